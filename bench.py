@@ -1,0 +1,198 @@
+#!/usr/bin/env python3
+"""Benchmark of the TW-Marlin W4A16 decode path on one MI355X.
+
+Workload (BASELINE.json configs[2]): the four M=1 GEMVs of a Qwen-7B-shaped layer
+    qkv 3584->4608, o 3584->3584, gate_up 3584->37888, down 18944->3584
+group-32 Q4 weights + FP16 scales, FP16 activations, FP32 outputs, each layer captured as one
+hipGraph.  One "step" = one layer = one graph replay.  Several distinct layers (default 4,
+525 MB of weights) are replayed round-robin so that the 256 MB Infinity Cache cannot hold the
+working set and the rate is an HBM rate.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers L] [--no-cpu] [--extra]
+
+Prints ONE JSON line. `value` = algorithmic bytes of a layer x K / time of K replays (inputs
+resident in HBM). `roofline` is for the dominant kernel, the gate_up GEMV, timed with HIP events
+on the stream it runs on. `cpu_baseline` is the CPU oracle (a port of the reference's CPU
+semantics: TW-Marlin unpack to dense f32, then the naive cpu_gemm loop) on one layer, one thread.
+"""
+import argparse
+import json
+import sys
+import time
+
+import numpy as np
+
+HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
+MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X dense FP16 matrix, published
+
+LAYER_7B = [("qkv", 3584, 4608), ("o", 3584, 3584), ("gate_up", 3584, 37888), ("down", 18944, 3584)]
+# HBM bytes per gate_up launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (see profiles/);
+# None until such a run has been made for the kernel in this tree.
+GATE_UP_TRAFFIC_BYTES = None
+
+
+def algo_bytes(k, n, m=1):
+    """K*N/2 nibbles + (K/32)*N*2 scales + M*K*2 FP16 activations + M*N*4 FP32 outputs"""
+    return k * n // 2 + (k // 32) * n * 2 + m * k * 2 + m * n * 4
+
+
+def make_layer(rng, shapes):
+    host = {}
+    for name, k, n in shapes:
+        packed = rng.integers(0, 256, size=(k // 32) * n * 16, dtype=np.uint8)          # nibbles uniform 0..15
+        scales = (np.abs(rng.standard_normal((k // 32) * n, dtype=np.float32)) * np.float32(0.02)).astype(np.float16)
+        act = rng.standard_normal(k, dtype=np.float32).astype(np.float16)               # f16(N(0,1))
+        host[name] = (packed, scales.view(np.uint16), act.view(np.uint16))
+    return host
+
+
+def time_launches(dev, fn, reps):
+    """average milliseconds per call of fn() over `reps` calls, HIP events on the context's stream"""
+    e0, e1 = dev.event(), dev.event()
+    dev.record(e0)
+    for i in range(reps):
+        fn(i)
+    dev.record(e1)
+    ms = dev.elapsed_ms(e0, e1)
+    dev.event_destroy(e0)
+    dev.event_destroy(e1)
+    return ms / reps
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=400)
+    ap.add_argument("--warmup", type=int, default=40)
+    ap.add_argument("--layers", type=int, default=4, help="distinct weight sets rotated through (>=3 defeats the 256 MB cache)")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
+    ap.add_argument("--extra", action="store_true", help="also time batched decode (M=4..32) on the gate_up shape")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on ONE GPU; --gpus %d is not supported (no collectives, no sharding)" % args.gpus)
+
+    import tensorwarp_amd as T
+
+    dev = T.WarpDevice(0)
+    rng = np.random.default_rng(20250101)
+    layers_host = [make_layer(rng, LAYER_7B) for _ in range(args.layers)]
+    layers = []
+    for host in layers_host:
+        entry = {}
+        for name, k, n in LAYER_7B:
+            packed, scales, act = host[name]
+            entry[name] = (T.MarlinWeight.upload(dev, packed, scales, k, n),
+                           T.GpuTensor.from_host(dev, act, "f16"),
+                           T.GpuTensor.zeros(dev, (n,), "f32"))
+        layers.append(entry)
+
+    def run_layer(li):
+        entry = layers[li]
+        for name, k, n in LAYER_7B:
+            w, a, c = entry[name]
+            T.gemm(dev, w, a, 1, c)
+
+    # eager warm-up (also loads every code object before capture), then one graph per layer
+    for li in range(args.layers):
+        run_layer(li)
+    dev.synchronize()
+    graphs = [T.GraphCapture.record_with_device(dev, lambda li=li: run_layer(li)) for li in range(args.layers)]
+
+    for i in range(args.warmup):
+        graphs[i % args.layers].replay()
+    dev.synchronize()
+    t0 = time.perf_counter()
+    ms_step = time_launches(dev, lambda i: graphs[i % args.layers].replay(), args.steps)
+    dev.synchronize()
+    wall = time.perf_counter() - t0
+
+    layer_bytes = sum(algo_bytes(k, n) for _, k, n in LAYER_7B)
+    value = layer_bytes / (ms_step * 1e-3) / 1e9
+
+    # per-projection timings, eager launches rotating over the distinct layers
+    per_shape = {}
+    for name, k, n in LAYER_7B:
+        def one(i, name=name):
+            w, a, c = layers[i % args.layers][name]
+            T.gemm(dev, w, a, 1, c)
+        for i in range(20):
+            one(i)
+        dev.synchronize()
+        ms = time_launches(dev, one, 200)
+        b = algo_bytes(k, n)
+        per_shape[name] = {"k": k, "n": n, "us": round(ms * 1e3, 3), "GBps": round(b / (ms * 1e-3) / 1e9, 1),
+                           "frac_hbm": round(b / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+                           "splits": T.pick_splits(k, n, 1)}
+
+    gu = per_shape["gate_up"]
+    gu_bytes = algo_bytes(3584, 37888)
+    roofline = {"bound": "hbm", "kernel": "k_decode (gate_up 3584->37888, M=1)",
+                "achieved": gu["GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                "frac": round(gu["GBps"] / HBM_PEAK_GBS, 4),
+                "bytes_per_launch": gu_bytes, "us_per_launch": gu["us"],
+                "traffic": GATE_UP_TRAFFIC_BYTES}
+
+    extra = {}
+    if args.extra:
+        k, n = 3584, 37888
+        for m in (4, 8, 16, 32):
+            a_m = T.GpuTensor.from_host(dev, rng.standard_normal((m, k), dtype=np.float32).astype(np.float16).view(np.uint16), "f16")
+            c_m = T.GpuTensor.zeros(dev, (m, n), "f32")
+
+            def one(i, a_m=a_m, c_m=c_m, m=m):
+                T.gemm(dev, layers[i % args.layers]["gate_up"][0], a_m, m, c_m)
+            for i in range(10):
+                one(i)
+            dev.synchronize()
+            ms = time_launches(dev, one, 100)
+            b = algo_bytes(k, n, m)
+            extra["gate_up_M%d" % m] = {"us": round(ms * 1e3, 2), "GBps": round(b / (ms * 1e-3) / 1e9, 1),
+                                        "frac_hbm": round(b / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
+
+    cpu = None
+    if not args.no_cpu:
+        # the checker, timed: reference CPU semantics on layer 0, one thread, whole layer once
+        from oracle import twm_oracle as O
+        host = layers_host[0]
+        t_cpu = 0.0
+        worst = 0.0
+        for name, k, n in LAYER_7B:
+            packed, scales, act = host[name]
+            a32 = act.view(np.float16).astype(np.float32).reshape(1, k)
+            t1 = time.perf_counter()
+            c_cpu = O.linear_dense(a32, packed, scales, 1, k, n)
+            t_cpu += time.perf_counter() - t1
+            w, a, c = layers[0][name]
+            T.gemm(dev, w, a, 1, c)
+            got = c.to_host().astype(np.float64)
+            truth = c_cpu[0].astype(np.float64)
+            denom = np.maximum(np.abs(truth), 1e-3 * np.abs(truth).max())
+            worst = max(worst, float((np.abs(got - truth) / denom).max()))
+        cpu = {"value": round(layer_bytes / t_cpu / 1e9, 4), "unit": "GB/s", "cores": 1, "kind": "port",
+               "sample": "one Qwen-7B-shaped layer (4 GEMVs, M=1, 131.3 MB algorithmic), unpack to dense f32 + naive cpu_gemm, run once",
+               "seconds": round(t_cpu, 3), "gpu_over_cpu": round(value / (layer_bytes / t_cpu / 1e9), 1),
+               "max_rel_err_gpu_vs_cpu": worst}
+
+    out = {
+        "metric": "achieved HBM GB/s of the W4A16 GEMV set at M=1 (Qwen-7B layer shapes, one hipGraph per layer)",
+        "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_step, 6), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f16 x int4 -> f32", "data": "synthetic",
+        "config": {"workload": "Qwen-7B decode linear set, M=1: qkv 3584->4608, o 3584->3584, gate_up 3584->37888, "
+                               "down 18944->3584; group-32 Q4 + FP16 scales; %d distinct layers rotated" % args.layers,
+                   "layer_bytes": layer_bytes, "frac_hbm_peak": round(value / HBM_PEAK_GBS, 4),
+                   "us_per_layer": round(ms_step * 1e3, 3), "wall_s": round(wall, 3)},
+        "roofline": roofline,
+        "cpu_baseline": cpu,
+        "per_projection": per_shape,
+    }
+    if extra:
+        out["batched_decode"] = extra
+    print(json.dumps(out))
+    for g in graphs:
+        g.destroy()
+    dev.close()
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,203 @@
+/*
+ * twmarlin.h - C ABI of libtwmarlin_hip.so, the MI355X (gfx950) implementation
+ * of TensorWarp's TW-Marlin W4A16 quantized-linear path.
+ *
+ * The library stands in for vendor/cudarc + the NVRTC kernel strings of
+ * crates/kernels/src/quantize.rs on this one path.  Every entry point cites the
+ * reference interface it replaces (paths relative to the reference checkout).
+ *
+ * Conventions (taken from the reference's own C API, crates/kernels/src/c_api.rs:26-67):
+ *   - opaque handles, every create paired with a destroy, NULL handles rejected;
+ *   - functions return an int status whose values equal c_api.rs `WarpError`;
+ *   - nothing panics or aborts across the ABI; twm_last_error() holds the text the
+ *     reference would have put in DeviceError::{Init,Memory,Launch}(String)
+ *     (crates/kernels/src/device.rs:278-292);
+ *   - all work is asynchronous and ordered on the context's stream; the caller
+ *     synchronises (device.rs:196-200).  A context must be driven by one host
+ *     thread / one stream at a time: split-K scratch memory is per context.
+ *   - pointers named *_dev are device pointers (from twm_malloc or any other
+ *     hipMalloc-compatible allocator, e.g. a torch tensor's data_ptr()); pointers
+ *     named *_host are host pointers.
+ *
+ * TW-Marlin format (quantize.rs:892-907, 1190-1191; gemma_moe_q4.rs:213-254), G = K/32:
+ *   packed : u8  [G][N][16]   byte i of a record = q[32g+2i] | q[32g+2i+1] << 4
+ *   scales : f16 [G][N]
+ *   weight : w[k][n] = f32(scales[k/32][n]) * (q[k][n] - 8)
+ */
+#ifndef TWMARLIN_H
+#define TWMARLIN_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* c_api.rs:41-50 `WarpError` */
+enum {
+    TWM_OK = 0,
+    TWM_DEVICE_ERROR = 1,
+    TWM_MEMORY_ERROR = 2,
+    TWM_SHAPE_ERROR = 3,
+    TWM_UNSUPPORTED_OP = 4,
+    TWM_INVALID_HANDLE = 5
+};
+
+/* c_api.rs:31-39 `WarpDType` */
+enum {
+    TWM_F32 = 0,
+    TWM_F16 = 1,
+    TWM_I32 = 2,
+    TWM_I8 = 3,
+    TWM_U8 = 4
+};
+
+typedef struct twm_ctx twm_ctx;       /* WarpDevice + KernelCache (device.rs, cache.rs) */
+typedef struct twm_weight twm_weight; /* one projection's (packed, scales) pair, repacked for gfx950 */
+typedef struct twm_graph twm_graph;   /* GraphCapture (cuda_graph.rs:72-118) */
+
+/* ---- library / device ------------------------------------------------------ */
+
+/* c_api.rs:107-112 warp_version */
+const char *twm_version(void);
+/* c_api.rs:101-105 warp_device_count */
+int twm_device_count(void);
+/* Text of the last failure on the calling thread ("" if none). */
+const char *twm_last_error(void);
+
+/* c_api.rs:52-59 warp_device_create / WarpDevice::new (device.rs) + KernelCache::new.
+ * All kernels are precompiled gfx950 code inside the library, so there is no
+ * JIT step.  Creates the context's own stream and its split-K scratch.
+ * Returns NULL on failure. */
+twm_ctx *twm_ctx_create(int ordinal);
+/* c_api.rs:61-67 warp_device_destroy */
+void twm_ctx_destroy(twm_ctx *ctx);
+/* c_api.rs:90-99 warp_device_sync / WarpDevice::synchronize (device.rs:196-200) */
+int twm_ctx_sync(twm_ctx *ctx);
+/* WarpDevice::with_stream (device.rs:230-265): run subsequent work on a caller-owned
+ * hipStream_t (e.g. the stream a framework already uses).  NULL restores the
+ * context's own stream. */
+int twm_ctx_set_stream(twm_ctx *ctx, void *hip_stream);
+/* The hipStream_t work is currently issued on. */
+void *twm_ctx_stream(twm_ctx *ctx);
+/* c_api.rs:69-80 warp_device_info: fills buf with "<name> | <CUs> CUs | <GiB> GiB". */
+int twm_ctx_info(twm_ctx *ctx, char *buf, size_t buf_len);
+/* Tuning knob for per-shape sweeps (the role AutoTuner::tune_gemm plays in
+ * crates/kernels/src/autotune.rs:254-396): key "nt" = 16-column tiles per workgroup,
+ * 0 = library's choice, else 1, 2 or 4. */
+int twm_ctx_set_option(twm_ctx *ctx, const char *key, int value);
+
+/* ---- device memory (GpuTensor::{zeros,from_host,to_host}, tensor.rs:9-104) ------ */
+
+void *twm_malloc(twm_ctx *ctx, size_t bytes);
+int twm_free(twm_ctx *ctx, void *ptr_dev);
+int twm_memcpy_h2d(twm_ctx *ctx, void *dst_dev, const void *src_host, size_t bytes); /* synchronous */
+int twm_memcpy_d2h(twm_ctx *ctx, void *dst_host, const void *src_dev, size_t bytes); /* synchronous */
+int twm_memcpy_d2d(twm_ctx *ctx, void *dst_dev, const void *src_dev, size_t bytes);  /* stream ordered */
+/* stream.memset_zeros (quantize.rs:1349); done by a fill kernel so that it may be graph captured */
+int twm_memset_zero(twm_ctx *ctx, void *ptr_dev, size_t bytes);
+
+/* ---- timing on the context's stream --------------------------------------------- */
+
+void *twm_event_create(twm_ctx *ctx);
+int twm_event_destroy(twm_ctx *ctx, void *event);
+int twm_event_record(twm_ctx *ctx, void *event);
+/* waits for `stop`, then returns the time between the two records in milliseconds */
+int twm_event_elapsed_ms(twm_ctx *ctx, void *start, void *stop, float *ms_out);
+
+/* ---- TW-Marlin format operations on device arrays in the reference layout -------- */
+
+/* quantize_weights_q4_0 (quantize.rs:414-474): w_kn_dev f32 row-major [K,N] ->
+ * Q4_0 20-byte blocks, column-major placement (col*G + g)*20 as documented at
+ * quantize.rs:410-413 and read by every consumer. */
+int twm_quantize_weights_q4_0(twm_ctx *ctx, const float *w_kn_dev, uint32_t k, uint32_t n,
+                              uint8_t *q4_dev);
+/* reorder_to_tw_marlin (quantize.rs:912-956): Q4_0 column-major -> (packed, scales f16). */
+int twm_reorder_to_tw_marlin(twm_ctx *ctx, const uint8_t *q4_dev, uint32_t k, uint32_t n,
+                             uint8_t *packed_dev, uint16_t *scales_dev);
+/* quantize_f32_to_tw_marlin (quantize.rs:1171-1180) in one pass; also equals
+ * cpu_quantize_tw_marlin (gemma_moe_q4.rs:218-254) when w_is_nk != 0 and the
+ * input is row-major [N,K]. */
+int twm_quantize_f32_to_tw_marlin(twm_ctx *ctx, const float *w_dev, int w_is_nk, uint32_t k,
+                                  uint32_t n, uint8_t *packed_dev, uint16_t *scales_dev);
+/* fuse_tw_marlin_n (quantize.rs:1018-1063): concatenate `count` matrices along N.
+ * packed_devs / scales_devs / ns are host arrays of `count` entries. */
+int twm_fuse_tw_marlin_n(twm_ctx *ctx, const uint8_t *const *packed_devs,
+                         const uint16_t *const *scales_devs, uint32_t k, const uint32_t *ns,
+                         uint32_t count, uint8_t *packed_out_dev, uint16_t *scales_out_dev);
+/* warp_dequant_q4_to_f16 / dequant_q4_to_f16 (quantize.rs:534-618) for TW-Marlin input:
+ * out[k][n] = f16_rne(f32(scale) * (q - 8)), row-major [K,N].  The "Q4 unpack". */
+int twm_dequant_to_f16(twm_ctx *ctx, const uint8_t *packed_dev, const uint16_t *scales_dev,
+                       uint32_t k, uint32_t n, uint16_t *out_kn_dev);
+/* same, f32 output (exact product) */
+int twm_dequant_to_f32(twm_ctx *ctx, const uint8_t *packed_dev, const uint16_t *scales_dev,
+                       uint32_t k, uint32_t n, float *out_kn_dev);
+/* split_qkv (ops.rs:2300-2321) and split_gate_up (ops.rs:2324-2343) */
+int twm_split_qkv(twm_ctx *ctx, const float *qkv_dev, float *q_dev, float *k_dev, float *v_dev,
+                  uint32_t h, uint32_t kv_dim, uint32_t batch);
+int twm_split_gate_up(twm_ctx *ctx, const float *gate_up_dev, float *gate_dev, float *up_dev,
+                      uint32_t ffn_dim, uint32_t batch);
+
+/* ---- the quantized-GEMM entry point, reference layout in, no repack ------------------ */
+
+/* gemm_tw_marlin_m1 (quantize.rs:1301-1360): C[1,N] = A[1,K] * dequant(packed, scales),
+ * f32 activations and output, arrays exactly as the reference holds them.
+ * K % 32 != 0 returns TWM_SHAPE_ERROR where the reference asserts (quantize.rs:1311). */
+int twm_gemm_tw_marlin_m1(twm_ctx *ctx, const float *a_dev, const uint8_t *packed_dev,
+                          const uint16_t *scales_dev, float *c_dev, uint32_t n, uint32_t k);
+/* gemm_tw_marlin_m1_from_buffer (quantize.rs:1731-1782): offsets in bytes (packed) and in
+ * f16 elements (scales) into larger slabs. */
+int twm_gemm_tw_marlin_m1_from_buffer(twm_ctx *ctx, const float *a_dev, const uint8_t *packed_buf_dev,
+                                      size_t packed_offset, const uint16_t *scales_buf_dev,
+                                      size_t scales_offset, float *c_dev, uint32_t n, uint32_t k);
+/* The reference's adaptive split-K rule, bit for bit (quantize.rs:1314-1325). */
+void twm_pick_splits_reference(uint32_t k, uint32_t n, uint32_t *n_blocks, uint32_t *splits,
+                               uint32_t *groups_per_split);
+
+/* ---- the same path with weights repacked once at upload (the fast path) ------------- */
+
+/* Takes exactly the reference's TW-Marlin arrays (host) and repacks them on the GPU into
+ * the wavefront tile order the gfx950 kernels stream.  Replaces the from_host uploads at
+ * quantize.rs:950-953 / 1057-1060. */
+twm_weight *twm_weight_upload(twm_ctx *ctx, const uint8_t *packed_host, const uint16_t *scales_host,
+                              uint32_t k, uint32_t n);
+/* Same from device arrays (e.g. the output of twm_fuse_tw_marlin_n). The inputs are not retained. */
+twm_weight *twm_weight_from_device(twm_ctx *ctx, const uint8_t *packed_dev, const uint16_t *scales_dev,
+                                   uint32_t k, uint32_t n);
+void twm_weight_destroy(twm_weight *w);
+int twm_weight_dims(const twm_weight *w, uint32_t *k, uint32_t *n);
+/* device bytes held by the repacked weight */
+size_t twm_weight_bytes(const twm_weight *w);
+/* "Q4 unpack" straight from the repacked form: out[k][n] f16 row-major [K,N]; must be
+ * bit-identical to twm_dequant_to_f16 of the arrays the weight was made from. */
+int twm_weight_dequant_f16(twm_ctx *ctx, const twm_weight *w, uint16_t *out_kn_dev);
+
+/* C[M,N] (f32, row-major) = A[M,K] (f16 or f32, row-major) * dequant(W), f32 accumulation.
+ * M = 1 is gemm_tw_marlin_m1 (quantize.rs:1301); M > 1 has the semantics of gemm_q4_0
+ * (quantize.rs:1825-1858).  splits = 0 lets the library choose (twm_pick_splits). */
+int twm_gemm(twm_ctx *ctx, const twm_weight *w, const void *a_dev, int a_dtype, uint32_t m,
+             float *c_dev, uint32_t splits);
+/* Fused projection with the split folded into the store: column ranges of the fused
+ * weight go straight to separate buffers, replacing gemm_tw_marlin_m1 + split_qkv /
+ * split_gate_up (generate.rs:2152-2155, 2195-2198).  outs_dev / ns are host arrays;
+ * sum(ns) must equal the weight's N; out i is row-major [M, ns[i]] f32. */
+int twm_gemm_split(twm_ctx *ctx, const twm_weight *w, const void *a_dev, int a_dtype, uint32_t m,
+                   float *const *outs_dev, const uint32_t *ns, uint32_t count, uint32_t splits);
+/* The library's split-K choice for MI355X (256 CUs); same role as quantize.rs:1317-1325. */
+uint32_t twm_pick_splits(uint32_t k, uint32_t n, uint32_t m);
+
+/* ---- graph capture / replay (GraphCapture::{record_with_device, replay}, cuda_graph.rs:85-117) */
+
+/* Starts capturing the work issued on the context's stream. */
+int twm_graph_begin(twm_ctx *ctx);
+/* Ends capture and instantiates; NULL on failure. */
+twm_graph *twm_graph_end(twm_ctx *ctx);
+/* GraphCapture::replay */
+int twm_graph_launch(twm_ctx *ctx, twm_graph *g);
+void twm_graph_destroy(twm_graph *g);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TWMARLIN_H */

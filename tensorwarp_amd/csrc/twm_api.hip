@@ -1,0 +1,701 @@
+// C ABI of libtwmarlin_hip.so (declared in include/twmarlin.h): contexts, device memory,
+// weight upload with one-time repack, the quantized-GEMM dispatcher with its split-K choice,
+// and hipGraph capture/replay.  Host-side counterpart of the reference's
+// crates/kernels/src/{quantize.rs:1301-1360, device.rs, tensor.rs, cuda_graph.rs}.
+#include "../../include/twmarlin.h"
+#include "twm_internal.h"
+
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include <new>
+#include <string>
+#include <vector>
+
+using namespace twm;
+
+static thread_local std::string g_err;
+
+static int fail(int code, const char *fmt, ...)
+{
+    char buf[512];
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(buf, sizeof buf, fmt, ap);
+    va_end(ap);
+    g_err = buf;
+    return code;
+}
+
+#define HIP_TRY(expr, code, what)                                                      \
+    do {                                                                               \
+        hipError_t e__ = (expr);                                                       \
+        if (e__ != hipSuccess) return fail(code, "%s: %s", what, hipGetErrorString(e__)); \
+    } while (0)
+
+struct twm_ctx {
+    int ordinal;
+    hipStream_t own_stream;
+    hipStream_t stream;
+    float *ws;            // split-K partial tiles
+    size_t ws_bytes;
+    unsigned *counters;   // one arrival counter per tile group, zero between launches
+    uint32_t n_counters;
+    bool capturing;
+    int force_nt;         // 0 = heuristic
+    hipDeviceProp_t prop;
+};
+
+struct twm_weight {
+    twm_ctx *ctx;
+    void *qw;
+    void *sc;
+    uint32_t k, n, groups, n_tiles, k_chunks;
+    size_t bytes;
+};
+
+struct twm_graph {
+    hipGraph_t graph;
+    hipGraphExec_t exec;
+};
+
+static const size_t kWsBytes = 64ull << 20;
+static const uint32_t kCounters = 1u << 16;
+
+extern "C" {
+
+const char *twm_version(void) { return "0.1.0"; }
+
+int twm_device_count(void)
+{
+    int n = 0;
+    if (hipGetDeviceCount(&n) != hipSuccess) return 0;
+    return n;
+}
+
+const char *twm_last_error(void) { return g_err.c_str(); }
+
+twm_ctx *twm_ctx_create(int ordinal)
+{
+    int count = 0;
+    hipError_t e = hipGetDeviceCount(&count);
+    if (e != hipSuccess || ordinal < 0 || ordinal >= count) {
+        fail(TWM_DEVICE_ERROR, "twm_ctx_create: no HIP device %d (%s)", ordinal,
+             e != hipSuccess ? hipGetErrorString(e) : "ordinal out of range");
+        return nullptr;
+    }
+    twm_ctx *c = new (std::nothrow) twm_ctx();
+    if (!c) { fail(TWM_MEMORY_ERROR, "twm_ctx_create: out of host memory"); return nullptr; }
+    c->ordinal = ordinal;
+    c->capturing = false;
+    c->force_nt = 0;
+    c->ws = nullptr;
+    c->counters = nullptr;
+    c->own_stream = nullptr;
+    bool ok = hipSetDevice(ordinal) == hipSuccess && hipGetDeviceProperties(&c->prop, ordinal) == hipSuccess;
+    if (ok && strncmp(c->prop.gcnArchName, "gfx950", 6) != 0) {
+        fail(TWM_DEVICE_ERROR, "twm_ctx_create: device %d is %s; this library holds gfx950 code only", ordinal,
+             c->prop.gcnArchName);
+        delete c;
+        return nullptr;
+    }
+    ok = ok && hipStreamCreateWithFlags(&c->own_stream, hipStreamNonBlocking) == hipSuccess;
+    c->stream = c->own_stream;
+    c->ws_bytes = kWsBytes;
+    c->n_counters = kCounters;
+    ok = ok && hipMalloc((void **)&c->ws, c->ws_bytes) == hipSuccess;
+    ok = ok && hipMalloc((void **)&c->counters, c->n_counters * sizeof(unsigned)) == hipSuccess;
+    ok = ok && hipMemset(c->counters, 0, c->n_counters * sizeof(unsigned)) == hipSuccess;
+    ok = ok && hipDeviceSynchronize() == hipSuccess;
+    if (!ok) {
+        fail(TWM_DEVICE_ERROR, "twm_ctx_create: %s", hipGetErrorString(hipGetLastError()));
+        if (c->ws) (void)hipFree(c->ws);
+        if (c->counters) (void)hipFree(c->counters);
+        if (c->own_stream) (void)hipStreamDestroy(c->own_stream);
+        delete c;
+        return nullptr;
+    }
+    return c;
+}
+
+void twm_ctx_destroy(twm_ctx *ctx)
+{
+    if (!ctx) return;
+    (void)hipSetDevice(ctx->ordinal);
+    (void)hipStreamSynchronize(ctx->stream);
+    (void)hipFree(ctx->ws);
+    (void)hipFree(ctx->counters);
+    (void)hipStreamDestroy(ctx->own_stream);
+    delete ctx;
+}
+
+int twm_ctx_sync(twm_ctx *ctx)
+{
+    if (!ctx) return fail(TWM_INVALID_HANDLE, "twm_ctx_sync: null context");
+    HIP_TRY(hipStreamSynchronize(ctx->stream), TWM_DEVICE_ERROR, "stream synchronize");
+    return TWM_OK;
+}
+
+int twm_ctx_set_stream(twm_ctx *ctx, void *hip_stream)
+{
+    if (!ctx) return fail(TWM_INVALID_HANDLE, "twm_ctx_set_stream: null context");
+    if (ctx->capturing) return fail(TWM_UNSUPPORTED_OP, "twm_ctx_set_stream: a graph capture is open");
+    ctx->stream = hip_stream ? (hipStream_t)hip_stream : ctx->own_stream;
+    return TWM_OK;
+}
+
+void *twm_ctx_stream(twm_ctx *ctx) { return ctx ? (void *)ctx->stream : nullptr; }
+
+int twm_ctx_info(twm_ctx *ctx, char *buf, size_t buf_len)
+{
+    if (!ctx || !buf || buf_len == 0) return fail(TWM_INVALID_HANDLE, "twm_ctx_info: null argument");
+    snprintf(buf, buf_len, "%s (%s) | %d CUs | %.1f GiB", ctx->prop.name, ctx->prop.gcnArchName,
+             ctx->prop.multiProcessorCount, (double)ctx->prop.totalGlobalMem / (1024.0 * 1024.0 * 1024.0));
+    return TWM_OK;
+}
+
+/* Tuning knob for sweeps: "nt" = n-tiles per workgroup (0 = heuristic, else 1, 2 or 4). */
+int twm_ctx_set_option(twm_ctx *ctx, const char *key, int value)
+{
+    if (!ctx || !key) return fail(TWM_INVALID_HANDLE, "twm_ctx_set_option: null argument");
+    if (strcmp(key, "nt") == 0) {
+        if (value != 0 && value != 1 && value != 2 && value != 4)
+            return fail(TWM_SHAPE_ERROR, "twm_ctx_set_option: nt must be 0, 1, 2 or 4");
+        ctx->force_nt = value;
+        return TWM_OK;
+    }
+    return fail(TWM_UNSUPPORTED_OP, "twm_ctx_set_option: unknown key %s", key);
+}
+
+/* ---- memory ---------------------------------------------------------------------------- */
+
+void *twm_malloc(twm_ctx *ctx, size_t bytes)
+{
+    if (!ctx) { fail(TWM_INVALID_HANDLE, "twm_malloc: null context"); return nullptr; }
+    if (ctx->capturing) { fail(TWM_UNSUPPORTED_OP, "twm_malloc: not allowed inside a graph capture"); return nullptr; }
+    void *p = nullptr;
+    hipError_t e = hipMalloc(&p, bytes ? bytes : 4);
+    if (e != hipSuccess) { fail(TWM_MEMORY_ERROR, "hipMalloc(%zu): %s", bytes, hipGetErrorString(e)); return nullptr; }
+    return p;
+}
+
+int twm_free(twm_ctx *ctx, void *ptr_dev)
+{
+    if (!ctx) return fail(TWM_INVALID_HANDLE, "twm_free: null context");
+    if (!ptr_dev) return TWM_OK;
+    HIP_TRY(hipFree(ptr_dev), TWM_MEMORY_ERROR, "hipFree");
+    return TWM_OK;
+}
+
+int twm_memcpy_h2d(twm_ctx *ctx, void *dst_dev, const void *src_host, size_t bytes)
+{
+    if (!ctx) return fail(TWM_INVALID_HANDLE, "twm_memcpy_h2d: null context");
+    if (bytes == 0) return TWM_OK;
+    if (!dst_dev || !src_host) return fail(TWM_INVALID_HANDLE, "twm_memcpy_h2d: null pointer");
+    if (ctx->capturing) return fail(TWM_UNSUPPORTED_OP, "twm_memcpy_h2d: not allowed inside a graph capture");
+    HIP_TRY(hipMemcpyAsync(dst_dev, src_host, bytes, hipMemcpyHostToDevice, ctx->stream), TWM_MEMORY_ERROR, "memcpy h2d");
+    HIP_TRY(hipStreamSynchronize(ctx->stream), TWM_DEVICE_ERROR, "memcpy h2d sync");
+    return TWM_OK;
+}
+
+int twm_memcpy_d2h(twm_ctx *ctx, void *dst_host, const void *src_dev, size_t bytes)
+{
+    if (!ctx) return fail(TWM_INVALID_HANDLE, "twm_memcpy_d2h: null context");
+    if (bytes == 0) return TWM_OK;
+    if (!dst_host || !src_dev) return fail(TWM_INVALID_HANDLE, "twm_memcpy_d2h: null pointer");
+    if (ctx->capturing) return fail(TWM_UNSUPPORTED_OP, "twm_memcpy_d2h: not allowed inside a graph capture");
+    HIP_TRY(hipMemcpyAsync(dst_host, src_dev, bytes, hipMemcpyDeviceToHost, ctx->stream), TWM_MEMORY_ERROR, "memcpy d2h");
+    HIP_TRY(hipStreamSynchronize(ctx->stream), TWM_DEVICE_ERROR, "memcpy d2h sync");
+    return TWM_OK;
+}
+
+int twm_memcpy_d2d(twm_ctx *ctx, void *dst_dev, const void *src_dev, size_t bytes)
+{
+    if (!ctx) return fail(TWM_INVALID_HANDLE, "twm_memcpy_d2d: null context");
+    if (bytes == 0) return TWM_OK;
+    if (!dst_dev || !src_dev) return fail(TWM_INVALID_HANDLE, "twm_memcpy_d2d: null pointer");
+    HIP_TRY(hipMemcpyAsync(dst_dev, src_dev, bytes, hipMemcpyDeviceToDevice, ctx->stream), TWM_MEMORY_ERROR, "memcpy d2d");
+    return TWM_OK;
+}
+
+int twm_memset_zero(twm_ctx *ctx, void *ptr_dev, size_t bytes)
+{
+    if (!ctx) return fail(TWM_INVALID_HANDLE, "twm_memset_zero: null context");
+    if (bytes == 0) return TWM_OK;
+    if (!ptr_dev) return fail(TWM_INVALID_HANDLE, "twm_memset_zero: null pointer");
+    if (bytes % 4 != 0 || ((uintptr_t)ptr_dev & 3) != 0)
+        return fail(TWM_SHAPE_ERROR, "twm_memset_zero: pointer and size must be multiples of 4 bytes");
+    HIP_TRY(launch_fill_zero(ctx->stream, ptr_dev, bytes), TWM_DEVICE_ERROR, "fill kernel launch");
+    return TWM_OK;
+}
+
+/* ---- events ------------------------------------------------------------------------------ */
+
+void *twm_event_create(twm_ctx *ctx)
+{
+    if (!ctx) { fail(TWM_INVALID_HANDLE, "twm_event_create: null context"); return nullptr; }
+    hipEvent_t ev = nullptr;
+    hipError_t e = hipEventCreate(&ev);
+    if (e != hipSuccess) { fail(TWM_DEVICE_ERROR, "hipEventCreate: %s", hipGetErrorString(e)); return nullptr; }
+    return (void *)ev;
+}
+
+int twm_event_destroy(twm_ctx *ctx, void *event)
+{
+    if (!ctx || !event) return fail(TWM_INVALID_HANDLE, "twm_event_destroy: null argument");
+    HIP_TRY(hipEventDestroy((hipEvent_t)event), TWM_DEVICE_ERROR, "hipEventDestroy");
+    return TWM_OK;
+}
+
+int twm_event_record(twm_ctx *ctx, void *event)
+{
+    if (!ctx || !event) return fail(TWM_INVALID_HANDLE, "twm_event_record: null argument");
+    HIP_TRY(hipEventRecord((hipEvent_t)event, ctx->stream), TWM_DEVICE_ERROR, "hipEventRecord");
+    return TWM_OK;
+}
+
+int twm_event_elapsed_ms(twm_ctx *ctx, void *start, void *stop, float *ms_out)
+{
+    if (!ctx || !start || !stop || !ms_out) return fail(TWM_INVALID_HANDLE, "twm_event_elapsed_ms: null argument");
+    HIP_TRY(hipEventSynchronize((hipEvent_t)stop), TWM_DEVICE_ERROR, "hipEventSynchronize");
+    HIP_TRY(hipEventElapsedTime(ms_out, (hipEvent_t)start, (hipEvent_t)stop), TWM_DEVICE_ERROR, "hipEventElapsedTime");
+    return TWM_OK;
+}
+
+/* ---- format operations -------------------------------------------------------------------- */
+
+static int check_kn(const char *who, uint32_t k, uint32_t n)
+{
+    if (k % 32 != 0) return fail(TWM_SHAPE_ERROR, "%s: K (%u) must be divisible by 32", who, k);
+    if ((uint64_t)(k / 32) * n * 16 > (1ull << 40)) return fail(TWM_SHAPE_ERROR, "%s: K x N too large", who);
+    return TWM_OK;
+}
+
+int twm_quantize_weights_q4_0(twm_ctx *ctx, const float *w_kn_dev, uint32_t k, uint32_t n, uint8_t *q4_dev)
+{
+    if (!ctx) return fail(TWM_INVALID_HANDLE, "twm_quantize_weights_q4_0: null context");
+    if (int rc = check_kn("twm_quantize_weights_q4_0", k, n)) return rc;
+    if (k == 0 || n == 0) return TWM_OK;
+    if (!w_kn_dev || !q4_dev) return fail(TWM_INVALID_HANDLE, "twm_quantize_weights_q4_0: null pointer");
+    HIP_TRY(launch_quantize_q4_0(ctx->stream, w_kn_dev, k, n, q4_dev), TWM_DEVICE_ERROR, "quantize launch");
+    return TWM_OK;
+}
+
+int twm_reorder_to_tw_marlin(twm_ctx *ctx, const uint8_t *q4_dev, uint32_t k, uint32_t n, uint8_t *packed_dev,
+                             uint16_t *scales_dev)
+{
+    if (!ctx) return fail(TWM_INVALID_HANDLE, "twm_reorder_to_tw_marlin: null context");
+    if (int rc = check_kn("twm_reorder_to_tw_marlin", k, n)) return rc;
+    if (k == 0 || n == 0) return TWM_OK;
+    if (!q4_dev || !packed_dev || !scales_dev) return fail(TWM_INVALID_HANDLE, "twm_reorder_to_tw_marlin: null pointer");
+    HIP_TRY(launch_reorder(ctx->stream, q4_dev, k, n, packed_dev, scales_dev), TWM_DEVICE_ERROR, "reorder launch");
+    return TWM_OK;
+}
+
+int twm_quantize_f32_to_tw_marlin(twm_ctx *ctx, const float *w_dev, int w_is_nk, uint32_t k, uint32_t n,
+                                  uint8_t *packed_dev, uint16_t *scales_dev)
+{
+    if (!ctx) return fail(TWM_INVALID_HANDLE, "twm_quantize_f32_to_tw_marlin: null context");
+    if (int rc = check_kn("twm_quantize_f32_to_tw_marlin", k, n)) return rc;
+    if (k == 0 || n == 0) return TWM_OK;
+    if (!w_dev || !packed_dev || !scales_dev)
+        return fail(TWM_INVALID_HANDLE, "twm_quantize_f32_to_tw_marlin: null pointer");
+    HIP_TRY(launch_quantize_twm(ctx->stream, w_dev, w_is_nk, k, n, packed_dev, scales_dev), TWM_DEVICE_ERROR,
+            "quantize launch");
+    return TWM_OK;
+}
+
+int twm_fuse_tw_marlin_n(twm_ctx *ctx, const uint8_t *const *packed_devs, const uint16_t *const *scales_devs, uint32_t k,
+                         const uint32_t *ns, uint32_t count, uint8_t *packed_out_dev, uint16_t *scales_out_dev)
+{
+    if (!ctx) return fail(TWM_INVALID_HANDLE, "twm_fuse_tw_marlin_n: null context");
+    if (!packed_devs || !scales_devs || !ns) return fail(TWM_INVALID_HANDLE, "twm_fuse_tw_marlin_n: null array");
+    uint64_t total = 0;
+    for (uint32_t i = 0; i < count; i++) total += ns[i];
+    if (total > 0xFFFFFFFFull) return fail(TWM_SHAPE_ERROR, "twm_fuse_tw_marlin_n: fused N overflows u32");
+    if (int rc = check_kn("twm_fuse_tw_marlin_n", k, (uint32_t)total)) return rc;
+    if (total == 0 || k == 0) return TWM_OK;
+    if (!packed_out_dev || !scales_out_dev) return fail(TWM_INVALID_HANDLE, "twm_fuse_tw_marlin_n: null output");
+    uint32_t off = 0;
+    for (uint32_t i = 0; i < count; i++) {
+        if (ns[i] == 0) continue;
+        if (!packed_devs[i] || !scales_devs[i]) return fail(TWM_INVALID_HANDLE, "twm_fuse_tw_marlin_n: null input %u", i);
+        HIP_TRY(launch_fuse_one(ctx->stream, packed_devs[i], scales_devs[i], k / 32, ns[i], (uint32_t)total, off,
+                                packed_out_dev, scales_out_dev),
+                TWM_DEVICE_ERROR, "fuse launch");
+        off += ns[i];
+    }
+    return TWM_OK;
+}
+
+static int dequant_common(twm_ctx *ctx, const uint8_t *packed_dev, const uint16_t *scales_dev, uint32_t k, uint32_t n,
+                          void *out, bool f16)
+{
+    if (!ctx) return fail(TWM_INVALID_HANDLE, "twm_dequant: null context");
+    if (int rc = check_kn("twm_dequant", k, n)) return rc;
+    if (k == 0 || n == 0) return TWM_OK;
+    if (!packed_dev || !scales_dev || !out) return fail(TWM_INVALID_HANDLE, "twm_dequant: null pointer");
+    HIP_TRY(launch_dequant(ctx->stream, packed_dev, scales_dev, k, n, out, f16), TWM_DEVICE_ERROR, "dequant launch");
+    return TWM_OK;
+}
+
+int twm_dequant_to_f16(twm_ctx *ctx, const uint8_t *packed_dev, const uint16_t *scales_dev, uint32_t k, uint32_t n,
+                       uint16_t *out_kn_dev)
+{
+    return dequant_common(ctx, packed_dev, scales_dev, k, n, out_kn_dev, true);
+}
+
+int twm_dequant_to_f32(twm_ctx *ctx, const uint8_t *packed_dev, const uint16_t *scales_dev, uint32_t k, uint32_t n,
+                       float *out_kn_dev)
+{
+    return dequant_common(ctx, packed_dev, scales_dev, k, n, out_kn_dev, false);
+}
+
+int twm_split_qkv(twm_ctx *ctx, const float *qkv_dev, float *q_dev, float *k_dev, float *v_dev, uint32_t h,
+                  uint32_t kv_dim, uint32_t batch)
+{
+    if (!ctx) return fail(TWM_INVALID_HANDLE, "twm_split_qkv: null context");
+    if ((uint64_t)batch * ((uint64_t)h + 2ull * kv_dim) == 0) return TWM_OK;
+    if (!qkv_dev || !q_dev || !k_dev || !v_dev) return fail(TWM_INVALID_HANDLE, "twm_split_qkv: null pointer");
+    HIP_TRY(launch_split_qkv(ctx->stream, qkv_dev, q_dev, k_dev, v_dev, h, kv_dim, batch), TWM_DEVICE_ERROR,
+            "split_qkv launch");
+    return TWM_OK;
+}
+
+int twm_split_gate_up(twm_ctx *ctx, const float *gate_up_dev, float *gate_dev, float *up_dev, uint32_t ffn_dim,
+                      uint32_t batch)
+{
+    if (!ctx) return fail(TWM_INVALID_HANDLE, "twm_split_gate_up: null context");
+    if ((uint64_t)batch * ffn_dim == 0) return TWM_OK;
+    if (!gate_up_dev || !gate_dev || !up_dev) return fail(TWM_INVALID_HANDLE, "twm_split_gate_up: null pointer");
+    HIP_TRY(launch_split_gate_up(ctx->stream, gate_up_dev, gate_dev, up_dev, ffn_dim, batch), TWM_DEVICE_ERROR,
+            "split_gate_up launch");
+    return TWM_OK;
+}
+
+/* ---- GEMV on the reference layout ------------------------------------------------------- */
+
+void twm_pick_splits_reference(uint32_t k, uint32_t n, uint32_t *n_blocks, uint32_t *splits, uint32_t *groups_per_split)
+{
+    uint32_t groups = k / 32u;
+    uint32_t nb = (n + 255u) / 256u;
+    uint32_t sp;
+    if (k < 2048u || nb >= 128u) {
+        sp = 1;
+    } else {
+        uint32_t max_splits = groups / 8u;
+        if (max_splits < 1u) max_splits = 1u;
+        sp = (256u + nb - 1u) / nb;
+        if (sp < 1u) sp = 1u;
+        if (sp > max_splits) sp = max_splits;
+    }
+    if (n_blocks) *n_blocks = nb;
+    if (splits) *splits = sp;
+    if (groups_per_split) *groups_per_split = (groups + sp - 1u) / sp;
+}
+
+int twm_gemm_tw_marlin_m1(twm_ctx *ctx, const float *a_dev, const uint8_t *packed_dev, const uint16_t *scales_dev,
+                          float *c_dev, uint32_t n, uint32_t k)
+{
+    if (!ctx) return fail(TWM_INVALID_HANDLE, "twm_gemm_tw_marlin_m1: null context");
+    if (int rc = check_kn("twm_gemm_tw_marlin_m1", k, n)) return rc;
+    if (n == 0) return TWM_OK;
+    if (!c_dev) return fail(TWM_INVALID_HANDLE, "twm_gemm_tw_marlin_m1: null output");
+    if (k == 0) return twm_memset_zero(ctx, c_dev, (size_t)n * 4);
+    if (!a_dev || !packed_dev || !scales_dev) return fail(TWM_INVALID_HANDLE, "twm_gemm_tw_marlin_m1: null input");
+    if (((uintptr_t)packed_dev & 15) != 0) return fail(TWM_SHAPE_ERROR, "twm_gemm_tw_marlin_m1: packed must be 16-byte aligned");
+    uint32_t nb, sp, gps;
+    twm_pick_splits_reference(k, n, &nb, &sp, &gps);
+    HIP_TRY(launch_ref_gemv(ctx->stream, a_dev, packed_dev, scales_dev, c_dev, n, k, sp, gps), TWM_DEVICE_ERROR,
+            "gemv launch");
+    return TWM_OK;
+}
+
+int twm_gemm_tw_marlin_m1_from_buffer(twm_ctx *ctx, const float *a_dev, const uint8_t *packed_buf_dev,
+                                      size_t packed_offset, const uint16_t *scales_buf_dev, size_t scales_offset,
+                                      float *c_dev, uint32_t n, uint32_t k)
+{
+    if (!packed_buf_dev || !scales_buf_dev)
+        return fail(TWM_INVALID_HANDLE, "twm_gemm_tw_marlin_m1_from_buffer: null slab");
+    return twm_gemm_tw_marlin_m1(ctx, a_dev, packed_buf_dev + packed_offset, scales_buf_dev + scales_offset, c_dev, n, k);
+}
+
+/* ---- repacked weights ----------------------------------------------------------------------- */
+
+static twm_weight *weight_alloc(twm_ctx *ctx, uint32_t k, uint32_t n)
+{
+    twm_weight *w = new (std::nothrow) twm_weight();
+    if (!w) { fail(TWM_MEMORY_ERROR, "twm_weight: out of host memory"); return nullptr; }
+    w->ctx = ctx;
+    w->k = k;
+    w->n = n;
+    w->groups = k / 32;
+    uint32_t n_pad = ((n + kNPadTo - 1) / kNPadTo) * kNPadTo;
+    w->n_tiles = n_pad / kTileN;
+    w->k_chunks = (w->groups + kChunkGroups - 1) / kChunkGroups;
+    size_t tiles = (size_t)w->n_tiles * w->k_chunks;
+    size_t qbytes = tiles * 1024, sbytes = tiles * 128;
+    w->bytes = qbytes + sbytes;
+    w->qw = nullptr;
+    w->sc = nullptr;
+    if (tiles == 0) return w;
+    hipError_t e = hipMalloc(&w->qw, qbytes + sbytes);
+    if (e != hipSuccess) {
+        fail(TWM_MEMORY_ERROR, "twm_weight: hipMalloc(%zu): %s", qbytes + sbytes, hipGetErrorString(e));
+        delete w;
+        return nullptr;
+    }
+    w->sc = (char *)w->qw + qbytes;
+    return w;
+}
+
+twm_weight *twm_weight_from_device(twm_ctx *ctx, const uint8_t *packed_dev, const uint16_t *scales_dev, uint32_t k,
+                                   uint32_t n)
+{
+    if (!ctx) { fail(TWM_INVALID_HANDLE, "twm_weight_from_device: null context"); return nullptr; }
+    if (ctx->capturing) { fail(TWM_UNSUPPORTED_OP, "twm_weight_from_device: not allowed inside a graph capture"); return nullptr; }
+    if (check_kn("twm_weight_from_device", k, n)) return nullptr;
+    if ((uint64_t)k * n != 0 && (!packed_dev || !scales_dev)) {
+        fail(TWM_INVALID_HANDLE, "twm_weight_from_device: null pointer");
+        return nullptr;
+    }
+    if (((uintptr_t)packed_dev & 3) != 0) { fail(TWM_SHAPE_ERROR, "twm_weight_from_device: packed must be 4-byte aligned"); return nullptr; }
+    twm_weight *w = weight_alloc(ctx, k, n);
+    if (!w) return nullptr;
+    if (w->qw) {
+        hipError_t e = launch_repack(ctx->stream, packed_dev, scales_dev, k, n, w->qw, w->sc, w->n_tiles, w->k_chunks);
+        if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
+        if (e != hipSuccess) {
+            fail(TWM_DEVICE_ERROR, "twm_weight_from_device: repack: %s", hipGetErrorString(e));
+            (void)hipFree(w->qw);
+            delete w;
+            return nullptr;
+        }
+    }
+    return w;
+}
+
+twm_weight *twm_weight_upload(twm_ctx *ctx, const uint8_t *packed_host, const uint16_t *scales_host, uint32_t k,
+                              uint32_t n)
+{
+    if (!ctx) { fail(TWM_INVALID_HANDLE, "twm_weight_upload: null context"); return nullptr; }
+    if (ctx->capturing) { fail(TWM_UNSUPPORTED_OP, "twm_weight_upload: not allowed inside a graph capture"); return nullptr; }
+    if (check_kn("twm_weight_upload", k, n)) return nullptr;
+    size_t pbytes = (size_t)(k / 32) * n * 16, sbytes = (size_t)(k / 32) * n * 2;
+    if (pbytes == 0) return twm_weight_from_device(ctx, nullptr, nullptr, k, n);
+    if (!packed_host || !scales_host) { fail(TWM_INVALID_HANDLE, "twm_weight_upload: null pointer"); return nullptr; }
+    void *stage = nullptr;
+    hipError_t e = hipMalloc(&stage, pbytes + sbytes);
+    if (e != hipSuccess) { fail(TWM_MEMORY_ERROR, "twm_weight_upload: staging hipMalloc: %s", hipGetErrorString(e)); return nullptr; }
+    uint8_t *p = (uint8_t *)stage;
+    uint16_t *s = (uint16_t *)(p + pbytes);
+    twm_weight *w = nullptr;
+    if (twm_memcpy_h2d(ctx, p, packed_host, pbytes) == TWM_OK && twm_memcpy_h2d(ctx, s, scales_host, sbytes) == TWM_OK)
+        w = twm_weight_from_device(ctx, p, s, k, n);
+    (void)hipFree(stage);
+    return w;
+}
+
+void twm_weight_destroy(twm_weight *w)
+{
+    if (!w) return;
+    if (w->qw) {
+        (void)hipStreamSynchronize(w->ctx->stream);
+        (void)hipFree(w->qw);
+    }
+    delete w;
+}
+
+int twm_weight_dims(const twm_weight *w, uint32_t *k, uint32_t *n)
+{
+    if (!w) return fail(TWM_INVALID_HANDLE, "twm_weight_dims: null weight");
+    if (k) *k = w->k;
+    if (n) *n = w->n;
+    return TWM_OK;
+}
+
+size_t twm_weight_bytes(const twm_weight *w) { return w ? w->bytes : 0; }
+
+static WeightView view_of(const twm_weight *w)
+{
+    WeightView v;
+    v.qw = w->qw;
+    v.sc = w->sc;
+    v.k = w->k;
+    v.n = w->n;
+    v.groups = w->groups;
+    v.n_tiles = w->n_tiles;
+    v.k_chunks = w->k_chunks;
+    return v;
+}
+
+int twm_weight_dequant_f16(twm_ctx *ctx, const twm_weight *w, uint16_t *out_kn_dev)
+{
+    if (!ctx || !w) return fail(TWM_INVALID_HANDLE, "twm_weight_dequant_f16: null handle");
+    if ((uint64_t)w->k * w->n == 0) return TWM_OK;
+    if (!out_kn_dev) return fail(TWM_INVALID_HANDLE, "twm_weight_dequant_f16: null output");
+    HIP_TRY(launch_weight_dequant_f16(ctx->stream, view_of(w), out_kn_dev), TWM_DEVICE_ERROR, "dequant launch");
+    return TWM_OK;
+}
+
+/* ---- dispatcher --------------------------------------------------------------------------- */
+
+// Split-K / tile choice for 256 CUs x 4 SIMDs.  A workgroup is 4 waves; aim for ~1024
+// workgroups (16 waves per CU) while every wave still has at least one 128-deep k-chunk.
+static DecodePlan plan_decode(uint32_t n_tiles, uint32_t k_chunks, uint32_t m, int force_nt, uint32_t force_splits)
+{
+    DecodePlan p;
+    p.nt = 1;
+    if (n_tiles >= 4096 && m <= 16) p.nt = 4;
+    else if (n_tiles >= 2048) p.nt = 2;
+    if (force_nt) p.nt = (uint32_t)force_nt;
+    uint32_t tg = n_tiles / p.nt;
+    uint32_t max_splits = k_chunks / 4;
+    if (max_splits < 1) max_splits = 1;
+    uint32_t sp = tg ? (1024u + tg / 2) / tg : 1;
+    if (sp < 1) sp = 1;
+    if (sp > max_splits) sp = max_splits;
+    if (force_splits) sp = force_splits;
+    if (sp > k_chunks) sp = k_chunks ? k_chunks : 1;
+    p.splits = sp;
+    return p;
+}
+
+uint32_t twm_pick_splits(uint32_t k, uint32_t n, uint32_t m)
+{
+    uint32_t n_tiles = ((n + kNPadTo - 1) / kNPadTo) * kNPadTo / kTileN;
+    uint32_t k_chunks = (k / 32 + kChunkGroups - 1) / kChunkGroups;
+    return plan_decode(n_tiles, k_chunks, m > kMaxDecodeM ? kMaxDecodeM : m, 0, 0).splits;
+}
+
+static int gemm_common(twm_ctx *ctx, const twm_weight *w, const void *a_dev, int a_dtype, uint32_t m, const OutSpec &out,
+                       uint32_t splits, const char *who)
+{
+    if (a_dtype != TWM_F16 && a_dtype != TWM_F32) return fail(TWM_UNSUPPORTED_OP, "%s: activations must be f16 or f32", who);
+    if (m == 0 || w->n == 0) return TWM_OK;
+    if (w->k == 0) {
+        for (uint32_t s = 0; s < out.count; s++)
+            if (int rc = twm_memset_zero(ctx, out.seg[s].ptr, (size_t)m * out.seg[s].width * 4)) return rc;
+        return TWM_OK;
+    }
+    if (!a_dev) return fail(TWM_INVALID_HANDLE, "%s: null activations", who);
+    if (((uintptr_t)a_dev & 15) != 0) return fail(TWM_SHAPE_ERROR, "%s: activations must be 16-byte aligned", who);
+    WeightView v = view_of(w);
+    size_t a_row_bytes = (size_t)w->k * (a_dtype == TWM_F16 ? 2 : 4);
+    uint32_t n_ld = w->n_tiles * kTileN;
+    for (uint32_t m0 = 0; m0 < m; m0 += kMaxDecodeM) {
+        uint32_t mb = m - m0 < (uint32_t)kMaxDecodeM ? m - m0 : (uint32_t)kMaxDecodeM;
+        DecodePlan plan = plan_decode(w->n_tiles, w->k_chunks, mb, ctx->force_nt, splits);
+        if (mb > 16 && plan.nt == 4) plan.nt = 2;
+        // the scratch must hold splits x mb x n_ld partials and one counter per tile group
+        while (plan.splits > 1 && (size_t)plan.splits * mb * n_ld * 4 > ctx->ws_bytes) plan.splits--;
+        if (w->n_tiles / plan.nt > ctx->n_counters) plan.splits = 1;
+        OutSpec o = out;
+        for (uint32_t s = 0; s < o.count; s++) o.seg[s].ptr += (size_t)m0 * o.seg[s].width;
+        const char *a_blk = (const char *)a_dev + (size_t)m0 * a_row_bytes;
+        HIP_TRY(launch_decode(ctx->stream, v, a_blk, a_dtype == TWM_F32, mb, o, ctx->ws, ctx->counters, plan),
+                TWM_DEVICE_ERROR, "gemm launch");
+    }
+    return TWM_OK;
+}
+
+int twm_gemm(twm_ctx *ctx, const twm_weight *w, const void *a_dev, int a_dtype, uint32_t m, float *c_dev, uint32_t splits)
+{
+    if (!ctx || !w) return fail(TWM_INVALID_HANDLE, "twm_gemm: null handle");
+    if (w->ctx != ctx) return fail(TWM_INVALID_HANDLE, "twm_gemm: weight belongs to another context");
+    if (m != 0 && w->n != 0 && !c_dev) return fail(TWM_INVALID_HANDLE, "twm_gemm: null output");
+    OutSpec out;
+    memset(&out, 0, sizeof out);
+    out.count = 1;
+    out.seg[0].ptr = c_dev;
+    out.seg[0].start = 0;
+    out.seg[0].width = w->n;
+    return gemm_common(ctx, w, a_dev, a_dtype, m, out, splits, "twm_gemm");
+}
+
+int twm_gemm_split(twm_ctx *ctx, const twm_weight *w, const void *a_dev, int a_dtype, uint32_t m, float *const *outs_dev,
+                   const uint32_t *ns, uint32_t count, uint32_t splits)
+{
+    if (!ctx || !w) return fail(TWM_INVALID_HANDLE, "twm_gemm_split: null handle");
+    if (w->ctx != ctx) return fail(TWM_INVALID_HANDLE, "twm_gemm_split: weight belongs to another context");
+    if (!outs_dev || !ns) return fail(TWM_INVALID_HANDLE, "twm_gemm_split: null array");
+    if (count == 0 || count > (uint32_t)kMaxSegs)
+        return fail(TWM_SHAPE_ERROR, "twm_gemm_split: between 1 and %d outputs are supported", kMaxSegs);
+    OutSpec out;
+    memset(&out, 0, sizeof out);
+    uint64_t total = 0;
+    uint32_t used = 0;
+    for (uint32_t i = 0; i < count; i++) {
+        if (ns[i] == 0) continue;
+        if (m != 0 && !outs_dev[i]) return fail(TWM_INVALID_HANDLE, "twm_gemm_split: null output %u", i);
+        out.seg[used].ptr = outs_dev[i];
+        out.seg[used].start = (uint32_t)total;
+        out.seg[used].width = ns[i];
+        used++;
+        total += ns[i];
+    }
+    out.count = used;
+    if (total != w->n) return fail(TWM_SHAPE_ERROR, "twm_gemm_split: outputs cover %llu columns, weight has %u",
+                                   (unsigned long long)total, w->n);
+    return gemm_common(ctx, w, a_dev, a_dtype, m, out, splits, "twm_gemm_split");
+}
+
+/* ---- graphs ---------------------------------------------------------------------------------- */
+
+int twm_graph_begin(twm_ctx *ctx)
+{
+    if (!ctx) return fail(TWM_INVALID_HANDLE, "twm_graph_begin: null context");
+    if (ctx->capturing) return fail(TWM_UNSUPPORTED_OP, "twm_graph_begin: a capture is already open");
+    if (ctx->stream == nullptr) return fail(TWM_UNSUPPORTED_OP, "twm_graph_begin: cannot capture the null stream");
+    HIP_TRY(hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeRelaxed), TWM_DEVICE_ERROR, "hipStreamBeginCapture");
+    ctx->capturing = true;
+    return TWM_OK;
+}
+
+twm_graph *twm_graph_end(twm_ctx *ctx)
+{
+    if (!ctx) { fail(TWM_INVALID_HANDLE, "twm_graph_end: null context"); return nullptr; }
+    if (!ctx->capturing) { fail(TWM_UNSUPPORTED_OP, "twm_graph_end: no capture is open"); return nullptr; }
+    ctx->capturing = false;
+    hipGraph_t graph = nullptr;
+    hipError_t e = hipStreamEndCapture(ctx->stream, &graph);
+    if (e != hipSuccess || !graph) {
+        fail(TWM_DEVICE_ERROR, "hipStreamEndCapture: %s", hipGetErrorString(e));
+        return nullptr;
+    }
+    hipGraphExec_t exec = nullptr;
+    e = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
+    if (e != hipSuccess) {
+        fail(TWM_DEVICE_ERROR, "hipGraphInstantiate: %s", hipGetErrorString(e));
+        (void)hipGraphDestroy(graph);
+        return nullptr;
+    }
+    twm_graph *g = new (std::nothrow) twm_graph();
+    if (!g) {
+        fail(TWM_MEMORY_ERROR, "twm_graph_end: out of host memory");
+        (void)hipGraphExecDestroy(exec);
+        (void)hipGraphDestroy(graph);
+        return nullptr;
+    }
+    g->graph = graph;
+    g->exec = exec;
+    return g;
+}
+
+int twm_graph_launch(twm_ctx *ctx, twm_graph *g)
+{
+    if (!ctx || !g) return fail(TWM_INVALID_HANDLE, "twm_graph_launch: null handle");
+    if (ctx->capturing) return fail(TWM_UNSUPPORTED_OP, "twm_graph_launch: a capture is open");
+    HIP_TRY(hipGraphLaunch(g->exec, ctx->stream), TWM_DEVICE_ERROR, "hipGraphLaunch");
+    return TWM_OK;
+}
+
+void twm_graph_destroy(twm_graph *g)
+{
+    if (!g) return;
+    (void)hipGraphExecDestroy(g->exec);
+    (void)hipGraphDestroy(g->graph);
+    delete g;
+}
+
+}  // extern "C"

@@ -1,0 +1,63 @@
+// Internal declarations shared by the kernel file and the C-ABI host file.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace twm {
+
+// ---- repacked ("wave tile") weight layout ---------------------------------------
+// n-tile  = 16 output columns, k-chunk = 4 groups = 128 input features.
+//   qw : uint4 [n_tiles][k_chunks][64]   lane l = (kb = l/16, c = l%16); component i of the
+//        uint4 is word kb (k = 8*kb .. 8*kb+7) of group 4*kc+i, column 16*nt+c, with its eight
+//        nibbles reordered so that bit position 4*p holds k-offset {0,2,4,6,1,3,5,7}[p].
+//   sc : uint2 [n_tiles][k_chunks][16]   four f16 scales (groups 4*kc .. 4*kc+3) of column c.
+// Columns >= N and groups >= G are padded with nibble 8 / scale 0 (weight exactly 0).
+constexpr int kTileN = 16;
+constexpr int kChunkGroups = 4;
+constexpr int kNPadTo = 64;      // N is padded to a multiple of this, so 1, 2 or 4 tiles per block divide
+constexpr int kMaxSegs = 4;
+constexpr int kMaxDecodeM = 32;
+
+struct OutSeg {
+    float *ptr;
+    uint32_t start;  // first fused column of this segment
+    uint32_t width;  // number of columns = row stride of ptr
+};
+struct OutSpec {
+    OutSeg seg[kMaxSegs];
+    uint32_t count;
+};
+
+struct WeightView {
+    const void *qw;
+    const void *sc;
+    uint32_t k, n, groups, n_tiles, k_chunks;
+};
+
+struct DecodePlan {
+    uint32_t nt;      // n-tiles per workgroup (1, 2, 4)
+    uint32_t splits;  // cross-workgroup split-K factor
+};
+
+// ---- launchers (all asynchronous on `s`, return the launch status) ---------------
+hipError_t launch_fill_zero(hipStream_t s, void *ptr, size_t bytes);
+hipError_t launch_quantize_q4_0(hipStream_t s, const float *w_kn, uint32_t k, uint32_t n, uint8_t *q4);
+hipError_t launch_reorder(hipStream_t s, const uint8_t *q4, uint32_t k, uint32_t n, uint8_t *packed, uint16_t *scales);
+hipError_t launch_quantize_twm(hipStream_t s, const float *w, int w_is_nk, uint32_t k, uint32_t n,
+                               uint8_t *packed, uint16_t *scales);
+hipError_t launch_fuse_one(hipStream_t s, const uint8_t *packed_in, const uint16_t *scales_in, uint32_t groups,
+                           uint32_t ni, uint32_t total_n, uint32_t col_off, uint8_t *packed_out, uint16_t *scales_out);
+hipError_t launch_dequant(hipStream_t s, const uint8_t *packed, const uint16_t *scales, uint32_t k, uint32_t n,
+                          void *out, bool f16_out);
+hipError_t launch_split_qkv(hipStream_t s, const float *qkv, float *q, float *kk, float *v, uint32_t h,
+                            uint32_t kv, uint32_t batch);
+hipError_t launch_split_gate_up(hipStream_t s, const float *gu, float *g, float *u, uint32_t ffn, uint32_t batch);
+hipError_t launch_ref_gemv(hipStream_t s, const float *a, const uint8_t *packed, const uint16_t *scales, float *c,
+                           uint32_t n, uint32_t k, uint32_t splits, uint32_t groups_per_split);
+hipError_t launch_repack(hipStream_t s, const uint8_t *packed, const uint16_t *scales, uint32_t k, uint32_t n,
+                         void *qw, void *sc, uint32_t n_tiles, uint32_t k_chunks);
+hipError_t launch_weight_dequant_f16(hipStream_t s, const WeightView &w, uint16_t *out_kn);
+hipError_t launch_decode(hipStream_t s, const WeightView &w, const void *a, bool a_f32, uint32_t m, const OutSpec &out,
+                         float *ws, unsigned *counters, DecodePlan plan);
+
+}  // namespace twm

@@ -1,0 +1,353 @@
+"""Host-side mirror of the reference's quantized-linear interface, over the C ABI.
+
+Names, argument order and error behaviour follow crates/kernels/src/quantize.rs,
+device.rs, tensor.rs, cuda_graph.rs and ops.rs of the reference so that tests read
+like the reference's own; every function is a thin call into libtwmarlin_hip.so.
+numpy is used only to move host bytes in and out.
+"""
+import ctypes as C
+
+import numpy as np
+
+from . import _lib
+
+BLOCK_SIZE = 32           # quantize.rs `BLOCK_SIZE`
+Q4_0_BLOCK_BYTES = 20     # quantize.rs `Q4_0_BLOCK_BYTES`
+
+
+class DeviceError(RuntimeError):
+    """device.rs:278-292 `DeviceError`; `.code` is the c_api.rs `WarpError` value."""
+
+    def __init__(self, code, message):
+        super().__init__("[%d] %s" % (code, message))
+        self.code = code
+
+
+def _check(rc):
+    if rc != _lib.OK:
+        raise DeviceError(rc, _lib.load().twm_last_error().decode())
+
+
+class WarpDevice:
+    """device.rs `WarpDevice` + cache.rs `KernelCache`: one context, one stream."""
+
+    def __init__(self, ordinal=0):
+        self._l = _lib.load()
+        self.handle = self._l.twm_ctx_create(ordinal)
+        if not self.handle:
+            raise DeviceError(_lib.DEVICE_ERROR, self._l.twm_last_error().decode())
+
+    def close(self):
+        if self.handle:
+            self._l.twm_ctx_destroy(self.handle)
+            self.handle = None
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        self.close()
+
+    def synchronize(self):
+        _check(self._l.twm_ctx_sync(self.handle))
+
+    def summary(self):
+        buf = C.create_string_buffer(256)
+        _check(self._l.twm_ctx_info(self.handle, buf, 256))
+        return buf.value.decode()
+
+    def with_stream(self, hip_stream):
+        _check(self._l.twm_ctx_set_stream(self.handle, hip_stream))
+
+    def set_option(self, key, value):
+        _check(self._l.twm_ctx_set_option(self.handle, key.encode(), int(value)))
+
+    # timing
+    def event(self):
+        ev = self._l.twm_event_create(self.handle)
+        if not ev:
+            raise DeviceError(_lib.DEVICE_ERROR, self._l.twm_last_error().decode())
+        return ev
+
+    def record(self, ev):
+        _check(self._l.twm_event_record(self.handle, ev))
+
+    def elapsed_ms(self, start, stop):
+        ms = C.c_float()
+        _check(self._l.twm_event_elapsed_ms(self.handle, start, stop, C.byref(ms)))
+        return ms.value
+
+    def event_destroy(self, ev):
+        _check(self._l.twm_event_destroy(self.handle, ev))
+
+
+_NP_DTYPES = {"f32": np.float32, "f16": np.uint16, "u8": np.uint8}
+
+
+class GpuTensor:
+    """tensor.rs `GpuTensor<T>`: an owned device allocation with a shape.  f16 data
+    travels as raw uint16 bit patterns on the host side."""
+
+    def __init__(self, device, shape, dtype):
+        self.device = device
+        self.shape = tuple(int(s) for s in (shape if isinstance(shape, (tuple, list)) else (shape,)))
+        self.dtype = dtype
+        self.numel = int(np.prod(self.shape)) if self.shape else 1
+        self.nbytes = self.numel * np.dtype(_NP_DTYPES[dtype]).itemsize
+        self.ptr = device._l.twm_malloc(device.handle, self.nbytes)
+        if not self.ptr:
+            raise DeviceError(_lib.MEMORY_ERROR, device._l.twm_last_error().decode())
+
+    @classmethod
+    def zeros(cls, device, shape, dtype):
+        t = cls(device, shape, dtype)
+        if t.nbytes:
+            t.copy_from_host(np.zeros(t.numel, _NP_DTYPES[dtype]))
+        return t
+
+    @classmethod
+    def from_host(cls, device, array, dtype=None):
+        array = np.ascontiguousarray(array)
+        if dtype is None:
+            dtype = {np.dtype(np.float32): "f32", np.dtype(np.uint16): "f16", np.dtype(np.float16): "f16",
+                     np.dtype(np.uint8): "u8"}[array.dtype]
+        if array.dtype == np.float16:
+            array = array.view(np.uint16)
+        t = cls(device, array.shape, dtype)
+        t.copy_from_host(array)
+        return t
+
+    def copy_from_host(self, array):
+        array = np.ascontiguousarray(array, dtype=_NP_DTYPES[self.dtype])
+        assert array.nbytes == self.nbytes
+        _check(self.device._l.twm_memcpy_h2d(self.device.handle, self.ptr, array.ctypes.data, self.nbytes))
+
+    def to_host(self):
+        out = np.empty(self.shape, _NP_DTYPES[self.dtype])
+        _check(self.device._l.twm_memcpy_d2h(self.device.handle, out.ctypes.data, self.ptr, self.nbytes))
+        return out
+
+    def free(self):
+        if self.ptr:
+            self.device._l.twm_free(self.device.handle, self.ptr)
+            self.ptr = None
+
+
+def _require_k(k):
+    # the reference asserts (quantize.rs:1311); here the library reports SHAPE_ERROR
+    if k % BLOCK_SIZE != 0:
+        raise DeviceError(_lib.SHAPE_ERROR, "K (%d) must be divisible by %d" % (k, BLOCK_SIZE))
+
+
+def pick_splits_reference(k, n):
+    """quantize.rs:1314-1325 -> (n_blocks, splits, k_blocks_per_split)."""
+    nb, sp, kb = C.c_uint32(), C.c_uint32(), C.c_uint32()
+    _lib.load().twm_pick_splits_reference(k, n, C.byref(nb), C.byref(sp), C.byref(kb))
+    return nb.value, sp.value, kb.value
+
+
+def pick_splits(k, n, m=1):
+    return _lib.load().twm_pick_splits(k, n, m)
+
+
+def quantize_weights_q4_0(device, weights, k, n):
+    """quantize.rs:414 — weights: GpuTensor f32 [K,N] -> GpuTensor u8 (Q4_0 column-major blocks)."""
+    _require_k(k)
+    out = GpuTensor(device, ((k // BLOCK_SIZE) * n * Q4_0_BLOCK_BYTES,), "u8")
+    _check(device._l.twm_quantize_weights_q4_0(device.handle, weights.ptr, k, n, out.ptr))
+    return out
+
+
+def reorder_to_tw_marlin(device, col_major_q4, k, n):
+    """quantize.rs:912 -> (packed GpuTensor u8, scales GpuTensor f16)."""
+    _require_k(k)
+    g = k // BLOCK_SIZE
+    packed = GpuTensor(device, (g * n * 16,), "u8")
+    scales = GpuTensor(device, (g * n,), "f16")
+    _check(device._l.twm_reorder_to_tw_marlin(device.handle, col_major_q4.ptr, k, n, packed.ptr, scales.ptr))
+    return packed, scales
+
+
+def quantize_f32_to_tw_marlin(device, weights, k, n, weights_are_nk=False):
+    """quantize.rs:1171 (weights [K,N]); weights_are_nk=True gives cpu_quantize_tw_marlin
+    (gemma_moe_q4.rs:218) on a [N,K] matrix."""
+    _require_k(k)
+    g = k // BLOCK_SIZE
+    packed = GpuTensor(device, (g * n * 16,), "u8")
+    scales = GpuTensor(device, (g * n,), "f16")
+    _check(device._l.twm_quantize_f32_to_tw_marlin(device.handle, weights.ptr, 1 if weights_are_nk else 0, k, n,
+                                                   packed.ptr, scales.ptr))
+    return packed, scales
+
+
+def fuse_tw_marlin_n(device, matrices, k, ns):
+    """quantize.rs:1018 — matrices: [(packed, scales), ...] GpuTensors; ns: their N."""
+    _require_k(k)
+    cnt = len(matrices)
+    total = int(sum(ns))
+    g = k // BLOCK_SIZE
+    packed = GpuTensor(device, (g * total * 16,), "u8")
+    scales = GpuTensor(device, (g * total,), "f16")
+    pp = (C.c_void_p * cnt)(*[m[0].ptr for m in matrices])
+    sp = (C.c_void_p * cnt)(*[m[1].ptr for m in matrices])
+    nsa = (C.c_uint32 * cnt)(*[int(x) for x in ns])
+    _check(device._l.twm_fuse_tw_marlin_n(device.handle, pp, sp, k, nsa, cnt, packed.ptr, scales.ptr))
+    return packed, scales
+
+
+def dequant_to_f16(device, packed, scales, k, n):
+    """quantize.rs:580 `dequant_q4_to_f16` for TW-Marlin arrays -> GpuTensor f16 [K,N]."""
+    _require_k(k)
+    out = GpuTensor(device, (k, n), "f16")
+    _check(device._l.twm_dequant_to_f16(device.handle, packed.ptr, scales.ptr, k, n, out.ptr))
+    return out
+
+
+def dequant_to_f32(device, packed, scales, k, n):
+    _require_k(k)
+    out = GpuTensor(device, (k, n), "f32")
+    _check(device._l.twm_dequant_to_f32(device.handle, packed.ptr, scales.ptr, k, n, out.ptr))
+    return out
+
+
+def split_qkv(device, qkv, q, k, v, h, kv_dim, batch):
+    """ops.rs:2300"""
+    _check(device._l.twm_split_qkv(device.handle, qkv.ptr, q.ptr, k.ptr, v.ptr, h, kv_dim, batch))
+
+
+def split_gate_up(device, gate_up, gate, up, ffn_dim, batch):
+    """ops.rs:2324"""
+    _check(device._l.twm_split_gate_up(device.handle, gate_up.ptr, gate.ptr, up.ptr, ffn_dim, batch))
+
+
+def gemm_tw_marlin_m1(device, a, packed, scales, c, n, k):
+    """quantize.rs:1301 — a: f32 [1,K]; packed/scales: reference TW-Marlin arrays; c: f32 [1,N]."""
+    _check(device._l.twm_gemm_tw_marlin_m1(device.handle, a.ptr, packed.ptr, scales.ptr, c.ptr, n, k))
+
+
+def gemm_tw_marlin_m1_from_buffer(device, a, packed_buf, packed_offset, scales_buf, scales_offset, c, n, k):
+    """quantize.rs:1731"""
+    _check(device._l.twm_gemm_tw_marlin_m1_from_buffer(device.handle, a.ptr, packed_buf.ptr, packed_offset,
+                                                       scales_buf.ptr, scales_offset, c.ptr, n, k))
+
+
+class MarlinWeight:
+    """One projection repacked for gfx950 (twm_weight)."""
+
+    def __init__(self, device, handle, k, n):
+        self.device, self.handle, self.k, self.n = device, handle, k, n
+
+    @classmethod
+    def upload(cls, device, packed_host, scales_host, k, n):
+        packed_host = np.ascontiguousarray(packed_host, np.uint8)
+        scales_host = np.ascontiguousarray(scales_host).view(np.uint16)
+        h = device._l.twm_weight_upload(device.handle, packed_host.ctypes.data, scales_host.ctypes.data, k, n)
+        if not h:
+            raise DeviceError(_lib.SHAPE_ERROR if k % 32 else _lib.DEVICE_ERROR, device._l.twm_last_error().decode())
+        return cls(device, h, k, n)
+
+    @classmethod
+    def from_device(cls, device, packed, scales, k, n):
+        h = device._l.twm_weight_from_device(device.handle, packed.ptr, scales.ptr, k, n)
+        if not h:
+            raise DeviceError(_lib.SHAPE_ERROR if k % 32 else _lib.DEVICE_ERROR, device._l.twm_last_error().decode())
+        return cls(device, h, k, n)
+
+    @property
+    def nbytes(self):
+        return self.device._l.twm_weight_bytes(self.handle)
+
+    def dequant_f16(self):
+        out = GpuTensor(self.device, (self.k, self.n), "f16")
+        _check(self.device._l.twm_weight_dequant_f16(self.device.handle, self.handle, out.ptr))
+        return out
+
+    def free(self):
+        if self.handle:
+            self.device._l.twm_weight_destroy(self.handle)
+            self.handle = None
+
+
+def gemm(device, weight, a, m, c, splits=0):
+    """C[M,N] f32 = A[M,K] (f16 or f32) x dequant(weight). M=1 is gemm_tw_marlin_m1."""
+    dt = _lib.F16 if a.dtype == "f16" else _lib.F32
+    _check(device._l.twm_gemm(device.handle, weight.handle, a.ptr, dt, m, c.ptr, splits))
+
+
+def gemm_split(device, weight, a, m, outs, ns, splits=0):
+    """Fused projection whose column ranges land in separate buffers (gemm + split_qkv/split_gate_up)."""
+    cnt = len(outs)
+    dt = _lib.F16 if a.dtype == "f16" else _lib.F32
+    op = (C.c_void_p * cnt)(*[o.ptr for o in outs])
+    nsa = (C.c_uint32 * cnt)(*[int(x) for x in ns])
+    _check(device._l.twm_gemm_split(device.handle, weight.handle, a.ptr, dt, m, op, nsa, cnt, splits))
+
+
+class TWMarlinWeights:
+    """quantize.rs:1067-1166 `TWMarlinWeights`: the seven projections of one layer as
+    (packed, scales) device pairs, plus the fused QKV / gate+up made by fuse_projections."""
+
+    NAMES = ("wq", "wk", "wv", "wo", "wg", "wu", "wd")
+
+    def __init__(self, device, hidden_size, kv_dim, ffn_dim, pairs):
+        self.device, self.h, self.kv, self.ffn = device, hidden_size, kv_dim, ffn_dim
+        for name in self.NAMES:
+            p, s = pairs[name]
+            setattr(self, name + "_packed", p)
+            setattr(self, name + "_scales", s)
+        self.wqkv_packed = self.wqkv_scales = self.wgu_packed = self.wgu_scales = None
+        self.repacked = {}
+
+    def fuse_projections(self):
+        """quantize.rs:1138"""
+        d, h, kv, ffn = self.device, self.h, self.kv, self.ffn
+        self.wqkv_packed, self.wqkv_scales = fuse_tw_marlin_n(
+            d, [(self.wq_packed, self.wq_scales), (self.wk_packed, self.wk_scales), (self.wv_packed, self.wv_scales)],
+            h, [h, kv, kv])
+        self.wgu_packed, self.wgu_scales = fuse_tw_marlin_n(
+            d, [(self.wg_packed, self.wg_scales), (self.wu_packed, self.wu_scales)], h, [ffn, ffn])
+
+    def repack_for_decode(self):
+        """Builds the gfx950 tile-order weights for the four GEMVs of the fused decode path."""
+        d, h, kv, ffn = self.device, self.h, self.kv, self.ffn
+        if self.wqkv_packed is None:
+            self.fuse_projections()
+        self.repacked = {
+            "qkv": MarlinWeight.from_device(d, self.wqkv_packed, self.wqkv_scales, h, h + 2 * kv),
+            "o": MarlinWeight.from_device(d, self.wo_packed, self.wo_scales, h, h),
+            "gate_up": MarlinWeight.from_device(d, self.wgu_packed, self.wgu_scales, h, 2 * ffn),
+            "down": MarlinWeight.from_device(d, self.wd_packed, self.wd_scales, ffn, h),
+        }
+        return self.repacked
+
+
+class GraphCapture:
+    """cuda_graph.rs:72-118"""
+
+    def __init__(self, device, handle):
+        self.device, self.handle = device, handle
+
+    @classmethod
+    def record_with_device(cls, device, fn):
+        _check(device._l.twm_graph_begin(device.handle))
+        err = None
+        try:
+            fn()
+        except Exception as e:  # end the capture before reporting, as the reference does (cuda_graph.rs:101-108)
+            err = e
+        h = device._l.twm_graph_end(device.handle)
+        if err is not None:
+            if h:
+                device._l.twm_graph_destroy(h)
+            raise err
+        if not h:
+            raise DeviceError(_lib.DEVICE_ERROR, device._l.twm_last_error().decode())
+        return cls(device, h)
+
+    def replay(self):
+        _check(self.device._l.twm_graph_launch(self.device.handle, self.handle))
+
+    def destroy(self):
+        if self.handle:
+            self.device._l.twm_graph_destroy(self.handle)
+            self.handle = None

@@ -1,0 +1,395 @@
+"""GPU parity tests: the HIP path, called through the C ABI, against the CPU oracle and
+the committed golden fixtures.
+
+Bars: bit-exact for byte/integer work (quantizer output, reorder, fuse, repack, Q4 unpack
+to FP16, splits); max relative error <= 1e-2 for GEMV/GEMM outputs (f32 accumulation), where
+    rel = max_i |c_i - t_i| / max(|t_i|, 1e-3 * max_j |t_j|)
+and t is the oracle's f64 dequant-then-matmul.  The floor keeps near-cancelling outputs from
+turning an absolute error of a few ulps into a huge ratio.  Observed errors are ~1e-6, so the
+tests also assert a much tighter 2e-4.
+"""
+import os
+
+import numpy as np
+import pytest
+
+import tensorwarp_amd as T
+from oracle import twm_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+GOLD = os.path.join(os.path.dirname(__file__), "golden")
+TOL = 1e-2         # the stated tolerance
+TIGHT = 2e-4       # what f32 accumulation actually delivers
+
+
+@pytest.fixture(scope="module")
+def dev():
+    d = T.WarpDevice(0)
+    print("device:", d.summary(), flush=True)
+    yield d
+    d.close()
+
+
+def rel_err(c, truth):
+    truth = np.asarray(truth, np.float64)
+    denom = np.maximum(np.abs(truth), 1e-3 * np.abs(truth).max() + 1e-30)
+    return float((np.abs(np.asarray(c, np.float64) - truth) / denom).max())
+
+
+def synth(k, n, m, seed):
+    packed = O.synth_packed(k, n, seed * 3 + 1)
+    scales = O.synth_scales(k, n, seed * 3 + 2)
+    a16 = O.synth_act_f16(m, k, seed * 3 + 3)
+    return packed, scales, a16
+
+
+def f16_as_f32(bits):
+    return bits.view(np.float16).astype(np.float32)
+
+
+# ---------------------------------------------------------------- format operations
+
+def test_quantize_reorder_fuse_bit_exact(dev):
+    k, n = 256, 200
+    w_kn = O.synth_normal_f32(k * n, 41).reshape(k, n) * np.float32(0.05)
+    w_kn[32:64, 7] = 0.0                       # an all-zero group
+    w_kn[0, 3] = 0.35                          # make some exact .5 ties likely irrelevant but harmless
+    wd = T.GpuTensor.from_host(dev, w_kn)
+    q4 = T.quantize_weights_q4_0(dev, wd, k, n)
+    assert np.array_equal(q4.to_host(), O.quantize_weights_q4_0_kn(w_kn, k, n))
+    packed, scales = T.reorder_to_tw_marlin(dev, q4, k, n)
+    op, os_ = O.reorder_to_tw_marlin(O.quantize_weights_q4_0_kn(w_kn, k, n), k, n)
+    assert np.array_equal(packed.to_host(), op) and np.array_equal(scales.to_host(), os_)
+    # one-pass quantizer from [K,N] and from [N,K]
+    p2, s2 = T.quantize_f32_to_tw_marlin(dev, wd, k, n)
+    assert np.array_equal(p2.to_host(), op) and np.array_equal(s2.to_host(), os_)
+    wnk = T.GpuTensor.from_host(dev, np.ascontiguousarray(w_kn.T))
+    p3, s3 = T.quantize_f32_to_tw_marlin(dev, wnk, k, n, weights_are_nk=True)
+    rp, rs = O.quantize_tw_marlin_nk(np.ascontiguousarray(w_kn.T), k, n)
+    assert np.array_equal(p3.to_host(), rp) and np.array_equal(s3.to_host(), rs)
+
+
+def test_quantizer_ties_round_half_away(dev):
+    v = np.zeros((1, 32), np.float32)
+    v[0, :8] = [7.0, -7.0, 0.5, -0.5, 1.5, -1.5, 2.5, -2.5]
+    p, s = T.quantize_f32_to_tw_marlin(dev, T.GpuTensor.from_host(dev, v), 32, 1, weights_are_nk=True)
+    rp, rs = O.quantize_tw_marlin_nk(v, 32, 1)
+    assert np.array_equal(p.to_host(), rp) and np.array_equal(s.to_host(), rs)
+
+
+def test_lcg_fixture_quantizes_to_golden_bytes(dev):
+    d = np.load(os.path.join(GOLD, "lcg_k128_n64_m4.npz"))
+    k, n = 128, 64
+    p, s = T.quantize_f32_to_tw_marlin(dev, T.GpuTensor.from_host(dev, d["w_kn"]), k, n)
+    assert np.array_equal(p.to_host(), d["packed"]) and np.array_equal(s.to_host(), d["scales"])
+
+
+def test_fuse_matches_oracle(dev):
+    k, ns = 96, [48, 16, 16]
+    mats_h = [(O.synth_packed(k, ni, 50 + i), O.synth_scales(k, ni, 60 + i)) for i, ni in enumerate(ns)]
+    mats_d = [(T.GpuTensor.from_host(dev, p), T.GpuTensor.from_host(dev, s, "f16")) for p, s in mats_h]
+    fp, fs = T.fuse_tw_marlin_n(dev, mats_d, k, ns)
+    op, os_ = O.fuse_tw_marlin_n(mats_h, k, ns)
+    assert np.array_equal(fp.to_host(), op) and np.array_equal(fs.to_host(), os_)
+
+
+def test_split_kernels(dev):
+    h, kv, batch = 96, 32, 3
+    x = O.synth_normal_f32(batch * (h + 2 * kv), 70)
+    q, kk, v = (T.GpuTensor.zeros(dev, (batch * h,), "f32"), T.GpuTensor.zeros(dev, (batch * kv,), "f32"),
+                T.GpuTensor.zeros(dev, (batch * kv,), "f32"))
+    T.split_qkv(dev, T.GpuTensor.from_host(dev, x), q, kk, v, h, kv, batch)
+    oq, ok_, ov = O.split_qkv(x, h, kv, batch)
+    assert np.array_equal(q.to_host(), oq) and np.array_equal(kk.to_host(), ok_) and np.array_equal(v.to_host(), ov)
+    ffn = 80
+    y = O.synth_normal_f32(batch * 2 * ffn, 71)
+    g, u = T.GpuTensor.zeros(dev, (batch * ffn,), "f32"), T.GpuTensor.zeros(dev, (batch * ffn,), "f32")
+    T.split_gate_up(dev, T.GpuTensor.from_host(dev, y), g, u, ffn, batch)
+    og, ou = O.split_gate_up(y, ffn, batch)
+    assert np.array_equal(g.to_host(), og) and np.array_equal(u.to_host(), ou)
+
+
+# ---------------------------------------------------------------- Q4 unpack, bit exact
+
+@pytest.mark.parametrize("name", ["lcg_k64_n8_m1", "lcg_k128_n64_m4", "synth_k128_n64_m1",
+                                  "synth_k256_n80_m5", "synth_k160_n33_m17"])
+def test_dequant_matches_golden_bits(dev, name):
+    d = np.load(os.path.join(GOLD, name + ".npz"))
+    k, n = int(d["k"]), int(d["n"])
+    p = T.GpuTensor.from_host(dev, d["packed"])
+    s = T.GpuTensor.from_host(dev, d["scales"], "f16")
+    assert np.array_equal(T.dequant_to_f16(dev, p, s, k, n).to_host(), d["dequant_f16"])
+    assert np.array_equal(T.dequant_to_f32(dev, p, s, k, n).to_host(), d["dequant_f32"])
+    w = T.MarlinWeight.from_device(dev, p, s, k, n)            # and straight from the repacked form
+    assert np.array_equal(w.dequant_f16().to_host(), d["dequant_f16"])
+    w.free()
+
+
+def test_dequant_f16_exhaustive_scales_times_nibbles(dev):
+    # all 65536 scale bit patterns x 16 nibble values; NaN payloads compare as NaN
+    n = 65536
+    s_bits = np.arange(n, dtype=np.uint16)
+    packed = np.zeros((1, n, 16), np.uint8)
+    for i in range(16):
+        packed[0, :, i // 2] |= np.uint8(i << (4 * (i & 1)))
+    want = O.dequant_f16(packed.reshape(-1), s_bits, 32, n)
+    p = T.GpuTensor.from_host(dev, packed.reshape(-1))
+    s = T.GpuTensor.from_host(dev, s_bits, "f16")
+    for got in (T.dequant_to_f16(dev, p, s, 32, n).to_host(),
+                T.MarlinWeight.from_device(dev, p, s, 32, n).dequant_f16().to_host()):
+        wn = np.isnan(want.view(np.float16))
+        assert np.array_equal(got[~wn], want[~wn])
+        assert np.all(np.isnan(got.view(np.float16)[wn]))
+
+
+def test_repack_is_lossless_at_7b_shape(dev):
+    k, n = 3584, 4608
+    packed, scales, _ = synth(k, n, 1, 5)
+    w = T.MarlinWeight.upload(dev, packed, scales, k, n)
+    assert np.array_equal(w.dequant_f16().to_host(), O.dequant_f16(packed, scales, k, n))
+    w.free()
+
+
+# ---------------------------------------------------------------- GEMV on the reference layout
+
+@pytest.mark.parametrize("k,n", [(64, 8), (128, 64), (896, 1152), (4096, 4096), (4864, 896), (3584, 300)])
+def test_gemm_tw_marlin_m1_reference_layout(dev, k, n):
+    packed, scales, a16 = synth(k, n, 1, k + n)
+    a = f16_as_f32(a16)
+    c = T.GpuTensor.zeros(dev, (n,), "f32")
+    T.gemm_tw_marlin_m1(dev, T.GpuTensor.from_host(dev, a), T.GpuTensor.from_host(dev, packed),
+                        T.GpuTensor.from_host(dev, scales, "f16"), c, n, k)
+    got = c.to_host()
+    truth = O.gemm_f64(a, packed, scales, 1, k, n)[0]
+    assert rel_err(got, truth) < TIGHT
+    _, splits, _ = T.pick_splits_reference(k, n)
+    if splits == 1:                                      # same order as the reference kernel: bitwise
+        assert np.array_equal(got, O.gemv_ref_order(a, packed, scales, 1, k, n, 1)[0])
+
+
+def test_gemm_tw_marlin_m1_from_buffer_and_errors(dev):
+    k, n = 128, 64
+    packed, scales, a16 = synth(k, n, 1, 9)
+    a = f16_as_f32(a16)
+    slab_p = np.concatenate([np.zeros(4096, np.uint8), packed])
+    slab_s = np.concatenate([np.zeros(100, np.uint16), scales])
+    c = T.GpuTensor.zeros(dev, (n,), "f32")
+    T.gemm_tw_marlin_m1_from_buffer(dev, T.GpuTensor.from_host(dev, a), T.GpuTensor.from_host(dev, slab_p), 4096,
+                                    T.GpuTensor.from_host(dev, slab_s, "f16"), 100, c, n, k)
+    assert np.array_equal(c.to_host(), O.gemv_ref_order(a, packed, scales, 1, k, n, 1)[0])
+    with pytest.raises(T.DeviceError) as e:              # the reference asserts k % 32 == 0 (quantize.rs:1311)
+        T.gemm_tw_marlin_m1(dev, c, c, c, c, n, 100)
+    assert e.value.code == T._lib.SHAPE_ERROR
+    with pytest.raises(T.DeviceError):
+        T.MarlinWeight.upload(dev, packed, scales, 100, n)
+
+
+# ---------------------------------------------------------------- the repacked fast path
+
+def run_gemm(dev, w, a16, m, n, splits=0, a_f32=False):
+    a_dev = T.GpuTensor.from_host(dev, f16_as_f32(a16)) if a_f32 else T.GpuTensor.from_host(dev, a16, "f16")
+    c = T.GpuTensor.from_host(dev, np.full((m, n), np.nan, np.float32))   # NaN canary: every output must be written
+    T.gemm(dev, w, a_dev, m, c, splits)
+    out = c.to_host()
+    a_dev.free()
+    c.free()
+    return out
+
+
+@pytest.mark.parametrize("name", ["lcg_k64_n8_m1", "lcg_k128_n64_m4", "synth_k128_n64_m1",
+                                  "synth_k256_n80_m5", "synth_k160_n33_m17"])
+def test_gemm_matches_golden(dev, name):
+    d = np.load(os.path.join(GOLD, name + ".npz"))
+    k, n, m = int(d["k"]), int(d["n"]), int(d["m"])
+    w = T.MarlinWeight.upload(dev, d["packed"], d["scales"], k, n)
+    for a_f32 in (False, True):
+        got = run_gemm(dev, w, d["a_f16"], m, n, a_f32=a_f32)
+        assert rel_err(got, d["c_f64"]) < TIGHT, (name, a_f32)
+    w.free()
+
+
+def test_gemv_closed_forms(dev):
+    k, n = 256, 96
+    scales = O.synth_scales(k, n, 77)
+    a16 = O.synth_act_f16(1, k, 78)
+    w0 = T.MarlinWeight.upload(dev, np.full((k // 32) * n * 16, 0x88, np.uint8), scales, k, n)
+    assert np.all(run_gemm(dev, w0, a16, 1, n) == 0)                 # all weights exactly zero
+    one = np.full((k // 32) * n, np.float16(1.0).view(np.uint16), np.uint16)
+    w1 = T.MarlinWeight.upload(dev, np.full((k // 32) * n * 16, 0x99, np.uint8), one, k, n)
+    assert np.allclose(run_gemm(dev, w1, a16, 1, n), f16_as_f32(a16).astype(np.float64).sum(), atol=1e-3)
+    packed = O.synth_packed(k, n, 79)
+    w2 = T.MarlinWeight.upload(dev, packed, scales, k, n)
+    deq = O.dequant_f32(packed, scales, k, n)
+    for kk in (0, 1, 7, 8, 31, 32, 100, 255):                        # one-hot A picks a dequantised row, exactly
+        e = np.zeros((1, k), np.float16)
+        e[0, kk] = 1.0
+        assert np.array_equal(run_gemm(dev, w2, e.view(np.uint16), 1, n)[0], deq[kk]), kk
+    for w in (w0, w1, w2):
+        w.free()
+
+
+SHAPES_05B = [(896, 1152), (896, 896), (896, 9728), (4864, 896)]
+SHAPES_7B = [(3584, 4608), (3584, 3584), (3584, 37888), (18944, 3584)]
+
+
+@pytest.mark.parametrize("k,n", [(4096, 4096)] + SHAPES_05B + SHAPES_7B)
+def test_gemv_m1_benchmark_shapes(dev, k, n):
+    packed, scales, a16 = synth(k, n, 1, k * 7 + n)
+    w = T.MarlinWeight.upload(dev, packed, scales, k, n)
+    truth = O.gemm_f64(f16_as_f32(a16), packed, scales, 1, k, n)
+    got = run_gemm(dev, w, a16, 1, n)
+    err = rel_err(got, truth)
+    print("M=1 %5d->%5d splits=%d rel_err=%.2e" % (k, n, T.pick_splits(k, n, 1), err), flush=True)
+    assert err < TIGHT and err < TOL
+    w.free()
+
+
+@pytest.mark.parametrize("m", [2, 3, 4, 5, 8, 15, 16, 17, 31, 32])
+def test_batched_decode_small_k(dev, m):
+    k, n = 896, 1152
+    packed, scales, a16 = synth(k, n, m, 1000 + m)
+    w = T.MarlinWeight.upload(dev, packed, scales, k, n)
+    truth = O.gemm_f64(f16_as_f32(a16), packed, scales, m, k, n)
+    for splits in (0, 1, 3):
+        assert rel_err(run_gemm(dev, w, a16, m, n, splits), truth) < TIGHT, splits
+    w.free()
+
+
+@pytest.mark.parametrize("m,k,n", [(4, 3584, 4608), (8, 3584, 37888), (16, 18944, 3584), (32, 3584, 4608)])
+def test_batched_decode_7b_shapes(dev, m, k, n):
+    packed, scales, a16 = synth(k, n, m, 2000 + m)
+    w = T.MarlinWeight.upload(dev, packed, scales, k, n)
+    truth = O.gemm_f64(f16_as_f32(a16), packed, scales, m, k, n)
+    got = run_gemm(dev, w, a16, m, n)
+    assert rel_err(got, truth) < TIGHT
+    # every row of the batch equals the same row run alone at the same split factor
+    sp = T.pick_splits(k, n, m)
+    alone = run_gemm(dev, w, a16[m - 1:m], 1, n, sp)
+    assert rel_err(alone[0], got[m - 1]) < 1e-5
+    w.free()
+
+
+def test_split_k_choice_does_not_change_the_result(dev):
+    k, n = 4096, 4096
+    packed, scales, a16 = synth(k, n, 1, 31)
+    w = T.MarlinWeight.upload(dev, packed, scales, k, n)
+    truth = O.gemm_f64(f16_as_f32(a16), packed, scales, 1, k, n)
+    base = run_gemm(dev, w, a16, 1, n, 1)
+    for nt in (1, 2, 4):
+        dev.set_option("nt", nt)
+        for splits in (1, 2, 5, 8, 32):
+            got = run_gemm(dev, w, a16, 1, n, splits)
+            assert rel_err(got, truth) < TIGHT, (nt, splits)
+            assert rel_err(got, base) < 1e-4
+        # same launch twice is bitwise repeatable (ordered reduction, no float atomics)
+        assert np.array_equal(run_gemm(dev, w, a16, 1, n, 8), run_gemm(dev, w, a16, 1, n, 8))
+    dev.set_option("nt", 0)
+    w.free()
+
+
+def test_m_larger_than_32_is_tiled(dev):
+    m, k, n = 70, 256, 128
+    packed, scales, a16 = synth(k, n, m, 33)
+    w = T.MarlinWeight.upload(dev, packed, scales, k, n)
+    truth = O.gemm_f64(f16_as_f32(a16), packed, scales, m, k, n)
+    assert rel_err(run_gemm(dev, w, a16, m, n), truth) < TIGHT
+    w.free()
+
+
+def test_empty_inputs(dev):
+    w = T.MarlinWeight.upload(dev, np.zeros(0, np.uint8), np.zeros(0, np.uint16), 64, 0)
+    c = T.GpuTensor.zeros(dev, (4,), "f32")
+    a = T.GpuTensor.zeros(dev, (64,), "f16")
+    T.gemm(dev, w, a, 1, c)          # N == 0: nothing to do
+    T.gemm(dev, w, a, 0, c)          # M == 0
+    w.free()
+    w0 = T.MarlinWeight.upload(dev, np.zeros(0, np.uint8), np.zeros(0, np.uint16), 0, 8)
+    c8 = T.GpuTensor.from_host(dev, np.ones(8, np.float32))
+    T.gemm(dev, w0, a, 1, c8)        # K == 0: the empty sum
+    assert np.all(c8.to_host() == 0)
+    w0.free()
+
+
+# ---------------------------------------------------------------- fused projections
+
+def test_fused_qkv_and_gate_up_equal_separate_projections(dev):
+    # fused-vs-unfused equality, the check the reference makes for F32 weights only
+    # (transformer.rs:2230-2287), here on TW-Marlin weights and bit for bit
+    h, kv, ffn = 896, 128, 4864
+    names = {"wq": (h, h), "wk": (h, kv), "wv": (h, kv), "wo": (h, h), "wg": (h, ffn), "wu": (h, ffn), "wd": (ffn, h)}
+    host, pairs = {}, {}
+    for i, (nm, (k, n)) in enumerate(names.items()):
+        host[nm] = (O.synth_packed(k, n, 300 + i), O.synth_scales(k, n, 400 + i))
+        pairs[nm] = (T.GpuTensor.from_host(dev, host[nm][0]), T.GpuTensor.from_host(dev, host[nm][1], "f16"))
+    layer = T.TWMarlinWeights(dev, h, kv, ffn, pairs)
+    layer.fuse_projections()
+    fp, fs = O.fuse_tw_marlin_n([host["wq"], host["wk"], host["wv"]], h, [h, kv, kv])
+    assert np.array_equal(layer.wqkv_packed.to_host(), fp) and np.array_equal(layer.wqkv_scales.to_host(), fs)
+    rp = layer.repack_for_decode()
+    a16 = O.synth_act_f16(1, h, 500)
+    a_dev = T.GpuTensor.from_host(dev, a16, "f16")
+    # (1) fused GEMV + split kernels, the reference's sequence (generate.rs:2152-2155)
+    qkv = T.GpuTensor.zeros(dev, (h + 2 * kv,), "f32")
+    T.gemm(dev, rp["qkv"], a_dev, 1, qkv, 1)
+    q, kk, v = (T.GpuTensor.zeros(dev, (h,), "f32"), T.GpuTensor.zeros(dev, (kv,), "f32"),
+                T.GpuTensor.zeros(dev, (kv,), "f32"))
+    T.split_qkv(dev, qkv, q, kk, v, h, kv, 1)
+    # (2) the split folded into the GEMV's store
+    q2, k2, v2 = (T.GpuTensor.zeros(dev, (h,), "f32"), T.GpuTensor.zeros(dev, (kv,), "f32"),
+                  T.GpuTensor.zeros(dev, (kv,), "f32"))
+    T.gemm_split(dev, rp["qkv"], a_dev, 1, [q2, k2, v2], [h, kv, kv], 1)
+    # (3) three separate projections
+    for nm, fused, direct in (("wq", q, q2), ("wk", kk, k2), ("wv", v, v2)):
+        k_, n_ = names[nm]
+        w = T.MarlinWeight.from_device(dev, pairs[nm][0], pairs[nm][1], k_, n_)
+        sep = T.GpuTensor.zeros(dev, (n_,), "f32")
+        T.gemm(dev, w, a_dev, 1, sep, 1)
+        assert np.array_equal(sep.to_host(), fused.to_host()), nm
+        assert np.array_equal(sep.to_host(), direct.to_host()), nm
+        truth = O.gemm_f64(f16_as_f32(a16), host[nm][0], host[nm][1], 1, k_, n_)[0]
+        assert rel_err(sep.to_host(), truth) < TIGHT
+    # gate+up with M = 3 and automatic split-K
+    a3 = O.synth_act_f16(3, h, 501)
+    a3d = T.GpuTensor.from_host(dev, a3, "f16")
+    g, u = T.GpuTensor.zeros(dev, (3, ffn), "f32"), T.GpuTensor.zeros(dev, (3, ffn), "f32")
+    T.gemm_split(dev, rp["gate_up"], a3d, 3, [g, u], [ffn, ffn])
+    tg = O.gemm_f64(f16_as_f32(a3), host["wg"][0], host["wg"][1], 3, h, ffn)
+    tu = O.gemm_f64(f16_as_f32(a3), host["wu"][0], host["wu"][1], 3, h, ffn)
+    assert rel_err(g.to_host(), tg) < TIGHT and rel_err(u.to_host(), tu) < TIGHT
+    with pytest.raises(T.DeviceError):
+        T.gemm_split(dev, rp["gate_up"], a3d, 3, [g, u], [ffn, ffn - 1])
+
+
+# ---------------------------------------------------------------- graph capture / replay
+
+def test_layer_graph_replays_match_eager(dev):
+    # the four projections of a Qwen-0.5B-shaped layer as one graph; replayed several times
+    # with eager work and synchronisations in between, every replay checked against eager
+    shapes = {"qkv": (896, 1152), "o": (896, 896), "gate_up": (896, 9728), "down": (4864, 896)}
+    ws, acts, outs, eager = {}, {}, {}, {}
+    for i, (nm, (k, n)) in enumerate(shapes.items()):
+        p, s, a16 = synth(k, n, 1, 600 + i)
+        ws[nm] = T.MarlinWeight.upload(dev, p, s, k, n)
+        acts[nm] = T.GpuTensor.from_host(dev, a16, "f16")
+        outs[nm] = T.GpuTensor.zeros(dev, (n,), "f32")
+        T.gemm(dev, ws[nm], acts[nm], 1, outs[nm])
+        eager[nm] = outs[nm].to_host()
+        truth = O.gemm_f64(f16_as_f32(a16), p, s, 1, k, n)[0]
+        assert rel_err(eager[nm], truth) < TIGHT
+
+    def body():
+        for nm in shapes:
+            T.gemm(dev, ws[nm], acts[nm], 1, outs[nm])
+
+    graph = T.GraphCapture.record_with_device(dev, body)
+    for rep in range(4):
+        for nm, (k, n) in shapes.items():
+            outs[nm].copy_from_host(np.full(n, np.nan, np.float32))
+        graph.replay()
+        dev.synchronize()
+        for nm in shapes:
+            assert np.array_equal(outs[nm].to_host(), eager[nm]), (rep, nm)
+        T.gemm(dev, ws["down"], acts["down"], 1, outs["down"], 7)      # eager work between replays
+        dev.synchronize()
+    graph.destroy()
