@@ -26,6 +26,18 @@ __device__ __forceinline__ float f16_bits_to_f32(uint16_t h)
     return (float)x.f;  // v_cvt_f32_f16: exact, subnormals kept
 }
 
+// scale * q for the Q4 unpack.  The value is pinned in a register between the convert and the
+// multiply: left alone, the compiler folds both into v_fma_mix*(s, q, +0), and x*y + (+0) turns
+// the product -0.0 (zero scale, negative q) into +0.0, which is not the reference's bit pattern.
+__device__ __forceinline__ float scale_times_q(uint16_t scale_bits, int q)
+{
+    float s = f16_bits_to_f32(scale_bits);
+    asm volatile("" : "+v"(s));
+    float w = s * (float)q;
+    asm volatile("" : "+v"(w));
+    return w;
+}
+
 __device__ __forceinline__ uint16_t f32_to_f16_bits(float f)
 {
     union { uint16_t u; _Float16 h; } x;
@@ -211,10 +223,9 @@ __global__ __launch_bounds__(256) void k_dequant(const uint8_t *__restrict__ pac
     if (idx >= (size_t)k * n) return;
     uint32_t row = (uint32_t)(idx / n), col = (uint32_t)(idx % n);
     uint32_t g = row / 32, e = row % 32;
-    float s = f16_bits_to_f32(scales[(size_t)g * n + col]);
     uint8_t byte = packed[((size_t)g * n + col) * 16 + e / 2];
     int q = (e & 1) ? (byte >> 4) : (byte & 0xF);
-    float w = s * (float)(q - 8);  // exact in f32: 11-bit x 4-bit significands
+    float w = scale_times_q(scales[(size_t)g * n + col], q - 8);  // exact in f32: 11-bit x 4-bit significands
     if (F16OUT) ((uint16_t *)out)[idx] = f32_to_f16_bits(w);
     else ((float *)out)[idx] = w;
 }
@@ -408,8 +419,7 @@ __global__ __launch_bounds__(256) void k_weight_dequant_f16(const uint32_t *__re
     uint32_t w = qw[(tile * 64 + kb * 16 + c) * 4 + i];
     int p = (j & 1) ? 4 + (j >> 1) : (j >> 1);
     int q = (int)((w >> (4 * p)) & 0xFu) - 8;
-    float s = f16_bits_to_f32(sc[(tile * 16 + c) * 4 + i]);
-    out[idx] = f32_to_f16_bits(s * (float)q);
+    out[idx] = f32_to_f16_bits(scale_times_q(sc[(tile * 16 + c) * 4 + i], q));
 }
 
 hipError_t launch_weight_dequant_f16(hipStream_t s, const WeightView &w, uint16_t *out_kn)
