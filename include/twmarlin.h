@@ -84,8 +84,8 @@ void *twm_ctx_stream(twm_ctx *ctx);
 /* c_api.rs:69-80 warp_device_info: fills buf with "<name> | <CUs> CUs | <GiB> GiB". */
 int twm_ctx_info(twm_ctx *ctx, char *buf, size_t buf_len);
 /* Tuning knob for per-shape sweeps (the role AutoTuner::tune_gemm plays in
- * crates/kernels/src/autotune.rs:254-396): key "nt" = 16-column tiles per workgroup,
- * 0 = library's choice, else 1, 2 or 4. */
+ * crates/kernels/src/autotune.rs:254-396): key "nt" = 16-column tiles per workgroup
+ * (1, 2, 4), key "waves" = waves per workgroup (4, 8, 16); 0 = library's choice. */
 int twm_ctx_set_option(twm_ctx *ctx, const char *key, int value);
 
 /* ---- device memory (GpuTensor::{zeros,from_host,to_host}, tensor.rs:9-104) ------ */

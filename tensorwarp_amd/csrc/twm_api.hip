@@ -43,6 +43,7 @@ struct twm_ctx {
     uint32_t n_counters;
     bool capturing;
     int force_nt;         // 0 = heuristic
+    int force_waves;      // 0 = heuristic
     hipDeviceProp_t prop;
 };
 
@@ -89,6 +90,7 @@ twm_ctx *twm_ctx_create(int ordinal)
     c->ordinal = ordinal;
     c->capturing = false;
     c->force_nt = 0;
+    c->force_waves = 0;
     c->ws = nullptr;
     c->counters = nullptr;
     c->own_stream = nullptr;
@@ -154,7 +156,8 @@ int twm_ctx_info(twm_ctx *ctx, char *buf, size_t buf_len)
     return TWM_OK;
 }
 
-/* Tuning knob for sweeps: "nt" = n-tiles per workgroup (0 = heuristic, else 1, 2 or 4). */
+/* Tuning knobs for sweeps: "nt" = n-tiles per workgroup (0 = heuristic, else 1, 2 or 4);
+ * "waves" = waves per workgroup (0 = heuristic, else 4, 8 or 16). */
 int twm_ctx_set_option(twm_ctx *ctx, const char *key, int value)
 {
     if (!ctx || !key) return fail(TWM_INVALID_HANDLE, "twm_ctx_set_option: null argument");
@@ -162,6 +165,12 @@ int twm_ctx_set_option(twm_ctx *ctx, const char *key, int value)
         if (value != 0 && value != 1 && value != 2 && value != 4)
             return fail(TWM_SHAPE_ERROR, "twm_ctx_set_option: nt must be 0, 1, 2 or 4");
         ctx->force_nt = value;
+        return TWM_OK;
+    }
+    if (strcmp(key, "waves") == 0) {
+        if (value != 0 && value != 4 && value != 8 && value != 16)
+            return fail(TWM_SHAPE_ERROR, "twm_ctx_set_option: waves must be 0, 4, 8 or 16");
+        ctx->force_waves = value;
         return TWM_OK;
     }
     return fail(TWM_UNSUPPORTED_OP, "twm_ctx_set_option: unknown key %s", key);
@@ -540,21 +549,30 @@ int twm_weight_dequant_f16(twm_ctx *ctx, const twm_weight *w, uint16_t *out_kn_d
 
 /* ---- dispatcher --------------------------------------------------------------------------- */
 
-// Split-K / tile choice for 256 CUs x 4 SIMDs.  A workgroup is 4 waves; aim for ~1024
-// workgroups (16 waves per CU) while every wave still has at least one 128-deep k-chunk.
-static DecodePlan plan_decode(uint32_t n_tiles, uint32_t k_chunks, uint32_t m, int force_nt, uint32_t force_splits)
+// Tile / wave / split-K choice for 256 CUs x 4 SIMDs.  Work comes in units of one n-tile x one
+// k-chunk (1 KiB of nibbles).  Aim for about 4096 waves (16 per CU), each with at least two units
+// when the matrix is big enough; split K inside the workgroup first (LDS reduction), across
+// workgroups only when there are too few n-tiles to occupy the CUs.
+static DecodePlan plan_decode(uint32_t n_tiles, uint32_t k_chunks, uint32_t m, int force_nt, int force_waves,
+                              uint32_t force_splits)
 {
     DecodePlan p;
+    uint32_t mt = m > 16 ? 2 : 1;
     p.nt = 1;
-    if (n_tiles >= 4096 && m <= 16) p.nt = 4;
-    else if (n_tiles >= 2048) p.nt = 2;
+    if (n_tiles >= 2048) p.nt = 2;
     if (force_nt) p.nt = (uint32_t)force_nt;
+    if (mt == 2 && p.nt == 4) p.nt = 2;
     uint32_t tg = n_tiles / p.nt;
-    uint32_t max_splits = k_chunks / 4;
-    if (max_splits < 1) max_splits = 1;
-    uint32_t sp = tg ? (1024u + tg / 2) / tg : 1;
-    if (sp < 1) sp = 1;
-    if (sp > max_splits) sp = max_splits;
+    if (tg == 0) tg = 1;
+    // waves per workgroup: enough that tg * waves reaches ~4096, bounded by the chunks available
+    p.waves = 4;
+    while (p.waves < 16 && tg * p.waves < 3072 && k_chunks >= p.waves * 2) p.waves *= 2;
+    if (force_waves) p.waves = (uint32_t)force_waves;
+    while (p.waves > 4 && p.waves * p.nt * mt > 64) p.waves /= 2;
+    // cross-workgroup splits: only when the tile groups alone leave CUs idle
+    uint32_t sp = 1;
+    uint32_t per_wg = p.waves * 2;  // keep >= 2 chunks per wave
+    while (tg * sp < 512 && (k_chunks / (sp * 2)) >= per_wg) sp *= 2;
     if (force_splits) sp = force_splits;
     if (sp > k_chunks) sp = k_chunks ? k_chunks : 1;
     p.splits = sp;
@@ -565,7 +583,7 @@ uint32_t twm_pick_splits(uint32_t k, uint32_t n, uint32_t m)
 {
     uint32_t n_tiles = ((n + kNPadTo - 1) / kNPadTo) * kNPadTo / kTileN;
     uint32_t k_chunks = (k / 32 + kChunkGroups - 1) / kChunkGroups;
-    return plan_decode(n_tiles, k_chunks, m > kMaxDecodeM ? kMaxDecodeM : m, 0, 0).splits;
+    return plan_decode(n_tiles, k_chunks, m > kMaxDecodeM ? kMaxDecodeM : m, 0, 0, 0).splits;
 }
 
 static int gemm_common(twm_ctx *ctx, const twm_weight *w, const void *a_dev, int a_dtype, uint32_t m, const OutSpec &out,
@@ -585,8 +603,7 @@ static int gemm_common(twm_ctx *ctx, const twm_weight *w, const void *a_dev, int
     uint32_t n_ld = w->n_tiles * kTileN;
     for (uint32_t m0 = 0; m0 < m; m0 += kMaxDecodeM) {
         uint32_t mb = m - m0 < (uint32_t)kMaxDecodeM ? m - m0 : (uint32_t)kMaxDecodeM;
-        DecodePlan plan = plan_decode(w->n_tiles, w->k_chunks, mb, ctx->force_nt, splits);
-        if (mb > 16 && plan.nt == 4) plan.nt = 2;
+        DecodePlan plan = plan_decode(w->n_tiles, w->k_chunks, mb, ctx->force_nt, ctx->force_waves, splits);
         // the scratch must hold splits x mb x n_ld partials and one counter per tile group
         while (plan.splits > 1 && (size_t)plan.splits * mb * n_ld * 4 > ctx->ws_bytes) plan.splits--;
         if (w->n_tiles / plan.nt > ctx->n_counters) plan.splits = 1;

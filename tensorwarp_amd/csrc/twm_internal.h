@@ -36,6 +36,7 @@ struct WeightView {
 
 struct DecodePlan {
     uint32_t nt;      // n-tiles per workgroup (1, 2, 4)
+    uint32_t waves;   // waves per workgroup (4, 8, 16); they split the workgroup's k-range
     uint32_t splits;  // cross-workgroup split-K factor
 };
 

@@ -6,18 +6,12 @@
 //   quantizer .................. :414-474, crates/loader/src/gemma_moe_q4.rs:218-254
 //   reorder / fuse ............. :912-956, :1018-1063
 //   split_qkv / split_gate_up .. crates/kernels/src/ops.rs:2255-2297
-// Nothing here is translated from those kernels: the decode kernels stream weights
-// repacked into a wave64 tile order, dequantise in registers with packed-f16 integer
-// tricks and contract on the 16x16x32 f16 MFMA with f32 accumulation.
-#include "twm_internal.h"
+// This file holds the format operations, the GEMV on the reference layout and the repack into
+// the wave tile order; the MFMA decode kernel that streams the repacked weights is in
+// twm_decode.hip.
+#include "twm_device.h"
 
 namespace twm {
-
-typedef _Float16 half8 __attribute__((ext_vector_type(8)));
-typedef _Float16 half2v __attribute__((ext_vector_type(2)));
-typedef float float4v __attribute__((ext_vector_type(4)));
-typedef unsigned int uint4v __attribute__((ext_vector_type(4)));
-typedef unsigned int uint2v __attribute__((ext_vector_type(2)));
 
 __device__ __forceinline__ float f16_bits_to_f32(uint16_t h)
 {
@@ -429,235 +423,6 @@ hipError_t launch_weight_dequant_f16(hipStream_t s, const WeightView &w, uint16_
     hipLaunchKernelGGL(k_weight_dequant_f16, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s,
                        (const uint32_t *)w.qw, (const uint16_t *)w.sc, w.k, w.n, w.k_chunks, out_kn);
     return hipGetLastError();
-}
-
-// ---------------------------------------------------------------------------------
-// decode kernel, M = 1..32
-// ---------------------------------------------------------------------------------
-// One u32 of the tile order -> eight f16 values (q - 8), exact.
-//   (w & 0x000F000F) | 0x6400 6400 : two halves 1024 + q       (nibbles at bits 0..3)
-//   (w & 0x00F000F0) | 0x5400 5400 : two halves   64 + q       (nibbles at bits 4..7)
-// then a packed subtract of 1032 / 72.  Thanks to the nibble permutation done at repack the
-// four resulting registers hold k-offsets (0,1) (2,3) (4,5) (6,7): the MFMA B-operand order.
-__device__ __forceinline__ uint32_t and_or(uint32_t x, uint32_t mask, uint32_t magic)
-{
-    uint32_t r;
-    asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(r) : "v"(x), "s"(mask), "v"(magic));
-    return r;
-}
-
-__device__ __forceinline__ half8 dequant_word(uint32_t w, uint32_t magic_lo, uint32_t magic_hi)
-{
-    union { uint32_t u[4]; half2v h2[4]; half8 h; } r;
-    uint32_t w8 = w >> 8;
-    r.u[0] = and_or(w, 0x000F000Fu, magic_lo);
-    r.u[1] = and_or(w, 0x00F000F0u, magic_hi);
-    r.u[2] = and_or(w8, 0x000F000Fu, magic_lo);
-    r.u[3] = and_or(w8, 0x00F000F0u, magic_hi);
-    const half2v b_lo = {(_Float16)-1032.0f, (_Float16)-1032.0f};
-    const half2v b_hi = {(_Float16)-72.0f, (_Float16)-72.0f};
-    r.h2[0] += b_lo;
-    r.h2[1] += b_hi;
-    r.h2[2] += b_lo;
-    r.h2[3] += b_hi;
-    return r.h;
-}
-
-__device__ __forceinline__ void store_out(const OutSpec &out, uint32_t m, uint32_t col, float v)
-{
-#pragma unroll
-    for (uint32_t s = 0; s < kMaxSegs; s++) {
-        if (s < out.count) {
-            uint32_t rel = col - out.seg[s].start;
-            if (rel < out.seg[s].width) out.seg[s].ptr[(size_t)m * out.seg[s].width + rel] = v;
-        }
-    }
-}
-
-// Workgroup = 4 waves. It owns NT n-tiles (16*NT columns) and the k-chunks
-// [split*cps, (split+1)*cps) of them; wave w takes chunks w, w+4, ... of that range, the four
-// partial tiles are summed through LDS, and, when the launch is split along K, the workgroup
-// parks its tile in `ws` and the last workgroup to arrive for the tile adds the `splits`
-// partials in ascending order (deterministic) and stores the result.
-//   MT : 16-row blocks of A (1 for M <= 16, 2 for M <= 32)
-//   RL : accumulator registers that can hold live rows (M for M < 4, else 4)
-// Block ids are dealt round-robin to the 8 XCDs; the id is unfolded so that every split of a
-// tile lands on the same XCD and the partials stay in that XCD's L2.
-template <int NT, int MT, int RL, bool AF32>
-__global__ __launch_bounds__(256) void k_decode(const uint4v *__restrict__ qw, const uint2v *__restrict__ sc,
-                                                 const void *__restrict__ a_any, OutSpec out, float *__restrict__ ws,
-                                                 unsigned *__restrict__ counters, uint32_t m_rows, uint32_t k,
-                                                 uint32_t n, uint32_t k_chunks, uint32_t tile_groups, uint32_t splits,
-                                                 uint32_t cps)
-{
-    constexpr int IDX = NT * MT * 4;
-    __shared__ float red[4][IDX][64];
-    __shared__ int s_last;
-
-    const uint32_t b = blockIdx.x;
-    const uint32_t xcd = b & 7u, jj = b >> 3;
-    const uint32_t sp = jj % splits;
-    const uint32_t tg = (jj / splits) * 8u + xcd;
-    if (tg >= tile_groups) return;  // whole workgroup leaves together
-
-    const uint32_t wave = threadIdx.x >> 6, lane = threadIdx.x & 63u;
-    const uint32_t c = lane & 15u, kb = lane >> 4;
-    const uint32_t nt0 = tg * NT;
-    const uint32_t kc0 = sp * cps;
-    const uint32_t kc1 = (kc0 + cps < k_chunks) ? kc0 + cps : k_chunks;
-
-    uint32_t magic_lo = 0x64006400u, magic_hi = 0x54005400u;
-    asm volatile("" : "+v"(magic_lo), "+v"(magic_hi));  // keep the two constants in VGPRs
-
-    float4v acc[NT][MT];
-#pragma unroll
-    for (int t = 0; t < NT; t++)
-#pragma unroll
-        for (int mt = 0; mt < MT; mt++) acc[t][mt] = float4v{0.f, 0.f, 0.f, 0.f};
-
-    for (uint32_t kc = kc0 + wave; kc < kc1; kc += 4) {
-        uint4v wq[NT];
-        uint2v ws4[NT];
-#pragma unroll
-        for (int t = 0; t < NT; t++) {
-            size_t tile = (size_t)(nt0 + t) * k_chunks + kc;
-            wq[t] = qw[tile * 64 + lane];
-            ws4[t] = sc[tile * 16 + c];
-        }
-        half8 af[4][MT];
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-            uint32_t k0 = kc * 128u + i * 32u + kb * 8u;
-#pragma unroll
-            for (int mt = 0; mt < MT; mt++) {
-                uint32_t row = mt * 16 + c;
-                half8 v = {0, 0, 0, 0, 0, 0, 0, 0};
-                if (row < m_rows && k0 < k) {
-                    if (AF32) {
-                        const float4 *p = (const float4 *)((const float *)a_any + (size_t)row * k + k0);
-                        float4 x = p[0], y = p[1];
-                        v = half8{(_Float16)x.x, (_Float16)x.y, (_Float16)x.z, (_Float16)x.w,
-                                  (_Float16)y.x, (_Float16)y.y, (_Float16)y.z, (_Float16)y.w};
-                    } else {
-                        v = *(const half8 *)((const _Float16 *)a_any + (size_t)row * k + k0);
-                    }
-                }
-                af[i][mt] = v;
-            }
-        }
-#pragma unroll
-        for (int t = 0; t < NT; t++) {
-            union { uint2v u; _Float16 h[4]; } sv;
-            sv.u = ws4[t];
-#pragma unroll
-            for (int i = 0; i < 4; i++) {
-                half8 bfrag = dequant_word(wq[t][i], magic_lo, magic_hi);
-                float s = (float)sv.h[i];
-#pragma unroll
-                for (int mt = 0; mt < MT; mt++) {
-                    float4v d = __builtin_amdgcn_mfma_f32_16x16x32_f16(af[i][mt], bfrag, float4v{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
-#pragma unroll
-                    for (int r = 0; r < RL; r++) acc[t][mt][r] = fmaf(d[r], s, acc[t][mt][r]);
-                }
-            }
-        }
-    }
-
-    // ---- sum the four waves through LDS ----
-#pragma unroll
-    for (int t = 0; t < NT; t++)
-#pragma unroll
-        for (int mt = 0; mt < MT; mt++)
-#pragma unroll
-            for (int r = 0; r < RL; r++) red[wave][(t * MT + mt) * 4 + r][lane] = acc[t][mt][r];
-    __syncthreads();
-
-    const uint32_t n_ld = ((n + kNPadTo - 1) / kNPadTo) * kNPadTo;  // row stride of the split-K scratch
-
-    float val[NT * MT];
-    bool live[NT * MT];
-    uint32_t om[NT * MT], on[NT * MT];
-#pragma unroll
-    for (int x = 0; x < NT * MT; x++) {
-        uint32_t idx = wave + 4 * x;        // this thread's entries: idx = (t*MT+mt)*4 + r, lane = lane
-        uint32_t r = idx & 3u, tm = idx >> 2;
-        uint32_t mt = tm % MT, t = tm / MT;
-        om[x] = mt * 16 + kb * 4 + r;
-        on[x] = (nt0 + t) * 16 + c;
-        live[x] = (r < (uint32_t)RL) && om[x] < m_rows && on[x] < n;
-        float v = 0.f;
-        if (live[x]) v = (red[0][idx][lane] + red[1][idx][lane]) + (red[2][idx][lane] + red[3][idx][lane]);
-        val[x] = v;
-    }
-
-    if (splits == 1) {
-#pragma unroll
-        for (int x = 0; x < NT * MT; x++)
-            if (live[x]) store_out(out, om[x], on[x], val[x]);
-        return;
-    }
-
-    // ---- cross-workgroup split-K: park the partial, last arrival reduces ----
-#pragma unroll
-    for (int x = 0; x < NT * MT; x++)
-        if (live[x]) ws[((size_t)sp * m_rows + om[x]) * n_ld + on[x]] = val[x];
-    __threadfence();
-    __syncthreads();
-    if (threadIdx.x == 0) {
-        unsigned prev = atomicAdd(&counters[tg], 1u);
-        s_last = (prev == splits - 1);
-    }
-    __syncthreads();
-    if (!s_last) return;
-    __threadfence();
-#pragma unroll
-    for (int x = 0; x < NT * MT; x++) {
-        if (live[x]) {
-            float v = 0.f;
-            for (uint32_t s = 0; s < splits; s++)
-                v += __builtin_nontemporal_load(&ws[((size_t)s * m_rows + om[x]) * n_ld + on[x]]);
-            store_out(out, om[x], on[x], v);
-        }
-    }
-    if (threadIdx.x == 0) counters[tg] = 0u;  // ready for the next launch
-}
-
-template <int NT, int MT, int RL>
-static hipError_t launch_decode_t(hipStream_t s, const WeightView &w, const void *a, bool a_f32, uint32_t m,
-                                  const OutSpec &out, float *ws, unsigned *counters, uint32_t splits)
-{
-    uint32_t tile_groups = w.n_tiles / NT;
-    uint32_t cps = (w.k_chunks + splits - 1) / splits;
-    uint32_t blocks = ((tile_groups + 7) / 8) * 8 * splits;
-    if (a_f32)
-        hipLaunchKernelGGL((k_decode<NT, MT, RL, true>), dim3(blocks), dim3(256), 0, s, (const uint4v *)w.qw,
-                           (const uint2v *)w.sc, a, out, ws, counters, m, w.k, w.n, w.k_chunks, tile_groups, splits, cps);
-    else
-        hipLaunchKernelGGL((k_decode<NT, MT, RL, false>), dim3(blocks), dim3(256), 0, s, (const uint4v *)w.qw,
-                           (const uint2v *)w.sc, a, out, ws, counters, m, w.k, w.n, w.k_chunks, tile_groups, splits, cps);
-    return hipGetLastError();
-}
-
-template <int NT>
-static hipError_t launch_decode_nt(hipStream_t s, const WeightView &w, const void *a, bool a_f32, uint32_t m,
-                                   const OutSpec &out, float *ws, unsigned *counters, uint32_t splits)
-{
-    if (m == 1) return launch_decode_t<NT, 1, 1>(s, w, a, a_f32, m, out, ws, counters, splits);
-    if (m == 2) return launch_decode_t<NT, 1, 2>(s, w, a, a_f32, m, out, ws, counters, splits);
-    if (m <= 16) return launch_decode_t<NT, 1, 4>(s, w, a, a_f32, m, out, ws, counters, splits);
-    return launch_decode_t<NT, 2, 4>(s, w, a, a_f32, m, out, ws, counters, splits);
-}
-
-hipError_t launch_decode(hipStream_t s, const WeightView &w, const void *a, bool a_f32, uint32_t m, const OutSpec &out,
-                         float *ws, unsigned *counters, DecodePlan plan)
-{
-    if (m == 0 || w.n == 0) return hipSuccess;
-    switch (plan.nt) {
-    case 1: return launch_decode_nt<1>(s, w, a, a_f32, m, out, ws, counters, plan.splits);
-    case 2: return launch_decode_nt<2>(s, w, a, a_f32, m, out, ws, counters, plan.splits);
-    case 4: return launch_decode_nt<4>(s, w, a, a_f32, m, out, ws, counters, plan.splits);
-    default: return hipErrorInvalidValue;
-    }
 }
 
 }  // namespace twm
