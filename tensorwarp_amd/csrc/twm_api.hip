@@ -44,6 +44,8 @@ struct twm_ctx {
     bool capturing;
     int force_nt;         // 0 = heuristic
     int force_waves;      // 0 = heuristic
+    int force_kernel;     // 0 = heuristic, 1 = generic decode kernel, 2 = small-M kernel with A in LDS
+    int force_depth;      // 0 = heuristic, else chunks in flight per wave (2 or 4) for the small-M kernel
     hipDeviceProp_t prop;
 };
 
@@ -91,6 +93,8 @@ twm_ctx *twm_ctx_create(int ordinal)
     c->capturing = false;
     c->force_nt = 0;
     c->force_waves = 0;
+    c->force_kernel = 0;
+    c->force_depth = 0;
     c->ws = nullptr;
     c->counters = nullptr;
     c->own_stream = nullptr;
@@ -156,8 +160,9 @@ int twm_ctx_info(twm_ctx *ctx, char *buf, size_t buf_len)
     return TWM_OK;
 }
 
-/* Tuning knobs for sweeps: "nt" = n-tiles per workgroup (0 = heuristic, else 1, 2 or 4);
- * "waves" = waves per workgroup (0 = heuristic, else 4, 8 or 16). */
+/* Tuning knobs for sweeps (0 = heuristic): "nt" = n-tiles per wave / workgroup (1, 2, 4); "waves" =
+ * waves per workgroup of the generic kernel (4, 8, 16); "kernel" = 1 generic, 2 small-M with A in LDS;
+ * "depth" = chunks in flight per wave in the small-M kernel (2, 4). */
 int twm_ctx_set_option(twm_ctx *ctx, const char *key, int value)
 {
     if (!ctx || !key) return fail(TWM_INVALID_HANDLE, "twm_ctx_set_option: null argument");
@@ -171,6 +176,16 @@ int twm_ctx_set_option(twm_ctx *ctx, const char *key, int value)
         if (value != 0 && value != 4 && value != 8 && value != 16)
             return fail(TWM_SHAPE_ERROR, "twm_ctx_set_option: waves must be 0, 4, 8 or 16");
         ctx->force_waves = value;
+        return TWM_OK;
+    }
+    if (strcmp(key, "kernel") == 0) {
+        if (value < 0 || value > 2) return fail(TWM_SHAPE_ERROR, "twm_ctx_set_option: kernel must be 0, 1 or 2");
+        ctx->force_kernel = value;
+        return TWM_OK;
+    }
+    if (strcmp(key, "depth") == 0) {
+        if (value != 0 && value != 2 && value != 4) return fail(TWM_SHAPE_ERROR, "twm_ctx_set_option: depth must be 0, 2 or 4");
+        ctx->force_depth = value;
         return TWM_OK;
     }
     return fail(TWM_UNSUPPORTED_OP, "twm_ctx_set_option: unknown key %s", key);
@@ -557,6 +572,8 @@ static DecodePlan plan_decode(uint32_t n_tiles, uint32_t k_chunks, uint32_t m, i
                               uint32_t force_splits)
 {
     DecodePlan p;
+    p.lds_a = 0;
+    p.depth = 0;
     uint32_t mt = m > 16 ? 2 : 1;
     p.nt = 1;
     if (n_tiles >= 2048) p.nt = 2;
@@ -579,10 +596,40 @@ static DecodePlan plan_decode(uint32_t n_tiles, uint32_t k_chunks, uint32_t m, i
     return p;
 }
 
+// Small-M kernel (A staged in LDS, a wave owns its n-tiles): a workgroup covers 4*nt n-tiles, so
+// split K across workgroups until about three workgroups per CU exist, while each still streams at
+// least one full ring of chunks, and until its slice of A fits the LDS budget.  Returns false when
+// no split factor fits (then the generic kernel runs).
+static bool plan_gemv(uint32_t n_tiles, uint32_t k_chunks, uint32_t m, int force_nt, int force_depth,
+                      uint32_t force_splits, DecodePlan *out)
+{
+    DecodePlan p;
+    p.lds_a = 1;
+    p.waves = 4;
+    p.nt = 1;
+    if (force_nt) p.nt = (uint32_t)force_nt;
+    if (p.nt > n_tiles) p.nt = 1;
+    p.depth = force_depth ? (uint32_t)force_depth : (p.nt == 4 ? 2u : 4u);
+    uint32_t tg = (n_tiles + 4 * p.nt - 1) / (4 * p.nt);
+    uint32_t sp = (768u + tg - 1) / tg;
+    uint32_t max_sp = k_chunks / p.depth;
+    if (max_sp < 1) max_sp = 1;
+    if (sp > max_sp) sp = max_sp;
+    if (force_splits) sp = force_splits;
+    if (sp > k_chunks) sp = k_chunks ? k_chunks : 1;
+    while (sp < k_chunks && gemv_lds_bytes(m, k_chunks, sp) > kGemvMaxLds) sp++;
+    if (gemv_lds_bytes(m, k_chunks, sp) > kGemvMaxLds) return false;
+    p.splits = sp;
+    *out = p;
+    return true;
+}
+
 uint32_t twm_pick_splits(uint32_t k, uint32_t n, uint32_t m)
 {
     uint32_t n_tiles = ((n + kNPadTo - 1) / kNPadTo) * kNPadTo / kTileN;
     uint32_t k_chunks = (k / 32 + kChunkGroups - 1) / kChunkGroups;
+    DecodePlan p;
+    if (m <= 16 && plan_gemv(n_tiles, k_chunks, m, 0, 0, 0, &p)) return p.splits;
     return plan_decode(n_tiles, k_chunks, m > kMaxDecodeM ? kMaxDecodeM : m, 0, 0, 0).splits;
 }
 
@@ -603,15 +650,30 @@ static int gemm_common(twm_ctx *ctx, const twm_weight *w, const void *a_dev, int
     uint32_t n_ld = w->n_tiles * kTileN;
     for (uint32_t m0 = 0; m0 < m; m0 += kMaxDecodeM) {
         uint32_t mb = m - m0 < (uint32_t)kMaxDecodeM ? m - m0 : (uint32_t)kMaxDecodeM;
-        DecodePlan plan = plan_decode(w->n_tiles, w->k_chunks, mb, ctx->force_nt, ctx->force_waves, splits);
+        DecodePlan plan;
+        bool small = mb <= 16 && ctx->force_kernel != 1 &&
+                     plan_gemv(w->n_tiles, w->k_chunks, mb, ctx->force_nt, ctx->force_depth, splits, &plan);
+        if (!small) {
+            if (ctx->force_kernel == 2) return fail(TWM_UNSUPPORTED_OP, "%s: the small-M kernel cannot run this shape", who);
+            plan = plan_decode(w->n_tiles, w->k_chunks, mb, ctx->force_nt, ctx->force_waves, splits);
+        }
         // the scratch must hold splits x mb x n_ld partials and one counter per tile group
         while (plan.splits > 1 && (size_t)plan.splits * mb * n_ld * 4 > ctx->ws_bytes) plan.splits--;
         if (w->n_tiles / plan.nt > ctx->n_counters) plan.splits = 1;
+        if (small && gemv_lds_bytes(mb, w->k_chunks, plan.splits) > kGemvMaxLds) {
+            small = false;
+            plan = plan_decode(w->n_tiles, w->k_chunks, mb, ctx->force_nt, ctx->force_waves, plan.splits);
+        }
         OutSpec o = out;
         for (uint32_t s = 0; s < o.count; s++) o.seg[s].ptr += (size_t)m0 * o.seg[s].width;
         const char *a_blk = (const char *)a_dev + (size_t)m0 * a_row_bytes;
-        HIP_TRY(launch_decode(ctx->stream, v, a_blk, a_dtype == TWM_F32, mb, o, ctx->ws, ctx->counters, plan),
-                TWM_DEVICE_ERROR, "gemm launch");
+        if (small)
+            HIP_TRY(launch_gemv_lds(ctx->stream, v, a_blk, a_dtype == TWM_F32, mb, o, ctx->ws, ctx->counters, plan.nt,
+                                    plan.depth, plan.splits),
+                    TWM_DEVICE_ERROR, "gemv launch");
+        else
+            HIP_TRY(launch_decode(ctx->stream, v, a_blk, a_dtype == TWM_F32, mb, o, ctx->ws, ctx->counters, plan),
+                    TWM_DEVICE_ERROR, "gemm launch");
     }
     return TWM_OK;
 }

@@ -102,8 +102,9 @@ __global__ __launch_bounds__(1024) void k_decode(const uint4v *__restrict__ qw, 
     const DequantConsts dq = make_dequant_consts();
 
     // per-lane bases; the loop only adds chunk offsets
-    const uint4v *qbase = qw + ((size_t)nt0 * k_chunks) * 64 + lane;
-    const uint2v *sbase = sc + ((size_t)nt0 * k_chunks) * 16 + c;
+    const uint32_t n_tiles = tile_groups * NT;
+    const uint4v *qbase = qw + (size_t)nt0 * 64 + lane;
+    const uint2v *sbase = sc + (size_t)nt0 * 16 + c;
     size_t a_row_off[MT];
 #pragma unroll
     for (int mt = 0; mt < MT; mt++) {
@@ -121,8 +122,8 @@ __global__ __launch_bounds__(1024) void k_decode(const uint4v *__restrict__ qw, 
     auto load_chunk = [&](ChunkRegs<NT, MT> &r, uint32_t kc) {
 #pragma unroll
         for (int t = 0; t < NT; t++) {
-            r.wq[t] = qbase[((size_t)t * k_chunks + kc) * 64];
-            r.sc[t] = sbase[((size_t)t * k_chunks + kc) * 16];
+            r.wq[t] = qbase[((size_t)kc * n_tiles + t) * 64];
+            r.sc[t] = sbase[((size_t)kc * n_tiles + t) * 16];
         }
 #pragma unroll
         for (int i = 0; i < 4; i++) {
@@ -256,15 +257,16 @@ static hipError_t launch_decode_t(hipStream_t s, const WeightView &w, const void
 {
     uint32_t tile_groups = w.n_tiles / NT;
     uint32_t cps = (w.k_chunks + plan.splits - 1) / plan.splits;
-    uint32_t blocks = ((tile_groups + 7) / 8) * 8 * plan.splits;
+    uint32_t nsplits = (w.k_chunks + cps - 1) / cps;  // no empty split
+    uint32_t blocks = ((tile_groups + 7) / 8) * 8 * nsplits;
     uint32_t threads = plan.waves * 64;
     size_t lds = (size_t)plan.waves * NT * MT * 4 * 64 * sizeof(float);
     if (a_f32)
         hipLaunchKernelGGL((k_decode<NT, MT, RL, true>), dim3(blocks), dim3(threads), lds, s, (const uint4v *)w.qw,
-                           (const uint2v *)w.sc, a, out, ws, counters, m, w.k, w.n, w.k_chunks, tile_groups, plan.splits, cps);
+                           (const uint2v *)w.sc, a, out, ws, counters, m, w.k, w.n, w.k_chunks, tile_groups, nsplits, cps);
     else
         hipLaunchKernelGGL((k_decode<NT, MT, RL, false>), dim3(blocks), dim3(threads), lds, s, (const uint4v *)w.qw,
-                           (const uint2v *)w.sc, a, out, ws, counters, m, w.k, w.n, w.k_chunks, tile_groups, plan.splits, cps);
+                           (const uint2v *)w.sc, a, out, ws, counters, m, w.k, w.n, w.k_chunks, tile_groups, nsplits, cps);
     return hipGetLastError();
 }
 

@@ -7,16 +7,20 @@ namespace twm {
 
 // ---- repacked ("wave tile") weight layout ---------------------------------------
 // n-tile  = 16 output columns, k-chunk = 4 groups = 128 input features.
-//   qw : uint4 [n_tiles][k_chunks][64]   lane l = (kb = l/16, c = l%16); component i of the
+//   qw : uint4 [k_chunks][n_tiles][64]   lane l = (kb = l/16, c = l%16); component i of the
 //        uint4 is word kb (k = 8*kb .. 8*kb+7) of group 4*kc+i, column 16*nt+c, with its eight
 //        nibbles reordered so that bit position 4*p holds k-offset {0,2,4,6,1,3,5,7}[p].
-//   sc : uint2 [n_tiles][k_chunks][16]   four f16 scales (groups 4*kc .. 4*kc+3) of column c.
+//   sc : uint2 [k_chunks][n_tiles][16]   four f16 scales (groups 4*kc .. 4*kc+3) of column c.
+// The k-chunk index is the slow one: waves working on neighbouring n-tiles advance through k
+// together, so at any moment the whole GPU reads one contiguous band of the array (DRAM pages
+// stay open) instead of thousands of far-apart streams.
 // Columns >= N and groups >= G are padded with nibble 8 / scale 0 (weight exactly 0).
 constexpr int kTileN = 16;
 constexpr int kChunkGroups = 4;
 constexpr int kNPadTo = 64;      // N is padded to a multiple of this, so 1, 2 or 4 tiles per block divide
 constexpr int kMaxSegs = 4;
 constexpr int kMaxDecodeM = 32;
+constexpr size_t kGemvMaxLds = 64 * 1024;  // LDS the small-M kernel may use for its slice of A
 
 struct OutSeg {
     float *ptr;
@@ -38,6 +42,8 @@ struct DecodePlan {
     uint32_t nt;      // n-tiles per workgroup (1, 2, 4)
     uint32_t waves;   // waves per workgroup (4, 8, 16); they split the workgroup's k-range
     uint32_t splits;  // cross-workgroup split-K factor
+    uint32_t lds_a;   // 1: small-M kernel with A staged in LDS (waves own n-tiles, `waves` unused)
+    uint32_t depth;   // chunks in flight per wave for the small-M kernel (2 or 4)
 };
 
 // ---- launchers (all asynchronous on `s`, return the launch status) ---------------
@@ -58,6 +64,9 @@ hipError_t launch_ref_gemv(hipStream_t s, const float *a, const uint8_t *packed,
 hipError_t launch_repack(hipStream_t s, const uint8_t *packed, const uint16_t *scales, uint32_t k, uint32_t n,
                          void *qw, void *sc, uint32_t n_tiles, uint32_t k_chunks);
 hipError_t launch_weight_dequant_f16(hipStream_t s, const WeightView &w, uint16_t *out_kn);
+size_t gemv_lds_bytes(uint32_t m, uint32_t k_chunks, uint32_t splits);
+hipError_t launch_gemv_lds(hipStream_t s, const WeightView &w, const void *a, bool a_f32, uint32_t m, const OutSpec &out,
+                           float *ws, unsigned *counters, uint32_t nt, uint32_t depth, uint32_t splits);
 hipError_t launch_decode(hipStream_t s, const WeightView &w, const void *a, bool a_f32, uint32_t m, const OutSpec &out,
                          float *ws, unsigned *counters, DecodePlan plan);
 

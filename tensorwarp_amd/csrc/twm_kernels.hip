@@ -351,11 +351,11 @@ __device__ __forceinline__ uint32_t permute_word(uint32_t w)
 __global__ __launch_bounds__(256) void k_repack_q(const uint32_t *__restrict__ packed, uint32_t groups, uint32_t n,
                                                    uint32_t n_tiles, uint32_t k_chunks, uint4v *__restrict__ qw)
 {
-    size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;  // (nt * k_chunks + kc) * 64 + lane
+    size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;  // (kc * n_tiles + nt) * 64 + lane
     if (idx >= (size_t)n_tiles * k_chunks * 64) return;
     uint32_t lane = (uint32_t)(idx & 63);
     size_t tile = idx >> 6;
-    uint32_t kc = (uint32_t)(tile % k_chunks), nt = (uint32_t)(tile / k_chunks);
+    uint32_t nt = (uint32_t)(tile % n_tiles), kc = (uint32_t)(tile / n_tiles);
     uint32_t col = nt * 16 + (lane & 15), kb = lane >> 4;
     uint4v o;
 #pragma unroll
@@ -371,11 +371,11 @@ __global__ __launch_bounds__(256) void k_repack_q(const uint32_t *__restrict__ p
 __global__ __launch_bounds__(256) void k_repack_s(const uint16_t *__restrict__ scales, uint32_t groups, uint32_t n,
                                                    uint32_t n_tiles, uint32_t k_chunks, uint2v *__restrict__ sc)
 {
-    size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;  // (nt * k_chunks + kc) * 16 + c
+    size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;  // (kc * n_tiles + nt) * 16 + c
     if (idx >= (size_t)n_tiles * k_chunks * 16) return;
     uint32_t c = (uint32_t)(idx & 15);
     size_t tile = idx >> 4;
-    uint32_t kc = (uint32_t)(tile % k_chunks), nt = (uint32_t)(tile / k_chunks);
+    uint32_t nt = (uint32_t)(tile % n_tiles), kc = (uint32_t)(tile / n_tiles);
     uint32_t col = nt * 16 + c;
     uint32_t h[4];
 #pragma unroll
@@ -402,14 +402,14 @@ hipError_t launch_repack(hipStream_t s, const uint8_t *packed, const uint16_t *s
 // Q4 unpack straight from the wave tile order (used to prove the repack lossless).
 __global__ __launch_bounds__(256) void k_weight_dequant_f16(const uint32_t *__restrict__ qw,
                                                              const uint16_t *__restrict__ sc, uint32_t k, uint32_t n,
-                                                             uint32_t k_chunks, uint16_t *__restrict__ out)
+                                                             uint32_t n_tiles, uint16_t *__restrict__ out)
 {
     size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;  // row * n + col
     if (idx >= (size_t)k * n) return;
     uint32_t row = (uint32_t)(idx / n), col = (uint32_t)(idx % n);
     uint32_t g = row / 32, e = row % 32;
     uint32_t nt = col / 16, c = col % 16, kc = g / 4, i = g % 4, kb = e / 8, j = e % 8;
-    size_t tile = (size_t)nt * k_chunks + kc;
+    size_t tile = (size_t)kc * n_tiles + nt;
     uint32_t w = qw[(tile * 64 + kb * 16 + c) * 4 + i];
     int p = (j & 1) ? 4 + (j >> 1) : (j >> 1);
     int q = (int)((w >> (4 * p)) & 0xFu) - 8;
@@ -421,7 +421,7 @@ hipError_t launch_weight_dequant_f16(hipStream_t s, const WeightView &w, uint16_
     size_t total = (size_t)w.k * w.n;
     if (total == 0) return hipSuccess;
     hipLaunchKernelGGL(k_weight_dequant_f16, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s,
-                       (const uint32_t *)w.qw, (const uint16_t *)w.sc, w.k, w.n, w.k_chunks, out_kn);
+                       (const uint32_t *)w.qw, (const uint16_t *)w.sc, w.k, w.n, w.n_tiles, out_kn);
     return hipGetLastError();
 }
 
