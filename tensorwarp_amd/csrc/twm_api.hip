@@ -46,13 +46,16 @@ struct twm_ctx {
     int force_waves;      // 0 = heuristic
     int force_kernel;     // 0 = heuristic, 1 = generic decode kernel, 2 = small-M kernel with A in LDS
     int force_depth;      // 0 = heuristic, else chunks in flight per wave (2 or 4) for the small-M kernel
+    int dequant_src;      // which copy twm_weight_dequant_f16 unpacks: 0 = 16-column tiles, 1 = column-lane
     hipDeviceProp_t prop;
 };
 
 struct twm_weight {
     twm_ctx *ctx;
-    void *qw;
+    void *qw;   // one allocation: 16-column tile order (qw, sc) then the column-lane copy (cq, cs)
     void *sc;
+    void *cq;
+    void *cs;
     uint32_t k, n, groups, n_tiles, k_chunks;
     size_t bytes;
 };
@@ -95,6 +98,7 @@ twm_ctx *twm_ctx_create(int ordinal)
     c->force_waves = 0;
     c->force_kernel = 0;
     c->force_depth = 0;
+    c->dequant_src = 0;
     c->ws = nullptr;
     c->counters = nullptr;
     c->own_stream = nullptr;
@@ -173,13 +177,18 @@ int twm_ctx_set_option(twm_ctx *ctx, const char *key, int value)
         return TWM_OK;
     }
     if (strcmp(key, "waves") == 0) {
-        if (value != 0 && value != 4 && value != 8 && value != 16)
-            return fail(TWM_SHAPE_ERROR, "twm_ctx_set_option: waves must be 0, 4, 8 or 16");
+        if (value != 0 && value != 1 && value != 2 && value != 4 && value != 8 && value != 16)
+            return fail(TWM_SHAPE_ERROR, "twm_ctx_set_option: waves must be 0, 1, 2, 4, 8 or 16");
         ctx->force_waves = value;
         return TWM_OK;
     }
+    if (strcmp(key, "dequant_src") == 0) {
+        if (value != 0 && value != 1) return fail(TWM_SHAPE_ERROR, "twm_ctx_set_option: dequant_src must be 0 or 1");
+        ctx->dequant_src = value;
+        return TWM_OK;
+    }
     if (strcmp(key, "kernel") == 0) {
-        if (value < 0 || value > 2) return fail(TWM_SHAPE_ERROR, "twm_ctx_set_option: kernel must be 0, 1 or 2");
+        if (value < 0 || value > 3) return fail(TWM_SHAPE_ERROR, "twm_ctx_set_option: kernel must be 0, 1, 2 or 3");
         ctx->force_kernel = value;
         return TWM_OK;
     }
@@ -458,18 +467,22 @@ static twm_weight *weight_alloc(twm_ctx *ctx, uint32_t k, uint32_t n)
     w->n_tiles = n_pad / kTileN;
     w->k_chunks = (w->groups + kChunkGroups - 1) / kChunkGroups;
     size_t tiles = (size_t)w->n_tiles * w->k_chunks;
+    // Both copies hold the same K x N weights (16-column tiles for M > 4, one lane per column for
+    // M <= 4); with 288 GB of HBM the second copy of a 4-bit model is cheap and each kernel streams
+    // the order that suits it.
     size_t qbytes = tiles * 1024, sbytes = tiles * 128;
-    w->bytes = qbytes + sbytes;
-    w->qw = nullptr;
-    w->sc = nullptr;
+    w->bytes = 2 * (qbytes + sbytes);
+    w->qw = w->sc = w->cq = w->cs = nullptr;
     if (tiles == 0) return w;
-    hipError_t e = hipMalloc(&w->qw, qbytes + sbytes);
+    hipError_t e = hipMalloc(&w->qw, w->bytes);
     if (e != hipSuccess) {
-        fail(TWM_MEMORY_ERROR, "twm_weight: hipMalloc(%zu): %s", qbytes + sbytes, hipGetErrorString(e));
+        fail(TWM_MEMORY_ERROR, "twm_weight: hipMalloc(%zu): %s", w->bytes, hipGetErrorString(e));
         delete w;
         return nullptr;
     }
     w->sc = (char *)w->qw + qbytes;
+    w->cq = (char *)w->sc + sbytes;
+    w->cs = (char *)w->cq + qbytes;
     return w;
 }
 
@@ -488,6 +501,8 @@ twm_weight *twm_weight_from_device(twm_ctx *ctx, const uint8_t *packed_dev, cons
     if (!w) return nullptr;
     if (w->qw) {
         hipError_t e = launch_repack(ctx->stream, packed_dev, scales_dev, k, n, w->qw, w->sc, w->n_tiles, w->k_chunks);
+        if (e == hipSuccess)
+            e = launch_repack_col(ctx->stream, packed_dev, scales_dev, k, n, w->cq, w->cs, w->n_tiles * kTileN, w->k_chunks);
         if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
         if (e != hipSuccess) {
             fail(TWM_DEVICE_ERROR, "twm_weight_from_device: repack: %s", hipGetErrorString(e));
@@ -545,6 +560,8 @@ static WeightView view_of(const twm_weight *w)
     WeightView v;
     v.qw = w->qw;
     v.sc = w->sc;
+    v.cq = w->cq;
+    v.cs = w->cs;
     v.k = w->k;
     v.n = w->n;
     v.groups = w->groups;
@@ -558,7 +575,11 @@ int twm_weight_dequant_f16(twm_ctx *ctx, const twm_weight *w, uint16_t *out_kn_d
     if (!ctx || !w) return fail(TWM_INVALID_HANDLE, "twm_weight_dequant_f16: null handle");
     if ((uint64_t)w->k * w->n == 0) return TWM_OK;
     if (!out_kn_dev) return fail(TWM_INVALID_HANDLE, "twm_weight_dequant_f16: null output");
-    HIP_TRY(launch_weight_dequant_f16(ctx->stream, view_of(w), out_kn_dev), TWM_DEVICE_ERROR, "dequant launch");
+    // "dequant_src" = 1 reads the column-lane copy instead of the 16-column tile order
+    if (ctx->dequant_src == 1)
+        HIP_TRY(launch_weight_dequant_f16_col(ctx->stream, view_of(w), out_kn_dev), TWM_DEVICE_ERROR, "dequant launch");
+    else
+        HIP_TRY(launch_weight_dequant_f16(ctx->stream, view_of(w), out_kn_dev), TWM_DEVICE_ERROR, "dequant launch");
     return TWM_OK;
 }
 
@@ -624,11 +645,35 @@ static bool plan_gemv(uint32_t n_tiles, uint32_t k_chunks, uint32_t m, int force
     return true;
 }
 
+// M <= 4 kernel (one lane per column): a workgroup of `waves` waves shares nt tiles of 64 columns
+// and splits its k-chunks among the waves; workgroups split K further when 64-column tiles alone
+// leave CUs idle.  Aim for about 16 waves per CU with at least two chunks per wave.
+static DecodePlan plan_gemv4(uint32_t n_tiles, uint32_t k_chunks, int force_nt, int force_waves, uint32_t force_splits)
+{
+    DecodePlan p;
+    p.lds_a = 2;
+    p.depth = 0;
+    uint32_t tiles64 = n_tiles * kTileN / 64;
+    p.nt = 1;
+    if (force_nt == 2 && tiles64 % 2 == 0) p.nt = 2;
+    uint32_t tg = tiles64 / p.nt;
+    p.waves = 8;
+    while (p.waves > 1 && k_chunks < p.waves * 2) p.waves /= 2;
+    if (force_waves) p.waves = (uint32_t)force_waves;
+    uint32_t sp = 1;
+    while (tg * p.waves * sp < 3072 && k_chunks / (sp * 2) >= p.waves * 2) sp *= 2;
+    if (force_splits) sp = force_splits;
+    if (sp > k_chunks) sp = k_chunks ? k_chunks : 1;
+    p.splits = sp;
+    return p;
+}
+
 uint32_t twm_pick_splits(uint32_t k, uint32_t n, uint32_t m)
 {
     uint32_t n_tiles = ((n + kNPadTo - 1) / kNPadTo) * kNPadTo / kTileN;
     uint32_t k_chunks = (k / 32 + kChunkGroups - 1) / kChunkGroups;
     DecodePlan p;
+    if (m <= 4) return plan_gemv4(n_tiles, k_chunks, 0, 0, 0).splits;
     if (m <= 16 && plan_gemv(n_tiles, k_chunks, m, 0, 0, 0, &p)) return p.splits;
     return plan_decode(n_tiles, k_chunks, m > kMaxDecodeM ? kMaxDecodeM : m, 0, 0, 0).splits;
 }
@@ -651,11 +696,18 @@ static int gemm_common(twm_ctx *ctx, const twm_weight *w, const void *a_dev, int
     for (uint32_t m0 = 0; m0 < m; m0 += kMaxDecodeM) {
         uint32_t mb = m - m0 < (uint32_t)kMaxDecodeM ? m - m0 : (uint32_t)kMaxDecodeM;
         DecodePlan plan;
-        bool small = mb <= 16 && ctx->force_kernel != 1 &&
-                     plan_gemv(w->n_tiles, w->k_chunks, mb, ctx->force_nt, ctx->force_depth, splits, &plan);
-        if (!small) {
-            if (ctx->force_kernel == 2) return fail(TWM_UNSUPPORTED_OP, "%s: the small-M kernel cannot run this shape", who);
-            plan = plan_decode(w->n_tiles, w->k_chunks, mb, ctx->force_nt, ctx->force_waves, splits);
+        bool lane_col = mb <= 4 && (ctx->force_kernel == 0 || ctx->force_kernel == 3);
+        if (ctx->force_kernel == 3 && !lane_col) return fail(TWM_UNSUPPORTED_OP, "%s: the column-lane kernel takes M <= 4", who);
+        bool small = false;
+        if (lane_col) {
+            plan = plan_gemv4(w->n_tiles, w->k_chunks, ctx->force_nt, ctx->force_waves, splits);
+        } else {
+            small = mb <= 16 && ctx->force_kernel != 1 &&
+                    plan_gemv(w->n_tiles, w->k_chunks, mb, ctx->force_nt, ctx->force_depth, splits, &plan);
+            if (!small) {
+                if (ctx->force_kernel == 2) return fail(TWM_UNSUPPORTED_OP, "%s: the small-M kernel cannot run this shape", who);
+                plan = plan_decode(w->n_tiles, w->k_chunks, mb, ctx->force_nt, ctx->force_waves, splits);
+            }
         }
         // the scratch must hold splits x mb x n_ld partials and one counter per tile group
         while (plan.splits > 1 && (size_t)plan.splits * mb * n_ld * 4 > ctx->ws_bytes) plan.splits--;
@@ -667,7 +719,11 @@ static int gemm_common(twm_ctx *ctx, const twm_weight *w, const void *a_dev, int
         OutSpec o = out;
         for (uint32_t s = 0; s < o.count; s++) o.seg[s].ptr += (size_t)m0 * o.seg[s].width;
         const char *a_blk = (const char *)a_dev + (size_t)m0 * a_row_bytes;
-        if (small)
+        if (lane_col)
+            HIP_TRY(launch_gemv4(ctx->stream, v, a_blk, a_dtype == TWM_F32, mb, o, ctx->ws, ctx->counters, plan.nt,
+                                 plan.waves, plan.splits),
+                    TWM_DEVICE_ERROR, "gemv launch");
+        else if (small)
             HIP_TRY(launch_gemv_lds(ctx->stream, v, a_blk, a_dtype == TWM_F32, mb, o, ctx->ws, ctx->counters, plan.nt,
                                     plan.depth, plan.splits),
                     TWM_DEVICE_ERROR, "gemv launch");

@@ -58,12 +58,6 @@ __device__ __forceinline__ void gemv_store_out(const OutSpec &out, uint32_t m, u
     }
 }
 
-template <int NT>
-struct WChunk {
-    uint4v wq[NT];
-    uint2v sc[NT];
-};
-
 // Workgroup = 4 waves; wave w owns n-tiles (tg*4 + w)*NT .. +NT and the k-chunks
 // [split*cps, (split+1)*cps).  RL = number of accumulator registers that hold live rows
 // (min(M, 4)); rows 4..15 of a 16-row tile live in lanes 16..63 of the same registers.
@@ -109,15 +103,20 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 8))) voi
     const uint32_t lane16 = lane * 16u, c8 = c * 8u;
     const size_t qstep = (size_t)n_tiles * 1024u, sstep = (size_t)n_tiles * 128u;  // bytes between k-chunks
     const uint32_t last = nchunks ? nchunks - 1 : 0;
-    WChunk<NT> ring[P];
+    // Two rings of P slots.  Nibbles of chunk j live in slot j % P and are refilled, in place, with
+    // chunk j + P as soon as they have been unpacked.  A scale is still needed after the MFMA, so the
+    // scale slot of step j is refilled one step later (with chunk j + P): no value is ever live
+    // across its own refill, hence no register copies and no wait for a load just issued.
+    uint4v wq_ring[P][NT];
+    uint2v sc_ring[P][NT];
 #pragma unroll
     for (int p = 0; p < P; p++) {
         uint32_t j = (uint32_t)p < last ? (uint32_t)p : last;
         if (nchunks == 0) break;  // never launched (the host normalises the split count); no load without a chunk
 #pragma unroll
         for (int t = 0; t < NT; t++) {
-            ring[p].wq[t] = *(const uint4v *)(qb[t] + (size_t)j * qstep + lane16);
-            ring[p].sc[t] = *(const uint2v *)(sb[t] + (size_t)j * sstep + c8);
+            wq_ring[p][t] = *(const uint4v *)(qb[t] + (size_t)j * qstep + lane16);
+            if (p < P - 1) sc_ring[p][t] = *(const uint2v *)(sb[t] + (size_t)j * sstep + c8);
         }
     }
 
@@ -154,24 +153,31 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 8))) voi
 #pragma unroll
         for (int r = 0; r < RL; r++) acc[t][r] = 0.f;
 
-    // One chunk: unpack (after which the ring slot's registers are dead), refill the slot in place
-    // with the chunk P ahead, then one MFMA per 32-wide group, scale and accumulate in f32.
-    auto process = [&](WChunk<NT> &slot, uint32_t j, bool refill) {
+    // One chunk (slot p = j % P): unpack, refill, then one MFMA per 32-wide group, scale and
+    // accumulate in f32.  The scheduling barriers keep the three phases in this order: left free, the
+    // instruction scheduler hoists the refill above the unpack (forcing copies) or sinks all loads of
+    // the unrolled body to its end (putting a full memory latency on every trip).
+    auto process = [&](const int p, uint32_t j, bool refill) {
         half8 bf[NT][4];
-        uint2v scv[NT];
 #pragma unroll
-        for (int t = 0; t < NT; t++) {
-            scv[t] = slot.sc[t];
+        for (int t = 0; t < NT; t++)
 #pragma unroll
-            for (int i = 0; i < 4; i++) bf[t][i] = gemv_dequant_word(slot.wq[t][i], dq);
-        }
+            for (int i = 0; i < 4; i++) bf[t][i] = gemv_dequant_word(wq_ring[p][t][i], dq);
         if (refill) {
-            const uint32_t jn = j + P < last ? j + P : last;  // the tail re-reads the last chunk
+            // an empty asm (no instruction) that consumes the unpacked registers and clobbers memory:
+            // the unpack cannot sink below it, the refill loads cannot rise above it
+#pragma unroll
+            for (int t = 0; t < NT; t++)
+                asm volatile("" : "+v"(bf[t][0]), "+v"(bf[t][1]), "+v"(bf[t][2]), "+v"(bf[t][3]) : : "memory");
+            const uint32_t jq = j + P < last ? j + P : last;          // the tail re-reads the last chunk
+            const uint32_t js = j + P - 1 < last ? j + P - 1 : last;
+            const int ps = (p + P - 1) % P;
 #pragma unroll
             for (int t = 0; t < NT; t++) {
-                slot.wq[t] = *(const uint4v *)(qb[t] + (size_t)jn * qstep + lane16);
-                slot.sc[t] = *(const uint2v *)(sb[t] + (size_t)jn * sstep + c8);
+                wq_ring[p][t] = *(const uint4v *)(qb[t] + (size_t)jq * qstep + lane16);
+                sc_ring[ps][t] = *(const uint2v *)(sb[t] + (size_t)js * sstep + c8);
             }
+            __builtin_amdgcn_sched_barrier(0);
         }
         half8 af[4];
 #pragma unroll
@@ -179,7 +185,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 8))) voi
 #pragma unroll
         for (int t = 0; t < NT; t++) {
             union { uint2v u; _Float16 h[4]; } sv;
-            sv.u = scv[t];
+            sv.u = sc_ring[p][t];
             float4v d[4];
 #pragma unroll
             for (int i = 0; i < 4; i++)
@@ -197,12 +203,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 8))) voi
     const uint32_t full = nchunks - nchunks % P;
     for (uint32_t j0 = 0; j0 < full; j0 += P) {
 #pragma unroll
-        for (int p = 0; p < P; p++) process(ring[p], j0 + p, true);
+        for (int p = 0; p < P; p++) process(p, j0 + p, true);
     }
-    // ---- tail: the last nchunks % P chunks are already in the ring ----
+    // ---- tail: the last nchunks % P chunks are already in the rings ----
 #pragma unroll
     for (int p = 0; p < P - 1; p++)
-        if (full + p < nchunks) process(ring[p], full + p, false);
+        if (full + p < nchunks) process(p, full + p, false);
 
     // ---- epilogue: lane (c, kb) holds rows kb*4 + r of column (nt_w + t)*16 + c ----
     const uint32_t n_ld = ((n + kNPadTo - 1) / kNPadTo) * kNPadTo;

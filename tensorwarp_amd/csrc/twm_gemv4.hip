@@ -1,0 +1,282 @@
+// Decode kernel for M <= 4 rows of activations: one lane per output column.
+//
+// C[m][n] = sum_g f32(scale[g][n]) * sum_{k in g} A[m][k] * (q[k][n] - 8), f32 accumulation (the
+// arithmetic of warp_gemm_tw_marlin_m1, crates/kernels/src/quantize.rs:1186-1298 in the reference),
+// on the "column-lane" copy of the weights:
+//   cq : uint4 [groups_pad][n_pad]     the 16-byte record of (group g, column n), nibbles permuted
+//                                       inside each 32-bit word as in twm_internal.h
+//   cs : uint2 [k_chunks][n_pad]       four f16 scales (groups 4*kc .. 4*kc+3) of column n
+// A wave owns 64 consecutive columns (lane = column) per tile.  The 32-term sum of a group is done by
+// eight chained v_mfma_f32_4x4x4_16B_f16: the instruction holds 16 independent 4x4 blocks, block b =
+// lanes 4b..4b+3 = four columns, and with CBSZ=4 every block takes its A matrix (4 rows x 4 k) from
+// the block named by ABID.  So ONE 16-byte-per-lane load of activations per 128-deep chunk (lane l
+// holds row l%4, k-piece l/4) feeds all 32 MFMAs of the chunk, the piece being chosen by the ABID
+// immediate: no LDS, no per-MFMA operand traffic, and the output row m of column n is register m of
+// lane n.  Per 1 KiB of nibbles the wave spends 36 VALU on the unpack, 8 MFMA and 1 scale-FMA.
+#include "twm_device.h"
+
+namespace twm {
+
+typedef _Float16 half4v __attribute__((ext_vector_type(4)));
+
+struct Gemv4Consts {
+    uint32_t mask_lo, mask_hi, magic_lo, magic_hi;
+};
+
+__device__ __forceinline__ Gemv4Consts make_gemv4_consts()
+{
+    // opaque to the optimiser so that (w & mask) | magic becomes one v_and_or_b32
+    Gemv4Consts c = {0x000F000Fu, 0x00F000F0u, 0x64006400u, 0x54005400u};
+    asm volatile("" : "+s"(c.mask_lo), "+s"(c.mask_hi), "+v"(c.magic_lo), "+v"(c.magic_hi));
+    return c;
+}
+
+// eight nibbles -> eight exact f16 values q - 8 in k order, as two half4 (k 0..3 and k 4..7)
+__device__ __forceinline__ void gemv4_dequant_word(uint32_t w, const Gemv4Consts &c, half4v &lo4, half4v &hi4)
+{
+    union { uint32_t u[2]; half2v h2[2]; half4v h; } a, b;
+    uint32_t w8 = w >> 8;
+    a.u[0] = (w & c.mask_lo) | c.magic_lo;    // 1024 + q of k0, k1
+    a.u[1] = (w & c.mask_hi) | c.magic_hi;    //   64 + q of k2, k3
+    b.u[0] = (w8 & c.mask_lo) | c.magic_lo;   // k4, k5
+    b.u[1] = (w8 & c.mask_hi) | c.magic_hi;   // k6, k7
+    const half2v b_lo = {(_Float16)-1032.0f, (_Float16)-1032.0f};
+    const half2v b_hi = {(_Float16)-72.0f, (_Float16)-72.0f};
+    a.h2[0] += b_lo;
+    a.h2[1] += b_hi;
+    b.h2[0] += b_lo;
+    b.h2[1] += b_hi;
+    lo4 = a.h;
+    hi4 = b.h;
+}
+
+__device__ __forceinline__ void gemv4_store_out(const OutSpec &out, uint32_t m, uint32_t col, float v)
+{
+#pragma unroll
+    for (uint32_t s = 0; s < kMaxSegs; s++) {
+        if (s < out.count) {
+            uint32_t rel = col - out.seg[s].start;
+            if (rel < out.seg[s].width) out.seg[s].ptr[(size_t)m * out.seg[s].width + rel] = v;
+        }
+    }
+}
+
+template <int NT>
+struct Chunk4 {
+    uint4v wq[NT][4];  // [tile][group in chunk]: this lane's column, 32 nibbles
+    uint2v sc[NT];     // four f16 scales
+    uint4v a;          // activations: row lane%4, k-piece lane/4 (8 halves)
+};
+
+template <int P>
+__device__ __forceinline__ float4v mfma_piece(half4v a, half4v b, float4v c)
+{
+    return __builtin_amdgcn_mfma_f32_4x4x4f16(a, b, c, 4, P, 0);  // CBSZ = 4: all 16 blocks use block P's A
+}
+
+// Workgroup = `waves` waves (blockDim.x / 64) that share NT tiles of 64 columns and split the
+// k-chunks [split*cps, (split+1)*cps) among themselves (wave w: chunks w, w + waves, ...).
+template <int NT, int RL, bool AF32>
+__global__ __launch_bounds__(1024) void k_gemv4(const uint4v *__restrict__ cq, const uint2v *__restrict__ cs,
+                                                 const void *__restrict__ a_any, OutSpec out, float *__restrict__ ws,
+                                                 unsigned *__restrict__ counters, uint32_t m_rows, uint32_t k,
+                                                 uint32_t n, uint32_t n_pad, uint32_t k_chunks, uint32_t tile_groups,
+                                                 uint32_t splits, uint32_t cps)
+{
+    extern __shared__ float red[];  // [waves][NT][RL][64]
+    __shared__ int s_last;
+
+    const uint32_t b = blockIdx.x;
+    const uint32_t xcd = b & 7u, jj = b >> 3;
+    const uint32_t sp = jj % splits;
+    const uint32_t tg = (jj / splits) * 8u + xcd;
+    if (tg >= tile_groups) return;
+
+    const uint32_t waves = blockDim.x >> 6;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const uint32_t lane = threadIdx.x & 63u;
+    const uint32_t kc0 = sp * cps;
+    const uint32_t kc1 = (kc0 + cps < k_chunks) ? kc0 + cps : k_chunks;
+    const uint32_t col0 = tg * NT * 64u + lane;  // this lane's column in tile 0; tile t adds 64*t
+
+    const Gemv4Consts dq = make_gemv4_consts();
+
+    // activations: lane l reads row min(l % 4, M-1), halves [kc*128 + 8*(l/4), +8)
+    uint32_t arow = lane & 3u;
+    if (arow > m_rows - 1) arow = m_rows - 1;
+    const uint32_t apiece = (lane >> 2) * 8u;
+
+    float acc[NT][RL];
+#pragma unroll
+    for (int t = 0; t < NT; t++)
+#pragma unroll
+        for (int r = 0; r < RL; r++) acc[t][r] = 0.f;
+
+    auto load_chunk = [&](Chunk4<NT> &r, uint32_t kc) {
+#pragma unroll
+        for (int t = 0; t < NT; t++) {
+#pragma unroll
+            for (int g = 0; g < 4; g++) r.wq[t][g] = cq[(size_t)(kc * 4u + g) * n_pad + col0 + 64u * t];
+            r.sc[t] = cs[(size_t)kc * n_pad + col0 + 64u * t];
+        }
+        uint32_t k0 = kc * 128u + apiece;
+        if (k0 > k - 8u) k0 = k - 8u;  // only the zero-padded groups of a last partial chunk get here
+        if (AF32) {
+            const float4 *p = (const float4 *)((const float *)a_any + (size_t)arow * k + k0);
+            float4 x = p[0], y = p[1];
+            union { half8 h; uint4v u; } cv;
+            cv.h = half8{(_Float16)x.x, (_Float16)x.y, (_Float16)x.z, (_Float16)x.w,
+                         (_Float16)y.x, (_Float16)y.y, (_Float16)y.z, (_Float16)y.w};
+            r.a = cv.u;
+        } else {
+            r.a = *(const uint4v *)((const _Float16 *)a_any + (size_t)arow * k + k0);
+        }
+    };
+
+    auto compute_chunk = [&](const Chunk4<NT> &r) {
+        union { uint4v u; half4v h[2]; } av;
+        av.u = r.a;  // h[0] = k 0..3 of the lane's piece, h[1] = k 4..7
+#pragma unroll
+        for (int t = 0; t < NT; t++) {
+            union { uint2v u; _Float16 h[4]; } sv;
+            sv.u = r.sc[t];
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+                float4v d = {0.f, 0.f, 0.f, 0.f};
+                half4v lo4, hi4;
+#define TWM_PIECE(W, PIECE)                                       \
+    gemv4_dequant_word(r.wq[t][g][W], dq, lo4, hi4);              \
+    d = mfma_piece<PIECE>(av.h[0], lo4, d);                       \
+    d = mfma_piece<PIECE>(av.h[1], hi4, d);
+                if (g == 0) { TWM_PIECE(0, 0) TWM_PIECE(1, 1) TWM_PIECE(2, 2) TWM_PIECE(3, 3) }
+                if (g == 1) { TWM_PIECE(0, 4) TWM_PIECE(1, 5) TWM_PIECE(2, 6) TWM_PIECE(3, 7) }
+                if (g == 2) { TWM_PIECE(0, 8) TWM_PIECE(1, 9) TWM_PIECE(2, 10) TWM_PIECE(3, 11) }
+                if (g == 3) { TWM_PIECE(0, 12) TWM_PIECE(1, 13) TWM_PIECE(2, 14) TWM_PIECE(3, 15) }
+#undef TWM_PIECE
+                float s = (float)sv.h[g];
+#pragma unroll
+                for (int rr = 0; rr < RL; rr++) acc[t][rr] = fmaf(d[rr], s, acc[t][rr]);
+            }
+        }
+    };
+
+    {
+        // two register sets used alternately: the loads of one are in flight while the other is consumed
+        Chunk4<NT> r0, r1;
+        uint32_t kc = kc0 + wave;
+        if (kc < kc1) {
+            load_chunk(r0, kc);
+            while (true) {
+                uint32_t kn = kc + waves;
+                if (kn < kc1) load_chunk(r1, kn);
+                compute_chunk(r0);
+                if (kn >= kc1) break;
+                kc = kn + waves;
+                if (kc < kc1) load_chunk(r0, kc);
+                compute_chunk(r1);
+                if (kc >= kc1) break;
+            }
+        }
+    }
+
+    // ---- sum the waves' partial vectors through LDS: thread (wave 0.., lane) adds column `lane` ----
+#pragma unroll
+    for (int t = 0; t < NT; t++)
+#pragma unroll
+        for (int r = 0; r < RL; r++) red[((wave * NT + t) * RL + r) * 64 + lane] = acc[t][r];
+    __syncthreads();
+
+    const uint32_t threads = blockDim.x;
+    const uint32_t entries = NT * RL * 64;  // entry e = (t*RL + r)*64 + lane
+    if (splits == 1) {
+        for (uint32_t e = threadIdx.x; e < entries; e += threads) {
+            uint32_t ln = e & 63u, tr = e >> 6, r = tr % RL, t = tr / RL;
+            uint32_t on = (tg * NT + t) * 64u + ln;
+            if (r < m_rows && on < n) {
+                float v = 0.f;
+                for (uint32_t w = 0; w < waves; w++) v += red[(w * NT * RL + tr) * 64 + ln];
+                gemv4_store_out(out, r, on, v);
+            }
+        }
+        return;
+    }
+
+    // cross-workgroup split-K: park the partial (agent-scope relaxed atomics: coherent across the XCDs'
+    // L2s without a cache write-back), bump the arrival counter once the stores have completed; the
+    // last workgroup to arrive adds the partials in ascending split order.
+    for (uint32_t e = threadIdx.x; e < entries; e += threads) {
+        uint32_t ln = e & 63u, tr = e >> 6, r = tr % RL, t = tr / RL;
+        uint32_t on = (tg * NT + t) * 64u + ln;
+        if (r < m_rows && on < n) {
+            float v = 0.f;
+            for (uint32_t w = 0; w < waves; w++) v += red[(w * NT * RL + tr) * 64 + ln];
+            __hip_atomic_store(&ws[((size_t)sp * m_rows + r) * n_pad + on], v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+    }
+    __builtin_amdgcn_s_waitcnt(0);  // vmcnt(0): this wave's scratch stores have completed
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        unsigned prev = __hip_atomic_fetch_add(&counters[tg], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        s_last = (prev == splits - 1);
+    }
+    __syncthreads();
+    if (!s_last) return;
+    for (uint32_t e = threadIdx.x; e < entries; e += threads) {
+        uint32_t ln = e & 63u, tr = e >> 6, r = tr % RL, t = tr / RL;
+        uint32_t on = (tg * NT + t) * 64u + ln;
+        if (r < m_rows && on < n) {
+            float v = 0.f;
+            for (uint32_t s = 0; s < splits; s++)
+                v += __hip_atomic_load(&ws[((size_t)s * m_rows + r) * n_pad + on], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            gemv4_store_out(out, r, on, v);
+        }
+    }
+    if (threadIdx.x == 0) __hip_atomic_store(&counters[tg], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+template <int NT, int RL>
+static hipError_t launch_gemv4_t(hipStream_t s, const WeightView &w, const void *a, bool a_f32, uint32_t m,
+                                 const OutSpec &out, float *ws, unsigned *counters, uint32_t waves, uint32_t splits)
+{
+    uint32_t n_pad = w.n_tiles * kTileN;                 // multiple of 64
+    uint32_t tiles64 = n_pad / 64;
+    uint32_t tile_groups = (tiles64 + NT - 1) / NT;
+    uint32_t cps = (w.k_chunks + splits - 1) / splits;
+    splits = (w.k_chunks + cps - 1) / cps;               // no empty split
+    uint32_t blocks = ((tile_groups + 7) / 8) * 8 * splits;
+    size_t lds = (size_t)waves * NT * RL * 64 * sizeof(float);
+    if (a_f32)
+        hipLaunchKernelGGL((k_gemv4<NT, RL, true>), dim3(blocks), dim3(waves * 64), lds, s, (const uint4v *)w.cq,
+                           (const uint2v *)w.cs, a, out, ws, counters, m, w.k, w.n, n_pad, w.k_chunks, tile_groups,
+                           splits, cps);
+    else
+        hipLaunchKernelGGL((k_gemv4<NT, RL, false>), dim3(blocks), dim3(waves * 64), lds, s, (const uint4v *)w.cq,
+                           (const uint2v *)w.cs, a, out, ws, counters, m, w.k, w.n, n_pad, w.k_chunks, tile_groups,
+                           splits, cps);
+    return hipGetLastError();
+}
+
+hipError_t launch_gemv4(hipStream_t s, const WeightView &w, const void *a, bool a_f32, uint32_t m, const OutSpec &out,
+                        float *ws, unsigned *counters, uint32_t nt, uint32_t waves, uint32_t splits)
+{
+    if (m == 0 || w.n == 0) return hipSuccess;
+    if (m > 4 || splits == 0 || !w.cq) return hipErrorInvalidValue;
+    if (waves != 1 && waves != 2 && waves != 4 && waves != 8 && waves != 16) return hipErrorInvalidValue;
+    // a tile group past the end of the padded columns must not exist: NT has to divide the 64-column tile count
+    uint32_t tiles64 = w.n_tiles * kTileN / 64;
+    if (nt == 0 || tiles64 % nt != 0) return hipErrorInvalidValue;
+    uint32_t rl = m;  // rows 0..m-1 live in registers 0..m-1
+    if (nt == 1) {
+        if (rl == 1) return launch_gemv4_t<1, 1>(s, w, a, a_f32, m, out, ws, counters, waves, splits);
+        if (rl == 2) return launch_gemv4_t<1, 2>(s, w, a, a_f32, m, out, ws, counters, waves, splits);
+        return launch_gemv4_t<1, 4>(s, w, a, a_f32, m, out, ws, counters, waves, splits);
+    }
+    if (nt == 2) {
+        if (rl == 1) return launch_gemv4_t<2, 1>(s, w, a, a_f32, m, out, ws, counters, waves, splits);
+        if (rl == 2) return launch_gemv4_t<2, 2>(s, w, a, a_f32, m, out, ws, counters, waves, splits);
+        return launch_gemv4_t<2, 4>(s, w, a, a_f32, m, out, ws, counters, waves, splits);
+    }
+    return hipErrorInvalidValue;
+}
+
+}  // namespace twm

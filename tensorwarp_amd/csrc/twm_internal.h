@@ -35,6 +35,8 @@ struct OutSpec {
 struct WeightView {
     const void *qw;
     const void *sc;
+    const void *cq;  // column-lane copy (see twm_gemv4.hip): uint4 [groups_pad][n_pad]
+    const void *cs;  //                                        uint2 [k_chunks][n_pad]
     uint32_t k, n, groups, n_tiles, k_chunks;
 };
 
@@ -42,7 +44,8 @@ struct DecodePlan {
     uint32_t nt;      // n-tiles per workgroup (1, 2, 4)
     uint32_t waves;   // waves per workgroup (4, 8, 16); they split the workgroup's k-range
     uint32_t splits;  // cross-workgroup split-K factor
-    uint32_t lds_a;   // 1: small-M kernel with A staged in LDS (waves own n-tiles, `waves` unused)
+    uint32_t lds_a;   // 1: small-M kernel with A staged in LDS (waves own n-tiles, `waves` unused);
+                      // 2: M <= 4 kernel, one lane per column (nt = 64-column tiles per workgroup)
     uint32_t depth;   // chunks in flight per wave for the small-M kernel (2 or 4)
 };
 
@@ -67,6 +70,11 @@ hipError_t launch_weight_dequant_f16(hipStream_t s, const WeightView &w, uint16_
 size_t gemv_lds_bytes(uint32_t m, uint32_t k_chunks, uint32_t splits);
 hipError_t launch_gemv_lds(hipStream_t s, const WeightView &w, const void *a, bool a_f32, uint32_t m, const OutSpec &out,
                            float *ws, unsigned *counters, uint32_t nt, uint32_t depth, uint32_t splits);
+hipError_t launch_repack_col(hipStream_t s, const uint8_t *packed, const uint16_t *scales, uint32_t k, uint32_t n,
+                             void *cq, void *cs, uint32_t n_pad, uint32_t k_chunks);
+hipError_t launch_weight_dequant_f16_col(hipStream_t s, const WeightView &w, uint16_t *out_kn);
+hipError_t launch_gemv4(hipStream_t s, const WeightView &w, const void *a, bool a_f32, uint32_t m, const OutSpec &out,
+                        float *ws, unsigned *counters, uint32_t nt, uint32_t waves, uint32_t splits);
 hipError_t launch_decode(hipStream_t s, const WeightView &w, const void *a, bool a_f32, uint32_t m, const OutSpec &out,
                          float *ws, unsigned *counters, DecodePlan plan);
 

@@ -121,8 +121,13 @@ def test_dequant_matches_golden_bits(dev, name):
     s = T.GpuTensor.from_host(dev, d["scales"], "f16")
     assert np.array_equal(T.dequant_to_f16(dev, p, s, k, n).to_host(), d["dequant_f16"])
     assert np.array_equal(T.dequant_to_f32(dev, p, s, k, n).to_host(), d["dequant_f32"])
-    w = T.MarlinWeight.from_device(dev, p, s, k, n)            # and straight from the repacked form
-    assert np.array_equal(w.dequant_f16().to_host(), d["dequant_f16"])
+    w = T.MarlinWeight.from_device(dev, p, s, k, n)            # and straight from both repacked copies
+    try:
+        for src in (0, 1):                                      # 0 = 16-column tile order, 1 = column-lane order
+            dev.set_option("dequant_src", src)
+            assert np.array_equal(w.dequant_f16().to_host(), d["dequant_f16"]), src
+    finally:
+        dev.set_option("dequant_src", 0)
     w.free()
 
 
@@ -147,7 +152,13 @@ def test_repack_is_lossless_at_7b_shape(dev):
     k, n = 3584, 4608
     packed, scales, _ = synth(k, n, 1, 5)
     w = T.MarlinWeight.upload(dev, packed, scales, k, n)
-    assert np.array_equal(w.dequant_f16().to_host(), O.dequant_f16(packed, scales, k, n))
+    want = O.dequant_f16(packed, scales, k, n)
+    try:
+        for src in (0, 1):
+            dev.set_option("dequant_src", src)
+            assert np.array_equal(w.dequant_f16().to_host(), want), src
+    finally:
+        dev.set_option("dequant_src", 0)
     w.free()
 
 
@@ -271,21 +282,29 @@ def test_batched_decode_7b_shapes(dev, m, k, n):
 
 
 def test_split_k_choice_does_not_change_the_result(dev):
-    # both decode kernels (1 = generic, 2 = small-M with A in LDS), every tile width, many split factors
+    # the decode kernels (1 = generic, 2 = small-M with A in LDS, 3 = one lane per column), every tile
+    # width, many split factors
     k, n = 4096, 4096
     packed, scales, a16 = synth(k, n, 1, 31)
     w = T.MarlinWeight.upload(dev, packed, scales, k, n)
     truth = O.gemm_f64(f16_as_f32(a16), packed, scales, 1, k, n)
     try:
-        for kernel in (1, 2):
+        for kernel in (1, 2, 3):
             dev.set_option("kernel", kernel)
-            for nt in (1, 2, 4):
+            for nt in ((1, 2) if kernel == 3 else (1, 2, 4)):
                 dev.set_option("nt", nt)
                 for splits in (1, 2, 5, 8, 32):
                     got = run_gemm(dev, w, a16, 1, n, splits)
                     assert rel_err(got, truth) < TIGHT, (kernel, nt, splits)
                 # same launch twice is bitwise repeatable (ordered reduction, no float atomics)
                 assert np.array_equal(run_gemm(dev, w, a16, 1, n, 8), run_gemm(dev, w, a16, 1, n, 8))
+            if kernel == 3:
+                dev.set_option("nt", 1)
+                for waves in (1, 2, 4, 8, 16):
+                    dev.set_option("waves", waves)
+                    for splits in (1, 3, 32):
+                        assert rel_err(run_gemm(dev, w, a16, 1, n, splits), truth) < TIGHT, (waves, splits)
+                dev.set_option("waves", 0)
             if kernel == 2:
                 for depth in (2, 4):
                     dev.set_option("depth", depth)
@@ -306,7 +325,7 @@ def test_split_factors_that_do_not_divide_the_k_chunks(dev):
     w = T.MarlinWeight.upload(dev, packed, scales, k, n)
     truth = O.gemm_f64(f16_as_f32(a16), packed, scales, 2, k, n)
     try:
-        for kernel in (1, 2):
+        for kernel in (1, 2, 3):
             dev.set_option("kernel", kernel)
             for depth in ((2, 4) if kernel == 2 else (0,)):
                 dev.set_option("depth", depth)
@@ -326,7 +345,7 @@ def test_small_m_kernel_rows_and_f32_activations(dev, m):
     w = T.MarlinWeight.upload(dev, packed, scales, k, n)
     truth = O.gemm_f64(f16_as_f32(a16), packed, scales, m, k, n)
     try:
-        for kernel in (1, 2):
+        for kernel in ((1, 2, 3) if m <= 4 else (1, 2)):
             dev.set_option("kernel", kernel)
             for splits in (0, 1, 2, 3):
                 for a_f32 in (False, True):
