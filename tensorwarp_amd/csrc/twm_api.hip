@@ -44,8 +44,7 @@ struct twm_ctx {
     bool capturing;
     int force_nt;         // 0 = heuristic
     int force_waves;      // 0 = heuristic
-    int force_kernel;     // 0 = heuristic, 1 = generic decode kernel, 2 = small-M kernel with A in LDS
-    int force_depth;      // 0 = heuristic, else chunks in flight per wave (2 or 4) for the small-M kernel
+    int force_kernel;     // 0 = heuristic, 1 = 16-column tile kernel, 2 = one-lane-per-column kernel (M <= 4)
     int dequant_src;      // which copy twm_weight_dequant_f16 unpacks: 0 = 16-column tiles, 1 = column-lane
     hipDeviceProp_t prop;
 };
@@ -54,8 +53,7 @@ struct twm_weight {
     twm_ctx *ctx;
     void *qw;   // one allocation: 16-column tile order (qw, sc) then the column-lane copy (cq, cs)
     void *sc;
-    void *cq;
-    void *cs;
+    void *cq;   // column-lane copy: 4608-byte blocks (nibbles + scales together)
     uint32_t k, n, groups, n_tiles, k_chunks;
     size_t bytes;
 };
@@ -97,7 +95,6 @@ twm_ctx *twm_ctx_create(int ordinal)
     c->force_nt = 0;
     c->force_waves = 0;
     c->force_kernel = 0;
-    c->force_depth = 0;
     c->dequant_src = 0;
     c->ws = nullptr;
     c->counters = nullptr;
@@ -164,9 +161,9 @@ int twm_ctx_info(twm_ctx *ctx, char *buf, size_t buf_len)
     return TWM_OK;
 }
 
-/* Tuning knobs for sweeps (0 = heuristic): "nt" = n-tiles per wave / workgroup (1, 2, 4); "waves" =
- * waves per workgroup of the generic kernel (4, 8, 16); "kernel" = 1 generic, 2 small-M with A in LDS;
- * "depth" = chunks in flight per wave in the small-M kernel (2, 4). */
+/* Tuning knobs for sweeps (0 = heuristic): "nt" = tiles per workgroup (1, 2, 4); "waves" = waves per
+ * workgroup; "kernel" = 1 the 16-column tile kernel, 2 the one-lane-per-column kernel (M <= 4);
+ * "dequant_src" = which weight copy twm_weight_dequant_f16 unpacks. */
 int twm_ctx_set_option(twm_ctx *ctx, const char *key, int value)
 {
     if (!ctx || !key) return fail(TWM_INVALID_HANDLE, "twm_ctx_set_option: null argument");
@@ -188,13 +185,8 @@ int twm_ctx_set_option(twm_ctx *ctx, const char *key, int value)
         return TWM_OK;
     }
     if (strcmp(key, "kernel") == 0) {
-        if (value < 0 || value > 3) return fail(TWM_SHAPE_ERROR, "twm_ctx_set_option: kernel must be 0, 1, 2 or 3");
+        if (value < 0 || value > 2) return fail(TWM_SHAPE_ERROR, "twm_ctx_set_option: kernel must be 0, 1 or 2");
         ctx->force_kernel = value;
-        return TWM_OK;
-    }
-    if (strcmp(key, "depth") == 0) {
-        if (value != 0 && value != 2 && value != 4) return fail(TWM_SHAPE_ERROR, "twm_ctx_set_option: depth must be 0, 2 or 4");
-        ctx->force_depth = value;
         return TWM_OK;
     }
     return fail(TWM_UNSUPPORTED_OP, "twm_ctx_set_option: unknown key %s", key);
@@ -472,7 +464,7 @@ static twm_weight *weight_alloc(twm_ctx *ctx, uint32_t k, uint32_t n)
     // the order that suits it.
     size_t qbytes = tiles * 1024, sbytes = tiles * 128;
     w->bytes = 2 * (qbytes + sbytes);
-    w->qw = w->sc = w->cq = w->cs = nullptr;
+    w->qw = w->sc = w->cq = nullptr;
     if (tiles == 0) return w;
     hipError_t e = hipMalloc(&w->qw, w->bytes);
     if (e != hipSuccess) {
@@ -482,7 +474,6 @@ static twm_weight *weight_alloc(twm_ctx *ctx, uint32_t k, uint32_t n)
     }
     w->sc = (char *)w->qw + qbytes;
     w->cq = (char *)w->sc + sbytes;
-    w->cs = (char *)w->cq + qbytes;
     return w;
 }
 
@@ -502,7 +493,7 @@ twm_weight *twm_weight_from_device(twm_ctx *ctx, const uint8_t *packed_dev, cons
     if (w->qw) {
         hipError_t e = launch_repack(ctx->stream, packed_dev, scales_dev, k, n, w->qw, w->sc, w->n_tiles, w->k_chunks);
         if (e == hipSuccess)
-            e = launch_repack_col(ctx->stream, packed_dev, scales_dev, k, n, w->cq, w->cs, w->n_tiles * kTileN, w->k_chunks);
+            e = launch_repack_col(ctx->stream, packed_dev, scales_dev, k, n, w->cq, w->n_tiles * kTileN, w->k_chunks);
         if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
         if (e != hipSuccess) {
             fail(TWM_DEVICE_ERROR, "twm_weight_from_device: repack: %s", hipGetErrorString(e));
@@ -561,7 +552,6 @@ static WeightView view_of(const twm_weight *w)
     v.qw = w->qw;
     v.sc = w->sc;
     v.cq = w->cq;
-    v.cs = w->cs;
     v.k = w->k;
     v.n = w->n;
     v.groups = w->groups;
@@ -593,20 +583,17 @@ static DecodePlan plan_decode(uint32_t n_tiles, uint32_t k_chunks, uint32_t m, i
                               uint32_t force_splits)
 {
     DecodePlan p;
-    p.lds_a = 0;
-    p.depth = 0;
-    uint32_t mt = m > 16 ? 2 : 1;
+    p.lane_col = 0;
     p.nt = 1;
     if (n_tiles >= 2048) p.nt = 2;
     if (force_nt) p.nt = (uint32_t)force_nt;
-    if (mt == 2 && p.nt == 4) p.nt = 2;
     uint32_t tg = n_tiles / p.nt;
     if (tg == 0) tg = 1;
     // waves per workgroup: enough that tg * waves reaches ~4096, bounded by the chunks available
     p.waves = 4;
     while (p.waves < 16 && tg * p.waves < 3072 && k_chunks >= p.waves * 2) p.waves *= 2;
     if (force_waves) p.waves = (uint32_t)force_waves;
-    while (p.waves > 4 && p.waves * p.nt * mt > 64) p.waves /= 2;
+    while (p.waves > 4 && p.waves * p.nt > 64) p.waves /= 2;
     // cross-workgroup splits: only when the tile groups alone leave CUs idle
     uint32_t sp = 1;
     uint32_t per_wg = p.waves * 2;  // keep >= 2 chunks per wave
@@ -617,42 +604,13 @@ static DecodePlan plan_decode(uint32_t n_tiles, uint32_t k_chunks, uint32_t m, i
     return p;
 }
 
-// Small-M kernel (A staged in LDS, a wave owns its n-tiles): a workgroup covers 4*nt n-tiles, so
-// split K across workgroups until about three workgroups per CU exist, while each still streams at
-// least one full ring of chunks, and until its slice of A fits the LDS budget.  Returns false when
-// no split factor fits (then the generic kernel runs).
-static bool plan_gemv(uint32_t n_tiles, uint32_t k_chunks, uint32_t m, int force_nt, int force_depth,
-                      uint32_t force_splits, DecodePlan *out)
-{
-    DecodePlan p;
-    p.lds_a = 1;
-    p.waves = 4;
-    p.nt = 1;
-    if (force_nt) p.nt = (uint32_t)force_nt;
-    if (p.nt > n_tiles) p.nt = 1;
-    p.depth = force_depth ? (uint32_t)force_depth : (p.nt == 4 ? 2u : 4u);
-    uint32_t tg = (n_tiles + 4 * p.nt - 1) / (4 * p.nt);
-    uint32_t sp = (768u + tg - 1) / tg;
-    uint32_t max_sp = k_chunks / p.depth;
-    if (max_sp < 1) max_sp = 1;
-    if (sp > max_sp) sp = max_sp;
-    if (force_splits) sp = force_splits;
-    if (sp > k_chunks) sp = k_chunks ? k_chunks : 1;
-    while (sp < k_chunks && gemv_lds_bytes(m, k_chunks, sp) > kGemvMaxLds) sp++;
-    if (gemv_lds_bytes(m, k_chunks, sp) > kGemvMaxLds) return false;
-    p.splits = sp;
-    *out = p;
-    return true;
-}
-
 // M <= 4 kernel (one lane per column): a workgroup of `waves` waves shares nt tiles of 64 columns
 // and splits its k-chunks among the waves; workgroups split K further when 64-column tiles alone
 // leave CUs idle.  Aim for about 16 waves per CU with at least two chunks per wave.
 static DecodePlan plan_gemv4(uint32_t n_tiles, uint32_t k_chunks, int force_nt, int force_waves, uint32_t force_splits)
 {
     DecodePlan p;
-    p.lds_a = 2;
-    p.depth = 0;
+    p.lane_col = 1;
     uint32_t tiles64 = n_tiles * kTileN / 64;
     p.nt = 1;
     if (force_nt == 2 && tiles64 % 2 == 0) p.nt = 2;
@@ -660,8 +618,8 @@ static DecodePlan plan_gemv4(uint32_t n_tiles, uint32_t k_chunks, int force_nt, 
     p.waves = 8;
     while (p.waves > 1 && k_chunks < p.waves * 2) p.waves /= 2;
     if (force_waves) p.waves = (uint32_t)force_waves;
-    uint32_t sp = 1;
-    while (tg * p.waves * sp < 3072 && k_chunks / (sp * 2) >= p.waves * 2) sp *= 2;
+    uint32_t sp = 1;  // splitting across workgroups costs a synchronisation: only for matrices with few tiles
+    while (tg * p.waves * sp < 1024 && k_chunks / (sp * 2) >= p.waves * 2) sp *= 2;
     if (force_splits) sp = force_splits;
     if (sp > k_chunks) sp = k_chunks ? k_chunks : 1;
     p.splits = sp;
@@ -672,9 +630,7 @@ uint32_t twm_pick_splits(uint32_t k, uint32_t n, uint32_t m)
 {
     uint32_t n_tiles = ((n + kNPadTo - 1) / kNPadTo) * kNPadTo / kTileN;
     uint32_t k_chunks = (k / 32 + kChunkGroups - 1) / kChunkGroups;
-    DecodePlan p;
     if (m <= 4) return plan_gemv4(n_tiles, k_chunks, 0, 0, 0).splits;
-    if (m <= 16 && plan_gemv(n_tiles, k_chunks, m, 0, 0, 0, &p)) return p.splits;
     return plan_decode(n_tiles, k_chunks, m > kMaxDecodeM ? kMaxDecodeM : m, 0, 0, 0).splits;
 }
 
@@ -696,36 +652,19 @@ static int gemm_common(twm_ctx *ctx, const twm_weight *w, const void *a_dev, int
     for (uint32_t m0 = 0; m0 < m; m0 += kMaxDecodeM) {
         uint32_t mb = m - m0 < (uint32_t)kMaxDecodeM ? m - m0 : (uint32_t)kMaxDecodeM;
         DecodePlan plan;
-        bool lane_col = mb <= 4 && (ctx->force_kernel == 0 || ctx->force_kernel == 3);
-        if (ctx->force_kernel == 3 && !lane_col) return fail(TWM_UNSUPPORTED_OP, "%s: the column-lane kernel takes M <= 4", who);
-        bool small = false;
-        if (lane_col) {
-            plan = plan_gemv4(w->n_tiles, w->k_chunks, ctx->force_nt, ctx->force_waves, splits);
-        } else {
-            small = mb <= 16 && ctx->force_kernel != 1 &&
-                    plan_gemv(w->n_tiles, w->k_chunks, mb, ctx->force_nt, ctx->force_depth, splits, &plan);
-            if (!small) {
-                if (ctx->force_kernel == 2) return fail(TWM_UNSUPPORTED_OP, "%s: the small-M kernel cannot run this shape", who);
-                plan = plan_decode(w->n_tiles, w->k_chunks, mb, ctx->force_nt, ctx->force_waves, splits);
-            }
-        }
+        bool lane_col = mb <= 4 && ctx->force_kernel != 1;
+        if (ctx->force_kernel == 2 && !lane_col) return fail(TWM_UNSUPPORTED_OP, "%s: the one-lane-per-column kernel takes M <= 4", who);
+        if (lane_col) plan = plan_gemv4(w->n_tiles, w->k_chunks, ctx->force_nt, ctx->force_waves, splits);
+        else plan = plan_decode(w->n_tiles, w->k_chunks, mb, ctx->force_nt, ctx->force_waves == 1 || ctx->force_waves == 2 ? 0 : ctx->force_waves, splits);
         // the scratch must hold splits x mb x n_ld partials and one counter per tile group
         while (plan.splits > 1 && (size_t)plan.splits * mb * n_ld * 4 > ctx->ws_bytes) plan.splits--;
         if (w->n_tiles / plan.nt > ctx->n_counters) plan.splits = 1;
-        if (small && gemv_lds_bytes(mb, w->k_chunks, plan.splits) > kGemvMaxLds) {
-            small = false;
-            plan = plan_decode(w->n_tiles, w->k_chunks, mb, ctx->force_nt, ctx->force_waves, plan.splits);
-        }
         OutSpec o = out;
         for (uint32_t s = 0; s < o.count; s++) o.seg[s].ptr += (size_t)m0 * o.seg[s].width;
         const char *a_blk = (const char *)a_dev + (size_t)m0 * a_row_bytes;
         if (lane_col)
             HIP_TRY(launch_gemv4(ctx->stream, v, a_blk, a_dtype == TWM_F32, mb, o, ctx->ws, ctx->counters, plan.nt,
                                  plan.waves, plan.splits),
-                    TWM_DEVICE_ERROR, "gemv launch");
-        else if (small)
-            HIP_TRY(launch_gemv_lds(ctx->stream, v, a_blk, a_dtype == TWM_F32, mb, o, ctx->ws, ctx->counters, plan.nt,
-                                    plan.depth, plan.splits),
                     TWM_DEVICE_ERROR, "gemv launch");
         else
             HIP_TRY(launch_decode(ctx->stream, v, a_blk, a_dtype == TWM_F32, mb, o, ctx->ws, ctx->counters, plan),

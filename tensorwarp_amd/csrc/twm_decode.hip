@@ -1,4 +1,5 @@
-// Decode kernel for the repacked TW-Marlin weights, M = 1..32 rows of activations.
+// Decode kernel on the 16-column tile order, M = 1..16 rows of activations (used for M = 5..16;
+// M <= 4 runs the one-lane-per-column kernel of twm_gemv4.hip).
 //
 // C[m][n] = sum_g f32(scale[g][n]) * sum_{k in g} A[m][k] * (q[k][n] - 8), f32 accumulation: the
 // arithmetic of warp_gemm_tw_marlin_m1 (crates/kernels/src/quantize.rs:1186-1245 in the
@@ -56,11 +57,11 @@ __device__ __forceinline__ void store_out(const OutSpec &out, uint32_t m, uint32
     }
 }
 
-template <int NT, int MT>
+template <int NT>
 struct ChunkRegs {
     uint4v wq[NT];     // 16 B of nibbles per lane per n-tile
     uint2v sc[NT];     // four f16 scales (the chunk's four groups) of this lane's column
-    half8 a[4][MT];    // MFMA A operands: 8 consecutive k of row (lane % 16) per group
+    half8 a[4];        // MFMA A operands: 8 consecutive k of row (lane % 16) per group
 };
 
 // Workgroup = `waves` waves (blockDim.x / 64).  It owns NT n-tiles (16*NT columns) and the
@@ -69,19 +70,19 @@ struct ChunkRegs {
 // tiles are summed through LDS, and, when the launch is also split along K across workgroups, the
 // workgroup parks its tile in `ws` and the last workgroup to arrive for the tile adds the `splits`
 // partials in ascending order (deterministic) and stores the result.
-//   MT : 16-row blocks of A (1 for M <= 16, 2 for M <= 32)
 //   RL : accumulator registers that can hold live rows (M for M < 4, else 4)
 // Rows of A beyond M are read from row M-1 instead of being zeroed (no branches in the loop);
 // the output rows they produce are never stored.
 // Block ids are dealt round-robin to the 8 XCDs; the id is unfolded so that every split of a
 // tile lands on the same XCD and the partials stay in that XCD's L2.
-template <int NT, int MT, int RL, bool AF32>
+template <int NT, int RL, bool AF32>
 __global__ __launch_bounds__(1024) void k_decode(const uint4v *__restrict__ qw, const uint2v *__restrict__ sc,
                                                   const void *__restrict__ a_any, OutSpec out, float *__restrict__ ws,
                                                   unsigned *__restrict__ counters, uint32_t m_rows, uint32_t k,
                                                   uint32_t n, uint32_t k_chunks, uint32_t tile_groups, uint32_t splits,
                                                   uint32_t cps)
 {
+    constexpr int MT = 1;  // one 16-row block of A
     constexpr int IDX = NT * MT * 4;
     extern __shared__ float red[];  // [waves][IDX][64]
     __shared__ int s_last;
@@ -119,7 +120,7 @@ __global__ __launch_bounds__(1024) void k_decode(const uint4v *__restrict__ qw, 
 #pragma unroll
         for (int mt = 0; mt < MT; mt++) acc[t][mt] = float4v{0.f, 0.f, 0.f, 0.f};
 
-    auto load_chunk = [&](ChunkRegs<NT, MT> &r, uint32_t kc) {
+    auto load_chunk = [&](ChunkRegs<NT> &r, uint32_t kc) {
 #pragma unroll
         for (int t = 0; t < NT; t++) {
             r.wq[t] = qbase[((size_t)kc * n_tiles + t) * 64];
@@ -134,16 +135,16 @@ __global__ __launch_bounds__(1024) void k_decode(const uint4v *__restrict__ qw, 
                 if (AF32) {
                     const float4 *p = (const float4 *)((const float *)a_any + a_row_off[mt] + k0);
                     float4 x = p[0], y = p[1];
-                    r.a[i][mt] = half8{(_Float16)x.x, (_Float16)x.y, (_Float16)x.z, (_Float16)x.w,
+                    r.a[i] = half8{(_Float16)x.x, (_Float16)x.y, (_Float16)x.z, (_Float16)x.w,
                                        (_Float16)y.x, (_Float16)y.y, (_Float16)y.z, (_Float16)y.w};
                 } else {
-                    r.a[i][mt] = *(const half8 *)((const _Float16 *)a_any + a_row_off[mt] + k0);
+                    r.a[i] = *(const half8 *)((const _Float16 *)a_any + a_row_off[mt] + k0);
                 }
             }
         }
     };
 
-    auto compute_chunk = [&](const ChunkRegs<NT, MT> &r) {
+    auto compute_chunk = [&](const ChunkRegs<NT> &r) {
 #pragma unroll
         for (int t = 0; t < NT; t++) {
             union { uint2v u; _Float16 h[4]; } sv;
@@ -156,7 +157,7 @@ __global__ __launch_bounds__(1024) void k_decode(const uint4v *__restrict__ qw, 
             for (int i = 0; i < 4; i++)
 #pragma unroll
                 for (int mt = 0; mt < MT; mt++)
-                    d[i][mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(r.a[i][mt], bf[i], float4v{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+                    d[i][mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(r.a[i], bf[i], float4v{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
 #pragma unroll
             for (int i = 0; i < 4; i++) {
                 float s = (float)sv.h[i];
@@ -171,7 +172,7 @@ __global__ __launch_bounds__(1024) void k_decode(const uint4v *__restrict__ qw, 
     {
         // two register sets used alternately: the loads of one are in flight while the other is
         // consumed, and no set is ever copied (a copy would have to wait for its loads)
-        ChunkRegs<NT, MT> r0, r1;
+        ChunkRegs<NT> r0, r1;
         uint32_t kc = kc0 + wave;
         if (kc < kc1) {
             load_chunk(r0, kc);
@@ -251,7 +252,7 @@ __global__ __launch_bounds__(1024) void k_decode(const uint4v *__restrict__ qw, 
     if (threadIdx.x == 0) __hip_atomic_store(&counters[tg], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // ready for the next launch
 }
 
-template <int NT, int MT, int RL>
+template <int NT, int RL>
 static hipError_t launch_decode_t(hipStream_t s, const WeightView &w, const void *a, bool a_f32, uint32_t m,
                                   const OutSpec &out, float *ws, unsigned *counters, const DecodePlan &plan)
 {
@@ -260,12 +261,12 @@ static hipError_t launch_decode_t(hipStream_t s, const WeightView &w, const void
     uint32_t nsplits = (w.k_chunks + cps - 1) / cps;  // no empty split
     uint32_t blocks = ((tile_groups + 7) / 8) * 8 * nsplits;
     uint32_t threads = plan.waves * 64;
-    size_t lds = (size_t)plan.waves * NT * MT * 4 * 64 * sizeof(float);
+    size_t lds = (size_t)plan.waves * NT * 4 * 64 * sizeof(float);
     if (a_f32)
-        hipLaunchKernelGGL((k_decode<NT, MT, RL, true>), dim3(blocks), dim3(threads), lds, s, (const uint4v *)w.qw,
+        hipLaunchKernelGGL((k_decode<NT, RL, true>), dim3(blocks), dim3(threads), lds, s, (const uint4v *)w.qw,
                            (const uint2v *)w.sc, a, out, ws, counters, m, w.k, w.n, w.k_chunks, tile_groups, nsplits, cps);
     else
-        hipLaunchKernelGGL((k_decode<NT, MT, RL, false>), dim3(blocks), dim3(threads), lds, s, (const uint4v *)w.qw,
+        hipLaunchKernelGGL((k_decode<NT, RL, false>), dim3(blocks), dim3(threads), lds, s, (const uint4v *)w.qw,
                            (const uint2v *)w.sc, a, out, ws, counters, m, w.k, w.n, w.k_chunks, tile_groups, nsplits, cps);
     return hipGetLastError();
 }
@@ -274,10 +275,9 @@ template <int NT>
 static hipError_t launch_decode_nt(hipStream_t s, const WeightView &w, const void *a, bool a_f32, uint32_t m,
                                    const OutSpec &out, float *ws, unsigned *counters, const DecodePlan &plan)
 {
-    if (m == 1) return launch_decode_t<NT, 1, 1>(s, w, a, a_f32, m, out, ws, counters, plan);
-    if (m == 2) return launch_decode_t<NT, 1, 2>(s, w, a, a_f32, m, out, ws, counters, plan);
-    if (m <= 16) return launch_decode_t<NT, 1, 4>(s, w, a, a_f32, m, out, ws, counters, plan);
-    return launch_decode_t<NT, 2, 4>(s, w, a, a_f32, m, out, ws, counters, plan);
+    if (m == 1) return launch_decode_t<NT, 1>(s, w, a, a_f32, m, out, ws, counters, plan);
+    if (m == 2) return launch_decode_t<NT, 2>(s, w, a, a_f32, m, out, ws, counters, plan);
+    return launch_decode_t<NT, 4>(s, w, a, a_f32, m, out, ws, counters, plan);
 }
 
 hipError_t launch_decode(hipStream_t s, const WeightView &w, const void *a, bool a_f32, uint32_t m, const OutSpec &out,
@@ -286,8 +286,7 @@ hipError_t launch_decode(hipStream_t s, const WeightView &w, const void *a, bool
     if (m == 0 || w.n == 0) return hipSuccess;
     if (m > (uint32_t)kMaxDecodeM || plan.splits == 0) return hipErrorInvalidValue;
     if (plan.waves != 4 && plan.waves != 8 && plan.waves != 16) return hipErrorInvalidValue;
-    uint32_t mt = m > 16 ? 2 : 1;
-    if (plan.waves * plan.nt * mt > 64) return hipErrorInvalidValue;  // LDS reduction buffer <= 64 KiB
+    if (plan.waves * plan.nt > 64) return hipErrorInvalidValue;  // LDS reduction buffer <= 64 KiB
     switch (plan.nt) {
     case 1: return launch_decode_nt<1>(s, w, a, a_f32, m, out, ws, counters, plan);
     case 2: return launch_decode_nt<2>(s, w, a, a_f32, m, out, ws, counters, plan);

@@ -2,10 +2,13 @@
 //
 // C[m][n] = sum_g f32(scale[g][n]) * sum_{k in g} A[m][k] * (q[k][n] - 8), f32 accumulation (the
 // arithmetic of warp_gemm_tw_marlin_m1, crates/kernels/src/quantize.rs:1186-1298 in the reference),
-// on the "column-lane" copy of the weights:
-//   cq : uint4 [groups_pad][n_pad]     the 16-byte record of (group g, column n), nibbles permuted
-//                                       inside each 32-bit word as in twm_internal.h
-//   cs : uint2 [k_chunks][n_pad]       four f16 scales (groups 4*kc .. 4*kc+3) of column n
+// on the "column-lane" copy of the weights: one 4608-byte block per (64-column tile, 128-deep chunk),
+//   block(tile, kc) at ((tile * k_chunks + kc) * 4608) bytes:
+//     [g = 0..3][lane = 0..63][16 B]   the 16-byte record of (group 4*kc+g, column 64*tile+lane),
+//                                       nibbles permuted inside each 32-bit word as in twm_internal.h
+//     [lane = 0..63][8 B]              the four f16 scales of that column for the chunk's groups
+// so a chunk is one contiguous read and a tile's chunks follow each other: a workgroup streams one
+// contiguous region (scales included) instead of touching every group row of the matrix.
 // A wave owns 64 consecutive columns (lane = column) per tile.  The 32-term sum of a group is done by
 // eight chained v_mfma_f32_4x4x4_16B_f16: the instruction holds 16 independent 4x4 blocks, block b =
 // lanes 4b..4b+3 = four columns, and with CBSZ=4 every block takes its A matrix (4 rows x 4 k) from
@@ -77,9 +80,8 @@ __device__ __forceinline__ float4v mfma_piece(half4v a, half4v b, float4v c)
 // Workgroup = `waves` waves (blockDim.x / 64) that share NT tiles of 64 columns and split the
 // k-chunks [split*cps, (split+1)*cps) among themselves (wave w: chunks w, w + waves, ...).
 template <int NT, int RL, bool AF32>
-__global__ __launch_bounds__(1024) void k_gemv4(const uint4v *__restrict__ cq, const uint2v *__restrict__ cs,
-                                                 const void *__restrict__ a_any, OutSpec out, float *__restrict__ ws,
-                                                 unsigned *__restrict__ counters, uint32_t m_rows, uint32_t k,
+__global__ __launch_bounds__(1024) void k_gemv4(const char *__restrict__ cw, const void *__restrict__ a_any,
+                                                 OutSpec out, float *__restrict__ ws, unsigned *__restrict__ counters, uint32_t m_rows, uint32_t k,
                                                  uint32_t n, uint32_t n_pad, uint32_t k_chunks, uint32_t tile_groups,
                                                  uint32_t splits, uint32_t cps)
 {
@@ -97,7 +99,11 @@ __global__ __launch_bounds__(1024) void k_gemv4(const uint4v *__restrict__ cq, c
     const uint32_t lane = threadIdx.x & 63u;
     const uint32_t kc0 = sp * cps;
     const uint32_t kc1 = (kc0 + cps < k_chunks) ? kc0 + cps : k_chunks;
-    const uint32_t col0 = tg * NT * 64u + lane;  // this lane's column in tile 0; tile t adds 64*t
+    // byte address of this lane's first record in block (tile tg*NT + t, chunk 0)
+    const char *wbase[NT];
+#pragma unroll
+    for (int t = 0; t < NT; t++) wbase[t] = cw + (size_t)(tg * NT + t) * k_chunks * kColBlockBytes;
+    const uint32_t lane16 = lane * 16u, lane8 = 4096u + lane * 8u;
 
     const Gemv4Consts dq = make_gemv4_consts();
 
@@ -115,9 +121,10 @@ __global__ __launch_bounds__(1024) void k_gemv4(const uint4v *__restrict__ cq, c
     auto load_chunk = [&](Chunk4<NT> &r, uint32_t kc) {
 #pragma unroll
         for (int t = 0; t < NT; t++) {
+            const char *blk = wbase[t] + (size_t)kc * kColBlockBytes;
 #pragma unroll
-            for (int g = 0; g < 4; g++) r.wq[t][g] = cq[(size_t)(kc * 4u + g) * n_pad + col0 + 64u * t];
-            r.sc[t] = cs[(size_t)kc * n_pad + col0 + 64u * t];
+            for (int g = 0; g < 4; g++) r.wq[t][g] = *(const uint4v *)(blk + g * 1024u + lane16);
+            r.sc[t] = *(const uint2v *)(blk + lane8);
         }
         uint32_t k0 = kc * 128u + apiece;
         if (k0 > k - 8u) k0 = k - 8u;  // only the zero-padded groups of a last partial chunk get here
@@ -246,12 +253,12 @@ static hipError_t launch_gemv4_t(hipStream_t s, const WeightView &w, const void 
     uint32_t blocks = ((tile_groups + 7) / 8) * 8 * splits;
     size_t lds = (size_t)waves * NT * RL * 64 * sizeof(float);
     if (a_f32)
-        hipLaunchKernelGGL((k_gemv4<NT, RL, true>), dim3(blocks), dim3(waves * 64), lds, s, (const uint4v *)w.cq,
-                           (const uint2v *)w.cs, a, out, ws, counters, m, w.k, w.n, n_pad, w.k_chunks, tile_groups,
+        hipLaunchKernelGGL((k_gemv4<NT, RL, true>), dim3(blocks), dim3(waves * 64), lds, s, (const char *)w.cq, a, out, ws,
+                           counters, m, w.k, w.n, n_pad, w.k_chunks, tile_groups,
                            splits, cps);
     else
-        hipLaunchKernelGGL((k_gemv4<NT, RL, false>), dim3(blocks), dim3(waves * 64), lds, s, (const uint4v *)w.cq,
-                           (const uint2v *)w.cs, a, out, ws, counters, m, w.k, w.n, n_pad, w.k_chunks, tile_groups,
+        hipLaunchKernelGGL((k_gemv4<NT, RL, false>), dim3(blocks), dim3(waves * 64), lds, s, (const char *)w.cq, a, out, ws,
+                           counters, m, w.k, w.n, n_pad, w.k_chunks, tile_groups,
                            splits, cps);
     return hipGetLastError();
 }

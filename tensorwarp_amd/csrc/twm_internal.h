@@ -19,8 +19,8 @@ constexpr int kTileN = 16;
 constexpr int kChunkGroups = 4;
 constexpr int kNPadTo = 64;      // N is padded to a multiple of this, so 1, 2 or 4 tiles per block divide
 constexpr int kMaxSegs = 4;
-constexpr int kMaxDecodeM = 32;
-constexpr size_t kGemvMaxLds = 64 * 1024;  // LDS the small-M kernel may use for its slice of A
+constexpr int kMaxDecodeM = 16;     // rows per launch of the tile kernel (one 16-row MFMA block)
+constexpr uint32_t kColBlockBytes = 4608;  // column-lane copy: 4 x 1024 B of nibbles + 512 B of scales per (tile, chunk)
 
 struct OutSeg {
     float *ptr;
@@ -35,18 +35,15 @@ struct OutSpec {
 struct WeightView {
     const void *qw;
     const void *sc;
-    const void *cq;  // column-lane copy (see twm_gemv4.hip): uint4 [groups_pad][n_pad]
-    const void *cs;  //                                        uint2 [k_chunks][n_pad]
+    const void *cq;  // column-lane copy (see twm_gemv4.hip): 4608-byte blocks [tiles64][k_chunks]
     uint32_t k, n, groups, n_tiles, k_chunks;
 };
 
 struct DecodePlan {
-    uint32_t nt;      // n-tiles per workgroup (1, 2, 4)
+    uint32_t nt;      // tiles per workgroup (1, 2, 4)
     uint32_t waves;   // waves per workgroup (4, 8, 16); they split the workgroup's k-range
     uint32_t splits;  // cross-workgroup split-K factor
-    uint32_t lds_a;   // 1: small-M kernel with A staged in LDS (waves own n-tiles, `waves` unused);
-                      // 2: M <= 4 kernel, one lane per column (nt = 64-column tiles per workgroup)
-    uint32_t depth;   // chunks in flight per wave for the small-M kernel (2 or 4)
+    uint32_t lane_col;  // 1: M <= 4 kernel, one lane per column (nt = 64-column tiles per workgroup)
 };
 
 // ---- launchers (all asynchronous on `s`, return the launch status) ---------------
@@ -67,11 +64,8 @@ hipError_t launch_ref_gemv(hipStream_t s, const float *a, const uint8_t *packed,
 hipError_t launch_repack(hipStream_t s, const uint8_t *packed, const uint16_t *scales, uint32_t k, uint32_t n,
                          void *qw, void *sc, uint32_t n_tiles, uint32_t k_chunks);
 hipError_t launch_weight_dequant_f16(hipStream_t s, const WeightView &w, uint16_t *out_kn);
-size_t gemv_lds_bytes(uint32_t m, uint32_t k_chunks, uint32_t splits);
-hipError_t launch_gemv_lds(hipStream_t s, const WeightView &w, const void *a, bool a_f32, uint32_t m, const OutSpec &out,
-                           float *ws, unsigned *counters, uint32_t nt, uint32_t depth, uint32_t splits);
 hipError_t launch_repack_col(hipStream_t s, const uint8_t *packed, const uint16_t *scales, uint32_t k, uint32_t n,
-                             void *cq, void *cs, uint32_t n_pad, uint32_t k_chunks);
+                             void *cq, uint32_t n_pad, uint32_t k_chunks);
 hipError_t launch_weight_dequant_f16_col(hipStream_t s, const WeightView &w, uint16_t *out_kn);
 hipError_t launch_gemv4(hipStream_t s, const WeightView &w, const void *a, bool a_f32, uint32_t m, const OutSpec &out,
                         float *ws, unsigned *counters, uint32_t nt, uint32_t waves, uint32_t splits);

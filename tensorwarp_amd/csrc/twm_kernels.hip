@@ -426,61 +426,55 @@ hipError_t launch_weight_dequant_f16(hipStream_t s, const WeightView &w, uint16_
 }
 
 // ---------------------------------------------------------------------------------
-// column-lane copy (layout in twm_gemv4.hip): the reference order [g][n] with N padded to a
-// multiple of 64, groups padded to a multiple of 4, nibbles permuted inside each word
+// column-lane copy (layout in twm_gemv4.hip): 4608-byte blocks [tile64][k_chunk], each
+// [4 groups][64 columns][16 B nibbles, permuted inside each word] + [64 columns][4 f16 scales]
 // ---------------------------------------------------------------------------------
-__global__ __launch_bounds__(256) void k_repack_col_q(const uint4v *__restrict__ packed, uint32_t groups, uint32_t n,
-                                                       uint32_t groups_pad, uint32_t n_pad, uint4v *__restrict__ cq)
+__global__ __launch_bounds__(256) void k_repack_col(const uint4v *__restrict__ packed, const uint16_t *__restrict__ scales,
+                                                     uint32_t groups, uint32_t n, uint32_t k_chunks, uint32_t tiles64,
+                                                     char *__restrict__ cw)
 {
-    size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;  // g * n_pad + col
-    if (idx >= (size_t)groups_pad * n_pad) return;
-    uint32_t g = (uint32_t)(idx / n_pad), col = (uint32_t)(idx % n_pad);
+    size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;  // ((tile * k_chunks + kc) * 4 + g) * 64 + lane
+    if (idx >= (size_t)tiles64 * k_chunks * 256) return;
+    uint32_t lane = (uint32_t)(idx & 63), gi = (uint32_t)((idx >> 6) & 3);
+    size_t blk = idx >> 8;
+    uint32_t kc = (uint32_t)(blk % k_chunks), tile = (uint32_t)(blk / k_chunks);
+    uint32_t g = kc * 4 + gi, col = tile * 64 + lane;
     uint4v w = {0x88888888u, 0x88888888u, 0x88888888u, 0x88888888u};
-    if (g < groups && col < n) w = packed[(size_t)g * n + col];
-    uint4v o = {permute_word(w[0]), permute_word(w[1]), permute_word(w[2]), permute_word(w[3])};
-    cq[idx] = o;
-}
-
-__global__ __launch_bounds__(256) void k_repack_col_s(const uint16_t *__restrict__ scales, uint32_t groups, uint32_t n,
-                                                       uint32_t k_chunks, uint32_t n_pad, uint2v *__restrict__ cs)
-{
-    size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;  // kc * n_pad + col
-    if (idx >= (size_t)k_chunks * n_pad) return;
-    uint32_t kc = (uint32_t)(idx / n_pad), col = (uint32_t)(idx % n_pad);
-    uint32_t h[4];
-#pragma unroll
-    for (int i = 0; i < 4; i++) {
-        uint32_t g = kc * 4 + i;
-        h[i] = (g < groups && col < n) ? scales[(size_t)g * n + col] : 0u;
+    uint32_t sbits = 0;
+    if (g < groups && col < n) {
+        w = packed[(size_t)g * n + col];
+        sbits = scales[(size_t)g * n + col];
     }
-    uint2v o = {h[0] | (h[1] << 16), h[2] | (h[3] << 16)};
-    cs[idx] = o;
+    uint4v o = {permute_word(w[0]), permute_word(w[1]), permute_word(w[2]), permute_word(w[3])};
+    char *base = cw + blk * kColBlockBytes;
+    *(uint4v *)(base + gi * 1024u + lane * 16u) = o;
+    *(uint16_t *)(base + 4096u + lane * 8u + gi * 2u) = (uint16_t)sbits;
 }
 
 hipError_t launch_repack_col(hipStream_t s, const uint8_t *packed, const uint16_t *scales, uint32_t k, uint32_t n,
-                             void *cq, void *cs, uint32_t n_pad, uint32_t k_chunks)
+                             void *cq, uint32_t n_pad, uint32_t k_chunks)
 {
-    size_t tq = (size_t)k_chunks * 4 * n_pad, ts = (size_t)k_chunks * n_pad;
-    if (tq == 0) return hipSuccess;
-    hipLaunchKernelGGL(k_repack_col_q, dim3((unsigned)((tq + 255) / 256)), dim3(256), 0, s, (const uint4v *)packed, k / 32,
-                       n, k_chunks * 4, n_pad, (uint4v *)cq);
-    hipLaunchKernelGGL(k_repack_col_s, dim3((unsigned)((ts + 255) / 256)), dim3(256), 0, s, scales, k / 32, n, k_chunks,
-                       n_pad, (uint2v *)cs);
+    size_t total = (size_t)(n_pad / 64) * k_chunks * 256;
+    if (total == 0) return hipSuccess;
+    hipLaunchKernelGGL(k_repack_col, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, (const uint4v *)packed,
+                       scales, k / 32, n, k_chunks, n_pad / 64, (char *)cq);
     return hipGetLastError();
 }
 
-__global__ __launch_bounds__(256) void k_weight_dequant_f16_col(const uint32_t *__restrict__ cq,
-                                                                 const uint16_t *__restrict__ cs, uint32_t k, uint32_t n,
-                                                                 uint32_t n_pad, uint16_t *__restrict__ out)
+__global__ __launch_bounds__(256) void k_weight_dequant_f16_col(const char *__restrict__ cw, uint32_t k, uint32_t n,
+                                                                 uint32_t k_chunks, uint16_t *__restrict__ out)
 {
     size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;  // row * n + col
     if (idx >= (size_t)k * n) return;
     uint32_t row = (uint32_t)(idx / n), col = (uint32_t)(idx % n);
     uint32_t g = row / 32, e = row % 32, j = e % 8;
-    uint32_t w = cq[((size_t)g * n_pad + col) * 4 + e / 8];
+    const char *base = cw + ((size_t)(col / 64) * k_chunks + g / 4) * kColBlockBytes;
+    uint32_t lane = col % 64, gi = g % 4;
+    uint32_t w = *(const uint32_t *)(base + gi * 1024u + lane * 16u + (e / 8) * 4u);
     int p = (j & 1) ? 4 + (j >> 1) : (j >> 1);
     int q = (int)((w >> (4 * p)) & 0xFu) - 8;
-    out[idx] = f32_to_f16_bits(scale_times_q(cs[((size_t)(g / 4) * n_pad + col) * 4 + g % 4], q));
+    uint16_t sbits = *(const uint16_t *)(base + 4096u + lane * 8u + gi * 2u);
+    out[idx] = f32_to_f16_bits(scale_times_q(sbits, q));
 }
 
 hipError_t launch_weight_dequant_f16_col(hipStream_t s, const WeightView &w, uint16_t *out_kn)
@@ -488,7 +482,7 @@ hipError_t launch_weight_dequant_f16_col(hipStream_t s, const WeightView &w, uin
     size_t total = (size_t)w.k * w.n;
     if (total == 0) return hipSuccess;
     hipLaunchKernelGGL(k_weight_dequant_f16_col, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s,
-                       (const uint32_t *)w.cq, (const uint16_t *)w.cs, w.k, w.n, w.n_tiles * kTileN, out_kn);
+                       (const char *)w.cq, w.k, w.n, w.k_chunks, out_kn);
     return hipGetLastError();
 }
 

@@ -282,37 +282,30 @@ def test_batched_decode_7b_shapes(dev, m, k, n):
 
 
 def test_split_k_choice_does_not_change_the_result(dev):
-    # the decode kernels (1 = generic, 2 = small-M with A in LDS, 3 = one lane per column), every tile
-    # width, many split factors
+    # both decode kernels (1 = 16-column tiles, 2 = one lane per column), every tile width, many split factors
     k, n = 4096, 4096
     packed, scales, a16 = synth(k, n, 1, 31)
     w = T.MarlinWeight.upload(dev, packed, scales, k, n)
     truth = O.gemm_f64(f16_as_f32(a16), packed, scales, 1, k, n)
     try:
-        for kernel in (1, 2, 3):
+        for kernel in (1, 2):
             dev.set_option("kernel", kernel)
-            for nt in ((1, 2) if kernel == 3 else (1, 2, 4)):
+            for nt in ((1, 2) if kernel == 2 else (1, 2, 4)):
                 dev.set_option("nt", nt)
                 for splits in (1, 2, 5, 8, 32):
                     got = run_gemm(dev, w, a16, 1, n, splits)
                     assert rel_err(got, truth) < TIGHT, (kernel, nt, splits)
                 # same launch twice is bitwise repeatable (ordered reduction, no float atomics)
                 assert np.array_equal(run_gemm(dev, w, a16, 1, n, 8), run_gemm(dev, w, a16, 1, n, 8))
-            if kernel == 3:
+            if kernel == 2:
                 dev.set_option("nt", 1)
                 for waves in (1, 2, 4, 8, 16):
                     dev.set_option("waves", waves)
                     for splits in (1, 3, 32):
                         assert rel_err(run_gemm(dev, w, a16, 1, n, splits), truth) < TIGHT, (waves, splits)
                 dev.set_option("waves", 0)
-            if kernel == 2:
-                for depth in (2, 4):
-                    dev.set_option("depth", depth)
-                    dev.set_option("nt", 1)
-                    for splits in (1, 3, 7, 16, 32):       # 32 chunks: whole rings, partial rings, single chunks
-                        assert rel_err(run_gemm(dev, w, a16, 1, n, splits), truth) < TIGHT, (depth, splits)
     finally:
-        for key in ("kernel", "nt", "depth", "waves"):
+        for key in ("kernel", "nt", "waves"):
             dev.set_option(key, 0)
     w.free()
 
@@ -325,27 +318,24 @@ def test_split_factors_that_do_not_divide_the_k_chunks(dev):
     w = T.MarlinWeight.upload(dev, packed, scales, k, n)
     truth = O.gemm_f64(f16_as_f32(a16), packed, scales, 2, k, n)
     try:
-        for kernel in (1, 2, 3):
+        for kernel in (1, 2):
             dev.set_option("kernel", kernel)
-            for depth in ((2, 4) if kernel == 2 else (0,)):
-                dev.set_option("depth", depth)
-                for splits in (5, 8, 9, 11, 12, 13, 15, 20, 27, 28):
-                    assert rel_err(run_gemm(dev, w, a16, 2, n, splits), truth) < TIGHT, (kernel, depth, splits)
+            for splits in (5, 8, 9, 11, 12, 13, 15, 20, 27, 28):
+                assert rel_err(run_gemm(dev, w, a16, 2, n, splits), truth) < TIGHT, (kernel, splits)
     finally:
         dev.set_option("kernel", 0)
-        dev.set_option("depth", 0)
     w.free()
 
 
 @pytest.mark.parametrize("m", [1, 2, 3, 4, 7, 16])
-def test_small_m_kernel_rows_and_f32_activations(dev, m):
+def test_decode_kernels_rows_and_f32_activations(dev, m):
     # K = 1184 is 37 groups: 9 full chunks + one chunk with three zero-padded groups; N = 200 is ragged
     k, n = 1184, 200
     packed, scales, a16 = synth(k, n, m, 3000 + m)
     w = T.MarlinWeight.upload(dev, packed, scales, k, n)
     truth = O.gemm_f64(f16_as_f32(a16), packed, scales, m, k, n)
     try:
-        for kernel in ((1, 2, 3) if m <= 4 else (1, 2)):
+        for kernel in ((1, 2) if m <= 4 else (1,)):
             dev.set_option("kernel", kernel)
             for splits in (0, 1, 2, 3):
                 for a_f32 in (False, True):
