@@ -28,9 +28,9 @@ HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X dense FP16 matrix, published
 
 LAYER_7B = [("qkv", 3584, 4608), ("o", 3584, 3584), ("gate_up", 3584, 37888), ("down", 18944, 3584)]
-# HBM bytes per gate_up launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (see profiles/);
-# None until such a run has been made for the kernel in this tree.
-GATE_UP_TRAFFIC_BYTES = None
+# HBM bytes per gate_up launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, each scaled by
+# what the same counter reads for a 64 MiB copy (profiles/k_gemv4_gate_up_m1_hbm_traffic.md).
+GATE_UP_TRAFFIC_BYTES = 76665000
 
 
 def algo_bytes(k, n, m=1):
@@ -69,6 +69,9 @@ def main():
     ap.add_argument("--layers", type=int, default=4, help="distinct weight sets rotated through (>=3 defeats the 256 MB cache)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--extra", action="store_true", help="also time batched decode (M=4..32) on the gate_up shape")
+    ap.add_argument("--pmc-copy", action="store_true",
+                    help="also run four 64 MiB device-to-device copies: a kernel of known traffic to scale rocprofv3 "
+                         "FETCH_SIZE / WRITE_SIZE readings by")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU; --gpus %d is not supported (no collectives, no sharding)" % args.gpus)
@@ -93,6 +96,13 @@ def main():
         for name, k, n in LAYER_7B:
             w, a, c = entry[name]
             T.gemm(dev, w, a, 1, c)
+
+    if args.pmc_copy:
+        src = T.GpuTensor.zeros(dev, (64 << 20,), "u8")
+        dst = T.GpuTensor.zeros(dev, (64 << 20,), "u8")
+        for _ in range(4):
+            dev._l.twm_memcpy_d2d(dev.handle, dst.ptr, src.ptr, 64 << 20)
+        dev.synchronize()
 
     # eager warm-up (also loads every code object before capture), then the graphs
     for li in range(args.layers):
