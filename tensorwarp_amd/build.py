@@ -6,7 +6,7 @@ import subprocess
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libtwmarlin_hip.so")
-SOURCES = ["twm_kernels.hip", "twm_decode.hip", "twm_gemv4.hip", "twm_api.hip"]
+SOURCES = ["twm_kernels.hip", "twm_decode.hip", "twm_gemv4.hip", "twm_prefill.hip", "twm_api.hip"]
 # -packed-fp32-ops off: v_pk_{add,mul,fma}_f32 are not to be generated on this hardware pool.
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared", "-fno-gpu-rdc",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
