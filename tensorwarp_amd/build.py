@@ -2,13 +2,18 @@
 import os
 import shutil
 import subprocess
+from concurrent.futures import ThreadPoolExecutor
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libtwmarlin_hip.so")
 SOURCES = ["twm_kernels.hip", "twm_decode.hip", "twm_gemv4.hip", "twm_prefill.hip", "twm_api.hip"]
+# The prefill kernel keeps its 64 accumulator registers per lane in architectural VGPRs: with the
+# default choice the compiler carries them across the k loop in VGPRs but feeds the MFMAs from AGPRs,
+# and copies all of them twice per iteration.
+PER_FILE_FLAGS = {}
 # -packed-fp32-ops off: v_pk_{add,mul,fma}_f32 are not to be generated on this hardware pool.
-FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared", "-fno-gpu-rdc",
+FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fno-gpu-rdc",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
          "-Wall", "-Wno-unused-function"]
 
@@ -17,11 +22,24 @@ def build(verbose=False):
     """Compile every HIP source for gfx950 and link the shared library. Always recompiles."""
     hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
     tmp = LIB + ".tmp"
-    cmd = [hipcc] + FLAGS + [os.path.join(CSRC, s) for s in SOURCES] + ["-o", tmp]
-    res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
-    out = "\n".join(l for l in res.stdout.splitlines() if "not a recognized feature" not in l)
-    if res.returncode != 0:
-        raise RuntimeError("hipcc failed:\n" + out)
+    objdir = os.path.join(HERE, "_build")
+    os.makedirs(objdir, exist_ok=True)
+
+    def run(cmd):
+        res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+        out = "\n".join(l for l in res.stdout.splitlines() if "not a recognized feature" not in l)
+        if res.returncode != 0:
+            raise RuntimeError("hipcc failed: %s\n%s" % (" ".join(cmd), out))
+        return out
+
+    def compile_one(src):
+        obj = os.path.join(objdir, src.replace(".hip", ".o"))
+        return obj, run([hipcc] + FLAGS + PER_FILE_FLAGS.get(src, []) + ["-c", os.path.join(CSRC, src), "-o", obj])
+
+    with ThreadPoolExecutor(max_workers=min(len(SOURCES), os.cpu_count() or 1)) as pool:
+        results = list(pool.map(compile_one, SOURCES))
+    out = "\n".join(o for _, o in results if o.strip())
+    out += run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-fno-gpu-rdc"] + [o for o, _ in results] + ["-o", tmp])
     os.replace(tmp, LIB)
     if verbose and out.strip():
         print(out)

@@ -45,6 +45,7 @@ struct twm_ctx {
     int force_nt;         // 0 = heuristic
     int force_waves;      // 0 = heuristic
     int force_kernel;     // 0 = heuristic, 1 = 16-column tile kernel, 2 = one-lane-per-column kernel (M <= 4)
+    int prefill_bm;       // rows of A per prefill workgroup: 0 = choose, 64 or 128
     int prefill_min_m;    // M from which the LDS/MFMA prefill kernel runs instead of 16-row decode blocks
     int dequant_src;      // which copy twm_weight_dequant_f16 unpacks: 0 = 16-column tiles, 1 = column-lane
     hipDeviceProp_t prop;
@@ -97,6 +98,7 @@ twm_ctx *twm_ctx_create(int ordinal)
     c->force_waves = 0;
     c->force_kernel = 0;
     c->dequant_src = 0;
+    c->prefill_bm = 0;
     c->prefill_min_m = 33;  // M <= 32 is batched decode: exact f32 weights, weights re-read per 16-row block
     c->ws = nullptr;
     c->counters = nullptr;
@@ -180,6 +182,11 @@ int twm_ctx_set_option(twm_ctx *ctx, const char *key, int value)
         if (value != 0 && value != 1 && value != 2 && value != 4 && value != 8 && value != 16)
             return fail(TWM_SHAPE_ERROR, "twm_ctx_set_option: waves must be 0, 1, 2, 4, 8 or 16");
         ctx->force_waves = value;
+        return TWM_OK;
+    }
+    if (strcmp(key, "prefill_bm") == 0) {
+        if (value != 0 && value != 64 && value != 128) return fail(TWM_SHAPE_ERROR, "twm_ctx_set_option: prefill_bm must be 0, 64 or 128");
+        ctx->prefill_bm = value;
         return TWM_OK;
     }
     if (strcmp(key, "prefill_min_m") == 0) {
@@ -658,7 +665,7 @@ static int gemm_common(twm_ctx *ctx, const twm_weight *w, const void *a_dev, int
     size_t a_row_bytes = (size_t)w->k * (a_dtype == TWM_F16 ? 2 : 4);
     uint32_t n_ld = w->n_tiles * kTileN;
     if (m >= (uint32_t)ctx->prefill_min_m) {
-        HIP_TRY(launch_prefill(ctx->stream, v, a_dev, a_dtype == TWM_F32, m, out), TWM_DEVICE_ERROR, "prefill launch");
+        HIP_TRY(launch_prefill(ctx->stream, v, a_dev, a_dtype == TWM_F32, m, out, (uint32_t)ctx->prefill_bm, ctx->ws, ctx->ws_bytes), TWM_DEVICE_ERROR, "prefill launch");
         return TWM_OK;
     }
     for (uint32_t m0 = 0; m0 < m; m0 += kMaxDecodeM) {

@@ -69,7 +69,8 @@ hipError_t launch_repack_col(hipStream_t s, const uint8_t *packed, const uint16_
 hipError_t launch_weight_dequant_f16_col(hipStream_t s, const WeightView &w, uint16_t *out_kn);
 hipError_t launch_gemv4(hipStream_t s, const WeightView &w, const void *a, bool a_f32, uint32_t m, const OutSpec &out,
                         float *ws, unsigned *counters, uint32_t nt, uint32_t waves, uint32_t splits);
-hipError_t launch_prefill(hipStream_t s, const WeightView &w, const void *a, bool a_f32, uint32_t m, const OutSpec &out);
+hipError_t launch_prefill(hipStream_t s, const WeightView &w, const void *a, bool a_f32, uint32_t m, const OutSpec &out,
+                          uint32_t block_rows, void *scratch, size_t scratch_bytes);
 hipError_t launch_decode(hipStream_t s, const WeightView &w, const void *a, bool a_f32, uint32_t m, const OutSpec &out,
                          float *ws, unsigned *counters, DecodePlan plan);
 

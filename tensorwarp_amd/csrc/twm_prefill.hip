@@ -1,25 +1,27 @@
-// Prefill kernel (M > 16): C[M,N] = A[M,K] * dequant(W), FP16 MFMA with FP32 accumulation.
+// Prefill kernel (M > 32): C[M,N] = A[M,K] * dequant(W), FP16 MFMA with FP32 accumulation.
 //
 // Semantics: gemm_q4_0 (crates/kernels/src/quantize.rs:1825-1858 / kernel :186-246 in the reference),
 // i.e. C[m][n] = sum_k A[m][k] * w[k][n].  Here w is the reference's Q4 unpack to FP16,
 // f16_rne(f32(scale) * (q - 8)) (quantize.rs:534-571), produced in registers: (q - 8) is exact in f16 and
 // one packed f16 multiply by the scale rounds exactly like the reference's __float2half(scale * q).
 //
-// Block = 128 rows x 256 columns, 4 waves; wave w owns 64 columns (four 16-column tiles of the tile-order
-// copy) for all 128 rows, so no weight is unpacked twice inside a block.  Per 128-deep k-chunk:
-//   A tile (128 x 128 f16) : global -> registers -> LDS, double buffered, row stride 272 B so that the
-//                            sixteen rows of a 16-byte-per-lane operand read hit distinct banks;
-//   B : 16 bytes of nibbles + four scales per lane per tile, straight from HBM into registers (prefetched
-//       one chunk ahead), unpacked to MFMA B operands;
-//   128 v_mfma_f32_16x16x32_f16 per wave (8 row blocks x 4 column tiles x 4 groups), 128 accumulator
-//   registers per lane.
+// Block = 16*MT rows x 256 columns (MT = 8 or 4), 4 waves; wave w owns 64 columns (four 16-column tiles of
+// the tile-order copy) for all rows of the block, so no weight is unpacked twice inside a block.  Per
+// 128-deep k-chunk and wave:
+//   A tile (16*MT x 128 f16): global -> registers -> LDS, double buffered, row stride 272 B so that the
+//                             sixteen rows of a 16-byte-per-lane operand read hit distinct banks;
+//   B : 16 bytes of nibbles + four scales per lane per tile, straight from HBM/L2 into registers, two
+//       chunks ahead (three register slots), unpacked to MFMA B operands one 32-deep group ahead;
+//   16*MT v_mfma_f32_16x16x32_f16 (MT row blocks x 4 column tiles x 4 groups), 16*MT accumulator registers.
+// One v_mfma issue slot hides about two other vector instructions, so the unpack (14 instructions per
+// tile and group, shared by MT row blocks) is only free from MT = 8 on.
 #include "twm_device.h"
+
+#include <type_traits>
 
 namespace twm {
 
-constexpr int kPfBM = 128;
 constexpr int kPfRowStride = 136;  // halves per LDS row: 128 + 8 (272 bytes)
-constexpr int kPfTileHalves = kPfBM * kPfRowStride;
 
 struct PfConsts {
     uint32_t mask_lo, mask_hi, magic_lo, magic_hi;
@@ -32,22 +34,37 @@ __device__ __forceinline__ PfConsts make_pf_consts()
     return c;
 }
 
-// eight nibbles -> eight FP16 weights f16(scale * (q - 8)); `s2` holds the scale in both halves
-__device__ __forceinline__ half8 pf_dequant_word(uint32_t w, half2v s2, const PfConsts &c)
+// Pins a uniform address in a scalar register pair so that the load takes it as its scalar base with the
+// per-lane part as a 32-bit offset (otherwise the loop-invariant per-lane part is folded into a 64-bit
+// vector base and every load costs a 64-bit vector add).
+#define TWM_GLOBAL __attribute__((address_space(1)))
+__device__ __forceinline__ const TWM_GLOBAL char *scalar_base(const void *p, size_t byte_offset)
 {
-    union { uint32_t u[4]; half2v h2[4]; half8 h; } r;
-    uint32_t w8 = w >> 8;
-    r.u[0] = (w & c.mask_lo) | c.magic_lo;
-    r.u[1] = (w & c.mask_hi) | c.magic_hi;
-    r.u[2] = (w8 & c.mask_lo) | c.magic_lo;
-    r.u[3] = (w8 & c.mask_hi) | c.magic_hi;
+    uint64_t v = (uint64_t)p + byte_offset;
+    asm("" : "+s"(v));  // not volatile: a volatile asm would cut the scheduling region in two
+    return (const TWM_GLOBAL char *)v;
+}
+
+// MFMA B operand of one tile and group: eight FP16 weights per lane
+union PfFrag {
+    uint32_t u[4];
+    half2v h2[4];
+    half8 h;
+};
+
+// Half of a fragment: nibbles 0..3 (half 0) or 4..7 (half 1) of word `w` -> f16(scale * (q - 8)).
+// 1024 + q and 64 + q are built by OR-ing the nibble into an f16 mantissa; the subtraction is exact.
+__device__ __forceinline__ void pf_unpack_half(PfFrag &r, int half, uint32_t w, uint32_t scale16, const PfConsts &c)
+{
+    union { uint32_t u; half2v h; } s2;
+    s2.u = scale16 | (scale16 << 16);
     const half2v b_lo = {(_Float16)-1032.0f, (_Float16)-1032.0f};
     const half2v b_hi = {(_Float16)-72.0f, (_Float16)-72.0f};
-    r.h2[0] = (r.h2[0] + b_lo) * s2;
-    r.h2[1] = (r.h2[1] + b_hi) * s2;
-    r.h2[2] = (r.h2[2] + b_lo) * s2;
-    r.h2[3] = (r.h2[3] + b_hi) * s2;
-    return r.h;
+    if (half) w >>= 8;
+    r.u[2 * half] = (w & c.mask_lo) | c.magic_lo;
+    r.u[2 * half + 1] = (w & c.mask_hi) | c.magic_hi;
+    r.h2[2 * half] = (r.h2[2 * half] + b_lo) * s2.h;
+    r.h2[2 * half + 1] = (r.h2[2 * half + 1] + b_hi) * s2.h;
 }
 
 __device__ __forceinline__ void pf_store_out(const OutSpec &out, uint32_t m, uint32_t col, float v)
@@ -61,18 +78,23 @@ __device__ __forceinline__ void pf_store_out(const OutSpec &out, uint32_t m, uin
     }
 }
 
-template <bool AF32>
+template <int MT>  // MT = 16-row blocks per workgroup tile (BM = 16 * MT rows)
 __global__ __launch_bounds__(256) void k_prefill(const uint4v *__restrict__ qw, const uint2v *__restrict__ sc,
-                                                  const void *__restrict__ a_any, OutSpec out, uint32_t m_rows,
+                                                  const _Float16 *__restrict__ a_any, OutSpec out, uint32_t m_rows,
                                                   uint32_t k, uint32_t n, uint32_t n_tiles, uint32_t k_chunks)
 {
+    constexpr int kPfTileHalves = 16 * MT * kPfRowStride;
+    constexpr int NV = MT;       // 16-byte vectors of A each thread stages per chunk (16 MT rows * 16 / 256)
+    constexpr int HV = NV / 2;
+    constexpr int PPU = 8 / MT;  // half fragments unpacked per unit (a unit = one row block's four MFMAs)
     extern __shared__ _Float16 a_lds[];  // two tiles of kPfTileHalves
 
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const uint32_t lane = threadIdx.x & 63u;
     const uint32_t c = lane & 15u, kb = lane >> 4;
-    const uint32_t m0 = blockIdx.y * kPfBM;
+    const uint32_t m0 = blockIdx.y * (16u * MT);
     const uint32_t nt0 = (blockIdx.x * 4u + wave) * 4u;  // first of this wave's four 16-column tiles
+    const uint32_t last = k_chunks - 1;
 
     const PfConsts dq = make_pf_consts();
 
@@ -81,96 +103,162 @@ __global__ __launch_bounds__(256) void k_prefill(const uint4v *__restrict__ qw, 
 #pragma unroll
     for (int t = 0; t < 4; t++) nt[t] = nt0 + t < n_tiles ? nt0 + t : n_tiles - 1;
 
-    float4v acc[8][4];
+    // Accumulators live in AGPRs.  The empty asm pins them there across the loop back edge; without it the
+    // compiler carries them in VGPRs and copies all of them to AGPRs and back every iteration.
+    float4v acc[MT][4];
 #pragma unroll
-    for (int mt = 0; mt < 8; mt++)
+    for (int mt = 0; mt < MT; mt++)
 #pragma unroll
         for (int t = 0; t < 4; t++) acc[mt][t] = float4v{0.f, 0.f, 0.f, 0.f};
-
-    // ---- A staging: thread handles eight 16-byte vectors: idx = tid + 256*j, row = idx/16, vec = idx%16 ----
-    uint4v a_stage[8];
-    auto load_a = [&](uint32_t kc) {
+    auto pin_acc = [&]() {
 #pragma unroll
-        for (int j = 0; j < 8; j++) {
-            uint32_t idx = threadIdx.x + 256u * j;
-            uint32_t row = m0 + (idx >> 4), kk = kc * 128u + (idx & 15u) * 8u;
-            uint4v v = {0u, 0u, 0u, 0u};
-            if (row < m_rows && kk < k) {
-                if (AF32) {
-                    const float4 *p = (const float4 *)((const float *)a_any + (size_t)row * k + kk);
-                    float4 x = p[0], y = p[1];
-                    union { half8 h; uint4v u; } cv;
-                    cv.h = half8{(_Float16)x.x, (_Float16)x.y, (_Float16)x.z, (_Float16)x.w,
-                                 (_Float16)y.x, (_Float16)y.y, (_Float16)y.z, (_Float16)y.w};
-                    v = cv.u;
-                } else {
-                    v = *(const uint4v *)((const _Float16 *)a_any + (size_t)row * k + kk);
-                }
-            }
-            a_stage[j] = v;
-        }
+        for (int mt = 0; mt < MT; mt++)
+#pragma unroll
+            for (int t = 0; t < 4; t++) asm volatile("" : "+a"(acc[mt][t]));
     };
-    auto store_a = [&](uint32_t buf) {
-#pragma unroll
-        for (int j = 0; j < 8; j++) {
-            uint32_t idx = threadIdx.x + 256u * j;
-            *(uint4v *)(a_lds + buf * kPfTileHalves + (idx >> 4) * kPfRowStride + (idx & 15u) * 8u) = a_stage[j];
-        }
-    };
+    pin_acc();
 
-    uint4v bq[2][4];
-    uint2v bs[2][4];
-    auto load_b = [&](int slot, uint32_t kc) {
+    // ---- A staging: thread handles NV 16-byte vectors: vector j is row (tid / 16) + 16 j, columns
+    // 8 (tid % 16) .. +7 of the chunk.  Loads are unconditional (clamped addresses) so that the k loop is
+    // straight-line code and the compiler can count outstanding loads exactly.  Rows past m_rows replay the
+    // last row and are never stored; columns past k replay the row's first columns, where the padded
+    // weights are exactly zero.  Address = uniform base of (row block, chunk) + a 32-bit per-thread offset.
+    const char *a_blk = (const char *)a_any + (size_t)m0 * k * 2u;
+    const uint32_t vec = threadIdx.x & 15u;
+    uint32_t a_off[NV];
 #pragma unroll
-        for (int t = 0; t < 4; t++) {
-            size_t tile = (size_t)kc * n_tiles + nt[t];
-            bq[slot][t] = qw[tile * 64 + lane];
-            bs[slot][t] = sc[tile * 16 + c];
-        }
-    };
-
-    auto compute = [&](int slot, uint32_t buf) {
-        const _Float16 *ap = a_lds + buf * kPfTileHalves + c * kPfRowStride + kb * 8u;
-#pragma unroll
-        for (int g = 0; g < 4; g++) {
-            half8 bf[4];
-#pragma unroll
-            for (int t = 0; t < 4; t++) {
-                uint32_t pair = bs[slot][t][g >> 1];
-                uint32_t s16 = (g & 1) ? (pair >> 16) : (pair & 0xFFFFu);
-                union { uint32_t u; half2v h; } s2;
-                s2.u = s16 | (s16 << 16);
-                bf[t] = pf_dequant_word(bq[slot][t][g], s2.h, dq);
-            }
-#pragma unroll
-            for (int mt = 0; mt < 8; mt++) {
-                half8 af = *(const half8 *)(ap + mt * 16 * kPfRowStride + g * 32);
-#pragma unroll
-                for (int t = 0; t < 4; t++)
-                    acc[mt][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(af, bf[t], acc[mt][t], 0, 0, 0);
-            }
-        }
-    };
-
-    // ---- pipeline over k-chunks ----
-    load_a(0);
-    load_b(0, 0);
-    store_a(0);
-    __syncthreads();
-    for (uint32_t kc = 0; kc < k_chunks; kc += 2) {
-        // even chunk: slot 0 / buffer 0
-        if (kc + 1 < k_chunks) { load_a(kc + 1); load_b(1, kc + 1); }
-        compute(0, 0);
-        if (kc + 1 >= k_chunks) break;
-        store_a(1);
-        __syncthreads();
-        // odd chunk: slot 1 / buffer 1
-        if (kc + 2 < k_chunks) { load_a(kc + 2); load_b(0, kc + 2); }
-        compute(1, 1);
-        if (kc + 2 >= k_chunks) break;
-        store_a(0);
-        __syncthreads();
+    for (int j = 0; j < NV; j++) {
+        uint32_t row = m0 + (threadIdx.x >> 4) + 16u * j;
+        row = (row < m_rows ? row : m_rows - 1) - m0;
+        a_off[j] = (row * k + vec * 8u) * 2u;
     }
+    uint4v a_stage[NV];
+    const char *a_src;
+    uint32_t a_back;
+    auto aim_a = [&](uint32_t kc) {  // addresses of chunk kc
+        a_src = a_blk + (size_t)kc * 256u;
+        a_back = kc * 128u + vec * 8u < k ? 0u : vec * 16u;
+    };
+    auto load_a = [&](int j) { a_stage[j] = *(const uint4v *)(a_src + (a_off[j] - a_back)); };
+    const uint32_t wr_off = (threadIdx.x >> 4) * kPfRowStride + vec * 8u;
+    auto store_a = [&](uint32_t buf, int j) {
+        *(uint4v *)(a_lds + buf * kPfTileHalves + wr_off + j * 16 * kPfRowStride) = a_stage[j];
+    };
+
+    // ---- B: chunk kc lives in register slot kc % 3 (one being multiplied, two in flight)
+    uint4v bq[3][4];
+    uint2v bs[3][4];
+    const uint32_t q_off = lane * 16u, s_off = c * 8u;
+    auto load_bq = [&](int slot, uint32_t kc, int t) {
+        bq[slot][t] = *(const TWM_GLOBAL uint4v *)(scalar_base(qw, (size_t)(kc * n_tiles + nt[t]) * 1024u) + q_off);
+    };
+    auto load_bs = [&](int slot, uint32_t kc, int t) {
+        bs[slot][t] = *(const TWM_GLOBAL uint2v *)(scalar_base(sc, (size_t)(kc * n_tiles + nt[t]) * 128u) + s_off);
+    };
+    // half fragment hp (tile hp / 2, half hp % 2) of group g
+    auto unpack = [&](int slot, int g, PfFrag (&bf)[4], int hp) {
+        const int t = hp >> 1;
+        uint32_t pair = bs[slot][t][g >> 1];
+        uint32_t s16 = (g & 1) ? (pair >> 16) : (pair & 0xFFFFu);
+        pf_unpack_half(bf[t], hp & 1, bq[slot][t][g], s16, dq);
+    };
+
+    const uint32_t rd_off = c * kPfRowStride + kb * 8u;
+    auto read_a = [&](uint32_t buf, int g, int mt) {
+        return *(const half8 *)(a_lds + buf * kPfTileHalves + rd_off + mt * 16 * kPfRowStride + g * 32);
+    };
+
+    half8 af0[MT], af1[MT];
+    PfFrag bf0[4], bf1[4];
+
+    // One step = the MFMAs of one 32-deep group, in MT units of four (one row block x four tiles).  Unit mt
+    // also fetches the next group's A operand for its row block, unpacks its share of the next group's B
+    // operands and issues `extra(mt)`, its share of the traffic for later chunks.  The scheduling barrier
+    // after each unit keeps this interleaving: one MFMA issue slot hides about two other instructions,
+    // but only if they sit next to it.
+    auto step = [&](const half8 (&af_cur)[MT], const PfFrag (&bf_cur)[4], half8 (&af_nxt)[MT], PfFrag (&bf_nxt)[4],
+                    uint32_t rd_buf, int rd_g, int uq_slot, int uq_g, auto extra) {
+#pragma unroll
+        for (int mt = 0; mt < MT; mt++) {
+            af_nxt[mt] = read_a(rd_buf, rd_g, mt);
+            extra(mt);
+#pragma unroll
+            for (int p = 0; p < PPU; p++) unpack(uq_slot, uq_g, bf_nxt, mt * PPU + p);
+#pragma unroll
+            for (int t = 0; t < 4; t++)
+                acc[mt][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(af_cur[mt], bf_cur[t].h, acc[mt][t], 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+
+    // One k-chunk (B slot S, LDS buffer kc & 1).  On entry af0 / bf0 hold group 0 of this chunk and a_stage
+    // holds A tile kc+1.
+    //   step 0, 1: write A tile kc+1 to the other LDS buffer; load B nibbles of chunk kc+2
+    //   step 2   : load first half of A tile kc+2; then the chunk's only barrier
+    //   step 3   : load the rest of A tile kc+2 and the B scales of chunk kc+2; its reads and unpack are
+    //              already those of chunk kc+1, group 0
+    // Barrier: tile kc+1 is complete before step 3 reads it, and all reads of buffer (kc+1) & 1 as tile
+    // kc-1 (issued up to step 2 of chunk kc-1 and completed before that chunk's barrier) precede its
+    // rewriting.  Past the end the last chunk is loaded again and never used.
+    auto chunk = [&](auto slot_c, uint32_t kc) {
+        constexpr int S = decltype(slot_c)::value, S1 = (S + 1) % 3, S2 = (S + 2) % 3;
+        const uint32_t buf = kc & 1u;
+        const uint32_t kc2 = kc + 2 < last ? kc + 2 : last;
+        step(af0, bf0, af1, bf1, buf, 1, S, 1, [&](int u) {
+            if (u < 2) load_bq(S2, kc2, u);
+            if (u < HV) store_a(buf ^ 1u, u);
+        });
+        step(af1, bf1, af0, bf0, buf, 2, S, 2, [&](int u) {
+            if (u < 2) load_bq(S2, kc2, 2 + u);
+            if (u < NV - HV) store_a(buf ^ 1u, HV + u);
+        });
+        aim_a(kc2);
+        step(af0, bf0, af1, bf1, buf, 3, S, 3, [&](int u) {
+            if (u < HV) load_a(u);
+        });
+        __syncthreads();
+        step(af1, bf1, af0, bf0, buf ^ 1u, 0, S1, 0, [&](int u) {
+            if (u < NV - HV) load_a(HV + u);
+            if (u >= MT - 4) load_bs(S2, kc2, u - (MT - 4));
+        });
+        pin_acc();
+    };
+    using S0 = std::integral_constant<int, 0>;
+    using S1 = std::integral_constant<int, 1>;
+    using S2 = std::integral_constant<int, 2>;
+
+    // prologue: tile 0 in LDS, tile 1 in the staging registers, B chunks 0 and 1 in slots 0 and 1
+    const uint32_t kc1 = 1 < last ? 1 : last;
+    aim_a(0);
+#pragma unroll
+    for (int j = 0; j < NV; j++) load_a(j);
+#pragma unroll
+    for (int t = 0; t < 4; t++) {
+        load_bq(0, 0, t);
+        load_bs(0, 0, t);
+        load_bq(1, kc1, t);
+        load_bs(1, kc1, t);
+    }
+#pragma unroll
+    for (int j = 0; j < NV; j++) store_a(0, j);
+    aim_a(kc1);
+#pragma unroll
+    for (int j = 0; j < NV; j++) load_a(j);
+    __syncthreads();
+#pragma unroll
+    for (int mt = 0; mt < MT; mt++) af0[mt] = read_a(0, 0, mt);
+#pragma unroll
+    for (int hp = 0; hp < 8; hp++) unpack(0, 0, bf0, hp);
+    __builtin_amdgcn_sched_barrier(0);
+
+    uint32_t kc = 0;
+    for (; kc + 3 <= k_chunks; kc += 3) {
+        chunk(S0{}, kc);
+        chunk(S1{}, kc + 1);
+        chunk(S2{}, kc + 2);
+    }
+    if (kc < k_chunks) chunk(S0{}, kc);
+    if (kc + 1 < k_chunks) chunk(S1{}, kc + 1);
 
     // ---- store: lane (c, kb) holds rows 4*kb + r of row block mt, column 16*tile + c ----
 #pragma unroll
@@ -179,7 +267,7 @@ __global__ __launch_bounds__(256) void k_prefill(const uint4v *__restrict__ qw, 
         uint32_t on = (nt0 + t) * 16u + c;
         if (on >= n) continue;
 #pragma unroll
-        for (int mt = 0; mt < 8; mt++)
+        for (int mt = 0; mt < MT; mt++)
 #pragma unroll
             for (int r = 0; r < 4; r++) {
                 uint32_t om = m0 + mt * 16u + kb * 4u + r;
@@ -188,25 +276,60 @@ __global__ __launch_bounds__(256) void k_prefill(const uint4v *__restrict__ qw, 
     }
 }
 
-hipError_t launch_prefill(hipStream_t s, const WeightView &w, const void *a, bool a_f32, uint32_t m, const OutSpec &out)
+// f32 activations are rounded to f16 (round-to-nearest-even, as the MFMA operand needs) into scratch first
+__global__ __launch_bounds__(256) void k_cvt_f32_f16(const float4 *__restrict__ src, uint2v *__restrict__ dst, size_t n4)
 {
-    if (m == 0 || w.n == 0) return hipSuccess;
+    size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n4) return;
+    float4 x = src[i];
+    union { half2v h[2]; uint2v u; } cv;
+    cv.h[0] = half2v{(_Float16)x.x, (_Float16)x.y};
+    cv.h[1] = half2v{(_Float16)x.z, (_Float16)x.w};
+    dst[i] = cv.u;
+}
+
+template <int MT>
+static hipError_t launch_prefill_t(hipStream_t s, const WeightView &w, const _Float16 *a, uint32_t m, const OutSpec &out)
+{
     static bool attr_set = false;
-    size_t lds = (size_t)2 * kPfTileHalves * sizeof(_Float16);
-    if (!attr_set) {
-        hipError_t e = hipFuncSetAttribute((const void *)k_prefill<true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-        if (e == hipSuccess)
-            e = hipFuncSetAttribute((const void *)k_prefill<false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    size_t lds = (size_t)2 * 16 * MT * kPfRowStride * sizeof(_Float16);
+    if (!attr_set && lds > 65536) {
+        hipError_t e = hipFuncSetAttribute((const void *)k_prefill<MT>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (e != hipSuccess) return e;
         attr_set = true;
     }
-    dim3 grid((w.n_tiles + 15) / 16, (m + kPfBM - 1) / kPfBM);
-    if (a_f32)
-        hipLaunchKernelGGL(k_prefill<true>, grid, dim3(256), lds, s, (const uint4v *)w.qw, (const uint2v *)w.sc, a, out, m,
-                           w.k, w.n, w.n_tiles, w.k_chunks);
-    else
-        hipLaunchKernelGGL(k_prefill<false>, grid, dim3(256), lds, s, (const uint4v *)w.qw, (const uint2v *)w.sc, a, out, m,
-                           w.k, w.n, w.n_tiles, w.k_chunks);
+    dim3 grid((w.n_tiles + 15) / 16, (m + 16 * MT - 1) / (16 * MT));
+    hipLaunchKernelGGL((k_prefill<MT>), grid, dim3(256), lds, s, (const uint4v *)w.qw, (const uint2v *)w.sc, a, out, m, w.k,
+                       w.n, w.n_tiles, w.k_chunks);
+    return hipGetLastError();
+}
+
+// block_rows: 64 or 128 rows of A per workgroup (0 = choose).  `scratch` (scratch_bytes) is only used for f32
+// activations; when it cannot hold all M rows as f16 the rows are processed in slabs.
+hipError_t launch_prefill(hipStream_t s, const WeightView &w, const void *a, bool a_f32, uint32_t m, const OutSpec &out,
+                          uint32_t block_rows, void *scratch, size_t scratch_bytes)
+{
+    if (m == 0 || w.n == 0) return hipSuccess;
+    if (block_rows == 0) block_rows = 128;
+    if (block_rows != 64 && block_rows != 128) return hipErrorInvalidValue;
+    auto run = [&](const _Float16 *a16, uint32_t rows, const OutSpec &o) {
+        return block_rows == 64 ? launch_prefill_t<4>(s, w, a16, rows, o) : launch_prefill_t<8>(s, w, a16, rows, o);
+    };
+    if (!a_f32) return run((const _Float16 *)a, m, out);
+    size_t row_bytes = (size_t)w.k * 2;
+    uint32_t slab = (uint32_t)(scratch_bytes / row_bytes < m ? scratch_bytes / row_bytes : m);
+    if (slab >= block_rows) slab -= slab % block_rows;
+    if (slab == 0 || !scratch) return hipErrorInvalidValue;
+    for (uint32_t r0 = 0; r0 < m; r0 += slab) {
+        uint32_t rows = m - r0 < slab ? m - r0 : slab;
+        size_t n4 = (size_t)rows * w.k / 4;  // k is a multiple of 32
+        hipLaunchKernelGGL(k_cvt_f32_f16, dim3((unsigned)((n4 + 255) / 256)), dim3(256), 0, s,
+                           (const float4 *)((const float *)a + (size_t)r0 * w.k), (uint2v *)scratch, n4);
+        OutSpec o = out;
+        for (uint32_t i = 0; i < o.count; i++) o.seg[i].ptr += (size_t)r0 * o.seg[i].width;
+        hipError_t e = run((const _Float16 *)scratch, rows, o);
+        if (e != hipSuccess) return e;
+    }
     return hipGetLastError();
 }
 

@@ -359,23 +359,30 @@ def test_m_larger_than_16_is_tiled_by_the_decode_kernel(dev):
     w.free()
 
 
-@pytest.mark.parametrize("m,k,n", [(33, 256, 128), (64, 896, 1152), (128, 1184, 200), (200, 4096, 704), (512, 4096, 1024)])
+@pytest.mark.parametrize("m,k,n", [(33, 256, 128), (40, 128, 64), (40, 384, 80), (70, 640, 64), (64, 896, 1152),
+                                   (128, 1184, 200), (200, 4096, 704), (512, 4096, 1024)])
 def test_prefill_kernel_matches_oracle(dev, m, k, n):
     # M > 32 runs the LDS/MFMA prefill kernel.  Its weights are the reference's FP16 Q4 unpack,
     # f16(scale*(q-8)) (quantize.rs:534-571), so its oracle is A x f16-dequant(W) in f64: tight match.
     # Against the f32-weight matmul the FP16 rounding of the weights (2^-12 relative each) shows on
     # near-cancelling outputs, so that comparison is made relative to the largest output.
-    # Ragged M (33, 200), K not a multiple of 128 (1184), N not a multiple of 256 / 64 (200, 704).
+    # Ragged M (33, 200), K not a multiple of 128 (1184), N not a multiple of 256 / 64 (200, 704); 1 to 5
+    # k-chunks (the k loop is unrolled by three with a remainder); both workgroup heights.
     packed, scales, a16 = synth(k, n, m, 4000 + m)
     w = T.MarlinWeight.upload(dev, packed, scales, k, n)
     a = f16_as_f32(a16)
     w16 = O.dequant_f16(packed, scales, k, n).view(np.float16).astype(np.float64)
     exact = a.astype(np.float64) @ w16
     truth = O.gemm_f64(a, packed, scales, m, k, n)
-    for a_f32 in (False, True):
-        got = run_gemm(dev, w, a16, m, n, a_f32=a_f32)
-        assert rel_err(got, exact) < 1e-3, a_f32          # one f32 accumulator over all of K: a few 1e-4 at K = 4096
-        assert np.abs(got - truth).max() / np.abs(truth).max() < 1e-3
+    try:
+        for bm in (64, 128):
+            dev.set_option("prefill_bm", bm)
+            for a_f32 in (False, True):
+                got = run_gemm(dev, w, a16, m, n, a_f32=a_f32)
+                assert rel_err(got, exact) < 1e-3, (bm, a_f32)   # one f32 accumulator over all of K: a few 1e-4 at K = 4096
+                assert np.abs(got - truth).max() / np.abs(truth).max() < 1e-3
+    finally:
+        dev.set_option("prefill_bm", 0)
     # the exact-weight decode blocks and the prefill kernel agree to the weight rounding
     try:
         dev.set_option("prefill_min_m", 1 << 30)
