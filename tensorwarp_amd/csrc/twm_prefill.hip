@@ -304,13 +304,17 @@ static hipError_t launch_prefill_t(hipStream_t s, const WeightView &w, const _Fl
     return hipGetLastError();
 }
 
-// block_rows: 64 or 128 rows of A per workgroup (0 = choose).  `scratch` (scratch_bytes) is only used for f32
+// block_rows: 64 or 128 rows of A per workgroup; 0 = choose: 128-row blocks unpack each weight for twice as
+// many rows and win once they fill the 256 CUs, below that 64-row blocks give twice the workgroups.  `scratch` (scratch_bytes) is only used for f32
 // activations; when it cannot hold all M rows as f16 the rows are processed in slabs.
 hipError_t launch_prefill(hipStream_t s, const WeightView &w, const void *a, bool a_f32, uint32_t m, const OutSpec &out,
                           uint32_t block_rows, void *scratch, size_t scratch_bytes)
 {
     if (m == 0 || w.n == 0) return hipSuccess;
-    if (block_rows == 0) block_rows = 128;
+    if (block_rows == 0) {
+        size_t wg128 = (size_t)((m + 127) / 128) * ((w.n_tiles + 15) / 16);
+        block_rows = wg128 >= 256 ? 128 : 64;
+    }
     if (block_rows != 64 && block_rows != 128) return hipErrorInvalidValue;
     auto run = [&](const _Float16 *a16, uint32_t rows, const OutSpec &o) {
         return block_rows == 64 ? launch_prefill_t<4>(s, w, a16, rows, o) : launch_prefill_t<8>(s, w, a16, rows, o);
