@@ -665,7 +665,7 @@ static int gemm_common(twm_ctx *ctx, const twm_weight *w, const void *a_dev, int
     size_t a_row_bytes = (size_t)w->k * (a_dtype == TWM_F16 ? 2 : 4);
     uint32_t n_ld = w->n_tiles * kTileN;
     if (m >= (uint32_t)ctx->prefill_min_m) {
-        HIP_TRY(launch_prefill(ctx->stream, v, a_dev, a_dtype == TWM_F32, m, out, (uint32_t)ctx->prefill_bm, ctx->ws, ctx->ws_bytes), TWM_DEVICE_ERROR, "prefill launch");
+        HIP_TRY(launch_prefill(ctx->stream, v, a_dev, a_dtype == TWM_F32, m, out, (uint32_t)ctx->prefill_bm, splits, ctx->ws, ctx->ws_bytes), TWM_DEVICE_ERROR, "prefill launch");
         return TWM_OK;
     }
     for (uint32_t m0 = 0; m0 < m; m0 += kMaxDecodeM) {

@@ -70,7 +70,7 @@ hipError_t launch_weight_dequant_f16_col(hipStream_t s, const WeightView &w, uin
 hipError_t launch_gemv4(hipStream_t s, const WeightView &w, const void *a, bool a_f32, uint32_t m, const OutSpec &out,
                         float *ws, unsigned *counters, uint32_t nt, uint32_t waves, uint32_t splits);
 hipError_t launch_prefill(hipStream_t s, const WeightView &w, const void *a, bool a_f32, uint32_t m, const OutSpec &out,
-                          uint32_t block_rows, void *scratch, size_t scratch_bytes);
+                          uint32_t block_rows, uint32_t splits, void *scratch, size_t scratch_bytes);
 hipError_t launch_decode(hipStream_t s, const WeightView &w, const void *a, bool a_f32, uint32_t m, const OutSpec &out,
                          float *ws, unsigned *counters, DecodePlan plan);
 

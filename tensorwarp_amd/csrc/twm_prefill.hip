@@ -81,7 +81,8 @@ __device__ __forceinline__ void pf_store_out(const OutSpec &out, uint32_t m, uin
 template <int MT>  // MT = 16-row blocks per workgroup tile (BM = 16 * MT rows)
 __global__ __launch_bounds__(256) void k_prefill(const uint4v *__restrict__ qw, const uint2v *__restrict__ sc,
                                                   const _Float16 *__restrict__ a_any, OutSpec out, uint32_t m_rows,
-                                                  uint32_t k, uint32_t n, uint32_t n_tiles, uint32_t k_chunks)
+                                                  uint32_t k, uint32_t n, uint32_t n_tiles, uint32_t k_chunks,
+                                                  uint32_t chunks_per_split, float *__restrict__ partials)
 {
     constexpr int kPfTileHalves = 16 * MT * kPfRowStride;
     constexpr int NV = MT;       // 16-byte vectors of A each thread stages per chunk (16 MT rows * 16 / 256)
@@ -94,7 +95,10 @@ __global__ __launch_bounds__(256) void k_prefill(const uint4v *__restrict__ qw, 
     const uint32_t c = lane & 15u, kb = lane >> 4;
     const uint32_t m0 = blockIdx.y * (16u * MT);
     const uint32_t nt0 = (blockIdx.x * 4u + wave) * 4u;  // first of this wave's four 16-column tiles
-    const uint32_t last = k_chunks - 1;
+    // split-K: blockIdx.z takes chunks [kc0, kc0 + nchunks); chunk indices below are relative to kc0
+    const uint32_t kc0 = blockIdx.z * chunks_per_split;
+    const uint32_t nchunks = k_chunks - kc0 < chunks_per_split ? k_chunks - kc0 : chunks_per_split;
+    const uint32_t last = nchunks - 1;
 
     const PfConsts dq = make_pf_consts();
 
@@ -136,8 +140,8 @@ __global__ __launch_bounds__(256) void k_prefill(const uint4v *__restrict__ qw, 
     const char *a_src;
     uint32_t a_back;
     auto aim_a = [&](uint32_t kc) {  // addresses of chunk kc
-        a_src = a_blk + (size_t)kc * 256u;
-        a_back = kc * 128u + vec * 8u < k ? 0u : vec * 16u;
+        a_src = a_blk + (size_t)(kc0 + kc) * 256u;
+        a_back = (kc0 + kc) * 128u + vec * 8u < k ? 0u : vec * 16u;
     };
     auto load_a = [&](int j) { a_stage[j] = *(const uint4v *)(a_src + (a_off[j] - a_back)); };
     const uint32_t wr_off = (threadIdx.x >> 4) * kPfRowStride + vec * 8u;
@@ -150,10 +154,10 @@ __global__ __launch_bounds__(256) void k_prefill(const uint4v *__restrict__ qw, 
     uint2v bs[3][4];
     const uint32_t q_off = lane * 16u, s_off = c * 8u;
     auto load_bq = [&](int slot, uint32_t kc, int t) {
-        bq[slot][t] = *(const TWM_GLOBAL uint4v *)(scalar_base(qw, (size_t)(kc * n_tiles + nt[t]) * 1024u) + q_off);
+        bq[slot][t] = *(const TWM_GLOBAL uint4v *)(scalar_base(qw, (size_t)((kc0 + kc) * n_tiles + nt[t]) * 1024u) + q_off);
     };
     auto load_bs = [&](int slot, uint32_t kc, int t) {
-        bs[slot][t] = *(const TWM_GLOBAL uint2v *)(scalar_base(sc, (size_t)(kc * n_tiles + nt[t]) * 128u) + s_off);
+        bs[slot][t] = *(const TWM_GLOBAL uint2v *)(scalar_base(sc, (size_t)((kc0 + kc) * n_tiles + nt[t]) * 128u) + s_off);
     };
     // half fragment hp (tile hp / 2, half hp % 2) of group g
     auto unpack = [&](int slot, int g, PfFrag (&bf)[4], int hp) {
@@ -252,15 +256,33 @@ __global__ __launch_bounds__(256) void k_prefill(const uint4v *__restrict__ qw, 
     __builtin_amdgcn_sched_barrier(0);
 
     uint32_t kc = 0;
-    for (; kc + 3 <= k_chunks; kc += 3) {
+    for (; kc + 3 <= nchunks; kc += 3) {
         chunk(S0{}, kc);
         chunk(S1{}, kc + 1);
         chunk(S2{}, kc + 2);
     }
-    if (kc < k_chunks) chunk(S0{}, kc);
-    if (kc + 1 < k_chunks) chunk(S1{}, kc + 1);
+    if (kc < nchunks) chunk(S0{}, kc);
+    if (kc + 1 < nchunks) chunk(S1{}, kc + 1);
 
     // ---- store: lane (c, kb) holds rows 4*kb + r of row block mt, column 16*tile + c ----
+    if (partials) {
+        // split-K: plain [split][row][padded column] partial sums, added up in split order by k_prefill_reduce
+        const uint32_t n_ld = n_tiles * 16u;
+        float *dst = partials + ((size_t)blockIdx.z * m_rows) * n_ld;
+#pragma unroll
+        for (int t = 0; t < 4; t++) {
+            if (nt0 + t >= n_tiles) continue;
+            uint32_t on = (nt0 + t) * 16u + c;
+#pragma unroll
+            for (int mt = 0; mt < MT; mt++)
+#pragma unroll
+                for (int r = 0; r < 4; r++) {
+                    uint32_t om = m0 + mt * 16u + kb * 4u + r;
+                    if (om < m_rows) dst[(size_t)om * n_ld + on] = acc[mt][t][r];
+                }
+        }
+        return;
+    }
 #pragma unroll
     for (int t = 0; t < 4; t++) {
         if (nt0 + t >= n_tiles) continue;
@@ -276,6 +298,27 @@ __global__ __launch_bounds__(256) void k_prefill(const uint4v *__restrict__ qw, 
     }
 }
 
+// out[row][col] = sum over splits, in split order (deterministic), of partials[split][row][col]
+__global__ __launch_bounds__(256) void k_prefill_reduce(const float *__restrict__ partials, OutSpec out, uint32_t m_rows, uint32_t n,
+                                                         uint32_t n_ld, uint32_t splits)
+{
+    size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;  // one thread per four padded columns
+    uint32_t quads = n_ld / 4;
+    if (idx >= (size_t)m_rows * quads) return;
+    uint32_t row = (uint32_t)(idx / quads), col = (uint32_t)(idx % quads) * 4u;
+    const float4 *src = (const float4 *)(partials + (size_t)row * n_ld + col);
+    size_t stride4 = (size_t)m_rows * n_ld / 4;
+    float4 s = src[0];
+    for (uint32_t z = 1; z < splits; z++) {
+        float4 v = src[z * stride4];
+        s.x += v.x; s.y += v.y; s.z += v.z; s.w += v.w;
+    }
+    if (col + 0 < n) pf_store_out(out, row, col + 0, s.x);
+    if (col + 1 < n) pf_store_out(out, row, col + 1, s.y);
+    if (col + 2 < n) pf_store_out(out, row, col + 2, s.z);
+    if (col + 3 < n) pf_store_out(out, row, col + 3, s.w);
+}
+
 // f32 activations are rounded to f16 (round-to-nearest-even, as the MFMA operand needs) into scratch first
 __global__ __launch_bounds__(256) void k_cvt_f32_f16(const float4 *__restrict__ src, uint2v *__restrict__ dst, size_t n4)
 {
@@ -289,7 +332,8 @@ __global__ __launch_bounds__(256) void k_cvt_f32_f16(const float4 *__restrict__ 
 }
 
 template <int MT>
-static hipError_t launch_prefill_t(hipStream_t s, const WeightView &w, const _Float16 *a, uint32_t m, const OutSpec &out)
+static hipError_t launch_prefill_t(hipStream_t s, const WeightView &w, const _Float16 *a, uint32_t m, const OutSpec &out,
+                                   uint32_t splits, float *partials)
 {
     static bool attr_set = false;
     size_t lds = (size_t)2 * 16 * MT * kPfRowStride * sizeof(_Float16);
@@ -298,17 +342,28 @@ static hipError_t launch_prefill_t(hipStream_t s, const WeightView &w, const _Fl
         if (e != hipSuccess) return e;
         attr_set = true;
     }
-    dim3 grid((w.n_tiles + 15) / 16, (m + 16 * MT - 1) / (16 * MT));
+    uint32_t cps = (w.k_chunks + splits - 1) / splits;
+    splits = (w.k_chunks + cps - 1) / cps;  // no empty split
+    dim3 grid((w.n_tiles + 15) / 16, (m + 16 * MT - 1) / (16 * MT), splits);
     hipLaunchKernelGGL((k_prefill<MT>), grid, dim3(256), lds, s, (const uint4v *)w.qw, (const uint2v *)w.sc, a, out, m, w.k,
-                       w.n, w.n_tiles, w.k_chunks);
+                       w.n, w.n_tiles, w.k_chunks, cps, splits > 1 ? partials : nullptr);
+    if (splits > 1) {
+        uint32_t n_ld = w.n_tiles * 16;
+        size_t quads = (size_t)m * n_ld / 4;
+        hipLaunchKernelGGL(k_prefill_reduce, dim3((unsigned)((quads + 255) / 256)), dim3(256), 0, s, partials, out, m, w.n, n_ld,
+                           splits);
+    }
     return hipGetLastError();
 }
 
 // block_rows: 64 or 128 rows of A per workgroup; 0 = choose: 128-row blocks unpack each weight for twice as
-// many rows and win once they fill the 256 CUs, below that 64-row blocks give twice the workgroups.  `scratch` (scratch_bytes) is only used for f32
-// activations; when it cannot hold all M rows as f16 the rows are processed in slabs.
+// many rows and win once they fill the 256 CUs, below that 64-row blocks give twice the workgroups.
+// splits: k-split factor, 0 = choose: when the grid leaves CUs idle, K is cut so that about 512 64-row
+// workgroups (two per CU) exist, within what `scratch` can hold as f32 partial sums.
+// `scratch` (scratch_bytes) holds the f16 copy of f32 activations and / or the split-K partials; when it
+// cannot hold all M rows the rows are processed in slabs.
 hipError_t launch_prefill(hipStream_t s, const WeightView &w, const void *a, bool a_f32, uint32_t m, const OutSpec &out,
-                          uint32_t block_rows, void *scratch, size_t scratch_bytes)
+                          uint32_t block_rows, uint32_t splits, void *scratch, size_t scratch_bytes)
 {
     if (m == 0 || w.n == 0) return hipSuccess;
     if (block_rows == 0) {
@@ -316,14 +371,29 @@ hipError_t launch_prefill(hipStream_t s, const WeightView &w, const void *a, boo
         block_rows = wg128 >= 256 ? 128 : 64;
     }
     if (block_rows != 64 && block_rows != 128) return hipErrorInvalidValue;
-    auto run = [&](const _Float16 *a16, uint32_t rows, const OutSpec &o) {
-        return block_rows == 64 ? launch_prefill_t<4>(s, w, a16, rows, o) : launch_prefill_t<8>(s, w, a16, rows, o);
+    const size_t n_ld = (size_t)w.n_tiles * 16;
+    auto run = [&](const _Float16 *a16, uint32_t rows, const OutSpec &o, void *ws, size_t ws_bytes) {
+        uint32_t sp = splits;
+        if (sp == 0) {
+            size_t wgs = (size_t)((rows + block_rows - 1) / block_rows) * ((w.n_tiles + 15) / 16);
+            size_t want = block_rows == 64 ? 512 : 256;
+            sp = (uint32_t)(want / wgs);
+            if (sp > w.k_chunks / 4) sp = w.k_chunks / 4;  // at least four chunks per split
+        }
+        size_t per_split = (size_t)rows * n_ld * 4;
+        if (!ws || per_split == 0) sp = 1;
+        else if (sp > ws_bytes / per_split) sp = (uint32_t)(ws_bytes / per_split);
+        if (sp < 2) sp = 1;
+        return block_rows == 64 ? launch_prefill_t<4>(s, w, a16, rows, o, sp, (float *)ws)
+                                : launch_prefill_t<8>(s, w, a16, rows, o, sp, (float *)ws);
     };
-    if (!a_f32) return run((const _Float16 *)a, m, out);
+    if (!a_f32) return run((const _Float16 *)a, m, out, scratch, scratch_bytes);
+    // f16 copy of the activations at the front of the scratch, partials behind it
     size_t row_bytes = (size_t)w.k * 2;
-    uint32_t slab = (uint32_t)(scratch_bytes / row_bytes < m ? scratch_bytes / row_bytes : m);
+    if (!scratch || scratch_bytes < row_bytes) return hipErrorInvalidValue;
+    uint32_t slab = (uint32_t)(scratch_bytes / 2 / row_bytes < m ? scratch_bytes / 2 / row_bytes : m);
+    if (slab == 0) slab = 1;
     if (slab >= block_rows) slab -= slab % block_rows;
-    if (slab == 0 || !scratch) return hipErrorInvalidValue;
     for (uint32_t r0 = 0; r0 < m; r0 += slab) {
         uint32_t rows = m - r0 < slab ? m - r0 : slab;
         size_t n4 = (size_t)rows * w.k / 4;  // k is a multiple of 32
@@ -331,7 +401,8 @@ hipError_t launch_prefill(hipStream_t s, const WeightView &w, const void *a, boo
                            (const float4 *)((const float *)a + (size_t)r0 * w.k), (uint2v *)scratch, n4);
         OutSpec o = out;
         for (uint32_t i = 0; i < o.count; i++) o.seg[i].ptr += (size_t)r0 * o.seg[i].width;
-        hipError_t e = run((const _Float16 *)scratch, rows, o);
+        size_t used = ((size_t)rows * row_bytes + 255) & ~(size_t)255;
+        hipError_t e = run((const _Float16 *)scratch, rows, o, (char *)scratch + used, scratch_bytes - used);
         if (e != hipSuccess) return e;
     }
     return hipGetLastError();

@@ -392,6 +392,33 @@ def test_prefill_kernel_matches_oracle(dev, m, k, n):
     w.free()
 
 
+@pytest.mark.parametrize("m,k,n", [(64, 4096, 704), (100, 1184, 200), (130, 2048, 320)])
+def test_prefill_split_k(dev, m, k, n):
+    # Few workgroups: K is cut across workgroups, f32 partial sums are added in split order by a second
+    # kernel.  Explicit factors (also ones that do not divide the chunk count, and more than there are
+    # chunks) and the automatic choice; f32 activations share the scratch with the partials.
+    packed, scales, a16 = synth(k, n, m, 5000 + m)
+    w = T.MarlinWeight.upload(dev, packed, scales, k, n)
+    a = f16_as_f32(a16)
+    w16 = O.dequant_f16(packed, scales, k, n).view(np.float16).astype(np.float64)
+    exact = a.astype(np.float64) @ w16
+    try:
+        for bm in (64, 128):
+            dev.set_option("prefill_bm", bm)
+            base = run_gemm(dev, w, a16, m, n, splits=1)
+            assert rel_err(base, exact) < 1e-3
+            for splits in (0, 2, 3, 7, 64):
+                for a_f32 in (False, True):
+                    got = run_gemm(dev, w, a16, m, n, splits=splits, a_f32=a_f32)
+                    assert rel_err(got, exact) < 1e-3, (bm, splits, a_f32)
+                    assert rel_err(got, base) < 1e-3, (bm, splits, a_f32)      # another summation order
+            again = run_gemm(dev, w, a16, m, n, splits=3)
+            assert np.array_equal(again, run_gemm(dev, w, a16, m, n, splits=3))   # no atomics: run-to-run identical
+    finally:
+        dev.set_option("prefill_bm", 0)
+    w.free()
+
+
 def test_empty_inputs(dev):
     w = T.MarlinWeight.upload(dev, np.zeros(0, np.uint8), np.zeros(0, np.uint16), 64, 0)
     c = T.GpuTensor.zeros(dev, (4,), "f32")
