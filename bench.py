@@ -10,7 +10,10 @@ captured once as a hipGraph (the reference captures all layers of a decode step 
 crates/kernels/src/generate.rs:2485-2536) and replayed; `config.us_per_layer_own_graph` is the
 same measurement with one graph per layer, which pays the graph-launch cost once per layer.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers L] [--no-cpu] [--extra]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers L] [--no-cpu] [--no-prefill] [--extra]
+
+`prefill` holds the W4A16 GEMM on the LLaMA-7B MLP shapes (BASELINE.json configs[4]) at M=512 and
+2048 as TFLOP/s against the 2.5 PFLOP/s dense FP16 MFMA peak; it is not part of `value`.
 
 Prints ONE JSON line. `value` = algorithmic bytes of a layer x K / time of K replays (inputs
 resident in HBM). `roofline` is for the dominant kernel, the gate_up GEMV, timed with HIP events
@@ -68,6 +71,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=40)
     ap.add_argument("--layers", type=int, default=4, help="distinct weight sets rotated through (>=3 defeats the 256 MB cache)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
+    ap.add_argument("--no-prefill", action="store_true", help="skip the prefill GEMM timings")
     ap.add_argument("--extra", action="store_true", help="also time batched decode (M=4..32) on the gate_up shape")
     ap.add_argument("--pmc-copy", action="store_true",
                     help="also run four 64 MiB device-to-device copies: a kernel of known traffic to scale rocprofv3 "
@@ -175,6 +179,30 @@ def main():
             extra["gate_up_M%d" % m] = {"us": round(ms * 1e3, 2), "GBps": round(b / (ms * 1e-3) / 1e9, 1),
                                         "frac_hbm": round(b / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
 
+    prefill = None
+    if not args.no_prefill:
+        prefill = {}
+        for k, n in ((4096, 11008), (11008, 4096)):
+            packed = rng.integers(0, 256, size=(k // 32) * n * 16, dtype=np.uint8)
+            scales = (np.abs(rng.standard_normal((k // 32) * n, dtype=np.float32)) * np.float32(0.02)).astype(np.float16)
+            w = T.MarlinWeight.upload(dev, packed, scales.view(np.uint16), k, n)
+            for m in (512, 2048):
+                a_m = T.GpuTensor.from_host(dev, rng.standard_normal((m, k), dtype=np.float32).astype(np.float16).view(np.uint16), "f16")
+                c_m = T.GpuTensor.zeros(dev, (m, n), "f32")
+
+                def one(i, w=w, a_m=a_m, c_m=c_m, m=m):
+                    T.gemm(dev, w, a_m, m, c_m)
+                for i in range(3):
+                    one(i)
+                dev.synchronize()
+                ms = time_launches(dev, one, 20)
+                tf = 2.0 * m * n * k / (ms * 1e-3) / 1e12
+                prefill["M%d_K%d_N%d" % (m, k, n)] = {"us": round(ms * 1e3, 1), "TFLOPs": round(tf, 1),
+                                                      "frac_mfma_f16_peak": round(tf / MFMA_F16_PEAK_TFLOPS, 4)}
+                a_m.free()
+                c_m.free()
+            w.free()
+
     cpu = None
     if not args.no_cpu:
         # the checker, timed: reference CPU semantics on layer 0, one thread, whole layer once
@@ -213,6 +241,8 @@ def main():
         "cpu_baseline": cpu,
         "per_projection": per_shape,
     }
+    if prefill:
+        out["prefill"] = prefill
     if extra:
         out["batched_decode"] = extra
     print(json.dumps(out))
