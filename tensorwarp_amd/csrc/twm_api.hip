@@ -99,7 +99,7 @@ twm_ctx *twm_ctx_create(int ordinal)
     c->force_kernel = 0;
     c->dequant_src = 0;
     c->prefill_bm = 0;
-    c->prefill_min_m = 33;  // M <= 32 is batched decode: exact f32 weights, weights re-read per 16-row block
+    c->prefill_min_m = 17;  // M <= 16 is batched decode (exact f32 scales); from 17 rows on the MFMA GEMM is faster
     c->ws = nullptr;
     c->counters = nullptr;
     c->own_stream = nullptr;

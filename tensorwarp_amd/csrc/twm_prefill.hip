@@ -1,4 +1,4 @@
-// Prefill kernel (M > 32): C[M,N] = A[M,K] * dequant(W), FP16 MFMA with FP32 accumulation.
+// Prefill kernel (M > 16): C[M,N] = A[M,K] * dequant(W), FP16 MFMA with FP32 accumulation.
 //
 // Semantics: gemm_q4_0 (crates/kernels/src/quantize.rs:1825-1858 / kernel :186-246 in the reference),
 // i.e. C[m][n] = sum_k A[m][k] * w[k][n].  Here w is the reference's Q4 unpack to FP16,
