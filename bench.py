@@ -73,6 +73,9 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--no-prefill", action="store_true", help="skip the prefill GEMM timings")
     ap.add_argument("--extra", action="store_true", help="also time batched decode (M=4..32) on the gate_up shape")
+    ap.add_argument("--sweep-splits", action="store_true",
+                    help="also time every projection at M=1,4,8,16,32 with forced split-K factors next to the library's "
+                         "own choice (BASELINE.json configs[3])")
     ap.add_argument("--pmc-copy", action="store_true",
                     help="also run four 64 MiB device-to-device copies: a kernel of known traffic to scale rocprofv3 "
                          "FETCH_SIZE / WRITE_SIZE readings by")
@@ -203,6 +206,26 @@ def main():
                 c_m.free()
             w.free()
 
+    sweep = None
+    if args.sweep_splits:
+        sweep = {}
+        for name, k, n in LAYER_7B:
+            for m in (1, 4, 8, 16, 32):
+                a_m = T.GpuTensor.from_host(dev, rng.standard_normal((m, k), dtype=np.float32).astype(np.float16).view(np.uint16), "f16")
+                c_m = T.GpuTensor.zeros(dev, (m, n), "f32")
+                row = {}
+                for sp in (0, 1, 2, 3, 4, 6, 8, 12, 16):
+                    def one(i, a_m=a_m, c_m=c_m, m=m, sp=sp, name=name):
+                        T.gemm(dev, layers[i % args.layers][name][0], a_m, m, c_m, sp)
+                    for i in range(8):
+                        one(i)
+                    dev.synchronize()
+                    row["auto" if sp == 0 else str(sp)] = round(time_launches(dev, one, 100) * 1e3, 2)
+                best = min((v, key) for key, v in row.items() if key != "auto")
+                sweep["%s_M%d" % (name, m)] = {"us": row, "auto_over_best": round(row["auto"] / best[0], 3), "best_splits": int(best[1])}
+                a_m.free()
+                c_m.free()
+
     cpu = None
     if not args.no_cpu:
         # the checker, timed: reference CPU semantics on layer 0, one thread, whole layer once
@@ -245,6 +268,8 @@ def main():
         out["prefill"] = prefill
     if extra:
         out["batched_decode"] = extra
+    if sweep:
+        out["split_sweep"] = sweep
     print(json.dumps(out))
     for g in graphs + [graph_all]:
         g.destroy()

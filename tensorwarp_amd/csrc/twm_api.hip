@@ -609,10 +609,12 @@ static DecodePlan plan_decode(uint32_t n_tiles, uint32_t k_chunks, uint32_t m, i
     while (p.waves < 16 && tg * p.waves < 3072 && k_chunks >= p.waves * 2) p.waves *= 2;
     if (force_waves) p.waves = (uint32_t)force_waves;
     while (p.waves > 4 && p.waves * p.nt > 64) p.waves /= 2;
-    // cross-workgroup splits: only when the tile groups alone leave CUs idle
+    // cross-workgroup splits: the partial tiles of this kernel are 16 rows deep, so parking and re-reading them
+    // costs more than idle CUs unless fewer than 128 workgroups exist (per-shape sweep: 224 tile groups of the
+    // 7B `down` run 15 us unsplit, 24 us with 4 splits)
     uint32_t sp = 1;
     uint32_t per_wg = p.waves * 2;  // keep >= 2 chunks per wave
-    while (tg * sp < 512 && (k_chunks / (sp * 2)) >= per_wg) sp *= 2;
+    while (tg * sp < 128 && (k_chunks / (sp * 2)) >= per_wg) sp *= 2;
     if (force_splits) sp = force_splits;
     if (sp > k_chunks) sp = k_chunks ? k_chunks : 1;
     p.splits = sp;

@@ -331,6 +331,31 @@ __global__ __launch_bounds__(256) void k_cvt_f32_f16(const float4 *__restrict__ 
     dst[i] = cv.u;
 }
 
+// Split-K factor by a small cost model fitted to per-shape sweeps on MI355X (microseconds):
+//   rounds * (chunks per split * t_chunk + t_start)  +  [split]  t_reduce + 2 * splits * partial bytes / 3 TB/s
+// t_chunk: 1.0 for 64-row blocks alone on a CU, 1.3 when two share it, 2.3 for 128-row blocks.
+static uint32_t pick_prefill_splits(uint32_t rows, uint32_t block_rows, uint32_t col_blocks, uint32_t k_chunks, size_t n_ld)
+{
+    const double wgs = (double)((rows + block_rows - 1) / block_rows) * col_blocks;
+    const double slots = block_rows == 128 ? 256.0 : 512.0;
+    const double partial_us = 2.0 * (double)rows * (double)n_ld * 4.0 / 3.0e6;  // write + read of one split's partials
+    uint32_t best = 1;
+    double best_t = 1e30;
+    for (uint32_t sp = 1; sp <= 64 && sp * 2 <= (k_chunks > 1 ? k_chunks : 2); sp++) {
+        uint32_t cps = (k_chunks + sp - 1) / sp;
+        if ((k_chunks + cps - 1) / cps != sp) continue;  // same work as a smaller factor
+        double total = wgs * sp;
+        double rounds = total <= slots ? 1.0 : (double)(uint64_t)((total + slots - 1) / slots);
+        double t_chunk = block_rows == 128 ? 2.3 : (total > 256.0 ? 1.3 : 1.0);
+        double t = rounds * (cps * t_chunk + 3.0) + (sp > 1 ? 3.0 + sp * partial_us : 0.0);
+        if (t < best_t * 0.97) {  // a larger factor has to pay for itself
+            best_t = t;
+            best = sp;
+        }
+    }
+    return best;
+}
+
 template <int MT>
 static hipError_t launch_prefill_t(hipStream_t s, const WeightView &w, const _Float16 *a, uint32_t m, const OutSpec &out,
                                    uint32_t splits, float *partials)
@@ -374,12 +399,7 @@ hipError_t launch_prefill(hipStream_t s, const WeightView &w, const void *a, boo
     const size_t n_ld = (size_t)w.n_tiles * 16;
     auto run = [&](const _Float16 *a16, uint32_t rows, const OutSpec &o, void *ws, size_t ws_bytes) {
         uint32_t sp = splits;
-        if (sp == 0) {
-            size_t wgs = (size_t)((rows + block_rows - 1) / block_rows) * ((w.n_tiles + 15) / 16);
-            size_t want = block_rows == 64 ? 512 : 256;
-            sp = (uint32_t)(want / wgs);
-            if (sp > w.k_chunks / 4) sp = w.k_chunks / 4;  // at least four chunks per split
-        }
+        if (sp == 0) sp = pick_prefill_splits(rows, block_rows, (w.n_tiles + 15) / 16, w.k_chunks, n_ld);
         size_t per_split = (size_t)rows * n_ld * 4;
         if (!ws || per_split == 0) sp = 1;
         else if (sp > ws_bytes / per_split) sp = (uint32_t)(ws_bytes / per_split);
