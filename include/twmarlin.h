@@ -86,10 +86,11 @@ int twm_ctx_info(twm_ctx *ctx, char *buf, size_t buf_len);
 /* Tuning knobs for per-shape sweeps (the role AutoTuner::tune_gemm plays in
  * crates/kernels/src/autotune.rs:254-396); 0 = library's choice unless noted:
  *   "nt"            column tiles per workgroup of the decode kernels (1, 2, 4)
- *   "waves"         waves per workgroup of the decode kernels (1, 2, 4, 8, 16)
- *   "kernel"        decode kernel: 1 = 16x16x32 tile kernel, 2 = one-lane-per-column kernel (M <= 4 only)
+ *   "waves"         waves per workgroup of the decode kernels (1, 2, 4, 8, 16; streaming kernel 4 or 8)
+ *   "kernel"        decode kernel: 1 = 16x16x32 tile kernel (16-row blocks), 2 = one-lane-per-column kernel
+ *                   (M <= 4 only), 3 = batched-decode streaming kernel (32-row blocks)
  *   "dequant_src"   which repacked copy twm_weight_dequant_f16 unpacks: 0 = 16-column tiles, 1 = column lanes
- *   "prefill_min_m" smallest M that runs the prefill GEMM (default 17; below it the decode kernels run)
+ *   "prefill_min_m" smallest M that runs the prefill GEMM (default 33; below it the decode kernels run)
  *   "prefill_bm"    rows of A per prefill workgroup (64 or 128)
  * Values outside these sets return TWM_SHAPE_ERROR, unknown keys TWM_UNSUPPORTED_OP. */
 int twm_ctx_set_option(twm_ctx *ctx, const char *key, int value);
@@ -182,8 +183,9 @@ int twm_weight_dequant_f16(twm_ctx *ctx, const twm_weight *w, uint16_t *out_kn_d
 /* C[M,N] (f32, row-major) = A[M,K] (f16 or f32, row-major) * dequant(W), f32 accumulation.
  * M = 1 is gemm_tw_marlin_m1 (quantize.rs:1301); M > 1 has the semantics of gemm_q4_0
  * (quantize.rs:1825-1858).  splits = 0 lets the library choose (twm_pick_splits).
- * M <= 16: decode kernels, weights exact, each group's f32 sum scaled by f32(scale).
- * M  > 16: prefill GEMM; weights are the reference's FP16 Q4 unpack, f16(scale * (q - 8)), as in
+ * M <= 32: decode kernels (M <= 4 one lane per column, M = 5..32 streaming tiles), weights exact,
+ *          each group's f32 sum scaled by f32(scale).
+ * M  > 32: prefill GEMM; weights are the reference's FP16 Q4 unpack, f16(scale * (q - 8)), as in
  * its dequant-then-matmul prefill route; f32 activations are rounded to f16 first.  Uses the
  * context's scratch: one context must not run two calls at the same time. */
 int twm_gemm(twm_ctx *ctx, const twm_weight *w, const void *a_dev, int a_dtype, uint32_t m,

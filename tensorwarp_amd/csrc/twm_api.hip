@@ -44,7 +44,7 @@ struct twm_ctx {
     bool capturing;
     int force_nt;         // 0 = heuristic
     int force_waves;      // 0 = heuristic
-    int force_kernel;     // 0 = heuristic, 1 = 16-column tile kernel, 2 = one-lane-per-column kernel (M <= 4)
+    int force_kernel;     // 0 = heuristic, 1 = 16-column tile kernel, 2 = one-lane-per-column kernel (M <= 4), 3 = streaming kernel (M <= 32)
     int prefill_bm;       // rows of A per prefill workgroup: 0 = choose, 64 or 128
     int prefill_min_m;    // M from which the LDS/MFMA prefill kernel runs instead of 16-row decode blocks
     int dequant_src;      // which copy twm_weight_dequant_f16 unpacks: 0 = 16-column tiles, 1 = column-lane
@@ -99,7 +99,7 @@ twm_ctx *twm_ctx_create(int ordinal)
     c->force_kernel = 0;
     c->dequant_src = 0;
     c->prefill_bm = 0;
-    c->prefill_min_m = 17;  // M <= 16 is batched decode (exact f32 scales); from 17 rows on the MFMA GEMM is faster
+    c->prefill_min_m = 33;  // M <= 32 is batched decode (exact f32 scales, weights streamed once)
     c->ws = nullptr;
     c->counters = nullptr;
     c->own_stream = nullptr;
@@ -200,7 +200,7 @@ int twm_ctx_set_option(twm_ctx *ctx, const char *key, int value)
         return TWM_OK;
     }
     if (strcmp(key, "kernel") == 0) {
-        if (value < 0 || value > 2) return fail(TWM_SHAPE_ERROR, "twm_ctx_set_option: kernel must be 0, 1 or 2");
+        if (value < 0 || value > 3) return fail(TWM_SHAPE_ERROR, "twm_ctx_set_option: kernel must be 0, 1, 2 or 3");
         ctx->force_kernel = value;
         return TWM_OK;
     }
@@ -643,12 +643,34 @@ static DecodePlan plan_gemv4(uint32_t n_tiles, uint32_t k_chunks, int force_nt, 
     return p;
 }
 
+// Batched-decode streaming kernel (M = 5 .. 32): one workgroup of eight waves per 64 columns and k-range.  K is
+// cut when the column quads alone leave CUs idle, up to about one workgroup per CU, keeping two chunks per
+// wave (one for the 32-row variant, whose chunks cost twice the arithmetic); the partial sums cost a second
+// kernel.  Fitted to the per-shape sweep (bench.py --sweep-splits).
+static uint32_t plan_stream(uint32_t n_tiles, uint32_t k_chunks, uint32_t m)
+{
+    uint32_t quads = n_tiles / 4;
+    if (quads == 0 || quads >= 256) return 1;
+    uint32_t sp = 256 / quads;
+    uint32_t cap = k_chunks / (m > 16 ? 8 : 16);
+    if (sp > cap) sp = cap;
+    return sp < 2 ? 1 : sp;
+}
+
+// Waves per workgroup of the streaming kernel: eight, except that the 32-row variant (158 registers) fits
+// only one eight-wave workgroup per CU, so with many column quads four-wave workgroups fill the CUs better.
+static uint32_t stream_waves(uint32_t n_tiles, uint32_t m, int force_waves)
+{
+    if (force_waves == 4 || force_waves == 8) return (uint32_t)force_waves;
+    return (m > 16 && n_tiles / 4 >= 256) ? 4 : 8;
+}
+
 uint32_t twm_pick_splits(uint32_t k, uint32_t n, uint32_t m)
 {
     uint32_t n_tiles = ((n + kNPadTo - 1) / kNPadTo) * kNPadTo / kTileN;
     uint32_t k_chunks = (k / 32 + kChunkGroups - 1) / kChunkGroups;
     if (m <= 4) return plan_gemv4(n_tiles, k_chunks, 0, 0, 0).splits;
-    return plan_decode(n_tiles, k_chunks, m > kMaxDecodeM ? kMaxDecodeM : m, 0, 0, 0).splits;
+    return plan_stream(n_tiles, k_chunks, m);
 }
 
 static int gemm_common(twm_ctx *ctx, const twm_weight *w, const void *a_dev, int a_dtype, uint32_t m, const OutSpec &out,
@@ -668,6 +690,19 @@ static int gemm_common(twm_ctx *ctx, const twm_weight *w, const void *a_dev, int
     uint32_t n_ld = w->n_tiles * kTileN;
     if (m >= (uint32_t)ctx->prefill_min_m) {
         HIP_TRY(launch_prefill(ctx->stream, v, a_dev, a_dtype == TWM_F32, m, out, (uint32_t)ctx->prefill_bm, splits, ctx->ws, ctx->ws_bytes), TWM_DEVICE_ERROR, "prefill launch");
+        return TWM_OK;
+    }
+    if (ctx->force_kernel == 3 || (ctx->force_kernel == 0 && m > 4)) {
+        // batched decode: 32-row blocks of the streaming kernel
+        for (uint32_t m0 = 0; m0 < m; m0 += kMaxStreamM) {
+            uint32_t mb = m - m0 < (uint32_t)kMaxStreamM ? m - m0 : (uint32_t)kMaxStreamM;
+            OutSpec o = out;
+            for (uint32_t s = 0; s < o.count; s++) o.seg[s].ptr += (size_t)m0 * o.seg[s].width;
+            const char *a_blk = (const char *)a_dev + (size_t)m0 * a_row_bytes;
+            HIP_TRY(launch_stream(ctx->stream, v, a_blk, a_dtype == TWM_F32, mb, o, splits ? splits : plan_stream(w->n_tiles, w->k_chunks, mb),
+                                  stream_waves(w->n_tiles, mb, ctx->force_waves), ctx->ws, ctx->ws_bytes),
+                    TWM_DEVICE_ERROR, "batched decode launch");
+        }
         return TWM_OK;
     }
     for (uint32_t m0 = 0; m0 < m; m0 += kMaxDecodeM) {

@@ -20,6 +20,7 @@ constexpr int kChunkGroups = 4;
 constexpr int kNPadTo = 64;      // N is padded to a multiple of this, so 1, 2 or 4 tiles per block divide
 constexpr int kMaxSegs = 4;
 constexpr int kMaxDecodeM = 16;     // rows per launch of the tile kernel (one 16-row MFMA block)
+constexpr int kMaxStreamM = 32;     // rows per launch of the batched-decode streaming kernel
 constexpr uint32_t kColBlockBytes = 4608;  // column-lane copy: 4 x 1024 B of nibbles + 512 B of scales per (tile, chunk)
 
 struct OutSeg {
@@ -71,6 +72,11 @@ hipError_t launch_gemv4(hipStream_t s, const WeightView &w, const void *a, bool 
                         float *ws, unsigned *counters, uint32_t nt, uint32_t waves, uint32_t splits);
 hipError_t launch_prefill(hipStream_t s, const WeightView &w, const void *a, bool a_f32, uint32_t m, const OutSpec &out,
                           uint32_t block_rows, uint32_t splits, void *scratch, size_t scratch_bytes);
+// out[row][col] = sum over splits (in order) of partials[split][row][col], partials rows n_ld floats wide
+hipError_t launch_splitk_reduce(hipStream_t s, const float *partials, const OutSpec &out, uint32_t m, uint32_t n,
+                                uint32_t n_ld, uint32_t splits);
+hipError_t launch_stream(hipStream_t s, const WeightView &w, const void *a, bool a_f32, uint32_t m, const OutSpec &out,
+                         uint32_t splits, uint32_t waves, float *partials, size_t partial_bytes);
 hipError_t launch_decode(hipStream_t s, const WeightView &w, const void *a, bool a_f32, uint32_t m, const OutSpec &out,
                          float *ws, unsigned *counters, DecodePlan plan);
 

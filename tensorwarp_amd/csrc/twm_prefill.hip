@@ -1,4 +1,4 @@
-// Prefill kernel (M > 16): C[M,N] = A[M,K] * dequant(W), FP16 MFMA with FP32 accumulation.
+// Prefill kernel (M > 32): C[M,N] = A[M,K] * dequant(W), FP16 MFMA with FP32 accumulation.
 //
 // Semantics: gemm_q4_0 (crates/kernels/src/quantize.rs:1825-1858 / kernel :186-246 in the reference),
 // i.e. C[m][n] = sum_k A[m][k] * w[k][n].  Here w is the reference's Q4 unpack to FP16,
@@ -266,7 +266,7 @@ __global__ __launch_bounds__(256) void k_prefill(const uint4v *__restrict__ qw, 
 
     // ---- store: lane (c, kb) holds rows 4*kb + r of row block mt, column 16*tile + c ----
     if (partials) {
-        // split-K: plain [split][row][padded column] partial sums, added up in split order by k_prefill_reduce
+        // split-K: plain [split][row][padded column] partial sums, added up in split order by k_splitk_reduce
         const uint32_t n_ld = n_tiles * 16u;
         float *dst = partials + ((size_t)blockIdx.z * m_rows) * n_ld;
 #pragma unroll
@@ -299,7 +299,7 @@ __global__ __launch_bounds__(256) void k_prefill(const uint4v *__restrict__ qw, 
 }
 
 // out[row][col] = sum over splits, in split order (deterministic), of partials[split][row][col]
-__global__ __launch_bounds__(256) void k_prefill_reduce(const float *__restrict__ partials, OutSpec out, uint32_t m_rows, uint32_t n,
+__global__ __launch_bounds__(256) void k_splitk_reduce(const float *__restrict__ partials, OutSpec out, uint32_t m_rows, uint32_t n,
                                                          uint32_t n_ld, uint32_t splits)
 {
     size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;  // one thread per four padded columns
@@ -329,6 +329,16 @@ __global__ __launch_bounds__(256) void k_cvt_f32_f16(const float4 *__restrict__ 
     cv.h[0] = half2v{(_Float16)x.x, (_Float16)x.y};
     cv.h[1] = half2v{(_Float16)x.z, (_Float16)x.w};
     dst[i] = cv.u;
+}
+
+hipError_t launch_splitk_reduce(hipStream_t s, const float *partials, const OutSpec &out, uint32_t m, uint32_t n,
+                                uint32_t n_ld, uint32_t splits)
+{
+    size_t quads = (size_t)m * n_ld / 4;
+    if (quads == 0) return hipSuccess;
+    hipLaunchKernelGGL(k_splitk_reduce, dim3((unsigned)((quads + 255) / 256)), dim3(256), 0, s, partials, out, m, n, n_ld,
+                       splits);
+    return hipGetLastError();
 }
 
 // Split-K factor by a small cost model fitted to per-shape sweeps on MI355X (microseconds):
@@ -372,12 +382,7 @@ static hipError_t launch_prefill_t(hipStream_t s, const WeightView &w, const _Fl
     dim3 grid((w.n_tiles + 15) / 16, (m + 16 * MT - 1) / (16 * MT), splits);
     hipLaunchKernelGGL((k_prefill<MT>), grid, dim3(256), lds, s, (const uint4v *)w.qw, (const uint2v *)w.sc, a, out, m, w.k,
                        w.n, w.n_tiles, w.k_chunks, cps, splits > 1 ? partials : nullptr);
-    if (splits > 1) {
-        uint32_t n_ld = w.n_tiles * 16;
-        size_t quads = (size_t)m * n_ld / 4;
-        hipLaunchKernelGGL(k_prefill_reduce, dim3((unsigned)((quads + 255) / 256)), dim3(256), 0, s, partials, out, m, w.n, n_ld,
-                           splits);
-    }
+    if (splits > 1) return launch_splitk_reduce(s, partials, out, m, w.n, w.n_tiles * 16, splits);
     return hipGetLastError();
 }
 

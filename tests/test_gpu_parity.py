@@ -50,10 +50,10 @@ def f16_as_f32(bits):
 
 def gemm_truth(a16, packed, scales, m, k, n):
     """f64 dequant-then-matmul the library's default path is held to: exact weights f32(scale)*(q-8) up to
-    M = 16 (decode kernels); from M = 17 on the FP16 Q4 unpack f16(scale*(q-8)) (prefill GEMM), which is
+    M = 32 (decode kernels); from M = 33 on the FP16 Q4 unpack f16(scale*(q-8)) (prefill GEMM), which is
     the reference's prefill route (quantize.rs:534-571 then an FP16 GEMM)."""
     a = f16_as_f32(a16).reshape(m, k)
-    if m <= 16:
+    if m <= 32:
         return O.gemm_f64(a, packed, scales, m, k, n)
     w16 = O.dequant_f16(packed, scales, k, n).view(np.float16).astype(np.float64).reshape(k, n)
     return a.astype(np.float64) @ w16
@@ -227,10 +227,10 @@ def test_gemm_matches_golden(dev, name):
     w = T.MarlinWeight.upload(dev, d["packed"], d["scales"], k, n)
     for a_f32 in (False, True):
         got = run_gemm(dev, w, d["a_f16"], m, n, a_f32=a_f32)
-        if m <= 16:
+        if m <= 32:
             assert rel_err(got, d["c_f64"]) < TIGHT, (name, a_f32)
         else:
-            # M > 16 runs the MFMA GEMM on the FP16 Q4 unpack (the fixture's dequant_f16), like the reference's
+            # M > 32 runs the MFMA GEMM on the FP16 Q4 unpack (the fixture's dequant_f16), like the reference's
             # dequant-then-matmul; against the f32-weight result the weight rounding (2^-12 each) shows
             w16 = d["dequant_f16"].view(np.float16).astype(np.float64).reshape(k, n)
             exact = f16_as_f32(d["a_f16"]).astype(np.float64).reshape(m, k) @ w16
@@ -297,10 +297,7 @@ def test_batched_decode_7b_shapes(dev, m, k, n):
     # summation order, so agreement is to f32 rounding, not bitwise; M = 32 also differs by the
     # FP16 rounding of the weights, 2^-12 each, which shows relative to the largest output)
     alone = run_gemm(dev, w, a16[m - 1:m], 1, n)
-    if m <= 16:
-        assert rel_err(alone[0], got[m - 1]) < TIGHT
-    else:
-        assert np.abs(alone[0] - got[m - 1]).max() / np.abs(alone[0]).max() < 1e-3
+    assert rel_err(alone[0], got[m - 1]) < TIGHT
     w.free()
 
 
@@ -358,15 +355,16 @@ def test_decode_kernels_rows_and_f32_activations(dev, m):
     w = T.MarlinWeight.upload(dev, packed, scales, k, n)
     truth = O.gemm_f64(f16_as_f32(a16), packed, scales, m, k, n)
     try:
-        dev.set_option("prefill_min_m", 1 << 30)      # M = 17..32 as two 16-row blocks of the decode kernel
-        for kernel in ((1, 2) if m <= 4 else (1,)):
+        dev.set_option("prefill_min_m", 1 << 30)
+        # 1 = 16-column tile kernel (16-row blocks), 2 = one lane per column (M <= 4), 3 = streaming kernel (32-row blocks)
+        for kernel in ((1, 2, 3) if m <= 4 else (1, 3)):
             dev.set_option("kernel", kernel)
             for splits in (0, 1, 2, 3):
                 for a_f32 in (False, True):
                     assert rel_err(run_gemm(dev, w, a16, m, n, splits, a_f32), truth) < TIGHT, (kernel, splits, a_f32)
     finally:
         dev.set_option("kernel", 0)
-        dev.set_option("prefill_min_m", 17)
+        dev.set_option("prefill_min_m", 33)
     w.free()
 
 
@@ -380,14 +378,14 @@ def test_m_larger_than_16_is_tiled_by_the_decode_kernel(dev):
         dev.set_option("prefill_min_m", 1 << 30)
         assert rel_err(run_gemm(dev, w, a16, m, n), truth) < TIGHT
     finally:
-        dev.set_option("prefill_min_m", 17)
+        dev.set_option("prefill_min_m", 33)
     w.free()
 
 
 @pytest.mark.parametrize("m,k,n", [(17, 256, 128), (32, 3584, 512), (33, 256, 128), (40, 128, 64), (40, 384, 80), (70, 640, 64), (64, 896, 1152),
                                    (128, 1184, 200), (200, 4096, 704), (512, 4096, 1024)])
 def test_prefill_kernel_matches_oracle(dev, m, k, n):
-    # M > 16 runs the LDS/MFMA prefill kernel.  Its weights are the reference's FP16 Q4 unpack,
+    # M > 32 runs the LDS/MFMA prefill kernel (here forced for every M).  Its weights are the reference's FP16 Q4 unpack,
     # f16(scale*(q-8)) (quantize.rs:534-571), so its oracle is A x f16-dequant(W) in f64: tight match.
     # Against the f32-weight matmul the FP16 rounding of the weights (2^-12 relative each) shows on
     # near-cancelling outputs, so that comparison is made relative to the largest output.
@@ -400,6 +398,7 @@ def test_prefill_kernel_matches_oracle(dev, m, k, n):
     exact = a.astype(np.float64) @ w16
     truth = O.gemm_f64(a, packed, scales, m, k, n)
     try:
+        dev.set_option("prefill_min_m", 1)
         for bm in (64, 128):
             dev.set_option("prefill_bm", bm)
             for a_f32 in (False, True):
@@ -408,12 +407,13 @@ def test_prefill_kernel_matches_oracle(dev, m, k, n):
                 assert np.abs(got - truth).max() / np.abs(truth).max() < 1e-3
     finally:
         dev.set_option("prefill_bm", 0)
+        dev.set_option("prefill_min_m", 33)
     # the exact-weight decode blocks and the prefill kernel agree to the weight rounding
     try:
         dev.set_option("prefill_min_m", 1 << 30)
         assert rel_err(run_gemm(dev, w, a16, m, n), truth) < TIGHT
     finally:
-        dev.set_option("prefill_min_m", 17)
+        dev.set_option("prefill_min_m", 33)
     w.free()
 
 
