@@ -508,6 +508,30 @@ def test_fused_qkv_and_gate_up_equal_separate_projections(dev):
         T.gemm_split(dev, rp["gate_up"], a3d, 3, [g, u], [ffn, ffn - 1])
 
 
+@pytest.mark.parametrize("m", [12, 24, 40, 130])
+def test_gemm_split_batched_and_prefill_rows(dev, m):
+    # segment stores of the streaming kernel (M = 12, 24), of the MFMA GEMM (M = 40, 130) and of the
+    # split-K reduce kernel: gemm_split equals slicing the fused result, bit for bit, for every split factor
+    k, ns = 1184, [96, 40, 168]
+    n = sum(ns)
+    packed, scales, a16 = synth(k, n, m, 7000 + m)
+    w = T.MarlinWeight.upload(dev, packed, scales, k, n)
+    a_dev = T.GpuTensor.from_host(dev, a16, "f16")
+    truth = gemm_truth(a16, packed, scales, m, k, n)
+    for splits in (0, 1, 3):
+        whole = T.GpuTensor.from_host(dev, np.full((m, n), np.nan, np.float32))
+        T.gemm(dev, w, a_dev, m, whole, splits)
+        got = whole.to_host()
+        assert rel_err(got, truth) < TIGHT, splits
+        parts = [T.GpuTensor.from_host(dev, np.full((m, ni), np.nan, np.float32)) for ni in ns]
+        T.gemm_split(dev, w, a_dev, m, parts, ns, splits)
+        off = 0
+        for pt, ni in zip(parts, ns):
+            assert np.array_equal(pt.to_host(), got[:, off:off + ni]), (splits, off)
+            off += ni
+    w.free()
+
+
 # ---------------------------------------------------------------- graph capture / replay
 
 def test_layer_graph_replays_match_eager(dev):
