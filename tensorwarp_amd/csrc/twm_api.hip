@@ -111,6 +111,7 @@ twm_ctx *twm_ctx_create(int ordinal)
         return nullptr;
     }
     ok = ok && hipStreamCreateWithFlags(&c->own_stream, hipStreamNonBlocking) == hipSuccess;
+    ok = ok && init_prefill() == hipSuccess;
     c->stream = c->own_stream;
     c->ws_bytes = kWsBytes;
     c->n_counters = kCounters;

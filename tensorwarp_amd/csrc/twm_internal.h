@@ -70,6 +70,7 @@ hipError_t launch_repack_col(hipStream_t s, const uint8_t *packed, const uint16_
 hipError_t launch_weight_dequant_f16_col(hipStream_t s, const WeightView &w, uint16_t *out_kn);
 hipError_t launch_gemv4(hipStream_t s, const WeightView &w, const void *a, bool a_f32, uint32_t m, const OutSpec &out,
                         float *ws, unsigned *counters, uint32_t nt, uint32_t waves, uint32_t splits);
+hipError_t init_prefill();
 hipError_t launch_prefill(hipStream_t s, const WeightView &w, const void *a, bool a_f32, uint32_t m, const OutSpec &out,
                           uint32_t block_rows, uint32_t splits, void *scratch, size_t scratch_bytes);
 // out[row][col] = sum over splits (in order) of partials[split][row][col], partials rows n_ld floats wide

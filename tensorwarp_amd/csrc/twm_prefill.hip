@@ -370,13 +370,7 @@ template <int MT>
 static hipError_t launch_prefill_t(hipStream_t s, const WeightView &w, const _Float16 *a, uint32_t m, const OutSpec &out,
                                    uint32_t splits, float *partials)
 {
-    static bool attr_set = false;
     size_t lds = (size_t)2 * 16 * MT * kPfRowStride * sizeof(_Float16);
-    if (!attr_set && lds > 65536) {
-        hipError_t e = hipFuncSetAttribute((const void *)k_prefill<MT>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-        if (e != hipSuccess) return e;
-        attr_set = true;
-    }
     uint32_t cps = (w.k_chunks + splits - 1) / splits;
     splits = (w.k_chunks + cps - 1) / cps;  // no empty split
     dim3 grid((w.n_tiles + 15) / 16, (m + 16 * MT - 1) / (16 * MT), splits);
@@ -384,6 +378,13 @@ static hipError_t launch_prefill_t(hipStream_t s, const WeightView &w, const _Fl
                        w.n, w.n_tiles, w.k_chunks, cps, splits > 1 ? partials : nullptr);
     if (splits > 1) return launch_splitk_reduce(s, partials, out, m, w.n, w.n_tiles * 16, splits);
     return hipGetLastError();
+}
+
+// Once per device, outside any stream capture: the 128-row variant needs 68 KB of dynamic LDS.
+hipError_t init_prefill()
+{
+    return hipFuncSetAttribute((const void *)k_prefill<8>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                               2 * 16 * 8 * kPfRowStride * (int)sizeof(_Float16));
 }
 
 // block_rows: 64 or 128 rows of A per workgroup; 0 = choose: 128-row blocks unpack each weight for twice as

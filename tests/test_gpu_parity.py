@@ -564,3 +564,43 @@ def test_layer_graph_replays_match_eager(dev):
         T.gemm(dev, ws["down"], acts["down"], 1, outs["down"], 7)      # eager work between replays
         dev.synchronize()
     graph.destroy()
+
+
+def test_graph_of_batched_and_prefill_launches():
+    # The multi-kernel paths (f32 -> f16 conversion, split-K partials + ordered reduce) captured in a graph
+    # as their FIRST use in a fresh context, then replayed with eager work in between; every replay must
+    # reproduce the eager result bit for bit (no memset nodes, no allocation, deterministic sums).
+    with T.WarpDevice(0) as d:
+        k, n = 2048, 320
+        packed, scales, a16 = synth(k, n, 130, 8100)
+        w = T.MarlinWeight.upload(d, packed, scales, k, n)
+        cases = []
+        for m, a_f32, splits in ((12, False, 3), (24, True, 0), (40, True, 2), (130, False, 0)):
+            bits = a16[:m]
+            a_dev = T.GpuTensor.from_host(d, f16_as_f32(bits)) if a_f32 else T.GpuTensor.from_host(d, bits, "f16")
+            cases.append((m, a_dev, T.GpuTensor.zeros(d, (m, n), "f32"), splits, bits))
+
+        def body():
+            for m, a_dev, c, splits, _ in cases:
+                T.gemm(d, w, a_dev, m, c, splits)
+
+        graph = T.GraphCapture.record_with_device(d, body)
+        graph.replay()
+        d.synchronize()
+        first = [c.to_host() for _, _, c, _, _ in cases]
+        for (m, _, _, _, bits), got in zip(cases, first):
+            assert rel_err(got, gemm_truth(bits, packed, scales, m, k, n)) < TIGHT, m
+        for rep in range(3):
+            for _, _, c, _, _ in cases:
+                c.copy_from_host(np.full(c.shape, np.nan, np.float32))
+            body()                                   # eager, between replays
+            d.synchronize()
+            for (_, _, c, _, _), want in zip(cases, first):
+                assert np.array_equal(c.to_host(), want), ("eager", rep)
+                c.copy_from_host(np.full(c.shape, np.nan, np.float32))
+            graph.replay()
+            d.synchronize()
+            for (_, _, c, _, _), want in zip(cases, first):
+                assert np.array_equal(c.to_host(), want), ("replay", rep)
+        graph.destroy()
+        w.free()
