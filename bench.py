@@ -12,7 +12,8 @@ same measurement with one graph per layer, which pays the graph-launch cost once
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers L] [--no-cpu] [--no-prefill] [--extra]
 
-`prefill` holds the W4A16 GEMM on the LLaMA-7B MLP shapes (BASELINE.json configs[4]) at M=512 and
+`small_shapes_m1` holds the launch-bound configurations (BASELINE.json configs[0] and [1]: 4096->4096 and
+the Qwen-0.5B layer) per projection and as a graph, `prefill` the W4A16 GEMM on the LLaMA-7B MLP shapes (BASELINE.json configs[4]) at M=512 and
 2048 as TFLOP/s against the 2.5 PFLOP/s dense FP16 MFMA peak; it is not part of `value`.
 
 Prints ONE JSON line. `value` = algorithmic bytes of a layer x K / time of K replays (inputs
@@ -31,6 +32,8 @@ HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X dense FP16 matrix, published
 
 LAYER_7B = [("qkv", 3584, 4608), ("o", 3584, 3584), ("gate_up", 3584, 37888), ("down", 18944, 3584)]
+LAYER_05B = [("qkv", 896, 1152), ("o", 896, 896), ("gate_up", 896, 9728), ("down", 4864, 896)]   # BASELINE.json configs[1]
+CFG0 = [("cfg0", 4096, 4096)]                                                                     # BASELINE.json configs[0]
 # HBM bytes per gate_up launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, each scaled by
 # what the same counter reads for a 64 MiB copy (profiles/k_gemv4_gate_up_m1_hbm_traffic.md).
 GATE_UP_TRAFFIC_BYTES = 76665000
@@ -182,6 +185,46 @@ def main():
             extra["gate_up_M%d" % m] = {"us": round(ms * 1e3, 2), "GBps": round(b / (ms * 1e-3) / 1e9, 1),
                                         "frac_hbm": round(b / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
 
+    # the small configurations: launch- and latency-bound, reported per projection and as one graph per layer
+    small = {}
+    for label, shapes in (("qwen05b", LAYER_05B), ("cfg0", CFG0)):
+        sets = []
+        for _ in range(8):                                   # 8 x 9.4 MB: still inside the 256 MB cache, as in a real
+            host = make_layer(rng, shapes)                   # 0.5B model (all weights 250 MB) these shapes would be
+            sets.append({name: (T.MarlinWeight.upload(dev, host[name][0], host[name][1], k, n),
+                                T.GpuTensor.from_host(dev, host[name][2], "f16"),
+                                T.GpuTensor.zeros(dev, (n,), "f32")) for name, k, n in shapes})
+        entry = {}
+        for name, k, n in shapes:
+            def one(i, name=name, sets=sets):
+                w, a, c = sets[i % len(sets)][name]
+                T.gemm(dev, w, a, 1, c)
+            for i in range(16):
+                one(i)
+            dev.synchronize()
+            ms = time_launches(dev, one, 200)
+            b = algo_bytes(k, n)
+            entry[name] = {"k": k, "n": n, "us": round(ms * 1e3, 3), "GBps": round(b / (ms * 1e-3) / 1e9, 1),
+                           "splits": T.pick_splits(k, n, 1)}
+
+        def run_sets(sets=sets, shapes=shapes):
+            for st in sets:
+                for name, k, n in shapes:
+                    w, a, c = st[name]
+                    T.gemm(dev, w, a, 1, c)
+        g = T.GraphCapture.record_with_device(dev, run_sets)
+        for _ in range(5):
+            g.replay()
+        dev.synchronize()
+        ms = time_launches(dev, lambda i: g.replay(), 50) / len(sets)
+        lb = sum(algo_bytes(k, n) for _, k, n in shapes)
+        entry["layer_graph"] = {"us": round(ms * 1e3, 3), "GBps": round(lb / (ms * 1e-3) / 1e9, 1), "bytes": lb}
+        g.destroy()
+        small[label] = entry
+        for st in sets:
+            for name in st:
+                st[name][0].free(); st[name][1].free(); st[name][2].free()
+
     prefill = None
     if not args.no_prefill:
         prefill = {}
@@ -276,6 +319,7 @@ def main():
         "cpu_baseline": cpu,
         "per_projection": per_shape,
     }
+    out["small_shapes_m1"] = small
     if prefill:
         out["prefill"] = prefill
     if extra:
