@@ -8,10 +8,11 @@
 // Block = 16*MT rows x 256 columns (MT = 8 or 4), 4 waves; wave w owns 64 columns (four 16-column tiles of
 // the tile-order copy) for all rows of the block, so no weight is unpacked twice inside a block.  Per
 // 128-deep k-chunk and wave:
-//   A tile (16*MT x 128 f16): global -> registers -> LDS, double buffered, row stride 272 B so that the
-//                             sixteen rows of a 16-byte-per-lane operand read hit distinct banks;
-//   B : 16 bytes of nibbles + four scales per lane per tile, straight from HBM/L2 into registers, two
-//       chunks ahead (three register slots), unpacked to MFMA B operands one 32-deep group ahead;
+//   A tile (16*MT x 128 f16): global -> LDS directly (global_load_lds_dwordx4), double buffered, 256-byte rows
+//                             whose 16-byte slots are XOR-swizzled so that the sixteen rows of an operand
+//                             read hit distinct banks;
+//   B : 16 bytes of nibbles + four scales per lane per tile, straight from HBM/L2 into registers, one
+//       chunk ahead (two register slots), unpacked to MFMA B operands one 32-deep group ahead;
 //   16*MT v_mfma_f32_16x16x32_f16 (MT row blocks x 4 column tiles x 4 groups), 16*MT accumulator registers.
 // One v_mfma issue slot hides about two other vector instructions, so the unpack (14 instructions per
 // tile and group, shared by MT row blocks) is only free from MT = 8 on.
@@ -21,7 +22,7 @@
 
 namespace twm {
 
-constexpr int kPfRowStride = 136;  // halves per LDS row: 128 + 8 (272 bytes)
+constexpr int kPfRowStride = 128;  // halves per LDS row (256 bytes, unpadded: the 16-byte slots of a row are XOR-swizzled)
 
 struct PfConsts {
     uint32_t mask_lo, mask_hi, magic_lo, magic_hi;
@@ -85,10 +86,9 @@ __global__ __launch_bounds__(256) void k_prefill(const uint4v *__restrict__ qw, 
                                                   uint32_t chunks_per_split, float *__restrict__ partials)
 {
     constexpr int kPfTileHalves = 16 * MT * kPfRowStride;
-    constexpr int NV = MT;       // 16-byte vectors of A each thread stages per chunk (16 MT rows * 16 / 256)
-    constexpr int HV = NV / 2;
+    constexpr int NV = MT;       // direct-to-LDS load instructions per wave and A tile (16 MT rows / 16)
     constexpr int PPU = 8 / MT;  // half fragments unpacked per unit (a unit = one row block's four MFMAs)
-    extern __shared__ _Float16 a_lds[];  // two tiles of kPfTileHalves
+    extern __shared__ _Float16 a_lds[];  // two tiles of kPfTileHalves (64 KB at MT = 8)
 
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const uint32_t lane = threadIdx.x & 63u;
@@ -122,36 +122,36 @@ __global__ __launch_bounds__(256) void k_prefill(const uint4v *__restrict__ qw, 
     };
     pin_acc();
 
-    // ---- A staging: thread handles NV 16-byte vectors: vector j is row (tid / 16) + 16 j, columns
-    // 8 (tid % 16) .. +7 of the chunk.  Loads are unconditional (clamped addresses) so that the k loop is
-    // straight-line code and the compiler can count outstanding loads exactly.  Rows past m_rows replay the
-    // last row and are never stored; columns past k replay the row's first columns, where the padded
-    // weights are exactly zero.  Address = uniform base of (row block, chunk) + a 32-bit per-thread offset.
+    // ---- A tile: global -> LDS directly (global_load_lds_dwordx4: lane L's 16 bytes land at the instruction's
+    // LDS base + 16 L, no registers, no LDS store instruction).  Instruction j of wave w fills rows
+    // 16 j + 4 w .. + 3 (256 bytes each).  Slot s of row r holds the row's vector s ^ (r % 16) (8 halves
+    // each): lane L = (row 4 w + L / 16 of the instruction, slot L % 16) therefore fetches vector
+    // (L % 16) ^ ((4 w + L / 16) % 16), and the sixteen rows of an operand read (one slot each, chosen by the
+    // same XOR) fall on distinct banks.  Loads are unconditional: rows past m_rows replay the last row and
+    // are never stored; vectors past k replay the row's first vector, where the padded weights are zero.
     const char *a_blk = (const char *)a_any + (size_t)m0 * k * 2u;
-    const uint32_t vec = threadIdx.x & 15u;
+    const uint32_t a_vec = (lane & 15u) ^ ((4u * wave + (lane >> 4)) & 15u);
     uint32_t a_off[NV];
 #pragma unroll
     for (int j = 0; j < NV; j++) {
-        uint32_t row = m0 + (threadIdx.x >> 4) + 16u * j;
+        uint32_t row = m0 + 16u * j + 4u * wave + (lane >> 4);
         row = (row < m_rows ? row : m_rows - 1) - m0;
-        a_off[j] = (row * k + vec * 8u) * 2u;
+        a_off[j] = (row * k + a_vec * 8u) * 2u;
     }
-    uint4v a_stage[NV];
-    const char *a_src;
-    uint32_t a_back;
-    auto aim_a = [&](uint32_t kc) {  // addresses of chunk kc
-        a_src = a_blk + (size_t)(kc0 + kc) * 256u;
-        a_back = (kc0 + kc) * 128u + vec * 8u < k ? 0u : vec * 16u;
+    auto load_a = [&](uint32_t buf, uint32_t kc, int j) {  // part j of tile kc (relative) into LDS buffer buf
+        const char *src = a_blk + (size_t)(kc0 + kc) * 256u;
+        const uint32_t back = (kc0 + kc) * 128u + a_vec * 8u < k ? 0u : a_vec * 16u;
+        __builtin_amdgcn_global_load_lds((const TWM_GLOBAL void *)(src + (a_off[j] - back)),
+                                         (__attribute__((address_space(3))) void *)(a_lds + buf * kPfTileHalves +
+                                                                                    (16 * j + 4 * wave) * kPfRowStride),
+                                         16, 0, 0);
     };
-    auto load_a = [&](int j) { a_stage[j] = *(const uint4v *)(a_src + (a_off[j] - a_back)); };
-    const uint32_t wr_off = (threadIdx.x >> 4) * kPfRowStride + vec * 8u;
-    auto store_a = [&](uint32_t buf, int j) {
-        *(uint4v *)(a_lds + buf * kPfTileHalves + wr_off + j * 16 * kPfRowStride) = a_stage[j];
-    };
+    // everything this wave has loaded (its parts of the A tile among it) has arrived: before a barrier
+    auto wait_loads = [&]() { __builtin_amdgcn_s_waitcnt(0x0F70); };  // vmcnt(0), other counters untouched
 
-    // ---- B: chunk kc lives in register slot kc % 3 (one being multiplied, two in flight)
-    uint4v bq[3][4];
-    uint2v bs[3][4];
+    // ---- B: chunk kc lives in register slot kc % 2
+    uint4v bq[2][4];
+    uint2v bs[2][4];
     const uint32_t q_off = lane * 16u, s_off = c * 8u;
     auto load_bq = [&](int slot, uint32_t kc, int t) {
         bq[slot][t] = *(const TWM_GLOBAL uint4v *)(scalar_base(qw, (size_t)((kc0 + kc) * n_tiles + nt[t]) * 1024u) + q_off);
@@ -167,9 +167,11 @@ __global__ __launch_bounds__(256) void k_prefill(const uint4v *__restrict__ qw, 
         pf_unpack_half(bf[t], hp & 1, bq[slot][t][g], s16, dq);
     };
 
-    const uint32_t rd_off = c * kPfRowStride + kb * 8u;
+    uint32_t rd_off[4];  // row c of a row block, vector 4 g + kb of the chunk -> slot (4 g + kb) ^ c
+#pragma unroll
+    for (int g = 0; g < 4; g++) rd_off[g] = c * kPfRowStride + (((4u * g + kb) ^ c) * 8u);
     auto read_a = [&](uint32_t buf, int g, int mt) {
-        return *(const half8 *)(a_lds + buf * kPfTileHalves + rd_off + mt * 16 * kPfRowStride + g * 32);
+        return *(const half8 *)(a_lds + buf * kPfTileHalves + rd_off[g] + mt * 16 * kPfRowStride);
     };
 
     half8 af0[MT], af1[MT];
@@ -195,59 +197,49 @@ __global__ __launch_bounds__(256) void k_prefill(const uint4v *__restrict__ qw, 
         }
     };
 
-    // One k-chunk (B slot S, LDS buffer kc & 1).  On entry af0 / bf0 hold group 0 of this chunk and a_stage
-    // holds A tile kc+1.
-    //   step 0, 1: write A tile kc+1 to the other LDS buffer; load B nibbles of chunk kc+2
-    //   step 2   : load first half of A tile kc+2; then the chunk's only barrier
-    //   step 3   : load the rest of A tile kc+2 and the B scales of chunk kc+2; its reads and unpack are
-    //              already those of chunk kc+1, group 0
-    // Barrier: tile kc+1 is complete before step 3 reads it, and all reads of buffer (kc+1) & 1 as tile
-    // kc-1 (issued up to step 2 of chunk kc-1 and completed before that chunk's barrier) precede its
-    // rewriting.  Past the end the last chunk is loaded again and never used.
+    // One k-chunk (B slot S = kc & 1, LDS buffer kc & 1).  On entry af0 / bf0 hold group 0 of this chunk.
+    //   step 0   : load B (nibbles, scales) of chunk kc+1 into the other slot
+    //   step 1, 2: no loads; at the end of step 2 wait for this wave's loads, then the chunk's only barrier:
+    //              A tile kc+1 is complete, and every wave is done reading buffer kc & 1 (tile kc: its reads
+    //              were issued up to step 2 and are waited for by the barrier)
+    //   step 3   : A tile kc+2 -> buffer kc & 1; the step's own reads and unpack are already those of chunk
+    //              kc+1, group 0
+    // Past the end the last chunk is loaded again and never used.
     auto chunk = [&](auto slot_c, uint32_t kc) {
-        constexpr int S = decltype(slot_c)::value, S1 = (S + 1) % 3, S2 = (S + 2) % 3;
+        constexpr int S = decltype(slot_c)::value, S1 = S ^ 1;
         const uint32_t buf = kc & 1u;
-        const uint32_t kc2 = kc + 2 < last ? kc + 2 : last;
+        const uint32_t kc1 = kc + 1 < last ? kc + 1 : last, kc2 = kc + 2 < last ? kc + 2 : last;
         step(af0, bf0, af1, bf1, buf, 1, S, 1, [&](int u) {
-            if (u < 2) load_bq(S2, kc2, u);
-            if (u < HV) store_a(buf ^ 1u, u);
+#pragma unroll
+            for (int t = 0; t < 4; t++) {
+                if (t * MT / 4 == u) load_bq(S1, kc1, t);
+                if (t * MT / 4 + (MT >= 8 ? 1 : 0) == u) load_bs(S1, kc1, t);
+            }
         });
-        step(af1, bf1, af0, bf0, buf, 2, S, 2, [&](int u) {
-            if (u < 2) load_bq(S2, kc2, 2 + u);
-            if (u < NV - HV) store_a(buf ^ 1u, HV + u);
-        });
-        aim_a(kc2);
-        step(af0, bf0, af1, bf1, buf, 3, S, 3, [&](int u) {
-            if (u < HV) load_a(u);
-        });
+        step(af1, bf1, af0, bf0, buf, 2, S, 2, [&](int) {});
+        step(af0, bf0, af1, bf1, buf, 3, S, 3, [&](int) {});
+        wait_loads();
         __syncthreads();
         step(af1, bf1, af0, bf0, buf ^ 1u, 0, S1, 0, [&](int u) {
-            if (u < NV - HV) load_a(HV + u);
-            if (u >= MT - 4) load_bs(S2, kc2, u - (MT - 4));
+            if (u < NV) load_a(buf, kc2, u);
         });
         pin_acc();
     };
     using S0 = std::integral_constant<int, 0>;
     using S1 = std::integral_constant<int, 1>;
-    using S2 = std::integral_constant<int, 2>;
 
-    // prologue: tile 0 in LDS, tile 1 in the staging registers, B chunks 0 and 1 in slots 0 and 1
-    const uint32_t kc1 = 1 < last ? 1 : last;
-    aim_a(0);
+    // prologue: tiles 0 and 1 -> LDS, B chunk 0 -> slot 0
+    const uint32_t kc1p = 1 < last ? 1 : last;
 #pragma unroll
-    for (int j = 0; j < NV; j++) load_a(j);
+    for (int j = 0; j < NV; j++) load_a(0, 0, j);
 #pragma unroll
     for (int t = 0; t < 4; t++) {
         load_bq(0, 0, t);
         load_bs(0, 0, t);
-        load_bq(1, kc1, t);
-        load_bs(1, kc1, t);
     }
 #pragma unroll
-    for (int j = 0; j < NV; j++) store_a(0, j);
-    aim_a(kc1);
-#pragma unroll
-    for (int j = 0; j < NV; j++) load_a(j);
+    for (int j = 0; j < NV; j++) load_a(1, kc1p, j);
+    wait_loads();
     __syncthreads();
 #pragma unroll
     for (int mt = 0; mt < MT; mt++) af0[mt] = read_a(0, 0, mt);
@@ -256,13 +248,11 @@ __global__ __launch_bounds__(256) void k_prefill(const uint4v *__restrict__ qw, 
     __builtin_amdgcn_sched_barrier(0);
 
     uint32_t kc = 0;
-    for (; kc + 3 <= nchunks; kc += 3) {
+    for (; kc + 2 <= nchunks; kc += 2) {
         chunk(S0{}, kc);
         chunk(S1{}, kc + 1);
-        chunk(S2{}, kc + 2);
     }
     if (kc < nchunks) chunk(S0{}, kc);
-    if (kc + 1 < nchunks) chunk(S1{}, kc + 1);
 
     // ---- store: lane (c, kb) holds rows 4*kb + r of row block mt, column 16*tile + c ----
     if (partials) {
@@ -380,7 +370,7 @@ static hipError_t launch_prefill_t(hipStream_t s, const WeightView &w, const _Fl
     return hipGetLastError();
 }
 
-// Once per device, outside any stream capture: the 128-row variant needs 68 KB of dynamic LDS.
+// Once per device, outside any stream capture: the 128-row variant asks for all 64 KB of dynamic LDS.
 hipError_t init_prefill()
 {
     return hipFuncSetAttribute((const void *)k_prefill<8>, hipFuncAttributeMaxDynamicSharedMemorySize,
