@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the TW-Marlin W4A16 decode path on one MI355X.
 
-Workload (BASELINE.json configs[2]): the four M=1 GEMVs of a Qwen-7B-shaped layer
+Workload: the four M=1 GEMVs of a Qwen-7B-shaped layer
     qkv 3584->4608, o 3584->3584, gate_up 3584->37888, down 18944->3584
 group-32 Q4 weights + FP16 scales, FP16 activations, FP32 outputs.  One "step" = one layer.
 Several distinct layers (default 4, 525 MB of weights) are walked in turn so that the 256 MB
@@ -12,8 +12,8 @@ same measurement with one graph per layer, which pays the graph-launch cost once
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers L] [--no-cpu] [--no-prefill] [--extra]
 
-`small_shapes_m1` holds the launch-bound configurations (BASELINE.json configs[0] and [1]: 4096->4096 and
-the Qwen-0.5B layer) per projection and as a graph, `prefill` the W4A16 GEMM on the LLaMA-7B MLP shapes (BASELINE.json configs[4]) at M=512 and
+`small_shapes_m1` holds the launch-bound configurations (4096->4096 and the Qwen-0.5B layer) per
+projection and as a graph, `prefill` the W4A16 GEMM on the LLaMA-7B MLP shapes at M=512 and
 2048 as TFLOP/s against the 2.5 PFLOP/s dense FP16 MFMA peak; it is not part of `value`.
 
 Prints ONE JSON line. `value` = algorithmic bytes of a layer x K / time of K replays (inputs
@@ -32,8 +32,8 @@ HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X dense FP16 matrix, published
 
 LAYER_7B = [("qkv", 3584, 4608), ("o", 3584, 3584), ("gate_up", 3584, 37888), ("down", 18944, 3584)]
-LAYER_05B = [("qkv", 896, 1152), ("o", 896, 896), ("gate_up", 896, 9728), ("down", 4864, 896)]   # BASELINE.json configs[1]
-CFG0 = [("cfg0", 4096, 4096)]                                                                     # BASELINE.json configs[0]
+LAYER_05B = [("qkv", 896, 1152), ("o", 896, 896), ("gate_up", 896, 9728), ("down", 4864, 896)]   # Qwen-0.5B layer
+CFG0 = [("cfg0", 4096, 4096)]                                                                     # the single-GEMV configuration
 # HBM bytes per gate_up launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, each scaled by
 # what the same counter reads for a 64 MiB copy (profiles/k_gemv4_gate_up_m1_hbm_traffic.md).
 GATE_UP_TRAFFIC_BYTES = 76665000
@@ -78,7 +78,7 @@ def main():
     ap.add_argument("--extra", action="store_true", help="also time batched decode (M=4..32) on the gate_up shape")
     ap.add_argument("--sweep-splits", action="store_true",
                     help="also time every projection at M=1,4,8,16,32 with forced split-K factors next to the library's "
-                         "own choice (BASELINE.json configs[3])")
+                         "own choice (batched decode configuration)")
     ap.add_argument("--pmc-copy", action="store_true",
                     help="also run four 64 MiB device-to-device copies: a kernel of known traffic to scale rocprofv3 "
                          "FETCH_SIZE / WRITE_SIZE readings by")

@@ -80,7 +80,7 @@ def lcg_act(m, k):
 
 def make_case(name, k, n, m, rng, synthetic):
     if synthetic:
-        # BASELINE-style synthetic: nibbles uniform 0..15, scales f16(|N(0,1)|*0.02)
+        # benchmark-style synthetic: nibbles uniform 0..15, scales f16(|N(0,1)|*0.02)
         packed = rng.integers(0, 256, size=(k // 32, n, 16), dtype=np.uint8)
         scales = (np.abs(rng.standard_normal((k // 32, n))) * 0.02).astype(np.float32).astype(np.float16)
         a16 = rng.standard_normal((m, k)).astype(np.float32).astype(np.float16)
