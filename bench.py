@@ -322,6 +322,10 @@ def main():
     out["small_shapes_m1"] = small
     if prefill:
         out["prefill"] = prefill
+        best = max(prefill.items(), key=lambda kv: kv[1]["TFLOPs"] if kv[0].startswith("M2048") else 0.0)
+        out["roofline_prefill"] = {"bound": "mfma", "kernel": "k_prefill (%s)" % best[0], "achieved": best[1]["TFLOPs"],
+                                   "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": best[1]["frac_mfma_f16_peak"],
+                                   "us_per_launch": best[1]["us"]}
     if extra:
         out["batched_decode"] = extra
     if sweep:
