@@ -89,3 +89,13 @@ def test_product_package_does_not_touch_the_oracle():
             if f.endswith((".py", ".hip", ".h", ".cpp")):
                 text = open(os.path.join(dirpath, f)).read()
                 assert "oracle" not in text.replace("no CPU fallback", ""), f
+
+
+def test_bench_refuses_more_than_one_gpu():
+    # one GPU per box: bench.py --gpus N (N != 1) exits with a message before touching any device
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    res = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True)
+    assert res.returncode != 0
+    assert "ONE GPU" in res.stderr
