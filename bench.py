@@ -10,7 +10,7 @@ captured once as a hipGraph (the reference captures all layers of a decode step 
 crates/kernels/src/generate.rs:2485-2536) and replayed; `config.us_per_layer_own_graph` is the
 same measurement with one graph per layer, which pays the graph-launch cost once per layer.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers L] [--no-cpu] [--no-prefill] [--extra]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers L] [--no-cpu] [--no-prefill] [--no-lm-head] [--extra]
 
 `small_shapes_m1` holds the launch-bound configurations (4096->4096 and the Qwen-0.5B layer) per
 projection and as a graph, `prefill` the W4A16 GEMM on the LLaMA-7B MLP shapes at M=512 and
@@ -75,6 +75,7 @@ def main():
     ap.add_argument("--layers", type=int, default=4, help="distinct weight sets rotated through (>=3 defeats the 256 MB cache)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--no-prefill", action="store_true", help="skip the prefill GEMM timings")
+    ap.add_argument("--no-lm-head", action="store_true", help="skip the LM-head GEMV + argmax timing")
     ap.add_argument("--extra", action="store_true", help="also time batched decode (M=4..32) on the gate_up shape")
     ap.add_argument("--sweep-splits", action="store_true",
                     help="also time every projection at M=1,4,8,16,32 with forced split-K factors next to the library's "
@@ -225,6 +226,42 @@ def main():
             for name in st:
                 st[name][0].free(); st[name][1].free(); st[name][2].free()
 
+    # The LM head of the same model class as a TW-Marlin GEMV with on-device argmax (the reference has
+    # forward_lm_head_tw_marlin, generate.rs:1748-1761, and a GPU argmax buffer, :1417): 3584 -> 152064, the
+    # largest GEMV of a decode step.  Two weight sets (616 MB) alternate so that the cache cannot hold them.
+    lm = None
+    if not args.no_lm_head:
+        k, n = 3584, 152064
+        sets = []
+        for _ in range(2):
+            packed = rng.integers(0, 256, size=(k // 32) * n * 16, dtype=np.uint8)
+            scales = (np.abs(rng.standard_normal((k // 32) * n, dtype=np.float32)) * np.float32(0.02)).astype(np.float16)
+            sets.append(T.MarlinWeight.upload(dev, packed, scales.view(np.uint16), k, n))
+        a1 = T.GpuTensor.from_host(dev, rng.standard_normal(k, dtype=np.float32).astype(np.float16).view(np.uint16), "f16")
+        logits = T.GpuTensor.zeros(dev, (n,), "f32")
+        token = T.GpuTensor.from_host(dev, np.zeros(1, np.int32))
+
+        def one_gemv(i):
+            T.gemm(dev, sets[i % 2], a1, 1, logits)
+
+        def one_argmax(i):
+            T.argmax(dev, logits, token, 1, n)
+        for i in range(6):
+            one_gemv(i)
+            one_argmax(i)
+        dev.synchronize()
+        ms_g = time_launches(dev, one_gemv, 100)
+        ms_a = time_launches(dev, one_argmax, 100)
+        picked = int(token.to_host()[0])
+        assert picked == int(np.argmax(logits.to_host())), "argmax disagrees with the host"
+        b = algo_bytes(k, n)
+        lm = {"k": k, "n": n, "gemv_us": round(ms_g * 1e3, 2), "GBps": round(b / (ms_g * 1e-3) / 1e9, 1),
+              "frac_hbm": round(b / (ms_g * 1e-3) / 1e9 / HBM_PEAK_GBS, 4), "argmax_us": round(ms_a * 1e3, 2),
+              "bytes": b}
+        for w in sets:
+            w.free()
+        logits.free()
+
     prefill = None
     if not args.no_prefill:
         prefill = {}
@@ -320,6 +357,8 @@ def main():
         "per_projection": per_shape,
     }
     out["small_shapes_m1"] = small
+    if lm:
+        out["lm_head_m1"] = lm
     if prefill:
         out["prefill"] = prefill
         best = max(prefill.items(), key=lambda kv: kv[1]["TFLOPs"] if kv[0].startswith("M2048") else 0.0)

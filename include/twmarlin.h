@@ -146,6 +146,12 @@ int twm_split_qkv(twm_ctx *ctx, const float *qkv_dev, float *q_dev, float *k_dev
 int twm_split_gate_up(twm_ctx *ctx, const float *gate_up_dev, float *gate_dev, float *up_dev,
                       uint32_t ffn_dim, uint32_t batch);
 
+/* argmax (crates/kernels/src/missing_ops.rs:24-58): out[row] = first index of the row's maximum, with the
+ * reference's starting value: only values > -1e30 compete, a row without any yields 0; NaNs never win.
+ * input [rows, cols] f32 row-major, out [rows] i32.  Used on the LM-head logits (generate.rs:1417-1418)
+ * so that greedy decoding reads back 4 bytes instead of the logits. */
+int twm_argmax_f32(twm_ctx *ctx, const float *input_dev, uint32_t rows, uint32_t cols, int32_t *out_dev);
+
 /* ---- the quantized-GEMM entry point, reference layout in, no repack ------------------ */
 
 /* gemm_tw_marlin_m1 (quantize.rs:1301-1360): C[1,N] = A[1,K] * dequant(packed, scales),

@@ -265,6 +265,23 @@ void twmo_split_gate_up(const float *gu, float *gate, float *up, uint32_t ffn, u
     }
 }
 
+/* warp_argmax (crates/kernels/src/missing_ops.rs:24-39): sequential scan, strict '>' from -1e30 at index 0 */
+void twmo_argmax(const float *in, uint32_t rows, uint32_t cols, int32_t *out)
+{
+    for (uint32_t r = 0; r < rows; r++) {
+        float max_val = -1e30f;
+        int32_t max_idx = 0;
+        for (uint32_t c = 0; c < cols; c++) {
+            float v = in[(size_t)r * cols + c];
+            if (v > max_val) {
+                max_val = v;
+                max_idx = (int32_t)c;
+            }
+        }
+        out[r] = max_idx;
+    }
+}
+
 /* ------------------------------------------------------------------ */
 /* Dequant                                                             */
 /* ------------------------------------------------------------------ */

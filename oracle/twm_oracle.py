@@ -135,6 +135,13 @@ def split_gate_up(gu, ffn, batch):
     return g, u
 
 
+def argmax(x, rows, cols):
+    x = _c(x, np.float32)
+    out = np.zeros(rows, np.int32)
+    lib().twmo_argmax(_p(x), C.c_uint32(rows), C.c_uint32(cols), _p(out))
+    return out
+
+
 def dequant_f32(packed, scales, k, n):
     out = np.empty((k, n), np.float32)
     lib().twmo_dequant_f32(_p(_c(packed, np.uint8)), _p(_c(scales, np.uint16)),

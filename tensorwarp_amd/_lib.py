@@ -43,6 +43,7 @@ SIGNATURES = {
     "twm_dequant_to_f16": (_int, [_vp, _vp, _vp, _u32, _u32, _vp]),
     "twm_dequant_to_f32": (_int, [_vp, _vp, _vp, _u32, _u32, _vp]),
     "twm_split_qkv": (_int, [_vp, _vp, _vp, _vp, _vp, _u32, _u32, _u32]),
+    "twm_argmax_f32": (_int, [_vp, _vp, _u32, _u32, _vp]),
     "twm_split_gate_up": (_int, [_vp, _vp, _vp, _vp, _u32, _u32]),
     "twm_gemm_tw_marlin_m1": (_int, [_vp, _vp, _vp, _vp, _vp, _u32, _u32]),
     "twm_gemm_tw_marlin_m1_from_buffer": (_int, [_vp, _vp, _vp, _sz, _vp, _sz, _vp, _u32, _u32]),

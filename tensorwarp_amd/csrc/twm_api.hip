@@ -403,6 +403,15 @@ int twm_split_qkv(twm_ctx *ctx, const float *qkv_dev, float *q_dev, float *k_dev
     return TWM_OK;
 }
 
+int twm_argmax_f32(twm_ctx *ctx, const float *input_dev, uint32_t rows, uint32_t cols, int32_t *out_dev)
+{
+    if (!ctx) return fail(TWM_INVALID_HANDLE, "twm_argmax_f32: null context");
+    if (rows == 0) return TWM_OK;
+    if (!out_dev || (cols != 0 && !input_dev)) return fail(TWM_INVALID_HANDLE, "twm_argmax_f32: null pointer");
+    HIP_TRY(launch_argmax(ctx->stream, input_dev, rows, cols, out_dev, ctx->ws, ctx->ws_bytes), TWM_DEVICE_ERROR, "argmax launch");
+    return TWM_OK;
+}
+
 int twm_split_gate_up(twm_ctx *ctx, const float *gate_up_dev, float *gate_dev, float *up_dev, uint32_t ffn_dim,
                       uint32_t batch)
 {

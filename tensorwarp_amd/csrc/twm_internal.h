@@ -60,6 +60,8 @@ hipError_t launch_dequant(hipStream_t s, const uint8_t *packed, const uint16_t *
 hipError_t launch_split_qkv(hipStream_t s, const float *qkv, float *q, float *kk, float *v, uint32_t h,
                             uint32_t kv, uint32_t batch);
 hipError_t launch_split_gate_up(hipStream_t s, const float *gu, float *g, float *u, uint32_t ffn, uint32_t batch);
+hipError_t launch_argmax(hipStream_t s, const float *in, uint32_t rows, uint32_t cols, int *out, void *scratch,
+                         size_t scratch_bytes);
 hipError_t launch_ref_gemv(hipStream_t s, const float *a, const uint8_t *packed, const uint16_t *scales, float *c,
                            uint32_t n, uint32_t k, uint32_t splits, uint32_t groups_per_split);
 hipError_t launch_repack(hipStream_t s, const uint8_t *packed, const uint16_t *scales, uint32_t k, uint32_t n,

@@ -263,6 +263,137 @@ __global__ __launch_bounds__(256) void k_split_gate_up(const float *__restrict__
     else u[(size_t)b * ffn + (d - ffn)] = x;
 }
 
+// ArgMax along the last dimension with the reference's rule (crates/kernels/src/missing_ops.rs:24-39): the
+// first index whose value is greater than every earlier candidate, starting from -1e30 at index 0 (so
+// values <= -1e30 and NaNs are never chosen, and an empty or all-small row yields 0).  One workgroup per row:
+// each thread scans a strided share in increasing order, then (value, index) pairs are merged preferring
+// the larger value and, among equal values, the smaller index.
+__global__ __launch_bounds__(1024) void k_argmax(const float *__restrict__ in, uint32_t cols, int *__restrict__ out)
+{
+    __shared__ float sv[1024];
+    __shared__ uint32_t si[1024];
+    const float *row = in + (size_t)blockIdx.x * cols;
+    float best = -1e30f;
+    uint32_t idx = 0xFFFFFFFFu;  // "none yet"
+    for (uint32_t c = threadIdx.x; c < cols; c += 1024u) {
+        float v = row[c];
+        if (v > best) {
+            best = v;
+            idx = c;
+        }
+    }
+    sv[threadIdx.x] = best;
+    si[threadIdx.x] = idx;
+    __syncthreads();
+    for (uint32_t step = 512; step > 0; step >>= 1) {
+        if (threadIdx.x < step) {
+            float ov = sv[threadIdx.x + step];
+            uint32_t oi = si[threadIdx.x + step];
+            if (ov > sv[threadIdx.x] || (ov == sv[threadIdx.x] && oi < si[threadIdx.x])) {
+                sv[threadIdx.x] = ov;
+                si[threadIdx.x] = oi;
+            }
+        }
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) out[blockIdx.x] = si[0] == 0xFFFFFFFFu ? 0 : (int)si[0];
+}
+
+// Long rows (a vocabulary): phase 1, one workgroup per 8192 columns leaves its (value, index) candidate in
+// scratch; phase 2 is k_argmax_merge over the candidates.  Same rule: larger value, then smaller index.
+constexpr uint32_t kArgmaxSpan = 8192;
+
+__global__ __launch_bounds__(1024) void k_argmax_partial(const float *__restrict__ in, uint32_t cols, uint32_t spans,
+                                                          float *__restrict__ cand_val, uint32_t *__restrict__ cand_idx)
+{
+    __shared__ float sv[1024];
+    __shared__ uint32_t si[1024];
+    const float *row = in + (size_t)blockIdx.y * cols;
+    const uint32_t c0 = blockIdx.x * kArgmaxSpan;
+    float v[8];
+#pragma unroll
+    for (int j = 0; j < 8; j++) {  // all eight loads first, then the compares in increasing index order
+        uint32_t c = c0 + threadIdx.x + 1024u * j;
+        v[j] = c < cols ? row[c] : -1e30f;
+    }
+    float best = -1e30f;
+    uint32_t idx = 0xFFFFFFFFu;
+#pragma unroll
+    for (int j = 0; j < 8; j++)
+        if (v[j] > best) {
+            best = v[j];
+            idx = c0 + threadIdx.x + 1024u * j;
+        }
+    sv[threadIdx.x] = best;
+    si[threadIdx.x] = idx;
+    __syncthreads();
+    for (uint32_t step = 512; step > 0; step >>= 1) {
+        if (threadIdx.x < step) {
+            float ov = sv[threadIdx.x + step];
+            uint32_t oi = si[threadIdx.x + step];
+            if (ov > sv[threadIdx.x] || (ov == sv[threadIdx.x] && oi < si[threadIdx.x])) {
+                sv[threadIdx.x] = ov;
+                si[threadIdx.x] = oi;
+            }
+        }
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) {
+        cand_val[(size_t)blockIdx.y * spans + blockIdx.x] = sv[0];
+        cand_idx[(size_t)blockIdx.y * spans + blockIdx.x] = si[0];
+    }
+}
+
+__global__ __launch_bounds__(256) void k_argmax_merge(const float *__restrict__ cand_val, const uint32_t *__restrict__ cand_idx,
+                                                       uint32_t spans, int *__restrict__ out)
+{
+    __shared__ float sv[256];
+    __shared__ uint32_t si[256];
+    float best = -1e30f;
+    uint32_t idx = 0xFFFFFFFFu;
+    for (uint32_t s = threadIdx.x; s < spans; s += 256u) {  // candidates of later spans have larger indices
+        float v = cand_val[(size_t)blockIdx.x * spans + s];
+        uint32_t i = cand_idx[(size_t)blockIdx.x * spans + s];
+        if (v > best || (v == best && i < idx)) {
+            best = v;
+            idx = i;
+        }
+    }
+    sv[threadIdx.x] = best;
+    si[threadIdx.x] = idx;
+    __syncthreads();
+    for (uint32_t step = 128; step > 0; step >>= 1) {
+        if (threadIdx.x < step) {
+            float ov = sv[threadIdx.x + step];
+            uint32_t oi = si[threadIdx.x + step];
+            if (ov > sv[threadIdx.x] || (ov == sv[threadIdx.x] && oi < si[threadIdx.x])) {
+                sv[threadIdx.x] = ov;
+                si[threadIdx.x] = oi;
+            }
+        }
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) out[blockIdx.x] = si[0] == 0xFFFFFFFFu ? 0 : (int)si[0];
+}
+
+// `scratch` (scratch_bytes) holds the candidates of the two-phase form; without enough of it, or for short
+// rows, one workgroup per row scans the whole row.
+hipError_t launch_argmax(hipStream_t s, const float *in, uint32_t rows, uint32_t cols, int *out, void *scratch,
+                         size_t scratch_bytes)
+{
+    if (rows == 0) return hipSuccess;
+    uint32_t spans = (cols + kArgmaxSpan - 1) / kArgmaxSpan;
+    if (spans >= 4 && rows <= 65535 && scratch && (size_t)rows * spans * 8 <= scratch_bytes) {
+        float *cv = (float *)scratch;
+        uint32_t *ci = (uint32_t *)(cv + (size_t)rows * spans);
+        hipLaunchKernelGGL(k_argmax_partial, dim3(spans, rows), dim3(1024), 0, s, in, cols, spans, cv, ci);
+        hipLaunchKernelGGL(k_argmax_merge, dim3(rows), dim3(256), 0, s, cv, ci, spans, out);
+        return hipGetLastError();
+    }
+    hipLaunchKernelGGL(k_argmax, dim3(rows), dim3(1024), 0, s, in, cols, out);
+    return hipGetLastError();
+}
+
 hipError_t launch_split_qkv(hipStream_t s, const float *qkv, float *q, float *kk, float *v, uint32_t h, uint32_t kv,
                             uint32_t batch)
 {

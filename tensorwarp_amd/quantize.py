@@ -81,7 +81,7 @@ class WarpDevice:
         _check(self._l.twm_event_destroy(self.handle, ev))
 
 
-_NP_DTYPES = {"f32": np.float32, "f16": np.uint16, "u8": np.uint8}
+_NP_DTYPES = {"f32": np.float32, "f16": np.uint16, "u8": np.uint8, "i32": np.int32}
 
 
 class GpuTensor:
@@ -110,7 +110,7 @@ class GpuTensor:
         array = np.ascontiguousarray(array)
         if dtype is None:
             dtype = {np.dtype(np.float32): "f32", np.dtype(np.uint16): "f16", np.dtype(np.float16): "f16",
-                     np.dtype(np.uint8): "u8"}[array.dtype]
+                     np.dtype(np.uint8): "u8", np.dtype(np.int32): "i32"}[array.dtype]
         if array.dtype == np.float16:
             array = array.view(np.uint16)
         t = cls(device, array.shape, dtype)
@@ -218,6 +218,11 @@ def split_qkv(device, qkv, q, k, v, h, kv_dim, batch):
 def split_gate_up(device, gate_up, gate, up, ffn_dim, batch):
     """ops.rs:2324"""
     _check(device._l.twm_split_gate_up(device.handle, gate_up.ptr, gate.ptr, up.ptr, ffn_dim, batch))
+
+
+def argmax(device, input, output, rows, cols):
+    """missing_ops.rs:42 — input f32 [rows, cols], output i32 [rows]."""
+    _check(device._l.twm_argmax_f32(device.handle, input.ptr, rows, cols, output.ptr))
 
 
 def gemm_tw_marlin_m1(device, a, packed, scales, c, n, k):

@@ -121,6 +121,32 @@ def test_split_kernels(dev):
     assert np.array_equal(g.to_host(), og) and np.array_equal(u.to_host(), ou)
 
 
+def test_argmax_bit_exact(dev):
+    # index output: bit exact against the oracle's sequential scan, including ties (first wins), values at or
+    # below the -1e30 starting value, NaN, infinities, a vocabulary-sized row and an empty one
+    rng = np.random.default_rng(11)
+    cases = [rng.standard_normal((5, 3000)).astype(np.float32),
+             rng.standard_normal((1, 152064)).astype(np.float32),
+             np.round(rng.standard_normal((8, 5000)) * 2).astype(np.float32),          # many ties
+             np.full((2, 2048), -2e30, np.float32),
+             np.array([[np.nan, 1.0, np.nan, 3.0, 3.0, np.nan]], np.float32),
+             np.array([[1.0, np.inf, np.inf, -np.inf]], np.float32),
+             np.full((1, 1500), np.nan, np.float32),
+             np.round(rng.standard_normal((3, 70000)) * 3).astype(np.float32),         # two-phase form with ties across spans
+             np.full((2, 40000), -2e30, np.float32),
+             np.full((1, 33000), np.nan, np.float32)]
+    cases[3][1, 1999] = np.float32(-9.9e29)
+    cases[8][1, 39999] = np.float32(-9.9e29)
+    for x in cases:
+        rows, cols = x.shape
+        out = T.GpuTensor.from_host(dev, np.full(rows, -7, np.int32))
+        T.argmax(dev, T.GpuTensor.from_host(dev, x), out, rows, cols)
+        assert np.array_equal(out.to_host(), O.argmax(x, rows, cols)), x.shape
+    out = T.GpuTensor.from_host(dev, np.full(3, -7, np.int32))
+    T.argmax(dev, T.GpuTensor.zeros(dev, (1,), "f32"), out, 3, 0)        # cols == 0: every row yields 0
+    assert out.to_host().tolist() == [0, 0, 0]
+
+
 # ---------------------------------------------------------------- Q4 unpack, bit exact
 
 @pytest.mark.parametrize("name", ["lcg_k64_n8_m1", "lcg_k128_n64_m4", "synth_k128_n64_m1",

@@ -309,3 +309,26 @@ def test_synthetic_generators_are_deterministic_and_shaped():
     assert s.min() >= 0 and abs(s.mean() - 0.02 * np.sqrt(2 / np.pi)) < 1e-3
     a = O.synth_act_f16(4, 4096, 5).view(np.float16).astype(np.float32)
     assert abs(a.mean()) < 0.03 and abs(a.std() - 1) < 0.03
+
+
+def test_argmax_follows_the_reference_scan():
+    # warp_argmax (missing_ops.rs:24-39): first index of the maximum; only values > -1e30 compete; NaN never wins.
+    # Pinned against numpy where the two definitions coincide and by hand where they do not.
+    rng = np.random.default_rng(5)
+    x = rng.standard_normal((7, 1000)).astype(np.float32)
+    assert np.array_equal(O.argmax(x, 7, 1000), np.argmax(x, axis=1).astype(np.int32))
+    ties = np.zeros((1, 9), np.float32)
+    ties[0, [3, 5, 8]] = 2.5
+    assert O.argmax(ties, 1, 9)[0] == 3                                   # first of equal maxima
+    low = np.full((1, 5), -2e30, np.float32)
+    assert O.argmax(low, 1, 5)[0] == 0                                    # nothing above the starting value
+    low[0, 4] = -1e30
+    assert O.argmax(low, 1, 5)[0] == 0                                    # equal to it does not count either
+    low[0, 2] = np.float32(-9.9e29)
+    assert O.argmax(low, 1, 5)[0] == 2
+    nan = np.array([[np.nan, 1.0, np.nan, 3.0, np.nan]], np.float32)
+    assert O.argmax(nan, 1, 5)[0] == 3                                    # comparisons with NaN are false
+    assert O.argmax(np.full((1, 4), np.nan, np.float32), 1, 4)[0] == 0
+    assert O.argmax(np.zeros((2, 0), np.float32), 2, 0).tolist() == [0, 0]  # empty rows
+    inf = np.array([[1.0, np.inf, np.inf, -np.inf]], np.float32)
+    assert O.argmax(inf, 1, 4)[0] == 1
