@@ -76,6 +76,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--no-prefill", action="store_true", help="skip the prefill GEMM timings")
     ap.add_argument("--no-lm-head", action="store_true", help="skip the LM-head GEMV + argmax timing")
+    ap.add_argument("--no-swiglu", action="store_true", help="skip the fused gate_up + SwiGLU timing")
     ap.add_argument("--extra", action="store_true", help="also time batched decode (M=4..32) on the gate_up shape")
     ap.add_argument("--sweep-splits", action="store_true",
                     help="also time every projection at M=1,4,8,16,32 with forced split-K factors next to the library's "
@@ -262,6 +263,56 @@ def main():
             w.free()
         logits.free()
 
+    # MLP front half at M=1: the reference's three launches (GEMV, split_gate_up, fused_silu_mul) against the
+    # single launch with the gate applied in the GEMV's store; graphs over distinct weight sets
+    mlp_front = None
+    if not args.no_swiglu:
+        k, ffn = 3584, 18944
+        plain, pairedw = [], []
+        for _ in range(L):
+            halves = []
+            for _h in range(2):
+                packed = rng.integers(0, 256, size=(k // 32) * ffn * 16, dtype=np.uint8)
+                scales = (np.abs(rng.standard_normal((k // 32) * ffn, dtype=np.float32)) * np.float32(0.02)).astype(np.float16)
+                halves.append((T.GpuTensor.from_host(dev, packed), T.GpuTensor.from_host(dev, scales.view(np.uint16), "f16")))
+            fp, fs = T.fuse_tw_marlin_n(dev, halves, k, [ffn, ffn])
+            plain.append(T.MarlinWeight.from_device(dev, fp, fs, k, 2 * ffn))
+            pairedw.append(T.MarlinWeight.gate_up(dev, halves[0], halves[1], k, ffn))
+            for t in (fp, fs, halves[0][0], halves[0][1], halves[1][0], halves[1][1]):
+                t.free()
+        a1 = T.GpuTensor.from_host(dev, rng.standard_normal(k, dtype=np.float32).astype(np.float16).view(np.uint16), "f16")
+        gate_up = T.GpuTensor.zeros(dev, (2 * ffn,), "f32")
+        g1, u1 = T.GpuTensor.zeros(dev, (ffn,), "f32"), T.GpuTensor.zeros(dev, (ffn,), "f32")
+        act3, act2, act1 = (T.GpuTensor.zeros(dev, (ffn,), "f32") for _ in range(3))
+
+        def three():
+            for w in plain:
+                T.gemm(dev, w, a1, 1, gate_up)
+                T.split_gate_up(dev, gate_up, g1, u1, ffn, 1)
+                T.fused_silu_mul(dev, g1, u1, act3)
+
+        def two():
+            for w in plain:
+                T.gemm_split(dev, w, a1, 1, [g1, u1], [ffn, ffn])
+                T.fused_silu_mul(dev, g1, u1, act2)
+
+        def fused():
+            for w in pairedw:
+                T.gemm_swiglu(dev, w, a1, 1, act1)
+        mlp_front = {"k": k, "ffn": ffn}
+        for label, fn in (("gemv_split_silu_us", three), ("gemv_with_split_store_silu_us", two), ("fused_us", fused)):
+            fn()
+            dev.synchronize()
+            gr = T.GraphCapture.record_with_device(dev, fn)
+            for _ in range(5):
+                gr.replay()
+            dev.synchronize()
+            mlp_front[label] = round(time_launches(dev, lambda i: gr.replay(), 50) / L * 1e3, 2)
+            gr.destroy()
+        assert np.array_equal(act1.to_host(), act3.to_host()), "fused SwiGLU differs from the three-launch sequence"
+        for w in plain + pairedw:
+            w.free()
+
     prefill = None
     if not args.no_prefill:
         prefill = {}
@@ -359,6 +410,8 @@ def main():
     out["small_shapes_m1"] = small
     if lm:
         out["lm_head_m1"] = lm
+    if mlp_front is not None:
+        out["mlp_front_m1"] = mlp_front
     if prefill:
         out["prefill"] = prefill
         best = max(prefill.items(), key=lambda kv: kv[1]["TFLOPs"] if kv[0].startswith("M2048") else 0.0)

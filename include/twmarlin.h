@@ -146,6 +146,23 @@ int twm_split_qkv(twm_ctx *ctx, const float *qkv_dev, float *q_dev, float *k_dev
 int twm_split_gate_up(twm_ctx *ctx, const float *gate_up_dev, float *gate_dev, float *up_dev,
                       uint32_t ffn_dim, uint32_t batch);
 
+/* fused_silu_mul (ops.rs:1139-1155, kernel warp_fused_silu_mul ops.rs:966-976): the SwiGLU gate,
+ * out[i] = gate[i] / (1 + expf(-gate[i])) * up[i] in f32, i < count. */
+int twm_silu_mul(twm_ctx *ctx, const float *gate_dev, const float *up_dev, float *out_dev, size_t count);
+/* split_gate_up + fused_silu_mul in one pass (generate.rs:1086-1093, 2198-2203):
+ * out[b][j] = silu(gate_up[b][gate column j]) * gate_up[b][up column j], gate_up [batch, 2*ffn_dim].
+ * paired = 0: the reference's fused order, gate columns then up columns.
+ * paired = 1: the order of twm_pair_gate_up (ffn_dim must be a multiple of 32). */
+int twm_swiglu_rows(twm_ctx *ctx, const float *gate_up_dev, uint32_t batch, uint32_t ffn_dim, int paired,
+                    float *out_dev);
+/* Like fuse_tw_marlin_n of (gate, up), but with the columns interleaved in runs of 32: output column
+ * 64*(j/32) + j%32 is gate column j and the up column j sits 32 further, so any kernel that owns 64
+ * consecutive columns has both halves of 32 features.  ffn_dim must be a multiple of 32.  Outputs are
+ * TW-Marlin arrays of shape [K/32][2*ffn_dim]; a byte permutation of the reference's fused arrays. */
+int twm_pair_gate_up(twm_ctx *ctx, const uint8_t *gate_packed_dev, const uint16_t *gate_scales_dev,
+                     const uint8_t *up_packed_dev, const uint16_t *up_scales_dev, uint32_t k,
+                     uint32_t ffn_dim, uint8_t *packed_out_dev, uint16_t *scales_out_dev);
+
 /* argmax (crates/kernels/src/missing_ops.rs:24-58): out[row] = first index of the row's maximum, with the
  * reference's starting value: only values > -1e30 compete, a row without any yields 0; NaNs never win.
  * input [rows, cols] f32 row-major, out [rows] i32.  Used on the LM-head logits (generate.rs:1417-1418)
@@ -202,6 +219,21 @@ int twm_gemm(twm_ctx *ctx, const twm_weight *w, const void *a_dev, int a_dtype, 
  * sum(ns) must equal the weight's N; out i is row-major [M, ns[i]] f32. */
 int twm_gemm_split(twm_ctx *ctx, const twm_weight *w, const void *a_dev, int a_dtype, uint32_t m,
                    float *const *outs_dev, const uint32_t *ns, uint32_t count, uint32_t splits);
+/* Gate/up weight for twm_gemm_swiglu: twm_pair_gate_up followed by twm_weight_from_device, with the
+ * handle marked as paired.  twm_gemm / twm_gemm_split on such a handle return the 2*ffn_dim columns
+ * in the paired order. */
+twm_weight *twm_weight_gate_up(twm_ctx *ctx, const uint8_t *gate_packed_dev, const uint16_t *gate_scales_dev,
+                               const uint8_t *up_packed_dev, const uint16_t *up_scales_dev, uint32_t k,
+                               uint32_t ffn_dim);
+int twm_weight_is_paired(const twm_weight *w);
+/* The MLP front half in one call: out[M][ffn_dim] = silu(A x W_gate) * (A x W_up), replacing
+ * gemm_tw_marlin_m1 + split_gate_up + fused_silu_mul (generate.rs:2195-2203).  w must come from
+ * twm_weight_gate_up.  M <= 4: a single launch, the gate is applied in the GEMV's store and the
+ * 2*ffn_dim intermediate never reaches memory.  Larger M: the GEMM writes tmp_dev (f32
+ * [M][2*ffn_dim], may be NULL only when M <= 4) and twm_swiglu_rows follows.  The arithmetic of the
+ * projections is twm_gemm's for the same M. */
+int twm_gemm_swiglu(twm_ctx *ctx, const twm_weight *w, const void *a_dev, int a_dtype, uint32_t m,
+                    float *out_dev, float *tmp_dev, uint32_t splits);
 /* The library's split-K choice for MI355X (256 CUs); same role as quantize.rs:1317-1325. */
 uint32_t twm_pick_splits(uint32_t k, uint32_t n, uint32_t m);
 

@@ -265,6 +265,38 @@ void twmo_split_gate_up(const float *gu, float *gate, float *up, uint32_t ffn, u
     }
 }
 
+/* warp_fused_silu_mul (crates/kernels/src/ops.rs:966-976): g / (1 + expf(-g)) * up, in f32 */
+void twmo_silu_mul(const float *gate, const float *up, float *out, size_t count)
+{
+    for (size_t i = 0; i < count; i++) {
+        float g = gate[i];
+        float silu_g = g / (1.0f + expf(-g));
+        out[i] = silu_g * up[i];
+    }
+}
+
+/* The paired column order of a gate_up weight (no counterpart in the reference, which keeps
+ * [gate | up]): output column 64*(j/32) + j%32 is gate column j, the up column j sits 32 further.
+ * Stated here as a plain gather so the device kernel has an independent twin. */
+void twmo_pair_gate_up(const uint8_t *gate_packed, const uint16_t *gate_scales,
+                       const uint8_t *up_packed, const uint16_t *up_scales, uint32_t k, uint32_t ffn,
+                       uint8_t *packed_out, uint16_t *scales_out)
+{
+    uint32_t G = k / TWM_GROUP;
+    size_t n2 = (size_t)2 * ffn;
+    for (uint32_t g = 0; g < G; g++) {
+        for (uint32_t j = 0; j < ffn; j++) {
+            size_t src = (size_t)g * ffn + j;
+            size_t dg = (size_t)g * n2 + (size_t)(j / 32) * 64 + j % 32;
+            size_t du = dg + 32;
+            memcpy(packed_out + dg * 16, gate_packed + src * 16, 16);
+            memcpy(packed_out + du * 16, up_packed + src * 16, 16);
+            scales_out[dg] = gate_scales[src];
+            scales_out[du] = up_scales[src];
+        }
+    }
+}
+
 /* warp_argmax (crates/kernels/src/missing_ops.rs:24-39): sequential scan, strict '>' from -1e30 at index 0 */
 void twmo_argmax(const float *in, uint32_t rows, uint32_t cols, int32_t *out)
 {

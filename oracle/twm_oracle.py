@@ -135,6 +135,22 @@ def split_gate_up(gu, ffn, batch):
     return g, u
 
 
+def silu_mul(gate, up):
+    gate, up = _c(gate, np.float32), _c(up, np.float32)
+    out = np.zeros(gate.size, np.float32)
+    lib().twmo_silu_mul(_p(gate), _p(up), _p(out), C.c_size_t(gate.size))
+    return out.reshape(gate.shape)
+
+
+def pair_gate_up(gate_packed, gate_scales, up_packed, up_scales, k, ffn):
+    po = np.zeros((k // 32) * 2 * ffn * 16, np.uint8)
+    so = np.zeros((k // 32) * 2 * ffn, np.uint16)
+    lib().twmo_pair_gate_up(_p(_c(gate_packed, np.uint8)), _p(_c(gate_scales, np.uint16)),
+                            _p(_c(up_packed, np.uint8)), _p(_c(up_scales, np.uint16)),
+                            C.c_uint32(k), C.c_uint32(ffn), _p(po), _p(so))
+    return po, so
+
+
 def argmax(x, rows, cols):
     x = _c(x, np.float32)
     out = np.zeros(rows, np.int32)

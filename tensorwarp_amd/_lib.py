@@ -45,6 +45,9 @@ SIGNATURES = {
     "twm_split_qkv": (_int, [_vp, _vp, _vp, _vp, _vp, _u32, _u32, _u32]),
     "twm_argmax_f32": (_int, [_vp, _vp, _u32, _u32, _vp]),
     "twm_split_gate_up": (_int, [_vp, _vp, _vp, _vp, _u32, _u32]),
+    "twm_silu_mul": (_int, [_vp, _vp, _vp, _vp, _sz]),
+    "twm_swiglu_rows": (_int, [_vp, _vp, _u32, _u32, _int, _vp]),
+    "twm_pair_gate_up": (_int, [_vp, _vp, _vp, _vp, _vp, _u32, _u32, _vp, _vp]),
     "twm_gemm_tw_marlin_m1": (_int, [_vp, _vp, _vp, _vp, _vp, _u32, _u32]),
     "twm_gemm_tw_marlin_m1_from_buffer": (_int, [_vp, _vp, _vp, _sz, _vp, _sz, _vp, _u32, _u32]),
     "twm_pick_splits_reference": (None, [_u32, _u32, C.POINTER(_u32), C.POINTER(_u32), C.POINTER(_u32)]),
@@ -56,6 +59,9 @@ SIGNATURES = {
     "twm_weight_dequant_f16": (_int, [_vp, _vp, _vp]),
     "twm_gemm": (_int, [_vp, _vp, _vp, _int, _u32, _vp, _u32]),
     "twm_gemm_split": (_int, [_vp, _vp, _vp, _int, _u32, C.POINTER(_vp), C.POINTER(_u32), _u32, _u32]),
+    "twm_weight_gate_up": (_vp, [_vp, _vp, _vp, _vp, _vp, _u32, _u32]),
+    "twm_weight_is_paired": (_int, [_vp]),
+    "twm_gemm_swiglu": (_int, [_vp, _vp, _vp, _int, _u32, _vp, _vp, _u32]),
     "twm_pick_splits": (_u32, [_u32, _u32, _u32]),
     "twm_graph_begin": (_int, [_vp]),
     "twm_graph_end": (_vp, [_vp]),

@@ -58,6 +58,7 @@ struct twm_weight {
     void *cq;   // column-lane copy: 4608-byte blocks (nibbles + scales together)
     uint32_t k, n, groups, n_tiles, k_chunks;
     size_t bytes;
+    bool paired;  // gate_up weight whose columns are in the paired order (32 gate, 32 up, ...)
 };
 
 struct twm_graph {
@@ -423,6 +424,50 @@ int twm_split_gate_up(twm_ctx *ctx, const float *gate_up_dev, float *gate_dev, f
     return TWM_OK;
 }
 
+int twm_silu_mul(twm_ctx *ctx, const float *gate_dev, const float *up_dev, float *out_dev, size_t count)
+{
+    if (!ctx) return fail(TWM_INVALID_HANDLE, "twm_silu_mul: null context");
+    if (count == 0) return TWM_OK;
+    if (!gate_dev || !up_dev || !out_dev) return fail(TWM_INVALID_HANDLE, "twm_silu_mul: null pointer");
+    HIP_TRY(launch_silu_mul(ctx->stream, gate_dev, up_dev, out_dev, count), TWM_DEVICE_ERROR, "silu_mul launch");
+    return TWM_OK;
+}
+
+int twm_swiglu_rows(twm_ctx *ctx, const float *gate_up_dev, uint32_t batch, uint32_t ffn_dim, int paired, float *out_dev)
+{
+    if (!ctx) return fail(TWM_INVALID_HANDLE, "twm_swiglu_rows: null context");
+    if (paired && ffn_dim % kPairWidth != 0)
+        return fail(TWM_SHAPE_ERROR, "twm_swiglu_rows: the paired order needs ffn_dim %% %u == 0, got %u", kPairWidth, ffn_dim);
+    if ((uint64_t)ffn_dim * 2 > 0xFFFFFFFFull) return fail(TWM_SHAPE_ERROR, "twm_swiglu_rows: 2 * ffn_dim overflows u32");
+    if ((uint64_t)batch * ffn_dim == 0) return TWM_OK;
+    if (!gate_up_dev || !out_dev) return fail(TWM_INVALID_HANDLE, "twm_swiglu_rows: null pointer");
+    HIP_TRY(launch_swiglu_rows(ctx->stream, gate_up_dev, out_dev, ffn_dim, batch, paired != 0), TWM_DEVICE_ERROR,
+            "swiglu_rows launch");
+    return TWM_OK;
+}
+
+static int check_pair_args(const char *who, uint32_t k, uint32_t ffn_dim)
+{
+    if (ffn_dim % kPairWidth != 0) return fail(TWM_SHAPE_ERROR, "%s: ffn_dim must be a multiple of %u, got %u", who, kPairWidth, ffn_dim);
+    if ((uint64_t)ffn_dim * 2 > 0xFFFFFFFFull) return fail(TWM_SHAPE_ERROR, "%s: 2 * ffn_dim overflows u32", who);
+    return check_kn(who, k, ffn_dim * 2);
+}
+
+int twm_pair_gate_up(twm_ctx *ctx, const uint8_t *gate_packed_dev, const uint16_t *gate_scales_dev,
+                     const uint8_t *up_packed_dev, const uint16_t *up_scales_dev, uint32_t k, uint32_t ffn_dim,
+                     uint8_t *packed_out_dev, uint16_t *scales_out_dev)
+{
+    if (!ctx) return fail(TWM_INVALID_HANDLE, "twm_pair_gate_up: null context");
+    if (int rc = check_pair_args("twm_pair_gate_up", k, ffn_dim)) return rc;
+    if (k == 0 || ffn_dim == 0) return TWM_OK;
+    if (!gate_packed_dev || !gate_scales_dev || !up_packed_dev || !up_scales_dev || !packed_out_dev || !scales_out_dev)
+        return fail(TWM_INVALID_HANDLE, "twm_pair_gate_up: null pointer");
+    HIP_TRY(launch_pair_gate_up(ctx->stream, gate_packed_dev, gate_scales_dev, up_packed_dev, up_scales_dev, k / 32,
+                                ffn_dim, packed_out_dev, scales_out_dev),
+            TWM_DEVICE_ERROR, "pair_gate_up launch");
+    return TWM_OK;
+}
+
 /* ---- GEMV on the reference layout ------------------------------------------------------- */
 
 void twm_pick_splits_reference(uint32_t k, uint32_t n, uint32_t *n_blocks, uint32_t *splits, uint32_t *groups_per_split)
@@ -490,6 +535,7 @@ static twm_weight *weight_alloc(twm_ctx *ctx, uint32_t k, uint32_t n)
     size_t qbytes = tiles * 1024, sbytes = tiles * 128;
     w->bytes = 2 * (qbytes + sbytes);
     w->qw = w->sc = w->cq = nullptr;
+    w->paired = false;
     if (tiles == 0) return w;
     hipError_t e = hipMalloc(&w->qw, w->bytes);
     if (e != hipSuccess) {
@@ -550,6 +596,35 @@ twm_weight *twm_weight_upload(twm_ctx *ctx, const uint8_t *packed_host, const ui
     (void)hipFree(stage);
     return w;
 }
+
+twm_weight *twm_weight_gate_up(twm_ctx *ctx, const uint8_t *gate_packed_dev, const uint16_t *gate_scales_dev,
+                               const uint8_t *up_packed_dev, const uint16_t *up_scales_dev, uint32_t k, uint32_t ffn_dim)
+{
+    if (!ctx) { fail(TWM_INVALID_HANDLE, "twm_weight_gate_up: null context"); return nullptr; }
+    if (ctx->capturing) { fail(TWM_UNSUPPORTED_OP, "twm_weight_gate_up: not allowed inside a graph capture"); return nullptr; }
+    if (check_pair_args("twm_weight_gate_up", k, ffn_dim)) return nullptr;
+    uint32_t n = ffn_dim * 2;
+    size_t pbytes = (size_t)(k / 32) * n * 16, sbytes = (size_t)(k / 32) * n * 2;
+    twm_weight *w = nullptr;
+    if (pbytes == 0) {
+        w = twm_weight_from_device(ctx, nullptr, nullptr, k, n);
+    } else {
+        void *stage = nullptr;
+        hipError_t e = hipMalloc(&stage, pbytes + sbytes);
+        if (e != hipSuccess) { fail(TWM_MEMORY_ERROR, "twm_weight_gate_up: staging hipMalloc: %s", hipGetErrorString(e)); return nullptr; }
+        uint8_t *p = (uint8_t *)stage;
+        uint16_t *sc = (uint16_t *)(p + pbytes);
+        if (twm_pair_gate_up(ctx, gate_packed_dev, gate_scales_dev, up_packed_dev, up_scales_dev, k, ffn_dim, p, sc) == TWM_OK)
+            w = twm_weight_from_device(ctx, p, sc, k, n);  // synchronises the stream before returning
+        else
+            (void)hipStreamSynchronize(ctx->stream);
+        (void)hipFree(stage);
+    }
+    if (w) w->paired = true;
+    return w;
+}
+
+int twm_weight_is_paired(const twm_weight *w) { return w && w->paired ? 1 : 0; }
 
 void twm_weight_destroy(twm_weight *w)
 {
@@ -683,8 +758,10 @@ uint32_t twm_pick_splits(uint32_t k, uint32_t n, uint32_t m)
     return plan_stream(n_tiles, k_chunks, m);
 }
 
+// swiglu_out (only with m <= 4 on the one-lane-per-column kernel, paired weight): the launch writes
+// silu(gate) * up to swiglu_out[m][n/2] instead of the columns to `out`.
 static int gemm_common(twm_ctx *ctx, const twm_weight *w, const void *a_dev, int a_dtype, uint32_t m, const OutSpec &out,
-                       uint32_t splits, const char *who)
+                       uint32_t splits, const char *who, float *swiglu_out = nullptr)
 {
     if (a_dtype != TWM_F16 && a_dtype != TWM_F32) return fail(TWM_UNSUPPORTED_OP, "%s: activations must be f16 or f32", who);
     if (m == 0 || w->n == 0) return TWM_OK;
@@ -698,6 +775,8 @@ static int gemm_common(twm_ctx *ctx, const twm_weight *w, const void *a_dev, int
     WeightView v = view_of(w);
     size_t a_row_bytes = (size_t)w->k * (a_dtype == TWM_F16 ? 2 : 4);
     uint32_t n_ld = w->n_tiles * kTileN;
+    if (swiglu_out && !(m <= 4 && m < (uint32_t)ctx->prefill_min_m && ctx->force_kernel != 1 && ctx->force_kernel != 3))
+        return fail(TWM_UNSUPPORTED_OP, "%s: the fused SwiGLU epilogue exists for M <= 4 on the one-lane-per-column kernel", who);
     if (m >= (uint32_t)ctx->prefill_min_m) {
         HIP_TRY(launch_prefill(ctx->stream, v, a_dev, a_dtype == TWM_F32, m, out, (uint32_t)ctx->prefill_bm, splits, ctx->ws, ctx->ws_bytes), TWM_DEVICE_ERROR, "prefill launch");
         return TWM_OK;
@@ -730,7 +809,7 @@ static int gemm_common(twm_ctx *ctx, const twm_weight *w, const void *a_dev, int
         const char *a_blk = (const char *)a_dev + (size_t)m0 * a_row_bytes;
         if (lane_col)
             HIP_TRY(launch_gemv4(ctx->stream, v, a_blk, a_dtype == TWM_F32, mb, o, ctx->ws, ctx->counters, plan.nt,
-                                 plan.waves, plan.splits),
+                                 plan.waves, plan.splits, swiglu_out ? swiglu_out + (size_t)m0 * (w->n / 2) : nullptr),
                     TWM_DEVICE_ERROR, "gemv launch");
         else
             HIP_TRY(launch_decode(ctx->stream, v, a_blk, a_dtype == TWM_F32, mb, o, ctx->ws, ctx->counters, plan),
@@ -778,6 +857,30 @@ int twm_gemm_split(twm_ctx *ctx, const twm_weight *w, const void *a_dev, int a_d
     if (total != w->n) return fail(TWM_SHAPE_ERROR, "twm_gemm_split: outputs cover %llu columns, weight has %u",
                                    (unsigned long long)total, w->n);
     return gemm_common(ctx, w, a_dev, a_dtype, m, out, splits, "twm_gemm_split");
+}
+
+int twm_gemm_swiglu(twm_ctx *ctx, const twm_weight *w, const void *a_dev, int a_dtype, uint32_t m, float *out_dev,
+                    float *tmp_dev, uint32_t splits)
+{
+    if (!ctx || !w) return fail(TWM_INVALID_HANDLE, "twm_gemm_swiglu: null handle");
+    if (w->ctx != ctx) return fail(TWM_INVALID_HANDLE, "twm_gemm_swiglu: weight belongs to another context");
+    if (!w->paired) return fail(TWM_UNSUPPORTED_OP, "twm_gemm_swiglu: the weight was not built by twm_weight_gate_up");
+    uint32_t ffn = w->n / 2;
+    if (m == 0 || ffn == 0) return TWM_OK;
+    if (!out_dev) return fail(TWM_INVALID_HANDLE, "twm_gemm_swiglu: null output");
+    if (w->k == 0) return twm_memset_zero(ctx, out_dev, (size_t)m * ffn * 4);  // silu(0) * 0
+    OutSpec out;
+    memset(&out, 0, sizeof out);
+    bool fused = m <= 4 && m < (uint32_t)ctx->prefill_min_m && ctx->force_kernel != 1 && ctx->force_kernel != 3;
+    if (fused) return gemm_common(ctx, w, a_dev, a_dtype, m, out, splits, "twm_gemm_swiglu", out_dev);
+    if (!tmp_dev) return fail(TWM_INVALID_HANDLE, "twm_gemm_swiglu: M = %u needs the [M][2*ffn] f32 temporary", m);
+    out.count = 1;
+    out.seg[0].ptr = tmp_dev;
+    out.seg[0].start = 0;
+    out.seg[0].width = w->n;
+    if (int rc = gemm_common(ctx, w, a_dev, a_dtype, m, out, splits, "twm_gemm_swiglu")) return rc;
+    HIP_TRY(launch_swiglu_rows(ctx->stream, tmp_dev, out_dev, ffn, m, true), TWM_DEVICE_ERROR, "swiglu_rows launch");
+    return TWM_OK;
 }
 
 /* ---- graphs ---------------------------------------------------------------------------------- */

@@ -83,7 +83,7 @@ template <int NT, int RL, bool AF32>
 __global__ __launch_bounds__(1024) void k_gemv4(const char *__restrict__ cw, const void *__restrict__ a_any,
                                                  OutSpec out, float *__restrict__ ws, unsigned *__restrict__ counters, uint32_t m_rows, uint32_t k,
                                                  uint32_t n, uint32_t n_pad, uint32_t k_chunks, uint32_t tile_groups,
-                                                 uint32_t splits, uint32_t cps)
+                                                 uint32_t splits, uint32_t cps, float *__restrict__ swiglu_out)
 {
     extern __shared__ float red[];  // [waves][NT][RL][64]
     __shared__ int s_last;
@@ -195,7 +195,27 @@ __global__ __launch_bounds__(1024) void k_gemv4(const char *__restrict__ cw, con
 
     const uint32_t threads = blockDim.x;
     const uint32_t entries = NT * RL * 64;  // entry e = (t*RL + r)*64 + lane
+    // Paired gate_up weight: every 64-column tile holds 32 gate columns followed by the up columns of the
+    // same 32 features, so the thread that sums lane ln < 32 also sums lane ln + 32 and writes silu(gate) * up.
+    const bool swiglu = swiglu_out != nullptr;
+    const uint32_t ffn = n >> 1;
+    const uint32_t pair_entries = NT * RL * 32;  // entry e = (t*RL + r)*32 + ln
     if (splits == 1) {
+        if (swiglu) {
+            for (uint32_t e = threadIdx.x; e < pair_entries; e += threads) {
+                uint32_t ln = e & 31u, tr = e >> 5, r = tr % RL, t = tr / RL;
+                uint32_t feat = (tg * NT + t) * 32u + ln;
+                if (r < m_rows && feat < ffn) {
+                    float g = 0.f, u = 0.f;
+                    for (uint32_t w = 0; w < waves; w++) {
+                        g += red[(w * NT * RL + tr) * 64 + ln];
+                        u += red[(w * NT * RL + tr) * 64 + 32 + ln];
+                    }
+                    swiglu_out[(size_t)r * ffn + feat] = silu_mul_f32(g, u);
+                }
+            }
+            return;
+        }
         for (uint32_t e = threadIdx.x; e < entries; e += threads) {
             uint32_t ln = e & 63u, tr = e >> 6, r = tr % RL, t = tr / RL;
             uint32_t on = (tg * NT + t) * 64u + ln;
@@ -228,6 +248,23 @@ __global__ __launch_bounds__(1024) void k_gemv4(const char *__restrict__ cw, con
     }
     __syncthreads();
     if (!s_last) return;
+    if (swiglu) {
+        for (uint32_t e = threadIdx.x; e < pair_entries; e += threads) {
+            uint32_t ln = e & 31u, tr = e >> 5, r = tr % RL, t = tr / RL;
+            uint32_t feat = (tg * NT + t) * 32u + ln, on = (tg * NT + t) * 64u + ln;
+            if (r < m_rows && feat < ffn) {
+                float g = 0.f, u = 0.f;
+                for (uint32_t s = 0; s < splits; s++) {
+                    const float *row = &ws[((size_t)s * m_rows + r) * n_pad + on];
+                    g += __hip_atomic_load(row, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    u += __hip_atomic_load(row + 32, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                }
+                swiglu_out[(size_t)r * ffn + feat] = silu_mul_f32(g, u);
+            }
+        }
+        if (threadIdx.x == 0) __hip_atomic_store(&counters[tg], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        return;
+    }
     for (uint32_t e = threadIdx.x; e < entries; e += threads) {
         uint32_t ln = e & 63u, tr = e >> 6, r = tr % RL, t = tr / RL;
         uint32_t on = (tg * NT + t) * 64u + ln;
@@ -243,7 +280,8 @@ __global__ __launch_bounds__(1024) void k_gemv4(const char *__restrict__ cw, con
 
 template <int NT, int RL>
 static hipError_t launch_gemv4_t(hipStream_t s, const WeightView &w, const void *a, bool a_f32, uint32_t m,
-                                 const OutSpec &out, float *ws, unsigned *counters, uint32_t waves, uint32_t splits)
+                                 const OutSpec &out, float *ws, unsigned *counters, uint32_t waves, uint32_t splits,
+                                 float *swiglu_out)
 {
     uint32_t n_pad = w.n_tiles * kTileN;                 // multiple of 64
     uint32_t tiles64 = n_pad / 64;
@@ -255,18 +293,19 @@ static hipError_t launch_gemv4_t(hipStream_t s, const WeightView &w, const void 
     if (a_f32)
         hipLaunchKernelGGL((k_gemv4<NT, RL, true>), dim3(blocks), dim3(waves * 64), lds, s, (const char *)w.cq, a, out, ws,
                            counters, m, w.k, w.n, n_pad, w.k_chunks, tile_groups,
-                           splits, cps);
+                           splits, cps, swiglu_out);
     else
         hipLaunchKernelGGL((k_gemv4<NT, RL, false>), dim3(blocks), dim3(waves * 64), lds, s, (const char *)w.cq, a, out, ws,
                            counters, m, w.k, w.n, n_pad, w.k_chunks, tile_groups,
-                           splits, cps);
+                           splits, cps, swiglu_out);
     return hipGetLastError();
 }
 
 hipError_t launch_gemv4(hipStream_t s, const WeightView &w, const void *a, bool a_f32, uint32_t m, const OutSpec &out,
-                        float *ws, unsigned *counters, uint32_t nt, uint32_t waves, uint32_t splits)
+                        float *ws, unsigned *counters, uint32_t nt, uint32_t waves, uint32_t splits, float *swiglu_out)
 {
     if (m == 0 || w.n == 0) return hipSuccess;
+    if (swiglu_out && w.n % 64 != 0) return hipErrorInvalidValue;
     if (m > 4 || splits == 0 || !w.cq) return hipErrorInvalidValue;
     if (waves != 1 && waves != 2 && waves != 4 && waves != 8 && waves != 16) return hipErrorInvalidValue;
     // a tile group past the end of the padded columns must not exist: NT has to divide the 64-column tile count
@@ -274,14 +313,14 @@ hipError_t launch_gemv4(hipStream_t s, const WeightView &w, const void *a, bool 
     if (nt == 0 || tiles64 % nt != 0) return hipErrorInvalidValue;
     uint32_t rl = m;  // rows 0..m-1 live in registers 0..m-1
     if (nt == 1) {
-        if (rl == 1) return launch_gemv4_t<1, 1>(s, w, a, a_f32, m, out, ws, counters, waves, splits);
-        if (rl == 2) return launch_gemv4_t<1, 2>(s, w, a, a_f32, m, out, ws, counters, waves, splits);
-        return launch_gemv4_t<1, 4>(s, w, a, a_f32, m, out, ws, counters, waves, splits);
+        if (rl == 1) return launch_gemv4_t<1, 1>(s, w, a, a_f32, m, out, ws, counters, waves, splits, swiglu_out);
+        if (rl == 2) return launch_gemv4_t<1, 2>(s, w, a, a_f32, m, out, ws, counters, waves, splits, swiglu_out);
+        return launch_gemv4_t<1, 4>(s, w, a, a_f32, m, out, ws, counters, waves, splits, swiglu_out);
     }
     if (nt == 2) {
-        if (rl == 1) return launch_gemv4_t<2, 1>(s, w, a, a_f32, m, out, ws, counters, waves, splits);
-        if (rl == 2) return launch_gemv4_t<2, 2>(s, w, a, a_f32, m, out, ws, counters, waves, splits);
-        return launch_gemv4_t<2, 4>(s, w, a, a_f32, m, out, ws, counters, waves, splits);
+        if (rl == 1) return launch_gemv4_t<2, 1>(s, w, a, a_f32, m, out, ws, counters, waves, splits, swiglu_out);
+        if (rl == 2) return launch_gemv4_t<2, 2>(s, w, a, a_f32, m, out, ws, counters, waves, splits, swiglu_out);
+        return launch_gemv4_t<2, 4>(s, w, a, a_f32, m, out, ws, counters, waves, splits, swiglu_out);
     }
     return hipErrorInvalidValue;
 }

@@ -23,6 +23,12 @@ constexpr int kMaxDecodeM = 16;     // rows per launch of the tile kernel (one 1
 constexpr int kMaxStreamM = 32;     // rows per launch of the batched-decode streaming kernel
 constexpr uint32_t kColBlockBytes = 4608;  // column-lane copy: 4 x 1024 B of nibbles + 512 B of scales per (tile, chunk)
 
+// Column order of a "paired" gate_up weight: 32 gate columns, then the 32 up columns of the same
+// features, and so on, so that every 64-column tile a kernel owns holds both halves of its features.
+// Column j of gate sits at paired_col(j), column j of up kPairWidth further.
+constexpr uint32_t kPairWidth = 32;
+__host__ __device__ __forceinline__ uint32_t paired_col(uint32_t j) { return (j >> 5) * 64u + (j & 31u); }
+
 struct OutSeg {
     float *ptr;
     uint32_t start;  // first fused column of this segment
@@ -60,6 +66,11 @@ hipError_t launch_dequant(hipStream_t s, const uint8_t *packed, const uint16_t *
 hipError_t launch_split_qkv(hipStream_t s, const float *qkv, float *q, float *kk, float *v, uint32_t h,
                             uint32_t kv, uint32_t batch);
 hipError_t launch_split_gate_up(hipStream_t s, const float *gu, float *g, float *u, uint32_t ffn, uint32_t batch);
+hipError_t launch_silu_mul(hipStream_t s, const float *gate, const float *up, float *out, size_t count);
+hipError_t launch_swiglu_rows(hipStream_t s, const float *gu, float *out, uint32_t ffn, uint32_t batch, bool paired);
+hipError_t launch_pair_gate_up(hipStream_t s, const uint8_t *gate_packed, const uint16_t *gate_scales,
+                               const uint8_t *up_packed, const uint16_t *up_scales, uint32_t groups, uint32_t ffn,
+                               uint8_t *packed_out, uint16_t *scales_out);
 hipError_t launch_argmax(hipStream_t s, const float *in, uint32_t rows, uint32_t cols, int *out, void *scratch,
                          size_t scratch_bytes);
 hipError_t launch_ref_gemv(hipStream_t s, const float *a, const uint8_t *packed, const uint16_t *scales, float *c,
@@ -70,8 +81,11 @@ hipError_t launch_weight_dequant_f16(hipStream_t s, const WeightView &w, uint16_
 hipError_t launch_repack_col(hipStream_t s, const uint8_t *packed, const uint16_t *scales, uint32_t k, uint32_t n,
                              void *cq, uint32_t n_pad, uint32_t k_chunks);
 hipError_t launch_weight_dequant_f16_col(hipStream_t s, const WeightView &w, uint16_t *out_kn);
+// swiglu_out != nullptr (the weight in the paired gate_up column order, N = 2*ffn a multiple of 64): instead
+// of the N columns, write silu(gate) * up of every feature to swiglu_out[m][ffn]; `out` is ignored.
 hipError_t launch_gemv4(hipStream_t s, const WeightView &w, const void *a, bool a_f32, uint32_t m, const OutSpec &out,
-                        float *ws, unsigned *counters, uint32_t nt, uint32_t waves, uint32_t splits);
+                        float *ws, unsigned *counters, uint32_t nt, uint32_t waves, uint32_t splits,
+                        float *swiglu_out = nullptr);
 hipError_t init_prefill();
 hipError_t launch_prefill(hipStream_t s, const WeightView &w, const void *a, bool a_f32, uint32_t m, const OutSpec &out,
                           uint32_t block_rows, uint32_t splits, void *scratch, size_t scratch_bytes);

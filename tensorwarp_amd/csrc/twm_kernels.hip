@@ -263,6 +263,55 @@ __global__ __launch_bounds__(256) void k_split_gate_up(const float *__restrict__
     else u[(size_t)b * ffn + (d - ffn)] = x;
 }
 
+// silu(gate) * up, elementwise (warp_fused_silu_mul, crates/kernels/src/ops.rs:966-976).
+__global__ __launch_bounds__(256) void k_silu_mul(const float *__restrict__ gate, const float *__restrict__ up,
+                                                   float *__restrict__ out, size_t count)
+{
+    size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx < count) out[idx] = silu_mul_f32(gate[idx], up[idx]);
+}
+
+// out[b][j] = silu(gate_up[b][gate column j]) * gate_up[b][up column j]: the split of
+// k_split_gate_up and the SwiGLU gate in one pass.  PAIRED selects where the two columns are:
+// [gate | up] halves (the reference's fused order) or the 32-column interleave of paired_col().
+template <bool PAIRED>
+__global__ __launch_bounds__(256) void k_swiglu_rows(const float *__restrict__ gu, float *__restrict__ out,
+                                                      uint32_t ffn, uint32_t batch)
+{
+    size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= (size_t)batch * ffn) return;
+    uint32_t b = (uint32_t)(idx / ffn), j = (uint32_t)(idx % ffn);
+    const float *row = gu + (size_t)b * 2 * ffn;
+    float g, u;
+    if (PAIRED) {
+        uint32_t c = paired_col(j);
+        g = row[c];
+        u = row[c + kPairWidth];
+    } else {
+        g = row[j];
+        u = row[ffn + j];
+    }
+    out[idx] = silu_mul_f32(g, u);
+}
+
+// TW-Marlin arrays of gate and up ([G][ffn] records and scales each) -> one [G][2*ffn] pair of
+// arrays in the paired column order.  Pure byte moves; one thread per (group, output column).
+__global__ __launch_bounds__(256) void k_pair_gate_up(const uint4v *__restrict__ gp, const uint16_t *__restrict__ gs,
+                                                       const uint4v *__restrict__ up, const uint16_t *__restrict__ us,
+                                                       uint32_t groups, uint32_t ffn, uint4v *__restrict__ pout,
+                                                       uint16_t *__restrict__ sout)
+{
+    size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;  // g * 2*ffn + c
+    size_t n2 = (size_t)2 * ffn;
+    if (idx >= (size_t)groups * n2) return;
+    uint32_t g = (uint32_t)(idx / n2), c = (uint32_t)(idx % n2);
+    uint32_t j = (c >> 6) * kPairWidth + (c & 31u);
+    size_t src = (size_t)g * ffn + j;
+    bool is_up = (c & kPairWidth) != 0;
+    pout[idx] = is_up ? up[src] : gp[src];
+    sout[idx] = is_up ? us[src] : gs[src];
+}
+
 // ArgMax along the last dimension with the reference's rule (crates/kernels/src/missing_ops.rs:24-39): the
 // first index whose value is greater than every earlier candidate, starting from -1e30 at index 0 (so
 // values <= -1e30 and NaNs are never chosen, and an empty or all-small row yields 0).  One workgroup per row:
@@ -408,6 +457,35 @@ hipError_t launch_split_gate_up(hipStream_t s, const float *gu, float *g, float 
     size_t total = (size_t)batch * 2 * ffn;
     if (total == 0) return hipSuccess;
     hipLaunchKernelGGL(k_split_gate_up, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, gu, g, u, ffn, batch);
+    return hipGetLastError();
+}
+
+hipError_t launch_silu_mul(hipStream_t s, const float *gate, const float *up, float *out, size_t count)
+{
+    if (count == 0) return hipSuccess;
+    hipLaunchKernelGGL(k_silu_mul, dim3((unsigned)((count + 255) / 256)), dim3(256), 0, s, gate, up, out, count);
+    return hipGetLastError();
+}
+
+hipError_t launch_swiglu_rows(hipStream_t s, const float *gu, float *out, uint32_t ffn, uint32_t batch, bool paired)
+{
+    size_t total = (size_t)batch * ffn;
+    if (total == 0) return hipSuccess;
+    dim3 grid((unsigned)((total + 255) / 256));
+    if (paired) hipLaunchKernelGGL(k_swiglu_rows<true>, grid, dim3(256), 0, s, gu, out, ffn, batch);
+    else hipLaunchKernelGGL(k_swiglu_rows<false>, grid, dim3(256), 0, s, gu, out, ffn, batch);
+    return hipGetLastError();
+}
+
+hipError_t launch_pair_gate_up(hipStream_t s, const uint8_t *gate_packed, const uint16_t *gate_scales,
+                               const uint8_t *up_packed, const uint16_t *up_scales, uint32_t groups, uint32_t ffn,
+                               uint8_t *packed_out, uint16_t *scales_out)
+{
+    size_t total = (size_t)groups * 2 * ffn;
+    if (total == 0) return hipSuccess;
+    hipLaunchKernelGGL(k_pair_gate_up, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s,
+                       (const uint4v *)gate_packed, gate_scales, (const uint4v *)up_packed, up_scales, groups, ffn,
+                       (uint4v *)packed_out, scales_out);
     return hipGetLastError();
 }
 

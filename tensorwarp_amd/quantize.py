@@ -220,6 +220,27 @@ def split_gate_up(device, gate_up, gate, up, ffn_dim, batch):
     _check(device._l.twm_split_gate_up(device.handle, gate_up.ptr, gate.ptr, up.ptr, ffn_dim, batch))
 
 
+def fused_silu_mul(device, gate, up, out):
+    """ops.rs:1139 — out = silu(gate) * up, elementwise f32."""
+    _check(device._l.twm_silu_mul(device.handle, gate.ptr, up.ptr, out.ptr, gate.numel))
+
+
+def swiglu_rows(device, gate_up, out, ffn_dim, batch, paired=False):
+    """split_gate_up + fused_silu_mul in one pass; paired=True reads the order of pair_gate_up."""
+    _check(device._l.twm_swiglu_rows(device.handle, gate_up.ptr, batch, ffn_dim, int(paired), out.ptr))
+
+
+def pair_gate_up(device, gate, up, k, ffn_dim):
+    """(packed, scales) of gate and up -> TW-Marlin arrays [K/32][2*ffn] with the columns interleaved in runs
+    of 32 (gate, up, gate, ...), the order the fused SwiGLU GEMV reads."""
+    g = k // 32
+    po = GpuTensor(device, (g * 2 * ffn_dim * 16,), "u8")
+    so = GpuTensor(device, (g * 2 * ffn_dim,), "f16")
+    _check(device._l.twm_pair_gate_up(device.handle, gate[0].ptr, gate[1].ptr, up[0].ptr, up[1].ptr, k, ffn_dim,
+                                      po.ptr, so.ptr))
+    return po, so
+
+
 def argmax(device, input, output, rows, cols):
     """missing_ops.rs:42 — input f32 [rows, cols], output i32 [rows]."""
     _check(device._l.twm_argmax_f32(device.handle, input.ptr, rows, cols, output.ptr))
@@ -258,6 +279,19 @@ class MarlinWeight:
             raise DeviceError(_lib.SHAPE_ERROR if k % 32 else _lib.DEVICE_ERROR, device._l.twm_last_error().decode())
         return cls(device, h, k, n)
 
+    @classmethod
+    def gate_up(cls, device, gate, up, k, ffn_dim):
+        """Paired gate/up weight for gemm_swiglu; gate and up are (packed, scales) device pairs."""
+        h = device._l.twm_weight_gate_up(device.handle, gate[0].ptr, gate[1].ptr, up[0].ptr, up[1].ptr, k, ffn_dim)
+        if not h:
+            raise DeviceError(_lib.SHAPE_ERROR if (k % 32 or ffn_dim % 32) else _lib.DEVICE_ERROR,
+                              device._l.twm_last_error().decode())
+        return cls(device, h, k, 2 * ffn_dim)
+
+    @property
+    def paired(self):
+        return bool(self.device._l.twm_weight_is_paired(self.handle))
+
     @property
     def nbytes(self):
         return self.device._l.twm_weight_bytes(self.handle)
@@ -277,6 +311,14 @@ def gemm(device, weight, a, m, c, splits=0):
     """C[M,N] f32 = A[M,K] (f16 or f32) x dequant(weight). M=1 is gemm_tw_marlin_m1."""
     dt = _lib.F16 if a.dtype == "f16" else _lib.F32
     _check(device._l.twm_gemm(device.handle, weight.handle, a.ptr, dt, m, c.ptr, splits))
+
+
+def gemm_swiglu(device, weight, a, m, out, tmp=None, splits=0):
+    """out[M, ffn] = silu(A x W_gate) * (A x W_up) on a MarlinWeight.gate_up weight: gemm_tw_marlin_m1 +
+    split_gate_up + fused_silu_mul of the decode step in one launch for M <= 4; larger M needs tmp [M, 2*ffn]."""
+    dt = _lib.F16 if a.dtype == "f16" else _lib.F32
+    _check(device._l.twm_gemm_swiglu(device.handle, weight.handle, a.ptr, dt, m, out.ptr,
+                                     tmp.ptr if tmp is not None else None, splits))
 
 
 def gemm_split(device, weight, a, m, outs, ns, splits=0):

@@ -121,6 +121,126 @@ def test_split_kernels(dev):
     assert np.array_equal(g.to_host(), og) and np.array_equal(u.to_host(), ou)
 
 
+def silu_close(got, want):
+    """f32 results of g / (1 + expf(-g)) * u from two correctly working libm's differ by a few ulps at most."""
+    got, want = np.asarray(got, np.float64), np.asarray(want, np.float64)
+    return bool(np.all(np.abs(got - want) <= 2e-6 * np.abs(want) + 1e-37))
+
+
+def test_silu_mul_and_swiglu_rows(dev):
+    batch, ffn = 3, 160
+    gu = (O.synth_normal_f32(batch * 2 * ffn, 930) * np.float32(3.0)).reshape(batch, 2 * ffn)
+    gu[0, :6] = [0.0, -0.0, 90.0, -90.0, 1e4, -1e4]
+    g, u = np.ascontiguousarray(gu[:, :ffn]), np.ascontiguousarray(gu[:, ffn:])
+    want = O.silu_mul(g, u)
+    gd, ud = T.GpuTensor.from_host(dev, g), T.GpuTensor.from_host(dev, u)
+    out = T.GpuTensor.zeros(dev, (batch, ffn), "f32")
+    T.fused_silu_mul(dev, gd, ud, out)
+    assert silu_close(out.to_host(), want)
+    first = out.to_host().copy()
+    # split + gate in one pass, on the reference's [gate | up] order: the same bits as the two-step route
+    out2 = T.GpuTensor.zeros(dev, (batch, ffn), "f32")
+    T.swiglu_rows(dev, T.GpuTensor.from_host(dev, gu), out2, ffn, batch)
+    assert np.array_equal(out2.to_host(), first)
+    # and on the paired order
+    j = np.arange(ffn)
+    col = (j // 32) * 64 + j % 32
+    paired = np.zeros_like(gu)
+    paired[:, col] = g
+    paired[:, col + 32] = u
+    out3 = T.GpuTensor.zeros(dev, (batch, ffn), "f32")
+    T.swiglu_rows(dev, T.GpuTensor.from_host(dev, paired), out3, ffn, batch, paired=True)
+    assert np.array_equal(out3.to_host(), first)
+    with pytest.raises(T.DeviceError):
+        T.swiglu_rows(dev, T.GpuTensor.from_host(dev, paired), out3, 40, 1, paired=True)
+
+
+def test_pair_gate_up_bit_exact(dev):
+    k, ffn = 128, 224
+    gp, gs = O.synth_packed(k, ffn, 940), O.synth_scales(k, ffn, 941)
+    up, us = O.synth_packed(k, ffn, 942), O.synth_scales(k, ffn, 943)
+    gd = (T.GpuTensor.from_host(dev, gp), T.GpuTensor.from_host(dev, gs, "f16"))
+    ud = (T.GpuTensor.from_host(dev, up), T.GpuTensor.from_host(dev, us, "f16"))
+    pp, ps = T.pair_gate_up(dev, gd, ud, k, ffn)
+    op, os_ = O.pair_gate_up(gp, gs, up, us, k, ffn)
+    assert np.array_equal(pp.to_host(), op) and np.array_equal(ps.to_host(), os_)
+    with pytest.raises(T.DeviceError):
+        T.pair_gate_up(dev, gd, ud, k, 48)   # not a multiple of 32
+
+
+@pytest.mark.parametrize("h,ffn,m,splits", [(896, 4864, 1, 0), (896, 4864, 3, 0), (3584, 18944, 1, 0),
+                                            (3584, 18944, 4, 0), (2048, 96, 1, 0), (2048, 96, 2, 4),
+                                            (256, 32, 1, 1), (1184, 160, 4, 3)])
+def test_gemm_swiglu_fused_epilogue(dev, h, ffn, m, splits):
+    # gemm_tw_marlin_m1 + split_gate_up + fused_silu_mul (generate.rs:2195-2203) against the single launch
+    gp, gs = O.synth_packed(h, ffn, 950), O.synth_scales(h, ffn, 951)
+    up, us = O.synth_packed(h, ffn, 952), O.synth_scales(h, ffn, 953)
+    gd = (T.GpuTensor.from_host(dev, gp), T.GpuTensor.from_host(dev, gs, "f16"))
+    ud = (T.GpuTensor.from_host(dev, up), T.GpuTensor.from_host(dev, us, "f16"))
+    a16 = O.synth_act_f16(m, h, 954)
+    ad = T.GpuTensor.from_host(dev, a16, "f16")
+    # the reference's sequence on the [gate | up] weight
+    fp, fs = T.fuse_tw_marlin_n(dev, [gd, ud], h, [ffn, ffn])
+    plain = T.MarlinWeight.from_device(dev, fp, fs, h, 2 * ffn)
+    gate_up = T.GpuTensor.zeros(dev, (m, 2 * ffn), "f32")
+    T.gemm(dev, plain, ad, m, gate_up, splits)
+    g, u = T.GpuTensor.zeros(dev, (m, ffn), "f32"), T.GpuTensor.zeros(dev, (m, ffn), "f32")
+    T.split_gate_up(dev, gate_up, g, u, ffn, m)
+    seq = T.GpuTensor.zeros(dev, (m, ffn), "f32")
+    T.fused_silu_mul(dev, g, u, seq)
+    # one launch on the paired weight
+    w = T.MarlinWeight.gate_up(dev, gd, ud, h, ffn)
+    assert w.paired and not plain.paired
+    out = T.GpuTensor.from_host(dev, np.full((m, ffn), np.nan, np.float32))
+    T.gemm_swiglu(dev, w, ad, m, out, None, splits)
+    assert np.array_equal(out.to_host(), seq.to_host())
+    # against the oracle: f64 projections, then the reference's gate in f32 (its input differs from the
+    # GPU's by the GEMV's rounding, so the bar is the GEMV's)
+    a = f16_as_f32(a16).reshape(m, h)
+    tg, tu = O.gemm_f64(a, gp, gs, m, h, ffn), O.gemm_f64(a, up, us, m, h, ffn)
+    truth = tg / (1.0 + np.exp(-tg)) * tu
+    assert rel_err(out.to_host(), truth) < TIGHT
+    # f32 activations take the same path
+    a32 = T.GpuTensor.from_host(dev, a)
+    out32 = T.GpuTensor.zeros(dev, (m, ffn), "f32")
+    T.gemm_swiglu(dev, w, a32, m, out32, None, splits)
+    assert np.array_equal(out32.to_host(), out.to_host())
+    with pytest.raises(T.DeviceError):
+        T.gemm_swiglu(dev, plain, ad, m, out)        # not a paired weight
+    w.free()
+    plain.free()
+
+
+@pytest.mark.parametrize("m", [8, 24, 40])
+def test_gemm_swiglu_larger_m_goes_through_the_temporary(dev, m):
+    h, ffn = 640, 224
+    gp, gs = O.synth_packed(h, ffn, 960), O.synth_scales(h, ffn, 961)
+    up, us = O.synth_packed(h, ffn, 962), O.synth_scales(h, ffn, 963)
+    gd = (T.GpuTensor.from_host(dev, gp), T.GpuTensor.from_host(dev, gs, "f16"))
+    ud = (T.GpuTensor.from_host(dev, up), T.GpuTensor.from_host(dev, us, "f16"))
+    a16 = O.synth_act_f16(m, h, 964)
+    ad = T.GpuTensor.from_host(dev, a16, "f16")
+    w = T.MarlinWeight.gate_up(dev, gd, ud, h, ffn)
+    out = T.GpuTensor.zeros(dev, (m, ffn), "f32")
+    with pytest.raises(T.DeviceError):
+        T.gemm_swiglu(dev, w, ad, m, out)            # no temporary
+    tmp = T.GpuTensor.zeros(dev, (m, 2 * ffn), "f32")
+    T.gemm_swiglu(dev, w, ad, m, out, tmp)
+    fp, fs = O.fuse_tw_marlin_n([(gp, gs), (up, us)], h, [ffn, ffn])
+    t = gemm_truth(a16, fp, fs, m, h, 2 * ffn)
+    tg, tu = t[:, :ffn], t[:, ffn:]
+    truth = tg / (1.0 + np.exp(-tg)) * tu
+    assert rel_err(out.to_host(), truth) < (TIGHT if m <= 32 else 1e-3)
+    # the plain GEMM on a paired handle returns the columns in the paired order
+    T.gemm(dev, w, ad, m, tmp)
+    j = np.arange(ffn)
+    col = (j // 32) * 64 + j % 32
+    got = tmp.to_host().reshape(m, 2 * ffn)
+    assert rel_err(got[:, col], tg) < (TIGHT if m <= 32 else 1e-3)
+    assert rel_err(got[:, col + 32], tu) < (TIGHT if m <= 32 else 1e-3)
+    w.free()
+
+
 def test_argmax_bit_exact(dev):
     # index output: bit exact against the oracle's sequential scan, including ties (first wins), values at or
     # below the -1e30 starting value, NaN, infinities, a vocabulary-sized row and an empty one

@@ -332,3 +332,42 @@ def test_argmax_follows_the_reference_scan():
     assert O.argmax(np.zeros((2, 0), np.float32), 2, 0).tolist() == [0, 0]  # empty rows
     inf = np.array([[1.0, np.inf, np.inf, -np.inf]], np.float32)
     assert O.argmax(inf, 1, 4)[0] == 1
+
+
+def test_silu_mul_against_f64_and_its_invariants():
+    # warp_fused_silu_mul (ops.rs:966-976): g / (1 + expf(-g)) * up.  Checked against the same expression in
+    # f64 (a few f32 ulps), the identity silu(g) - silu(-g) = g, and the limits at 0 and at both tails.
+    g = (O.synth_normal_f32(5000, 910) * np.float32(4.0)).astype(np.float32)
+    u = O.synth_normal_f32(5000, 911)
+    out = O.silu_mul(g, u)
+    g64, u64 = g.astype(np.float64), u.astype(np.float64)
+    truth = g64 / (1.0 + np.exp(-g64)) * u64
+    assert np.max(np.abs(out - truth) / np.maximum(np.abs(truth), 1e-30)) < 1e-6
+    ones = np.ones_like(g)
+    assert np.allclose(O.silu_mul(g, ones).astype(np.float64) - O.silu_mul(-g, ones), g64, rtol=0, atol=2e-6)
+    edge = np.array([0.0, -0.0, 100.0, -100.0, 1e4, -1e4, 1.0], np.float32)
+    r = O.silu_mul(edge, np.full(7, 2.0, np.float32))
+    assert r[0] == 0.0 and r[1] == 0.0
+    assert r[2] == 200.0 and r[4] == 2e4                 # exp(-g) vanishes: silu(g) = g
+    assert abs(r[3]) < 1e-40 and r[5] == 0.0             # exp(-g) overflows to inf: g / inf = -0
+    assert abs(r[6] - 2.0 / (1.0 + np.exp(-1.0))) < 1e-6
+    assert O.silu_mul(np.zeros(0, np.float32), np.zeros(0, np.float32)).size == 0
+
+
+def test_pair_gate_up_is_the_32_column_interleave():
+    # independent restatement with reshapes: [G][ffn/32][32] blocks of gate and up stacked side by side
+    k, ffn = 96, 160
+    gp, gs = O.synth_packed(k, ffn, 920), O.synth_scales(k, ffn, 921)
+    up, us = O.synth_packed(k, ffn, 922), O.synth_scales(k, ffn, 923)
+    pp, ps = O.pair_gate_up(gp, gs, up, us, k, ffn)
+    G = k // 32
+    want_p = np.stack([gp.reshape(G, ffn // 32, 32, 16), up.reshape(G, ffn // 32, 32, 16)], axis=2).reshape(-1)
+    want_s = np.stack([gs.reshape(G, ffn // 32, 32), us.reshape(G, ffn // 32, 32)], axis=2).reshape(-1)
+    assert np.array_equal(pp, want_p) and np.array_equal(ps, want_s)
+    # the weights are those of fuse_tw_marlin_n([gate, up]) with the columns permuted
+    fp, fs = O.fuse_tw_marlin_n([(gp, gs), (up, us)], k, [ffn, ffn])
+    wf = O.dequant_f32(fp, fs, k, 2 * ffn)
+    wp = O.dequant_f32(pp, ps, k, 2 * ffn)
+    j = np.arange(ffn)
+    col = (j // 32) * 64 + j % 32
+    assert np.array_equal(wp[:, col], wf[:, :ffn]) and np.array_equal(wp[:, col + 32], wf[:, ffn:])
