@@ -219,6 +219,14 @@ int twm_gemm(twm_ctx *ctx, const twm_weight *w, const void *a_dev, int a_dtype, 
  * sum(ns) must equal the weight's N; out i is row-major [M, ns[i]] f32. */
 int twm_gemm_split(twm_ctx *ctx, const twm_weight *w, const void *a_dev, int a_dtype, uint32_t m,
                    float *const *outs_dev, const uint32_t *ns, uint32_t count, uint32_t splits);
+/* twm_gemm_split with an f32 bias per output: out i = A x W_i + biases_dev[i][0..ns[i]) on every row
+ * (one f32 add per element, GEMV result first).  biases_dev is a host array of `count` device
+ * pointers, entries may be NULL; biases_dev itself may be NULL.  For the Q/K/V biases bq/bk/bv
+ * (quantize.rs:1078-1080), which the reference adds in its fused bias + RoPE kernel
+ * (generate.rs:2162-2178): with the sum already in q/k/v that kernel runs with has_bias = false. */
+int twm_gemm_split_bias(twm_ctx *ctx, const twm_weight *w, const void *a_dev, int a_dtype, uint32_t m,
+                        float *const *outs_dev, const float *const *biases_dev, const uint32_t *ns,
+                        uint32_t count, uint32_t splits);
 /* Gate/up weight for twm_gemm_swiglu: twm_pair_gate_up followed by twm_weight_from_device, with the
  * handle marked as paired.  twm_gemm / twm_gemm_split on such a handle return the 2*ffn_dim columns
  * in the paired order. */

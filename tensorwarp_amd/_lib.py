@@ -62,6 +62,7 @@ SIGNATURES = {
     "twm_weight_gate_up": (_vp, [_vp, _vp, _vp, _vp, _vp, _u32, _u32]),
     "twm_weight_is_paired": (_int, [_vp]),
     "twm_gemm_swiglu": (_int, [_vp, _vp, _vp, _int, _u32, _vp, _vp, _u32]),
+    "twm_gemm_split_bias": (_int, [_vp, _vp, _vp, _int, _u32, C.POINTER(_vp), C.POINTER(_vp), C.POINTER(_u32), _u32, _u32]),
     "twm_pick_splits": (_u32, [_u32, _u32, _u32]),
     "twm_graph_begin": (_int, [_vp]),
     "twm_graph_end": (_vp, [_vp]),

@@ -766,8 +766,16 @@ static int gemm_common(twm_ctx *ctx, const twm_weight *w, const void *a_dev, int
     if (a_dtype != TWM_F16 && a_dtype != TWM_F32) return fail(TWM_UNSUPPORTED_OP, "%s: activations must be f16 or f32", who);
     if (m == 0 || w->n == 0) return TWM_OK;
     if (w->k == 0) {
-        for (uint32_t s = 0; s < out.count; s++)
-            if (int rc = twm_memset_zero(ctx, out.seg[s].ptr, (size_t)m * out.seg[s].width * 4)) return rc;
+        for (uint32_t s = 0; s < out.count; s++) {
+            if (!out.seg[s].bias) {
+                if (int rc = twm_memset_zero(ctx, out.seg[s].ptr, (size_t)m * out.seg[s].width * 4)) return rc;
+                continue;
+            }
+            for (uint32_t r = 0; r < m; r++)  // an empty sum plus the bias
+                if (int rc = twm_memcpy_d2d(ctx, out.seg[s].ptr + (size_t)r * out.seg[s].width, out.seg[s].bias,
+                                            (size_t)out.seg[s].width * 4))
+                    return rc;
+        }
         return TWM_OK;
     }
     if (!a_dev) return fail(TWM_INVALID_HANDLE, "%s: null activations", who);
@@ -832,31 +840,39 @@ int twm_gemm(twm_ctx *ctx, const twm_weight *w, const void *a_dev, int a_dtype, 
     return gemm_common(ctx, w, a_dev, a_dtype, m, out, splits, "twm_gemm");
 }
 
-int twm_gemm_split(twm_ctx *ctx, const twm_weight *w, const void *a_dev, int a_dtype, uint32_t m, float *const *outs_dev,
-                   const uint32_t *ns, uint32_t count, uint32_t splits)
+int twm_gemm_split_bias(twm_ctx *ctx, const twm_weight *w, const void *a_dev, int a_dtype, uint32_t m,
+                        float *const *outs_dev, const float *const *biases_dev, const uint32_t *ns, uint32_t count,
+                        uint32_t splits)
 {
-    if (!ctx || !w) return fail(TWM_INVALID_HANDLE, "twm_gemm_split: null handle");
-    if (w->ctx != ctx) return fail(TWM_INVALID_HANDLE, "twm_gemm_split: weight belongs to another context");
-    if (!outs_dev || !ns) return fail(TWM_INVALID_HANDLE, "twm_gemm_split: null array");
+    if (!ctx || !w) return fail(TWM_INVALID_HANDLE, "twm_gemm_split_bias: null handle");
+    if (w->ctx != ctx) return fail(TWM_INVALID_HANDLE, "twm_gemm_split_bias: weight belongs to another context");
+    if (!outs_dev || !ns) return fail(TWM_INVALID_HANDLE, "twm_gemm_split_bias: null array");
     if (count == 0 || count > (uint32_t)kMaxSegs)
-        return fail(TWM_SHAPE_ERROR, "twm_gemm_split: between 1 and %d outputs are supported", kMaxSegs);
+        return fail(TWM_SHAPE_ERROR, "twm_gemm_split_bias: between 1 and %d outputs are supported", kMaxSegs);
     OutSpec out;
     memset(&out, 0, sizeof out);
     uint64_t total = 0;
     uint32_t used = 0;
     for (uint32_t i = 0; i < count; i++) {
         if (ns[i] == 0) continue;
-        if (m != 0 && !outs_dev[i]) return fail(TWM_INVALID_HANDLE, "twm_gemm_split: null output %u", i);
+        if (m != 0 && !outs_dev[i]) return fail(TWM_INVALID_HANDLE, "twm_gemm_split_bias: null output %u", i);
         out.seg[used].ptr = outs_dev[i];
         out.seg[used].start = (uint32_t)total;
         out.seg[used].width = ns[i];
+        out.seg[used].bias = biases_dev ? biases_dev[i] : nullptr;
         used++;
         total += ns[i];
     }
     out.count = used;
-    if (total != w->n) return fail(TWM_SHAPE_ERROR, "twm_gemm_split: outputs cover %llu columns, weight has %u",
+    if (total != w->n) return fail(TWM_SHAPE_ERROR, "twm_gemm_split_bias: outputs cover %llu columns, weight has %u",
                                    (unsigned long long)total, w->n);
-    return gemm_common(ctx, w, a_dev, a_dtype, m, out, splits, "twm_gemm_split");
+    return gemm_common(ctx, w, a_dev, a_dtype, m, out, splits, "twm_gemm_split_bias");
+}
+
+int twm_gemm_split(twm_ctx *ctx, const twm_weight *w, const void *a_dev, int a_dtype, uint32_t m, float *const *outs_dev,
+                   const uint32_t *ns, uint32_t count, uint32_t splits)
+{
+    return twm_gemm_split_bias(ctx, w, a_dev, a_dtype, m, outs_dev, nullptr, ns, count, splits);
 }
 
 int twm_gemm_swiglu(twm_ctx *ctx, const twm_weight *w, const void *a_dev, int a_dtype, uint32_t m, float *out_dev,

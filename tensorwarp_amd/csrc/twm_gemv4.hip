@@ -59,7 +59,7 @@ __device__ __forceinline__ void gemv4_store_out(const OutSpec &out, uint32_t m, 
     for (uint32_t s = 0; s < kMaxSegs; s++) {
         if (s < out.count) {
             uint32_t rel = col - out.seg[s].start;
-            if (rel < out.seg[s].width) out.seg[s].ptr[(size_t)m * out.seg[s].width + rel] = v;
+            if (rel < out.seg[s].width) out.seg[s].ptr[(size_t)m * out.seg[s].width + rel] = out.seg[s].bias ? v + out.seg[s].bias[rel] : v;
         }
     }
 }

@@ -33,6 +33,7 @@ struct OutSeg {
     float *ptr;
     uint32_t start;  // first fused column of this segment
     uint32_t width;  // number of columns = row stride of ptr
+    const float *bias;  // optional [width] f32 added to every row in the store (nullptr: none)
 };
 struct OutSpec {
     OutSeg seg[kMaxSegs];

@@ -209,7 +209,7 @@ __global__ __launch_bounds__(WAVES * 64) void k_stream(const uint4v *__restrict_
             for (uint32_t sg = 0; sg < kMaxSegs; sg++) {
                 if (sg < out.count) {
                     uint32_t rel = on - out.seg[sg].start;
-                    if (rel < out.seg[sg].width) out.seg[sg].ptr[(size_t)row * out.seg[sg].width + rel] = s;
+                    if (rel < out.seg[sg].width) out.seg[sg].ptr[(size_t)row * out.seg[sg].width + rel] = out.seg[sg].bias ? s + out.seg[sg].bias[rel] : s;
                 }
             }
         }

@@ -321,13 +321,18 @@ def gemm_swiglu(device, weight, a, m, out, tmp=None, splits=0):
                                      tmp.ptr if tmp is not None else None, splits))
 
 
-def gemm_split(device, weight, a, m, outs, ns, splits=0):
-    """Fused projection whose column ranges land in separate buffers (gemm + split_qkv/split_gate_up)."""
+def gemm_split(device, weight, a, m, outs, ns, splits=0, biases=None):
+    """Fused projection whose column ranges land in separate buffers (gemm + split_qkv/split_gate_up);
+    biases: optional list of f32 [ns[i]] tensors (or None entries) added in the store (bq/bk/bv)."""
     cnt = len(outs)
     dt = _lib.F16 if a.dtype == "f16" else _lib.F32
     op = (C.c_void_p * cnt)(*[o.ptr for o in outs])
     nsa = (C.c_uint32 * cnt)(*[int(x) for x in ns])
-    _check(device._l.twm_gemm_split(device.handle, weight.handle, a.ptr, dt, m, op, nsa, cnt, splits))
+    if biases is None:
+        _check(device._l.twm_gemm_split(device.handle, weight.handle, a.ptr, dt, m, op, nsa, cnt, splits))
+        return
+    bp = (C.c_void_p * cnt)(*[(b.ptr if b is not None else None) for b in biases])
+    _check(device._l.twm_gemm_split_bias(device.handle, weight.handle, a.ptr, dt, m, op, bp, nsa, cnt, splits))
 
 
 class TWMarlinWeights:

@@ -654,6 +654,39 @@ def test_fused_qkv_and_gate_up_equal_separate_projections(dev):
         T.gemm_split(dev, rp["gate_up"], a3d, 3, [g, u], [ffn, ffn - 1])
 
 
+@pytest.mark.parametrize("m,splits", [(1, 0), (1, 4), (3, 0), (12, 0), (12, 2), (40, 0), (70, 2)])
+def test_gemm_split_bias_adds_bq_bk_bv_in_the_store(dev, m, splits):
+    # q = gemv + bq etc. (the add the reference makes in its bias + RoPE kernel): one f32 add per element on
+    # top of the unbiased result, so the comparison with numpy's f32 add is bit for bit, on every kernel
+    h, kv = 640, 128
+    ns = [h, kv, kv]
+    packed, scales, a16 = synth(h, sum(ns), m, 970 + m)
+    w = T.MarlinWeight.upload(dev, packed, scales, h, sum(ns))
+    ad = T.GpuTensor.from_host(dev, a16, "f16")
+    plain = [T.GpuTensor.zeros(dev, (m, n), "f32") for n in ns]
+    T.gemm_split(dev, w, ad, m, plain, ns, splits)
+    bias_h = [O.synth_normal_f32(n, 980 + i) for i, n in enumerate(ns)]
+    bias_h[1] = None                                             # K without a bias
+    bias_d = [T.GpuTensor.from_host(dev, b) if b is not None else None for b in bias_h]
+    outs = [T.GpuTensor.from_host(dev, np.full((m, n), np.nan, np.float32)) for n in ns]
+    T.gemm_split(dev, w, ad, m, outs, ns, splits, biases=bias_d)
+    for o, p, b in zip(outs, plain, bias_h):
+        want = p.to_host() if b is None else (p.to_host() + b[None, :]).astype(np.float32)
+        assert np.array_equal(o.to_host(), want)
+    w.free()
+
+
+def test_gemm_split_bias_with_empty_k(dev):
+    ns = [64, 32]
+    w = T.MarlinWeight.upload(dev, np.zeros(0, np.uint8), np.zeros(0, np.uint16), 0, 96)
+    a = T.GpuTensor.zeros(dev, (1,), "f16")
+    b0 = O.synth_normal_f32(64, 990)
+    outs = [T.GpuTensor.from_host(dev, np.full((2, n), np.nan, np.float32)) for n in ns]
+    T.gemm_split(dev, w, a, 2, outs, ns, 0, biases=[T.GpuTensor.from_host(dev, b0), None])
+    assert np.array_equal(outs[0].to_host(), np.stack([b0, b0])) and not outs[1].to_host().any()
+    w.free()
+
+
 @pytest.mark.parametrize("m", [12, 24, 40, 130])
 def test_gemm_split_batched_and_prefill_rows(dev, m):
     # segment stores of the streaming kernel (M = 12, 24), of the MFMA GEMM (M = 40, 130) and of the
