@@ -199,6 +199,15 @@ void twm_weight_destroy(twm_weight *w);
 int twm_weight_dims(const twm_weight *w, uint32_t *k, uint32_t *n);
 /* device bytes held by the repacked weight */
 size_t twm_weight_bytes(const twm_weight *w);
+/* The repacked weight as a self-describing byte blob, for an on-disk cache of the internal order
+ * beside the reference's pre-quantized `.warp` cache (crates/loader/src/warp_cache.rs:1-21: store
+ * it there as one U8 tensor per projection).  Import skips quantize / reorder / fuse / repack: it
+ * is one host-to-device copy.  The blob carries a layout number; a library whose repacked order
+ * differs refuses it (TWM_UNSUPPORTED_OP) and the caller repacks from the TW-Marlin arrays.
+ * A checksum catches truncated or corrupt blobs (TWM_SHAPE_ERROR).  Both calls synchronise. */
+size_t twm_weight_blob_bytes(const twm_weight *w);
+int twm_weight_export(twm_ctx *ctx, const twm_weight *w, void *blob_host, size_t blob_bytes);
+twm_weight *twm_weight_import(twm_ctx *ctx, const void *blob_host, size_t blob_bytes);
 /* "Q4 unpack" straight from the repacked form: out[k][n] f16 row-major [K,N]; must be
  * bit-identical to twm_dequant_to_f16 of the arrays the weight was made from. */
 int twm_weight_dequant_f16(twm_ctx *ctx, const twm_weight *w, uint16_t *out_kn_dev);

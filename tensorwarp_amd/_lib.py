@@ -56,6 +56,9 @@ SIGNATURES = {
     "twm_weight_destroy": (None, [_vp]),
     "twm_weight_dims": (_int, [_vp, C.POINTER(_u32), C.POINTER(_u32)]),
     "twm_weight_bytes": (_sz, [_vp]),
+    "twm_weight_blob_bytes": (_sz, [_vp]),
+    "twm_weight_export": (_int, [_vp, _vp, _vp, _sz]),
+    "twm_weight_import": (_vp, [_vp, _vp, _sz]),
     "twm_weight_dequant_f16": (_int, [_vp, _vp, _vp]),
     "twm_gemm": (_int, [_vp, _vp, _vp, _int, _u32, _vp, _u32]),
     "twm_gemm_split": (_int, [_vp, _vp, _vp, _int, _u32, C.POINTER(_vp), C.POINTER(_u32), _u32, _u32]),

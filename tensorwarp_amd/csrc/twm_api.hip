@@ -646,6 +646,106 @@ int twm_weight_dims(const twm_weight *w, uint32_t *k, uint32_t *n)
 
 size_t twm_weight_bytes(const twm_weight *w) { return w ? w->bytes : 0; }
 
+/* ---- repacked weights as a byte blob (for an on-disk cache) -------------------------------- */
+
+// 64-byte little-endian header followed by the device allocation as it is.
+struct WeightBlobHeader {
+    char magic[8];          // "TWMWGT01"
+    uint32_t layout;        // changes whenever the repacked byte order does
+    uint32_t k, n, n_tiles, k_chunks;
+    uint32_t paired;
+    uint64_t payload_bytes;
+    uint64_t checksum;      // of the payload
+    uint8_t reserved[16];
+};
+static_assert(sizeof(WeightBlobHeader) == 64, "blob header is 64 bytes");
+static const char kBlobMagic[8] = {'T', 'W', 'M', 'W', 'G', 'T', '0', '1'};
+static const uint32_t kBlobLayout = 3;
+
+// Four independent multiply-rotate lanes over 64-bit words (memory-bound on the host), folded at the end.
+static uint64_t blob_checksum(const uint8_t *p, size_t bytes)
+{
+    uint64_t h[4] = {0x9E3779B97F4A7C15ull, 0xC2B2AE3D27D4EB4Full, 0x165667B19E3779F9ull, 0x27D4EB2F165667C5ull};
+    size_t words = bytes / 8, i = 0;
+    for (; i + 4 <= words; i += 4) {
+        for (int l = 0; l < 4; l++) {
+            uint64_t v;
+            memcpy(&v, p + (i + l) * 8, 8);
+            h[l] = (h[l] ^ v) * 0x100000001B3ull;
+            h[l] = (h[l] << 29) | (h[l] >> 35);
+        }
+    }
+    uint64_t tail = 0;
+    for (size_t b = i * 8; b < bytes; b++) tail = tail * 257 + p[b];
+    uint64_t r = tail ^ (uint64_t)bytes;
+    for (int l = 0; l < 4; l++) r = (r ^ h[l]) * 0xFF51AFD7ED558CCDull + (r >> 31);
+    return r;
+}
+
+size_t twm_weight_blob_bytes(const twm_weight *w) { return w ? sizeof(WeightBlobHeader) + w->bytes : 0; }
+
+int twm_weight_export(twm_ctx *ctx, const twm_weight *w, void *blob_host, size_t blob_bytes)
+{
+    if (!ctx || !w) return fail(TWM_INVALID_HANDLE, "twm_weight_export: null handle");
+    if (w->ctx != ctx) return fail(TWM_INVALID_HANDLE, "twm_weight_export: weight belongs to another context");
+    if (ctx->capturing) return fail(TWM_UNSUPPORTED_OP, "twm_weight_export: not allowed inside a graph capture");
+    if (!blob_host) return fail(TWM_INVALID_HANDLE, "twm_weight_export: null buffer");
+    if (blob_bytes != twm_weight_blob_bytes(w))
+        return fail(TWM_SHAPE_ERROR, "twm_weight_export: the buffer must hold %zu bytes, got %zu", twm_weight_blob_bytes(w), blob_bytes);
+    uint8_t *payload = (uint8_t *)blob_host + sizeof(WeightBlobHeader);
+    size_t payload_bytes = (w->qw != nullptr) ? w->bytes : 0;
+    if (payload_bytes)
+        if (int rc = twm_memcpy_d2h(ctx, payload, w->qw, payload_bytes)) return rc;
+    WeightBlobHeader hd;
+    memset(&hd, 0, sizeof hd);
+    memcpy(hd.magic, kBlobMagic, 8);
+    hd.layout = kBlobLayout;
+    hd.k = w->k;
+    hd.n = w->n;
+    hd.n_tiles = w->n_tiles;
+    hd.k_chunks = w->k_chunks;
+    hd.paired = w->paired ? 1u : 0u;
+    hd.payload_bytes = w->bytes;
+    hd.checksum = blob_checksum(payload, payload_bytes);
+    memcpy(blob_host, &hd, sizeof hd);
+    return TWM_OK;
+}
+
+twm_weight *twm_weight_import(twm_ctx *ctx, const void *blob_host, size_t blob_bytes)
+{
+    if (!ctx) { fail(TWM_INVALID_HANDLE, "twm_weight_import: null context"); return nullptr; }
+    if (ctx->capturing) { fail(TWM_UNSUPPORTED_OP, "twm_weight_import: not allowed inside a graph capture"); return nullptr; }
+    if (!blob_host || blob_bytes < sizeof(WeightBlobHeader)) { fail(TWM_SHAPE_ERROR, "twm_weight_import: blob shorter than its header"); return nullptr; }
+    WeightBlobHeader hd;
+    memcpy(&hd, blob_host, sizeof hd);
+    if (memcmp(hd.magic, kBlobMagic, 8) != 0) { fail(TWM_SHAPE_ERROR, "twm_weight_import: not a repacked-weight blob (bad magic)"); return nullptr; }
+    if (hd.layout != kBlobLayout) {
+        fail(TWM_UNSUPPORTED_OP, "twm_weight_import: blob has layout %u, this library writes %u: repack from the TW-Marlin arrays", hd.layout, kBlobLayout);
+        return nullptr;
+    }
+    if (check_kn("twm_weight_import", hd.k, hd.n)) return nullptr;
+    twm_weight *w = weight_alloc(ctx, hd.k, hd.n);
+    if (!w) return nullptr;
+    const uint8_t *payload = (const uint8_t *)blob_host + sizeof(WeightBlobHeader);
+    bool ok = w->n_tiles == hd.n_tiles && w->k_chunks == hd.k_chunks && w->bytes == hd.payload_bytes &&
+              blob_bytes == sizeof(WeightBlobHeader) + hd.payload_bytes && hd.paired <= 1 &&
+              (!hd.paired || hd.n % (2 * kPairWidth) == 0);
+    if (!ok) fail(TWM_SHAPE_ERROR, "twm_weight_import: header does not describe a %u x %u weight of %zu bytes", hd.k, hd.n, blob_bytes);
+    size_t payload_bytes = w->qw ? w->bytes : 0;
+    if (ok && blob_checksum(payload, payload_bytes) != hd.checksum) {
+        ok = false;
+        fail(TWM_SHAPE_ERROR, "twm_weight_import: checksum mismatch (corrupt or truncated blob)");
+    }
+    if (ok && payload_bytes) ok = twm_memcpy_h2d(ctx, w->qw, payload, payload_bytes) == TWM_OK;
+    if (!ok) {
+        if (w->qw) (void)hipFree(w->qw);
+        delete w;
+        return nullptr;
+    }
+    w->paired = hd.paired != 0;
+    return w;
+}
+
 static WeightView view_of(const twm_weight *w)
 {
     WeightView v;

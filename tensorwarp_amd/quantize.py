@@ -296,6 +296,23 @@ class MarlinWeight:
     def nbytes(self):
         return self.device._l.twm_weight_bytes(self.handle)
 
+    def export_blob(self):
+        """The repacked weight as a uint8 array (header + device bytes) for an on-disk cache."""
+        size = self.device._l.twm_weight_blob_bytes(self.handle)
+        blob = np.empty(size, np.uint8)
+        _check(self.device._l.twm_weight_export(self.device.handle, self.handle, blob.ctypes.data, size))
+        return blob
+
+    @classmethod
+    def import_blob(cls, device, blob):
+        blob = np.ascontiguousarray(blob, np.uint8)
+        h = device._l.twm_weight_import(device.handle, blob.ctypes.data, blob.size)
+        if not h:
+            raise DeviceError(_lib.SHAPE_ERROR, device._l.twm_last_error().decode())
+        k, n = C.c_uint32(), C.c_uint32()
+        device._l.twm_weight_dims(h, C.byref(k), C.byref(n))
+        return cls(device, h, k.value, n.value)
+
     def dequant_f16(self):
         out = GpuTensor(self.device, (self.k, self.n), "f16")
         _check(self.device._l.twm_weight_dequant_f16(self.device.handle, self.handle, out.ptr))

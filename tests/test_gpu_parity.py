@@ -604,6 +604,52 @@ def test_empty_inputs(dev):
     w0.free()
 
 
+def test_repacked_weight_blob_round_trip_through_a_warp_file(dev, tmp_path):
+    from tensorwarp_amd import warp_cache as W
+    k, n, ffn = 640, 200, 96
+    packed, scales, a16 = synth(k, n, 3, 1000)
+    w = T.MarlinWeight.upload(dev, packed, scales, k, n)
+    gp, gs = O.synth_packed(k, ffn, 1001), O.synth_scales(k, ffn, 1002)
+    up, us = O.synth_packed(k, ffn, 1003), O.synth_scales(k, ffn, 1004)
+    wp = T.MarlinWeight.gate_up(dev, (T.GpuTensor.from_host(dev, gp), T.GpuTensor.from_host(dev, gs, "f16")),
+                                (T.GpuTensor.from_host(dev, up), T.GpuTensor.from_host(dev, us, "f16")), k, ffn)
+    blob, blob_p = w.export_blob(), wp.export_blob()
+    assert blob.size == 64 + w.nbytes and bytes(blob[:8]) == b"TWMWGT01"
+    path = tmp_path / "model.warp"
+    W.save_warp_cache(path, '{"layout": "gfx950"}', [("l0.w", W.DTYPE_U8, blob.shape, blob),
+                                                    ("l0.gate_up", W.DTYPE_U8, blob_p.shape, blob_p)])
+    _, tensors = W.load_warp_cache(path)
+    w2 = T.MarlinWeight.import_blob(dev, tensors[0].array())
+    wp2 = T.MarlinWeight.import_blob(dev, tensors[1].array())
+    assert (w2.k, w2.n, w2.paired) == (k, n, False) and (wp2.k, wp2.n, wp2.paired) == (k, 2 * ffn, True)
+    ad = T.GpuTensor.from_host(dev, a16, "f16")
+    for m in (1, 3):
+        c1, c2 = T.GpuTensor.zeros(dev, (m, n), "f32"), T.GpuTensor.zeros(dev, (m, n), "f32")
+        T.gemm(dev, w, ad, m, c1)
+        T.gemm(dev, w2, ad, m, c2)
+        assert np.array_equal(c1.to_host(), c2.to_host())
+        s1, s2 = T.GpuTensor.zeros(dev, (m, ffn), "f32"), T.GpuTensor.zeros(dev, (m, ffn), "f32")
+        T.gemm_swiglu(dev, wp, ad, m, s1)
+        T.gemm_swiglu(dev, wp2, ad, m, s2)
+        assert np.array_equal(s1.to_host(), s2.to_host())
+    assert np.array_equal(w2.dequant_f16().to_host(), O.dequant_f16(packed, scales, k, n).reshape(k, n))
+    assert np.array_equal(w2.export_blob(), blob)
+    # refusals: flipped payload byte, truncated blob, other layout number, foreign bytes
+    bad = blob.copy()
+    bad[64 + 1234] ^= 1
+    short = blob[:-16]
+    other = blob.copy()
+    other[8] ^= 0x40
+    for b in (bad, short, other, np.zeros(64, np.uint8), np.zeros(10, np.uint8)):
+        with pytest.raises(T.DeviceError):
+            T.MarlinWeight.import_blob(dev, b)
+    empty = T.MarlinWeight.upload(dev, np.zeros(0, np.uint8), np.zeros(0, np.uint16), 64, 0)
+    e2 = T.MarlinWeight.import_blob(dev, empty.export_blob())
+    assert (e2.k, e2.n) == (64, 0)
+    for x in (w, w2, wp, wp2, empty, e2):
+        x.free()
+
+
 # ---------------------------------------------------------------- fused projections
 
 def test_fused_qkv_and_gate_up_equal_separate_projections(dev):
