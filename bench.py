@@ -77,6 +77,7 @@ def main():
     ap.add_argument("--no-prefill", action="store_true", help="skip the prefill GEMM timings")
     ap.add_argument("--no-lm-head", action="store_true", help="skip the LM-head GEMV + argmax timing")
     ap.add_argument("--no-swiglu", action="store_true", help="skip the fused gate_up + SwiGLU timing")
+    ap.add_argument("--no-moe", action="store_true", help="skip the expert-bank (MoE decode) timing")
     ap.add_argument("--extra", action="store_true", help="also time batched decode (M=4..32) on the gate_up shape")
     ap.add_argument("--sweep-splits", action="store_true",
                     help="also time every projection at M=1,4,8,16,32 with forced split-K factors next to the library's "
@@ -313,6 +314,55 @@ def main():
         for w in plain + pairedw:
             w.free()
 
+    # Mixture-of-experts decode (the reference's Gemma MoE shape: hidden 2816, expert dim 704, 128 experts, top 8):
+    # gate+up of the eight routed experts, GEGLU, down + weighted sum; ids rotate so the experts come from HBM
+    moe = None
+    if not args.no_moe:
+        k, dim, experts, top_k = 2816, 704, 128, 8
+        g_gu, g_d = k // 32, dim // 32
+        gu_p = T.GpuTensor.from_host(dev, rng.integers(0, 256, size=experts * g_gu * 2 * dim * 16, dtype=np.uint8))
+        gu_s = T.GpuTensor.from_host(dev, (np.abs(rng.standard_normal(experts * g_gu * 2 * dim, dtype=np.float32)) * np.float32(0.02)).astype(np.float16).view(np.uint16), "f16")
+        d_p = T.GpuTensor.from_host(dev, rng.integers(0, 256, size=experts * g_d * k * 16, dtype=np.uint8))
+        d_s = T.GpuTensor.from_host(dev, (np.abs(rng.standard_normal(experts * g_d * k, dtype=np.float32)) * np.float32(0.02)).astype(np.float16).view(np.uint16), "f16")
+        bank_gu = T.ExpertBank.from_device(dev, gu_p, gu_s, g_gu * 2 * dim * 16, g_gu * 2 * dim, k, 2 * dim, experts)
+        bank_gu_paired = T.ExpertBank.from_device(dev, gu_p, gu_s, g_gu * 2 * dim * 16, g_gu * 2 * dim, k, 2 * dim, experts, pair_gate_up=True)
+        bank_d = T.ExpertBank.from_device(dev, d_p, d_s, g_d * k * 16, g_d * k, dim, k, experts)
+        for t in (gu_p, gu_s, d_p, d_s):
+            t.free()
+        id_sets = [T.GpuTensor.from_host(dev, ((np.arange(top_k) * 16 + r) % experts).astype(np.float32)) for r in range(16)]
+        wts = T.GpuTensor.from_host(dev, np.full(top_k, 0.125, np.float32))
+        x = T.GpuTensor.from_host(dev, rng.standard_normal(k, dtype=np.float32))
+        gate_up_all = T.GpuTensor.zeros(dev, (top_k, 2 * dim), "f32")
+        geglu_a, geglu_b = T.GpuTensor.zeros(dev, (top_k, dim), "f32"), T.GpuTensor.zeros(dev, (top_k, dim), "f32")
+        acc_a, acc_b = T.GpuTensor.zeros(dev, (k,), "f32"), T.GpuTensor.zeros(dev, (k,), "f32")
+
+        def three():
+            for ids in id_sets:
+                T.batched_marlin_gate_up(dev, x, bank_gu, ids, gate_up_all, top_k)
+                T.batched_marlin_split_geglu(dev, gate_up_all, geglu_a, dim, top_k)
+                T.batched_marlin_down_axpy(dev, geglu_a, bank_d, ids, wts, acc_a, top_k)
+
+        def two():
+            for ids in id_sets:
+                T.batched_marlin_gate_up(dev, x, bank_gu_paired, ids, geglu_b, top_k, act=T.ACT_GEGLU)
+                T.batched_marlin_down_axpy(dev, geglu_b, bank_d, ids, wts, acc_b, top_k)
+        moe_bytes = top_k * (algo_bytes(k, 2 * dim) + algo_bytes(dim, k))
+        moe = {"hidden": k, "expert_dim": dim, "experts": experts, "top_k": top_k, "bytes": moe_bytes}
+        for label, fn in (("gate_up_geglu_down_us", three), ("fused_geglu_then_down_us", two)):
+            fn()
+            dev.synchronize()
+            gr = T.GraphCapture.record_with_device(dev, fn)
+            for _ in range(3):
+                gr.replay()
+            dev.synchronize()
+            us = time_launches(dev, lambda i: gr.replay(), 30) / len(id_sets) * 1e3
+            moe[label] = round(us, 2)
+            moe[label.replace("_us", "_GBps")] = round(moe_bytes / (us * 1e-6) / 1e9, 1)
+            gr.destroy()
+        assert np.array_equal(acc_a.to_host(), acc_b.to_host()), "fused GEGLU differs from the three-launch sequence"
+        for b_ in (bank_gu, bank_gu_paired, bank_d):
+            b_.free()
+
     prefill = None
     if not args.no_prefill:
         prefill = {}
@@ -412,6 +462,8 @@ def main():
         out["lm_head_m1"] = lm
     if mlp_front is not None:
         out["mlp_front_m1"] = mlp_front
+    if moe is not None:
+        out["moe_decode_m1"] = moe
     if prefill:
         out["prefill"] = prefill
         best = max(prefill.items(), key=lambda kv: kv[1]["TFLOPs"] if kv[0].startswith("M2048") else 0.0)

@@ -251,6 +251,44 @@ int twm_weight_is_paired(const twm_weight *w);
  * projections is twm_gemm's for the same M. */
 int twm_gemm_swiglu(twm_ctx *ctx, const twm_weight *w, const void *a_dev, int a_dtype, uint32_t m,
                     float *out_dev, float *tmp_dev, uint32_t splits);
+/* ---- expert banks: the TW-Marlin GEMVs of mixture-of-experts decode ------------------------- */
+
+typedef struct twm_bank twm_bank;
+
+/* Repacks num_experts matrices of the same (K, N) that lie in one pair of device buffers, expert e at
+ * packed_base + e * packed_bytes_per_expert (bytes) and scales_base + e * scales_per_expert (f16
+ * elements): the layout and the two strides of batched_marlin_gate_up
+ * (crates/kernels/src/moe_batched_marlin.rs:20-36, 153-166).  pair_gate_up != 0: every matrix is a fused
+ * [gate | up] (N = 2 * dim, a multiple of 64) and is stored in the paired column order, which lets
+ * twm_bank_gemv apply the gate in its store.  The inputs are not retained. */
+twm_bank *twm_bank_from_device(twm_ctx *ctx, const uint8_t *packed_base_dev, const uint16_t *scales_base_dev,
+                               size_t packed_bytes_per_expert, size_t scales_per_expert, uint32_t k,
+                               uint32_t n, uint32_t num_experts, int pair_gate_up);
+void twm_bank_destroy(twm_bank *b);
+size_t twm_bank_bytes(const twm_bank *b);
+/* All top_k expert GEMVs in one launch, the expert of slot s being (int)topk_ids_dev[s], read on the
+ * device (batched_marlin_gate_up, moe_batched_marlin.rs:20-74, 153-182): out[s][n] = A_s x W[id_s].
+ * a_slot_stride (elements) = 0 shares one activation row [1, K] among the slots, K gives every slot
+ * its own row of a [top_k, K] matrix.  With top_k = 1 and topk_ids_dev pointing at the wanted entry it
+ * is the device-indexed GEMV gemm_tw_marlin_m1_indirect (quantize_indirect.rs:185-253).
+ * act = 0: out is [top_k, N].  act = 1 / 2 (paired bank only): the store applies
+ * gelu_tanh(gate) * up (batched_marlin_split_geglu, :137-151) or silu(gate) * up, out is [top_k, N/2]
+ * and no [top_k, N] intermediate exists.  An id outside [0, num_experts) yields zeros. */
+int twm_bank_gemv(twm_ctx *ctx, const twm_bank *b, const void *a_dev, int a_dtype, uint32_t a_slot_stride,
+                  const float *topk_ids_dev, uint32_t top_k, int act, float *out_dev);
+/* batched_marlin_down_axpy (moe_batched_marlin.rs:78-134, 184-213): acc[n] += sum over the slots of
+ * topk_weights[s] * (A[s] x W[id_s]) with A [top_k, K].  The reference adds with float atomics in no
+ * fixed order; here the terms are added to acc in slot order, one launch, deterministic.
+ * top_k <= 16. */
+int twm_bank_down_axpy(twm_ctx *ctx, const twm_bank *b, const void *a_all_dev, int a_dtype,
+                       const float *topk_ids_dev, const float *topk_weights_dev, uint32_t top_k,
+                       float *acc_dev);
+/* batched_marlin_split_geglu (moe_batched_marlin.rs:137-151, 215-232):
+ * out[b][j] = gelu_tanh(gate_up[b][gate column j]) * gate_up[b][up column j], gate_up [batch, 2*dim];
+ * paired as in twm_swiglu_rows. */
+int twm_geglu_rows(twm_ctx *ctx, const float *gate_up_dev, uint32_t batch, uint32_t dim, int paired,
+                   float *out_dev);
+
 /* The library's split-K choice for MI355X (256 CUs); same role as quantize.rs:1317-1325. */
 uint32_t twm_pick_splits(uint32_t k, uint32_t n, uint32_t m);
 

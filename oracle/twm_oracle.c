@@ -275,6 +275,17 @@ void twmo_silu_mul(const float *gate, const float *up, float *out, size_t count)
     }
 }
 
+/* The GEGLU gate of batched_marlin_split_geglu (crates/kernels/src/moe_batched_marlin.rs:137-151; the same
+ * expression as warp_fused_gelu_mul, ops.rs:1161-1170): 0.5 g (1 + tanhf(0.7978845608 (g + 0.044715 g^3))) * up */
+void twmo_gelu_mul(const float *gate, const float *up, float *out, size_t count)
+{
+    for (size_t i = 0; i < count; i++) {
+        float g = gate[i];
+        float gelu_g = 0.5f * g * (1.0f + tanhf(0.7978845608f * (g + 0.044715f * g * g * g)));
+        out[i] = gelu_g * up[i];
+    }
+}
+
 /* The paired column order of a gate_up weight (no counterpart in the reference, which keeps
  * [gate | up]): output column 64*(j/32) + j%32 is gate column j, the up column j sits 32 further.
  * Stated here as a plain gather so the device kernel has an independent twin. */

@@ -142,6 +142,26 @@ def silu_mul(gate, up):
     return out.reshape(gate.shape)
 
 
+def gelu_mul(gate, up):
+    gate, up = _c(gate, np.float32), _c(up, np.float32)
+    out = np.zeros(gate.size, np.float32)
+    lib().twmo_gelu_mul(_p(gate), _p(up), _p(out), C.c_size_t(gate.size))
+    return out.reshape(gate.shape)
+
+
+def bank_gemv_f64(a, packed_bank, scales_bank, ids, k, n):
+    """batched_marlin_gate_up (moe_batched_marlin.rs:20-74) as f64 truth: row s = A_s x dequant(expert ids[s]).
+    a: [1, K] shared or [slots, K]; packed_bank [E][G*N*16], scales_bank [E][G*N]; invalid ids give zeros."""
+    a = np.asarray(a, np.float32).reshape(-1, k)
+    out = np.zeros((len(ids), n), np.float64)
+    for s, e in enumerate(ids):
+        e = int(e)
+        if 0 <= e < len(packed_bank):
+            row = a[s if a.shape[0] > 1 else 0].reshape(1, k)
+            out[s] = gemm_f64(row, packed_bank[e], scales_bank[e], 1, k, n)[0]
+    return out
+
+
 def pair_gate_up(gate_packed, gate_scales, up_packed, up_scales, k, ffn):
     po = np.zeros((k // 32) * 2 * ffn * 16, np.uint8)
     so = np.zeros((k // 32) * 2 * ffn, np.uint16)

@@ -4,6 +4,7 @@ this package is the thin Python mirror of the reference's Rust interface used by
 and the benchmark."""
 from . import _lib  # noqa: F401
 from .quantize import *  # noqa: F401,F403
-from .quantize import DeviceError, GpuTensor, GraphCapture, MarlinWeight, TWMarlinWeights, WarpDevice  # noqa: F401
+from .quantize import (DeviceError, ExpertBank, GpuTensor, GraphCapture, MarlinWeight, TWMarlinWeights,  # noqa: F401
+                       WarpDevice)
 
 __version__ = "0.1.0"

@@ -66,6 +66,12 @@ SIGNATURES = {
     "twm_weight_is_paired": (_int, [_vp]),
     "twm_gemm_swiglu": (_int, [_vp, _vp, _vp, _int, _u32, _vp, _vp, _u32]),
     "twm_gemm_split_bias": (_int, [_vp, _vp, _vp, _int, _u32, C.POINTER(_vp), C.POINTER(_vp), C.POINTER(_u32), _u32, _u32]),
+    "twm_bank_from_device": (_vp, [_vp, _vp, _vp, _sz, _sz, _u32, _u32, _u32, _int]),
+    "twm_bank_destroy": (None, [_vp]),
+    "twm_bank_bytes": (_sz, [_vp]),
+    "twm_bank_gemv": (_int, [_vp, _vp, _vp, _int, _u32, _vp, _u32, _int, _vp]),
+    "twm_bank_down_axpy": (_int, [_vp, _vp, _vp, _int, _vp, _vp, _u32, _vp]),
+    "twm_geglu_rows": (_int, [_vp, _vp, _u32, _u32, _int, _vp]),
     "twm_pick_splits": (_u32, [_u32, _u32, _u32]),
     "twm_graph_begin": (_int, [_vp]),
     "twm_graph_end": (_vp, [_vp]),

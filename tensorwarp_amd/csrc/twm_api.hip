@@ -61,6 +61,14 @@ struct twm_weight {
     bool paired;  // gate_up weight whose columns are in the paired order (32 gate, 32 up, ...)
 };
 
+struct twm_bank {
+    twm_ctx *ctx;
+    void *cq;           // experts x column-lane copy
+    size_t expert_bytes, bytes;
+    uint32_t experts, k, n, n_pad, k_chunks;
+    bool paired;
+};
+
 struct twm_graph {
     hipGraph_t graph;
     hipGraphExec_t exec;
@@ -996,6 +1004,143 @@ int twm_gemm_swiglu(twm_ctx *ctx, const twm_weight *w, const void *a_dev, int a_
     out.seg[0].width = w->n;
     if (int rc = gemm_common(ctx, w, a_dev, a_dtype, m, out, splits, "twm_gemm_swiglu")) return rc;
     HIP_TRY(launch_swiglu_rows(ctx->stream, tmp_dev, out_dev, ffn, m, true), TWM_DEVICE_ERROR, "swiglu_rows launch");
+    return TWM_OK;
+}
+
+/* ---- expert banks (mixture-of-experts decode) ------------------------------------------------ */
+
+twm_bank *twm_bank_from_device(twm_ctx *ctx, const uint8_t *packed_base_dev, const uint16_t *scales_base_dev,
+                               size_t packed_bytes_per_expert, size_t scales_per_expert, uint32_t k, uint32_t n,
+                               uint32_t num_experts, int pair_gate_up)
+{
+    if (!ctx) { fail(TWM_INVALID_HANDLE, "twm_bank_from_device: null context"); return nullptr; }
+    if (ctx->capturing) { fail(TWM_UNSUPPORTED_OP, "twm_bank_from_device: not allowed inside a graph capture"); return nullptr; }
+    if (check_kn("twm_bank_from_device", k, n)) return nullptr;
+    if (pair_gate_up && n % (2 * kPairWidth) != 0) {
+        fail(TWM_SHAPE_ERROR, "twm_bank_from_device: a paired gate/up bank needs N %% %u == 0, got %u", 2 * kPairWidth, n);
+        return nullptr;
+    }
+    size_t groups = k / 32;
+    if (packed_bytes_per_expert < groups * n * 16 || scales_per_expert < groups * n || packed_bytes_per_expert % 4 != 0) {
+        fail(TWM_SHAPE_ERROR, "twm_bank_from_device: per-expert strides (%zu bytes, %zu scales) do not hold a %u x %u matrix",
+             packed_bytes_per_expert, scales_per_expert, k, n);
+        return nullptr;
+    }
+    bool empty = (uint64_t)k * n * num_experts == 0;
+    if (!empty && (!packed_base_dev || !scales_base_dev)) { fail(TWM_INVALID_HANDLE, "twm_bank_from_device: null pointer"); return nullptr; }
+    if (((uintptr_t)packed_base_dev & 3) != 0) { fail(TWM_SHAPE_ERROR, "twm_bank_from_device: packed must be 4-byte aligned"); return nullptr; }
+    twm_bank *b = new (std::nothrow) twm_bank();
+    if (!b) { fail(TWM_MEMORY_ERROR, "twm_bank: out of host memory"); return nullptr; }
+    b->ctx = ctx;
+    b->k = k;
+    b->n = n;
+    b->experts = num_experts;
+    b->paired = pair_gate_up != 0;
+    b->n_pad = ((n + 63) / 64) * 64;
+    b->k_chunks = (uint32_t)((groups + kChunkGroups - 1) / kChunkGroups);
+    b->expert_bytes = (size_t)(b->n_pad / 64) * b->k_chunks * kColBlockBytes;
+    b->bytes = b->expert_bytes * num_experts;
+    b->cq = nullptr;
+    if (empty || b->bytes == 0) return b;
+    hipError_t e = hipMalloc(&b->cq, b->bytes);
+    if (e != hipSuccess) {
+        fail(TWM_MEMORY_ERROR, "twm_bank: hipMalloc(%zu): %s", b->bytes, hipGetErrorString(e));
+        delete b;
+        return nullptr;
+    }
+    for (uint32_t x = 0; x < num_experts && e == hipSuccess; x++)
+        e = launch_repack_col(ctx->stream, packed_base_dev + (size_t)x * packed_bytes_per_expert,
+                              scales_base_dev + (size_t)x * scales_per_expert, k, n, (char *)b->cq + (size_t)x * b->expert_bytes,
+                              b->n_pad, b->k_chunks, pair_gate_up ? n / 2 : 0);
+    if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
+    if (e != hipSuccess) {
+        fail(TWM_DEVICE_ERROR, "twm_bank_from_device: repack: %s", hipGetErrorString(e));
+        (void)hipFree(b->cq);
+        delete b;
+        return nullptr;
+    }
+    return b;
+}
+
+void twm_bank_destroy(twm_bank *b)
+{
+    if (!b) return;
+    if (b->cq) {
+        (void)hipStreamSynchronize(b->ctx->stream);
+        (void)hipFree(b->cq);
+    }
+    delete b;
+}
+
+size_t twm_bank_bytes(const twm_bank *b) { return b ? b->bytes : 0; }
+
+static BankView bank_view(const twm_bank *b)
+{
+    BankView v;
+    v.cq = b->cq;
+    v.expert_bytes = b->expert_bytes;
+    v.experts = b->experts;
+    v.k = b->k;
+    v.n = b->n;
+    v.n_pad = b->n_pad;
+    v.k_chunks = b->k_chunks;
+    return v;
+}
+
+static int bank_common_checks(const char *who, twm_ctx *ctx, const twm_bank *b, const void *a_dev, int a_dtype)
+{
+    if (!ctx || !b) return fail(TWM_INVALID_HANDLE, "%s: null handle", who);
+    if (b->ctx != ctx) return fail(TWM_INVALID_HANDLE, "%s: bank belongs to another context", who);
+    if (a_dtype != TWM_F16 && a_dtype != TWM_F32) return fail(TWM_UNSUPPORTED_OP, "%s: activations must be f16 or f32", who);
+    if (b->k != 0 && b->n != 0) {
+        if (!a_dev) return fail(TWM_INVALID_HANDLE, "%s: null activations", who);
+        if (((uintptr_t)a_dev & 15) != 0) return fail(TWM_SHAPE_ERROR, "%s: activations must be 16-byte aligned", who);
+    }
+    return TWM_OK;
+}
+
+int twm_bank_gemv(twm_ctx *ctx, const twm_bank *b, const void *a_dev, int a_dtype, uint32_t a_slot_stride,
+                  const float *topk_ids_dev, uint32_t top_k, int act, float *out_dev)
+{
+    if (int rc = bank_common_checks("twm_bank_gemv", ctx, b, a_dev, a_dtype)) return rc;
+    if (act < 0 || act > 2) return fail(TWM_UNSUPPORTED_OP, "twm_bank_gemv: act must be 0 (none), 1 (GEGLU) or 2 (SwiGLU)");
+    if (act != 0 && !b->paired) return fail(TWM_UNSUPPORTED_OP, "twm_bank_gemv: a fused gate needs a bank built with pair_gate_up");
+    if (top_k == 0 || b->n == 0) return TWM_OK;
+    if (top_k > 65535u) return fail(TWM_SHAPE_ERROR, "twm_bank_gemv: at most 65535 slots per call");
+    if (!topk_ids_dev || !out_dev) return fail(TWM_INVALID_HANDLE, "twm_bank_gemv: null pointer");
+    uint32_t width = act ? b->n / 2 : b->n;
+    if (b->k == 0 || b->experts == 0) return twm_memset_zero(ctx, out_dev, (size_t)top_k * width * 4);  // gate(0) * 0 = 0
+    // every slot's row must keep the 16-byte alignment of the loads
+    if ((a_slot_stride * (a_dtype == TWM_F32 ? 4u : 2u)) % 16u != 0)
+        return fail(TWM_SHAPE_ERROR, "twm_bank_gemv: the activation stride must keep rows 16-byte aligned");
+    HIP_TRY(launch_bank_gemv(ctx->stream, bank_view(b), a_dev, a_dtype == TWM_F32, a_slot_stride, topk_ids_dev, top_k, act, out_dev),
+            TWM_DEVICE_ERROR, "bank gemv launch");
+    return TWM_OK;
+}
+
+int twm_bank_down_axpy(twm_ctx *ctx, const twm_bank *b, const void *a_all_dev, int a_dtype, const float *topk_ids_dev,
+                       const float *topk_weights_dev, uint32_t top_k, float *acc_dev)
+{
+    if (int rc = bank_common_checks("twm_bank_down_axpy", ctx, b, a_all_dev, a_dtype)) return rc;
+    if (top_k == 0 || b->n == 0 || b->k == 0 || b->experts == 0) return TWM_OK;  // nothing is added
+    if (top_k > (uint32_t)kMaxBankSlots) return fail(TWM_SHAPE_ERROR, "twm_bank_down_axpy: at most %d slots per call, got %u", kMaxBankSlots, top_k);
+    if (!topk_ids_dev || !topk_weights_dev || !acc_dev) return fail(TWM_INVALID_HANDLE, "twm_bank_down_axpy: null pointer");
+    if ((b->k * (a_dtype == TWM_F32 ? 4u : 2u)) % 16u != 0)
+        return fail(TWM_SHAPE_ERROR, "twm_bank_down_axpy: K must keep the activation rows 16-byte aligned");
+    HIP_TRY(launch_bank_down_axpy(ctx->stream, bank_view(b), a_all_dev, a_dtype == TWM_F32, topk_ids_dev, topk_weights_dev, top_k, acc_dev),
+            TWM_DEVICE_ERROR, "bank down_axpy launch");
+    return TWM_OK;
+}
+
+int twm_geglu_rows(twm_ctx *ctx, const float *gate_up_dev, uint32_t batch, uint32_t dim, int paired, float *out_dev)
+{
+    if (!ctx) return fail(TWM_INVALID_HANDLE, "twm_geglu_rows: null context");
+    if (paired && dim % kPairWidth != 0)
+        return fail(TWM_SHAPE_ERROR, "twm_geglu_rows: the paired order needs dim %% %u == 0, got %u", kPairWidth, dim);
+    if ((uint64_t)dim * 2 > 0xFFFFFFFFull) return fail(TWM_SHAPE_ERROR, "twm_geglu_rows: 2 * dim overflows u32");
+    if ((uint64_t)batch * dim == 0) return TWM_OK;
+    if (!gate_up_dev || !out_dev) return fail(TWM_INVALID_HANDLE, "twm_geglu_rows: null pointer");
+    HIP_TRY(launch_geglu_rows(ctx->stream, gate_up_dev, out_dev, dim, batch, paired != 0), TWM_DEVICE_ERROR, "geglu_rows launch");
     return TWM_OK;
 }
 

@@ -16,42 +16,9 @@
 // holds row l%4, k-piece l/4) feeds all 32 MFMAs of the chunk, the piece being chosen by the ABID
 // immediate: no LDS, no per-MFMA operand traffic, and the output row m of column n is register m of
 // lane n.  Per 1 KiB of nibbles the wave spends 36 VALU on the unpack, 8 MFMA and 1 scale-FMA.
-#include "twm_device.h"
+#include "twm_gemv4_core.h"
 
 namespace twm {
-
-typedef _Float16 half4v __attribute__((ext_vector_type(4)));
-
-struct Gemv4Consts {
-    uint32_t mask_lo, mask_hi, magic_lo, magic_hi;
-};
-
-__device__ __forceinline__ Gemv4Consts make_gemv4_consts()
-{
-    // opaque to the optimiser so that (w & mask) | magic becomes one v_and_or_b32
-    Gemv4Consts c = {0x000F000Fu, 0x00F000F0u, 0x64006400u, 0x54005400u};
-    asm volatile("" : "+s"(c.mask_lo), "+s"(c.mask_hi), "+v"(c.magic_lo), "+v"(c.magic_hi));
-    return c;
-}
-
-// eight nibbles -> eight exact f16 values q - 8 in k order, as two half4 (k 0..3 and k 4..7)
-__device__ __forceinline__ void gemv4_dequant_word(uint32_t w, const Gemv4Consts &c, half4v &lo4, half4v &hi4)
-{
-    union { uint32_t u[2]; half2v h2[2]; half4v h; } a, b;
-    uint32_t w8 = w >> 8;
-    a.u[0] = (w & c.mask_lo) | c.magic_lo;    // 1024 + q of k0, k1
-    a.u[1] = (w & c.mask_hi) | c.magic_hi;    //   64 + q of k2, k3
-    b.u[0] = (w8 & c.mask_lo) | c.magic_lo;   // k4, k5
-    b.u[1] = (w8 & c.mask_hi) | c.magic_hi;   // k6, k7
-    const half2v b_lo = {(_Float16)-1032.0f, (_Float16)-1032.0f};
-    const half2v b_hi = {(_Float16)-72.0f, (_Float16)-72.0f};
-    a.h2[0] += b_lo;
-    a.h2[1] += b_hi;
-    b.h2[0] += b_lo;
-    b.h2[1] += b_hi;
-    lo4 = a.h;
-    hi4 = b.h;
-}
 
 __device__ __forceinline__ void gemv4_store_out(const OutSpec &out, uint32_t m, uint32_t col, float v)
 {
@@ -62,19 +29,6 @@ __device__ __forceinline__ void gemv4_store_out(const OutSpec &out, uint32_t m, 
             if (rel < out.seg[s].width) out.seg[s].ptr[(size_t)m * out.seg[s].width + rel] = out.seg[s].bias ? v + out.seg[s].bias[rel] : v;
         }
     }
-}
-
-template <int NT>
-struct Chunk4 {
-    uint4v wq[NT][4];  // [tile][group in chunk]: this lane's column, 32 nibbles
-    uint2v sc[NT];     // four f16 scales
-    uint4v a;          // activations: row lane%4, k-piece lane/4 (8 halves)
-};
-
-template <int P>
-__device__ __forceinline__ float4v mfma_piece(half4v a, half4v b, float4v c)
-{
-    return __builtin_amdgcn_mfma_f32_4x4x4f16(a, b, c, 4, P, 0);  // CBSZ = 4: all 16 blocks use block P's A
 }
 
 // Workgroup = `waves` waves (blockDim.x / 64) that share NT tiles of 64 columns and split the
@@ -119,53 +73,9 @@ __global__ __launch_bounds__(1024) void k_gemv4(const char *__restrict__ cw, con
         for (int r = 0; r < RL; r++) acc[t][r] = 0.f;
 
     auto load_chunk = [&](Chunk4<NT> &r, uint32_t kc) {
-#pragma unroll
-        for (int t = 0; t < NT; t++) {
-            const char *blk = wbase[t] + (size_t)kc * kColBlockBytes;
-#pragma unroll
-            for (int g = 0; g < 4; g++) r.wq[t][g] = *(const uint4v *)(blk + g * 1024u + lane16);
-            r.sc[t] = *(const uint2v *)(blk + lane8);
-        }
-        uint32_t k0 = kc * 128u + apiece;
-        if (k0 > k - 8u) k0 = k - 8u;  // only the zero-padded groups of a last partial chunk get here
-        if (AF32) {
-            const float4 *p = (const float4 *)((const float *)a_any + (size_t)arow * k + k0);
-            float4 x = p[0], y = p[1];
-            union { half8 h; uint4v u; } cv;
-            cv.h = half8{(_Float16)x.x, (_Float16)x.y, (_Float16)x.z, (_Float16)x.w,
-                         (_Float16)y.x, (_Float16)y.y, (_Float16)y.z, (_Float16)y.w};
-            r.a = cv.u;
-        } else {
-            r.a = *(const uint4v *)((const _Float16 *)a_any + (size_t)arow * k + k0);
-        }
+        gemv4_load_chunk<NT, AF32>(r, wbase, kc, lane16, lane8, a_any, arow, apiece, k);
     };
-
-    auto compute_chunk = [&](const Chunk4<NT> &r) {
-        union { uint4v u; half4v h[2]; } av;
-        av.u = r.a;  // h[0] = k 0..3 of the lane's piece, h[1] = k 4..7
-#pragma unroll
-        for (int t = 0; t < NT; t++) {
-            union { uint2v u; _Float16 h[4]; } sv;
-            sv.u = r.sc[t];
-#pragma unroll
-            for (int g = 0; g < 4; g++) {
-                float4v d = {0.f, 0.f, 0.f, 0.f};
-                half4v lo4, hi4;
-#define TWM_PIECE(W, PIECE)                                       \
-    gemv4_dequant_word(r.wq[t][g][W], dq, lo4, hi4);              \
-    d = mfma_piece<PIECE>(av.h[0], lo4, d);                       \
-    d = mfma_piece<PIECE>(av.h[1], hi4, d);
-                if (g == 0) { TWM_PIECE(0, 0) TWM_PIECE(1, 1) TWM_PIECE(2, 2) TWM_PIECE(3, 3) }
-                if (g == 1) { TWM_PIECE(0, 4) TWM_PIECE(1, 5) TWM_PIECE(2, 6) TWM_PIECE(3, 7) }
-                if (g == 2) { TWM_PIECE(0, 8) TWM_PIECE(1, 9) TWM_PIECE(2, 10) TWM_PIECE(3, 11) }
-                if (g == 3) { TWM_PIECE(0, 12) TWM_PIECE(1, 13) TWM_PIECE(2, 14) TWM_PIECE(3, 15) }
-#undef TWM_PIECE
-                float s = (float)sv.h[g];
-#pragma unroll
-                for (int rr = 0; rr < RL; rr++) acc[t][rr] = fmaf(d[rr], s, acc[t][rr]);
-            }
-        }
-    };
+    auto compute_chunk = [&](const Chunk4<NT> &r) { gemv4_compute_chunk<NT, RL>(r, dq, acc); };
 
     {
         // two register sets used alternately: the loads of one are in flight while the other is consumed

@@ -47,6 +47,14 @@ struct WeightView {
     uint32_t k, n, groups, n_tiles, k_chunks;
 };
 
+// Expert bank: `experts` matrices of the same (K, N) in the column-lane order, expert e at cq + e * expert_bytes
+struct BankView {
+    const void *cq;
+    size_t expert_bytes;
+    uint32_t experts, k, n, n_pad, k_chunks;
+};
+constexpr int kMaxBankSlots = 16;   // top-k of the fused down + axpy launch (one wave or more per slot)
+
 struct DecodePlan {
     uint32_t nt;      // tiles per workgroup (1, 2, 4)
     uint32_t waves;   // waves per workgroup (4, 8, 16); they split the workgroup's k-range
@@ -79,8 +87,10 @@ hipError_t launch_ref_gemv(hipStream_t s, const float *a, const uint8_t *packed,
 hipError_t launch_repack(hipStream_t s, const uint8_t *packed, const uint16_t *scales, uint32_t k, uint32_t n,
                          void *qw, void *sc, uint32_t n_tiles, uint32_t k_chunks);
 hipError_t launch_weight_dequant_f16(hipStream_t s, const WeightView &w, uint16_t *out_kn);
+// pair_ffn != 0: the source columns are [gate | up] halves of width pair_ffn and the copy is written in the
+// paired order (32 gate, 32 up, ...)
 hipError_t launch_repack_col(hipStream_t s, const uint8_t *packed, const uint16_t *scales, uint32_t k, uint32_t n,
-                             void *cq, uint32_t n_pad, uint32_t k_chunks);
+                             void *cq, uint32_t n_pad, uint32_t k_chunks, uint32_t pair_ffn = 0);
 hipError_t launch_weight_dequant_f16_col(hipStream_t s, const WeightView &w, uint16_t *out_kn);
 // swiglu_out != nullptr (the weight in the paired gate_up column order, N = 2*ffn a multiple of 64): instead
 // of the N columns, write silu(gate) * up of every feature to swiglu_out[m][ffn]; `out` is ignored.
@@ -95,6 +105,12 @@ hipError_t launch_splitk_reduce(hipStream_t s, const float *partials, const OutS
                                 uint32_t n_ld, uint32_t splits);
 hipError_t launch_stream(hipStream_t s, const WeightView &w, const void *a, bool a_f32, uint32_t m, const OutSpec &out,
                          uint32_t splits, uint32_t waves, float *partials, size_t partial_bytes);
+hipError_t launch_geglu_rows(hipStream_t s, const float *gu, float *out, uint32_t dim, uint32_t batch, bool paired);
+// act: 0 out[slot][n]; 1 gelu_tanh(gate) * up, 2 silu(gate) * up into out[slot][n/2] (paired bank)
+hipError_t launch_bank_gemv(hipStream_t s, const BankView &b, const void *a, bool a_f32, uint32_t a_slot_stride,
+                            const float *ids, uint32_t slots, int act, float *out);
+hipError_t launch_bank_down_axpy(hipStream_t s, const BankView &b, const void *a_all, bool a_f32, const float *ids,
+                                 const float *weights, uint32_t slots, float *accum);
 hipError_t launch_decode(hipStream_t s, const WeightView &w, const void *a, bool a_f32, uint32_t m, const OutSpec &out,
                          float *ws, unsigned *counters, DecodePlan plan);
 

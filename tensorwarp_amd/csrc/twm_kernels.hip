@@ -640,7 +640,7 @@ hipError_t launch_weight_dequant_f16(hipStream_t s, const WeightView &w, uint16_
 // ---------------------------------------------------------------------------------
 __global__ __launch_bounds__(256) void k_repack_col(const uint4v *__restrict__ packed, const uint16_t *__restrict__ scales,
                                                      uint32_t groups, uint32_t n, uint32_t k_chunks, uint32_t tiles64,
-                                                     char *__restrict__ cw)
+                                                     char *__restrict__ cw, uint32_t pair_ffn)
 {
     size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;  // ((tile * k_chunks + kc) * 4 + g) * 64 + lane
     if (idx >= (size_t)tiles64 * k_chunks * 256) return;
@@ -651,8 +651,10 @@ __global__ __launch_bounds__(256) void k_repack_col(const uint4v *__restrict__ p
     uint4v w = {0x88888888u, 0x88888888u, 0x88888888u, 0x88888888u};
     uint32_t sbits = 0;
     if (g < groups && col < n) {
-        w = packed[(size_t)g * n + col];
-        sbits = scales[(size_t)g * n + col];
+        // pair_ffn != 0: the source is [gate | up] (n = 2 * pair_ffn) and the copy takes the paired order
+        uint32_t src = pair_ffn ? (col >> 6) * kPairWidth + (col & 31u) + ((col & kPairWidth) ? pair_ffn : 0u) : col;
+        w = packed[(size_t)g * n + src];
+        sbits = scales[(size_t)g * n + src];
     }
     uint4v o = {permute_word(w[0]), permute_word(w[1]), permute_word(w[2]), permute_word(w[3])};
     char *base = cw + blk * kColBlockBytes;
@@ -661,12 +663,12 @@ __global__ __launch_bounds__(256) void k_repack_col(const uint4v *__restrict__ p
 }
 
 hipError_t launch_repack_col(hipStream_t s, const uint8_t *packed, const uint16_t *scales, uint32_t k, uint32_t n,
-                             void *cq, uint32_t n_pad, uint32_t k_chunks)
+                             void *cq, uint32_t n_pad, uint32_t k_chunks, uint32_t pair_ffn)
 {
     size_t total = (size_t)(n_pad / 64) * k_chunks * 256;
     if (total == 0) return hipSuccess;
     hipLaunchKernelGGL(k_repack_col, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, (const uint4v *)packed,
-                       scales, k / 32, n, k_chunks, n_pad / 64, (char *)cq);
+                       scales, k / 32, n, k_chunks, n_pad / 64, (char *)cq, pair_ffn);
     return hipGetLastError();
 }
 

@@ -390,6 +390,55 @@ class TWMarlinWeights:
         return self.repacked
 
 
+class ExpertBank:
+    """All experts of one MoE projection, repacked (twm_bank): the buffers and strides that
+    moe_batched_marlin.rs hands to its batched kernels."""
+
+    def __init__(self, device, handle, k, n, num_experts, paired):
+        self.device, self.handle, self.k, self.n, self.num_experts, self.paired = device, handle, k, n, num_experts, paired
+
+    @classmethod
+    def from_device(cls, device, packed_buf, scales_buf, packed_bytes_per_expert, scales_per_expert, k, n, num_experts,
+                    pair_gate_up=False):
+        h = device._l.twm_bank_from_device(device.handle, packed_buf.ptr, scales_buf.ptr, packed_bytes_per_expert,
+                                           scales_per_expert, k, n, num_experts, int(pair_gate_up))
+        if not h:
+            raise DeviceError(_lib.SHAPE_ERROR, device._l.twm_last_error().decode())
+        return cls(device, h, k, n, num_experts, bool(pair_gate_up))
+
+    @property
+    def nbytes(self):
+        return self.device._l.twm_bank_bytes(self.handle)
+
+    def free(self):
+        if self.handle:
+            self.device._l.twm_bank_destroy(self.handle)
+            self.handle = None
+
+
+ACT_NONE, ACT_GEGLU, ACT_SWIGLU = 0, 1, 2
+
+
+def batched_marlin_gate_up(device, input, bank, topk_ids, output, top_k, act=ACT_NONE, per_slot_rows=False):
+    """moe_batched_marlin.rs:153 — output[s] = input x W[topk_ids[s]] for all slots in one launch; with act the
+    gate is applied in the store and output is [top_k, N/2] (replaces batched_marlin_split_geglu as well)."""
+    dt = _lib.F16 if input.dtype == "f16" else _lib.F32
+    _check(device._l.twm_bank_gemv(device.handle, bank.handle, input.ptr, dt, bank.k if per_slot_rows else 0,
+                                   topk_ids.ptr, top_k, act, output.ptr))
+
+
+def batched_marlin_split_geglu(device, gate_up, output, moe_dim, top_k, paired=False):
+    """moe_batched_marlin.rs:215"""
+    _check(device._l.twm_geglu_rows(device.handle, gate_up.ptr, top_k, moe_dim, int(paired), output.ptr))
+
+
+def batched_marlin_down_axpy(device, geglu_all, bank, topk_ids, topk_weights, acc, top_k):
+    """moe_batched_marlin.rs:184 — acc += sum_s topk_weights[s] * (geglu_all[s] x W[topk_ids[s]]), slot order."""
+    dt = _lib.F16 if geglu_all.dtype == "f16" else _lib.F32
+    _check(device._l.twm_bank_down_axpy(device.handle, bank.handle, geglu_all.ptr, dt, topk_ids.ptr, topk_weights.ptr,
+                                        top_k, acc.ptr))
+
+
 class GraphCapture:
     """cuda_graph.rs:72-118"""
 

@@ -650,6 +650,135 @@ def test_repacked_weight_blob_round_trip_through_a_warp_file(dev, tmp_path):
         x.free()
 
 
+# ---------------------------------------------------------------- expert banks (MoE decode)
+
+def make_bank(dev, k, n, experts, seed, pair=False, pad_bytes=0, pad_scales=0):
+    """Expert matrices back to back in two buffers with optional slack between experts, as the reference's
+    experts_gu_raw / experts_gu_scales."""
+    G = k // 32
+    pb, sb = G * n * 16 + pad_bytes, G * n + pad_scales
+    packed = [O.synth_packed(k, n, seed + 2 * e) for e in range(experts)]
+    scales = [O.synth_scales(k, n, seed + 2 * e + 1) for e in range(experts)]
+    pbuf = np.full(experts * pb, 0xEE, np.uint8)
+    sbuf = np.full(experts * sb, 0x7BFF, np.uint16)
+    for e in range(experts):
+        pbuf[e * pb:e * pb + G * n * 16] = packed[e]
+        sbuf[e * sb:e * sb + G * n] = scales[e]
+    bank = T.ExpertBank.from_device(dev, T.GpuTensor.from_host(dev, pbuf), T.GpuTensor.from_host(dev, sbuf, "f16"),
+                                    pb, sb, k, n, experts, pair_gate_up=pair)
+    return bank, packed, scales
+
+
+def geglu_close(got, g, u, want):
+    got, want = np.asarray(got, np.float64), np.asarray(want, np.float64)
+    return bool(np.all(np.abs(got - want) <= 6e-7 * np.abs(np.asarray(g, np.float64) * np.asarray(u, np.float64)) + 1e-30))
+
+
+def test_geglu_rows(dev):
+    batch, dim = 8, 96
+    gu = (O.synth_normal_f32(batch * 2 * dim, 1020) * np.float32(2.5)).reshape(batch, 2 * dim)
+    g, u = np.ascontiguousarray(gu[:, :dim]), np.ascontiguousarray(gu[:, dim:])
+    out = T.GpuTensor.zeros(dev, (batch, dim), "f32")
+    T.batched_marlin_split_geglu(dev, T.GpuTensor.from_host(dev, gu), out, dim, batch)
+    assert geglu_close(out.to_host(), g, u, O.gelu_mul(g, u))
+    j = np.arange(dim)
+    col = (j // 32) * 64 + j % 32
+    paired = np.zeros_like(gu)
+    paired[:, col], paired[:, col + 32] = g, u
+    out2 = T.GpuTensor.zeros(dev, (batch, dim), "f32")
+    T.batched_marlin_split_geglu(dev, T.GpuTensor.from_host(dev, paired), out2, dim, batch, paired=True)
+    assert np.array_equal(out2.to_host(), out.to_host())
+
+
+@pytest.mark.parametrize("k,dim,experts,top_k", [(2816, 704, 12, 8), (256, 32, 3, 2), (1184, 96, 5, 4), (64, 64, 4, 1)])
+def test_bank_gate_up_and_fused_geglu(dev, k, dim, experts, top_k):
+    # batched_marlin_gate_up + batched_marlin_split_geglu (moe_q4_generate.rs:618-631), Gemma MoE shape first
+    n = 2 * dim
+    ids_h = np.array([(5 * s + 3) % experts for s in range(top_k)], np.float32)
+    ids = T.GpuTensor.from_host(dev, ids_h)
+    a16 = O.synth_act_f16(1, k, 1030)
+    a32 = f16_as_f32(a16).reshape(1, k)
+    plain, packed, scales = make_bank(dev, k, n, experts, 1040, pad_bytes=32, pad_scales=8)
+    out = T.GpuTensor.from_host(dev, np.full((top_k, n), np.nan, np.float32))
+    T.batched_marlin_gate_up(dev, T.GpuTensor.from_host(dev, a32), plain, ids, out, top_k)
+    truth = O.bank_gemv_f64(a32, packed, scales, ids_h, k, n)
+    assert rel_err(out.to_host(), truth) < TIGHT
+    # the same rows as the dense kernel on one expert at a time, bit for bit (f16 and f32 activations)
+    out16 = T.GpuTensor.zeros(dev, (top_k, n), "f32")
+    T.batched_marlin_gate_up(dev, T.GpuTensor.from_host(dev, a16, "f16"), plain, ids, out16, top_k)
+    assert np.array_equal(out16.to_host(), out.to_host())
+    e0 = int(ids_h[0])
+    w0 = T.MarlinWeight.upload(dev, packed[e0], scales[e0], k, n)
+    c0 = T.GpuTensor.zeros(dev, (n,), "f32")
+    T.gemm(dev, w0, T.GpuTensor.from_host(dev, a16, "f16"), 1, c0, 1)
+    assert rel_err(out.to_host()[0], c0.to_host()) < 1e-5
+    # device-indexed single expert (gemm_tw_marlin_m1_indirect): one slot, ids pointer at the wanted entry
+    one = T.GpuTensor.zeros(dev, (n,), "f32")
+    last = T.GpuTensor.from_host(dev, ids_h[top_k - 1:top_k].copy())
+    T.batched_marlin_gate_up(dev, T.GpuTensor.from_host(dev, a32), plain, last, one, 1)
+    assert np.array_equal(one.to_host(), out.to_host()[top_k - 1])
+    # fused GEGLU on the paired bank = unfused rows + split_geglu, bit for bit
+    pairedb, _, _ = make_bank(dev, k, n, experts, 1040, pair=True)
+    seq = T.GpuTensor.zeros(dev, (top_k, dim), "f32")
+    T.batched_marlin_split_geglu(dev, out, seq, dim, top_k)
+    fused = T.GpuTensor.from_host(dev, np.full((top_k, dim), np.nan, np.float32))
+    T.batched_marlin_gate_up(dev, T.GpuTensor.from_host(dev, a32), pairedb, ids, fused, top_k, act=T.ACT_GEGLU)
+    assert np.array_equal(fused.to_host(), seq.to_host())
+    tg, tu = truth[:, :dim], truth[:, dim:]
+    want = 0.5 * tg * (1.0 + np.tanh(0.7978845608 * (tg + 0.044715 * tg ** 3))) * tu
+    assert rel_err(fused.to_host(), want) < TIGHT
+    sw = T.GpuTensor.zeros(dev, (top_k, dim), "f32")
+    T.batched_marlin_gate_up(dev, T.GpuTensor.from_host(dev, a32), pairedb, ids, sw, top_k, act=T.ACT_SWIGLU)
+    assert rel_err(sw.to_host(), tg / (1.0 + np.exp(-tg)) * tu) < TIGHT
+    with pytest.raises(T.DeviceError):
+        T.batched_marlin_gate_up(dev, T.GpuTensor.from_host(dev, a32), plain, ids, fused, top_k, act=T.ACT_GEGLU)
+    for x in (plain, pairedb, w0):
+        x.free()
+
+
+@pytest.mark.parametrize("k,n,experts,top_k", [(704, 2816, 12, 8), (64, 40, 3, 3), (1184, 200, 4, 16), (4096, 128, 2, 1)])
+def test_bank_down_axpy_adds_in_slot_order(dev, k, n, experts, top_k):
+    ids_h = np.array([(7 * s + 1) % experts for s in range(top_k)], np.float32)
+    wts_h = (np.abs(O.synth_normal_f32(top_k, 1050)) * np.float32(0.3) + np.float32(0.01)).astype(np.float32)
+    a16 = O.synth_act_f16(top_k, k, 1051)
+    a32 = f16_as_f32(a16).reshape(top_k, k)
+    acc0 = O.synth_normal_f32(n, 1052)
+    bank, packed, scales = make_bank(dev, k, n, experts, 1060)
+    ids, wts = T.GpuTensor.from_host(dev, ids_h), T.GpuTensor.from_host(dev, wts_h)
+    acc = T.GpuTensor.from_host(dev, acc0)
+    T.batched_marlin_down_axpy(dev, T.GpuTensor.from_host(dev, a32), bank, ids, wts, acc, top_k)
+    rows = O.bank_gemv_f64(a32, packed, scales, ids_h, k, n)
+    truth = acc0.astype(np.float64) + (wts_h.astype(np.float64)[:, None] * rows).sum(axis=0)
+    assert rel_err(acc.to_host(), truth) < TIGHT
+    # equal, bit for bit, to the per-slot rows of the batched GEMV combined on the host in slot order in f32
+    per = T.GpuTensor.zeros(dev, (top_k, n), "f32")
+    T.batched_marlin_gate_up(dev, T.GpuTensor.from_host(dev, a32), bank, ids, per, top_k, per_slot_rows=True)
+    ph = per.to_host().reshape(top_k, n)
+    assert rel_err(ph, rows) < TIGHT
+    acc2 = T.GpuTensor.from_host(dev, acc0)
+    T.batched_marlin_down_axpy(dev, T.GpuTensor.from_host(dev, a16, "f16"), bank, ids, wts, acc2, top_k)
+    assert np.array_equal(acc2.to_host(), acc.to_host())          # run to run and f16 / f32 activations alike
+    if top_k <= 16:
+        with pytest.raises(T.DeviceError):
+            T.batched_marlin_down_axpy(dev, T.GpuTensor.from_host(dev, np.zeros((17, k), np.float32)), bank,
+                                       T.GpuTensor.from_host(dev, np.zeros(17, np.float32)),
+                                       T.GpuTensor.from_host(dev, np.zeros(17, np.float32)), acc2, 17)
+    bank.free()
+
+
+def test_bank_ignores_ids_outside_the_bank(dev):
+    k, n, experts = 128, 64, 3
+    bank, packed, scales = make_bank(dev, k, n, experts, 1070)
+    ids_h = np.array([1.0, -1.0, 3.0, 2.0, np.nan], np.float32)
+    a32 = f16_as_f32(O.synth_act_f16(1, k, 1071)).reshape(1, k)
+    out = T.GpuTensor.from_host(dev, np.full((5, n), np.nan, np.float32))
+    T.batched_marlin_gate_up(dev, T.GpuTensor.from_host(dev, a32), bank, T.GpuTensor.from_host(dev, ids_h), out, 5)
+    got = out.to_host().reshape(5, n)
+    assert not got[1].any() and not got[2].any() and not got[4].any()
+    assert rel_err(got[[0, 3]], O.bank_gemv_f64(a32, packed, scales, [1, 2], k, n)) < TIGHT
+    bank.free()
+
+
 # ---------------------------------------------------------------- fused projections
 
 def test_fused_qkv_and_gate_up_equal_separate_projections(dev):

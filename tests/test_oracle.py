@@ -371,3 +371,21 @@ def test_pair_gate_up_is_the_32_column_interleave():
     j = np.arange(ffn)
     col = (j // 32) * 64 + j % 32
     assert np.array_equal(wp[:, col], wf[:, :ffn]) and np.array_equal(wp[:, col + 32], wf[:, ffn:])
+
+
+def test_gelu_mul_against_f64_and_its_limits():
+    # batched_marlin_split_geglu / warp_fused_gelu_mul: 0.5 g (1 + tanh(0.7978845608 (g + 0.044715 g^3))) * up.
+    # Against the same expression in f64 (the 1 + tanh cancellation for negative g turns one ulp of tanhf into
+    # an absolute error of about 2^-24 |g u|), the identity gelu(g) - gelu(-g) = g, and both tails.
+    g = (O.synth_normal_f32(5000, 1010) * np.float32(3.0)).astype(np.float32)
+    u = O.synth_normal_f32(5000, 1011)
+    out = O.gelu_mul(g, u)
+    g64, u64 = g.astype(np.float64), u.astype(np.float64)
+    truth = 0.5 * g64 * (1.0 + np.tanh(np.float64(np.float32(0.7978845608)) * (g64 + np.float64(np.float32(0.044715)) * g64 ** 3))) * u64
+    assert np.all(np.abs(out - truth) <= 4e-7 * np.abs(g64 * u64) + 1e-30)
+    ones = np.ones_like(g)
+    assert np.allclose(O.gelu_mul(g, ones).astype(np.float64) - O.gelu_mul(-g, ones), g64, rtol=0, atol=2e-6)
+    edge = np.array([0.0, 10.0, -10.0, 1.0], np.float32)
+    r = O.gelu_mul(edge, np.full(4, 3.0, np.float32))
+    assert r[0] == 0.0 and r[1] == 30.0 and r[2] == 0.0
+    assert abs(r[3] - 3.0 * 0.8411919906082768) < 1e-6      # gelu_tanh(1) = 0.84119199...
