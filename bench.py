@@ -54,6 +54,46 @@ def make_layer(rng, shapes):
     return host
 
 
+class VendorGemm:
+    """rocBLAS gemm_ex (f16 x f16 -> f32, f32 accumulation) on the context's stream, through ctypes: a
+    yardstick for the prefill kernel, not part of the product.  Row-major C[M,N] = A[M,K] W[K,N] is the
+    column-major product C^T = W^T A^T, so W goes in as the first operand with leading dimension N."""
+    OP_NONE, F16_R, F32_R, ALGO_STANDARD = 111, 150, 151, 0
+
+    def __init__(self, dev):
+        import ctypes as C
+        self.C, self.dev, self.ok = C, dev, False
+        try:
+            self.lib = C.CDLL("librocblas.so")
+            self.handle = C.c_void_p()
+            if self.lib.rocblas_create_handle(C.byref(self.handle)) != 0:
+                return
+            if self.lib.rocblas_set_stream(self.handle, C.c_void_p(dev._l.twm_ctx_stream(dev.handle))) != 0:
+                return
+            self.lib.rocblas_gemm_ex.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p,
+                                                 C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_int, C.c_int, C.c_void_p,
+                                                 C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_int, C.c_int, C.c_int,
+                                                 C.c_int, C.c_int32, C.c_uint32]
+            self.ok = True
+        except OSError:
+            pass
+
+    def time(self, a, w16, c, m, n, k, reps):
+        C = self.C
+        alpha, beta = C.c_float(1.0), C.c_float(0.0)
+
+        def call(i):
+            return self.lib.rocblas_gemm_ex(self.handle, self.OP_NONE, self.OP_NONE, n, m, k, C.byref(alpha),
+                                            w16.ptr, self.F16_R, n, a.ptr, self.F16_R, k, C.byref(beta),
+                                            c.ptr, self.F32_R, n, c.ptr, self.F32_R, n, self.F32_R, self.ALGO_STANDARD, 0, 0)
+        if call(0) != 0:
+            return None
+        for i in range(3):
+            call(i)
+        self.dev.synchronize()
+        return time_launches(self.dev, call, reps)
+
+
 def time_launches(dev, fn, reps):
     """average milliseconds per call of fn() over `reps` calls, HIP events on the context's stream"""
     e0, e1 = dev.event(), dev.event()
@@ -78,6 +118,8 @@ def main():
     ap.add_argument("--no-lm-head", action="store_true", help="skip the LM-head GEMV + argmax timing")
     ap.add_argument("--no-swiglu", action="store_true", help="skip the fused gate_up + SwiGLU timing")
     ap.add_argument("--no-moe", action="store_true", help="skip the expert-bank (MoE decode) timing")
+    ap.add_argument("--no-vendor-gemm", action="store_true",
+                    help="skip timing rocBLAS' dense FP16 GEMM beside the prefill kernel")
     ap.add_argument("--extra", action="store_true", help="also time batched decode (M=4..32) on the gate_up shape")
     ap.add_argument("--sweep-splits", action="store_true",
                     help="also time every projection at M=1,4,8,16,32 with forced split-K factors next to the library's "
@@ -366,6 +408,7 @@ def main():
     prefill = None
     if not args.no_prefill:
         prefill = {}
+        vendor = None if args.no_vendor_gemm else VendorGemm(dev)
         for k, n in ((4096, 11008), (11008, 4096)):
             packed = rng.integers(0, 256, size=(k // 32) * n * 16, dtype=np.uint8)
             scales = (np.abs(rng.standard_normal((k // 32) * n, dtype=np.float32)) * np.float32(0.02)).astype(np.float16)
@@ -383,6 +426,21 @@ def main():
                 tf = 2.0 * m * n * k / (ms * 1e-3) / 1e12
                 prefill["M%d_K%d_N%d" % (m, k, n)] = {"us": round(ms * 1e3, 1), "TFLOPs": round(tf, 1),
                                                       "frac_mfma_f16_peak": round(tf / MFMA_F16_PEAK_TFLOPS, 4)}
+                if vendor is not None and vendor.ok:
+                    # the vendor library's dense FP16 GEMM on the already unpacked weights (no Q4 unpack in the
+                    # timed region): what the reference's dequant + library-GEMM prefill route would cost here
+                    if m == 512:
+                        w16 = w.dequant_f16()
+                    ours = c_m.to_host() if m == 512 else None
+                    v_ms = vendor.time(a_m, w16, c_m, m, n, k, 20)
+                    if v_ms is not None and ours is not None:
+                        theirs = c_m.to_host()
+                        assert np.abs(theirs - ours).max() <= 2e-3 * np.abs(ours).max(), "rocBLAS result differs"
+                    if v_ms is not None:
+                        prefill["M%d_K%d_N%d" % (m, k, n)]["rocblas_dense_f16_us"] = round(v_ms * 1e3, 1)
+                        prefill["M%d_K%d_N%d" % (m, k, n)]["rocblas_dense_f16_TFLOPs"] = round(2.0 * m * n * k / (v_ms * 1e-3) / 1e12, 1)
+                    if m == 2048:
+                        w16.free()
                 a_m.free()
                 c_m.free()
             w.free()
