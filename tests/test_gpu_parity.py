@@ -920,6 +920,59 @@ def test_layer_graph_replays_match_eager(dev):
     graph.destroy()
 
 
+def test_graph_of_fused_epilogues_and_expert_banks(dev):
+    # SwiGLU GEMV (split-K inside the launch), biased QKV split, the MoE block (fused GEGLU, then down + weighted
+    # sum onto an accumulator that the graph itself clears) and the argmax, captured together and replayed with
+    # eager work in between; every replay must reproduce the eager results bit for bit
+    h, ffn, kv = 2048, 96, 64
+    gp, gs = O.synth_packed(h, ffn, 1100), O.synth_scales(h, ffn, 1101)
+    up, us = O.synth_packed(h, ffn, 1102), O.synth_scales(h, ffn, 1103)
+    wgu = T.MarlinWeight.gate_up(dev, (T.GpuTensor.from_host(dev, gp), T.GpuTensor.from_host(dev, gs, "f16")),
+                                 (T.GpuTensor.from_host(dev, up), T.GpuTensor.from_host(dev, us, "f16")), h, ffn)
+    qp, qs, a16 = synth(h, h + 2 * kv, 1, 1104)
+    wqkv = T.MarlinWeight.upload(dev, qp, qs, h, h + 2 * kv)
+    x = T.GpuTensor.from_host(dev, a16, "f16")
+    biases = [T.GpuTensor.from_host(dev, O.synth_normal_f32(n, 1105 + i)) for i, n in enumerate((h, kv, kv))]
+    dim, experts, top_k = 64, 6, 4
+    gub, _, _ = make_bank(dev, h, 2 * dim, experts, 1110, pair=True)
+    db, _, _ = make_bank(dev, dim, h, experts, 1130)
+    ids = T.GpuTensor.from_host(dev, np.array([4, 0, 5, 2], np.float32))
+    wts = T.GpuTensor.from_host(dev, np.array([0.4, 0.3, 0.2, 0.1], np.float32))
+    act = T.GpuTensor.zeros(dev, (ffn,), "f32")
+    q, kk, v = (T.GpuTensor.zeros(dev, (n,), "f32") for n in (h, kv, kv))
+    geglu = T.GpuTensor.zeros(dev, (top_k, dim), "f32")
+    moe_acc = T.GpuTensor.zeros(dev, (h,), "f32")
+    token = T.GpuTensor.from_host(dev, np.zeros(1, np.int32))
+
+    def body():
+        T.gemm_swiglu(dev, wgu, x, 1, act)
+        T.gemm_split(dev, wqkv, x, 1, [q, kk, v], [h, kv, kv], 0, biases=biases)
+        T.batched_marlin_gate_up(dev, x, gub, ids, geglu, top_k, act=T.ACT_GEGLU)
+        dev._l.twm_memset_zero(dev.handle, moe_acc.ptr, h * 4)
+        T.batched_marlin_down_axpy(dev, geglu, db, ids, wts, moe_acc, top_k)
+        T.argmax(dev, moe_acc, token, 1, h)
+
+    body()
+    dev.synchronize()
+    bufs = {"act": act, "q": q, "k": kk, "v": v, "geglu": geglu, "moe": moe_acc, "token": token}
+    eager = {nm: t.to_host().copy() for nm, t in bufs.items()}
+    assert int(eager["token"][0]) == int(np.argmax(eager["moe"])) and np.isfinite(eager["moe"]).all()
+    graph = T.GraphCapture.record_with_device(dev, body)
+    for rep in range(4):
+        for nm, t in bufs.items():
+            if nm != "token":
+                t.copy_from_host(np.full(t.numel, np.nan, np.float32))
+        graph.replay()
+        dev.synchronize()
+        for nm, t in bufs.items():
+            assert np.array_equal(t.to_host(), eager[nm]), (rep, nm)
+        T.gemm_swiglu(dev, wgu, x, 1, act, None, 3)                 # eager work between replays
+        dev.synchronize()
+    graph.destroy()
+    for wobj in (wgu, wqkv, gub, db):
+        wobj.free()
+
+
 def test_graph_of_batched_and_prefill_launches():
     # The multi-kernel paths (f32 -> f16 conversion, split-K partials + ordered reduce) captured in a graph
     # as their FIRST use in a fresh context, then replayed with eager work in between; every replay must
