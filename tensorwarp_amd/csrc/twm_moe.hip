@@ -36,6 +36,36 @@ __device__ __forceinline__ uint32_t expert_of(float id, uint32_t experts)
     return (id >= 0.f && id < (float)experts) ? (uint32_t)id : experts;
 }
 
+// This wave's chunks first, first + stride, ... of one 64-column tile with three register sets: for the short
+// K loops of expert matrices (two or three chunks per wave) every load is in flight before the first unpack.
+template <bool AF32>
+__device__ __forceinline__ void bank_accumulate(const char *tile_base, const void *a_row, uint32_t first, uint32_t stride,
+                                                uint32_t k_chunks, uint32_t k, uint32_t lane, float (&acc)[1][1])
+{
+    const char *wbase[1] = {tile_base};
+    const uint32_t lane16 = lane * 16u, lane8 = 4096u + lane * 8u, apiece = (lane >> 2) * 8u;
+    const Gemv4Consts dq = make_gemv4_consts();
+    Chunk4<1> r0, r1, r2;
+    uint32_t c0 = first, c1 = first + stride, c2 = first + 2u * stride;
+    if (c0 < k_chunks) gemv4_load_chunk<1, AF32>(r0, wbase, c0, lane16, lane8, a_row, 0, apiece, k);
+    if (c1 < k_chunks) gemv4_load_chunk<1, AF32>(r1, wbase, c1, lane16, lane8, a_row, 0, apiece, k);
+    if (c2 < k_chunks) gemv4_load_chunk<1, AF32>(r2, wbase, c2, lane16, lane8, a_row, 0, apiece, k);
+    for (;;) {
+        if (c0 >= k_chunks) break;
+        gemv4_compute_chunk<1, 1>(r0, dq, acc);
+        c0 += 3u * stride;
+        if (c0 < k_chunks) gemv4_load_chunk<1, AF32>(r0, wbase, c0, lane16, lane8, a_row, 0, apiece, k);
+        if (c1 >= k_chunks) break;
+        gemv4_compute_chunk<1, 1>(r1, dq, acc);
+        c1 += 3u * stride;
+        if (c1 < k_chunks) gemv4_load_chunk<1, AF32>(r1, wbase, c1, lane16, lane8, a_row, 0, apiece, k);
+        if (c2 >= k_chunks) break;
+        gemv4_compute_chunk<1, 1>(r2, dq, acc);
+        c2 += 3u * stride;
+        if (c2 < k_chunks) gemv4_load_chunk<1, AF32>(r2, wbase, c2, lane16, lane8, a_row, 0, apiece, k);
+    }
+}
+
 // Workgroup = `waves` waves on one 64-column tile of one slot's expert; wave w takes chunks w, w + waves, ...
 // grid = (tiles64 rounded up to the 8 XCDs, slots).  ACT 0: out[slot][n]; 1 / 2: paired bank,
 // out[slot][n/2] = gelu_tanh / silu (gate) * up.
@@ -54,27 +84,10 @@ __global__ __launch_bounds__(1024) void k_bank_gemv(const char *__restrict__ ban
     const uint32_t eid = __builtin_amdgcn_readfirstlane(expert_of(ids[slot], experts));
 
     float acc[1][1] = {{0.f}};
-    if (eid < experts) {
-        const char *wbase[1] = {bank + (size_t)eid * expert_bytes + (size_t)tile * k_chunks * kColBlockBytes};
-        const void *a_slot = (const char *)a_any + (size_t)slot * a_slot_stride * (AF32 ? 4 : 2);
-        const uint32_t lane16 = lane * 16u, lane8 = 4096u + lane * 8u, apiece = (lane >> 2) * 8u;
-        const Gemv4Consts dq = make_gemv4_consts();
-        Chunk4<1> r0, r1;
-        uint32_t kc = wave;
-        if (kc < k_chunks) {
-            gemv4_load_chunk<1, AF32>(r0, wbase, kc, lane16, lane8, a_slot, 0, apiece, k);
-            while (true) {
-                uint32_t kn = kc + waves;
-                if (kn < k_chunks) gemv4_load_chunk<1, AF32>(r1, wbase, kn, lane16, lane8, a_slot, 0, apiece, k);
-                gemv4_compute_chunk<1, 1>(r0, dq, acc);
-                if (kn >= k_chunks) break;
-                kc = kn + waves;
-                if (kc < k_chunks) gemv4_load_chunk<1, AF32>(r0, wbase, kc, lane16, lane8, a_slot, 0, apiece, k);
-                gemv4_compute_chunk<1, 1>(r1, dq, acc);
-                if (kc >= k_chunks) break;
-            }
-        }
-    }
+    if (eid < experts)
+        bank_accumulate<AF32>(bank + (size_t)eid * expert_bytes + (size_t)tile * k_chunks * kColBlockBytes,
+                              (const char *)a_any + (size_t)slot * a_slot_stride * (AF32 ? 4 : 2), wave, waves, k_chunks, k,
+                              lane, acc);
     red[wave * 64 + lane] = acc[0][0];
     __syncthreads();
     if (ACT == 0) {
@@ -121,27 +134,9 @@ __global__ __launch_bounds__(1024) void k_bank_down_axpy(const char *__restrict_
     const uint32_t eid = __builtin_amdgcn_readfirstlane(expert_of(ids[slot], experts));
 
     float acc[1][1] = {{0.f}};
-    if (eid < experts) {
-        const char *wbase[1] = {bank + (size_t)eid * expert_bytes + (size_t)tile * k_chunks * kColBlockBytes};
-        const void *a_slot = (const char *)a_all + (size_t)slot * k * (AF32 ? 4 : 2);
-        const uint32_t lane16 = lane * 16u, lane8 = 4096u + lane * 8u, apiece = (lane >> 2) * 8u;
-        const Gemv4Consts dq = make_gemv4_consts();
-        Chunk4<1> r0, r1;
-        uint32_t kc = j;
-        if (kc < k_chunks) {
-            gemv4_load_chunk<1, AF32>(r0, wbase, kc, lane16, lane8, a_slot, 0, apiece, k);
-            while (true) {
-                uint32_t kn = kc + wps;
-                if (kn < k_chunks) gemv4_load_chunk<1, AF32>(r1, wbase, kn, lane16, lane8, a_slot, 0, apiece, k);
-                gemv4_compute_chunk<1, 1>(r0, dq, acc);
-                if (kn >= k_chunks) break;
-                kc = kn + wps;
-                if (kc < k_chunks) gemv4_load_chunk<1, AF32>(r0, wbase, kc, lane16, lane8, a_slot, 0, apiece, k);
-                gemv4_compute_chunk<1, 1>(r1, dq, acc);
-                if (kc >= k_chunks) break;
-            }
-        }
-    }
+    if (eid < experts)
+        bank_accumulate<AF32>(bank + (size_t)eid * expert_bytes + (size_t)tile * k_chunks * kColBlockBytes,
+                              (const char *)a_all + (size_t)slot * k * (AF32 ? 4 : 2), j, wps, k_chunks, k, lane, acc);
     red[wave * 64 + lane] = acc[0][0];
     __syncthreads();
     if (threadIdx.x < 64) {
@@ -182,7 +177,7 @@ hipError_t launch_geglu_rows(hipStream_t s, const float *gu, float *out, uint32_
 
 static uint32_t bank_waves(uint32_t k_chunks)
 {
-    uint32_t waves = 8;
+    uint32_t waves = 16;
     while (waves > 1 && k_chunks < waves * 2) waves /= 2;
     return waves;
 }
