@@ -205,6 +205,35 @@ def main():
                            "frac_hbm": round(b / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
                            "splits": T.pick_splits(k, n, 1)}
 
+    # the literal drop-in: gemm_tw_marlin_m1 on the reference's arrays (no repack), f32 activations
+    drop_in = {}
+    for name, k, n in LAYER_7B:
+        sets = []
+        for li in range(args.layers):
+            packed, scales, act = layers_host[li][name]
+            sets.append((T.GpuTensor.from_host(dev, packed), T.GpuTensor.from_host(dev, scales, "f16")))
+        a32 = T.GpuTensor.from_host(dev, layers_host[0][name][2].view(np.float16).astype(np.float32))
+        c32 = T.GpuTensor.zeros(dev, (n,), "f32")
+
+        def one(i, sets=sets, a32=a32, c32=c32, n=n, k=k):
+            p_, s_ = sets[i % args.layers]
+            T.gemm_tw_marlin_m1(dev, a32, p_, s_, c32, n, k)
+        for i in range(8):
+            one(i)
+        dev.synchronize()
+        ms = time_launches(dev, one, 100)
+        b = k * n // 2 + (k // 32) * n * 2 + k * 4 + n * 4
+        drop_in[name] = {"us": round(ms * 1e3, 2), "GBps": round(b / (ms * 1e-3) / 1e9, 1)}
+        one(0)                                             # layer 0 again, for the comparison
+        w, a, c = layers[0][name]
+        T.gemm(dev, w, a, 1, c)
+        ref = c.to_host()
+        assert np.abs(c32.to_host() - ref).max() <= 1e-4 * np.abs(ref).max(), "drop-in differs from the repacked path"
+        for p_, s_ in sets:
+            p_.free()
+            s_.free()
+    drop_in["layer_us"] = round(sum(v["us"] for v in drop_in.values()), 2)
+
     gu = per_shape["gate_up"]
     gu_bytes = algo_bytes(3584, 37888)
     roofline = {"bound": "hbm", "kernel": "k_gemv4 (gate_up 3584->37888, M=1)",
@@ -521,6 +550,7 @@ def main():
         "roofline": roofline,
         "cpu_baseline": cpu,
         "per_projection": per_shape,
+        "drop_in_reference_layout_m1": drop_in,
     }
     out["small_shapes_m1"] = small
     if lm:

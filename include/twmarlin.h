@@ -92,6 +92,10 @@ int twm_ctx_info(twm_ctx *ctx, char *buf, size_t buf_len);
  *   "dequant_src"   which repacked copy twm_weight_dequant_f16 unpacks: 0 = 16-column tiles, 1 = column lanes
  *   "prefill_min_m" smallest M that runs the prefill GEMM (default 33; below it the decode kernels run)
  *   "prefill_bm"    rows of A per prefill workgroup (64 or 128)
+ *   "m1_exact"      twm_gemm_tw_marlin_m1: 1 = f32 activations and f32 FMAs in the reference kernel's order with
+ *                   the reference's split-K rule and float atomics (bit-equal to the reference order when that
+ *                   rule yields one split); 0 (default) = the MFMA kernel
+ *   "m1_splits"     twm_gemm_tw_marlin_m1: split-K factor of the MFMA kernel (0 .. 64)
  * Values outside these sets return TWM_SHAPE_ERROR, unknown keys TWM_UNSUPPORTED_OP. */
 int twm_ctx_set_option(twm_ctx *ctx, const char *key, int value);
 
@@ -172,8 +176,13 @@ int twm_argmax_f32(twm_ctx *ctx, const float *input_dev, uint32_t rows, uint32_t
 /* ---- the quantized-GEMM entry point, reference layout in, no repack ------------------ */
 
 /* gemm_tw_marlin_m1 (quantize.rs:1301-1360): C[1,N] = A[1,K] * dequant(packed, scales),
- * f32 activations and output, arrays exactly as the reference holds them.
- * K % 32 != 0 returns TWM_SHAPE_ERROR where the reference asserts (quantize.rs:1311). */
+ * f32 activations and output, arrays exactly as the reference holds them (packed 16-byte aligned).
+ * Runs the M <= 4 MFMA kernel straight on those arrays: weights (q - 8) exact, every f32 activation
+ * enters as two f16 terms a = f16(a) + f16(a - f16(a)) (about 22 bits; |a| must stay inside the f16
+ * range), f32 sum per group times f32(scale), deterministic split-K.  Option "m1_exact" selects the
+ * plain f32 kernel in the reference's order instead (also taken when a_dev is not 16-byte aligned).
+ * K % 32 != 0 returns TWM_SHAPE_ERROR where the reference asserts (quantize.rs:1311).
+ * Uses the context's scratch like twm_gemm. */
 int twm_gemm_tw_marlin_m1(twm_ctx *ctx, const float *a_dev, const uint8_t *packed_dev,
                           const uint16_t *scales_dev, float *c_dev, uint32_t n, uint32_t k);
 /* gemm_tw_marlin_m1_from_buffer (quantize.rs:1731-1782): offsets in bytes (packed) and in
@@ -216,7 +225,8 @@ int twm_weight_dequant_f16(twm_ctx *ctx, const twm_weight *w, uint16_t *out_kn_d
  * M = 1 is gemm_tw_marlin_m1 (quantize.rs:1301); M > 1 has the semantics of gemm_q4_0
  * (quantize.rs:1825-1858).  splits = 0 lets the library choose (twm_pick_splits).
  * M <= 32: decode kernels (M <= 4 one lane per column, M = 5..32 streaming tiles), weights exact,
- *          each group's f32 sum scaled by f32(scale).
+ *          each group's f32 sum scaled by f32(scale).  f32 activations enter as two f16 terms,
+ *          f16(a) + f16(a - f16(a)), about 22 bits (|a| inside the f16 range).
  * M  > 32: prefill GEMM; weights are the reference's FP16 Q4 unpack, f16(scale * (q - 8)), as in
  * its dequant-then-matmul prefill route; f32 activations are rounded to f16 first.  Uses the
  * context's scratch: one context must not run two calls at the same time. */

@@ -48,6 +48,8 @@ struct twm_ctx {
     int prefill_bm;       // rows of A per prefill workgroup: 0 = choose, 64 or 128
     int prefill_min_m;    // M from which the LDS/MFMA prefill kernel runs instead of 16-row decode blocks
     int dequant_src;      // which copy twm_weight_dequant_f16 unpacks: 0 = 16-column tiles, 1 = column-lane
+    int m1_exact;         // twm_gemm_tw_marlin_m1: 1 = f32 activations and f32 FMAs in the reference's order
+    int m1_splits;        // twm_gemm_tw_marlin_m1: split-K factor of the MFMA kernel, 0 = heuristic
     hipDeviceProp_t prop;
 };
 
@@ -107,6 +109,8 @@ twm_ctx *twm_ctx_create(int ordinal)
     c->force_waves = 0;
     c->force_kernel = 0;
     c->dequant_src = 0;
+    c->m1_exact = 0;
+    c->m1_splits = 0;
     c->prefill_bm = 0;
     c->prefill_min_m = 33;  // M <= 32 is batched decode (exact f32 scales, weights streamed once)
     c->ws = nullptr;
@@ -207,6 +211,16 @@ int twm_ctx_set_option(twm_ctx *ctx, const char *key, int value)
     if (strcmp(key, "dequant_src") == 0) {
         if (value != 0 && value != 1) return fail(TWM_SHAPE_ERROR, "twm_ctx_set_option: dequant_src must be 0 or 1");
         ctx->dequant_src = value;
+        return TWM_OK;
+    }
+    if (strcmp(key, "m1_exact") == 0) {
+        if (value != 0 && value != 1) return fail(TWM_SHAPE_ERROR, "twm_ctx_set_option: m1_exact must be 0 or 1");
+        ctx->m1_exact = value;
+        return TWM_OK;
+    }
+    if (strcmp(key, "m1_splits") == 0) {
+        if (value < 0 || value > 64) return fail(TWM_SHAPE_ERROR, "twm_ctx_set_option: m1_splits must be 0 .. 64");
+        ctx->m1_splits = value;
         return TWM_OK;
     }
     if (strcmp(key, "kernel") == 0) {
@@ -507,10 +521,36 @@ int twm_gemm_tw_marlin_m1(twm_ctx *ctx, const float *a_dev, const uint8_t *packe
     if (k == 0) return twm_memset_zero(ctx, c_dev, (size_t)n * 4);
     if (!a_dev || !packed_dev || !scales_dev) return fail(TWM_INVALID_HANDLE, "twm_gemm_tw_marlin_m1: null input");
     if (((uintptr_t)packed_dev & 15) != 0) return fail(TWM_SHAPE_ERROR, "twm_gemm_tw_marlin_m1: packed must be 16-byte aligned");
-    uint32_t nb, sp, gps;
-    twm_pick_splits_reference(k, n, &nb, &sp, &gps);
-    HIP_TRY(launch_ref_gemv(ctx->stream, a_dev, packed_dev, scales_dev, c_dev, n, k, sp, gps), TWM_DEVICE_ERROR,
-            "gemv launch");
+    if (ctx->m1_exact || ((uintptr_t)a_dev & 15) != 0) {
+        // f32 activations, f32 FMAs, the reference kernel's order and its own split-K rule (float atomics)
+        uint32_t nb, sp, gps;
+        twm_pick_splits_reference(k, n, &nb, &sp, &gps);
+        HIP_TRY(launch_ref_gemv(ctx->stream, a_dev, packed_dev, scales_dev, c_dev, n, k, sp, gps), TWM_DEVICE_ERROR,
+                "gemv launch");
+        return TWM_OK;
+    }
+    // the M <= 4 MFMA kernel reading the reference's arrays as they are (activations rounded to f16)
+    uint32_t n_pad = ((n + 63) / 64) * 64, k_chunks = (k / 32 + kChunkGroups - 1) / kChunkGroups;
+    // On the reference's arrays a wave's four group rows of a chunk are N x 16 bytes apart, and more waves in
+    // flight pay better than on the contiguous copy: sixteen waves per tile and a split-K of up to about one
+    // workgroup per CU, unless the tiles alone fill the GPU (fitted to a sweep over the benchmark shapes).
+    DecodePlan plan;
+    plan.lane_col = 1;
+    plan.nt = 1;
+    plan.waves = 8;
+    plan.splits = 1;
+    if (n_pad / 64 < 256) {
+        plan.waves = 16;
+        while ((n_pad / 64) * plan.splits * 2 <= 256 && k_chunks >= plan.splits * 2 * 8) plan.splits *= 2;
+    }
+    if (ctx->force_waves) plan.waves = (uint32_t)ctx->force_waves;
+    if (ctx->m1_splits) plan.splits = (uint32_t)ctx->m1_splits;
+    if (plan.splits > k_chunks) plan.splits = k_chunks;
+    while (plan.splits > 1 && (size_t)plan.splits * n_pad * 4 > ctx->ws_bytes) plan.splits--;
+    if (n_pad / 64 > ctx->n_counters) plan.splits = 1;
+    HIP_TRY(launch_gemv4_ref(ctx->stream, packed_dev, scales_dev, k, n, a_dev, c_dev, ctx->ws, ctx->counters, plan.waves,
+                             plan.splits),
+            TWM_DEVICE_ERROR, "gemv launch");
     return TWM_OK;
 }
 

@@ -18,6 +18,8 @@
 // lane n.  Per 1 KiB of nibbles the wave spends 36 VALU on the unpack, 8 MFMA and 1 scale-FMA.
 #include "twm_gemv4_core.h"
 
+#include <cstring>
+
 namespace twm {
 
 __device__ __forceinline__ void gemv4_store_out(const OutSpec &out, uint32_t m, uint32_t col, float v)
@@ -33,11 +35,13 @@ __device__ __forceinline__ void gemv4_store_out(const OutSpec &out, uint32_t m, 
 
 // Workgroup = `waves` waves (blockDim.x / 64) that share NT tiles of 64 columns and split the
 // k-chunks [split*cps, (split+1)*cps) among themselves (wave w: chunks w, w + waves, ...).
-template <int NT, int RL, bool AF32>
+// REFL: cw is the reference's packed array and ref_scales its scales (no repack; M = 1, f32 activations).
+template <int NT, int RL, bool AF32, bool REFL = false>
 __global__ __launch_bounds__(1024) void k_gemv4(const char *__restrict__ cw, const void *__restrict__ a_any,
                                                  OutSpec out, float *__restrict__ ws, unsigned *__restrict__ counters, uint32_t m_rows, uint32_t k,
                                                  uint32_t n, uint32_t n_pad, uint32_t k_chunks, uint32_t tile_groups,
-                                                 uint32_t splits, uint32_t cps, float *__restrict__ swiglu_out)
+                                                 uint32_t splits, uint32_t cps, float *__restrict__ swiglu_out,
+                                                 const uint16_t *__restrict__ ref_scales = nullptr)
 {
     extern __shared__ float red[];  // [waves][NT][RL][64]
     __shared__ int s_last;
@@ -73,9 +77,12 @@ __global__ __launch_bounds__(1024) void k_gemv4(const char *__restrict__ cw, con
         for (int r = 0; r < RL; r++) acc[t][r] = 0.f;
 
     auto load_chunk = [&](Chunk4<NT> &r, uint32_t kc) {
-        gemv4_load_chunk<NT, AF32>(r, wbase, kc, lane16, lane8, a_any, arow, apiece, k);
+        if constexpr (REFL)
+            gemv4_load_chunk_ref<NT>(r, cw, ref_scales, tg * NT, kc, lane, n, k / 32u, (const float *)a_any, apiece, k);
+        else
+            gemv4_load_chunk<NT, AF32>(r, wbase, kc, lane16, lane8, a_any, arow, apiece, k);
     };
-    auto compute_chunk = [&](const Chunk4<NT> &r) { gemv4_compute_chunk<NT, RL>(r, dq, acc); };
+    auto compute_chunk = [&](const Chunk4<NT> &r) { gemv4_compute_chunk<NT, RL, AF32>(r, dq, acc); };
 
     {
         // two register sets used alternately: the loads of one are in flight while the other is consumed
@@ -208,6 +215,31 @@ static hipError_t launch_gemv4_t(hipStream_t s, const WeightView &w, const void 
         hipLaunchKernelGGL((k_gemv4<NT, RL, false>), dim3(blocks), dim3(waves * 64), lds, s, (const char *)w.cq, a, out, ws,
                            counters, m, w.k, w.n, n_pad, w.k_chunks, tile_groups,
                            splits, cps, swiglu_out);
+    return hipGetLastError();
+}
+
+// M = 1 on the reference's arrays (no repack), f32 activations; one 64-column tile per workgroup.
+hipError_t launch_gemv4_ref(hipStream_t s, const uint8_t *packed, const uint16_t *scales, uint32_t k, uint32_t n,
+                            const float *a, float *c, float *ws, unsigned *counters, uint32_t waves, uint32_t splits)
+{
+    if (n == 0) return hipSuccess;
+    if (k == 0 || k % 32 != 0 || splits == 0) return hipErrorInvalidValue;
+    if (waves != 1 && waves != 2 && waves != 4 && waves != 8 && waves != 16) return hipErrorInvalidValue;
+    uint32_t tiles64 = (n + 63) / 64, n_pad = tiles64 * 64;
+    uint32_t k_chunks = (k / 32 + 3) / 4;
+    uint32_t cps = (k_chunks + splits - 1) / splits;
+    splits = (k_chunks + cps - 1) / cps;
+    uint32_t blocks = ((tiles64 + 7) / 8) * 8 * splits;
+    size_t lds = (size_t)waves * 64 * sizeof(float);
+    OutSpec out;
+    memset(&out, 0, sizeof out);
+    out.count = 1;
+    out.seg[0].ptr = c;
+    out.seg[0].start = 0;
+    out.seg[0].width = n;
+    hipLaunchKernelGGL((k_gemv4<1, 1, true, true>), dim3(blocks), dim3(waves * 64), lds, s, (const char *)packed,
+                       (const void *)a, out, ws, counters, 1u, k, n, n_pad, k_chunks, tiles64, splits, cps,
+                       (float *)nullptr, scales);
     return hipGetLastError();
 }
 

@@ -44,7 +44,24 @@ struct Chunk4 {
     uint4v wq[NT][4];  // [tile][group in chunk]: this lane's column, 32 nibbles
     uint2v sc[NT];     // four f16 scales
     uint4v a;          // activations: row lane%4, k-piece lane/4 (8 halves)
+    uint4v a_lo;       // f32 activations only: the f16 residuals a - f16(a) of the same eight values
 };
+
+// f32 activations enter the f16 MFMA as two terms, a = f16(a) + f16(a - f16(a)) (about 22 significant bits;
+// the subtraction is exact), so that a caller's f32 values are not silently cut to 11 bits.  Values beyond the
+// f16 range (|a| > 65504) are not supported by this path.
+__device__ __forceinline__ void split_f32x8(const float (&v)[8], uint4v &hi, uint4v &lo)
+{
+    union { half8 h; uint4v u; } ch, cl;
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+        _Float16 h = (_Float16)v[i];
+        ch.h[i] = h;
+        cl.h[i] = (_Float16)(v[i] - (float)h);
+    }
+    hi = ch.u;
+    lo = cl.u;
+}
 
 template <int P>
 __device__ __forceinline__ float4v mfma_piece(half4v a, half4v b, float4v c)
@@ -71,21 +88,55 @@ __device__ __forceinline__ void gemv4_load_chunk(Chunk4<NT> &r, const char *(&wb
     if (AF32) {
         const float4 *p = (const float4 *)((const float *)a_any + (size_t)arow * k + k0);
         float4 x = p[0], y = p[1];
-        union { half8 h; uint4v u; } cv;
-        cv.h = half8{(_Float16)x.x, (_Float16)x.y, (_Float16)x.z, (_Float16)x.w,
-                     (_Float16)y.x, (_Float16)y.y, (_Float16)y.z, (_Float16)y.w};
-        r.a = cv.u;
+        const float v[8] = {x.x, x.y, x.z, x.w, y.x, y.y, y.z, y.w};
+        split_f32x8(v, r.a, r.a_lo);
     } else {
         r.a = *(const uint4v *)((const _Float16 *)a_any + (size_t)arow * k + k0);
     }
 }
 
-// acc[t][row] += f32(scale) * (sum over the group of A * (q - 8)) for the four groups of the chunk
-template <int NT, int RL>
+// The same chunk taken from the reference's own arrays, without a repack (packed u8 [G][N][16], scales f16
+// [G][N], crates/kernels/src/quantize.rs:892-907): lane = column, so a wave still reads 1 KiB contiguous per
+// group.  Columns past n and groups past the end replay the last valid one with scale 0 (weight exactly 0).
+// The nibbles are in their natural order here, which the mask-and-magic unpack turns into the k order
+// (0,4,1,5 | 2,6,3,7) per eight; the f32 activations (one row) are converted into that same order.
+template <int NT>
+__device__ __forceinline__ void gemv4_load_chunk_ref(Chunk4<NT> &r, const char *packed, const uint16_t *scales,
+                                                     uint32_t tile0, uint32_t kc, uint32_t lane, uint32_t n,
+                                                     uint32_t groups, const float *a, uint32_t apiece, uint32_t k)
+{
+#pragma unroll
+    for (int t = 0; t < NT; t++) {
+        const uint32_t col = (tile0 + t) * 64u + lane;
+        const uint32_t colc = col < n ? col : n - 1u;
+        uint32_t sb[4];
+#pragma unroll
+        for (int g = 0; g < 4; g++) {
+            const uint32_t gg = kc * 4u + g;
+            const uint32_t ggc = gg < groups ? gg : groups - 1u;
+            const size_t idx = (size_t)ggc * n + colc;
+            r.wq[t][g] = *(const uint4v *)(packed + idx * 16u);
+            const uint32_t sbits = scales[idx];
+            sb[g] = (gg < groups && col < n) ? sbits : 0u;
+        }
+        r.sc[t] = uint2v{sb[0] | (sb[1] << 16), sb[2] | (sb[3] << 16)};
+    }
+    uint32_t k0 = kc * 128u + apiece;
+    if (k0 > k - 8u) k0 = k - 8u;
+    const float4 *p = (const float4 *)(a + k0);
+    float4 x = p[0], y = p[1];
+    const float v[8] = {x.x, y.x, x.y, y.y, x.z, y.z, x.w, y.w};
+    split_f32x8(v, r.a, r.a_lo);
+}
+
+// acc[t][row] += f32(scale) * (sum over the group of A * (q - 8)) for the four groups of the chunk;
+// A2: the activations came as f32 and have a second (residual) term
+template <int NT, int RL, bool A2 = false>
 __device__ __forceinline__ void gemv4_compute_chunk(const Chunk4<NT> &r, const Gemv4Consts &dq, float (&acc)[NT][RL])
 {
-    union { uint4v u; half4v h[2]; } av;
+    union { uint4v u; half4v h[2]; } av, al;
     av.u = r.a;  // h[0] = k 0..3 of the lane's piece, h[1] = k 4..7
+    if (A2) al.u = r.a_lo;
 #pragma unroll
     for (int t = 0; t < NT; t++) {
         union { uint2v u; _Float16 h[4]; } sv;
@@ -97,7 +148,11 @@ __device__ __forceinline__ void gemv4_compute_chunk(const Chunk4<NT> &r, const G
 #define TWM_PIECE(W, PIECE)                                       \
     gemv4_dequant_word(r.wq[t][g][W], dq, lo4, hi4);              \
     d = mfma_piece<PIECE>(av.h[0], lo4, d);                       \
-    d = mfma_piece<PIECE>(av.h[1], hi4, d);
+    d = mfma_piece<PIECE>(av.h[1], hi4, d);                       \
+    if (A2) {                                                     \
+        d = mfma_piece<PIECE>(al.h[0], lo4, d);                   \
+        d = mfma_piece<PIECE>(al.h[1], hi4, d);                   \
+    }
             if (g == 0) { TWM_PIECE(0, 0) TWM_PIECE(1, 1) TWM_PIECE(2, 2) TWM_PIECE(3, 3) }
             if (g == 1) { TWM_PIECE(0, 4) TWM_PIECE(1, 5) TWM_PIECE(2, 6) TWM_PIECE(3, 7) }
             if (g == 2) { TWM_PIECE(0, 8) TWM_PIECE(1, 9) TWM_PIECE(2, 10) TWM_PIECE(3, 11) }

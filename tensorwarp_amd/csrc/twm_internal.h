@@ -97,6 +97,8 @@ hipError_t launch_weight_dequant_f16_col(hipStream_t s, const WeightView &w, uin
 hipError_t launch_gemv4(hipStream_t s, const WeightView &w, const void *a, bool a_f32, uint32_t m, const OutSpec &out,
                         float *ws, unsigned *counters, uint32_t nt, uint32_t waves, uint32_t splits,
                         float *swiglu_out = nullptr);
+hipError_t launch_gemv4_ref(hipStream_t s, const uint8_t *packed, const uint16_t *scales, uint32_t k, uint32_t n,
+                            const float *a, float *c, float *ws, unsigned *counters, uint32_t waves, uint32_t splits);
 hipError_t init_prefill();
 hipError_t launch_prefill(hipStream_t s, const WeightView &w, const void *a, bool a_f32, uint32_t m, const OutSpec &out,
                           uint32_t block_rows, uint32_t splits, void *scratch, size_t scratch_bytes);

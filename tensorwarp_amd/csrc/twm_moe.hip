@@ -52,15 +52,15 @@ __device__ __forceinline__ void bank_accumulate(const char *tile_base, const voi
     if (c2 < k_chunks) gemv4_load_chunk<1, AF32>(r2, wbase, c2, lane16, lane8, a_row, 0, apiece, k);
     for (;;) {
         if (c0 >= k_chunks) break;
-        gemv4_compute_chunk<1, 1>(r0, dq, acc);
+        gemv4_compute_chunk<1, 1, AF32>(r0, dq, acc);
         c0 += 3u * stride;
         if (c0 < k_chunks) gemv4_load_chunk<1, AF32>(r0, wbase, c0, lane16, lane8, a_row, 0, apiece, k);
         if (c1 >= k_chunks) break;
-        gemv4_compute_chunk<1, 1>(r1, dq, acc);
+        gemv4_compute_chunk<1, 1, AF32>(r1, dq, acc);
         c1 += 3u * stride;
         if (c1 < k_chunks) gemv4_load_chunk<1, AF32>(r1, wbase, c1, lane16, lane8, a_row, 0, apiece, k);
         if (c2 >= k_chunks) break;
-        gemv4_compute_chunk<1, 1>(r2, dq, acc);
+        gemv4_compute_chunk<1, 1, AF32>(r2, dq, acc);
         c2 += 3u * stride;
         if (c2 < k_chunks) gemv4_load_chunk<1, AF32>(r2, wbase, c2, lane16, lane8, a_row, 0, apiece, k);
     }

@@ -9,6 +9,7 @@
 // take the chunks of that range in turn (wave w: chunks w, w + 4, ...), each with its own registers:
 //   B : 4 x 16 B nibbles + 4 x 8 B scales per lane and chunk (one tile each), straight from HBM;
 //   A : MT x 4 x 16 B per lane and chunk (row = lane % 16 of row block mt, eight k per group), from L2;
+//       f32 activations are split once per launch into two f16 arrays (hi, lo) and both terms are multiplied;
 // one chunk ahead in a second register set (the loop is unrolled by two, loads are unconditional with
 // clamped chunk indices so that the compiler can count them).  At the end the four waves add their sums
 // through LDS and the workgroup stores 16 MT x 64 outputs, or parks them as split-K partials for
@@ -50,12 +51,14 @@ __device__ __forceinline__ half8 st_unpack(uint32_t w, const StConsts &c)
     return r.h;
 }
 
-template <bool AF32>
-struct AFrag;  // one lane's eight activations of one group, as loaded
+// One lane's eight activations of one group.  TWO: the activations came as f32 and were split beforehand into
+// two f16 arrays, hi = f16(a) and lo = f16(a - hi) (about 22 bits together); both terms go through the MFMA.
+template <bool TWO>
+struct AFrag;
 template <>
 struct AFrag<false> {
     uint4v v;
-    __device__ __forceinline__ void load(const TWM_GLOBAL char *p) { v = *(const TWM_GLOBAL uint4v *)p; }
+    __device__ __forceinline__ void load(const TWM_GLOBAL char *p, uint32_t) { v = *(const TWM_GLOBAL uint4v *)p; }
     __device__ __forceinline__ half8 get() const
     {
         union { uint4v u; half8 h; } cv;
@@ -65,16 +68,23 @@ struct AFrag<false> {
 };
 template <>
 struct AFrag<true> {
-    float4v x, y;
-    __device__ __forceinline__ void load(const TWM_GLOBAL char *p)
+    uint4v v, w;
+    __device__ __forceinline__ void load(const TWM_GLOBAL char *p, uint32_t lo_offset)
     {
-        x = *(const TWM_GLOBAL float4v *)p;
-        y = *(const TWM_GLOBAL float4v *)(p + 16);
+        v = *(const TWM_GLOBAL uint4v *)p;
+        w = *(const TWM_GLOBAL uint4v *)(p + lo_offset);
     }
     __device__ __forceinline__ half8 get() const
     {
-        return half8{(_Float16)x[0], (_Float16)x[1], (_Float16)x[2], (_Float16)x[3],
-                     (_Float16)y[0], (_Float16)y[1], (_Float16)y[2], (_Float16)y[3]};
+        union { uint4v u; half8 h; } cv;
+        cv.u = v;
+        return cv.h;
+    }
+    __device__ __forceinline__ half8 get_lo() const
+    {
+        union { uint4v u; half8 h; } cv;
+        cv.u = w;
+        return cv.h;
     }
 };
 
@@ -91,9 +101,9 @@ template <int MT, bool AF32, int WAVES>
 __global__ __launch_bounds__(WAVES * 64) void k_stream(const uint4v *__restrict__ qw, const uint2v *__restrict__ sc,
                                                  const void *__restrict__ a_any, OutSpec out, float *__restrict__ partials,
                                                  uint32_t m_rows, uint32_t k, uint32_t n, uint32_t n_tiles,
-                                                 uint32_t k_chunks, uint32_t chunks_per_split)
+                                                 uint32_t k_chunks, uint32_t chunks_per_split, uint32_t lo_offset)
 {
-    constexpr uint32_t kABytes = AF32 ? 4u : 2u;
+    constexpr uint32_t kABytes = 2u;  // f16 rows; with AF32 a_any holds the hi rows and, lo_offset bytes on, the lo rows
     __shared__ float red[WAVES][16 * MT][64];
 
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -137,15 +147,18 @@ __global__ __launch_bounds__(WAVES * 64) void k_stream(const uint4v *__restrict_
             kk = kk < k ? kk : 0u;
             const TWM_GLOBAL char *base = st_scalar_base(a_any, (size_t)kk * kABytes);
 #pragma unroll
-            for (int mt = 0; mt < MT; mt++) r.a[mt][g].load(base + a_off[mt]);
+            for (int mt = 0; mt < MT; mt++) r.a[mt][g].load(base + a_off[mt], lo_offset);
         }
     };
     auto compute = [&](const ChunkRegs<MT, AF32> &r) {
 #pragma unroll
         for (int g = 0; g < 4; g++) {
-            half8 af[MT];
+            half8 af[MT], al[MT];
 #pragma unroll
-            for (int mt = 0; mt < MT; mt++) af[mt] = r.a[mt][g].get();
+            for (int mt = 0; mt < MT; mt++) {
+                af[mt] = r.a[mt][g].get();
+                if constexpr (AF32) al[mt] = r.a[mt][g].get_lo();
+            }
 #pragma unroll
             for (int t = 0; t < 4; t++) {
                 half8 bf = st_unpack(r.bq[t][g], dq);
@@ -156,6 +169,7 @@ __global__ __launch_bounds__(WAVES * 64) void k_stream(const uint4v *__restrict_
 #pragma unroll
                 for (int mt = 0; mt < MT; mt++) {
                     float4v d = __builtin_amdgcn_mfma_f32_16x16x32_f16(af[mt], bf, float4v{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+                    if constexpr (AF32) d = __builtin_amdgcn_mfma_f32_16x16x32_f16(al[mt], bf, d, 0, 0, 0);
 #pragma unroll
                     for (int i = 0; i < 4; i++) acc[mt][t][i] += d[i] * scale;
                 }
@@ -216,15 +230,27 @@ __global__ __launch_bounds__(WAVES * 64) void k_stream(const uint4v *__restrict_
     }
 }
 
+// f32 activations -> two f16 arrays: hi = f16(a), lo = f16(a - hi) (the subtraction is exact)
+__global__ __launch_bounds__(256) void k_split_f32_hi_lo(const float *__restrict__ a, _Float16 *__restrict__ hi,
+                                                          _Float16 *__restrict__ lo, size_t count)
+{
+    size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= count) return;
+    float v = a[i];
+    _Float16 h = (_Float16)v;
+    hi[i] = h;
+    lo[i] = (_Float16)(v - (float)h);
+}
+
 template <int MT, bool AF32, int WAVES>
 static hipError_t launch_stream_t(hipStream_t s, const WeightView &w, const void *a, uint32_t m, const OutSpec &out,
-                                  uint32_t splits, float *partials)
+                                  uint32_t splits, float *partials, uint32_t lo_offset)
 {
     uint32_t cps = (w.k_chunks + splits - 1) / splits;
     splits = (w.k_chunks + cps - 1) / cps;  // no empty split
     dim3 grid(w.n_tiles / 4, splits);
     hipLaunchKernelGGL((k_stream<MT, AF32, WAVES>), grid, dim3(WAVES * 64), 0, s, (const uint4v *)w.qw, (const uint2v *)w.sc, a, out,
-                       splits > 1 ? partials : nullptr, m, w.k, w.n, w.n_tiles, w.k_chunks, cps);
+                       splits > 1 ? partials : nullptr, m, w.k, w.n, w.n_tiles, w.k_chunks, cps, lo_offset);
     if (splits > 1) {
         hipError_t e = launch_splitk_reduce(s, partials, out, m, w.n, w.n_tiles * 16, splits);
         if (e != hipSuccess) return e;
@@ -232,19 +258,34 @@ static hipError_t launch_stream_t(hipStream_t s, const WeightView &w, const void
     return hipGetLastError();
 }
 
-// M <= 32.  splits > 1 needs `partials` with room for splits x M x (n_tiles * 16) floats.
+// M <= 32.  `scratch` holds, for f32 activations, their two f16 terms (2 x M x K halves) and after them the
+// split-K partials (splits x M x (n_tiles * 16) floats); the split factor is cut to what fits.
 hipError_t launch_stream(hipStream_t s, const WeightView &w, const void *a, bool a_f32, uint32_t m, const OutSpec &out,
-                         uint32_t splits, uint32_t waves, float *partials, size_t partial_bytes)
+                         uint32_t splits, uint32_t waves, float *scratch, size_t scratch_bytes)
 {
     if (m == 0 || w.n == 0) return hipSuccess;
     if (m > 32 || w.k_chunks == 0) return hipErrorInvalidValue;
+    if (waves != 4 && waves != 8) return hipErrorInvalidValue;
+    float *partials = scratch;
+    size_t partial_bytes = scratch ? scratch_bytes : 0;
+    uint32_t lo_offset = 0;
+    if (a_f32) {
+        size_t term_bytes = (((size_t)m * w.k * 2) + 255) & ~(size_t)255;
+        if (!scratch || scratch_bytes < 2 * term_bytes || term_bytes > 0x7FFFFFFFu) return hipErrorInvalidValue;
+        _Float16 *hi = (_Float16 *)scratch, *lo = (_Float16 *)((char *)scratch + term_bytes);
+        size_t count = (size_t)m * w.k;
+        hipLaunchKernelGGL(k_split_f32_hi_lo, dim3((unsigned)((count + 255) / 256)), dim3(256), 0, s, (const float *)a, hi, lo, count);
+        a = hi;
+        lo_offset = (uint32_t)term_bytes;
+        partials = (float *)((char *)scratch + 2 * term_bytes);
+        partial_bytes = scratch_bytes - 2 * term_bytes;
+    }
     if (splits < 1) splits = 1;
     size_t per_split = (size_t)m * w.n_tiles * 16 * 4;
     if (!partials || per_split == 0) splits = 1;
     else if (splits > partial_bytes / per_split) splits = (uint32_t)(partial_bytes / per_split);
     if (splits < 1) splits = 1;
-    if (waves != 4 && waves != 8) return hipErrorInvalidValue;
-#define TWM_STREAM_CASE(MT, F32, W) return launch_stream_t<MT, F32, W>(s, w, a, m, out, splits, partials)
+#define TWM_STREAM_CASE(MT, F32, W) return launch_stream_t<MT, F32, W>(s, w, a, m, out, splits, partials, lo_offset)
     if (m <= 16) {
         if (waves == 8) { if (a_f32) TWM_STREAM_CASE(1, true, 8); TWM_STREAM_CASE(1, false, 8); }
         if (a_f32) TWM_STREAM_CASE(1, true, 4);

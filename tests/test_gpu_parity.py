@@ -326,14 +326,32 @@ def test_gemm_tw_marlin_m1_reference_layout(dev, k, n):
     packed, scales, a16 = synth(k, n, 1, k + n)
     a = f16_as_f32(a16)
     c = T.GpuTensor.zeros(dev, (n,), "f32")
-    T.gemm_tw_marlin_m1(dev, T.GpuTensor.from_host(dev, a), T.GpuTensor.from_host(dev, packed),
-                        T.GpuTensor.from_host(dev, scales, "f16"), c, n, k)
-    got = c.to_host()
+    pd, sd = T.GpuTensor.from_host(dev, packed), T.GpuTensor.from_host(dev, scales, "f16")
     truth = O.gemm_f64(a, packed, scales, 1, k, n)[0]
-    assert rel_err(got, truth) < TIGHT
-    _, splits, _ = T.pick_splits_reference(k, n)
-    if splits == 1:                                      # same order as the reference kernel: bitwise
-        assert np.array_equal(got, O.gemv_ref_order(a, packed, scales, 1, k, n, 1)[0])
+    # default: the MFMA kernel on the reference's arrays as they are
+    T.gemm_tw_marlin_m1(dev, T.GpuTensor.from_host(dev, a), pd, sd, c, n, k)
+    assert rel_err(c.to_host(), truth) < TIGHT
+    # activations that are not f16 numbers
+    a_raw = (O.synth_normal_f32(k, k + n + 1) * np.float32(1.37)).astype(np.float32)
+    T.gemm_tw_marlin_m1(dev, T.GpuTensor.from_host(dev, a_raw), pd, sd, c, n, k)
+    t_raw = O.gemm_f64(a_raw.reshape(1, k), packed, scales, 1, k, n)[0]
+    # two f16 terms per activation, about 22 bits (one term, plain rounding to f16, is off by up to 9e-2 on the
+    # near-cancelling outputs of the larger shapes)
+    assert rel_err(c.to_host(), t_raw) < TIGHT
+    # "m1_exact": f32 activations, f32 FMAs in the reference kernel's order and its split-K rule
+    try:
+        dev.set_option("m1_exact", 1)
+        c.copy_from_host(np.full(n, np.nan, np.float32))
+        T.gemm_tw_marlin_m1(dev, T.GpuTensor.from_host(dev, a), pd, sd, c, n, k)
+        got = c.to_host()
+        assert rel_err(got, truth) < TIGHT
+        _, splits, _ = T.pick_splits_reference(k, n)
+        if splits == 1:                                      # same order as the reference kernel: bitwise
+            assert np.array_equal(got, O.gemv_ref_order(a, packed, scales, 1, k, n, 1)[0])
+        T.gemm_tw_marlin_m1(dev, T.GpuTensor.from_host(dev, a_raw), pd, sd, c, n, k)
+        assert rel_err(c.to_host(), t_raw) < TIGHT
+    finally:
+        dev.set_option("m1_exact", 0)
 
 
 def test_gemm_tw_marlin_m1_from_buffer_and_errors(dev):
@@ -345,6 +363,13 @@ def test_gemm_tw_marlin_m1_from_buffer_and_errors(dev):
     c = T.GpuTensor.zeros(dev, (n,), "f32")
     T.gemm_tw_marlin_m1_from_buffer(dev, T.GpuTensor.from_host(dev, a), T.GpuTensor.from_host(dev, slab_p), 4096,
                                     T.GpuTensor.from_host(dev, slab_s, "f16"), 100, c, n, k)
+    assert rel_err(c.to_host(), O.gemm_f64(a, packed, scales, 1, k, n)[0]) < TIGHT
+    try:
+        dev.set_option("m1_exact", 1)
+        T.gemm_tw_marlin_m1_from_buffer(dev, T.GpuTensor.from_host(dev, a), T.GpuTensor.from_host(dev, slab_p), 4096,
+                                        T.GpuTensor.from_host(dev, slab_s, "f16"), 100, c, n, k)
+    finally:
+        dev.set_option("m1_exact", 0)
     assert np.array_equal(c.to_host(), O.gemv_ref_order(a, packed, scales, 1, k, n, 1)[0])
     with pytest.raises(T.DeviceError) as e:              # the reference asserts k % 32 == 0 (quantize.rs:1311)
         T.gemm_tw_marlin_m1(dev, c, c, c, c, n, 100)
@@ -511,6 +536,25 @@ def test_decode_kernels_rows_and_f32_activations(dev, m):
     finally:
         dev.set_option("kernel", 0)
         dev.set_option("prefill_min_m", 33)
+    w.free()
+
+
+@pytest.mark.parametrize("m", [1, 3, 4, 5, 16, 32])
+def test_f32_activations_keep_their_precision(dev, m):
+    # The reference's decode activations are f32 (generate.rs:2153).  Cutting them to f16 would move
+    # near-cancelling outputs of a 3584-deep sum by several percent of their value; the decode kernels take
+    # every f32 activation as two f16 terms instead, so the f64 truth on the raw values holds to the same bar.
+    k, n = 3584, 1152
+    packed, scales, _ = synth(k, n, 1, 4000 + m)
+    a_raw = (O.synth_normal_f32(m * k, 4100 + m) * np.float32(1.37)).reshape(m, k)
+    w = T.MarlinWeight.upload(dev, packed, scales, k, n)
+    truth = O.gemm_f64(a_raw, packed, scales, m, k, n)
+    for splits in (0, 1, 3):
+        c = T.GpuTensor.from_host(dev, np.full((m, n), np.nan, np.float32))
+        T.gemm(dev, w, T.GpuTensor.from_host(dev, a_raw), m, c, splits)
+        assert rel_err(c.to_host(), truth) < TIGHT, splits
+    rounded = O.gemm_f64(a_raw.astype(np.float16).astype(np.float32), packed, scales, m, k, n)
+    assert rel_err(rounded, truth) > TOL       # what a single f16 term would give: outside the stated tolerance
     w.free()
 
 
