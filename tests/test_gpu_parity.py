@@ -410,6 +410,36 @@ def test_gemm_matches_golden(dev, name):
     w.free()
 
 
+@pytest.mark.parametrize("m", [1, 4, 64])
+def test_reference_gemm_q4_0_correctness_case(dev, m):
+    # The reference's own test of the quantized GEMM (gemm_q4_0_correctness, quantize.rs:3043-3106): its
+    # generators for A and B, B quantized on the GPU, result against the full-precision product with
+    # NRMSE < 0.15 (the quantization error of group-32 Q4) -- here also against the oracle on the quantized
+    # weights at the library's own bar.  M = 64 is the reference's shape; 1 and 4 run the decode kernels.
+    n, k = 64, 128
+    a = (((np.arange(m * k) * 7 + 13) % 100).astype(np.float32) * np.float32(0.01) - np.float32(0.5)).reshape(m, k)
+    b = (((np.arange(k * n) * 11 + 3) % 100).astype(np.float32) * np.float32(0.01) - np.float32(0.5)).reshape(k, n)
+    packed, scales = T.quantize_f32_to_tw_marlin(dev, T.GpuTensor.from_host(dev, b), k, n)
+    ph, sh = packed.to_host(), scales.to_host()
+    w = T.MarlinWeight.from_device(dev, packed, scales, k, n)
+    c = T.GpuTensor.from_host(dev, np.full((m, n), np.nan, np.float32))
+    T.gemm(dev, w, T.GpuTensor.from_host(dev, a), m, c)
+    got = c.to_host().reshape(m, n).astype(np.float64)
+    full = a.astype(np.float64) @ b.astype(np.float64)
+    nrmse = np.sqrt(((got - full) ** 2).sum() / max((full ** 2).sum(), 1e-10))
+    assert nrmse < 0.15
+    if m <= 32:
+        assert rel_err(got, O.gemm_f64(a, ph, sh, m, k, n)) < TIGHT
+    else:   # prefill GEMM: f16 activations and the FP16 Q4 unpack
+        w16 = O.dequant_f16(ph, sh, k, n).view(np.float16).astype(np.float64).reshape(k, n)
+        assert rel_err(got, a.astype(np.float16).astype(np.float64) @ w16) < TIGHT
+    if m == 1:
+        c1 = T.GpuTensor.zeros(dev, (n,), "f32")
+        T.gemm_tw_marlin_m1(dev, T.GpuTensor.from_host(dev, a), packed, scales, c1, n, k)
+        assert rel_err(c1.to_host(), O.gemm_f64(a, ph, sh, 1, k, n)[0]) < TIGHT
+    w.free()
+
+
 def test_gemv_closed_forms(dev):
     k, n = 256, 96
     scales = O.synth_scales(k, n, 77)
