@@ -65,9 +65,12 @@ __global__ __launch_bounds__(1024) void k_gemv4(const char *__restrict__ cw, con
 
     const Gemv4Consts dq = make_gemv4_consts();
 
-    // activations: lane l reads row min(l % 4, M-1), halves [kc*128 + 8*(l/4), +8)
-    uint32_t arow = lane & 3u;
+    // activations: lane l reads row min(l % 4, M-1), halves [kc*128 + 8*(l/4), +8); with row-packed f32 terms
+    // row min((l % 4) / 2, M-1), odd lanes holding the residual term
+    constexpr int TERMS = REFL ? kTermsRowPacked : gemv4_terms<AF32, RL>();
+    uint32_t arow = TERMS == kTermsRowPacked ? (lane & 3u) >> 1 : lane & 3u;
     if (arow > m_rows - 1) arow = m_rows - 1;
+    const bool lane_is_lo = TERMS == kTermsRowPacked && (lane & 1u) != 0;
     const uint32_t apiece = (lane >> 2) * 8u;
 
     float acc[NT][RL];
@@ -78,11 +81,12 @@ __global__ __launch_bounds__(1024) void k_gemv4(const char *__restrict__ cw, con
 
     auto load_chunk = [&](Chunk4<NT> &r, uint32_t kc) {
         if constexpr (REFL)
-            gemv4_load_chunk_ref<NT>(r, cw, ref_scales, tg * NT, kc, lane, n, k / 32u, (const float *)a_any, apiece, k);
+            gemv4_load_chunk_ref<NT>(r, cw, ref_scales, tg * NT, kc, lane, n, k / 32u, (const float *)a_any, apiece, k,
+                                     lane_is_lo);
         else
-            gemv4_load_chunk<NT, AF32>(r, wbase, kc, lane16, lane8, a_any, arow, apiece, k);
+            gemv4_load_chunk<NT, AF32, TERMS>(r, wbase, kc, lane16, lane8, a_any, arow, apiece, k, lane_is_lo);
     };
-    auto compute_chunk = [&](const Chunk4<NT> &r) { gemv4_compute_chunk<NT, RL, AF32>(r, dq, acc); };
+    auto compute_chunk = [&](const Chunk4<NT> &r) { gemv4_compute_chunk<NT, RL, TERMS>(r, dq, acc); };
 
     {
         // two register sets used alternately: the loads of one are in flight while the other is consumed

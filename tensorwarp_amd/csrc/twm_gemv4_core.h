@@ -71,10 +71,19 @@ __device__ __forceinline__ float4v mfma_piece(half4v a, half4v b, float4v c)
 
 // Loads chunk kc of NT tiles (wbase[t] = this tile's block 0) and the lane's 16 bytes of activations:
 // lane l reads row arow, halves [kc*128 + apiece, +8).
-template <int NT, bool AF32>
+// Term modes of the activations: one f16 term; two terms as two MFMA passes (a_lo holds the second); or, for
+// at most two rows, two terms packed into the four MFMA rows (lane l: row (l % 4) / 2, term l % 2), which
+// costs no extra MFMA: the 4x4x4 instruction computes four rows anyway.
+enum { kTermsOne = 0, kTermsTwoPasses = 1, kTermsRowPacked = 2 };
+template <bool AF32, int RL>
+constexpr int gemv4_terms() { return AF32 ? (RL <= 2 ? kTermsRowPacked : kTermsTwoPasses) : kTermsOne; }
+
+// arow: the activation row this lane reads (see the term modes); lane_is_lo: row-packed mode, this lane holds
+// the residual term
+template <int NT, bool AF32, int TERMS = AF32 ? kTermsTwoPasses : kTermsOne>
 __device__ __forceinline__ void gemv4_load_chunk(Chunk4<NT> &r, const char *(&wbase)[NT], uint32_t kc,
                                                  uint32_t lane16, uint32_t lane8, const void *a_any, uint32_t arow,
-                                                 uint32_t apiece, uint32_t k)
+                                                 uint32_t apiece, uint32_t k, bool lane_is_lo = false)
 {
 #pragma unroll
     for (int t = 0; t < NT; t++) {
@@ -90,6 +99,10 @@ __device__ __forceinline__ void gemv4_load_chunk(Chunk4<NT> &r, const char *(&wb
         float4 x = p[0], y = p[1];
         const float v[8] = {x.x, x.y, x.z, x.w, y.x, y.y, y.z, y.w};
         split_f32x8(v, r.a, r.a_lo);
+        if (TERMS == kTermsRowPacked) {
+#pragma unroll
+            for (int i = 0; i < 4; i++) r.a[i] = lane_is_lo ? r.a_lo[i] : r.a[i];
+        }
     } else {
         r.a = *(const uint4v *)((const _Float16 *)a_any + (size_t)arow * k + k0);
     }
@@ -103,7 +116,8 @@ __device__ __forceinline__ void gemv4_load_chunk(Chunk4<NT> &r, const char *(&wb
 template <int NT>
 __device__ __forceinline__ void gemv4_load_chunk_ref(Chunk4<NT> &r, const char *packed, const uint16_t *scales,
                                                      uint32_t tile0, uint32_t kc, uint32_t lane, uint32_t n,
-                                                     uint32_t groups, const float *a, uint32_t apiece, uint32_t k)
+                                                     uint32_t groups, const float *a, uint32_t apiece, uint32_t k,
+                                                     bool lane_is_lo)
 {
 #pragma unroll
     for (int t = 0; t < NT; t++) {
@@ -127,13 +141,16 @@ __device__ __forceinline__ void gemv4_load_chunk_ref(Chunk4<NT> &r, const char *
     float4 x = p[0], y = p[1];
     const float v[8] = {x.x, y.x, x.y, y.y, x.z, y.z, x.w, y.w};
     split_f32x8(v, r.a, r.a_lo);
+#pragma unroll
+    for (int i = 0; i < 4; i++) r.a[i] = lane_is_lo ? r.a_lo[i] : r.a[i];  // one row: row-packed terms
 }
 
-// acc[t][row] += f32(scale) * (sum over the group of A * (q - 8)) for the four groups of the chunk;
-// A2: the activations came as f32 and have a second (residual) term
-template <int NT, int RL, bool A2 = false>
+// acc[t][row] += f32(scale) * (sum over the group of A * (q - 8)) for the four groups of the chunk
+template <int NT, int RL, int TERMS = kTermsOne>
 __device__ __forceinline__ void gemv4_compute_chunk(const Chunk4<NT> &r, const Gemv4Consts &dq, float (&acc)[NT][RL])
 {
+    constexpr bool A2 = TERMS == kTermsTwoPasses;
+    static_assert(TERMS != kTermsRowPacked || RL <= 2, "row-packed terms hold at most two rows");
     union { uint4v u; half4v h[2]; } av, al;
     av.u = r.a;  // h[0] = k 0..3 of the lane's piece, h[1] = k 4..7
     if (A2) al.u = r.a_lo;
@@ -160,7 +177,10 @@ __device__ __forceinline__ void gemv4_compute_chunk(const Chunk4<NT> &r, const G
 #undef TWM_PIECE
             float s = (float)sv.h[g];
 #pragma unroll
-            for (int rr = 0; rr < RL; rr++) acc[t][rr] = fmaf(d[rr], s, acc[t][rr]);
+            for (int rr = 0; rr < RL; rr++) {
+                if (TERMS == kTermsRowPacked) acc[t][rr] = fmaf(d[2 * rr] + d[2 * rr + 1], s, acc[t][rr]);
+                else acc[t][rr] = fmaf(d[rr], s, acc[t][rr]);
+            }
         }
     }
 }

@@ -45,24 +45,26 @@ __device__ __forceinline__ void bank_accumulate(const char *tile_base, const voi
     const char *wbase[1] = {tile_base};
     const uint32_t lane16 = lane * 16u, lane8 = 4096u + lane * 8u, apiece = (lane >> 2) * 8u;
     const Gemv4Consts dq = make_gemv4_consts();
+    constexpr int TERMS = gemv4_terms<AF32, 1>();   // one row: f32 activations as two row-packed terms
+    const bool is_lo = (lane & 1u) != 0;
     Chunk4<1> r0, r1, r2;
     uint32_t c0 = first, c1 = first + stride, c2 = first + 2u * stride;
-    if (c0 < k_chunks) gemv4_load_chunk<1, AF32>(r0, wbase, c0, lane16, lane8, a_row, 0, apiece, k);
-    if (c1 < k_chunks) gemv4_load_chunk<1, AF32>(r1, wbase, c1, lane16, lane8, a_row, 0, apiece, k);
-    if (c2 < k_chunks) gemv4_load_chunk<1, AF32>(r2, wbase, c2, lane16, lane8, a_row, 0, apiece, k);
+    if (c0 < k_chunks) gemv4_load_chunk<1, AF32, TERMS>(r0, wbase, c0, lane16, lane8, a_row, 0, apiece, k, is_lo);
+    if (c1 < k_chunks) gemv4_load_chunk<1, AF32, TERMS>(r1, wbase, c1, lane16, lane8, a_row, 0, apiece, k, is_lo);
+    if (c2 < k_chunks) gemv4_load_chunk<1, AF32, TERMS>(r2, wbase, c2, lane16, lane8, a_row, 0, apiece, k, is_lo);
     for (;;) {
         if (c0 >= k_chunks) break;
-        gemv4_compute_chunk<1, 1, AF32>(r0, dq, acc);
+        gemv4_compute_chunk<1, 1, TERMS>(r0, dq, acc);
         c0 += 3u * stride;
-        if (c0 < k_chunks) gemv4_load_chunk<1, AF32>(r0, wbase, c0, lane16, lane8, a_row, 0, apiece, k);
+        if (c0 < k_chunks) gemv4_load_chunk<1, AF32, TERMS>(r0, wbase, c0, lane16, lane8, a_row, 0, apiece, k, is_lo);
         if (c1 >= k_chunks) break;
-        gemv4_compute_chunk<1, 1, AF32>(r1, dq, acc);
+        gemv4_compute_chunk<1, 1, TERMS>(r1, dq, acc);
         c1 += 3u * stride;
-        if (c1 < k_chunks) gemv4_load_chunk<1, AF32>(r1, wbase, c1, lane16, lane8, a_row, 0, apiece, k);
+        if (c1 < k_chunks) gemv4_load_chunk<1, AF32, TERMS>(r1, wbase, c1, lane16, lane8, a_row, 0, apiece, k, is_lo);
         if (c2 >= k_chunks) break;
-        gemv4_compute_chunk<1, 1, AF32>(r2, dq, acc);
+        gemv4_compute_chunk<1, 1, TERMS>(r2, dq, acc);
         c2 += 3u * stride;
-        if (c2 < k_chunks) gemv4_load_chunk<1, AF32>(r2, wbase, c2, lane16, lane8, a_row, 0, apiece, k);
+        if (c2 < k_chunks) gemv4_load_chunk<1, AF32, TERMS>(r2, wbase, c2, lane16, lane8, a_row, 0, apiece, k, is_lo);
     }
 }
 
