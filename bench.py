@@ -135,6 +135,10 @@ def main():
 
     dev = T.WarpDevice(0)
     rng = np.random.default_rng(20250101)
+    graphs_done = []        # graphs stay alive until the end: nothing is destroyed between timed sections
+
+    def log(section):       # progress on stderr: a run that dies names the section it died in
+        print("[bench] " + section, file=sys.stderr, flush=True)
     layers_host = [make_layer(rng, LAYER_7B) for _ in range(args.layers)]
     layers = []
     for host in layers_host:
@@ -159,6 +163,7 @@ def main():
             dev._l.twm_memcpy_d2d(dev.handle, dst.ptr, src.ptr, 64 << 20)
         dev.synchronize()
 
+    log("decode layer: warm-up and graphs")
     # eager warm-up (also loads every code object before capture), then the graphs
     for li in range(args.layers):
         run_layer(li)
@@ -190,6 +195,7 @@ def main():
     layer_bytes = sum(algo_bytes(k, n) for _, k, n in LAYER_7B)
     value = layer_bytes / (ms_step * 1e-3) / 1e9
 
+    log("per-projection timings")
     # per-projection timings, eager launches rotating over the distinct layers
     per_shape = {}
     for name, k, n in LAYER_7B:
@@ -205,6 +211,7 @@ def main():
                            "frac_hbm": round(b / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
                            "splits": T.pick_splits(k, n, 1)}
 
+    log("drop-in on the reference layout")
     # the literal drop-in: gemm_tw_marlin_m1 on the reference's arrays (no repack), f32 activations
     drop_in = {}
     for name, k, n in LAYER_7B:
@@ -259,6 +266,7 @@ def main():
             extra["gate_up_M%d" % m] = {"us": round(ms * 1e3, 2), "GBps": round(b / (ms * 1e-3) / 1e9, 1),
                                         "frac_hbm": round(b / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
 
+    log("small configurations")
     # the small configurations: launch- and latency-bound, reported per projection and as one graph per layer
     small = {}
     for label, shapes in (("qwen05b", LAYER_05B), ("cfg0", CFG0)):
@@ -293,7 +301,7 @@ def main():
         ms = time_launches(dev, lambda i: g.replay(), 50) / len(sets)
         lb = sum(algo_bytes(k, n) for _, k, n in shapes)
         entry["layer_graph"] = {"us": round(ms * 1e3, 3), "GBps": round(lb / (ms * 1e-3) / 1e9, 1), "bytes": lb}
-        g.destroy()
+        graphs_done.append(g)
         small[label] = entry
         for st in sets:
             for name in st:
@@ -302,6 +310,7 @@ def main():
     # The LM head of the same model class as a TW-Marlin GEMV with on-device argmax (the reference has
     # forward_lm_head_tw_marlin, generate.rs:1748-1761, and a GPU argmax buffer, :1417): 3584 -> 152064, the
     # largest GEMV of a decode step.  Two weight sets (616 MB) alternate so that the cache cannot hold them.
+    log("LM head")
     lm = None
     if not args.no_lm_head:
         k, n = 3584, 152064
@@ -337,6 +346,7 @@ def main():
 
     # MLP front half at M=1: the reference's three launches (GEMV, split_gate_up, fused_silu_mul) against the
     # single launch with the gate applied in the GEMV's store; graphs over distinct weight sets
+    log("MLP front half")
     mlp_front = None
     if not args.no_swiglu:
         k, ffn = 3584, 18944
@@ -380,13 +390,14 @@ def main():
                 gr.replay()
             dev.synchronize()
             mlp_front[label] = round(time_launches(dev, lambda i: gr.replay(), 50) / L * 1e3, 2)
-            gr.destroy()
+            graphs_done.append(gr)
         assert np.array_equal(act1.to_host(), act3.to_host()), "fused SwiGLU differs from the three-launch sequence"
         for w in plain + pairedw:
             w.free()
 
     # Mixture-of-experts decode (the reference's Gemma MoE shape: hidden 2816, expert dim 704, 128 experts, top 8):
     # gate+up of the eight routed experts, GEGLU, down + weighted sum; ids rotate so the experts come from HBM
+    log("MoE decode")
     moe = None
     if not args.no_moe:
         k, dim, experts, top_k = 2816, 704, 128, 8
@@ -429,11 +440,12 @@ def main():
             us = time_launches(dev, lambda i: gr.replay(), 30) / len(id_sets) * 1e3
             moe[label] = round(us, 2)
             moe[label.replace("_us", "_GBps")] = round(moe_bytes / (us * 1e-6) / 1e9, 1)
-            gr.destroy()
+            graphs_done.append(gr)
         assert np.array_equal(acc_a.to_host(), acc_b.to_host()), "fused GEGLU differs from the three-launch sequence"
         for b_ in (bank_gu, bank_gu_paired, bank_d):
             b_.free()
 
+    log("prefill")
     prefill = None
     if not args.no_prefill:
         prefill = {}
@@ -494,6 +506,7 @@ def main():
                 a_m.free()
                 c_m.free()
 
+    log("cpu baseline")
     cpu = None
     if not args.no_cpu:
         # the checker, timed: reference CPU semantics, one thread, whole layers (a different weight set each pass)
@@ -570,7 +583,7 @@ def main():
     if sweep:
         out["split_sweep"] = sweep
     print(json.dumps(out))
-    for g in graphs + [graph_all]:
+    for g in graphs + [graph_all] + graphs_done:
         g.destroy()
     dev.close()
 
