@@ -486,6 +486,41 @@ def main():
                 c_m.free()
             w.free()
 
+    # prefill MLP front half (LLaMA-7B: 4096 -> 2 x 11008, M = 2048): GEMM to [M, 2*ffn] + split/gate kernel
+    # against the gate applied in the GEMM's store
+    prefill_mlp = None
+    if not args.no_prefill and not args.no_swiglu:
+        log("prefill MLP front half")
+        k, ffn, m = 4096, 11008, 2048
+        halves = []
+        for _h in range(2):
+            packed = rng.integers(0, 256, size=(k // 32) * ffn * 16, dtype=np.uint8)
+            scales = (np.abs(rng.standard_normal((k // 32) * ffn, dtype=np.float32)) * np.float32(0.02)).astype(np.float16)
+            halves.append((T.GpuTensor.from_host(dev, packed), T.GpuTensor.from_host(dev, scales.view(np.uint16), "f16")))
+        wp = T.MarlinWeight.gate_up(dev, halves[0], halves[1], k, ffn)
+        a_m = T.GpuTensor.from_host(dev, rng.standard_normal((m, k), dtype=np.float32).astype(np.float16).view(np.uint16), "f16")
+        tmp = T.GpuTensor.zeros(dev, (m, 2 * ffn), "f32")
+        seq, fused_out = T.GpuTensor.zeros(dev, (m, ffn), "f32"), T.GpuTensor.zeros(dev, (m, ffn), "f32")
+
+        def two_step(i):
+            T.gemm(dev, wp, a_m, m, tmp)
+            T.swiglu_rows(dev, tmp, seq, ffn, m, paired=True)
+
+        def one_step(i):
+            T.gemm_swiglu(dev, wp, a_m, m, fused_out)
+        prefill_mlp = {"m": m, "k": k, "ffn": ffn}
+        for label, fn in (("gemm_then_gate_us", two_step), ("fused_us", one_step)):
+            for i in range(3):
+                fn(i)
+            dev.synchronize()
+            ms = time_launches(dev, fn, 10)
+            prefill_mlp[label] = round(ms * 1e3, 1)
+            prefill_mlp[label.replace("_us", "_TFLOPs")] = round(2.0 * m * 2 * ffn * k / (ms * 1e-3) / 1e12, 1)
+        assert np.array_equal(fused_out.to_host(), seq.to_host()), "fused prefill SwiGLU differs from GEMM + gate"
+        for t in (tmp, seq, fused_out, a_m, halves[0][0], halves[0][1], halves[1][0], halves[1][1]):
+            t.free()
+        wp.free()
+
     sweep = None
     if args.sweep_splits:
         sweep = {}
@@ -572,6 +607,8 @@ def main():
         out["mlp_front_m1"] = mlp_front
     if moe is not None:
         out["moe_decode_m1"] = moe
+    if prefill_mlp:
+        out["prefill_mlp_front"] = prefill_mlp
     if prefill:
         out["prefill"] = prefill
         best = max(prefill.items(), key=lambda kv: kv[1]["TFLOPs"] if kv[0].startswith("M2048") else 0.0)

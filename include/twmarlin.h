@@ -254,13 +254,13 @@ twm_weight *twm_weight_gate_up(twm_ctx *ctx, const uint8_t *gate_packed_dev, con
                                uint32_t ffn_dim);
 int twm_weight_is_paired(const twm_weight *w);
 /* The MLP front half in one call: out[M][ffn_dim] = silu(A x W_gate) * (A x W_up), replacing
- * gemm_tw_marlin_m1 + split_gate_up + fused_silu_mul (generate.rs:2195-2203).  w must come from
- * twm_weight_gate_up.  M <= 4: a single launch, the gate is applied in the GEMV's store and the
- * 2*ffn_dim intermediate never reaches memory.  Larger M: the GEMM writes tmp_dev (f32
- * [M][2*ffn_dim], may be NULL only when M <= 4) and twm_swiglu_rows follows.  The arithmetic of the
- * projections is twm_gemm's for the same M. */
+ * gemm_tw_marlin_m1 + split_gate_up + fused_silu_mul (generate.rs:2195-2203; prefill: 1086-1093).
+ * w must come from twm_weight_gate_up.  The gate is applied in the GEMM's store (or, with split-K,
+ * in the kernel that adds the partial sums), so the [M][2*ffn_dim] intermediate never reaches
+ * memory, for every M.  The arithmetic of the projections is twm_gemm's for the same M.
+ * out_dev must be 16-byte aligned. */
 int twm_gemm_swiglu(twm_ctx *ctx, const twm_weight *w, const void *a_dev, int a_dtype, uint32_t m,
-                    float *out_dev, float *tmp_dev, uint32_t splits);
+                    float *out_dev, uint32_t splits);
 /* ---- expert banks: the TW-Marlin GEMVs of mixture-of-experts decode ------------------------- */
 
 typedef struct twm_bank twm_bank;

@@ -906,8 +906,8 @@ uint32_t twm_pick_splits(uint32_t k, uint32_t n, uint32_t m)
     return plan_stream(n_tiles, k_chunks, m);
 }
 
-// swiglu_out (only with m <= 4 on the one-lane-per-column kernel, paired weight): the launch writes
-// silu(gate) * up to swiglu_out[m][n/2] instead of the columns to `out`.
+// swiglu_out (paired weight): the launch writes silu(gate) * up to swiglu_out[m][n/2] instead of the columns
+// to `out`.
 static int gemm_common(twm_ctx *ctx, const twm_weight *w, const void *a_dev, int a_dtype, uint32_t m, const OutSpec &out,
                        uint32_t splits, const char *who, float *swiglu_out = nullptr)
 {
@@ -931,18 +931,20 @@ static int gemm_common(twm_ctx *ctx, const twm_weight *w, const void *a_dev, int
     WeightView v = view_of(w);
     size_t a_row_bytes = (size_t)w->k * (a_dtype == TWM_F16 ? 2 : 4);
     uint32_t n_ld = w->n_tiles * kTileN;
-    if (swiglu_out && !(m <= 4 && m < (uint32_t)ctx->prefill_min_m && ctx->force_kernel != 1 && ctx->force_kernel != 3))
-        return fail(TWM_UNSUPPORTED_OP, "%s: the fused SwiGLU epilogue exists for M <= 4 on the one-lane-per-column kernel", who);
+    // the paired store: every kernel but the 16-column tile kernel of option "kernel" = 1 has it
+    OutSpec gated = out;
+    gated.swiglu = swiglu_out;
     if (m >= (uint32_t)ctx->prefill_min_m) {
-        HIP_TRY(launch_prefill(ctx->stream, v, a_dev, a_dtype == TWM_F32, m, out, (uint32_t)ctx->prefill_bm, splits, ctx->ws, ctx->ws_bytes), TWM_DEVICE_ERROR, "prefill launch");
+        HIP_TRY(launch_prefill(ctx->stream, v, a_dev, a_dtype == TWM_F32, m, gated, (uint32_t)ctx->prefill_bm, splits, ctx->ws, ctx->ws_bytes), TWM_DEVICE_ERROR, "prefill launch");
         return TWM_OK;
     }
     if (ctx->force_kernel == 3 || (ctx->force_kernel == 0 && m > 4)) {
         // batched decode: 32-row blocks of the streaming kernel
         for (uint32_t m0 = 0; m0 < m; m0 += kMaxStreamM) {
             uint32_t mb = m - m0 < (uint32_t)kMaxStreamM ? m - m0 : (uint32_t)kMaxStreamM;
-            OutSpec o = out;
+            OutSpec o = gated;
             for (uint32_t s = 0; s < o.count; s++) o.seg[s].ptr += (size_t)m0 * o.seg[s].width;
+            if (o.swiglu) o.swiglu += (size_t)m0 * (w->n / 2);
             const char *a_blk = (const char *)a_dev + (size_t)m0 * a_row_bytes;
             HIP_TRY(launch_stream(ctx->stream, v, a_blk, a_dtype == TWM_F32, mb, o, splits ? splits : plan_stream(w->n_tiles, w->k_chunks, mb),
                                   stream_waves(w->n_tiles, mb, ctx->force_waves), ctx->ws, ctx->ws_bytes),
@@ -954,6 +956,7 @@ static int gemm_common(twm_ctx *ctx, const twm_weight *w, const void *a_dev, int
         uint32_t mb = m - m0 < (uint32_t)kMaxDecodeM ? m - m0 : (uint32_t)kMaxDecodeM;
         DecodePlan plan;
         bool lane_col = mb <= 4 && ctx->force_kernel != 1;
+        if (swiglu_out && !lane_col) return fail(TWM_UNSUPPORTED_OP, "%s: the 16-column tile kernel has no gated store", who);
         if (ctx->force_kernel == 2 && !lane_col) return fail(TWM_UNSUPPORTED_OP, "%s: the one-lane-per-column kernel takes M <= 4", who);
         if (lane_col) plan = plan_gemv4(w->n_tiles, w->k_chunks, ctx->force_nt, ctx->force_waves, splits);
         else plan = plan_decode(w->n_tiles, w->k_chunks, mb, ctx->force_nt, ctx->force_waves == 1 || ctx->force_waves == 2 ? 0 : ctx->force_waves, splits);
@@ -1024,7 +1027,7 @@ int twm_gemm_split(twm_ctx *ctx, const twm_weight *w, const void *a_dev, int a_d
 }
 
 int twm_gemm_swiglu(twm_ctx *ctx, const twm_weight *w, const void *a_dev, int a_dtype, uint32_t m, float *out_dev,
-                    float *tmp_dev, uint32_t splits)
+                    uint32_t splits)
 {
     if (!ctx || !w) return fail(TWM_INVALID_HANDLE, "twm_gemm_swiglu: null handle");
     if (w->ctx != ctx) return fail(TWM_INVALID_HANDLE, "twm_gemm_swiglu: weight belongs to another context");
@@ -1032,19 +1035,11 @@ int twm_gemm_swiglu(twm_ctx *ctx, const twm_weight *w, const void *a_dev, int a_
     uint32_t ffn = w->n / 2;
     if (m == 0 || ffn == 0) return TWM_OK;
     if (!out_dev) return fail(TWM_INVALID_HANDLE, "twm_gemm_swiglu: null output");
+    if (((uintptr_t)out_dev & 15) != 0) return fail(TWM_SHAPE_ERROR, "twm_gemm_swiglu: the output must be 16-byte aligned");
     if (w->k == 0) return twm_memset_zero(ctx, out_dev, (size_t)m * ffn * 4);  // silu(0) * 0
     OutSpec out;
     memset(&out, 0, sizeof out);
-    bool fused = m <= 4 && m < (uint32_t)ctx->prefill_min_m && ctx->force_kernel != 1 && ctx->force_kernel != 3;
-    if (fused) return gemm_common(ctx, w, a_dev, a_dtype, m, out, splits, "twm_gemm_swiglu", out_dev);
-    if (!tmp_dev) return fail(TWM_INVALID_HANDLE, "twm_gemm_swiglu: M = %u needs the [M][2*ffn] f32 temporary", m);
-    out.count = 1;
-    out.seg[0].ptr = tmp_dev;
-    out.seg[0].start = 0;
-    out.seg[0].width = w->n;
-    if (int rc = gemm_common(ctx, w, a_dev, a_dtype, m, out, splits, "twm_gemm_swiglu")) return rc;
-    HIP_TRY(launch_swiglu_rows(ctx->stream, tmp_dev, out_dev, ffn, m, true), TWM_DEVICE_ERROR, "swiglu_rows launch");
-    return TWM_OK;
+    return gemm_common(ctx, w, a_dev, a_dtype, m, out, splits, "twm_gemm_swiglu", out_dev);
 }
 
 /* ---- expert banks (mixture-of-experts decode) ------------------------------------------------ */

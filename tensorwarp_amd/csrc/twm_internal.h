@@ -38,7 +38,13 @@ struct OutSeg {
 struct OutSpec {
     OutSeg seg[kMaxSegs];
     uint32_t count;
+    // Paired gate/up weight only: when set, the store writes silu(gate) * up of every feature to
+    // swiglu[row][n / 2] instead of the n columns to the segments.
+    float *swiglu;
 };
+
+// feature index of internal column `col` of a paired weight (col % 64 < 32: the gate column; + 32: its up column)
+__host__ __device__ __forceinline__ uint32_t paired_feature(uint32_t col) { return (col >> 6) * kPairWidth + (col & 31u); }
 
 struct WeightView {
     const void *qw;

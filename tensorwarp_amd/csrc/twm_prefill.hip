@@ -273,6 +273,25 @@ __global__ __launch_bounds__(256) void k_prefill(const uint4v *__restrict__ qw, 
         }
         return;
     }
+    if (out.swiglu) {
+        // paired gate/up weight: this wave's tiles 0, 1 are 32 gate columns and tiles 2, 3 the up columns of the
+        // same features, in the same lanes and registers
+        const uint32_t ffn = n >> 1;
+#pragma unroll
+        for (int t = 0; t < 2; t++) {
+            if (nt0 + t + 2 >= n_tiles) continue;
+            const uint32_t feat = paired_feature((nt0 + t) * 16u + c);
+            if (feat >= ffn) continue;
+#pragma unroll
+            for (int mt = 0; mt < MT; mt++)
+#pragma unroll
+                for (int r = 0; r < 4; r++) {
+                    uint32_t om = m0 + mt * 16u + kb * 4u + r;
+                    if (om < m_rows) out.swiglu[(size_t)om * ffn + feat] = silu_mul_f32(acc[mt][t][r], acc[mt][t + 2][r]);
+                }
+        }
+        return;
+    }
 #pragma unroll
     for (int t = 0; t < 4; t++) {
         if (nt0 + t >= n_tiles) continue;
@@ -309,6 +328,28 @@ __global__ __launch_bounds__(256) void k_splitk_reduce(const float *__restrict__
     if (col + 3 < n) pf_store_out(out, row, col + 3, s.w);
 }
 
+// The same sum for a paired gate/up weight: one thread per four features adds the gate and the up partials
+// (32 columns apart) in split order and stores silu(gate) * up.
+__global__ __launch_bounds__(256) void k_splitk_reduce_swiglu(const float *__restrict__ partials, float *__restrict__ gate_out,
+                                                                uint32_t m_rows, uint32_t ffn, uint32_t n_ld, uint32_t splits)
+{
+    size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+    uint32_t quads = ffn / 4;  // ffn is a multiple of 32
+    if (idx >= (size_t)m_rows * quads) return;
+    uint32_t row = (uint32_t)(idx / quads), feat = (uint32_t)(idx % quads) * 4u;
+    uint32_t col = (feat >> 5) * 64u + (feat & 31u);
+    const float4 *src = (const float4 *)(partials + (size_t)row * n_ld + col);
+    size_t stride4 = (size_t)m_rows * n_ld / 4;
+    float4 g = src[0], u = src[8];
+    for (uint32_t z = 1; z < splits; z++) {
+        float4 v = src[z * stride4], w = src[z * stride4 + 8];
+        g.x += v.x; g.y += v.y; g.z += v.z; g.w += v.w;
+        u.x += w.x; u.y += w.y; u.z += w.z; u.w += w.w;
+    }
+    float4 o = {silu_mul_f32(g.x, u.x), silu_mul_f32(g.y, u.y), silu_mul_f32(g.z, u.z), silu_mul_f32(g.w, u.w)};
+    *(float4 *)(gate_out + (size_t)row * ffn + feat) = o;
+}
+
 // f32 activations are rounded to f16 (round-to-nearest-even, as the MFMA operand needs) into scratch first
 __global__ __launch_bounds__(256) void k_cvt_f32_f16(const float4 *__restrict__ src, uint2v *__restrict__ dst, size_t n4)
 {
@@ -326,6 +367,13 @@ hipError_t launch_splitk_reduce(hipStream_t s, const float *partials, const OutS
 {
     size_t quads = (size_t)m * n_ld / 4;
     if (quads == 0) return hipSuccess;
+    if (out.swiglu) {
+        if (n % (2 * kPairWidth) != 0) return hipErrorInvalidValue;
+        size_t fq = (size_t)m * (n / 2) / 4;
+        hipLaunchKernelGGL(k_splitk_reduce_swiglu, dim3((unsigned)((fq + 255) / 256)), dim3(256), 0, s, partials, out.swiglu, m,
+                           n / 2, n_ld, splits);
+        return hipGetLastError();
+    }
     hipLaunchKernelGGL(k_splitk_reduce, dim3((unsigned)((quads + 255) / 256)), dim3(256), 0, s, partials, out, m, n, n_ld,
                        splits);
     return hipGetLastError();
@@ -417,6 +465,7 @@ hipError_t launch_prefill(hipStream_t s, const WeightView &w, const void *a, boo
                            (const float4 *)((const float *)a + (size_t)r0 * w.k), (uint2v *)scratch, n4);
         OutSpec o = out;
         for (uint32_t i = 0; i < o.count; i++) o.seg[i].ptr += (size_t)r0 * o.seg[i].width;
+        if (o.swiglu) o.swiglu += (size_t)r0 * (w.n / 2);
         size_t used = ((size_t)rows * row_bytes + 255) & ~(size_t)255;
         hipError_t e = run((const _Float16 *)scratch, rows, o, (char *)scratch + used, scratch_bytes - used);
         if (e != hipSuccess) return e;

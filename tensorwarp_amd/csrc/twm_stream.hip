@@ -218,6 +218,16 @@ __global__ __launch_bounds__(WAVES * 64) void k_stream(const uint4v *__restrict_
         if (row >= m_rows) continue;
         if (partials) {
             partials[((size_t)blockIdx.y * m_rows + row) * n_ld + on] = s;
+        } else if (out.swiglu) {
+            // paired gate/up weight: columns 0..31 of the quad are gate columns, 32..63 the up columns of the same
+            // features (two tiles = eight registers further in the same lane)
+            if (col < 32u) {
+                float u = red[0][reg + 8][src_lane];
+#pragma unroll
+                for (int w = 1; w < WAVES; w++) u += red[w][reg + 8][src_lane];
+                const uint32_t ffn = n >> 1, feat = paired_feature(on);
+                if (feat < ffn) out.swiglu[(size_t)row * ffn + feat] = silu_mul_f32(s, u);
+            }
         } else if (on < n) {
 #pragma unroll
             for (uint32_t sg = 0; sg < kMaxSegs; sg++) {

@@ -330,12 +330,11 @@ def gemm(device, weight, a, m, c, splits=0):
     _check(device._l.twm_gemm(device.handle, weight.handle, a.ptr, dt, m, c.ptr, splits))
 
 
-def gemm_swiglu(device, weight, a, m, out, tmp=None, splits=0):
+def gemm_swiglu(device, weight, a, m, out, splits=0):
     """out[M, ffn] = silu(A x W_gate) * (A x W_up) on a MarlinWeight.gate_up weight: gemm_tw_marlin_m1 +
-    split_gate_up + fused_silu_mul of the decode step in one launch for M <= 4; larger M needs tmp [M, 2*ffn]."""
+    split_gate_up + fused_silu_mul of the decode step (and of prefill) with the gate applied in the GEMM's store."""
     dt = _lib.F16 if a.dtype == "f16" else _lib.F32
-    _check(device._l.twm_gemm_swiglu(device.handle, weight.handle, a.ptr, dt, m, out.ptr,
-                                     tmp.ptr if tmp is not None else None, splits))
+    _check(device._l.twm_gemm_swiglu(device.handle, weight.handle, a.ptr, dt, m, out.ptr, splits))
 
 
 def gemm_split(device, weight, a, m, outs, ns, splits=0, biases=None):

@@ -192,7 +192,7 @@ def test_gemm_swiglu_fused_epilogue(dev, h, ffn, m, splits):
     w = T.MarlinWeight.gate_up(dev, gd, ud, h, ffn)
     assert w.paired and not plain.paired
     out = T.GpuTensor.from_host(dev, np.full((m, ffn), np.nan, np.float32))
-    T.gemm_swiglu(dev, w, ad, m, out, None, splits)
+    T.gemm_swiglu(dev, w, ad, m, out, splits)
     assert np.array_equal(out.to_host(), seq.to_host())
     # against the oracle: f64 projections, then the reference's gate in f32 (its input differs from the
     # GPU's by the GEMV's rounding, so the bar is the GEMV's)
@@ -203,7 +203,7 @@ def test_gemm_swiglu_fused_epilogue(dev, h, ffn, m, splits):
     # f32 activations take the same path
     a32 = T.GpuTensor.from_host(dev, a)
     out32 = T.GpuTensor.zeros(dev, (m, ffn), "f32")
-    T.gemm_swiglu(dev, w, a32, m, out32, None, splits)
+    T.gemm_swiglu(dev, w, a32, m, out32, splits)
     assert np.array_equal(out32.to_host(), out.to_host())
     with pytest.raises(T.DeviceError):
         T.gemm_swiglu(dev, plain, ad, m, out)        # not a paired weight
@@ -211,8 +211,9 @@ def test_gemm_swiglu_fused_epilogue(dev, h, ffn, m, splits):
     plain.free()
 
 
-@pytest.mark.parametrize("m", [8, 24, 40])
-def test_gemm_swiglu_larger_m_goes_through_the_temporary(dev, m):
+@pytest.mark.parametrize("m,splits", [(8, 0), (8, 3), (24, 0), (32, 2), (40, 0), (40, 2), (150, 0)])
+def test_gemm_swiglu_batched_and_prefill_rows(dev, m, splits):
+    # the gated store of the streaming kernel (M = 5..32), of the prefill GEMM, and of the split-K sum
     h, ffn = 640, 224
     gp, gs = O.synth_packed(h, ffn, 960), O.synth_scales(h, ffn, 961)
     up, us = O.synth_packed(h, ffn, 962), O.synth_scales(h, ffn, 963)
@@ -221,23 +222,32 @@ def test_gemm_swiglu_larger_m_goes_through_the_temporary(dev, m):
     a16 = O.synth_act_f16(m, h, 964)
     ad = T.GpuTensor.from_host(dev, a16, "f16")
     w = T.MarlinWeight.gate_up(dev, gd, ud, h, ffn)
-    out = T.GpuTensor.zeros(dev, (m, ffn), "f32")
-    with pytest.raises(T.DeviceError):
-        T.gemm_swiglu(dev, w, ad, m, out)            # no temporary
+    out = T.GpuTensor.from_host(dev, np.full((m, ffn), np.nan, np.float32))
+    T.gemm_swiglu(dev, w, ad, m, out, splits)
+    # the plain GEMM on a paired handle returns the columns in the paired order; gating them afterwards gives the
+    # same bits as the fused store
     tmp = T.GpuTensor.zeros(dev, (m, 2 * ffn), "f32")
-    T.gemm_swiglu(dev, w, ad, m, out, tmp)
+    T.gemm(dev, w, ad, m, tmp, splits)
+    seq = T.GpuTensor.zeros(dev, (m, ffn), "f32")
+    T.swiglu_rows(dev, tmp, seq, ffn, m, paired=True)
+    assert np.array_equal(out.to_host(), seq.to_host())
     fp, fs = O.fuse_tw_marlin_n([(gp, gs), (up, us)], h, [ffn, ffn])
     t = gemm_truth(a16, fp, fs, m, h, 2 * ffn)
     tg, tu = t[:, :ffn], t[:, ffn:]
     truth = tg / (1.0 + np.exp(-tg)) * tu
-    assert rel_err(out.to_host(), truth) < (TIGHT if m <= 32 else 1e-3)
-    # the plain GEMM on a paired handle returns the columns in the paired order
-    T.gemm(dev, w, ad, m, tmp)
+    bar = TIGHT if m <= 32 else 1e-3
+    assert rel_err(out.to_host(), truth) < bar
     j = np.arange(ffn)
     col = (j // 32) * 64 + j % 32
     got = tmp.to_host().reshape(m, 2 * ffn)
-    assert rel_err(got[:, col], tg) < (TIGHT if m <= 32 else 1e-3)
-    assert rel_err(got[:, col + 32], tu) < (TIGHT if m <= 32 else 1e-3)
+    assert rel_err(got[:, col], tg) < bar and rel_err(got[:, col + 32], tu) < bar
+    try:
+        dev.set_option("kernel", 1)                      # the 16-column tile kernel has no gated store
+        if m < 33:
+            with pytest.raises(T.DeviceError):
+                T.gemm_swiglu(dev, w, ad, m, out, splits)
+    finally:
+        dev.set_option("kernel", 0)
     w.free()
 
 
@@ -1040,7 +1050,7 @@ def test_graph_of_fused_epilogues_and_expert_banks(dev):
         dev.synchronize()
         for nm, t in bufs.items():
             assert np.array_equal(t.to_host(), eager[nm]), (rep, nm)
-        T.gemm_swiglu(dev, wgu, x, 1, act, None, 3)                 # eager work between replays
+        T.gemm_swiglu(dev, wgu, x, 1, act, 3)                 # eager work between replays
         dev.synchronize()
     graph.destroy()
     for wobj in (wgu, wqkv, gub, db):
