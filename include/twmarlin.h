@@ -261,6 +261,10 @@ int twm_weight_is_paired(const twm_weight *w);
  * out_dev must be 16-byte aligned. */
 int twm_gemm_swiglu(twm_ctx *ctx, const twm_weight *w, const void *a_dev, int a_dtype, uint32_t m,
                     float *out_dev, uint32_t splits);
+/* The same with the GEGLU gate of the Gemma models, gelu_tanh(gate) * up (fused_gelu_mul,
+ * ops.rs:1157-1190; callers gemma_generate.rs:463, 623). */
+int twm_gemm_geglu(twm_ctx *ctx, const twm_weight *w, const void *a_dev, int a_dtype, uint32_t m,
+                   float *out_dev, uint32_t splits);
 /* ---- expert banks: the TW-Marlin GEMVs of mixture-of-experts decode ------------------------- */
 
 typedef struct twm_bank twm_bank;

@@ -65,6 +65,7 @@ SIGNATURES = {
     "twm_weight_gate_up": (_vp, [_vp, _vp, _vp, _vp, _vp, _u32, _u32]),
     "twm_weight_is_paired": (_int, [_vp]),
     "twm_gemm_swiglu": (_int, [_vp, _vp, _vp, _int, _u32, _vp, _u32]),
+    "twm_gemm_geglu": (_int, [_vp, _vp, _vp, _int, _u32, _vp, _u32]),
     "twm_gemm_split_bias": (_int, [_vp, _vp, _vp, _int, _u32, C.POINTER(_vp), C.POINTER(_vp), C.POINTER(_u32), _u32, _u32]),
     "twm_bank_from_device": (_vp, [_vp, _vp, _vp, _sz, _sz, _u32, _u32, _u32, _int]),
     "twm_bank_destroy": (None, [_vp]),

@@ -909,7 +909,7 @@ uint32_t twm_pick_splits(uint32_t k, uint32_t n, uint32_t m)
 // swiglu_out (paired weight): the launch writes silu(gate) * up to swiglu_out[m][n/2] instead of the columns
 // to `out`.
 static int gemm_common(twm_ctx *ctx, const twm_weight *w, const void *a_dev, int a_dtype, uint32_t m, const OutSpec &out,
-                       uint32_t splits, const char *who, float *swiglu_out = nullptr)
+                       uint32_t splits, const char *who, float *swiglu_out = nullptr, uint32_t gate_act = 2)
 {
     if (a_dtype != TWM_F16 && a_dtype != TWM_F32) return fail(TWM_UNSUPPORTED_OP, "%s: activations must be f16 or f32", who);
     if (m == 0 || w->n == 0) return TWM_OK;
@@ -934,6 +934,7 @@ static int gemm_common(twm_ctx *ctx, const twm_weight *w, const void *a_dev, int
     // the paired store: every kernel but the 16-column tile kernel of option "kernel" = 1 has it
     OutSpec gated = out;
     gated.swiglu = swiglu_out;
+    gated.gate_act = gate_act;
     if (m >= (uint32_t)ctx->prefill_min_m) {
         HIP_TRY(launch_prefill(ctx->stream, v, a_dev, a_dtype == TWM_F32, m, gated, (uint32_t)ctx->prefill_bm, splits, ctx->ws, ctx->ws_bytes), TWM_DEVICE_ERROR, "prefill launch");
         return TWM_OK;
@@ -963,7 +964,7 @@ static int gemm_common(twm_ctx *ctx, const twm_weight *w, const void *a_dev, int
         // the scratch must hold splits x mb x n_ld partials and one counter per tile group
         while (plan.splits > 1 && (size_t)plan.splits * mb * n_ld * 4 > ctx->ws_bytes) plan.splits--;
         if (w->n_tiles / plan.nt > ctx->n_counters) plan.splits = 1;
-        OutSpec o = out;
+        OutSpec o = gated;   // (the one-lane-per-column kernel takes the gated output as its own argument)
         for (uint32_t s = 0; s < o.count; s++) o.seg[s].ptr += (size_t)m0 * o.seg[s].width;
         const char *a_blk = (const char *)a_dev + (size_t)m0 * a_row_bytes;
         if (lane_col)
@@ -1026,20 +1027,32 @@ int twm_gemm_split(twm_ctx *ctx, const twm_weight *w, const void *a_dev, int a_d
     return twm_gemm_split_bias(ctx, w, a_dev, a_dtype, m, outs_dev, nullptr, ns, count, splits);
 }
 
+static int gemm_gated(twm_ctx *ctx, const twm_weight *w, const void *a_dev, int a_dtype, uint32_t m, float *out_dev,
+                      uint32_t splits, uint32_t act, const char *who)
+{
+    if (!ctx || !w) return fail(TWM_INVALID_HANDLE, "%s: null handle", who);
+    if (w->ctx != ctx) return fail(TWM_INVALID_HANDLE, "%s: weight belongs to another context", who);
+    if (!w->paired) return fail(TWM_UNSUPPORTED_OP, "%s: the weight was not built by twm_weight_gate_up", who);
+    uint32_t ffn = w->n / 2;
+    if (m == 0 || ffn == 0) return TWM_OK;
+    if (!out_dev) return fail(TWM_INVALID_HANDLE, "%s: null output", who);
+    if (((uintptr_t)out_dev & 15) != 0) return fail(TWM_SHAPE_ERROR, "%s: the output must be 16-byte aligned", who);
+    if (w->k == 0) return twm_memset_zero(ctx, out_dev, (size_t)m * ffn * 4);  // gate(0) * 0
+    OutSpec out;
+    memset(&out, 0, sizeof out);
+    return gemm_common(ctx, w, a_dev, a_dtype, m, out, splits, who, out_dev, act);
+}
+
 int twm_gemm_swiglu(twm_ctx *ctx, const twm_weight *w, const void *a_dev, int a_dtype, uint32_t m, float *out_dev,
                     uint32_t splits)
 {
-    if (!ctx || !w) return fail(TWM_INVALID_HANDLE, "twm_gemm_swiglu: null handle");
-    if (w->ctx != ctx) return fail(TWM_INVALID_HANDLE, "twm_gemm_swiglu: weight belongs to another context");
-    if (!w->paired) return fail(TWM_UNSUPPORTED_OP, "twm_gemm_swiglu: the weight was not built by twm_weight_gate_up");
-    uint32_t ffn = w->n / 2;
-    if (m == 0 || ffn == 0) return TWM_OK;
-    if (!out_dev) return fail(TWM_INVALID_HANDLE, "twm_gemm_swiglu: null output");
-    if (((uintptr_t)out_dev & 15) != 0) return fail(TWM_SHAPE_ERROR, "twm_gemm_swiglu: the output must be 16-byte aligned");
-    if (w->k == 0) return twm_memset_zero(ctx, out_dev, (size_t)m * ffn * 4);  // silu(0) * 0
-    OutSpec out;
-    memset(&out, 0, sizeof out);
-    return gemm_common(ctx, w, a_dev, a_dtype, m, out, splits, "twm_gemm_swiglu", out_dev);
+    return gemm_gated(ctx, w, a_dev, a_dtype, m, out_dev, splits, 2, "twm_gemm_swiglu");
+}
+
+int twm_gemm_geglu(twm_ctx *ctx, const twm_weight *w, const void *a_dev, int a_dtype, uint32_t m, float *out_dev,
+                   uint32_t splits)
+{
+    return gemm_gated(ctx, w, a_dev, a_dtype, m, out_dev, splits, 1, "twm_gemm_geglu");
 }
 
 /* ---- expert banks (mixture-of-experts decode) ------------------------------------------------ */

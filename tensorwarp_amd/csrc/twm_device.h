@@ -19,4 +19,18 @@ __device__ __forceinline__ float silu_mul_f32(float g, float u)
     return silu_g * u;
 }
 
+// warp_fused_gelu_mul's gate (crates/kernels/src/ops.rs:1161-1170, the tanh form), used by the reference's
+// batched_marlin_split_geglu as well
+__device__ __forceinline__ float gelu_mul_f32(float g, float u)
+{
+    float gelu_g = 0.5f * g * (1.0f + tanhf(0.7978845608f * (g + 0.044715f * g * g * g)));
+    return gelu_g * u;
+}
+
+// the gate of a paired store: act 1 = gelu_tanh(g) * u, otherwise silu(g) * u (act is uniform over the launch)
+__device__ __forceinline__ float gated_mul(uint32_t act, float g, float u)
+{
+    return act == 1u ? gelu_mul_f32(g, u) : silu_mul_f32(g, u);
+}
+
 }  // namespace twm

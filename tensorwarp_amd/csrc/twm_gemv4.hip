@@ -132,7 +132,7 @@ __global__ __launch_bounds__(1024) void k_gemv4(const char *__restrict__ cw, con
                         g += red[(w * NT * RL + tr) * 64 + ln];
                         u += red[(w * NT * RL + tr) * 64 + 32 + ln];
                     }
-                    swiglu_out[(size_t)r * ffn + feat] = silu_mul_f32(g, u);
+                    swiglu_out[(size_t)r * ffn + feat] = gated_mul(out.gate_act, g, u);
                 }
             }
             return;
@@ -180,7 +180,7 @@ __global__ __launch_bounds__(1024) void k_gemv4(const char *__restrict__ cw, con
                     g += __hip_atomic_load(row, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                     u += __hip_atomic_load(row + 32, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                 }
-                swiglu_out[(size_t)r * ffn + feat] = silu_mul_f32(g, u);
+                swiglu_out[(size_t)r * ffn + feat] = gated_mul(out.gate_act, g, u);
             }
         }
         if (threadIdx.x == 0) __hip_atomic_store(&counters[tg], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);

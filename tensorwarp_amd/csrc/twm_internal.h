@@ -41,6 +41,7 @@ struct OutSpec {
     // Paired gate/up weight only: when set, the store writes silu(gate) * up of every feature to
     // swiglu[row][n / 2] instead of the n columns to the segments.
     float *swiglu;
+    uint32_t gate_act;  // 1 = gelu_tanh(gate) * up (GEGLU), otherwise silu(gate) * up
 };
 
 // feature index of internal column `col` of a paired weight (col % 64 < 32: the gate column; + 32: its up column)

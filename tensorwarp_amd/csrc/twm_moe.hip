@@ -16,14 +16,6 @@
 
 namespace twm {
 
-// warp_fused_gelu_mul's gate (crates/kernels/src/ops.rs:1161-1170, the tanh form), used by the reference's
-// batched_marlin_split_geglu as well
-__device__ __forceinline__ float gelu_mul_f32(float g, float u)
-{
-    float gelu_g = 0.5f * g * (1.0f + tanhf(0.7978845608f * (g + 0.044715f * g * g * g)));
-    return gelu_g * u;
-}
-
 template <int ACT>
 __device__ __forceinline__ float gate_mul(float g, float u)
 {

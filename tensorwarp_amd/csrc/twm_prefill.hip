@@ -287,7 +287,7 @@ __global__ __launch_bounds__(256) void k_prefill(const uint4v *__restrict__ qw, 
 #pragma unroll
                 for (int r = 0; r < 4; r++) {
                     uint32_t om = m0 + mt * 16u + kb * 4u + r;
-                    if (om < m_rows) out.swiglu[(size_t)om * ffn + feat] = silu_mul_f32(acc[mt][t][r], acc[mt][t + 2][r]);
+                    if (om < m_rows) out.swiglu[(size_t)om * ffn + feat] = gated_mul(out.gate_act, acc[mt][t][r], acc[mt][t + 2][r]);
                 }
         }
         return;
@@ -331,7 +331,8 @@ __global__ __launch_bounds__(256) void k_splitk_reduce(const float *__restrict__
 // The same sum for a paired gate/up weight: one thread per four features adds the gate and the up partials
 // (32 columns apart) in split order and stores silu(gate) * up.
 __global__ __launch_bounds__(256) void k_splitk_reduce_swiglu(const float *__restrict__ partials, float *__restrict__ gate_out,
-                                                                uint32_t m_rows, uint32_t ffn, uint32_t n_ld, uint32_t splits)
+                                                                uint32_t m_rows, uint32_t ffn, uint32_t n_ld, uint32_t splits,
+                                                                uint32_t act)
 {
     size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
     uint32_t quads = ffn / 4;  // ffn is a multiple of 32
@@ -346,7 +347,7 @@ __global__ __launch_bounds__(256) void k_splitk_reduce_swiglu(const float *__res
         g.x += v.x; g.y += v.y; g.z += v.z; g.w += v.w;
         u.x += w.x; u.y += w.y; u.z += w.z; u.w += w.w;
     }
-    float4 o = {silu_mul_f32(g.x, u.x), silu_mul_f32(g.y, u.y), silu_mul_f32(g.z, u.z), silu_mul_f32(g.w, u.w)};
+    float4 o = {gated_mul(act, g.x, u.x), gated_mul(act, g.y, u.y), gated_mul(act, g.z, u.z), gated_mul(act, g.w, u.w)};
     *(float4 *)(gate_out + (size_t)row * ffn + feat) = o;
 }
 
@@ -371,7 +372,7 @@ hipError_t launch_splitk_reduce(hipStream_t s, const float *partials, const OutS
         if (n % (2 * kPairWidth) != 0) return hipErrorInvalidValue;
         size_t fq = (size_t)m * (n / 2) / 4;
         hipLaunchKernelGGL(k_splitk_reduce_swiglu, dim3((unsigned)((fq + 255) / 256)), dim3(256), 0, s, partials, out.swiglu, m,
-                           n / 2, n_ld, splits);
+                           n / 2, n_ld, splits, out.gate_act);
         return hipGetLastError();
     }
     hipLaunchKernelGGL(k_splitk_reduce, dim3((unsigned)((quads + 255) / 256)), dim3(256), 0, s, partials, out, m, n, n_ld,

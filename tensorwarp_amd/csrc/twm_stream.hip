@@ -226,7 +226,7 @@ __global__ __launch_bounds__(WAVES * 64) void k_stream(const uint4v *__restrict_
 #pragma unroll
                 for (int w = 1; w < WAVES; w++) u += red[w][reg + 8][src_lane];
                 const uint32_t ffn = n >> 1, feat = paired_feature(on);
-                if (feat < ffn) out.swiglu[(size_t)row * ffn + feat] = silu_mul_f32(s, u);
+                if (feat < ffn) out.swiglu[(size_t)row * ffn + feat] = gated_mul(out.gate_act, s, u);
             }
         } else if (on < n) {
 #pragma unroll

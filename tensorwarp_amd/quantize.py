@@ -337,6 +337,12 @@ def gemm_swiglu(device, weight, a, m, out, splits=0):
     _check(device._l.twm_gemm_swiglu(device.handle, weight.handle, a.ptr, dt, m, out.ptr, splits))
 
 
+def gemm_geglu(device, weight, a, m, out, splits=0):
+    """gemm_swiglu with the Gemma gate: out = gelu_tanh(A x W_gate) * (A x W_up)."""
+    dt = _lib.F16 if a.dtype == "f16" else _lib.F32
+    _check(device._l.twm_gemm_geglu(device.handle, weight.handle, a.ptr, dt, m, out.ptr, splits))
+
+
 def gemm_split(device, weight, a, m, outs, ns, splits=0, biases=None):
     """Fused projection whose column ranges land in separate buffers (gemm + split_qkv/split_gate_up);
     biases: optional list of f32 [ns[i]] tensors (or None entries) added in the store (bq/bk/bv)."""

@@ -251,6 +251,32 @@ def test_gemm_swiglu_batched_and_prefill_rows(dev, m, splits):
     w.free()
 
 
+@pytest.mark.parametrize("m,splits", [(1, 0), (2, 3), (4, 0), (12, 2), (40, 0), (40, 2)])
+def test_gemm_geglu_gate(dev, m, splits):
+    # Gemma's gate (fused_gelu_mul, ops.rs:1157-1190) in the same stores
+    h, ffn = 640, 224
+    gp, gs = O.synth_packed(h, ffn, 1200), O.synth_scales(h, ffn, 1201)
+    up, us = O.synth_packed(h, ffn, 1202), O.synth_scales(h, ffn, 1203)
+    gd = (T.GpuTensor.from_host(dev, gp), T.GpuTensor.from_host(dev, gs, "f16"))
+    ud = (T.GpuTensor.from_host(dev, up), T.GpuTensor.from_host(dev, us, "f16"))
+    a16 = O.synth_act_f16(m, h, 1204)
+    ad = T.GpuTensor.from_host(dev, a16, "f16")
+    w = T.MarlinWeight.gate_up(dev, gd, ud, h, ffn)
+    out = T.GpuTensor.from_host(dev, np.full((m, ffn), np.nan, np.float32))
+    T.gemm_geglu(dev, w, ad, m, out, splits)
+    tmp = T.GpuTensor.zeros(dev, (m, 2 * ffn), "f32")
+    T.gemm(dev, w, ad, m, tmp, splits)
+    seq = T.GpuTensor.zeros(dev, (m, ffn), "f32")
+    T.batched_marlin_split_geglu(dev, tmp, seq, ffn, m, paired=True)
+    assert np.array_equal(out.to_host(), seq.to_host())
+    fp, fs = O.fuse_tw_marlin_n([(gp, gs), (up, us)], h, [ffn, ffn])
+    t = gemm_truth(a16, fp, fs, m, h, 2 * ffn)
+    tg, tu = t[:, :ffn], t[:, ffn:]
+    truth = 0.5 * tg * (1.0 + np.tanh(0.7978845608 * (tg + 0.044715 * tg ** 3))) * tu
+    assert rel_err(out.to_host(), truth) < (TIGHT if m <= 32 else 1e-3)
+    w.free()
+
+
 def test_argmax_bit_exact(dev):
     # index output: bit exact against the oracle's sequential scan, including ties (first wins), values at or
     # below the -1e30 starting value, NaN, infinities, a vocabulary-sized row and an empty one
