@@ -865,8 +865,10 @@ static DecodePlan plan_gemv4(uint32_t n_tiles, uint32_t k_chunks, int force_nt, 
     p.nt = 1;
     if (force_nt == 2 && tiles64 % 2 == 0) p.nt = 2;
     uint32_t tg = tiles64 / p.nt;
+    // eight waves unless half of them would find no chunk: with a shallow K one chunk per wave puts every load
+    // in flight at once (896-deep: 3.6 us with eight waves, 4.2 us with two)
     p.waves = 8;
-    while (p.waves > 1 && k_chunks < p.waves * 2) p.waves /= 2;
+    while (p.waves > 1 && k_chunks <= p.waves / 2) p.waves /= 2;
     // 64 .. 127 tiles with a deep K (4096 -> 4096 is the case): sixteen waves per tile put as many waves in flight
     // as a two-way split-K of eight-wave workgroups would, without its partial sums (5.9 against 6.5 us)
     if (p.waves == 8 && tg >= 64 && tg < 128 && k_chunks >= 32) p.waves = 16;

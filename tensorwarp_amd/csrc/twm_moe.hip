@@ -171,8 +171,8 @@ hipError_t launch_geglu_rows(hipStream_t s, const float *gu, float *out, uint32_
 
 static uint32_t bank_waves(uint32_t k_chunks)
 {
-    uint32_t waves = 16;
-    while (waves > 1 && k_chunks < waves * 2) waves /= 2;
+    uint32_t waves = 8;
+    while (waves > 1 && k_chunks <= waves / 2) waves /= 2;  // as the dense M <= 4 plan: idle waves only below half
     return waves;
 }
 
