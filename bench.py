@@ -391,7 +391,8 @@ def main():
             dev.synchronize()
             mlp_front[label] = round(time_launches(dev, lambda i: gr.replay(), 50) / L * 1e3, 2)
             graphs_done.append(gr)
-        assert np.array_equal(act1.to_host(), act3.to_host()), "fused SwiGLU differs from the three-launch sequence"
+        a1h, a3h = act1.to_host(), act3.to_host()     # same sums, possibly another split order per column
+        assert np.abs(a1h - a3h).max() <= 1e-4 * np.abs(a3h).max(), "fused SwiGLU differs from the three-launch sequence"
         for w in plain + pairedw:
             w.free()
 
