@@ -83,7 +83,8 @@ template <int MT>  // MT = 16-row blocks per workgroup tile (BM = 16 * MT rows)
 __global__ __launch_bounds__(256) void k_prefill(const uint4v *__restrict__ qw, const uint2v *__restrict__ sc,
                                                   const _Float16 *__restrict__ a_any, OutSpec out, uint32_t m_rows,
                                                   uint32_t k, uint32_t n, uint32_t n_tiles, uint32_t k_chunks,
-                                                  uint32_t chunks_per_split, float *__restrict__ partials)
+                                                  uint32_t chunks_per_split, float *__restrict__ partials,
+                                                  uint32_t row_store)
 {
     constexpr int kPfTileHalves = 16 * MT * kPfRowStride;
     constexpr int NV = MT;       // direct-to-LDS load instructions per wave and A tile (16 MT rows / 16)
@@ -255,6 +256,33 @@ __global__ __launch_bounds__(256) void k_prefill(const uint4v *__restrict__ qw, 
     if (kc < nchunks) chunk(S0{}, kc);
 
     // ---- store: lane (c, kb) holds rows 4*kb + r of row block mt, column 16*tile + c ----
+    if (row_store) {
+        // One destination (the output itself or this split's partial sums), rows 16-byte aligned: each wave turns
+        // its 16 x 64 block of a row block through LDS (272-byte rows: the four row groups kb fall on different
+        // banks) so that a lane stores 16 bytes and sixteen lanes cover 256 consecutive bytes of a row, instead
+        // of 64-byte pieces of four rows from 4-byte stores.
+        float *dst = partials ? partials + ((size_t)blockIdx.z * m_rows) * (n_tiles * 16u) : out.seg[0].ptr;
+        const uint32_t ld = partials ? n_tiles * 16u : n;
+        const uint32_t n_lim = partials ? n_tiles * 16u : n;  // a multiple of 4
+        __syncthreads();                                       // every wave is done with the A tiles
+        float *stage = (float *)a_lds + wave * (16 * 68);
+        const uint32_t col = nt0 * 16u + (lane & 15u) * 4u;
+#pragma unroll
+        for (int mt = 0; mt < MT; mt++) {
+#pragma unroll
+            for (int t = 0; t < 4; t++)
+#pragma unroll
+                for (int r = 0; r < 4; r++) stage[(kb * 4 + r) * 68 + t * 16 + c] = acc[mt][t][r];
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const uint32_t row = (lane >> 4) + 4u * i;
+                const float4v v = *(const float4v *)(stage + row * 68 + (lane & 15u) * 4u);
+                const uint32_t om = m0 + mt * 16u + row;
+                if (om < m_rows && col < n_lim) __builtin_nontemporal_store(v, (float4v *)(dst + (size_t)om * ld + col));
+            }
+        }
+        return;
+    }
     if (partials) {
         // split-K: plain [split][row][padded column] partial sums, added up in split order by k_splitk_reduce
         const uint32_t n_ld = n_tiles * 16u;
@@ -275,20 +303,34 @@ __global__ __launch_bounds__(256) void k_prefill(const uint4v *__restrict__ qw, 
     }
     if (out.swiglu) {
         // paired gate/up weight: this wave's tiles 0, 1 are 32 gate columns and tiles 2, 3 the up columns of the
-        // same features, in the same lanes and registers
-        const uint32_t ffn = n >> 1;
+        // same features, in the same lanes and registers.  The 16 x 32 gated block of a row block goes through
+        // LDS like the plain store: a lane stores 16 bytes, eight lanes cover the wave's 128 bytes of a row.
+        const uint32_t ffn = n >> 1;  // a multiple of 32
+        __syncthreads();
+        float *stage = (float *)a_lds + wave * (16 * 36);
+        const uint32_t feat = paired_feature(nt0 * 16u) + (lane & 7u) * 4u;
+        const bool aligned = ((uintptr_t)out.swiglu & 15) == 0;
 #pragma unroll
-        for (int t = 0; t < 2; t++) {
-            if (nt0 + t + 2 >= n_tiles) continue;
-            const uint32_t feat = paired_feature((nt0 + t) * 16u + c);
-            if (feat >= ffn) continue;
+        for (int mt = 0; mt < MT; mt++) {
 #pragma unroll
-            for (int mt = 0; mt < MT; mt++)
+            for (int t = 0; t < 2; t++)
 #pragma unroll
-                for (int r = 0; r < 4; r++) {
-                    uint32_t om = m0 + mt * 16u + kb * 4u + r;
-                    if (om < m_rows) out.swiglu[(size_t)om * ffn + feat] = gated_mul(out.gate_act, acc[mt][t][r], acc[mt][t + 2][r]);
+                for (int r = 0; r < 4; r++)
+                    stage[(kb * 4 + r) * 36 + t * 16 + c] = gated_mul(out.gate_act, acc[mt][t][r], acc[mt][t + 2][r]);
+#pragma unroll
+            for (int i = 0; i < 2; i++) {
+                const uint32_t row = (lane >> 3) + 8u * i;
+                const float4v v = *(const float4v *)(stage + row * 36 + (lane & 7u) * 4u);
+                const uint32_t om = m0 + mt * 16u + row;
+                if (om < m_rows && feat < ffn && nt0 + 3 < n_tiles) {
+                    float *p = out.swiglu + (size_t)om * ffn + feat;
+                    if (aligned) {
+                        __builtin_nontemporal_store(v, (float4v *)p);
+                    } else {
+                        p[0] = v[0]; p[1] = v[1]; p[2] = v[2]; p[3] = v[3];
+                    }
                 }
+            }
         }
         return;
     }
@@ -413,8 +455,14 @@ static hipError_t launch_prefill_t(hipStream_t s, const WeightView &w, const _Fl
     uint32_t cps = (w.k_chunks + splits - 1) / splits;
     splits = (w.k_chunks + cps - 1) / cps;  // no empty split
     dim3 grid((w.n_tiles + 15) / 16, (m + 16 * MT - 1) / (16 * MT), splits);
+    // 16-byte row stores: into the partial sums always (padded width, a multiple of 64); into the output when it
+    // is one plain [M, N] matrix with N a multiple of 4 at a 16-byte aligned address
+    uint32_t row_store = 1;
+    if (splits == 1)
+        row_store = !out.swiglu && out.count == 1 && out.seg[0].start == 0 && out.seg[0].width == w.n && !out.seg[0].bias &&
+                    w.n % 4 == 0 && ((uintptr_t)out.seg[0].ptr & 15) == 0;
     hipLaunchKernelGGL((k_prefill<MT>), grid, dim3(256), lds, s, (const uint4v *)w.qw, (const uint2v *)w.sc, a, out, m, w.k,
-                       w.n, w.n_tiles, w.k_chunks, cps, splits > 1 ? partials : nullptr);
+                       w.n, w.n_tiles, w.k_chunks, cps, splits > 1 ? partials : nullptr, row_store);
     if (splits > 1) return launch_splitk_reduce(s, partials, out, m, w.n, w.n_tiles * 16, splits);
     return hipGetLastError();
 }
