@@ -50,8 +50,26 @@ def test_null_handles_are_rejected_not_crashed():
     assert lib.twm_malloc(None, 16) is None
     assert lib.twm_weight_upload(None, None, None, 64, 64) is None
     assert lib.twm_weight_bytes(None) == 0
+    # the fused stores, the weight cache and the expert banks
+    assert lib.twm_gemm_swiglu(None, None, None, _lib.F16, 1, None, 0) == _lib.INVALID_HANDLE
+    assert lib.twm_gemm_geglu(None, None, None, _lib.F16, 1, None, 0) == _lib.INVALID_HANDLE
+    assert lib.twm_gemm_split_bias(None, None, None, _lib.F16, 1, None, None, None, 1, 0) == _lib.INVALID_HANDLE
+    assert lib.twm_silu_mul(None, None, None, None, 4) == _lib.INVALID_HANDLE
+    assert lib.twm_pair_gate_up(None, None, None, None, None, 64, 64, None, None) == _lib.INVALID_HANDLE
+    assert lib.twm_weight_gate_up(None, None, None, None, None, 64, 64) is None
+    assert lib.twm_weight_is_paired(None) == 0
+    assert lib.twm_weight_blob_bytes(None) == 0
+    assert lib.twm_weight_export(None, None, None, 0) == _lib.INVALID_HANDLE
+    assert lib.twm_weight_import(None, None, 0) is None
+    assert lib.twm_bank_from_device(None, None, None, 0, 0, 64, 64, 1, 0) is None
+    assert lib.twm_bank_bytes(None) == 0
+    assert lib.twm_bank_gemv(None, None, None, _lib.F32, 0, None, 1, 0, None) == _lib.INVALID_HANDLE
+    assert lib.twm_bank_down_axpy(None, None, None, _lib.F32, None, None, 1, None) == _lib.INVALID_HANDLE
+    assert lib.twm_geglu_rows(None, None, 1, 32, 0, None) == _lib.INVALID_HANDLE
+    assert lib.twm_argmax_f32(None, None, 1, 1, None) == _lib.INVALID_HANDLE
     lib.twm_ctx_destroy(None)
     lib.twm_weight_destroy(None)
+    lib.twm_bank_destroy(None)
     lib.twm_graph_destroy(None)
 
 
