@@ -638,6 +638,31 @@ def test_f32_activations_keep_their_precision(dev, m):
     w.free()
 
 
+def test_random_shapes_against_the_oracle(dev):
+    # seeded sweep over ragged shapes: K any multiple of 32, N with and without tile padding, M across the three
+    # kernels, forced and automatic split-K, f16 and f32 activations
+    rng = np.random.default_rng(20250607)
+    for case in range(48):
+        k = 32 * int(rng.integers(1, 40))
+        n = int(rng.choice([1, 7, 15, 16, 17, 63, 64, 65, 100, 129, 200, 333, 512, 600]))
+        m = int(rng.choice([1, 2, 3, 4, 5, 9, 16, 17, 31, 32, 33, 47, 64, 70]))
+        splits = int(rng.choice([0, 0, 1, 2, 3, 5]))
+        a_f32 = bool(rng.integers(0, 2))
+        print("case %d: k=%d n=%d m=%d splits=%d f32=%d" % (case, k, n, m, splits, a_f32), flush=True)
+        packed, scales, a16 = synth(k, n, m, 5000 + case)
+        w = T.MarlinWeight.upload(dev, packed, scales, k, n)
+        got = run_gemm(dev, w, a16, m, n, splits, a_f32)
+        truth = gemm_truth(a16, packed, scales, m, k, n)
+        assert rel_err(got, truth) < (TIGHT if m <= 32 else 1e-3), (case, k, n, m, splits, a_f32)
+        assert np.array_equal(w.dequant_f16().to_host().reshape(-1), O.dequant_f16(packed, scales, k, n).reshape(-1)), case
+        if m == 1:
+            c = T.GpuTensor.from_host(dev, np.full(n, np.nan, np.float32))
+            T.gemm_tw_marlin_m1(dev, T.GpuTensor.from_host(dev, f16_as_f32(a16)), T.GpuTensor.from_host(dev, packed),
+                                T.GpuTensor.from_host(dev, scales, "f16"), c, n, k)
+            assert rel_err(c.to_host(), truth[0]) < TIGHT, (case, "drop-in")
+        w.free()
+
+
 def test_m_larger_than_16_is_tiled_by_the_decode_kernel(dev):
     # with the prefill kernel switched off, any M runs as 16-row blocks of the exact-weight decode kernel
     m, k, n = 70, 256, 128
