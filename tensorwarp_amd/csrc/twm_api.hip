@@ -44,6 +44,7 @@ struct twm_ctx {
     bool capturing;
     int force_nt;         // 0 = heuristic
     int force_waves;      // 0 = heuristic
+    int force_sub;        // M <= 4: 0 = heuristic, 1 = whole 64-column tiles per workgroup, 32 or 16 = the sub-tile kernel
     int force_kernel;     // 0 = heuristic, 1 = 16-column tile kernel, 2 = one-lane-per-column kernel (M <= 4), 3 = streaming kernel (M <= 32)
     int prefill_bm;       // rows of A per prefill workgroup: 0 = choose, 64 or 128
     int prefill_min_m;    // M from which the LDS/MFMA prefill kernel runs instead of 16-row decode blocks
@@ -107,6 +108,7 @@ twm_ctx *twm_ctx_create(int ordinal)
     c->capturing = false;
     c->force_nt = 0;
     c->force_waves = 0;
+    c->force_sub = 0;
     c->force_kernel = 0;
     c->dequant_src = 0;
     c->m1_exact = 0;
@@ -196,6 +198,12 @@ int twm_ctx_set_option(twm_ctx *ctx, const char *key, int value)
         if (value != 0 && value != 1 && value != 2 && value != 4 && value != 8 && value != 16)
             return fail(TWM_SHAPE_ERROR, "twm_ctx_set_option: waves must be 0, 1, 2, 4, 8 or 16");
         ctx->force_waves = value;
+        return TWM_OK;
+    }
+    if (strcmp(key, "sub") == 0) {
+        if (value != 0 && value != 1 && value != 16 && value != 32)
+            return fail(TWM_SHAPE_ERROR, "twm_ctx_set_option: sub must be 0, 1, 16 or 32");
+        ctx->force_sub = value;
         return TWM_OK;
     }
     if (strcmp(key, "prefill_bm") == 0) {
@@ -529,25 +537,44 @@ int twm_gemm_tw_marlin_m1(twm_ctx *ctx, const float *a_dev, const uint8_t *packe
                 "gemv launch");
         return TWM_OK;
     }
-    // the M <= 4 MFMA kernel reading the reference's arrays as they are (activations rounded to f16)
+    // the M <= 4 MFMA kernels reading the reference's arrays as they are (f32 activations as two f16 terms)
     uint32_t n_pad = ((n + 63) / 64) * 64, k_chunks = (k / 32 + kChunkGroups - 1) / kChunkGroups;
-    // On the reference's arrays a wave's four group rows of a chunk are N x 16 bytes apart, and more waves in
-    // flight pay better than on the contiguous copy: sixteen waves per tile and a split-K of up to about one
-    // workgroup per CU, unless the tiles alone fill the GPU (fitted to a sweep over the benchmark shapes).
+    // On the reference's arrays a wave's four group rows of a chunk are N x 16 bytes apart, and many waves in flight
+    // with one pass each pay better than on the contiguous copy: the sub-tile kernel with sixteen waves on 32
+    // columns, or with 16 columns when 64-column tiles number no more than 64; a very deep K is cut in two
+    // (fitted to a sweep over the benchmark shapes; option "sub" = 1 keeps the 64-column kernel).
+    const uint32_t tiles64 = n_pad / 64, passes16 = (k_chunks + 3) / 4;
+    if (ctx->force_sub != 1) {
+        uint32_t sub = tiles64 <= 64 ? 16 : 32, waves = (sub == 16 && passes16 <= 8) ? 8 : 16, sp = 1;
+        if (passes16 > 32) { sub = 32; waves = 16; sp = 2; }
+        if (ctx->force_sub >= 16) {
+            sub = (uint32_t)ctx->force_sub;
+            waves = 8;
+            sp = 1;
+        }
+        if (ctx->force_waves) waves = (uint32_t)ctx->force_waves;
+        if (ctx->m1_splits) sp = (uint32_t)ctx->m1_splits;
+        if (sp > k_chunks) sp = k_chunks;
+        while (sp > 1 && (size_t)sp * n_pad * 4 > ctx->ws_bytes) sp--;
+        if (n_pad / sub > ctx->n_counters) sp = 1;
+        HIP_TRY(launch_gemv4s_ref(ctx->stream, packed_dev, scales_dev, k, n, a_dev, c_dev, ctx->ws, ctx->counters, sub, waves, sp),
+                TWM_DEVICE_ERROR, "sub-tile gemv launch");
+        return TWM_OK;
+    }
     DecodePlan plan;
     plan.lane_col = 1;
     plan.nt = 1;
     plan.waves = 8;
     plan.splits = 1;
-    if (n_pad / 64 < 256) {
+    if (tiles64 < 256) {
         plan.waves = 16;
-        while ((n_pad / 64) * plan.splits * 2 <= 256 && k_chunks >= plan.splits * 2 * 8) plan.splits *= 2;
+        while (tiles64 * plan.splits * 2 <= 256 && k_chunks >= plan.splits * 2 * 8) plan.splits *= 2;
     }
     if (ctx->force_waves) plan.waves = (uint32_t)ctx->force_waves;
     if (ctx->m1_splits) plan.splits = (uint32_t)ctx->m1_splits;
     if (plan.splits > k_chunks) plan.splits = k_chunks;
     while (plan.splits > 1 && (size_t)plan.splits * n_pad * 4 > ctx->ws_bytes) plan.splits--;
-    if (n_pad / 64 > ctx->n_counters) plan.splits = 1;
+    if (tiles64 > ctx->n_counters) plan.splits = 1;
     HIP_TRY(launch_gemv4_ref(ctx->stream, packed_dev, scales_dev, k, n, a_dev, c_dev, ctx->ws, ctx->counters, plan.waves,
                              plan.splits),
             TWM_DEVICE_ERROR, "gemv launch");
@@ -881,6 +908,33 @@ static DecodePlan plan_gemv4(uint32_t n_tiles, uint32_t k_chunks, int force_nt, 
     return p;
 }
 
+// Sub-tile variant of the M <= 4 kernel: 16 or 32 columns per workgroup, each wave one pass (4 or 2 chunks) of
+// them, so that narrow matrices fill the CUs without a cross-workgroup split-K and wide ones run as many
+// short-lived workgroups.  sub = 0: keep the 64-column plan.  Fitted to sweeps over the Qwen2.5-7B, Llama-7B and
+// Qwen2.5-0.5B projections (M = 1, 2, 4; f16 and f32 activations); what it loses on are the activations, which
+// every lane reads 64 / sub times per chunk: four distinct rows, or f32 rows cut into two terms, shift the
+// balance back to wider workgroups.
+struct SubPlan {
+    uint32_t sub, waves;
+};
+static SubPlan plan_gemv4_sub(uint32_t tiles64, uint32_t k_chunks, uint32_t m, bool a_f32)
+{
+    const SubPlan none = {0, 0};
+    if (k_chunks < 16) return none;  // shallow K: nothing to gain over one chunk per wave of the 64-column plan
+    const bool two_pass = a_f32 && m > 2;
+    const uint32_t passes16 = (k_chunks + 3) / 4;
+    const SubPlan narrow16 = {16, passes16 <= 8 ? 8u : 16u};
+    if (tiles64 > 128) {
+        if (two_pass) return none;
+        if (a_f32) return tiles64 >= 1024 ? none : SubPlan{32, 16};
+        if (m > 2) return tiles64 >= 256 ? SubPlan{32, 8} : none;
+        return narrow16;
+    }
+    if (two_pass && passes16 > 16) return k_chunks <= 100 ? SubPlan{32, 8} : none;  // (the looping 16-column variant spills)
+    if (tiles64 > 64) return SubPlan{32, 16};  // 16 columns would leave a second, quarter-full round of workgroups
+    return narrow16;
+}
+
 // Batched-decode streaming kernel (M = 5 .. 32): one workgroup of eight waves per 64 columns and k-range.  K is
 // cut when the column quads alone leave CUs idle, up to about one workgroup per CU, keeping two chunks per
 // wave (one for the 32-row variant, whose chunks cost twice the arithmetic); the partial sums cost a second
@@ -972,7 +1026,23 @@ static int gemm_common(twm_ctx *ctx, const twm_weight *w, const void *a_dev, int
         OutSpec o = gated;   // (the one-lane-per-column kernel takes the gated output as its own argument)
         for (uint32_t s = 0; s < o.count; s++) o.seg[s].ptr += (size_t)m0 * o.seg[s].width;
         const char *a_blk = (const char *)a_dev + (size_t)m0 * a_row_bytes;
-        if (lane_col)
+        SubPlan sub = {0, 0};
+        if (lane_col && ctx->force_sub >= 16) {
+            sub.sub = (uint32_t)ctx->force_sub;
+            sub.waves = ctx->force_waves ? (uint32_t)ctx->force_waves : 8;
+        } else if (lane_col && ctx->force_sub == 0 && !ctx->force_nt && !ctx->force_waves && !splits) {
+            // (an explicit nt, waves or split factor asks for the 64-column kernel's plan)
+            sub = plan_gemv4_sub(n_ld / 64, w->k_chunks, mb, a_dtype == TWM_F32);
+        }
+        if (sub.sub) {
+            uint32_t ssp = splits ? splits : 1;
+            if (ssp > w->k_chunks) ssp = w->k_chunks;
+            while (ssp > 1 && (size_t)ssp * mb * n_ld * 4 > ctx->ws_bytes) ssp--;
+            if (n_ld / sub.sub > ctx->n_counters) ssp = 1;
+            if (swiglu_out) o.swiglu = swiglu_out + (size_t)m0 * (w->n / 2);
+            HIP_TRY(launch_gemv4s(ctx->stream, v, a_blk, a_dtype == TWM_F32, mb, o, ctx->ws, ctx->counters, sub.sub, sub.waves, ssp),
+                    TWM_DEVICE_ERROR, "sub-tile gemv launch");
+        } else if (lane_col)
             HIP_TRY(launch_gemv4(ctx->stream, v, a_blk, a_dtype == TWM_F32, mb, o, ctx->ws, ctx->counters, plan.nt,
                                  plan.waves, plan.splits, swiglu_out ? swiglu_out + (size_t)m0 * (w->n / 2) : nullptr),
                     TWM_DEVICE_ERROR, "gemv launch");

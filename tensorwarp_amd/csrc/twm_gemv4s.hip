@@ -1,0 +1,366 @@
+// Sub-tile variant of the M <= 4 decode kernel: finer workgroups without a cross-workgroup reduction.
+//
+// k_gemv4 gives a workgroup a whole 64-column tile; with 592 tiles on 256 CUs that is 2.3 long-lived
+// workgroups per CU, and a plain read of the same bytes in that decomposition is 1.3 - 1.6 us slower than in
+// many short-lived workgroups.  Here a workgroup owns SUB = 32 or 16 columns of a tile and a wave covers
+// 64 / SUB consecutive k-chunks of them in one pass: lane l = (chunk l / SUB of the pass, column l % SUB).
+// The column-lane copy is read as it is (a sub-tile's 16-byte records of one group are SUB * 16 contiguous
+// bytes).  The 4x4x4 MFMA broadcasts its A block inside groups of 2^CBSZ blocks, so with CBSZ = log2(SUB / 4)
+// every group of SUB lanes takes the activations of its own chunk: one A register holds 2 * SUB of the
+// chunk's 128 k-values (SUB / 4 pieces of eight), 64 / SUB registers the whole chunk.  The MFMA count per
+// byte of weights is unchanged (every lane of every MFMA is a live column).  With 28 chunks and SUB = 32 a
+// workgroup of 14 waves makes exactly one pass: every load of the launch is issued at once.
+//
+// Arithmetic and output as k_gemv4 (crates/kernels/src/quantize.rs:1186-1298).
+#include "twm_gemv4_core.h"
+#include "twm_internal.h"
+#include <cstring>
+
+namespace twm {
+
+namespace {
+
+template <int SUB>
+struct ChunkS {
+    uint4v wq[4];            // this lane's column, its chunk: four groups of 32 nibbles
+    uint2v sc;               // four f16 scales
+    uint4v a[64 / SUB];      // activations: row (lane % SUB) % 4, piece (lane % SUB) / 4 of every 2*SUB-wide slice
+    uint4v a_lo[64 / SUB];   // f32 activations as two passes: the residual terms
+};
+
+template <int SUB, int P>
+__device__ __forceinline__ float4v mfma_sub(half4v a, half4v b, float4v c)
+{
+    constexpr int CBSZ = SUB == 32 ? 3 : 2;
+    return __builtin_amdgcn_mfma_f32_4x4x4f16(a, b, c, CBSZ, P, 0);
+}
+
+__device__ __forceinline__ void gemv4s_store_out(const OutSpec &out, uint32_t m, uint32_t col, float v)
+{
+#pragma unroll
+    for (uint32_t s = 0; s < kMaxSegs; s++) {
+        if (s < out.count) {
+            uint32_t rel = col - out.seg[s].start;
+            if (rel < out.seg[s].width) out.seg[s].ptr[(size_t)m * out.seg[s].width + rel] = out.seg[s].bias ? v + out.seg[s].bias[rel] : v;
+        }
+    }
+}
+
+}  // namespace
+
+// grid: sub-tiles (rounded up to the 8 XCDs) x splits, unfolded like k_gemv4; workgroup = `waves` waves that
+// take the passes (64 / SUB chunks each) of the k-range in turn.
+// REFL: cw is the reference's packed array u8 [G][N][16] and ref_scales its f16 [G][N] (no repack; one row of f32
+// activations): a sub-tile's records of one group are still SUB * 16 contiguous bytes.
+template <int SUB, int RL, bool AF32, bool ONE, bool REFL = false>
+__global__ __launch_bounds__(1024) void k_gemv4s(const char *__restrict__ cw, const void *__restrict__ a_any, OutSpec out,
+                                                  float *__restrict__ ws, unsigned *__restrict__ counters, uint32_t m_rows,
+                                                  uint32_t k, uint32_t n, uint32_t n_pad, uint32_t k_chunks,
+                                                  uint32_t sub_tiles, uint32_t splits, uint32_t cps,
+                                                  const uint16_t *__restrict__ ref_scales = nullptr)
+{
+    static_assert(!REFL || (AF32 && RL == 1), "the reference-layout variant is the M = 1, f32-activation entry point");
+    constexpr int CPP = 64 / SUB;     // chunks per pass
+    constexpr int PIECES = SUB / 4;   // 8-wide k pieces per A register
+    constexpr int TERMS = gemv4_terms<AF32, RL>();
+    extern __shared__ float red[];    // [waves][RL][64]
+    __shared__ int s_last;
+
+    const uint32_t b = blockIdx.x;
+    const uint32_t xcd = b & 7u, jj = b >> 3;
+    const uint32_t sp = jj % splits;
+    const uint32_t st = (jj / splits) * 8u + xcd;
+    if (st >= sub_tiles) return;
+
+    const uint32_t waves = blockDim.x >> 6;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const uint32_t lane = threadIdx.x & 63u;
+    const uint32_t cl = lane % SUB, cg = lane / SUB;          // column in the sub-tile, chunk of the pass
+    const uint32_t tile = st / CPP, part = st % CPP;           // CPP sub-tiles per 64-column tile
+    const uint32_t kc0 = sp * cps;
+    const uint32_t kc1 = (kc0 + cps < k_chunks) ? kc0 + cps : k_chunks;
+    const uint32_t passes = (kc1 - kc0 + CPP - 1) / CPP;
+
+    // Gated store (paired gate_up weight: each 64-column tile is 32 gate columns, then the up columns of the same
+    // features): the workgroup takes SUB / 2 gate columns and their up columns, so that it can write the products.
+    const bool gated = !REFL && out.swiglu != nullptr;
+    auto col_in_tile = [&](uint32_t c) {
+        return gated ? (c / (SUB / 2)) * 32u + part * (SUB / 2) + c % (SUB / 2) : part * SUB + c;
+    };
+    const char *tbase = cw + (size_t)tile * k_chunks * kColBlockBytes;
+    const uint32_t rec_off = col_in_tile(cl) * 16u, sc_off = 4096u + col_in_tile(cl) * 8u;
+    const uint32_t ref_col = st * SUB + cl < n ? st * SUB + cl : n - 1u;  // REFL: columns past n replay the last one
+    const uint32_t ref_groups = k / 32u;
+    const Gemv4Consts dq = make_gemv4_consts();
+
+    uint32_t arow = TERMS == kTermsRowPacked ? (cl & 3u) >> 1 : cl & 3u;
+    if (arow > m_rows - 1) arow = m_rows - 1;
+    const bool lane_is_lo = TERMS == kTermsRowPacked && (cl & 1u) != 0;
+    const uint32_t apiece = (cl >> 2) * 8u;
+
+    float acc[RL];
+#pragma unroll
+    for (int r = 0; r < RL; r++) acc[r] = 0.f;
+
+    auto load_pass = [&](ChunkS<SUB> &r, uint32_t pass) {
+        uint32_t kc = kc0 + pass * CPP + cg;
+        const bool live = kc < kc1;
+        kc = live ? kc : kc1 - 1u;  // a chunk past the k-range replays the last one with scale 0
+        if (REFL) {
+            uint32_t sb[4];
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+                const uint32_t gg = kc * 4u + g;
+                const size_t idx = (size_t)(gg < ref_groups ? gg : ref_groups - 1u) * n + ref_col;
+                r.wq[g] = *(const uint4v *)(cw + idx * 16u);
+                const uint32_t sbits = ref_scales[idx];
+                sb[g] = (live && gg < ref_groups && st * SUB + cl < n) ? sbits : 0u;  // weight exactly 0 otherwise
+            }
+            r.sc = uint2v{sb[0] | (sb[1] << 16), sb[2] | (sb[3] << 16)};
+        } else {
+            const char *blk = tbase + (size_t)kc * kColBlockBytes;
+#pragma unroll
+            for (int g = 0; g < 4; g++) r.wq[g] = *(const uint4v *)(blk + g * 1024u + rec_off);
+            uint2v s = *(const uint2v *)(blk + sc_off);
+            r.sc = live ? s : uint2v{0u, 0u};
+        }
+#pragma unroll
+        for (int j = 0; j < CPP; j++) {
+            uint32_t k0 = kc * 128u + j * (2u * SUB) + apiece;
+            if (k0 > k - 8u) k0 = k - 8u;  // only the zero-padded groups of a last partial chunk get here
+            if (REFL) {
+                // the nibbles are in their natural order there, which the mask-and-magic unpack turns into the k
+                // order (0,4,1,5 | 2,6,3,7) per eight: the activations take the same order
+                const float4 *p = (const float4 *)((const float *)a_any + k0);
+                float4 x = p[0], y = p[1];
+                const float v[8] = {x.x, y.x, x.y, y.y, x.z, y.z, x.w, y.w};
+                split_f32x8(v, r.a[j], r.a_lo[j]);
+#pragma unroll
+                for (int i = 0; i < 4; i++) r.a[j][i] = lane_is_lo ? r.a_lo[j][i] : r.a[j][i];
+            } else if (AF32) {
+                const float4 *p = (const float4 *)((const float *)a_any + (size_t)arow * k + k0);
+                float4 x = p[0], y = p[1];
+                const float v[8] = {x.x, x.y, x.z, x.w, y.x, y.y, y.z, y.w};
+                split_f32x8(v, r.a[j], r.a_lo[j]);
+                if (TERMS == kTermsRowPacked) {
+#pragma unroll
+                    for (int i = 0; i < 4; i++) r.a[j][i] = lane_is_lo ? r.a_lo[j][i] : r.a[j][i];
+                }
+            } else {
+                r.a[j] = *(const uint4v *)((const _Float16 *)a_any + (size_t)arow * k + k0);
+            }
+        }
+    };
+
+    auto compute_pass = [&](const ChunkS<SUB> &r) {
+        union { uint2v u; _Float16 h[4]; } sv;
+        sv.u = r.sc;
+#pragma unroll
+        for (int g = 0; g < 4; g++) {
+            float4v d = {0.f, 0.f, 0.f, 0.f};
+            half4v lo4, hi4;
+            // word W of group g is the 8-wide piece 4g + W of the chunk: register (4g + W) / PIECES, block
+            // (4g + W) % PIECES of the lane group
+#define TWM_SUB_PIECE(W)                                                                   \
+    {                                                                                      \
+        constexpr int PG = 4 * G + W, J = PG / PIECES, ABID = PG % PIECES;                 \
+        union { uint4v u; half4v h[2]; } av, al;                                           \
+        av.u = r.a[J];                                                                     \
+        gemv4_dequant_word(r.wq[G][W], dq, lo4, hi4);                                      \
+        d = mfma_sub<SUB, ABID>(av.h[0], lo4, d);                                          \
+        d = mfma_sub<SUB, ABID>(av.h[1], hi4, d);                                          \
+        if (TERMS == kTermsTwoPasses) {                                                    \
+            al.u = r.a_lo[J];                                                              \
+            d = mfma_sub<SUB, ABID>(al.h[0], lo4, d);                                      \
+            d = mfma_sub<SUB, ABID>(al.h[1], hi4, d);                                      \
+        }                                                                                  \
+    }
+#define TWM_SUB_GROUP(GV)                                                                  \
+    if (g == GV) {                                                                         \
+        constexpr int G = GV;                                                              \
+        TWM_SUB_PIECE(0) TWM_SUB_PIECE(1) TWM_SUB_PIECE(2) TWM_SUB_PIECE(3)                \
+    }
+            TWM_SUB_GROUP(0) TWM_SUB_GROUP(1) TWM_SUB_GROUP(2) TWM_SUB_GROUP(3)
+#undef TWM_SUB_GROUP
+#undef TWM_SUB_PIECE
+            const float s = (float)sv.h[g];
+#pragma unroll
+            for (int rr = 0; rr < RL; rr++) {
+                if (TERMS == kTermsRowPacked) acc[rr] = fmaf(d[2 * rr] + d[2 * rr + 1], s, acc[rr]);
+                else acc[rr] = fmaf(d[rr], s, acc[rr]);
+            }
+        }
+    };
+
+    if (ONE) {  // the launcher saw that no wave has a second pass: one register set, no loop
+        ChunkS<SUB> r0;
+        if (wave < passes) {
+            load_pass(r0, wave);
+            compute_pass(r0);
+        }
+    } else {
+        ChunkS<SUB> r0, r1;
+        uint32_t p = wave;
+        if (p < passes) {
+            load_pass(r0, p);
+            while (true) {
+                uint32_t pn = p + waves;
+                if (pn < passes) load_pass(r1, pn);
+                compute_pass(r0);
+                if (pn >= passes) break;
+                p = pn + waves;
+                if (p < passes) load_pass(r0, p);
+                compute_pass(r1);
+                if (p >= passes) break;
+            }
+        }
+    }
+
+    // ---- sum over the waves and over the chunks of a pass (lane groups) through LDS ----
+#pragma unroll
+    for (int r = 0; r < RL; r++) red[(wave * RL + r) * 64 + lane] = acc[r];
+    __syncthreads();
+
+    const uint32_t threads = blockDim.x;
+    const uint32_t entries = RL * SUB;  // entry e = r * SUB + column
+    const uint32_t pair_entries = RL * (SUB / 2), ffn = n >> 1;  // gated: entry e = r * SUB/2 + feature
+    auto summed = [&](uint32_t r, uint32_t c) {
+        float v = 0.f;
+        for (uint32_t w = 0; w < waves; w++)
+#pragma unroll
+            for (int q = 0; q < CPP; q++) v += red[(w * RL + r) * 64 + q * SUB + c];
+        return v;
+    };
+    auto col_of = [&](uint32_t c) { return REFL ? st * SUB + c : tile * 64u + col_in_tile(c); };
+    if (splits == 1) {
+        if (gated) {
+            for (uint32_t e = threadIdx.x; e < pair_entries; e += threads) {
+                uint32_t i = e % (SUB / 2), r = e / (SUB / 2), feat = tile * 32u + part * (SUB / 2) + i;
+                if (r < m_rows && feat < ffn)
+                    out.swiglu[(size_t)r * ffn + feat] = gated_mul(out.gate_act, summed(r, i), summed(r, SUB / 2 + i));
+            }
+            return;
+        }
+        for (uint32_t e = threadIdx.x; e < entries; e += threads) {
+            uint32_t c = e % SUB, r = e / SUB, on = col_of(c);
+            if (r < m_rows && on < n) gemv4s_store_out(out, r, on, summed(r, c));
+        }
+        return;
+    }
+    // cross-workgroup split-K as in k_gemv4: park the partial, count arrivals, the last one adds in split order
+    for (uint32_t e = threadIdx.x; e < entries; e += threads) {
+        uint32_t c = e % SUB, r = e / SUB, on = col_of(c);
+        if (r < m_rows && on < n)
+            __hip_atomic_store(&ws[((size_t)sp * m_rows + r) * n_pad + on], summed(r, c), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    __builtin_amdgcn_s_waitcnt(0);  // vmcnt(0): this wave's scratch stores have completed
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        unsigned prev = __hip_atomic_fetch_add(&counters[st], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        s_last = (prev == splits - 1);
+    }
+    __syncthreads();
+    if (!s_last) return;
+    auto parked = [&](uint32_t r, uint32_t on) {
+        float v = 0.f;
+        for (uint32_t s = 0; s < splits; s++)
+            v += __hip_atomic_load(&ws[((size_t)s * m_rows + r) * n_pad + on], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        return v;
+    };
+    if (gated) {
+        for (uint32_t e = threadIdx.x; e < pair_entries; e += threads) {
+            uint32_t i = e % (SUB / 2), r = e / (SUB / 2), feat = tile * 32u + part * (SUB / 2) + i;
+            if (r < m_rows && feat < ffn)
+                out.swiglu[(size_t)r * ffn + feat] = gated_mul(out.gate_act, parked(r, col_of(i)), parked(r, col_of(SUB / 2 + i)));
+        }
+    } else {
+        for (uint32_t e = threadIdx.x; e < entries; e += threads) {
+            uint32_t c = e % SUB, r = e / SUB, on = col_of(c);
+            if (r < m_rows && on < n) gemv4s_store_out(out, r, on, parked(r, on));
+        }
+    }
+    if (threadIdx.x == 0) __hip_atomic_store(&counters[st], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+template <int SUB, int RL>
+static hipError_t launch_gemv4s_t(hipStream_t s, const WeightView &w, const void *a, bool a_f32, uint32_t m,
+                                  const OutSpec &out, float *ws, unsigned *counters, uint32_t waves, uint32_t splits)
+{
+    uint32_t n_pad = w.n_tiles * kTileN;  // whole 64-column tiles
+    uint32_t sub_tiles = n_pad / SUB;
+    uint32_t cps = (w.k_chunks + splits - 1) / splits;
+    splits = (w.k_chunks + cps - 1) / cps;
+    uint32_t blocks = ((sub_tiles + 7) / 8) * 8 * splits;
+    size_t lds = (size_t)waves * RL * 64 * sizeof(float);
+    const bool one = (cps + 64 / SUB - 1) / (64 / SUB) <= waves;
+#define TWM_S_LAUNCH(AF, ONEV)                                                                                          \
+    hipLaunchKernelGGL((k_gemv4s<SUB, RL, AF, ONEV>), dim3(blocks), dim3(waves * 64), lds, s, (const char *)w.cq, a, out, \
+                       ws, counters, m, w.k, w.n, n_pad, w.k_chunks, sub_tiles, splits, cps)
+    if (a_f32) {
+        if (one) TWM_S_LAUNCH(true, true);
+        else TWM_S_LAUNCH(true, false);
+    } else {
+        if (one) TWM_S_LAUNCH(false, true);
+        else TWM_S_LAUNCH(false, false);
+    }
+#undef TWM_S_LAUNCH
+    return hipGetLastError();
+}
+
+// sub = 32 or 16 columns per workgroup; waves 1 .. 16; out.swiglu set: the gated store of a paired weight.
+hipError_t launch_gemv4s(hipStream_t s, const WeightView &w, const void *a, bool a_f32, uint32_t m, const OutSpec &out,
+                         float *ws, unsigned *counters, uint32_t sub, uint32_t waves, uint32_t splits)
+{
+    if (m == 0 || w.n == 0) return hipSuccess;
+    if (m > 4 || splits == 0 || !w.cq) return hipErrorInvalidValue;
+    if (out.swiglu && w.n % 64 != 0) return hipErrorInvalidValue;
+    if (waves < 1 || waves > 16) return hipErrorInvalidValue;
+    if (sub != 32 && sub != 16) return hipErrorInvalidValue;
+#define TWM_S_CASE(SUBV)                                                                                       \
+    if (sub == SUBV) {                                                                                         \
+        if (m == 1) return launch_gemv4s_t<SUBV, 1>(s, w, a, a_f32, m, out, ws, counters, waves, splits);      \
+        if (m == 2) return launch_gemv4s_t<SUBV, 2>(s, w, a, a_f32, m, out, ws, counters, waves, splits);      \
+        return launch_gemv4s_t<SUBV, 4>(s, w, a, a_f32, m, out, ws, counters, waves, splits);                  \
+    }
+    TWM_S_CASE(32)
+    TWM_S_CASE(16)
+#undef TWM_S_CASE
+    return hipErrorInvalidValue;
+}
+
+// M = 1 on the reference's arrays (no repack), f32 activations.
+hipError_t launch_gemv4s_ref(hipStream_t s, const uint8_t *packed, const uint16_t *scales, uint32_t k, uint32_t n,
+                             const float *a, float *c, float *ws, unsigned *counters, uint32_t sub, uint32_t waves,
+                             uint32_t splits)
+{
+    if (n == 0) return hipSuccess;
+    if (k == 0 || k % 32 != 0 || splits == 0) return hipErrorInvalidValue;
+    if (waves < 1 || waves > 16 || (sub != 32 && sub != 16)) return hipErrorInvalidValue;
+    const uint32_t n_pad = ((n + 63) / 64) * 64, sub_tiles = n_pad / sub;
+    const uint32_t k_chunks = (k / 32 + 3) / 4;
+    const uint32_t cps = (k_chunks + splits - 1) / splits;
+    splits = (k_chunks + cps - 1) / cps;
+    const uint32_t blocks = ((sub_tiles + 7) / 8) * 8 * splits;
+    const size_t lds = (size_t)waves * 64 * sizeof(float);
+    const bool one = (cps + 64 / sub - 1) / (64 / sub) <= waves;
+    OutSpec out;
+    memset(&out, 0, sizeof out);
+    out.count = 1;
+    out.seg[0].ptr = c;
+    out.seg[0].start = 0;
+    out.seg[0].width = n;
+#define TWM_S_REF(SUBV, ONEV)                                                                                          \
+    hipLaunchKernelGGL((k_gemv4s<SUBV, 1, true, ONEV, true>), dim3(blocks), dim3(waves * 64), lds, s, (const char *)packed, \
+                       (const void *)a, out, ws, counters, 1u, k, n, n_pad, k_chunks, sub_tiles, splits, cps, scales)
+    if (sub == 32) {
+        if (one) TWM_S_REF(32, true);
+        else TWM_S_REF(32, false);
+    } else {
+        if (one) TWM_S_REF(16, true);
+        else TWM_S_REF(16, false);
+    }
+#undef TWM_S_REF
+    return hipGetLastError();
+}
+
+}  // namespace twm

@@ -101,6 +101,11 @@ hipError_t launch_repack_col(hipStream_t s, const uint8_t *packed, const uint16_
 hipError_t launch_weight_dequant_f16_col(hipStream_t s, const WeightView &w, uint16_t *out_kn);
 // swiglu_out != nullptr (the weight in the paired gate_up column order, N = 2*ffn a multiple of 64): instead
 // of the N columns, write silu(gate) * up of every feature to swiglu_out[m][ffn]; `out` is ignored.
+hipError_t launch_gemv4s(hipStream_t s, const WeightView &w, const void *a, bool a_f32, uint32_t m, const OutSpec &out,
+                         float *ws, unsigned *counters, uint32_t sub, uint32_t waves, uint32_t splits);
+hipError_t launch_gemv4s_ref(hipStream_t s, const uint8_t *packed, const uint16_t *scales, uint32_t k, uint32_t n,
+                             const float *a, float *c, float *ws, unsigned *counters, uint32_t sub, uint32_t waves,
+                             uint32_t splits);
 hipError_t launch_gemv4(hipStream_t s, const WeightView &w, const void *a, bool a_f32, uint32_t m, const OutSpec &out,
                         float *ws, unsigned *counters, uint32_t nt, uint32_t waves, uint32_t splits,
                         float *swiglu_out = nullptr);
