@@ -1236,7 +1236,8 @@ int twm_bank_gemv(twm_ctx *ctx, const twm_bank *b, const void *a_dev, int a_dtyp
     // every slot's row must keep the 16-byte alignment of the loads
     if ((a_slot_stride * (a_dtype == TWM_F32 ? 4u : 2u)) % 16u != 0)
         return fail(TWM_SHAPE_ERROR, "twm_bank_gemv: the activation stride must keep rows 16-byte aligned");
-    HIP_TRY(launch_bank_gemv(ctx->stream, bank_view(b), a_dev, a_dtype == TWM_F32, a_slot_stride, topk_ids_dev, top_k, act, out_dev),
+    HIP_TRY(launch_bank_gemv(ctx->stream, bank_view(b), a_dev, a_dtype == TWM_F32, a_slot_stride, topk_ids_dev, top_k, act, out_dev,
+                             ctx->force_sub, ctx->force_waves),
             TWM_DEVICE_ERROR, "bank gemv launch");
     return TWM_OK;
 }
@@ -1250,7 +1251,8 @@ int twm_bank_down_axpy(twm_ctx *ctx, const twm_bank *b, const void *a_all_dev, i
     if (!topk_ids_dev || !topk_weights_dev || !acc_dev) return fail(TWM_INVALID_HANDLE, "twm_bank_down_axpy: null pointer");
     if ((b->k * (a_dtype == TWM_F32 ? 4u : 2u)) % 16u != 0)
         return fail(TWM_SHAPE_ERROR, "twm_bank_down_axpy: K must keep the activation rows 16-byte aligned");
-    HIP_TRY(launch_bank_down_axpy(ctx->stream, bank_view(b), a_all_dev, a_dtype == TWM_F32, topk_ids_dev, topk_weights_dev, top_k, acc_dev),
+    HIP_TRY(launch_bank_down_axpy(ctx->stream, bank_view(b), a_all_dev, a_dtype == TWM_F32, topk_ids_dev, topk_weights_dev, top_k, acc_dev,
+                                  ctx->force_sub, ctx->force_waves),
             TWM_DEVICE_ERROR, "bank down_axpy launch");
     return TWM_OK;
 }

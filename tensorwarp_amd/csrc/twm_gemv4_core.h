@@ -1,6 +1,6 @@
 // Building blocks of the one-lane-per-column GEMV (M <= 4): nibble unpack, the chunk's register set, its
-// loads and its 32 chained 4x4x4 MFMAs.  Shared by the dense kernel (twm_gemv4.hip) and the expert-bank
-// kernels (twm_moe.hip); everything is force-inlined.
+// loads and its 32 chained 4x4x4 MFMAs, in the 64-column form (twm_gemv4.hip) and the sub-tile form
+// (twm_gemv4s.hip, twm_moe.hip); everything is force-inlined.
 #pragma once
 #include "twm_device.h"
 
@@ -182,6 +182,138 @@ __device__ __forceinline__ void gemv4_compute_chunk(const Chunk4<NT> &r, const G
                 else acc[t][rr] = fmaf(d[rr], s, acc[t][rr]);
             }
         }
+    }
+}
+
+// ---- sub-tile form: a wave covers 64 / SUB consecutive chunks of SUB columns in one pass ------------------
+// Lane l = (chunk l / SUB of the pass, column l % SUB).  With CBSZ = log2(SUB / 4) the MFMA broadcasts an A block
+// inside groups of SUB lanes only, so every lane group takes the activations of its own chunk: one A register
+// holds 2 * SUB of the chunk's 128 k-values (SUB / 4 pieces of eight), 64 / SUB registers the whole chunk.
+template <int SUB>
+struct ChunkS {
+    uint4v wq[4];            // this lane's column, its chunk: four groups of 32 nibbles
+    uint2v sc;               // four f16 scales
+    uint4v a[64 / SUB];      // activations: row (lane % SUB) % 4, piece (lane % SUB) / 4 of every 2*SUB-wide slice
+    uint4v a_lo[64 / SUB];   // f32 activations as two passes: the residual terms
+};
+
+template <int SUB, int P>
+__device__ __forceinline__ float4v mfma_sub(half4v a, half4v b, float4v c)
+{
+    static_assert(SUB == 32 || SUB == 16, "sub-tiles are 32 or 16 columns wide");
+    constexpr int CBSZ = SUB == 32 ? 3 : 2;
+    return __builtin_amdgcn_mfma_f32_4x4x4f16(a, b, c, CBSZ, P, 0);
+}
+
+// The lane's activations of chunk kc: 64 / SUB pieces of eight, row arow (term modes as gemv4_load_chunk).
+// ref_order: the weights' nibbles are in the reference's natural order, which the mask-and-magic unpack turns
+// into the k order (0,4,1,5 | 2,6,3,7) per eight; the (f32) activations take the same order.
+template <int SUB, bool AF32, int TERMS, bool REF_ORDER = false>
+__device__ __forceinline__ void gemv4s_load_a(ChunkS<SUB> &r, const void *a_any, uint32_t arow, uint32_t kc, uint32_t cl,
+                                              uint32_t k, bool lane_is_lo)
+{
+#pragma unroll
+    for (int j = 0; j < 64 / SUB; j++) {
+        uint32_t k0 = kc * 128u + j * (2u * SUB) + (cl >> 2) * 8u;
+        if (k0 > k - 8u) k0 = k - 8u;  // only the zero-padded groups of a last partial chunk get here
+        if (AF32) {
+            const float4 *p = (const float4 *)((const float *)a_any + (size_t)arow * k + k0);
+            float4 x = p[0], y = p[1];
+            const float v[8] = {x.x, REF_ORDER ? y.x : x.y, REF_ORDER ? x.y : x.z, REF_ORDER ? y.y : x.w,
+                                REF_ORDER ? x.z : y.x, REF_ORDER ? y.z : y.y, REF_ORDER ? x.w : y.z, y.w};
+            split_f32x8(v, r.a[j], r.a_lo[j]);
+            if (TERMS == kTermsRowPacked) {
+#pragma unroll
+                for (int i = 0; i < 4; i++) r.a[j][i] = lane_is_lo ? r.a_lo[j][i] : r.a[j][i];
+            }
+        } else {
+            r.a[j] = *(const uint4v *)((const _Float16 *)a_any + (size_t)arow * k + k0);
+        }
+    }
+}
+
+// The lane's weights from the column-lane copy: blk = the block of the lane's chunk, col = column in the
+// 64-column tile; live = false zeroes the scales (a chunk past the k-range replays a valid one as zeros).
+template <int SUB>
+__device__ __forceinline__ void gemv4s_load_w(ChunkS<SUB> &r, const char *blk, uint32_t col, bool live)
+{
+#pragma unroll
+    for (int g = 0; g < 4; g++) r.wq[g] = *(const uint4v *)(blk + g * 1024u + col * 16u);
+    uint2v s = *(const uint2v *)(blk + 4096u + col * 8u);
+    r.sc = live ? s : uint2v{0u, 0u};
+}
+
+// acc[row] += f32(scale) * (sum over the group of A * (q - 8)) for the four groups of the lane's chunk
+template <int SUB, int RL, int TERMS>
+__device__ __forceinline__ void gemv4s_compute(const ChunkS<SUB> &r, const Gemv4Consts &dq, float (&acc)[RL])
+{
+    constexpr int PIECES = SUB / 4;  // 8-wide k pieces per A register
+    static_assert(TERMS != kTermsRowPacked || RL <= 2, "row-packed terms hold at most two rows");
+    union { uint2v u; _Float16 h[4]; } sv;
+    sv.u = r.sc;
+#pragma unroll
+    for (int g = 0; g < 4; g++) {
+        float4v d = {0.f, 0.f, 0.f, 0.f};
+        half4v lo4, hi4;
+        // word W of group g is the 8-wide piece 4g + W of the chunk: register (4g + W) / PIECES, block
+        // (4g + W) % PIECES of the lane group
+#define TWM_SUB_PIECE(W)                                                                   \
+    {                                                                                      \
+        constexpr int PG = 4 * G + W, J = PG / PIECES, ABID = PG % PIECES;                 \
+        union { uint4v u; half4v h[2]; } av, al;                                           \
+        av.u = r.a[J];                                                                     \
+        gemv4_dequant_word(r.wq[G][W], dq, lo4, hi4);                                      \
+        d = mfma_sub<SUB, ABID>(av.h[0], lo4, d);                                          \
+        d = mfma_sub<SUB, ABID>(av.h[1], hi4, d);                                          \
+        if (TERMS == kTermsTwoPasses) {                                                    \
+            al.u = r.a_lo[J];                                                              \
+            d = mfma_sub<SUB, ABID>(al.h[0], lo4, d);                                      \
+            d = mfma_sub<SUB, ABID>(al.h[1], hi4, d);                                      \
+        }                                                                                  \
+    }
+#define TWM_SUB_GROUP(GV)                                                                  \
+    if (g == GV) {                                                                         \
+        constexpr int G = GV;                                                              \
+        TWM_SUB_PIECE(0) TWM_SUB_PIECE(1) TWM_SUB_PIECE(2) TWM_SUB_PIECE(3)                \
+    }
+        TWM_SUB_GROUP(0) TWM_SUB_GROUP(1) TWM_SUB_GROUP(2) TWM_SUB_GROUP(3)
+#undef TWM_SUB_GROUP
+#undef TWM_SUB_PIECE
+        const float s = (float)sv.h[g];
+#pragma unroll
+        for (int rr = 0; rr < RL; rr++) {
+            if (TERMS == kTermsRowPacked) acc[rr] = fmaf(d[2 * rr] + d[2 * rr + 1], s, acc[rr]);
+            else acc[rr] = fmaf(d[rr], s, acc[rr]);
+        }
+    }
+}
+
+// The passes first, first + stride, ... < passes with two register sets: the next pass's loads are in flight
+// while this one is unpacked.  ONE: the caller knows that no wave has a second pass.
+template <int SUB, bool ONE, class Load, class Compute>
+__device__ __forceinline__ void gemv4s_run_passes(uint32_t first, uint32_t stride, uint32_t passes, Load load, Compute compute)
+{
+    if (ONE) {
+        ChunkS<SUB> r0;
+        if (first < passes) {
+            load(r0, first);
+            compute(r0);
+        }
+        return;
+    }
+    ChunkS<SUB> r0, r1;
+    uint32_t p = first;
+    if (p >= passes) return;
+    load(r0, p);
+    while (true) {
+        uint32_t pn = p + stride;
+        if (pn < passes) load(r1, pn);
+        compute(r0);
+        if (pn >= passes) break;
+        p = pn + stride;
+        if (p < passes) load(r0, p);
+        compute(r1);
+        if (p >= passes) break;
     }
 }
 

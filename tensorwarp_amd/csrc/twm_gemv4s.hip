@@ -20,21 +20,6 @@ namespace twm {
 
 namespace {
 
-template <int SUB>
-struct ChunkS {
-    uint4v wq[4];            // this lane's column, its chunk: four groups of 32 nibbles
-    uint2v sc;               // four f16 scales
-    uint4v a[64 / SUB];      // activations: row (lane % SUB) % 4, piece (lane % SUB) / 4 of every 2*SUB-wide slice
-    uint4v a_lo[64 / SUB];   // f32 activations as two passes: the residual terms
-};
-
-template <int SUB, int P>
-__device__ __forceinline__ float4v mfma_sub(half4v a, half4v b, float4v c)
-{
-    constexpr int CBSZ = SUB == 32 ? 3 : 2;
-    return __builtin_amdgcn_mfma_f32_4x4x4f16(a, b, c, CBSZ, P, 0);
-}
-
 __device__ __forceinline__ void gemv4s_store_out(const OutSpec &out, uint32_t m, uint32_t col, float v)
 {
 #pragma unroll
@@ -61,7 +46,6 @@ __global__ __launch_bounds__(1024) void k_gemv4s(const char *__restrict__ cw, co
 {
     static_assert(!REFL || (AF32 && RL == 1), "the reference-layout variant is the M = 1, f32-activation entry point");
     constexpr int CPP = 64 / SUB;     // chunks per pass
-    constexpr int PIECES = SUB / 4;   // 8-wide k pieces per A register
     constexpr int TERMS = gemv4_terms<AF32, RL>();
     extern __shared__ float red[];    // [waves][RL][64]
     __shared__ int s_last;
@@ -88,7 +72,6 @@ __global__ __launch_bounds__(1024) void k_gemv4s(const char *__restrict__ cw, co
         return gated ? (c / (SUB / 2)) * 32u + part * (SUB / 2) + c % (SUB / 2) : part * SUB + c;
     };
     const char *tbase = cw + (size_t)tile * k_chunks * kColBlockBytes;
-    const uint32_t rec_off = col_in_tile(cl) * 16u, sc_off = 4096u + col_in_tile(cl) * 8u;
     const uint32_t ref_col = st * SUB + cl < n ? st * SUB + cl : n - 1u;  // REFL: columns past n replay the last one
     const uint32_t ref_groups = k / 32u;
     const Gemv4Consts dq = make_gemv4_consts();
@@ -96,7 +79,6 @@ __global__ __launch_bounds__(1024) void k_gemv4s(const char *__restrict__ cw, co
     uint32_t arow = TERMS == kTermsRowPacked ? (cl & 3u) >> 1 : cl & 3u;
     if (arow > m_rows - 1) arow = m_rows - 1;
     const bool lane_is_lo = TERMS == kTermsRowPacked && (cl & 1u) != 0;
-    const uint32_t apiece = (cl >> 2) * 8u;
 
     float acc[RL];
 #pragma unroll
@@ -118,103 +100,13 @@ __global__ __launch_bounds__(1024) void k_gemv4s(const char *__restrict__ cw, co
             }
             r.sc = uint2v{sb[0] | (sb[1] << 16), sb[2] | (sb[3] << 16)};
         } else {
-            const char *blk = tbase + (size_t)kc * kColBlockBytes;
-#pragma unroll
-            for (int g = 0; g < 4; g++) r.wq[g] = *(const uint4v *)(blk + g * 1024u + rec_off);
-            uint2v s = *(const uint2v *)(blk + sc_off);
-            r.sc = live ? s : uint2v{0u, 0u};
+            gemv4s_load_w<SUB>(r, tbase + (size_t)kc * kColBlockBytes, col_in_tile(cl), live);
         }
-#pragma unroll
-        for (int j = 0; j < CPP; j++) {
-            uint32_t k0 = kc * 128u + j * (2u * SUB) + apiece;
-            if (k0 > k - 8u) k0 = k - 8u;  // only the zero-padded groups of a last partial chunk get here
-            if (REFL) {
-                // the nibbles are in their natural order there, which the mask-and-magic unpack turns into the k
-                // order (0,4,1,5 | 2,6,3,7) per eight: the activations take the same order
-                const float4 *p = (const float4 *)((const float *)a_any + k0);
-                float4 x = p[0], y = p[1];
-                const float v[8] = {x.x, y.x, x.y, y.y, x.z, y.z, x.w, y.w};
-                split_f32x8(v, r.a[j], r.a_lo[j]);
-#pragma unroll
-                for (int i = 0; i < 4; i++) r.a[j][i] = lane_is_lo ? r.a_lo[j][i] : r.a[j][i];
-            } else if (AF32) {
-                const float4 *p = (const float4 *)((const float *)a_any + (size_t)arow * k + k0);
-                float4 x = p[0], y = p[1];
-                const float v[8] = {x.x, x.y, x.z, x.w, y.x, y.y, y.z, y.w};
-                split_f32x8(v, r.a[j], r.a_lo[j]);
-                if (TERMS == kTermsRowPacked) {
-#pragma unroll
-                    for (int i = 0; i < 4; i++) r.a[j][i] = lane_is_lo ? r.a_lo[j][i] : r.a[j][i];
-                }
-            } else {
-                r.a[j] = *(const uint4v *)((const _Float16 *)a_any + (size_t)arow * k + k0);
-            }
-        }
+        gemv4s_load_a<SUB, AF32, TERMS, REFL>(r, a_any, arow, kc, cl, k, lane_is_lo);
     };
-
-    auto compute_pass = [&](const ChunkS<SUB> &r) {
-        union { uint2v u; _Float16 h[4]; } sv;
-        sv.u = r.sc;
-#pragma unroll
-        for (int g = 0; g < 4; g++) {
-            float4v d = {0.f, 0.f, 0.f, 0.f};
-            half4v lo4, hi4;
-            // word W of group g is the 8-wide piece 4g + W of the chunk: register (4g + W) / PIECES, block
-            // (4g + W) % PIECES of the lane group
-#define TWM_SUB_PIECE(W)                                                                   \
-    {                                                                                      \
-        constexpr int PG = 4 * G + W, J = PG / PIECES, ABID = PG % PIECES;                 \
-        union { uint4v u; half4v h[2]; } av, al;                                           \
-        av.u = r.a[J];                                                                     \
-        gemv4_dequant_word(r.wq[G][W], dq, lo4, hi4);                                      \
-        d = mfma_sub<SUB, ABID>(av.h[0], lo4, d);                                          \
-        d = mfma_sub<SUB, ABID>(av.h[1], hi4, d);                                          \
-        if (TERMS == kTermsTwoPasses) {                                                    \
-            al.u = r.a_lo[J];                                                              \
-            d = mfma_sub<SUB, ABID>(al.h[0], lo4, d);                                      \
-            d = mfma_sub<SUB, ABID>(al.h[1], hi4, d);                                      \
-        }                                                                                  \
-    }
-#define TWM_SUB_GROUP(GV)                                                                  \
-    if (g == GV) {                                                                         \
-        constexpr int G = GV;                                                              \
-        TWM_SUB_PIECE(0) TWM_SUB_PIECE(1) TWM_SUB_PIECE(2) TWM_SUB_PIECE(3)                \
-    }
-            TWM_SUB_GROUP(0) TWM_SUB_GROUP(1) TWM_SUB_GROUP(2) TWM_SUB_GROUP(3)
-#undef TWM_SUB_GROUP
-#undef TWM_SUB_PIECE
-            const float s = (float)sv.h[g];
-#pragma unroll
-            for (int rr = 0; rr < RL; rr++) {
-                if (TERMS == kTermsRowPacked) acc[rr] = fmaf(d[2 * rr] + d[2 * rr + 1], s, acc[rr]);
-                else acc[rr] = fmaf(d[rr], s, acc[rr]);
-            }
-        }
-    };
-
-    if (ONE) {  // the launcher saw that no wave has a second pass: one register set, no loop
-        ChunkS<SUB> r0;
-        if (wave < passes) {
-            load_pass(r0, wave);
-            compute_pass(r0);
-        }
-    } else {
-        ChunkS<SUB> r0, r1;
-        uint32_t p = wave;
-        if (p < passes) {
-            load_pass(r0, p);
-            while (true) {
-                uint32_t pn = p + waves;
-                if (pn < passes) load_pass(r1, pn);
-                compute_pass(r0);
-                if (pn >= passes) break;
-                p = pn + waves;
-                if (p < passes) load_pass(r0, p);
-                compute_pass(r1);
-                if (p >= passes) break;
-            }
-        }
-    }
+    auto compute_pass = [&](const ChunkS<SUB> &r) { gemv4s_compute<SUB, RL, TERMS>(r, dq, acc); };
+    // (ONE: the launcher saw that no wave has a second pass: one register set, no loop)
+    gemv4s_run_passes<SUB, ONE>(wave, waves, passes, load_pass, compute_pass);
 
     // ---- sum over the waves and over the chunks of a pass (lane groups) through LDS ----
 #pragma unroll

@@ -122,9 +122,9 @@ hipError_t launch_stream(hipStream_t s, const WeightView &w, const void *a, bool
 hipError_t launch_geglu_rows(hipStream_t s, const float *gu, float *out, uint32_t dim, uint32_t batch, bool paired);
 // act: 0 out[slot][n]; 1 gelu_tanh(gate) * up, 2 silu(gate) * up into out[slot][n/2] (paired bank)
 hipError_t launch_bank_gemv(hipStream_t s, const BankView &b, const void *a, bool a_f32, uint32_t a_slot_stride,
-                            const float *ids, uint32_t slots, int act, float *out);
+                            const float *ids, uint32_t slots, int act, float *out, int force_sub = 0, int force_waves = 0);
 hipError_t launch_bank_down_axpy(hipStream_t s, const BankView &b, const void *a_all, bool a_f32, const float *ids,
-                                 const float *weights, uint32_t slots, float *accum);
+                                 const float *weights, uint32_t slots, float *accum, int force_sub = 0, int force_waves = 0);
 hipError_t launch_decode(hipStream_t s, const WeightView &w, const void *a, bool a_f32, uint32_t m, const OutSpec &out,
                          float *ws, unsigned *counters, DecodePlan plan);
 

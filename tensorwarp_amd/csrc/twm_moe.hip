@@ -28,118 +28,120 @@ __device__ __forceinline__ uint32_t expert_of(float id, uint32_t experts)
     return (id >= 0.f && id < (float)experts) ? (uint32_t)id : experts;
 }
 
-// This wave's chunks first, first + stride, ... of one 64-column tile with three register sets: for the short
-// K loops of expert matrices (two or three chunks per wave) every load is in flight before the first unpack.
-template <bool AF32>
-__device__ __forceinline__ void bank_accumulate(const char *tile_base, const void *a_row, uint32_t first, uint32_t stride,
-                                                uint32_t k_chunks, uint32_t k, uint32_t lane, float (&acc)[1][1])
-{
-    const char *wbase[1] = {tile_base};
-    const uint32_t lane16 = lane * 16u, lane8 = 4096u + lane * 8u, apiece = (lane >> 2) * 8u;
-    const Gemv4Consts dq = make_gemv4_consts();
-    constexpr int TERMS = gemv4_terms<AF32, 1>();   // one row: f32 activations as two row-packed terms
-    const bool is_lo = (lane & 1u) != 0;
-    Chunk4<1> r0, r1, r2;
-    uint32_t c0 = first, c1 = first + stride, c2 = first + 2u * stride;
-    if (c0 < k_chunks) gemv4_load_chunk<1, AF32, TERMS>(r0, wbase, c0, lane16, lane8, a_row, 0, apiece, k, is_lo);
-    if (c1 < k_chunks) gemv4_load_chunk<1, AF32, TERMS>(r1, wbase, c1, lane16, lane8, a_row, 0, apiece, k, is_lo);
-    if (c2 < k_chunks) gemv4_load_chunk<1, AF32, TERMS>(r2, wbase, c2, lane16, lane8, a_row, 0, apiece, k, is_lo);
-    for (;;) {
-        if (c0 >= k_chunks) break;
-        gemv4_compute_chunk<1, 1, TERMS>(r0, dq, acc);
-        c0 += 3u * stride;
-        if (c0 < k_chunks) gemv4_load_chunk<1, AF32, TERMS>(r0, wbase, c0, lane16, lane8, a_row, 0, apiece, k, is_lo);
-        if (c1 >= k_chunks) break;
-        gemv4_compute_chunk<1, 1, TERMS>(r1, dq, acc);
-        c1 += 3u * stride;
-        if (c1 < k_chunks) gemv4_load_chunk<1, AF32, TERMS>(r1, wbase, c1, lane16, lane8, a_row, 0, apiece, k, is_lo);
-        if (c2 >= k_chunks) break;
-        gemv4_compute_chunk<1, 1, TERMS>(r2, dq, acc);
-        c2 += 3u * stride;
-        if (c2 < k_chunks) gemv4_load_chunk<1, AF32, TERMS>(r2, wbase, c2, lane16, lane8, a_row, 0, apiece, k, is_lo);
-    }
-}
+// Both kernels work on sub-tiles of SUB = 16 or 32 columns (see twm_gemv4_core.h): a wave covers 64 / SUB
+// consecutive chunks of them in one pass, so that the short K of an expert matrix (a few chunks) still gives
+// every wave of a workgroup one pass and the launch many workgroups.
 
-// Workgroup = `waves` waves on one 64-column tile of one slot's expert; wave w takes chunks w, w + waves, ...
-// grid = (tiles64 rounded up to the 8 XCDs, slots).  ACT 0: out[slot][n]; 1 / 2: paired bank,
+// Workgroup = `waves` waves on one sub-tile of one slot's expert; wave w takes passes w, w + waves, ...
+// grid = (sub-tiles, slots).  ACT 0: out[slot][n]; 1 / 2: paired bank (each 64-column tile is 32 gate columns,
+// then the up columns of the same features; the workgroup takes SUB / 2 of each),
 // out[slot][n/2] = gelu_tanh / silu (gate) * up.
-template <bool AF32, int ACT>
+template <int SUB, bool AF32, int ACT, bool ONE>
 __global__ __launch_bounds__(1024) void k_bank_gemv(const char *__restrict__ bank, size_t expert_bytes, uint32_t experts,
                                                      const void *__restrict__ a_any, uint32_t a_slot_stride,
                                                      const float *__restrict__ ids, float *__restrict__ out,
-                                                     uint32_t k, uint32_t n, uint32_t k_chunks, uint32_t tiles64)
+                                                     uint32_t k, uint32_t n, uint32_t k_chunks, uint32_t sub_tiles)
 {
+    constexpr int CPP = 64 / SUB;
+    constexpr int TERMS = gemv4_terms<AF32, 1>();   // one row: f32 activations as two row-packed terms
     extern __shared__ float red[];  // [waves][64]
-    const uint32_t tile = blockIdx.x, slot = blockIdx.y;
-    if (tile >= tiles64) return;
+    const uint32_t st = blockIdx.x, slot = blockIdx.y;
+    if (st >= sub_tiles) return;
     const uint32_t waves = blockDim.x >> 6;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const uint32_t lane = threadIdx.x & 63u;
+    const uint32_t lane = threadIdx.x & 63u, cl = lane % SUB, cg = lane / SUB;
+    const uint32_t tile = st / CPP, part = st % CPP;
     const uint32_t eid = __builtin_amdgcn_readfirstlane(expert_of(ids[slot], experts));
+    const uint32_t col = ACT ? (cl / (SUB / 2)) * 32u + part * (SUB / 2) + cl % (SUB / 2) : part * SUB + cl;
+    const uint32_t passes = (k_chunks + CPP - 1) / CPP;
 
-    float acc[1][1] = {{0.f}};
-    if (eid < experts)
-        bank_accumulate<AF32>(bank + (size_t)eid * expert_bytes + (size_t)tile * k_chunks * kColBlockBytes,
-                              (const char *)a_any + (size_t)slot * a_slot_stride * (AF32 ? 4 : 2), wave, waves, k_chunks, k,
-                              lane, acc);
-    red[wave * 64 + lane] = acc[0][0];
+    float acc[1] = {0.f};
+    if (eid < experts) {
+        const char *tbase = bank + (size_t)eid * expert_bytes + (size_t)tile * k_chunks * kColBlockBytes;
+        const void *a_row = (const char *)a_any + (size_t)slot * a_slot_stride * (AF32 ? 4 : 2);
+        const Gemv4Consts dq = make_gemv4_consts();
+        const bool is_lo = (cl & 1u) != 0;
+        gemv4s_run_passes<SUB, ONE>(
+            wave, waves, passes,
+            [&](ChunkS<SUB> &r, uint32_t pass) {
+                uint32_t kc = pass * CPP + cg;
+                const bool live = kc < k_chunks;
+                kc = live ? kc : k_chunks - 1u;
+                gemv4s_load_w<SUB>(r, tbase + (size_t)kc * kColBlockBytes, col, live);
+                gemv4s_load_a<SUB, AF32, TERMS>(r, a_row, 0, kc, cl, k, is_lo);
+            },
+            [&](const ChunkS<SUB> &r) { gemv4s_compute<SUB, 1, TERMS>(r, dq, acc); });
+    }
+    red[wave * 64 + lane] = acc[0];
     __syncthreads();
+    auto summed = [&](uint32_t c) {
+        float v = 0.f;
+        for (uint32_t w = 0; w < waves; w++)
+#pragma unroll
+            for (int q = 0; q < CPP; q++) v += red[w * 64 + q * SUB + c];
+        return v;
+    };
     if (ACT == 0) {
-        if (threadIdx.x < 64) {
-            uint32_t on = tile * 64u + lane;
-            if (on < n) {
-                float v = 0.f;
-                for (uint32_t w = 0; w < waves; w++) v += red[w * 64 + lane];
-                out[(size_t)slot * n + on] = v;
-            }
+        if (threadIdx.x < SUB) {
+            uint32_t on = st * SUB + threadIdx.x;
+            if (on < n) out[(size_t)slot * n + on] = summed(threadIdx.x);
         }
-    } else {
-        // paired order: lanes 0..31 of the tile are gate columns, lanes 32..63 the up columns of the same features
-        if (threadIdx.x < 32) {
-            uint32_t dim = n >> 1, feat = tile * 32u + lane;
-            if (feat < dim) {
-                float g = 0.f, u = 0.f;
-                for (uint32_t w = 0; w < waves; w++) {
-                    g += red[w * 64 + lane];
-                    u += red[w * 64 + 32 + lane];
-                }
-                out[(size_t)slot * dim + feat] = gate_mul<ACT>(g, u);
-            }
-        }
+    } else if (threadIdx.x < SUB / 2) {
+        uint32_t dim = n >> 1, feat = tile * 32u + part * (SUB / 2) + threadIdx.x;
+        if (feat < dim) out[(size_t)slot * dim + feat] = gate_mul<ACT>(summed(threadIdx.x), summed(SUB / 2 + threadIdx.x));
     }
 }
 
-// Workgroup = slots * wps waves on one 64-column tile: wave (slot, j) takes chunks j, j + wps, ... of its
-// slot's expert with its slot's activation row; one thread per column then adds weight[slot] * dot to the
-// accumulator slot by slot.
-template <bool AF32>
+// Workgroup = slots * wps waves on one sub-tile: wave (slot, j) takes passes j, j + wps, ... of its slot's
+// expert with its slot's activation row; one thread per column then adds weight[slot] * dot to the accumulator
+// slot by slot.
+template <int SUB, bool AF32, bool ONE>
 __global__ __launch_bounds__(1024) void k_bank_down_axpy(const char *__restrict__ bank, size_t expert_bytes, uint32_t experts,
                                                           const void *__restrict__ a_all, const float *__restrict__ ids,
                                                           const float *__restrict__ weights, float *__restrict__ accum,
-                                                          uint32_t k, uint32_t n, uint32_t k_chunks, uint32_t tiles64,
+                                                          uint32_t k, uint32_t n, uint32_t k_chunks, uint32_t sub_tiles,
                                                           uint32_t slots, uint32_t wps)
 {
+    constexpr int CPP = 64 / SUB;
+    constexpr int TERMS = gemv4_terms<AF32, 1>();
     extern __shared__ float red[];  // [slots * wps][64]
-    const uint32_t tile = blockIdx.x;
-    if (tile >= tiles64) return;
+    const uint32_t st = blockIdx.x;
+    if (st >= sub_tiles) return;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const uint32_t lane = threadIdx.x & 63u;
+    const uint32_t lane = threadIdx.x & 63u, cl = lane % SUB, cg = lane / SUB;
+    const uint32_t tile = st / CPP, part = st % CPP;
     const uint32_t slot = wave / wps, j = wave % wps;
     const uint32_t eid = __builtin_amdgcn_readfirstlane(expert_of(ids[slot], experts));
+    const uint32_t passes = (k_chunks + CPP - 1) / CPP;
 
-    float acc[1][1] = {{0.f}};
-    if (eid < experts)
-        bank_accumulate<AF32>(bank + (size_t)eid * expert_bytes + (size_t)tile * k_chunks * kColBlockBytes,
-                              (const char *)a_all + (size_t)slot * k * (AF32 ? 4 : 2), j, wps, k_chunks, k, lane, acc);
-    red[wave * 64 + lane] = acc[0][0];
+    float acc[1] = {0.f};
+    if (eid < experts) {
+        const char *tbase = bank + (size_t)eid * expert_bytes + (size_t)tile * k_chunks * kColBlockBytes;
+        const void *a_row = (const char *)a_all + (size_t)slot * k * (AF32 ? 4 : 2);
+        const Gemv4Consts dq = make_gemv4_consts();
+        const bool is_lo = (cl & 1u) != 0;
+        gemv4s_run_passes<SUB, ONE>(
+            j, wps, passes,
+            [&](ChunkS<SUB> &r, uint32_t pass) {
+                uint32_t kc = pass * CPP + cg;
+                const bool live = kc < k_chunks;
+                kc = live ? kc : k_chunks - 1u;
+                gemv4s_load_w<SUB>(r, tbase + (size_t)kc * kColBlockBytes, part * SUB + cl, live);
+                gemv4s_load_a<SUB, AF32, TERMS>(r, a_row, 0, kc, cl, k, is_lo);
+            },
+            [&](const ChunkS<SUB> &r) { gemv4s_compute<SUB, 1, TERMS>(r, dq, acc); });
+    }
+    red[wave * 64 + lane] = acc[0];
     __syncthreads();
-    if (threadIdx.x < 64) {
-        uint32_t on = tile * 64u + lane;
+    if (threadIdx.x < SUB) {
+        uint32_t on = st * SUB + threadIdx.x;
         if (on < n) {
             float total = accum[on];
             for (uint32_t s = 0; s < slots; s++) {
                 float dot = 0.f;
-                for (uint32_t q = 0; q < wps; q++) dot += red[(s * wps + q) * 64 + lane];
+                for (uint32_t q = 0; q < wps; q++)
+#pragma unroll
+                    for (int c = 0; c < CPP; c++) dot += red[(s * wps + q) * 64 + c * SUB + threadIdx.x];
                 total += weights[s] * dot;
             }
             accum[on] = total;
@@ -169,53 +171,77 @@ hipError_t launch_geglu_rows(hipStream_t s, const float *gu, float *out, uint32_
     return hipGetLastError();
 }
 
-static uint32_t bank_waves(uint32_t k_chunks)
+// Sub-tile width of the bank kernels (force_sub = 16 or 32 overrides: a tuning knob of the context).  The
+// per-slot GEMV runs best on 32 columns once that gives a workgroup per CU (Gemma, Qwen and Mixtral expert
+// shapes: 7.0 against 7.6, 5.5 against 5.9, 26.9 against 29.7 us); the down projection, whose workgroups hold
+// every slot, on 16 (6.6 against 7.9, 5.6 against 7.6, 15.4 against 18.6 us).
+static uint32_t bank_sub(uint32_t n_pad, uint32_t slots, bool per_slot, int force_sub)
 {
-    uint32_t waves = 8;
-    while (waves > 1 && k_chunks <= waves / 2) waves /= 2;  // as the dense M <= 4 plan: idle waves only below half
-    return waves;
+    if (force_sub == 16 || force_sub == 32) return (uint32_t)force_sub;
+    return per_slot && (uint64_t)(n_pad / 32) * slots >= 256 ? 32 : 16;
 }
 
 hipError_t launch_bank_gemv(hipStream_t s, const BankView &b, const void *a, bool a_f32, uint32_t a_slot_stride,
-                            const float *ids, uint32_t slots, int act, float *out)
+                            const float *ids, uint32_t slots, int act, float *out, int force_sub, int force_waves)
 {
     if (slots == 0 || b.n == 0) return hipSuccess;
     if (!b.cq || act < 0 || act > 2 || slots > 65535u) return hipErrorInvalidValue;
     if (act != 0 && b.n % (2 * kPairWidth) != 0) return hipErrorInvalidValue;
-    uint32_t tiles64 = b.n_pad / 64, waves = bank_waves(b.k_chunks);
-    dim3 grid(tiles64, slots), block(waves * 64);
+    const uint32_t sub = bank_sub(b.n_pad, slots, true, force_sub), sub_tiles = b.n_pad / sub;
+    const uint32_t passes = (b.k_chunks + 64 / sub - 1) / (64 / sub);
+    uint32_t waves = passes < 16 ? passes : 16;
+    if (force_waves >= 1 && force_waves <= 16) waves = (uint32_t)force_waves;
+    const bool one = passes <= waves;
+    dim3 grid(sub_tiles, slots), block(waves * 64);
     size_t lds = (size_t)waves * 64 * sizeof(float);
-#define TWM_BANK_LAUNCH(F32, A)                                                                                        \
-    hipLaunchKernelGGL((k_bank_gemv<F32, A>), grid, block, lds, s, (const char *)b.cq, b.expert_bytes, b.experts, a,   \
-                       a_slot_stride, ids, out, b.k, b.n, b.k_chunks, tiles64)
-    if (a_f32) {
-        if (act == 0) TWM_BANK_LAUNCH(true, 0);
-        else if (act == 1) TWM_BANK_LAUNCH(true, 1);
-        else TWM_BANK_LAUNCH(true, 2);
+#define TWM_BANK_LAUNCH(SUBV, F32, A, ONEV)                                                                            \
+    hipLaunchKernelGGL((k_bank_gemv<SUBV, F32, A, ONEV>), grid, block, lds, s, (const char *)b.cq, b.expert_bytes,      \
+                       b.experts, a, a_slot_stride, ids, out, b.k, b.n, b.k_chunks, sub_tiles)
+#define TWM_BANK_ONE(SUBV, F32, A)                  \
+    if (one) TWM_BANK_LAUNCH(SUBV, F32, A, true);   \
+    else TWM_BANK_LAUNCH(SUBV, F32, A, false)
+#define TWM_BANK_ACT(SUBV, F32)                     \
+    if (act == 0) { TWM_BANK_ONE(SUBV, F32, 0); }   \
+    else if (act == 1) { TWM_BANK_ONE(SUBV, F32, 1); } \
+    else { TWM_BANK_ONE(SUBV, F32, 2); }
+    if (sub == 16) {
+        if (a_f32) { TWM_BANK_ACT(16, true) } else { TWM_BANK_ACT(16, false) }
     } else {
-        if (act == 0) TWM_BANK_LAUNCH(false, 0);
-        else if (act == 1) TWM_BANK_LAUNCH(false, 1);
-        else TWM_BANK_LAUNCH(false, 2);
+        if (a_f32) { TWM_BANK_ACT(32, true) } else { TWM_BANK_ACT(32, false) }
     }
+#undef TWM_BANK_ACT
+#undef TWM_BANK_ONE
 #undef TWM_BANK_LAUNCH
     return hipGetLastError();
 }
 
 hipError_t launch_bank_down_axpy(hipStream_t s, const BankView &b, const void *a_all, bool a_f32, const float *ids,
-                                 const float *weights, uint32_t slots, float *accum)
+                                 const float *weights, uint32_t slots, float *accum, int force_sub, int force_waves)
 {
     if (slots == 0 || b.n == 0) return hipSuccess;
     if (!b.cq || slots > (uint32_t)kMaxBankSlots) return hipErrorInvalidValue;
-    uint32_t wps = 1;
-    while (slots * wps * 2 <= 16 && b.k_chunks >= wps * 4) wps *= 2;  // at least two chunks per wave
-    uint32_t tiles64 = b.n_pad / 64, waves = slots * wps;
+    const uint32_t sub = bank_sub(b.n_pad, slots, false, force_sub), sub_tiles = b.n_pad / sub;
+    const uint32_t passes = (b.k_chunks + 64 / sub - 1) / (64 / sub);
+    uint32_t wps = 16 / slots;                // waves per slot: up to one per pass, sixteen waves in all
+    if (wps > passes) wps = passes;
+    if (force_waves >= 1 && (uint32_t)force_waves * slots <= 16) wps = (uint32_t)force_waves;
+    if (wps == 0) wps = 1;
+    const bool one = passes <= wps;
+    const uint32_t waves = slots * wps;
     size_t lds = (size_t)waves * 64 * sizeof(float);
-    if (a_f32)
-        hipLaunchKernelGGL((k_bank_down_axpy<true>), dim3(tiles64), dim3(waves * 64), lds, s, (const char *)b.cq,
-                           b.expert_bytes, b.experts, a_all, ids, weights, accum, b.k, b.n, b.k_chunks, tiles64, slots, wps);
-    else
-        hipLaunchKernelGGL((k_bank_down_axpy<false>), dim3(tiles64), dim3(waves * 64), lds, s, (const char *)b.cq,
-                           b.expert_bytes, b.experts, a_all, ids, weights, accum, b.k, b.n, b.k_chunks, tiles64, slots, wps);
+#define TWM_DOWN_LAUNCH(SUBV, F32, ONEV)                                                                               \
+    hipLaunchKernelGGL((k_bank_down_axpy<SUBV, F32, ONEV>), dim3(sub_tiles), dim3(waves * 64), lds, s, (const char *)b.cq, \
+                       b.expert_bytes, b.experts, a_all, ids, weights, accum, b.k, b.n, b.k_chunks, sub_tiles, slots, wps)
+#define TWM_DOWN_ONE(SUBV, F32)                  \
+    if (one) TWM_DOWN_LAUNCH(SUBV, F32, true);   \
+    else TWM_DOWN_LAUNCH(SUBV, F32, false)
+    if (sub == 16) {
+        if (a_f32) { TWM_DOWN_ONE(16, true); } else { TWM_DOWN_ONE(16, false); }
+    } else {
+        if (a_f32) { TWM_DOWN_ONE(32, true); } else { TWM_DOWN_ONE(32, false); }
+    }
+#undef TWM_DOWN_ONE
+#undef TWM_DOWN_LAUNCH
     return hipGetLastError();
 }
 
