@@ -925,12 +925,14 @@ static SubPlan plan_gemv4_sub(uint32_t tiles64, uint32_t k_chunks, uint32_t m, b
     const uint32_t passes16 = (k_chunks + 3) / 4;
     const SubPlan narrow16 = {16, passes16 <= 8 ? 8u : 16u};
     if (tiles64 > 128) {
-        if (two_pass) return none;
-        if (a_f32) return tiles64 >= 1024 ? none : SubPlan{32, 16};
-        if (m > 2) return tiles64 >= 256 ? SubPlan{32, 8} : none;
-        return narrow16;
+        // wide matrices: only the cheapest activations (f16, up to two rows) leave the sub-tiles ahead
+        // (3584 -> 37888: 15.8 against 17.0 us at M = 1, 18.3 against 17.3 at M = 4, 19.9 against 17.9 with f32 rows)
+        if (!a_f32 && m <= 2) return narrow16;
+        if (a_f32 && m <= 2 && tiles64 < 256) return SubPlan{32, 16};
+        return none;
     }
     if (two_pass && passes16 > 16) return k_chunks <= 100 ? SubPlan{32, 8} : none;  // (the looping 16-column variant spills)
+    if (m > 2 && passes16 > 32) return none;   // very deep K, four rows: the 64-column split-K plan is level or ahead
     if (tiles64 > 64) return SubPlan{32, 16};  // 16 columns would leave a second, quarter-full round of workgroups
     return narrow16;
 }
@@ -1033,6 +1035,9 @@ static int gemm_common(twm_ctx *ctx, const twm_weight *w, const void *a_dev, int
         } else if (lane_col && ctx->force_sub == 0 && !ctx->force_nt && !ctx->force_waves && !splits) {
             // (an explicit nt, waves or split factor asks for the 64-column kernel's plan)
             sub = plan_gemv4_sub(n_ld / 64, w->k_chunks, mb, a_dtype == TWM_F32);
+            // the gated store splits a sub-tile into a gate and an up half: 16 columns would read 128-byte runs
+            // (3584 -> 2 x 18944 at M = 1: 17.0 us on 16 columns, 16.3 on 32, 17.1 on whole tiles)
+            if (swiglu_out && sub.sub == 16) sub = SubPlan{32, 8};
         }
         if (sub.sub) {
             uint32_t ssp = splits ? splits : 1;

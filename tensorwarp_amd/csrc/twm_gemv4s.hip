@@ -89,14 +89,22 @@ __global__ __launch_bounds__(1024) void k_gemv4s(const char *__restrict__ cw, co
         const bool live = kc < kc1;
         kc = live ? kc : kc1 - 1u;  // a chunk past the k-range replays the last one with scale 0
         if (REFL) {
+            // (all eight loads into locals first: written straight into r, each pair was followed by a full wait)
+            uint4v wq[4];
             uint32_t sb[4];
+            bool ok[4];
 #pragma unroll
             for (int g = 0; g < 4; g++) {
                 const uint32_t gg = kc * 4u + g;
                 const size_t idx = (size_t)(gg < ref_groups ? gg : ref_groups - 1u) * n + ref_col;
-                r.wq[g] = *(const uint4v *)(cw + idx * 16u);
-                const uint32_t sbits = ref_scales[idx];
-                sb[g] = (live && gg < ref_groups && st * SUB + cl < n) ? sbits : 0u;  // weight exactly 0 otherwise
+                wq[g] = *(const uint4v *)(cw + idx * 16u);
+                sb[g] = ref_scales[idx];
+                ok[g] = live && gg < ref_groups && st * SUB + cl < n;  // weight exactly 0 otherwise
+            }
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+                r.wq[g] = wq[g];
+                sb[g] = ok[g] ? sb[g] : 0u;
             }
             r.sc = uint2v{sb[0] | (sb[1] << 16), sb[2] | (sb[3] << 16)};
         } else {

@@ -193,13 +193,14 @@ def test_gemm_swiglu_fused_epilogue(dev, h, ffn, m, splits):
     assert w.paired and not plain.paired
     out = T.GpuTensor.from_host(dev, np.full((m, ffn), np.nan, np.float32))
     T.gemm_swiglu(dev, w, ad, m, out, splits)
-    # The same columns, unfused, on the paired handle: bit for bit.  (Against the [gate | up] handle a column can
-    # sit in another part of the grid and be summed in another split order, so that comparison is to rounding.)
+    # the same columns, unfused, on the paired handle and on the [gate | up] handle
     tmp = T.GpuTensor.zeros(dev, (m, 2 * ffn), "f32")
     T.gemm(dev, w, ad, m, tmp, splits)
     seq_p = T.GpuTensor.zeros(dev, (m, ffn), "f32")
     T.swiglu_rows(dev, tmp, seq_p, ffn, m, paired=True)
-    assert np.array_equal(out.to_host(), seq_p.to_host())
+    # (bit for bit under one plan, see test_sub_tile_gated_store; the planner may give the gated launch wider
+    # sub-tiles than the plain one, which changes the order of the f32 sum)
+    assert rel_err(out.to_host(), seq_p.to_host()) < 1e-4
     assert rel_err(out.to_host(), seq.to_host()) < 1e-4
     # against the oracle: f64 projections, then the reference's gate in f32 (its input differs from the
     # GPU's by the GEMV's rounding, so the bar is the GEMV's)
