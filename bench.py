@@ -35,8 +35,8 @@ LAYER_7B = [("qkv", 3584, 4608), ("o", 3584, 3584), ("gate_up", 3584, 37888), ("
 LAYER_05B = [("qkv", 896, 1152), ("o", 896, 896), ("gate_up", 896, 9728), ("down", 4864, 896)]   # Qwen-0.5B layer
 CFG0 = [("cfg0", 4096, 4096)]                                                                     # the single-GEMV configuration
 # HBM bytes per gate_up launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, each scaled by
-# what the same counter reads for a 64 MiB copy (profiles/k_gemv4_gate_up_m1_hbm_traffic.md).
-GATE_UP_TRAFFIC_BYTES = 76665000
+# what the same counter reads for a 64 MiB copy (profiles/k_gemv4s_gate_up_m1_hbm_traffic.md).
+GATE_UP_TRAFFIC_BYTES = 76684800
 
 
 def algo_bytes(k, n, m=1):
@@ -271,7 +271,7 @@ def main():
 
     gu = per_shape["gate_up"]
     gu_bytes = algo_bytes(3584, 37888)
-    roofline = {"bound": "hbm", "kernel": "k_gemv4 (gate_up 3584->37888, M=1)",
+    roofline = {"bound": "hbm", "kernel": "k_gemv4s (gate_up 3584->37888, M=1)",
                 "achieved": gu["GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
                 "frac": round(gu["GBps"] / HBM_PEAK_GBS, 4),
                 "bytes_per_launch": gu_bytes, "us_per_launch": gu["us"],
