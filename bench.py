@@ -568,7 +568,7 @@ def main():
                     for i in range(8):
                         one(i)
                     dev.synchronize()
-                    row["auto" if sp == 0 else str(sp)] = round(time_launches(dev, one, 100) * 1e3, 2)
+                    row["auto" if sp == 0 else str(sp)] = round(time_short_launches(dev, T, one, 104, graphs_done)[0] * 1e3, 2)
                 best = min((v, key) for key, v in row.items() if key != "auto")
                 sweep["%s_M%d" % (name, m)] = {"us": row, "auto_over_best": round(row["auto"] / best[0], 3), "best_splits": int(best[1])}
                 a_m.free()

@@ -87,6 +87,8 @@ int twm_ctx_info(twm_ctx *ctx, char *buf, size_t buf_len);
  * crates/kernels/src/autotune.rs:254-396); 0 = library's choice unless noted:
  *   "nt"            column tiles per workgroup of the decode kernels (1, 2, 4)
  *   "waves"         waves per workgroup of the decode kernels (1, 2, 4, 8, 16; streaming kernel 4 or 8)
+ *   "sub"           M <= 4 and expert-bank kernels: 1 = whole 64-column tiles per workgroup, 16 or 32 = sub-tiles
+ *                   of that many columns (with "waves" waves, default 8), 0 = the planner's choice per shape
  *   "kernel"        decode kernel: 1 = 16x16x32 tile kernel (16-row blocks), 2 = one-lane-per-column kernel
  *                   (M <= 4 only), 3 = batched-decode streaming kernel (32-row blocks)
  *   "dequant_src"   which repacked copy twm_weight_dequant_f16 unpacks: 0 = 16-column tiles, 1 = column lanes
