@@ -937,6 +937,20 @@ static SubPlan plan_gemv4_sub(uint32_t tiles64, uint32_t k_chunks, uint32_t m, b
     return narrow16;
 }
 
+// M = 5 .. 16 (f16 rows): the same kernel repeats its MFMA chain per group of four rows on the unpacked weights.
+// It pays where the streaming kernel's 64-column workgroups leave most CUs idle, i.e. on narrow matrices, and
+// only in the one-pass form (the looping form runs out of registers): 3584 -> 3584 at M = 8 / 16: 4.8 / 6.5 us
+// against 6.9 / 8.2; 3584 -> 4608: 5.5 / 7.4 against 6.9 / 8.2; 3584 -> 37888: 21.7 / 35 against 19.5 / 23.2.
+static SubPlan plan_gemv4_sub_rows(uint32_t tiles64, uint32_t k_chunks)
+{
+    const SubPlan none = {0, 0};
+    if (k_chunks < 16 || tiles64 > 128) return none;
+    const uint32_t passes16 = (k_chunks + 3) / 4, passes32 = (k_chunks + 1) / 2;
+    if (tiles64 <= 64 && passes16 <= 16) return SubPlan{16, passes16 <= 8 ? 8u : 16u};
+    if (passes32 <= 16) return SubPlan{32, 16};
+    return none;
+}
+
 // Batched-decode streaming kernel (M = 5 .. 32): one workgroup of eight waves per 64 columns and k-range.  K is
 // cut when the column quads alone leave CUs idle, up to about one workgroup per CU, keeping two chunks per
 // wave (one for the 32-row variant, whose chunks cost twice the arithmetic); the partial sums cost a second
@@ -999,6 +1013,21 @@ static int gemm_common(twm_ctx *ctx, const twm_weight *w, const void *a_dev, int
     if (m >= (uint32_t)ctx->prefill_min_m) {
         HIP_TRY(launch_prefill(ctx->stream, v, a_dev, a_dtype == TWM_F32, m, gated, (uint32_t)ctx->prefill_bm, splits, ctx->ws, ctx->ws_bytes), TWM_DEVICE_ERROR, "prefill launch");
         return TWM_OK;
+    }
+    if (ctx->force_kernel == 0 && m > 4 && m <= 16 && a_dtype == TWM_F16 && ctx->force_sub != 1) {
+        // M = 5 .. 16 on narrow matrices: the lane-per-column sub-tile kernel with two to four row groups
+        SubPlan sub = {0, 0};
+        if (ctx->force_sub >= 16) sub = SubPlan{(uint32_t)ctx->force_sub, ctx->force_waves ? (uint32_t)ctx->force_waves : 8};
+        else if (!ctx->force_nt && !ctx->force_waves && !splits) sub = plan_gemv4_sub_rows(n_ld / 64, w->k_chunks);
+        if (sub.sub) {
+            uint32_t ssp = splits ? splits : 1;
+            if (ssp > w->k_chunks) ssp = w->k_chunks;
+            while (ssp > 1 && (size_t)ssp * m * n_ld * 4 > ctx->ws_bytes) ssp--;
+            if (n_ld / sub.sub > ctx->n_counters) ssp = 1;
+            HIP_TRY(launch_gemv4s(ctx->stream, v, a_dev, false, m, gated, ctx->ws, ctx->counters, sub.sub, sub.waves, ssp),
+                    TWM_DEVICE_ERROR, "sub-tile gemv launch");
+            return TWM_OK;
+        }
     }
     if (ctx->force_kernel == 3 || (ctx->force_kernel == 0 && m > 4)) {
         // batched decode: 32-row blocks of the streaming kernel

@@ -189,12 +189,13 @@ __device__ __forceinline__ void gemv4_compute_chunk(const Chunk4<NT> &r, const G
 // Lane l = (chunk l / SUB of the pass, column l % SUB).  With CBSZ = log2(SUB / 4) the MFMA broadcasts an A block
 // inside groups of SUB lanes only, so every lane group takes the activations of its own chunk: one A register
 // holds 2 * SUB of the chunk's 128 k-values (SUB / 4 pieces of eight), 64 / SUB registers the whole chunk.
-template <int SUB>
+// RG = row groups of four: rows 4 .. 4*RG-1 repeat the MFMA chain on the same unpacked weights (f16 rows only).
+template <int SUB, int RG = 1>
 struct ChunkS {
-    uint4v wq[4];            // this lane's column, its chunk: four groups of 32 nibbles
-    uint2v sc;               // four f16 scales
-    uint4v a[64 / SUB];      // activations: row (lane % SUB) % 4, piece (lane % SUB) / 4 of every 2*SUB-wide slice
-    uint4v a_lo[64 / SUB];   // f32 activations as two passes: the residual terms
+    uint4v wq[4];                 // this lane's column, its chunk: four groups of 32 nibbles
+    uint2v sc;                    // four f16 scales
+    uint4v a[RG][64 / SUB];       // activations: row 4*rg + (lane % SUB) % 4, piece (lane % SUB) / 4 of every 2*SUB-wide slice
+    uint4v a_lo[64 / SUB];        // f32 activations as two passes: the residual terms
 };
 
 template <int SUB, int P>
@@ -208,10 +209,12 @@ __device__ __forceinline__ float4v mfma_sub(half4v a, half4v b, float4v c)
 // The lane's activations of chunk kc: 64 / SUB pieces of eight, row arow (term modes as gemv4_load_chunk).
 // ref_order: the weights' nibbles are in the reference's natural order, which the mask-and-magic unpack turns
 // into the k order (0,4,1,5 | 2,6,3,7) per eight; the (f32) activations take the same order.
-template <int SUB, bool AF32, int TERMS, bool REF_ORDER = false>
-__device__ __forceinline__ void gemv4s_load_a(ChunkS<SUB> &r, const void *a_any, uint32_t arow, uint32_t kc, uint32_t cl,
-                                              uint32_t k, bool lane_is_lo)
+// With RG row groups, group rg reads row min(4*rg + arow, m_rows - 1).
+template <int SUB, bool AF32, int TERMS, bool REF_ORDER = false, int RG = 1>
+__device__ __forceinline__ void gemv4s_load_a(ChunkS<SUB, RG> &r, const void *a_any, uint32_t arow, uint32_t kc, uint32_t cl,
+                                              uint32_t k, bool lane_is_lo, uint32_t m_rows = 0)
 {
+    static_assert(RG == 1 || !AF32, "more than four rows: f16 activations only");
 #pragma unroll
     for (int j = 0; j < 64 / SUB; j++) {
         uint32_t k0 = kc * 128u + j * (2u * SUB) + (cl >> 2) * 8u;
@@ -221,21 +224,26 @@ __device__ __forceinline__ void gemv4s_load_a(ChunkS<SUB> &r, const void *a_any,
             float4 x = p[0], y = p[1];
             const float v[8] = {x.x, REF_ORDER ? y.x : x.y, REF_ORDER ? x.y : x.z, REF_ORDER ? y.y : x.w,
                                 REF_ORDER ? x.z : y.x, REF_ORDER ? y.z : y.y, REF_ORDER ? x.w : y.z, y.w};
-            split_f32x8(v, r.a[j], r.a_lo[j]);
+            split_f32x8(v, r.a[0][j], r.a_lo[j]);
             if (TERMS == kTermsRowPacked) {
 #pragma unroll
-                for (int i = 0; i < 4; i++) r.a[j][i] = lane_is_lo ? r.a_lo[j][i] : r.a[j][i];
+                for (int i = 0; i < 4; i++) r.a[0][j][i] = lane_is_lo ? r.a_lo[j][i] : r.a[0][j][i];
             }
         } else {
-            r.a[j] = *(const uint4v *)((const _Float16 *)a_any + (size_t)arow * k + k0);
+#pragma unroll
+            for (int rg = 0; rg < RG; rg++) {
+                uint32_t row = arow + 4u * rg;
+                if (RG > 1 && row > m_rows - 1u) row = m_rows - 1u;
+                r.a[rg][j] = *(const uint4v *)((const _Float16 *)a_any + (size_t)row * k + k0);
+            }
         }
     }
 }
 
 // The lane's weights from the column-lane copy: blk = the block of the lane's chunk, col = column in the
 // 64-column tile; live = false zeroes the scales (a chunk past the k-range replays a valid one as zeros).
-template <int SUB>
-__device__ __forceinline__ void gemv4s_load_w(ChunkS<SUB> &r, const char *blk, uint32_t col, bool live)
+template <int SUB, int RG>
+__device__ __forceinline__ void gemv4s_load_w(ChunkS<SUB, RG> &r, const char *blk, uint32_t col, bool live)
 {
 #pragma unroll
     for (int g = 0; g < 4; g++) r.wq[g] = *(const uint4v *)(blk + g * 1024u + col * 16u);
@@ -245,15 +253,19 @@ __device__ __forceinline__ void gemv4s_load_w(ChunkS<SUB> &r, const char *blk, u
 
 // acc[row] += f32(scale) * (sum over the group of A * (q - 8)) for the four groups of the lane's chunk
 template <int SUB, int RL, int TERMS>
-__device__ __forceinline__ void gemv4s_compute(const ChunkS<SUB> &r, const Gemv4Consts &dq, float (&acc)[RL])
+__device__ __forceinline__ void gemv4s_compute(const ChunkS<SUB, (RL + 3) / 4> &r, const Gemv4Consts &dq, float (&acc)[RL])
 {
     constexpr int PIECES = SUB / 4;  // 8-wide k pieces per A register
+    constexpr int RG = (RL + 3) / 4;
     static_assert(TERMS != kTermsRowPacked || RL <= 2, "row-packed terms hold at most two rows");
+    static_assert(RG == 1 || TERMS == kTermsOne, "more than four rows: one f16 term");
     union { uint2v u; _Float16 h[4]; } sv;
     sv.u = r.sc;
 #pragma unroll
     for (int g = 0; g < 4; g++) {
-        float4v d = {0.f, 0.f, 0.f, 0.f};
+        float4v d[RG];
+#pragma unroll
+        for (int rg = 0; rg < RG; rg++) d[rg] = float4v{0.f, 0.f, 0.f, 0.f};
         half4v lo4, hi4;
         // word W of group g is the 8-wide piece 4g + W of the chunk: register (4g + W) / PIECES, block
         // (4g + W) % PIECES of the lane group
@@ -261,14 +273,16 @@ __device__ __forceinline__ void gemv4s_compute(const ChunkS<SUB> &r, const Gemv4
     {                                                                                      \
         constexpr int PG = 4 * G + W, J = PG / PIECES, ABID = PG % PIECES;                 \
         union { uint4v u; half4v h[2]; } av, al;                                           \
-        av.u = r.a[J];                                                                     \
         gemv4_dequant_word(r.wq[G][W], dq, lo4, hi4);                                      \
-        d = mfma_sub<SUB, ABID>(av.h[0], lo4, d);                                          \
-        d = mfma_sub<SUB, ABID>(av.h[1], hi4, d);                                          \
+        _Pragma("unroll") for (int rg = 0; rg < RG; rg++) {                                \
+            av.u = r.a[rg][J];                                                             \
+            d[rg] = mfma_sub<SUB, ABID>(av.h[0], lo4, d[rg]);                              \
+            d[rg] = mfma_sub<SUB, ABID>(av.h[1], hi4, d[rg]);                              \
+        }                                                                                  \
         if (TERMS == kTermsTwoPasses) {                                                    \
             al.u = r.a_lo[J];                                                              \
-            d = mfma_sub<SUB, ABID>(al.h[0], lo4, d);                                      \
-            d = mfma_sub<SUB, ABID>(al.h[1], hi4, d);                                      \
+            d[0] = mfma_sub<SUB, ABID>(al.h[0], lo4, d[0]);                                \
+            d[0] = mfma_sub<SUB, ABID>(al.h[1], hi4, d[0]);                                \
         }                                                                                  \
     }
 #define TWM_SUB_GROUP(GV)                                                                  \
@@ -282,26 +296,26 @@ __device__ __forceinline__ void gemv4s_compute(const ChunkS<SUB> &r, const Gemv4
         const float s = (float)sv.h[g];
 #pragma unroll
         for (int rr = 0; rr < RL; rr++) {
-            if (TERMS == kTermsRowPacked) acc[rr] = fmaf(d[2 * rr] + d[2 * rr + 1], s, acc[rr]);
-            else acc[rr] = fmaf(d[rr], s, acc[rr]);
+            if (TERMS == kTermsRowPacked) acc[rr] = fmaf(d[0][2 * rr] + d[0][2 * rr + 1], s, acc[rr]);
+            else acc[rr] = fmaf(d[rr / 4][rr % 4], s, acc[rr]);
         }
     }
 }
 
 // The passes first, first + stride, ... < passes with two register sets: the next pass's loads are in flight
 // while this one is unpacked.  ONE: the caller knows that no wave has a second pass.
-template <int SUB, bool ONE, class Load, class Compute>
+template <int SUB, bool ONE, int RG = 1, class Load, class Compute>
 __device__ __forceinline__ void gemv4s_run_passes(uint32_t first, uint32_t stride, uint32_t passes, Load load, Compute compute)
 {
     if (ONE) {
-        ChunkS<SUB> r0;
+        ChunkS<SUB, RG> r0;
         if (first < passes) {
             load(r0, first);
             compute(r0);
         }
         return;
     }
-    ChunkS<SUB> r0, r1;
+    ChunkS<SUB, RG> r0, r1;
     uint32_t p = first;
     if (p >= passes) return;
     load(r0, p);

@@ -84,7 +84,8 @@ __global__ __launch_bounds__(1024) void k_gemv4s(const char *__restrict__ cw, co
 #pragma unroll
     for (int r = 0; r < RL; r++) acc[r] = 0.f;
 
-    auto load_pass = [&](ChunkS<SUB> &r, uint32_t pass) {
+    constexpr int RG = (RL + 3) / 4;  // rows beyond four repeat the MFMA chain (f16 activations)
+    auto load_pass = [&](ChunkS<SUB, RG> &r, uint32_t pass) {
         uint32_t kc = kc0 + pass * CPP + cg;
         const bool live = kc < kc1;
         kc = live ? kc : kc1 - 1u;  // a chunk past the k-range replays the last one with scale 0
@@ -110,11 +111,11 @@ __global__ __launch_bounds__(1024) void k_gemv4s(const char *__restrict__ cw, co
         } else {
             gemv4s_load_w<SUB>(r, tbase + (size_t)kc * kColBlockBytes, col_in_tile(cl), live);
         }
-        gemv4s_load_a<SUB, AF32, TERMS, REFL>(r, a_any, arow, kc, cl, k, lane_is_lo);
+        gemv4s_load_a<SUB, AF32, TERMS, REFL, RG>(r, a_any, arow, kc, cl, k, lane_is_lo, m_rows);
     };
-    auto compute_pass = [&](const ChunkS<SUB> &r) { gemv4s_compute<SUB, RL, TERMS>(r, dq, acc); };
+    auto compute_pass = [&](const ChunkS<SUB, RG> &r) { gemv4s_compute<SUB, RL, TERMS>(r, dq, acc); };
     // (ONE: the launcher saw that no wave has a second pass: one register set, no loop)
-    gemv4s_run_passes<SUB, ONE>(wave, waves, passes, load_pass, compute_pass);
+    gemv4s_run_passes<SUB, ONE, RG>(wave, waves, passes, load_pass, compute_pass);
 
     // ---- sum over the waves and over the chunks of a pass (lane groups) through LDS ----
 #pragma unroll
@@ -197,8 +198,12 @@ static hipError_t launch_gemv4s_t(hipStream_t s, const WeightView &w, const void
     hipLaunchKernelGGL((k_gemv4s<SUB, RL, AF, ONEV>), dim3(blocks), dim3(waves * 64), lds, s, (const char *)w.cq, a, out, \
                        ws, counters, m, w.k, w.n, n_pad, w.k_chunks, sub_tiles, splits, cps)
     if (a_f32) {
-        if (one) TWM_S_LAUNCH(true, true);
-        else TWM_S_LAUNCH(true, false);
+        if constexpr (RL <= 4) {
+            if (one) TWM_S_LAUNCH(true, true);
+            else TWM_S_LAUNCH(true, false);
+        } else {
+            return hipErrorInvalidValue;  // more than four rows: f16 activations only
+        }
     } else {
         if (one) TWM_S_LAUNCH(false, true);
         else TWM_S_LAUNCH(false, false);
@@ -208,11 +213,12 @@ static hipError_t launch_gemv4s_t(hipStream_t s, const WeightView &w, const void
 }
 
 // sub = 32 or 16 columns per workgroup; waves 1 .. 16; out.swiglu set: the gated store of a paired weight.
+// m <= 4 with f16 or f32 activations, m = 5 .. 16 with f16 activations.
 hipError_t launch_gemv4s(hipStream_t s, const WeightView &w, const void *a, bool a_f32, uint32_t m, const OutSpec &out,
                          float *ws, unsigned *counters, uint32_t sub, uint32_t waves, uint32_t splits)
 {
     if (m == 0 || w.n == 0) return hipSuccess;
-    if (m > 4 || splits == 0 || !w.cq) return hipErrorInvalidValue;
+    if (m > 16 || (m > 4 && a_f32) || splits == 0 || !w.cq) return hipErrorInvalidValue;
     if (out.swiglu && w.n % 64 != 0) return hipErrorInvalidValue;
     if (waves < 1 || waves > 16) return hipErrorInvalidValue;
     if (sub != 32 && sub != 16) return hipErrorInvalidValue;
@@ -220,7 +226,9 @@ hipError_t launch_gemv4s(hipStream_t s, const WeightView &w, const void *a, bool
     if (sub == SUBV) {                                                                                         \
         if (m == 1) return launch_gemv4s_t<SUBV, 1>(s, w, a, a_f32, m, out, ws, counters, waves, splits);      \
         if (m == 2) return launch_gemv4s_t<SUBV, 2>(s, w, a, a_f32, m, out, ws, counters, waves, splits);      \
-        return launch_gemv4s_t<SUBV, 4>(s, w, a, a_f32, m, out, ws, counters, waves, splits);                  \
+        if (m <= 4) return launch_gemv4s_t<SUBV, 4>(s, w, a, a_f32, m, out, ws, counters, waves, splits);      \
+        if (m <= 8) return launch_gemv4s_t<SUBV, 8>(s, w, a, a_f32, m, out, ws, counters, waves, splits);      \
+        return launch_gemv4s_t<SUBV, 16>(s, w, a, a_f32, m, out, ws, counters, waves, splits);                 \
     }
     TWM_S_CASE(32)
     TWM_S_CASE(16)
