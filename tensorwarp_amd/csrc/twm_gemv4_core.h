@@ -12,6 +12,14 @@ struct Gemv4Consts {
     uint32_t mask_lo, mask_hi, magic_lo, magic_hi;
 };
 
+// Weights are read once per launch: a non-temporal load keeps them from displacing the activations (and the
+// next launch's working set) in the caches.  3584 -> 37888 at M = 1: 14.8 against 15.8 us; LM head 48.5 against 51.
+template <class T>
+__device__ __forceinline__ T ld_once(const T *p)
+{
+    return __builtin_nontemporal_load(p);
+}
+
 __device__ __forceinline__ Gemv4Consts make_gemv4_consts()
 {
     // opaque to the optimiser so that (w & mask) | magic becomes one v_and_or_b32
@@ -89,8 +97,8 @@ __device__ __forceinline__ void gemv4_load_chunk(Chunk4<NT> &r, const char *(&wb
     for (int t = 0; t < NT; t++) {
         const char *blk = wbase[t] + (size_t)kc * kColBlockBytes;
 #pragma unroll
-        for (int g = 0; g < 4; g++) r.wq[t][g] = *(const uint4v *)(blk + g * 1024u + lane16);
-        r.sc[t] = *(const uint2v *)(blk + lane8);
+        for (int g = 0; g < 4; g++) r.wq[t][g] = ld_once((const uint4v *)(blk + g * 1024u + lane16));
+        r.sc[t] = ld_once((const uint2v *)(blk + lane8));
     }
     uint32_t k0 = kc * 128u + apiece;
     if (k0 > k - 8u) k0 = k - 8u;  // only the zero-padded groups of a last partial chunk get here
@@ -129,8 +137,8 @@ __device__ __forceinline__ void gemv4_load_chunk_ref(Chunk4<NT> &r, const char *
             const uint32_t gg = kc * 4u + g;
             const uint32_t ggc = gg < groups ? gg : groups - 1u;
             const size_t idx = (size_t)ggc * n + colc;
-            r.wq[t][g] = *(const uint4v *)(packed + idx * 16u);
-            const uint32_t sbits = scales[idx];
+            r.wq[t][g] = ld_once((const uint4v *)(packed + idx * 16u));
+            const uint32_t sbits = ld_once(scales + idx);
             sb[g] = (gg < groups && col < n) ? sbits : 0u;
         }
         r.sc[t] = uint2v{sb[0] | (sb[1] << 16), sb[2] | (sb[3] << 16)};
@@ -246,8 +254,8 @@ template <int SUB, int RG>
 __device__ __forceinline__ void gemv4s_load_w(ChunkS<SUB, RG> &r, const char *blk, uint32_t col, bool live)
 {
 #pragma unroll
-    for (int g = 0; g < 4; g++) r.wq[g] = *(const uint4v *)(blk + g * 1024u + col * 16u);
-    uint2v s = *(const uint2v *)(blk + 4096u + col * 8u);
+    for (int g = 0; g < 4; g++) r.wq[g] = ld_once((const uint4v *)(blk + g * 1024u + col * 16u));
+    uint2v s = ld_once((const uint2v *)(blk + 4096u + col * 8u));
     r.sc = live ? s : uint2v{0u, 0u};
 }
 

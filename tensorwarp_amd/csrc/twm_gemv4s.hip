@@ -98,8 +98,8 @@ __global__ __launch_bounds__(1024) void k_gemv4s(const char *__restrict__ cw, co
             for (int g = 0; g < 4; g++) {
                 const uint32_t gg = kc * 4u + g;
                 const size_t idx = (size_t)(gg < ref_groups ? gg : ref_groups - 1u) * n + ref_col;
-                wq[g] = *(const uint4v *)(cw + idx * 16u);
-                sb[g] = ref_scales[idx];
+                wq[g] = ld_once((const uint4v *)(cw + idx * 16u));
+                sb[g] = ld_once(ref_scales + idx);
                 ok[g] = live && gg < ref_groups && st * SUB + cl < n;  // weight exactly 0 otherwise
             }
 #pragma unroll

@@ -136,8 +136,9 @@ __global__ __launch_bounds__(WAVES * 64) void k_stream(const uint4v *__restrict_
 #pragma unroll
         for (int t = 0; t < 4; t++) {
             size_t tile = (size_t)kc * n_tiles + nt0 + t;
-            r.bq[t] = *(const TWM_GLOBAL uint4v *)(st_scalar_base(qw, tile * 1024u) + q_off);
-            r.bs[t] = *(const TWM_GLOBAL uint2v *)(st_scalar_base(sc, tile * 128u) + s_off);
+            // (weights are read once per launch: non-temporal)
+            r.bq[t] = __builtin_nontemporal_load((const TWM_GLOBAL uint4v *)(st_scalar_base(qw, tile * 1024u) + q_off));
+            r.bs[t] = __builtin_nontemporal_load((const TWM_GLOBAL uint2v *)(st_scalar_base(sc, tile * 128u) + s_off));
         }
 #pragma unroll
         for (int g = 0; g < 4; g++) {
