@@ -305,7 +305,8 @@ int twm_bank_down_axpy(twm_ctx *ctx, const twm_bank *b, const void *a_all_dev, i
 int twm_geglu_rows(twm_ctx *ctx, const float *gate_up_dev, uint32_t batch, uint32_t dim, int paired,
                    float *out_dev);
 
-/* The library's split-K choice for MI355X (256 CUs); same role as quantize.rs:1317-1325. */
+/* The library's split-K choice for MI355X (256 CUs) with f16 activations; same role as quantize.rs:1317-1325.
+ * 1 where the plan needs no split (among others wherever M <= 16 runs on column sub-tiles). */
 uint32_t twm_pick_splits(uint32_t k, uint32_t n, uint32_t m);
 
 /* ---- graph capture / replay (GraphCapture::{record_with_device, replay}, cuda_graph.rs:85-117) */

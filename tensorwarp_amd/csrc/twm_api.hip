@@ -977,7 +977,9 @@ uint32_t twm_pick_splits(uint32_t k, uint32_t n, uint32_t m)
 {
     uint32_t n_tiles = ((n + kNPadTo - 1) / kNPadTo) * kNPadTo / kTileN;
     uint32_t k_chunks = (k / 32 + kChunkGroups - 1) / kChunkGroups;
-    if (m <= 4) return plan_gemv4(n_tiles, k_chunks, 0, 0, 0).splits;
+    // (f16 activations assumed; where the planner takes the sub-tile kernel, K is not split at all)
+    if (m <= 4) return plan_gemv4_sub(n_tiles * kTileN / 64, k_chunks, m, false).sub ? 1 : plan_gemv4(n_tiles, k_chunks, 0, 0, 0).splits;
+    if (m <= 16 && plan_gemv4_sub_rows(n_tiles * kTileN / 64, k_chunks).sub) return 1;
     return plan_stream(n_tiles, k_chunks, m);
 }
 
