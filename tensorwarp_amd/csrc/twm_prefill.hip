@@ -422,26 +422,46 @@ hipError_t launch_splitk_reduce(hipStream_t s, const float *partials, const OutS
     return hipGetLastError();
 }
 
-// Split-K factor by a small cost model fitted to per-shape sweeps on MI355X (microseconds):
-//   rounds * (chunks per split * t_chunk + t_start)  +  [split]  t_reduce + 2 * splits * partial bytes / 3 TB/s
-// t_chunk: 1.0 for 64-row blocks alone on a CU, 1.3 when two share it, 2.3 for 128-row blocks.
-static uint32_t pick_prefill_splits(uint32_t rows, uint32_t block_rows, uint32_t col_blocks, uint32_t k_chunks, size_t n_ld)
+// Block height and split-K factor by a small cost model fitted to per-shape sweeps on MI355X (microseconds per
+// 128-deep chunk and workgroup): a 64-row block alone on a CU 1.1, two sharing a CU 2.0 each, a 128-row block 1.5
+// with few workgroups in flight up to 1.8 with all 256 CUs busy; 3 per round of workgroups for the start and the
+// store; a split costs the second kernel, 2.5 + its read of the partial sums at 4 TB/s.  (128-row blocks unpack
+// every weight for twice the rows: per row they are the cheapest form as soon as there is a workgroup for most
+// CUs, and K 4096 -> N 11008 at M = 512 runs in 50 us on 172 of them against 61 us on 344 64-row blocks.)
+struct PrefillPlan {
+    uint32_t block_rows, splits;
+    double us;
+};
+static PrefillPlan plan_prefill(uint32_t rows, uint32_t force_rows, uint32_t force_splits, uint32_t col_blocks,
+                                uint32_t k_chunks, size_t n_ld)
 {
-    const double wgs = (double)((rows + block_rows - 1) / block_rows) * col_blocks;
-    const double slots = block_rows == 128 ? 256.0 : 512.0;
-    const double partial_us = 2.0 * (double)rows * (double)n_ld * 4.0 / 3.0e6;  // write + read of one split's partials
-    uint32_t best = 1;
-    double best_t = 1e30;
-    for (uint32_t sp = 1; sp <= 64 && sp * 2 <= (k_chunks > 1 ? k_chunks : 2); sp++) {
-        uint32_t cps = (k_chunks + sp - 1) / sp;
-        if ((k_chunks + cps - 1) / cps != sp) continue;  // same work as a smaller factor
-        double total = wgs * sp;
-        double rounds = total <= slots ? 1.0 : (double)(uint64_t)((total + slots - 1) / slots);
-        double t_chunk = block_rows == 128 ? 2.3 : (total > 256.0 ? 1.3 : 1.0);
-        double t = rounds * (cps * t_chunk + 3.0) + (sp > 1 ? 3.0 + sp * partial_us : 0.0);
-        if (t < best_t * 0.97) {  // a larger factor has to pay for itself
-            best_t = t;
-            best = sp;
+    PrefillPlan best = {force_rows ? force_rows : 64u, force_splits ? force_splits : 1u, 1e30};
+    const double partial_us = (double)rows * (double)n_ld * 4.0 / 4.0e6;  // the reduce kernel's read of one split
+    for (uint32_t bm = 64; bm <= 128; bm += 64) {
+        if (force_rows && bm != force_rows) continue;
+        const double wgs = (double)((rows + bm - 1) / bm) * col_blocks;
+        for (uint32_t sp = 1; sp <= 64; sp++) {
+            if (force_splits ? sp != force_splits : sp * 2 > (k_chunks > 1 ? k_chunks : 2) && sp > 1) continue;
+            const uint32_t cps = (k_chunks + sp - 1) / sp;
+            if (!force_splits && (k_chunks + cps - 1) / cps != sp) continue;  // same work as a smaller factor
+            const double total = wgs * sp;
+            double t;
+            if (bm == 128) {
+                const double rounds = (double)(uint64_t)((total + 255.0) / 256.0);
+                const double load = total >= 256.0 ? 1.0 : total / 256.0;
+                t = rounds * (cps * (1.5 + 0.3 * load) + 3.0);
+            } else if (total <= 256.0) {
+                t = cps * 1.1 + 3.0;
+            } else {
+                const double full = (double)(uint64_t)(total / 512.0), rem = total - 512.0 * full;
+                t = full * (cps * 2.0 + 3.0) + (rem == 0.0 ? 0.0 : (rem <= 256.0 ? cps * 1.1 : cps * 2.0) + 3.0);
+            }
+            if (sp > 1) t += 2.5 + sp * partial_us;
+            if (t < best.us * (sp > best.splits && bm == best.block_rows ? 0.97 : 1.0)) {  // a larger factor has to pay for itself
+                best.block_rows = bm;
+                best.splits = sp;
+                best.us = t;
+            }
         }
     }
     return best;
@@ -474,31 +494,35 @@ hipError_t init_prefill()
                                2 * 16 * 8 * kPfRowStride * (int)sizeof(_Float16));
 }
 
-// block_rows: 64 or 128 rows of A per workgroup; 0 = choose: 128-row blocks unpack each weight for twice as
-// many rows and win once they fill the 256 CUs, below that 64-row blocks give twice the workgroups.
-// splits: k-split factor, 0 = choose: when the grid leaves CUs idle, K is cut so that about 512 64-row
-// workgroups (two per CU) exist, within what `scratch` can hold as f32 partial sums.
+// block_rows: 64 or 128 rows of A per workgroup, splits: k-split factor; 0 = choose (plan_prefill), within what
+// `scratch` can hold as f32 partial sums.
 // `scratch` (scratch_bytes) holds the f16 copy of f32 activations and / or the split-K partials; when it
 // cannot hold all M rows the rows are processed in slabs.
 hipError_t launch_prefill(hipStream_t s, const WeightView &w, const void *a, bool a_f32, uint32_t m, const OutSpec &out,
                           uint32_t block_rows, uint32_t splits, void *scratch, size_t scratch_bytes)
 {
     if (m == 0 || w.n == 0) return hipSuccess;
-    if (block_rows == 0) {
-        size_t wg128 = (size_t)((m + 127) / 128) * ((w.n_tiles + 15) / 16);
-        block_rows = wg128 >= 256 ? 128 : 64;
-    }
-    if (block_rows != 64 && block_rows != 128) return hipErrorInvalidValue;
+    if (block_rows != 0 && block_rows != 64 && block_rows != 128) return hipErrorInvalidValue;
     const size_t n_ld = (size_t)w.n_tiles * 16;
     auto run = [&](const _Float16 *a16, uint32_t rows, const OutSpec &o, void *ws, size_t ws_bytes) {
-        uint32_t sp = splits;
-        if (sp == 0) sp = pick_prefill_splits(rows, block_rows, (w.n_tiles + 15) / 16, w.k_chunks, n_ld);
+        PrefillPlan plan = plan_prefill(rows, block_rows, splits, (w.n_tiles + 15) / 16, w.k_chunks, n_ld);
         size_t per_split = (size_t)rows * n_ld * 4;
-        if (!ws || per_split == 0) sp = 1;
-        else if (sp > ws_bytes / per_split) sp = (uint32_t)(ws_bytes / per_split);
-        if (sp < 2) sp = 1;
-        return block_rows == 64 ? launch_prefill_t<4>(s, w, a16, rows, o, sp, (float *)ws)
-                                : launch_prefill_t<8>(s, w, a16, rows, o, sp, (float *)ws);
+        if (plan.splits > 1 && (!ws || per_split == 0 || plan.splits > ws_bytes / per_split)) {
+            // the scratch cannot hold that many partial sums: plan again within what it holds (at least unsplit)
+            uint32_t cap = (!ws || per_split == 0) ? 1u : (uint32_t)(ws_bytes / per_split);
+            if (cap < 2) cap = 1;
+            if (splits) plan.splits = cap;  // a forced factor is cut, the forced height kept
+            else {
+                PrefillPlan capped = {0, 0, 1e30};
+                for (uint32_t sp = 1; sp <= cap; sp++) {
+                    PrefillPlan c = plan_prefill(rows, block_rows, sp, (w.n_tiles + 15) / 16, w.k_chunks, n_ld);
+                    if (c.us < capped.us) capped = c;
+                }
+                plan = capped;
+            }
+        }
+        return plan.block_rows == 64 ? launch_prefill_t<4>(s, w, a16, rows, o, plan.splits, (float *)ws)
+                                     : launch_prefill_t<8>(s, w, a16, rows, o, plan.splits, (float *)ws);
     };
     if (!a_f32) return run((const _Float16 *)a, m, out, scratch, scratch_bytes);
     // f16 copy of the activations at the front of the scratch, partials behind it
@@ -506,7 +530,7 @@ hipError_t launch_prefill(hipStream_t s, const WeightView &w, const void *a, boo
     if (!scratch || scratch_bytes < row_bytes) return hipErrorInvalidValue;
     uint32_t slab = (uint32_t)(scratch_bytes / 2 / row_bytes < m ? scratch_bytes / 2 / row_bytes : m);
     if (slab == 0) slab = 1;
-    if (slab >= block_rows) slab -= slab % block_rows;
+    if (slab >= 128) slab -= slab % 128;
     for (uint32_t r0 = 0; r0 < m; r0 += slab) {
         uint32_t rows = m - r0 < slab ? m - r0 : slab;
         size_t n4 = (size_t)rows * w.k / 4;  // k is a multiple of 32
