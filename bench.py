@@ -152,6 +152,9 @@ def main():
     ap.add_argument("--sweep-splits", action="store_true",
                     help="also time every projection at M=1,4,8,16,32 with forced split-K factors next to the library's "
                          "own choice (batched decode configuration)")
+    ap.add_argument("--sweep-prefill", action="store_true",
+                    help="also time the prefill GEMM at M = 128 .. 2048 with the library's own block height and split-K "
+                         "against forced ones")
     ap.add_argument("--pmc-copy", action="store_true",
                     help="also run four 64 MiB device-to-device copies: a kernel of known traffic to scale rocprofv3 "
                          "FETCH_SIZE / WRITE_SIZE readings by")
@@ -574,6 +577,34 @@ def main():
                 a_m.free()
                 c_m.free()
 
+    prefill_sweep = None
+    if args.sweep_prefill:
+        # block height (64 / 128 rows per workgroup) x split-K forced against the library's plan; the plan is timed
+        # after the forced cases, every case after ~200 untimed launches
+        prefill_sweep = {}
+        for k, n in ((4096, 11008), (11008, 4096), (3584, 37888), (18944, 3584), (3584, 4608)):
+            packed = rng.integers(0, 256, size=(k // 32) * n * 16, dtype=np.uint8)
+            scales = (np.abs(rng.standard_normal((k // 32) * n, dtype=np.float32)) * np.float32(0.02)).astype(np.float16)
+            w = T.MarlinWeight.upload(dev, packed, scales.view(np.uint16), k, n)
+            for m in (128, 256, 512, 1024, 2048):
+                a_m = T.GpuTensor.from_host(dev, rng.standard_normal((m, k), dtype=np.float32).astype(np.float16).view(np.uint16), "f16")
+                c_m = T.GpuTensor.zeros(dev, (m, n), "f32")
+                row = {}
+                for bm, sp in ((64, 1), (64, 2), (64, 4), (128, 1), (128, 2), (128, 4), (0, 0)):
+                    dev.set_option("prefill_bm", bm)
+                    for _ in range(200):
+                        T.gemm(dev, w, a_m, m, c_m, sp)
+                    dev.synchronize()
+                    us = min(time_launches(dev, lambda i: T.gemm(dev, w, a_m, m, c_m, sp), 20, settle_ms=0) for _ in range(3)) * 1e3
+                    row["auto" if bm == 0 else "%dx%d" % (bm, sp)] = round(us, 1)
+                dev.set_option("prefill_bm", 0)
+                best = min((v, key) for key, v in row.items() if key != "auto")
+                prefill_sweep["K%d_N%d_M%d" % (k, n, m)] = {"us": row, "auto_over_best": round(row["auto"] / best[0], 3),
+                                                            "auto_TFLOPs": round(2.0 * m * n * k / row["auto"] / 1e6, 1)}
+                a_m.free()
+                c_m.free()
+            w.free()
+
     log("cpu baseline")
     cpu = None
     if not args.no_cpu:
@@ -652,6 +683,8 @@ def main():
         out["batched_decode"] = extra
     if sweep:
         out["split_sweep"] = sweep
+    if prefill_sweep is not None:
+        out["prefill_sweep"] = prefill_sweep
     print(json.dumps(out))
     for g in graphs + [graph_all] + graphs_done:
         g.destroy()
