@@ -1030,6 +1030,17 @@ static int gemm_common(twm_ctx *ctx, const twm_weight *w, const void *a_dev, int
                     TWM_DEVICE_ERROR, "sub-tile gemv launch");
             return TWM_OK;
         }
+        if (m <= 8 && !ctx->force_nt && !splits) {
+            // M = 5 .. 8 elsewhere: the 64-column lane-per-column kernel with two row groups, which unpacks with
+            // fewer vector instructions than the streaming kernel (3584 -> 37888 at M = 8: 18.0 against 19.2 us,
+            // 3584 -> 152064: 54.8 against 60.0; with four row groups, M = 9 .. 16, it needs 127 registers and loses)
+            DecodePlan plan = plan_gemv4(w->n_tiles, w->k_chunks, 1, ctx->force_waves, 0);
+            while (plan.splits > 1 && (size_t)plan.splits * m * n_ld * 4 > ctx->ws_bytes) plan.splits--;
+            if (w->n_tiles / plan.nt > ctx->n_counters) plan.splits = 1;
+            HIP_TRY(launch_gemv4(ctx->stream, v, a_dev, false, m, gated, ctx->ws, ctx->counters, 1, plan.waves, plan.splits, swiglu_out),
+                    TWM_DEVICE_ERROR, "gemv launch");
+            return TWM_OK;
+        }
     }
     if (ctx->force_kernel == 3 || (ctx->force_kernel == 0 && m > 4)) {
         // batched decode: 32-row blocks of the streaming kernel

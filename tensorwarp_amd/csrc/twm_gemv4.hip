@@ -79,18 +79,19 @@ __global__ __launch_bounds__(1024) void k_gemv4(const char *__restrict__ cw, con
 #pragma unroll
         for (int r = 0; r < RL; r++) acc[t][r] = 0.f;
 
-    auto load_chunk = [&](Chunk4<NT> &r, uint32_t kc) {
+    constexpr int RG = (RL + 3) / 4;  // rows beyond four repeat the MFMA chain (f16 activations)
+    auto load_chunk = [&](Chunk4<NT, RG> &r, uint32_t kc) {
         if constexpr (REFL)
             gemv4_load_chunk_ref<NT>(r, cw, ref_scales, tg * NT, kc, lane, n, k / 32u, (const float *)a_any, apiece, k,
                                      lane_is_lo);
         else
-            gemv4_load_chunk<NT, AF32, TERMS>(r, wbase, kc, lane16, lane8, a_any, arow, apiece, k, lane_is_lo);
+            gemv4_load_chunk<NT, AF32, TERMS, RG>(r, wbase, kc, lane16, lane8, a_any, arow, apiece, k, lane_is_lo, m_rows);
     };
-    auto compute_chunk = [&](const Chunk4<NT> &r) { gemv4_compute_chunk<NT, RL, TERMS>(r, dq, acc); };
+    auto compute_chunk = [&](const Chunk4<NT, RG> &r) { gemv4_compute_chunk<NT, RL, TERMS>(r, dq, acc); };
 
     {
         // two register sets used alternately: the loads of one are in flight while the other is consumed
-        Chunk4<NT> r0, r1;
+        Chunk4<NT, RG> r0, r1;
         uint32_t kc = kc0 + wave;
         if (kc < kc1) {
             load_chunk(r0, kc);
@@ -211,11 +212,14 @@ static hipError_t launch_gemv4_t(hipStream_t s, const WeightView &w, const void 
     splits = (w.k_chunks + cps - 1) / cps;               // no empty split
     uint32_t blocks = ((tile_groups + 7) / 8) * 8 * splits;
     size_t lds = (size_t)waves * NT * RL * 64 * sizeof(float);
-    if (a_f32)
-        hipLaunchKernelGGL((k_gemv4<NT, RL, true>), dim3(blocks), dim3(waves * 64), lds, s, (const char *)w.cq, a, out, ws,
-                           counters, m, w.k, w.n, n_pad, w.k_chunks, tile_groups,
-                           splits, cps, swiglu_out);
-    else
+    if (a_f32) {
+        if constexpr (RL <= 4)
+            hipLaunchKernelGGL((k_gemv4<NT, RL, true>), dim3(blocks), dim3(waves * 64), lds, s, (const char *)w.cq, a, out, ws,
+                               counters, m, w.k, w.n, n_pad, w.k_chunks, tile_groups,
+                               splits, cps, swiglu_out);
+        else
+            return hipErrorInvalidValue;  // more than four rows: f16 activations only
+    } else
         hipLaunchKernelGGL((k_gemv4<NT, RL, false>), dim3(blocks), dim3(waves * 64), lds, s, (const char *)w.cq, a, out, ws,
                            counters, m, w.k, w.n, n_pad, w.k_chunks, tile_groups,
                            splits, cps, swiglu_out);
@@ -252,7 +256,7 @@ hipError_t launch_gemv4(hipStream_t s, const WeightView &w, const void *a, bool 
 {
     if (m == 0 || w.n == 0) return hipSuccess;
     if (swiglu_out && w.n % 64 != 0) return hipErrorInvalidValue;
-    if (m > 4 || splits == 0 || !w.cq) return hipErrorInvalidValue;
+    if (m > 8 || (m > 4 && (a_f32 || nt != 1)) || splits == 0 || !w.cq) return hipErrorInvalidValue;
     if (waves != 1 && waves != 2 && waves != 4 && waves != 8 && waves != 16) return hipErrorInvalidValue;
     // a tile group past the end of the padded columns must not exist: NT has to divide the 64-column tile count
     uint32_t tiles64 = w.n_tiles * kTileN / 64;
@@ -261,7 +265,9 @@ hipError_t launch_gemv4(hipStream_t s, const WeightView &w, const void *a, bool 
     if (nt == 1) {
         if (rl == 1) return launch_gemv4_t<1, 1>(s, w, a, a_f32, m, out, ws, counters, waves, splits, swiglu_out);
         if (rl == 2) return launch_gemv4_t<1, 2>(s, w, a, a_f32, m, out, ws, counters, waves, splits, swiglu_out);
-        return launch_gemv4_t<1, 4>(s, w, a, a_f32, m, out, ws, counters, waves, splits, swiglu_out);
+        if (rl <= 4) return launch_gemv4_t<1, 4>(s, w, a, a_f32, m, out, ws, counters, waves, splits, swiglu_out);
+        // five to eight rows (f16): a second group of four rows repeats the MFMA chain on the unpacked weights
+        return launch_gemv4_t<1, 8>(s, w, a, a_f32, m, out, ws, counters, waves, splits, swiglu_out);
     }
     if (nt == 2) {
         if (rl == 1) return launch_gemv4_t<2, 1>(s, w, a, a_f32, m, out, ws, counters, waves, splits, swiglu_out);

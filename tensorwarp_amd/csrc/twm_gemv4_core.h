@@ -47,11 +47,12 @@ __device__ __forceinline__ void gemv4_dequant_word(uint32_t w, const Gemv4Consts
     hi4 = b.h;
 }
 
-template <int NT>
+// RG = row groups of four: rows 4 .. 4*RG-1 repeat the MFMA chain on the same unpacked weights (f16 rows only).
+template <int NT, int RG = 1>
 struct Chunk4 {
     uint4v wq[NT][4];  // [tile][group in chunk]: this lane's column, 32 nibbles
     uint2v sc[NT];     // four f16 scales
-    uint4v a;          // activations: row lane%4, k-piece lane/4 (8 halves)
+    uint4v a[RG];      // activations: row 4*rg + lane%4, k-piece lane/4 (8 halves)
     uint4v a_lo;       // f32 activations only: the f16 residuals a - f16(a) of the same eight values
 };
 
@@ -88,11 +89,12 @@ constexpr int gemv4_terms() { return AF32 ? (RL <= 2 ? kTermsRowPacked : kTermsT
 
 // arow: the activation row this lane reads (see the term modes); lane_is_lo: row-packed mode, this lane holds
 // the residual term
-template <int NT, bool AF32, int TERMS = AF32 ? kTermsTwoPasses : kTermsOne>
-__device__ __forceinline__ void gemv4_load_chunk(Chunk4<NT> &r, const char *(&wbase)[NT], uint32_t kc,
+template <int NT, bool AF32, int TERMS = AF32 ? kTermsTwoPasses : kTermsOne, int RG = 1>
+__device__ __forceinline__ void gemv4_load_chunk(Chunk4<NT, RG> &r, const char *(&wbase)[NT], uint32_t kc,
                                                  uint32_t lane16, uint32_t lane8, const void *a_any, uint32_t arow,
-                                                 uint32_t apiece, uint32_t k, bool lane_is_lo = false)
+                                                 uint32_t apiece, uint32_t k, bool lane_is_lo = false, uint32_t m_rows = 0)
 {
+    static_assert(RG == 1 || !AF32, "more than four rows: f16 activations only");
 #pragma unroll
     for (int t = 0; t < NT; t++) {
         const char *blk = wbase[t] + (size_t)kc * kColBlockBytes;
@@ -106,13 +108,18 @@ __device__ __forceinline__ void gemv4_load_chunk(Chunk4<NT> &r, const char *(&wb
         const float4 *p = (const float4 *)((const float *)a_any + (size_t)arow * k + k0);
         float4 x = p[0], y = p[1];
         const float v[8] = {x.x, x.y, x.z, x.w, y.x, y.y, y.z, y.w};
-        split_f32x8(v, r.a, r.a_lo);
+        split_f32x8(v, r.a[0], r.a_lo);
         if (TERMS == kTermsRowPacked) {
 #pragma unroll
-            for (int i = 0; i < 4; i++) r.a[i] = lane_is_lo ? r.a_lo[i] : r.a[i];
+            for (int i = 0; i < 4; i++) r.a[0][i] = lane_is_lo ? r.a_lo[i] : r.a[0][i];
         }
     } else {
-        r.a = *(const uint4v *)((const _Float16 *)a_any + (size_t)arow * k + k0);
+#pragma unroll
+        for (int rg = 0; rg < RG; rg++) {
+            uint32_t row = arow + 4u * rg;
+            if (RG > 1 && row > m_rows - 1u) row = m_rows - 1u;
+            r.a[rg] = *(const uint4v *)((const _Float16 *)a_any + (size_t)row * k + k0);
+        }
     }
 }
 
@@ -122,7 +129,7 @@ __device__ __forceinline__ void gemv4_load_chunk(Chunk4<NT> &r, const char *(&wb
 // The nibbles are in their natural order here, which the mask-and-magic unpack turns into the k order
 // (0,4,1,5 | 2,6,3,7) per eight; the f32 activations (one row) are converted into that same order.
 template <int NT>
-__device__ __forceinline__ void gemv4_load_chunk_ref(Chunk4<NT> &r, const char *packed, const uint16_t *scales,
+__device__ __forceinline__ void gemv4_load_chunk_ref(Chunk4<NT, 1> &r, const char *packed, const uint16_t *scales,
                                                      uint32_t tile0, uint32_t kc, uint32_t lane, uint32_t n,
                                                      uint32_t groups, const float *a, uint32_t apiece, uint32_t k,
                                                      bool lane_is_lo)
@@ -148,19 +155,22 @@ __device__ __forceinline__ void gemv4_load_chunk_ref(Chunk4<NT> &r, const char *
     const float4 *p = (const float4 *)(a + k0);
     float4 x = p[0], y = p[1];
     const float v[8] = {x.x, y.x, x.y, y.y, x.z, y.z, x.w, y.w};
-    split_f32x8(v, r.a, r.a_lo);
+    split_f32x8(v, r.a[0], r.a_lo);
 #pragma unroll
-    for (int i = 0; i < 4; i++) r.a[i] = lane_is_lo ? r.a_lo[i] : r.a[i];  // one row: row-packed terms
+    for (int i = 0; i < 4; i++) r.a[0][i] = lane_is_lo ? r.a_lo[i] : r.a[0][i];  // one row: row-packed terms
 }
 
 // acc[t][row] += f32(scale) * (sum over the group of A * (q - 8)) for the four groups of the chunk
 template <int NT, int RL, int TERMS = kTermsOne>
-__device__ __forceinline__ void gemv4_compute_chunk(const Chunk4<NT> &r, const Gemv4Consts &dq, float (&acc)[NT][RL])
+__device__ __forceinline__ void gemv4_compute_chunk(const Chunk4<NT, (RL + 3) / 4> &r, const Gemv4Consts &dq, float (&acc)[NT][RL])
 {
     constexpr bool A2 = TERMS == kTermsTwoPasses;
+    constexpr int RG = (RL + 3) / 4;
     static_assert(TERMS != kTermsRowPacked || RL <= 2, "row-packed terms hold at most two rows");
-    union { uint4v u; half4v h[2]; } av, al;
-    av.u = r.a;  // h[0] = k 0..3 of the lane's piece, h[1] = k 4..7
+    static_assert(RG == 1 || TERMS == kTermsOne, "more than four rows: one f16 term");
+    union { uint4v u; half4v h[2]; } av[RG], al;
+#pragma unroll
+    for (int rg = 0; rg < RG; rg++) av[rg].u = r.a[rg];  // h[0] = k 0..3 of the lane's piece, h[1] = k 4..7
     if (A2) al.u = r.a_lo;
 #pragma unroll
     for (int t = 0; t < NT; t++) {
@@ -168,15 +178,19 @@ __device__ __forceinline__ void gemv4_compute_chunk(const Chunk4<NT> &r, const G
         sv.u = r.sc[t];
 #pragma unroll
         for (int g = 0; g < 4; g++) {
-            float4v d = {0.f, 0.f, 0.f, 0.f};
+            float4v d[RG];
+#pragma unroll
+            for (int rg = 0; rg < RG; rg++) d[rg] = float4v{0.f, 0.f, 0.f, 0.f};
             half4v lo4, hi4;
 #define TWM_PIECE(W, PIECE)                                       \
     gemv4_dequant_word(r.wq[t][g][W], dq, lo4, hi4);              \
-    d = mfma_piece<PIECE>(av.h[0], lo4, d);                       \
-    d = mfma_piece<PIECE>(av.h[1], hi4, d);                       \
+    _Pragma("unroll") for (int rg = 0; rg < RG; rg++) {           \
+        d[rg] = mfma_piece<PIECE>(av[rg].h[0], lo4, d[rg]);       \
+        d[rg] = mfma_piece<PIECE>(av[rg].h[1], hi4, d[rg]);       \
+    }                                                             \
     if (A2) {                                                     \
-        d = mfma_piece<PIECE>(al.h[0], lo4, d);                   \
-        d = mfma_piece<PIECE>(al.h[1], hi4, d);                   \
+        d[0] = mfma_piece<PIECE>(al.h[0], lo4, d[0]);             \
+        d[0] = mfma_piece<PIECE>(al.h[1], hi4, d[0]);             \
     }
             if (g == 0) { TWM_PIECE(0, 0) TWM_PIECE(1, 1) TWM_PIECE(2, 2) TWM_PIECE(3, 3) }
             if (g == 1) { TWM_PIECE(0, 4) TWM_PIECE(1, 5) TWM_PIECE(2, 6) TWM_PIECE(3, 7) }
@@ -186,8 +200,8 @@ __device__ __forceinline__ void gemv4_compute_chunk(const Chunk4<NT> &r, const G
             float s = (float)sv.h[g];
 #pragma unroll
             for (int rr = 0; rr < RL; rr++) {
-                if (TERMS == kTermsRowPacked) acc[t][rr] = fmaf(d[2 * rr] + d[2 * rr + 1], s, acc[t][rr]);
-                else acc[t][rr] = fmaf(d[rr], s, acc[t][rr]);
+                if (TERMS == kTermsRowPacked) acc[t][rr] = fmaf(d[0][2 * rr] + d[0][2 * rr + 1], s, acc[t][rr]);
+                else acc[t][rr] = fmaf(d[rr / 4][rr % 4], s, acc[t][rr]);
             }
         }
     }

@@ -660,6 +660,48 @@ def test_sub_tile_gated_store(dev):
         w.free()
 
 
+def test_five_to_eight_rows_on_wide_matrices(dev):
+    # M = 5 .. 8 with f16 rows on more than 128 column tiles: the 64-column lane-per-column kernel with two row
+    # groups (f32 rows and forced split factors keep the streaming kernel); both against the oracle
+    k, n = 416, 9000
+    packed, scales, a16 = synth(k, n, 8, 4500)
+    w = T.MarlinWeight.upload(dev, packed, scales, k, n)
+    try:
+        for m in (5, 6, 7, 8):
+            truth = gemm_truth(a16[:m], packed, scales, m, k, n)
+            got = run_gemm(dev, w, a16[:m], m, n)
+            assert rel_err(got, truth) < TIGHT, m
+            dev.set_option("kernel", 3)
+            streamed = run_gemm(dev, w, a16[:m], m, n)
+            dev.set_option("kernel", 0)
+            assert rel_err(streamed, truth) < TIGHT, m
+            assert rel_err(got, streamed) < 1e-4, m
+            assert rel_err(run_gemm(dev, w, a16[:m], m, n, a_f32=True), truth) < TIGHT, m
+            for waves in (1, 16):
+                dev.set_option("waves", waves)
+                assert rel_err(run_gemm(dev, w, a16[:m], m, n), truth) < TIGHT, (m, waves)
+            dev.set_option("waves", 0)
+    finally:
+        dev.set_option("kernel", 0)
+        dev.set_option("waves", 0)
+    w.free()
+    # the gated store of the same kernel
+    h, ffn = 288, 4608
+    gp, gs = O.synth_packed(h, ffn, 4510), O.synth_scales(h, ffn, 4511)
+    up, us = O.synth_packed(h, ffn, 4512), O.synth_scales(h, ffn, 4513)
+    gd = (T.GpuTensor.from_host(dev, gp), T.GpuTensor.from_host(dev, gs, "f16"))
+    ud = (T.GpuTensor.from_host(dev, up), T.GpuTensor.from_host(dev, us, "f16"))
+    wp = T.MarlinWeight.gate_up(dev, gd, ud, h, ffn)
+    for m in (5, 8):
+        a16 = O.synth_act_f16(m, h, 4514 + m)
+        a = f16_as_f32(a16).reshape(m, h)
+        tg, tu = O.gemm_f64(a, gp, gs, m, h, ffn), O.gemm_f64(a, up, us, m, h, ffn)
+        out = T.GpuTensor.from_host(dev, np.full((m, ffn), np.nan, np.float32))
+        T.gemm_swiglu(dev, wp, T.GpuTensor.from_host(dev, a16, "f16"), m, out)
+        assert rel_err(out.to_host(), tg / (1.0 + np.exp(-tg)) * tu) < TIGHT, m
+    wp.free()
+
+
 def test_split_factors_that_do_not_divide_the_k_chunks(dev):
     # 28 k-chunks: 8, 9, 11, 12, 13 ... splits leave trailing splits without any chunk; the launch
     # must fold them away (an empty split used to read past the end of the weight array)
