@@ -1,4 +1,5 @@
-// Sub-tile variant of the M <= 4 decode kernel: finer workgroups without a cross-workgroup reduction.
+// Sub-tile variant of the lane-per-column decode kernel (M <= 4; up to M = 16 with f16 rows): finer workgroups
+// without a cross-workgroup reduction.
 //
 // k_gemv4 gives a workgroup a whole 64-column tile; with 592 tiles on 256 CUs that is 2.3 long-lived
 // workgroups per CU, and a plain read of the same bytes in that decomposition is 1.3 - 1.6 us slower than in
@@ -8,8 +9,10 @@
 // bytes).  The 4x4x4 MFMA broadcasts its A block inside groups of 2^CBSZ blocks, so with CBSZ = log2(SUB / 4)
 // every group of SUB lanes takes the activations of its own chunk: one A register holds 2 * SUB of the
 // chunk's 128 k-values (SUB / 4 pieces of eight), 64 / SUB registers the whole chunk.  The MFMA count per
-// byte of weights is unchanged (every lane of every MFMA is a live column).  With 28 chunks and SUB = 32 a
-// workgroup of 14 waves makes exactly one pass: every load of the launch is issued at once.
+// byte of weights is unchanged (every lane of every MFMA is a live column).  With 28 chunks and SUB = 16 a
+// workgroup of eight waves makes exactly one pass: every load of the launch is issued at once, the kernel has
+// no loop and needs about 50 registers, and 3584 -> 37888 becomes 2368 short-lived workgroups.
+// Rows five to sixteen (f16) repeat the MFMA chain on the unpacked weights per group of four rows.
 //
 // Arithmetic and output as k_gemv4 (crates/kernels/src/quantize.rs:1186-1298).
 #include "twm_gemv4_core.h"
