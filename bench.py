@@ -155,6 +155,9 @@ def main():
     ap.add_argument("--sweep-prefill", action="store_true",
                     help="also time the prefill GEMM at M = 128 .. 2048 with the library's own block height and split-K "
                          "against forced ones")
+    ap.add_argument("--sweep-models", action="store_true",
+                    help="also time the projections of other model sizes (Llama-3-8B, 13B, 70B, Qwen-1.5B shapes) at "
+                         "M = 1, 4, 8, 16 with the library's plan against the 64-column / streaming kernels alone")
     ap.add_argument("--pmc-copy", action="store_true",
                     help="also run four 64 MiB device-to-device copies: a kernel of known traffic to scale rocprofv3 "
                          "FETCH_SIZE / WRITE_SIZE readings by")
@@ -577,6 +580,46 @@ def main():
                 a_m.free()
                 c_m.free()
 
+    model_sweep = None
+    if args.sweep_models:
+        # the planner away from the shapes it was fitted on: option "sub" = 1 (and "kernel" = 3 from M = 5 on) keeps
+        # the 64-column lane-per-column kernel / the streaming kernel, 0 is the library's plan
+        model_sweep = {}
+        other = [("llama3_8b_qkv", 4096, 6144), ("llama3_8b_o", 4096, 4096), ("llama3_8b_gate_up", 4096, 28672),
+                 ("llama3_8b_down", 14336, 4096), ("13b_qkv", 5120, 15360), ("13b_down", 13824, 5120),
+                 ("70b_qkv", 8192, 10240), ("70b_o", 8192, 8192), ("70b_gate_up", 8192, 57344), ("70b_down", 28672, 8192),
+                 ("qwen15b_qkv", 1536, 2048), ("qwen15b_gate_up", 1536, 17920), ("qwen15b_down", 8960, 1536)]
+        for name, k, n in other:
+            sets = []
+            for _ in range(max(3, min(12, int(600e6 // (k * n * 0.5625)) + 1))):
+                packed = rng.integers(0, 256, size=(k // 32) * n * 16, dtype=np.uint8)
+                scales = (np.abs(rng.standard_normal((k // 32) * n, dtype=np.float32)) * np.float32(0.02)).astype(np.float16)
+                sets.append(T.MarlinWeight.upload(dev, packed, scales.view(np.uint16), k, n))
+            for m, dt in ((1, "f16"), (1, "f32"), (4, "f16"), (8, "f16"), (16, "f16")):
+                ah = rng.standard_normal((m, k), dtype=np.float32)
+                a_m = (T.GpuTensor.from_host(dev, ah.astype(np.float16).view(np.uint16), "f16") if dt == "f16"
+                       else T.GpuTensor.from_host(dev, ah))
+                c_m = T.GpuTensor.zeros(dev, (m, n), "f32")
+
+                def one(i, a_m=a_m, c_m=c_m, m=m, sets=sets):
+                    T.gemm(dev, sets[i % len(sets)], a_m, m, c_m)
+                row = {}
+                for label in ("whole_tiles", "plan"):
+                    dev.set_option("sub", 1 if label == "whole_tiles" else 0)
+                    dev.set_option("kernel", 3 if (label == "whole_tiles" and m > 4) else 0)
+                    for i in range(8):
+                        one(i)
+                    dev.synchronize()
+                    row[label] = round(time_short_launches(dev, T, one, 96, graphs_done, below_ms=1.0)[0] * 1e3, 2)
+                dev.set_option("sub", 0)
+                dev.set_option("kernel", 0)
+                row["plan_GBps"] = round(algo_bytes(k, n, m) / (row["plan"] * 1e-6) / 1e9, 1)
+                model_sweep["%s_K%d_N%d_M%d_%s" % (name, k, n, m, dt)] = row
+                a_m.free()
+                c_m.free()
+            for w in sets:
+                w.free()
+
     prefill_sweep = None
     if args.sweep_prefill:
         # block height (64 / 128 rows per workgroup) x split-K forced against the library's plan; the plan is timed
@@ -685,6 +728,8 @@ def main():
         out["split_sweep"] = sweep
     if prefill_sweep is not None:
         out["prefill_sweep"] = prefill_sweep
+    if model_sweep is not None:
+        out["model_sweep"] = model_sweep
     print(json.dumps(out))
     for g in graphs + [graph_all] + graphs_done:
         g.destroy()

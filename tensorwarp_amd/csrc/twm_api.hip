@@ -927,8 +927,10 @@ static SubPlan plan_gemv4_sub(uint32_t tiles64, uint32_t k_chunks, uint32_t m, b
     if (tiles64 > 128) {
         // wide matrices: only the cheapest activations (f16, up to two rows) leave the sub-tiles ahead
         // (3584 -> 37888: 15.8 against 17.0 us at M = 1, 18.3 against 17.3 at M = 4, 19.9 against 17.9 with f32 rows)
-        if (!a_f32 && m <= 2) return narrow16;
-        if (a_f32 && m <= 2 && tiles64 < 256) return SubPlan{32, 16};
+        // and only while every wave gets exactly one pass (K <= 4096): beyond that the 64-column kernel is ahead
+        // again (5120 -> 15360: 9.2 against 12.5 us; 8192 -> 57344: 42.3 against 49.7)
+        if (!a_f32 && m <= 2 && passes16 <= 8) return narrow16;
+        if (a_f32 && m <= 2 && tiles64 < 256 && k_chunks <= 32) return SubPlan{32, 16};
         return none;
     }
     if (two_pass && passes16 > 16) return k_chunks <= 100 ? SubPlan{32, 8} : none;  // (the looping 16-column variant spills)
@@ -1030,10 +1032,11 @@ static int gemm_common(twm_ctx *ctx, const twm_weight *w, const void *a_dev, int
                     TWM_DEVICE_ERROR, "sub-tile gemv launch");
             return TWM_OK;
         }
-        if (m <= 8 && !ctx->force_nt && !splits) {
-            // M = 5 .. 8 elsewhere: the 64-column lane-per-column kernel with two row groups, which unpacks with
+        if (m <= 8 && n_ld / 64 > 128 && !ctx->force_nt && !splits) {
+            // M = 5 .. 8 on wide matrices: the 64-column lane-per-column kernel with two row groups, which unpacks with
             // fewer vector instructions than the streaming kernel (3584 -> 37888 at M = 8: 18.0 against 19.2 us,
-            // 3584 -> 152064: 54.8 against 60.0; with four row groups, M = 9 .. 16, it needs 127 registers and loses)
+            // 3584 -> 152064: 54.8 against 60.0; with four row groups, M = 9 .. 16, it needs 127 registers and loses;
+            // on 128 tiles or fewer the streaming kernel's split-K is ahead: 14336 -> 4096 11.4 against 19.8 us)
             DecodePlan plan = plan_gemv4(w->n_tiles, w->k_chunks, 1, ctx->force_waves, 0);
             while (plan.splits > 1 && (size_t)plan.splits * m * n_ld * 4 > ctx->ws_bytes) plan.splits--;
             if (w->n_tiles / plan.nt > ctx->n_counters) plan.splits = 1;
