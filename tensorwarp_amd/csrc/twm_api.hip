@@ -541,23 +541,25 @@ int twm_gemm_tw_marlin_m1(twm_ctx *ctx, const float *a_dev, const uint8_t *packe
     uint32_t n_pad = ((n + 63) / 64) * 64, k_chunks = (k / 32 + kChunkGroups - 1) / kChunkGroups;
     // On the reference's arrays a wave's four group rows of a chunk are N x 16 bytes apart, and many waves in flight
     // with one pass each pay better than on the contiguous copy: the sub-tile kernel with sixteen waves on 32
-    // columns, or with 16 columns when 64-column tiles number no more than 64; a very deep K is cut in two
-    // (fitted to a sweep over the benchmark shapes; option "sub" = 1 keeps the 64-column kernel).
-    const uint32_t tiles64 = n_pad / 64, passes16 = (k_chunks + 3) / 4;
-    if (ctx->force_sub != 1) {
-        uint32_t sub = tiles64 <= 64 ? 16 : 32, waves = (sub == 16 && passes16 <= 8) ? 8 : 16, sp = 1;
-        if (passes16 > 32) { sub = 32; waves = 16; sp = 2; }
-        if (ctx->force_sub >= 16) {
-            sub = (uint32_t)ctx->force_sub;
-            waves = 8;
-            sp = 1;
-        }
-        if (ctx->force_waves) waves = (uint32_t)ctx->force_waves;
-        if (ctx->m1_splits) sp = (uint32_t)ctx->m1_splits;
+    // columns, or with 16 columns when 64-column tiles number no more than 64 -- as long as every wave gets a
+    // single pass (K <= 4096, or 8192 on 16 columns).  Deeper matrices keep the 64-column kernel and its split-K
+    // (8192 -> 57344: 46.6 against 63.7 us; 14336 -> 4096: 11.0 against 12.5).  Fitted to sweeps over the
+    // Qwen2.5-7B, Llama-3-8B, 13B and 70B projections; option "sub" = 1 keeps the 64-column kernel.
+    const uint32_t tiles64 = n_pad / 64, passes16 = (k_chunks + 3) / 4, passes32 = (k_chunks + 1) / 2;
+    uint32_t sub = tiles64 <= 64 ? 16 : 32, sub_waves = (sub == 16 && passes16 <= 8) ? 8 : 16;
+    bool use_sub = ctx->force_sub != 1 && (sub == 16 ? passes16 : passes32) <= 16;
+    if (ctx->force_sub >= 16) {
+        sub = (uint32_t)ctx->force_sub;
+        sub_waves = 8;
+        use_sub = true;
+    }
+    if (use_sub) {
+        uint32_t sp = ctx->m1_splits ? (uint32_t)ctx->m1_splits : 1;
+        if (ctx->force_waves) sub_waves = (uint32_t)ctx->force_waves;
         if (sp > k_chunks) sp = k_chunks;
         while (sp > 1 && (size_t)sp * n_pad * 4 > ctx->ws_bytes) sp--;
         if (n_pad / sub > ctx->n_counters) sp = 1;
-        HIP_TRY(launch_gemv4s_ref(ctx->stream, packed_dev, scales_dev, k, n, a_dev, c_dev, ctx->ws, ctx->counters, sub, waves, sp),
+        HIP_TRY(launch_gemv4s_ref(ctx->stream, packed_dev, scales_dev, k, n, a_dev, c_dev, ctx->ws, ctx->counters, sub, sub_waves, sp),
                 TWM_DEVICE_ERROR, "sub-tile gemv launch");
         return TWM_OK;
     }
