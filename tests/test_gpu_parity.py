@@ -784,6 +784,28 @@ def test_random_shapes_against_the_oracle(dev):
         w.free()
 
 
+def test_random_deep_shapes_against_the_oracle(dev):
+    # the same with K from 2048 to 6400, where the planners take sub-tiles, row groups or whole tiles by shape:
+    # narrow, middling and wide N (up to 64, 128 and more column tiles), one to sixteen rows
+    rng = np.random.default_rng(20251101)
+    for case in range(20):
+        k = 32 * int(rng.integers(64, 201))
+        n = int(rng.choice([16, 72, 200, 1000, 4100, 6000, 8300]))
+        m = int(rng.choice([1, 1, 2, 3, 4, 5, 8, 12, 16]))
+        a_f32 = bool(rng.integers(0, 2))
+        print("case %d: k=%d n=%d m=%d f32=%d" % (case, k, n, m, a_f32), flush=True)
+        packed, scales, a16 = synth(k, n, m, 5200 + case)
+        w = T.MarlinWeight.upload(dev, packed, scales, k, n)
+        truth = gemm_truth(a16, packed, scales, m, k, n)
+        assert rel_err(run_gemm(dev, w, a16, m, n, 0, a_f32), truth) < TIGHT, (case, k, n, m, a_f32)
+        if m == 1:
+            c = T.GpuTensor.from_host(dev, np.full(n, np.nan, np.float32))
+            T.gemm_tw_marlin_m1(dev, T.GpuTensor.from_host(dev, f16_as_f32(a16)), T.GpuTensor.from_host(dev, packed),
+                                T.GpuTensor.from_host(dev, scales, "f16"), c, n, k)
+            assert rel_err(c.to_host(), truth[0]) < TIGHT, (case, "drop-in")
+        w.free()
+
+
 def test_m_larger_than_16_is_tiled_by_the_decode_kernel(dev):
     # with the prefill kernel switched off, any M runs as 16-row blocks of the exact-weight decode kernel
     m, k, n = 70, 256, 128
