@@ -931,7 +931,13 @@ static SubPlan plan_gemv4_sub(uint32_t tiles64, uint32_t k_chunks, uint32_t m, b
         // (3584 -> 37888: 15.8 against 17.0 us at M = 1, 18.3 against 17.3 at M = 4, 19.9 against 17.9 with f32 rows)
         // and only while every wave gets exactly one pass (K <= 4096): beyond that the 64-column kernel is ahead
         // again (5120 -> 15360: 9.2 against 12.5 us; 8192 -> 57344: 42.3 against 49.7)
-        if (!a_f32 && m <= 2 && passes16 <= 8) return narrow16;
+        // and where whole tiles would leave their last round of 256 workgroups under 80 % full, which is the loss the
+        // finer workgroups remove (4096 -> 22016, 344 tiles = 1.34 rounds: 10.6 against 12.1 us; 3584 -> 37888, 2.31
+        // rounds: 14.8 against 15.5; but 4096 -> 28672, 1.75 rounds: 13.2 against 12.7, and 3584 -> 152064, 9.3
+        // rounds: 49.3 against 47.8)
+        const uint32_t rounds = (tiles64 + 255) / 256;
+        const bool poor_fill = tiles64 * 5 < rounds * 256 * 4;
+        if (!a_f32 && m <= 2 && passes16 <= 8 && poor_fill) return narrow16;
         if (a_f32 && m <= 2 && tiles64 < 256 && k_chunks <= 32) return SubPlan{32, 16};
         return none;
     }
