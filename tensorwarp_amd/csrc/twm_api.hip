@@ -45,7 +45,8 @@ struct twm_ctx {
     int force_nt;         // 0 = heuristic
     int force_waves;      // 0 = heuristic
     int force_sub;        // M <= 4: 0 = heuristic, 1 = whole 64-column tiles per workgroup, 32 or 16 = the sub-tile kernel
-    int force_kernel;     // 0 = heuristic, 1 = 16-column tile kernel, 2 = one-lane-per-column kernel (M <= 4), 3 = streaming kernel (M <= 32)
+    int force_kernel;     // 0 = heuristic, 1 = 16-column tile kernel, 2 = one-lane-per-column kernel (M <= 4), 3 = streaming kernel (M <= 32),
+                          // 4 = batched-decode kernel with LDS-shared activations (M <= 32; "nt" = tiles per wave, "waves" 8 / 16 = 2 / 4 k-slices)
     int prefill_bm;       // rows of A per prefill workgroup: 0 = choose, 64 or 128
     int prefill_min_m;    // M from which the LDS/MFMA prefill kernel runs instead of 16-row decode blocks
     int dequant_src;      // which copy twm_weight_dequant_f16 unpacks: 0 = 16-column tiles, 1 = column-lane
@@ -182,7 +183,8 @@ int twm_ctx_info(twm_ctx *ctx, char *buf, size_t buf_len)
 }
 
 /* Tuning knobs for sweeps (0 = heuristic): "nt" = tiles per workgroup (1, 2, 4); "waves" = waves per
- * workgroup; "kernel" = 1 the 16-column tile kernel, 2 the one-lane-per-column kernel (M <= 4);
+ * workgroup; "kernel" = 1 the 16-column tile kernel, 2 the one-lane-per-column kernel (M <= 4), 3 the
+ * streaming kernel, 4 the batched-decode kernel with LDS-shared activations;
  * "dequant_src" = which weight copy twm_weight_dequant_f16 unpacks; "prefill_min_m" = smallest M that
  * runs the prefill kernel. */
 int twm_ctx_set_option(twm_ctx *ctx, const char *key, int value)
@@ -232,7 +234,7 @@ int twm_ctx_set_option(twm_ctx *ctx, const char *key, int value)
         return TWM_OK;
     }
     if (strcmp(key, "kernel") == 0) {
-        if (value < 0 || value > 3) return fail(TWM_SHAPE_ERROR, "twm_ctx_set_option: kernel must be 0, 1, 2 or 3");
+        if (value < 0 || value > 4) return fail(TWM_SHAPE_ERROR, "twm_ctx_set_option: kernel must be 0 .. 4");
         ctx->force_kernel = value;
         return TWM_OK;
     }
@@ -983,6 +985,23 @@ static uint32_t stream_waves(uint32_t n_tiles, uint32_t m, int force_waves)
     return (m > 16 && n_tiles / 4 >= 256) ? 4 : 8;
 }
 
+// Batched-decode kernel with LDS-shared activations: K is cut over workgroups as for the streaming kernel's 32-row
+// variant (about one workgroup per CU, seven chunks or more each); with fewer than 512 workgroups of eight chunks
+// or more, each workgroup runs two k-slices (eight waves) that add their sums through LDS
+// (18944 -> 3584 at M = 32: 4 splits x 2 slices 17.3 us, 4 x 1 about 22, 9 x 1 18.8; 3584 -> 37888, 592 quads: 1 x 1
+// 26.7, 1 x 2 28.1).
+struct BatchPlan {
+    uint32_t splits, slices;
+};
+static BatchPlan plan_batch(uint32_t n_tiles, uint32_t k_chunks, uint32_t force_splits = 0)
+{
+    BatchPlan p = {force_splits ? force_splits : plan_stream(n_tiles, k_chunks, 32), 1};
+    if (p.splits > k_chunks) p.splits = k_chunks;
+    const uint32_t chunks_per_split = (k_chunks + p.splits - 1) / p.splits;
+    if ((n_tiles / 4) * p.splits < 512 && chunks_per_split >= 8) p.slices = 2;
+    return p;
+}
+
 uint32_t twm_pick_splits(uint32_t k, uint32_t n, uint32_t m)
 {
     uint32_t n_tiles = ((n + kNPadTo - 1) / kNPadTo) * kNPadTo / kTileN;
@@ -990,6 +1009,7 @@ uint32_t twm_pick_splits(uint32_t k, uint32_t n, uint32_t m)
     // (f16 activations assumed; where the planner takes the sub-tile kernel, K is not split at all)
     if (m <= 4) return plan_gemv4_sub(n_tiles * kTileN / 64, k_chunks, m, false).sub ? 1 : plan_gemv4(n_tiles, k_chunks, 0, 0, 0).splits;
     if (m <= 16 && plan_gemv4_sub_rows(n_tiles * kTileN / 64, k_chunks).sub) return 1;
+    if (m > 16 || (m > 8 && n_tiles * kTileN / 64 > 128)) return plan_batch(n_tiles, k_chunks).splits;
     return plan_stream(n_tiles, k_chunks, m);
 }
 
@@ -1052,6 +1072,27 @@ static int gemm_common(twm_ctx *ctx, const twm_weight *w, const void *a_dev, int
                     TWM_DEVICE_ERROR, "gemv launch");
             return TWM_OK;
         }
+    }
+    const bool batch_auto = ctx->force_kernel == 0 && !ctx->force_nt && !ctx->force_waves &&
+                            (m > 16 || (m > 8 && n_ld / 64 > 128 && !splits));
+    if (ctx->force_kernel == 4 || batch_auto) {
+        // batched decode with the activations shared through LDS, in 32-row blocks: from 17 rows on (there it runs the
+        // reference's M > 1 arithmetic on f16-rounded weights, like the prefill kernel), and from 9 rows on wide
+        // matrices (3584 -> 37888: M = 16 19.8 against 22.8 us of the streaming kernel, M = 32 26.7 against
+        // 33.3; 18944 -> 3584 at M = 32 17.3 against 21.8; at M = 9 .. 16 on narrow matrices the two are within 3 %)
+        for (uint32_t m0 = 0; m0 < m; m0 += kMaxStreamM) {
+            uint32_t mb = m - m0 < (uint32_t)kMaxStreamM ? m - m0 : (uint32_t)kMaxStreamM;
+            OutSpec o = gated;
+            for (uint32_t s = 0; s < o.count; s++) o.seg[s].ptr += (size_t)m0 * o.seg[s].width;
+            if (o.swiglu) o.swiglu += (size_t)m0 * (w->n / 2);
+            const char *a_blk = (const char *)a_dev + (size_t)m0 * a_row_bytes;
+            BatchPlan bp = {splits ? splits : 1, ctx->force_waves == 8 ? 2u : ctx->force_waves == 16 ? 4u : 1u};
+            if (batch_auto) bp = plan_batch(w->n_tiles, w->k_chunks, splits);
+            HIP_TRY(launch_batch(ctx->stream, v, a_blk, a_dtype == TWM_F32, mb, o, bp.splits, ctx->force_nt == 2 ? 2 : 1,
+                                 bp.slices, m > 16, ctx->ws, ctx->ws_bytes),
+                    TWM_DEVICE_ERROR, "batched decode launch");
+        }
+        return TWM_OK;
     }
     if (ctx->force_kernel == 3 || (ctx->force_kernel == 0 && m > 4)) {
         // batched decode: 32-row blocks of the streaming kernel

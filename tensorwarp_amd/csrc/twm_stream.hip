@@ -253,6 +253,13 @@ __global__ __launch_bounds__(256) void k_split_f32_hi_lo(const float *__restrict
     lo[i] = (_Float16)(v - (float)h);
 }
 
+hipError_t launch_split_hi_lo(hipStream_t s, const float *a, _Float16 *hi, _Float16 *lo, size_t count)
+{
+    if (count == 0) return hipSuccess;
+    hipLaunchKernelGGL(k_split_f32_hi_lo, dim3((unsigned)((count + 255) / 256)), dim3(256), 0, s, a, hi, lo, count);
+    return hipGetLastError();
+}
+
 template <int MT, bool AF32, int WAVES>
 static hipError_t launch_stream_t(hipStream_t s, const WeightView &w, const void *a, uint32_t m, const OutSpec &out,
                                   uint32_t splits, float *partials, uint32_t lo_offset)
@@ -284,8 +291,8 @@ hipError_t launch_stream(hipStream_t s, const WeightView &w, const void *a, bool
         size_t term_bytes = (((size_t)m * w.k * 2) + 255) & ~(size_t)255;
         if (!scratch || scratch_bytes < 2 * term_bytes || term_bytes > 0x7FFFFFFFu) return hipErrorInvalidValue;
         _Float16 *hi = (_Float16 *)scratch, *lo = (_Float16 *)((char *)scratch + term_bytes);
-        size_t count = (size_t)m * w.k;
-        hipLaunchKernelGGL(k_split_f32_hi_lo, dim3((unsigned)((count + 255) / 256)), dim3(256), 0, s, (const float *)a, hi, lo, count);
+        hipError_t e = launch_split_hi_lo(s, (const float *)a, hi, lo, (size_t)m * w.k);
+        if (e != hipSuccess) return e;
         a = hi;
         lo_offset = (uint32_t)term_bytes;
         partials = (float *)((char *)scratch + 2 * term_bytes);
