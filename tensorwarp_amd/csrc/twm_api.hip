@@ -985,21 +985,44 @@ static uint32_t stream_waves(uint32_t n_tiles, uint32_t m, int force_waves)
     return (m > 16 && n_tiles / 4 >= 256) ? 4 : 8;
 }
 
-// Batched-decode kernel with LDS-shared activations: K is cut over workgroups as for the streaming kernel's 32-row
-// variant (about one workgroup per CU, seven chunks or more each); with fewer than 512 workgroups of eight chunks
-// or more, each workgroup runs two k-slices (eight waves) that add their sums through LDS
-// (18944 -> 3584 at M = 32: 4 splits x 2 slices 17.3 us, 4 x 1 about 22, 9 x 1 18.8; 3584 -> 37888, 592 quads: 1 x 1
-// 26.7, 1 x 2 28.1).
+// Batched-decode kernel with LDS-shared activations: split-K factor over workgroups and k-slices inside a workgroup
+// by a small cost model fitted to forced sweeps on eleven projection shapes of 1.5B .. 70B models (microseconds).  A
+// CU works through chunk steps (one 128-deep chunk of one 64-column quad) at up to 3.5 per us with two row blocks
+// (4.9 with one) when it holds enough waves; a single slice (four waves) alone advances at 1.9 (2.5) steps per us,
+// the latency of its barrier-and-load chain.  The busiest CU holds ceil(workgroups / 256) workgroups of `slices`
+// slices, each with chunks / (splits * slices) steps; a K-split over workgroups costs the second kernel (2.5) and
+// the partial sums written and read back at 4 TB/s.  More slices or splits have to win by 3 %.
+// (3584 -> 37888, 592 quads x 28 chunks, M = 32: 1 x 1 26.7 us, 1 x 2 28.1, 2 x 1 30.3; 18944 -> 3584, 56 x 148:
+// 4 splits x 2 slices 17.3, 9 x 1 18.8; 8192 -> 10240, 160 x 64: 3 x 1 19.4, 1 x 4 19.7, 1 x 2 21.6.)
 struct BatchPlan {
     uint32_t splits, slices;
 };
-static BatchPlan plan_batch(uint32_t n_tiles, uint32_t k_chunks, uint32_t force_splits = 0)
+static BatchPlan plan_batch(uint32_t n_tiles, uint32_t k_chunks, uint32_t m, uint32_t force_splits = 0)
 {
-    BatchPlan p = {force_splits ? force_splits : plan_stream(n_tiles, k_chunks, 32), 1};
-    if (p.splits > k_chunks) p.splits = k_chunks;
-    const uint32_t chunks_per_split = (k_chunks + p.splits - 1) / p.splits;
-    if ((n_tiles / 4) * p.splits < 512 && chunks_per_split >= 8) p.slices = 2;
-    return p;
+    const uint32_t quads = n_tiles / 4;
+    const double full_rate = m > 16 ? 3.5 : 4.9, lone_rate = m > 16 ? 1.9 : 2.5;
+    const double partial_us = (double)m * n_tiles * 16.0 * 4.0 * 2.0 / 4.0e6;  // one split's partial sums, written and read
+    BatchPlan best = {force_splits ? (force_splits < k_chunks ? force_splits : k_chunks) : 1u, 1u};
+    double best_us = 1e30;
+    for (uint32_t sp = 1; sp <= 16 && sp <= k_chunks; sp++) {
+        if (force_splits && sp != best.splits) continue;
+        const uint32_t cps = (k_chunks + sp - 1) / sp;
+        if (!force_splits && (k_chunks + cps - 1) / cps != sp) continue;  // same work as a smaller factor
+        const double wgs_on_cu = (double)(((uint64_t)quads * sp + 255) / 256);
+        for (uint32_t ks = 1; ks <= 4; ks *= 2) {
+            if (ks > 1 && cps < 2 * ks) continue;  // two chunks per slice at least
+            const double steps = (double)((cps + ks - 1) / ks);
+            const double busy = wgs_on_cu * ks * steps / full_rate, chain = steps / lone_rate;
+            double t = busy > chain ? busy : chain;
+            if (sp > 1) t += 2.5 + sp * partial_us;
+            if (t < best_us * 0.97) {
+                best_us = t;
+                best.splits = sp;
+                best.slices = ks;
+            }
+        }
+    }
+    return best;
 }
 
 uint32_t twm_pick_splits(uint32_t k, uint32_t n, uint32_t m)
@@ -1009,7 +1032,7 @@ uint32_t twm_pick_splits(uint32_t k, uint32_t n, uint32_t m)
     // (f16 activations assumed; where the planner takes the sub-tile kernel, K is not split at all)
     if (m <= 4) return plan_gemv4_sub(n_tiles * kTileN / 64, k_chunks, m, false).sub ? 1 : plan_gemv4(n_tiles, k_chunks, 0, 0, 0).splits;
     if (m <= 16 && plan_gemv4_sub_rows(n_tiles * kTileN / 64, k_chunks).sub) return 1;
-    if (m > 16 || (m > 8 && n_tiles * kTileN / 64 > 128)) return plan_batch(n_tiles, k_chunks).splits;
+    if (m > 16 || (m > 8 && n_tiles * kTileN / 64 > 128)) return plan_batch(n_tiles, k_chunks, m).splits;
     return plan_stream(n_tiles, k_chunks, m);
 }
 
@@ -1087,7 +1110,7 @@ static int gemm_common(twm_ctx *ctx, const twm_weight *w, const void *a_dev, int
             if (o.swiglu) o.swiglu += (size_t)m0 * (w->n / 2);
             const char *a_blk = (const char *)a_dev + (size_t)m0 * a_row_bytes;
             BatchPlan bp = {splits ? splits : 1, ctx->force_waves == 8 ? 2u : ctx->force_waves == 16 ? 4u : 1u};
-            if (batch_auto) bp = plan_batch(w->n_tiles, w->k_chunks, splits);
+            if (batch_auto) bp = plan_batch(w->n_tiles, w->k_chunks, m > 16 ? 32 : mb, splits);
             HIP_TRY(launch_batch(ctx->stream, v, a_blk, a_dtype == TWM_F32, mb, o, bp.splits, ctx->force_nt == 2 ? 2 : 1,
                                  bp.slices, m > 16, ctx->ws, ctx->ws_bytes),
                     TWM_DEVICE_ERROR, "batched decode launch");
