@@ -1096,13 +1096,18 @@ static int gemm_common(twm_ctx *ctx, const twm_weight *w, const void *a_dev, int
             return TWM_OK;
         }
     }
+    const bool rows_f32 = a_dtype == TWM_F32;
     const bool batch_auto = ctx->force_kernel == 0 && !ctx->force_nt && !ctx->force_waves &&
-                            (m > 16 || (m > 8 && n_ld / 64 > 128 && !splits));
+                            (m > 16 || (!splits && ((m > 8 && (n_ld / 64 > 128 || rows_f32)) ||
+                                                    (rows_f32 && m > 4 && w->k_chunks <= 64))));
     if (ctx->force_kernel == 4 || batch_auto) {
         // batched decode with the activations shared through LDS, in 32-row blocks: from 17 rows on (there it runs the
         // reference's M > 1 arithmetic on f16-rounded weights, like the prefill kernel), and from 9 rows on wide
         // matrices (3584 -> 37888: M = 16 19.8 against 22.8 us of the streaming kernel, M = 32 26.7 against
-        // 33.3; 18944 -> 3584 at M = 32 17.3 against 21.8; at M = 9 .. 16 on narrow matrices the two are within 3 %)
+        // 33.3; 18944 -> 3584 at M = 32 17.3 against 21.8; at M = 9 .. 16 on narrow matrices the two are within 3 %
+        // with f16 rows).  f32 rows, which the streaming kernel holds twice in registers: from 9 rows on everywhere
+        // (3584 -> 4608 at M = 16 10.9 against 15.1 us, 18944 -> 3584 20.6 against 23.3), from 5 rows on up to 64
+        // chunks deep (3584 -> 4608 at M = 8 10.5 against 11.4; 13824 -> 5120 would lose 18.6 against 18.5)
         for (uint32_t m0 = 0; m0 < m; m0 += kMaxStreamM) {
             uint32_t mb = m - m0 < (uint32_t)kMaxStreamM ? m - m0 : (uint32_t)kMaxStreamM;
             OutSpec o = gated;
