@@ -148,7 +148,7 @@ def main():
     ap.add_argument("--no-moe", action="store_true", help="skip the expert-bank (MoE decode) timing")
     ap.add_argument("--no-vendor-gemm", action="store_true",
                     help="skip timing rocBLAS' dense FP16 GEMM beside the prefill kernel")
-    ap.add_argument("--extra", action="store_true", help="also time batched decode (M=4..32) on the gate_up shape")
+    ap.add_argument("--no-batched", action="store_true", help="skip the batched-decode layer (M = 4 .. 32)")
     ap.add_argument("--sweep-splits", action="store_true",
                     help="also time every projection at M=1,4,8,16,32 with forced split-K factors next to the library's "
                          "own choice (batched decode configuration)")
@@ -284,21 +284,25 @@ def main():
                 "traffic": GATE_UP_TRAFFIC_BYTES}
 
     extra = {}
-    if args.extra:
-        k, n = 3584, 37888
+    if not args.no_batched:
+        log("batched decode")
+        # the same layer at M = 4 .. 32 f16 rows: one graph of the four projections over the rotating layers
         for m in (4, 8, 16, 32):
-            a_m = T.GpuTensor.from_host(dev, rng.standard_normal((m, k), dtype=np.float32).astype(np.float16).view(np.uint16), "f16")
-            c_m = T.GpuTensor.zeros(dev, (m, n), "f32")
+            bufs = {name: (T.GpuTensor.from_host(dev, rng.standard_normal((m, k), dtype=np.float32).astype(np.float16).view(np.uint16), "f16"),
+                           T.GpuTensor.zeros(dev, (m, n), "f32")) for name, k, n in LAYER_7B}
 
-            def one(i, a_m=a_m, c_m=c_m, m=m):
-                T.gemm(dev, layers[i % args.layers]["gate_up"][0], a_m, m, c_m)
-            for i in range(10):
-                one(i)
+            def run_rows(m=m, bufs=bufs):
+                for li in range(L):
+                    for name, k, n in LAYER_7B:
+                        T.gemm(dev, layers[li][name][0], bufs[name][0], m, bufs[name][1])
+            run_rows()
             dev.synchronize()
-            ms = time_launches(dev, one, 100)
-            b = algo_bytes(k, n, m)
-            extra["gate_up_M%d" % m] = {"us": round(ms * 1e3, 2), "GBps": round(b / (ms * 1e-3) / 1e9, 1),
-                                        "frac_hbm": round(b / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
+            g_rows = T.GraphCapture.record_with_device(dev, run_rows)
+            ms = time_launches(dev, lambda i: g_rows.replay(), max(4, steps // L // 4)) / L
+            graphs_done.append(g_rows)
+            lb = sum(algo_bytes(k, n, m) for _, k, n in LAYER_7B)
+            extra["layer_M%d" % m] = {"us": round(ms * 1e3, 2), "GBps": round(lb / (ms * 1e-3) / 1e9, 1),
+                                      "frac_hbm": round(lb / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
 
     log("small configurations")
     # the small configurations: launch- and latency-bound, reported per projection and as one graph per layer
