@@ -599,7 +599,7 @@ def main():
                 packed = rng.integers(0, 256, size=(k // 32) * n * 16, dtype=np.uint8)
                 scales = (np.abs(rng.standard_normal((k // 32) * n, dtype=np.float32)) * np.float32(0.02)).astype(np.float16)
                 sets.append(T.MarlinWeight.upload(dev, packed, scales.view(np.uint16), k, n))
-            for m, dt in ((1, "f16"), (1, "f32"), (4, "f16"), (8, "f16"), (16, "f16")):
+            for m, dt in ((1, "f16"), (1, "f32"), (4, "f16"), (8, "f16"), (16, "f16"), (32, "f16")):
                 ah = rng.standard_normal((m, k), dtype=np.float32)
                 a_m = (T.GpuTensor.from_host(dev, ah.astype(np.float16).view(np.uint16), "f16") if dt == "f16"
                        else T.GpuTensor.from_host(dev, ah))
