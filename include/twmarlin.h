@@ -228,11 +228,13 @@ int twm_weight_dequant_f16(twm_ctx *ctx, const twm_weight *w, uint16_t *out_kn_d
 /* C[M,N] (f32, row-major) = A[M,K] (f16 or f32, row-major) * dequant(W), f32 accumulation.
  * M = 1 is gemm_tw_marlin_m1 (quantize.rs:1301); M > 1 has the semantics of gemm_q4_0
  * (quantize.rs:1825-1858).  splits = 0 lets the library choose (twm_pick_splits).
- * M <= 32: decode kernels (M <= 4 one lane per column, M = 5..32 streaming tiles), weights exact,
- *          each group's f32 sum scaled by f32(scale).  f32 activations enter as two f16 terms,
- *          f16(a) + f16(a - f16(a)), about 22 bits (|a| inside the f16 range).
- * M  > 32: prefill GEMM; weights are the reference's FP16 Q4 unpack, f16(scale * (q - 8)), as in
- * its dequant-then-matmul prefill route; f32 activations are rounded to f16 first.  Uses the
+ * M <= 16: decode kernels (M <= 4 one lane per column, above that 16-column tiles), weights exact,
+ *          each group's f32 sum scaled by f32(scale).
+ * M = 17 .. 32: batched-decode kernel on the reference's FP16 Q4 unpack, f16(scale * (q - 8)), as in
+ *          its dequant-then-matmul route for M > 1.
+ * Up to M = 32 f32 activations enter as two f16 terms, f16(a) + f16(a - f16(a)), about 22 bits (|a|
+ * inside the f16 range).
+ * M  > 32: prefill GEMM on the same FP16 unpack; f32 activations are rounded to f16 first.  Uses the
  * context's scratch: one context must not run two calls at the same time. */
 int twm_gemm(twm_ctx *ctx, const twm_weight *w, const void *a_dev, int a_dtype, uint32_t m,
              float *c_dev, uint32_t splits);
