@@ -985,40 +985,52 @@ static uint32_t stream_waves(uint32_t n_tiles, uint32_t m, int force_waves)
     return (m > 16 && n_tiles / 4 >= 256) ? 4 : 8;
 }
 
-// Batched-decode kernel with LDS-shared activations: split-K factor over workgroups and k-slices inside a workgroup
-// by a small cost model fitted to forced sweeps on eleven projection shapes of 1.5B .. 70B models (microseconds).  A
-// CU works through chunk steps (one 128-deep chunk of one 64-column quad) at up to 3.5 per us with two row blocks
-// (4.9 with one) when it holds enough waves; a single slice (four waves) alone advances at 1.9 (2.5) steps per us,
-// the latency of its barrier-and-load chain.  The busiest CU holds ceil(workgroups / 256) workgroups of `slices`
-// slices, each with chunks / (splits * slices) steps; a K-split over workgroups costs the second kernel (2.5) and
-// the partial sums written and read back at 4 TB/s.  More slices or splits have to win by 3 %.
-// (3584 -> 37888, 592 quads x 28 chunks, M = 32: 1 x 1 26.7 us, 1 x 2 28.1, 2 x 1 30.3; 18944 -> 3584, 56 x 148:
-// 4 splits x 2 slices 17.3, 9 x 1 18.8; 8192 -> 10240, 160 x 64: 3 x 1 19.4, 1 x 4 19.7, 1 x 2 21.6.)
+// Batched-decode kernel with LDS-shared activations: split-K factor over workgroups, k-slices inside a workgroup and
+// tiles per wave by a small cost model fitted to forced sweeps on fifteen projection shapes of 1.5B .. 70B models
+// (microseconds).  A CU works through quad steps (one 128-deep chunk of one 64-column quad) at up to 3.5 per us
+// with two row blocks (4.9 with one) when it holds enough waves; with two tiles per wave -- 128 columns per
+// workgroup, so half the activation loads per weight, which compete with the weight stream for the CU's memory
+// requests in flight -- at up to 3.95 (5.5).  A single slice (four waves) alone advances at 1.9 (2.5) steps per us,
+// 1.7 (2.2) with two tiles per wave: the latency of its barrier-and-load chain.  The busiest CU holds
+// ceil(workgroups / 256) workgroups of `slices` slices, each with chunks / (splits * slices) steps; a K-split over
+// workgroups costs the second kernel (2.5) and, per split, 0.2 plus the partial sums written and read back at
+// 2.7 TB/s (18944 -> 3584 at M = 32 read 19.0 us on nine splits against 17.2 on four).  More slices,
+// splits or tiles per wave have to win by 3 %; a slice keeps two chunks or more (eight with two tiles per wave).
+// (3584 -> 37888, 592 quads x 28 chunks, M = 32: 1 split x 1 slice x 1 tile 26.7 us, 1 x 2 x 1 28.1, 2 x 1 x 1 30.3,
+// 1 x 1 x 2 27.8 -- 296 workgroups put four quads on some CUs instead of three; 8192 -> 57344, 896 x 64: 1 x 1 x 1
+// 70.7, 1 x 1 x 2 62.1; 18944 -> 3584, 56 x 148: 4 x 2 x 1 17.3, 9 x 1 x 1 18.8; 8192 -> 10240, 160 x 64: 3 x 2 x 2
+// 18.2, 3 x 1 x 1 19.0, 1 x 4 x 1 19.7.)
 struct BatchPlan {
-    uint32_t splits, slices;
+    uint32_t splits, slices, tiles_per_wave;
 };
 static BatchPlan plan_batch(uint32_t n_tiles, uint32_t k_chunks, uint32_t m, uint32_t force_splits = 0)
 {
     const uint32_t quads = n_tiles / 4;
-    const double full_rate = m > 16 ? 3.5 : 4.9, lone_rate = m > 16 ? 1.9 : 2.5;
+    const bool two_blocks = m > 16;
     const double partial_us = (double)m * n_tiles * 16.0 * 4.0 * 2.0 / 4.0e6;  // one split's partial sums, written and read
-    BatchPlan best = {force_splits ? (force_splits < k_chunks ? force_splits : k_chunks) : 1u, 1u};
+    BatchPlan best = {force_splits ? (force_splits < k_chunks ? force_splits : k_chunks) : 1u, 1u, 1u};
     double best_us = 1e30;
-    for (uint32_t sp = 1; sp <= 16 && sp <= k_chunks; sp++) {
-        if (force_splits && sp != best.splits) continue;
-        const uint32_t cps = (k_chunks + sp - 1) / sp;
-        if (!force_splits && (k_chunks + cps - 1) / cps != sp) continue;  // same work as a smaller factor
-        const double wgs_on_cu = (double)(((uint64_t)quads * sp + 255) / 256);
-        for (uint32_t ks = 1; ks <= 4; ks *= 2) {
-            if (ks > 1 && cps < 2 * ks) continue;  // two chunks per slice at least
-            const double steps = (double)((cps + ks - 1) / ks);
-            const double busy = wgs_on_cu * ks * steps / full_rate, chain = steps / lone_rate;
-            double t = busy > chain ? busy : chain;
-            if (sp > 1) t += 2.5 + sp * partial_us;
-            if (t < best_us * 0.97) {
-                best_us = t;
-                best.splits = sp;
-                best.slices = ks;
+    for (uint32_t tpw = 1; tpw <= 2; tpw++) {
+        const double full_rate = two_blocks ? (tpw == 1 ? 3.5 : 3.95) : (tpw == 1 ? 4.9 : 5.5);
+        const double lone_rate = two_blocks ? (tpw == 1 ? 1.9 : 1.7) : (tpw == 1 ? 2.5 : 2.2);
+        const uint64_t groups = (quads + tpw - 1) / tpw;
+        for (uint32_t sp = 1; sp <= 16 && sp <= k_chunks; sp++) {
+            if (force_splits && sp != best.splits) continue;
+            const uint32_t cps = (k_chunks + sp - 1) / sp;
+            if (!force_splits && (k_chunks + cps - 1) / cps != sp) continue;  // same work as a smaller factor
+            const double wgs_on_cu = (double)((groups * sp + 255) / 256);
+            for (uint32_t ks = 1; ks <= (tpw == 1 ? 4u : 2u); ks *= 2) {
+                if (ks > 1 && cps < (tpw == 1 ? 2 : 8) * ks) continue;
+                const double steps = (double)((cps + ks - 1) / ks);
+                const double busy = wgs_on_cu * tpw * ks * steps / full_rate, chain = steps / lone_rate;
+                double t = busy > chain ? busy : chain;
+                if (sp > 1) t += 2.5 + sp * (0.2 + 1.5 * partial_us);
+                if (t < best_us * 0.97) {
+                    best_us = t;
+                    best.splits = sp;
+                    best.slices = ks;
+                    best.tiles_per_wave = tpw;
+                }
             }
         }
     }
@@ -1114,10 +1126,11 @@ static int gemm_common(twm_ctx *ctx, const twm_weight *w, const void *a_dev, int
             for (uint32_t s = 0; s < o.count; s++) o.seg[s].ptr += (size_t)m0 * o.seg[s].width;
             if (o.swiglu) o.swiglu += (size_t)m0 * (w->n / 2);
             const char *a_blk = (const char *)a_dev + (size_t)m0 * a_row_bytes;
-            BatchPlan bp = {splits ? splits : 1, ctx->force_waves == 8 ? 2u : ctx->force_waves == 16 ? 4u : 1u};
+            BatchPlan bp = {splits ? splits : 1, ctx->force_waves == 8 ? 2u : ctx->force_waves == 16 ? 4u : 1u,
+                            ctx->force_nt == 2 ? 2u : 1u};
             if (batch_auto) bp = plan_batch(w->n_tiles, w->k_chunks, m > 16 ? 32 : mb, splits);
-            HIP_TRY(launch_batch(ctx->stream, v, a_blk, a_dtype == TWM_F32, mb, o, bp.splits, ctx->force_nt == 2 ? 2 : 1,
-                                 bp.slices, m > 16, ctx->ws, ctx->ws_bytes),
+            HIP_TRY(launch_batch(ctx->stream, v, a_blk, a_dtype == TWM_F32, mb, o, bp.splits, bp.tiles_per_wave, bp.slices,
+                                 m > 16, ctx->ws, ctx->ws_bytes),
                     TWM_DEVICE_ERROR, "batched decode launch");
         }
         return TWM_OK;
