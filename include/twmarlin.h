@@ -91,8 +91,8 @@ int twm_ctx_info(twm_ctx *ctx, char *buf, size_t buf_len);
  *                   of that many columns (with "waves" waves, default 8), 0 = the planner's choice per shape
  *   "kernel"        decode kernel: 1 = 16x16x32 tile kernel (16-row blocks), 2 = one-lane-per-column kernel
  *                   (M <= 4 only), 3 = batched-decode streaming kernel (32-row blocks), 4 = batched-decode kernel
- *                   with the activations shared through LDS (32-row blocks; "nt" 1 / 2 = tiles per wave,
- *                   "waves" 8 / 16 = two / four k-slices per workgroup)
+ *                   with the activations shared through LDS (32-row blocks; "nt" 1 / 2 = tiles per wave, 4 / 3 =
+ *                   two / three column quads per workgroup, "waves" 8 / 16 = two / four k-slices per workgroup)
  *   "dequant_src"   which repacked copy twm_weight_dequant_f16 unpacks: 0 = 16-column tiles, 1 = column lanes
  *   "prefill_min_m" smallest M that runs the prefill GEMM (default 33; below it the decode kernels run)
  *   "prefill_bm"    rows of A per prefill workgroup (64 or 128)

@@ -191,8 +191,7 @@ int twm_ctx_set_option(twm_ctx *ctx, const char *key, int value)
 {
     if (!ctx || !key) return fail(TWM_INVALID_HANDLE, "twm_ctx_set_option: null argument");
     if (strcmp(key, "nt") == 0) {
-        if (value != 0 && value != 1 && value != 2 && value != 4)
-            return fail(TWM_SHAPE_ERROR, "twm_ctx_set_option: nt must be 0, 1, 2 or 4");
+        if (value < 0 || value > 4) return fail(TWM_SHAPE_ERROR, "twm_ctx_set_option: nt must be 0 .. 4");
         ctx->force_nt = value;
         return TWM_OK;
     }
@@ -865,7 +864,7 @@ static DecodePlan plan_decode(uint32_t n_tiles, uint32_t k_chunks, uint32_t m, i
     p.lane_col = 0;
     p.nt = 1;
     if (n_tiles >= 2048) p.nt = 2;
-    if (force_nt) p.nt = (uint32_t)force_nt;
+    if (force_nt && force_nt != 3) p.nt = (uint32_t)force_nt;  // (3 is a choice of the batched-decode kernel only)
     uint32_t tg = n_tiles / p.nt;
     if (tg == 0) tg = 1;
     // waves per workgroup: enough that tg * waves reaches ~4096, bounded by the chunks available
@@ -986,50 +985,61 @@ static uint32_t stream_waves(uint32_t n_tiles, uint32_t m, int force_waves)
 }
 
 // Batched-decode kernel with LDS-shared activations: split-K factor over workgroups, k-slices inside a workgroup and
-// tiles per wave by a small cost model fitted to forced sweeps on fifteen projection shapes of 1.5B .. 70B models
-// (microseconds).  A CU works through quad steps (one 128-deep chunk of one 64-column quad) at up to 3.5 per us
-// with two row blocks (4.9 with one) when it holds enough waves; with two tiles per wave -- 128 columns per
-// workgroup, so half the activation loads per weight, which compete with the weight stream for the CU's memory
-// requests in flight -- at up to 3.95 (5.5).  A single slice (four waves) alone advances at 1.9 (2.5) steps per us,
-// 1.7 (2.2) with two tiles per wave: the latency of its barrier-and-load chain.  The busiest CU holds
-// ceil(workgroups / 256) workgroups of `slices` slices, each with chunks / (splits * slices) steps; a K-split over
-// workgroups costs the second kernel (2.5) and, per split, 0.2 plus the partial sums written and read back at
-// 2.7 TB/s (18944 -> 3584 at M = 32 read 19.0 us on nine splits against 17.2 on four).  More slices,
-// splits or tiles per wave have to win by 3 %; a slice keeps two chunks or more (eight with two tiles per wave).
-// (3584 -> 37888, 592 quads x 28 chunks, M = 32: 1 split x 1 slice x 1 tile 26.7 us, 1 x 2 x 1 28.1, 2 x 1 x 1 30.3,
-// 1 x 1 x 2 27.8 -- 296 workgroups put four quads on some CUs instead of three; 8192 -> 57344, 896 x 64: 1 x 1 x 1
-// 70.7, 1 x 1 x 2 62.1; 18944 -> 3584, 56 x 148: 4 x 2 x 1 17.3, 9 x 1 x 1 18.8; 8192 -> 10240, 160 x 64: 3 x 2 x 2
-// 18.2, 3 x 1 x 1 19.0, 1 x 4 x 1 19.7.)
+// the columns that share one activation tile (one, two or three 64-column quads per workgroup with one tile per
+// wave, or two quads with two tiles per wave) by a small cost model fitted to forced sweeps on fifteen projection
+// shapes of 1.5B .. 70B models (microseconds).  A CU works through quad steps (one 128-deep chunk of one 64-column
+// quad) at up to 3.5 per us with two row blocks (4.9 with one) when it holds enough waves.  The activation tile
+// comes from L2 once per workgroup and chunk, and those requests compete with the weight stream for the CU's memory
+// requests in flight: with two or three quads per workgroup the rate is 4.3 (5.2), with two tiles per wave 3.95
+// (5.1).  A single slice alone advances at 1.9 (2.5) steps per us, 1.8 (2.4) with eight or twelve waves, 1.7 (2.2)
+// with two tiles per wave: the latency of its barrier-and-load chain.  The busiest CU holds ceil(workgroups / 256)
+// workgroups of `slices` slices, each with chunks / (splits * slices) steps (the time is the larger of the two
+// bounds plus 15 % of the smaller: 8192 -> 10240 at M = 16 on 160 workgroups of two slices, both bounds 13, read 17.5 us
+// with the launch, with four slices 15.4); a K-split over workgroups costs the
+// second kernel (2.5) and, per split, 0.2 plus the partial sums written and read back at 2.7 TB/s
+// (18944 -> 3584 at M = 32 read 19.0 us on nine splits against 17.2 on four).  A more elaborate plan has to win by
+// 3 %; a slice keeps two chunks or more (eight with two tiles per wave).
+// (3584 -> 37888, 592 quads x 28 chunks, M = 32: one quad per workgroup 26.1 us, two 26.0 -- 296 workgroups put four
+// quads on some CUs instead of three --, three 22.4, two k-slices 27.3, two K-splits 30.3; 4096 -> 22016, 344 x 32:
+// one quad 20.5, two quads x two slices 16.8; 8192 -> 57344, 896 x 64: one quad 72.4, two 63.2, two tiles per wave
+// 61.9; 18944 -> 3584, 56 x 148: 4 splits x 2 slices 17.1, 4 x 1 20.7; 8192 -> 10240, 160 x 64: 3 splits, two quads x
+// two slices 17.0, one quad 18.5.)
 struct BatchPlan {
-    uint32_t splits, slices, tiles_per_wave;
+    uint32_t splits, slices, tiles_per_wave, quads_per_group;
 };
-static BatchPlan plan_batch(uint32_t n_tiles, uint32_t k_chunks, uint32_t m, uint32_t force_splits = 0)
+static BatchPlan plan_batch(uint32_t n_tiles, uint32_t k_chunks, uint32_t m, bool rows_f32, uint32_t force_splits = 0)
 {
     const uint32_t quads = n_tiles / 4;
     const bool two_blocks = m > 16;
     const double partial_us = (double)m * n_tiles * 16.0 * 4.0 * 2.0 / 4.0e6;  // one split's partial sums, written and read
-    BatchPlan best = {force_splits ? (force_splits < k_chunks ? force_splits : k_chunks) : 1u, 1u, 1u};
+    BatchPlan best = {force_splits ? (force_splits < k_chunks ? force_splits : k_chunks) : 1u, 1u, 1u, 1u};
     double best_us = 1e30;
-    for (uint32_t tpw = 1; tpw <= 2; tpw++) {
-        const double full_rate = two_blocks ? (tpw == 1 ? 3.5 : 3.95) : (tpw == 1 ? 4.9 : 5.5);
-        const double lone_rate = two_blocks ? (tpw == 1 ? 1.9 : 1.7) : (tpw == 1 ? 2.5 : 2.2);
-        const uint64_t groups = (quads + tpw - 1) / tpw;
+    static const struct { uint32_t tpw, qpg, max_slices; double full2, full1, lone2, lone1; } kForms[] = {
+        {1, 1, 4, 3.5, 4.9, 1.9, 2.5}, {1, 2, 2, 4.3, 5.2, 1.8, 2.4}, {1, 3, 1, 4.3, 5.2, 1.8, 2.4}, {2, 1, 2, 3.95, 5.1, 1.7, 2.2}};
+    for (const auto &f : kForms) {
+        const double full_rate = two_blocks ? f.full2 : f.full1, lone_rate = two_blocks ? f.lone2 : f.lone1;
+        const uint32_t share = f.tpw * f.qpg;  // quads per workgroup
+        const uint64_t groups = (quads + share - 1) / share;
+        // (the 32-row two-term variant has LDS for one slice of eight waves, two of four)
+        const uint32_t max_slices = two_blocks && rows_f32 ? (f.qpg == 2 ? 1u : f.max_slices < 2 ? f.max_slices : 2u) : f.max_slices;
         for (uint32_t sp = 1; sp <= 16 && sp <= k_chunks; sp++) {
             if (force_splits && sp != best.splits) continue;
             const uint32_t cps = (k_chunks + sp - 1) / sp;
             if (!force_splits && (k_chunks + cps - 1) / cps != sp) continue;  // same work as a smaller factor
             const double wgs_on_cu = (double)((groups * sp + 255) / 256);
-            for (uint32_t ks = 1; ks <= (tpw == 1 ? 4u : 2u); ks *= 2) {
-                if (ks > 1 && cps < (tpw == 1 ? 2 : 8) * ks) continue;
+            for (uint32_t ks = 1; ks <= max_slices; ks *= 2) {
+                if (ks > 1 && cps < (f.tpw == 1 ? 2 : 8) * ks) continue;
                 const double steps = (double)((cps + ks - 1) / ks);
-                const double busy = wgs_on_cu * tpw * ks * steps / full_rate, chain = steps / lone_rate;
-                double t = busy > chain ? busy : chain;
+                const double busy = wgs_on_cu * share * ks * steps / full_rate, chain = steps / lone_rate;
+                double t = busy > chain ? busy + 0.15 * chain : chain + 0.15 * busy;  // (neither hides the other entirely)
+                if (ks > 1) t += 0.3 * ks;  // the slices' sums through LDS, the wider barriers
                 if (sp > 1) t += 2.5 + sp * (0.2 + 1.5 * partial_us);
                 if (t < best_us * 0.97) {
                     best_us = t;
                     best.splits = sp;
                     best.slices = ks;
-                    best.tiles_per_wave = tpw;
+                    best.tiles_per_wave = f.tpw;
+                    best.quads_per_group = f.qpg;
                 }
             }
         }
@@ -1044,7 +1054,7 @@ uint32_t twm_pick_splits(uint32_t k, uint32_t n, uint32_t m)
     // (f16 activations assumed; where the planner takes the sub-tile kernel, K is not split at all)
     if (m <= 4) return plan_gemv4_sub(n_tiles * kTileN / 64, k_chunks, m, false).sub ? 1 : plan_gemv4(n_tiles, k_chunks, 0, 0, 0).splits;
     if (m <= 16 && plan_gemv4_sub_rows(n_tiles * kTileN / 64, k_chunks).sub) return 1;
-    if (m > 16 || (m > 8 && n_tiles * kTileN / 64 > 128)) return plan_batch(n_tiles, k_chunks, m).splits;
+    if (m > 16 || (m > 8 && n_tiles * kTileN / 64 > 128)) return plan_batch(n_tiles, k_chunks, m, false).splits;
     return plan_stream(n_tiles, k_chunks, m);
 }
 
@@ -1126,11 +1136,12 @@ static int gemm_common(twm_ctx *ctx, const twm_weight *w, const void *a_dev, int
             for (uint32_t s = 0; s < o.count; s++) o.seg[s].ptr += (size_t)m0 * o.seg[s].width;
             if (o.swiglu) o.swiglu += (size_t)m0 * (w->n / 2);
             const char *a_blk = (const char *)a_dev + (size_t)m0 * a_row_bytes;
+            // forced: "nt" 2 = two tiles per wave, 4 = two quads per workgroup, 3 = three; "waves" 8 / 16 = 2 / 4 k-slices
             BatchPlan bp = {splits ? splits : 1, ctx->force_waves == 8 ? 2u : ctx->force_waves == 16 ? 4u : 1u,
-                            ctx->force_nt == 2 ? 2u : 1u};
-            if (batch_auto) bp = plan_batch(w->n_tiles, w->k_chunks, m > 16 ? 32 : mb, splits);
+                            ctx->force_nt == 2 ? 2u : 1u, ctx->force_nt == 4 ? 2u : ctx->force_nt == 3 ? 3u : 1u};
+            if (batch_auto) bp = plan_batch(w->n_tiles, w->k_chunks, m > 16 ? 32 : mb, rows_f32, splits);
             HIP_TRY(launch_batch(ctx->stream, v, a_blk, a_dtype == TWM_F32, mb, o, bp.splits, bp.tiles_per_wave, bp.slices,
-                                 m > 16, ctx->ws, ctx->ws_bytes),
+                                 bp.quads_per_group, m > 16, ctx->ws, ctx->ws_bytes),
                     TWM_DEVICE_ERROR, "batched decode launch");
         }
         return TWM_OK;

@@ -73,8 +73,13 @@ constexpr int kBtRow = 128;  // halves per LDS row (256 bytes)
 // of the workgroup's k-range with its own LDS buffers, and the slices' sums are added through LDS at the end -- more
 // waves per CU where the column quads alone are too few workgroups, without the partial-sum traffic of a K-split
 // over workgroups.
-template <int MT, int TERMS, int TPW, int KS>
-__global__ __launch_bounds__(256 * KS) void k_batch(const uint4v *__restrict__ qw, const uint2v *__restrict__ sc,
+// WPS: waves per slice (4, 8 or 12; TPW = 1 above 4): WPS / 4 quads per workgroup share one activation tile, so the
+// tile is fetched from L2 once per 64 WPS / 4 columns -- its requests compete with the weight stream for the CU's
+// memory requests in flight.  The first 4 MT waves of a slice stage the tile (four rows each, or MT times four with
+// WPS = 4); the others issue the same load on one 16-byte address and write a spare LDS row, which keeps every
+// wave's count of loads in flight the same.
+template <int MT, int TERMS, int TPW, int KS, int WPS>
+__global__ __launch_bounds__(64 * WPS * KS) void k_batch(const uint4v *__restrict__ qw, const uint2v *__restrict__ sc,
                                                 const void *__restrict__ a_any, OutSpec out, float *__restrict__ partials,
                                                 uint32_t m_rows, uint32_t k, uint32_t n, uint32_t n_tiles,
                                                 uint32_t k_chunks, uint32_t chunks_per_split, uint32_t lo_offset)
@@ -83,11 +88,15 @@ __global__ __launch_bounds__(256 * KS) void k_batch(const uint4v *__restrict__ q
     constexpr int S = 4;                     // register slots: chunk kc lives in slot kc % S, three chunks are in flight
     constexpr int kTile = 16 * MT * kBtRow;  // halves of one term's tile
     constexpr int kBuf = TERMS * kTile;      // halves of one LDS buffer
-    __shared__ __attribute__((aligned(16))) _Float16 lds_all[KS * 2 * kBuf];
+    static_assert(TPW == 1 || WPS == 4, "two tiles per wave: four waves per slice");
+    static_assert(64 * WPS * KS <= 1024, "workgroup size");
+    constexpr int NVW = (4 * MT + WPS - 1) / WPS;  // A loads per wave and chunk (four rows of the tile each)
+    constexpr int kSpare = NVW * WPS > 4 * MT ? 512 : 0;  // halves: where the waves without a part of the tile write
+    __shared__ __attribute__((aligned(16))) _Float16 lds_all[KS * (2 * kBuf + kSpare)];
 
     const uint32_t wave_all = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const uint32_t wave = wave_all & 3u, slice = wave_all >> 2;  // wave: index inside the slice
-    _Float16 *a_lds = lds_all + slice * (2 * kBuf);
+    const uint32_t wave = wave_all % WPS, slice = wave_all / WPS;  // wave: index inside the slice
+    _Float16 *a_lds = lds_all + slice * (2 * kBuf + kSpare);
     const uint32_t lane = threadIdx.x & 63u;
     const uint32_t c = lane & 15u, kb = lane >> 4;
     const uint32_t kc0 = blockIdx.y * chunks_per_split;
@@ -103,7 +112,7 @@ __global__ __launch_bounds__(256 * KS) void k_batch(const uint4v *__restrict__ q
     uint32_t tile_of[TPW], nt[TPW];
 #pragma unroll
     for (int i = 0; i < TPW; i++) {
-        tile_of[i] = TPW == 1 ? blockIdx.x * 4u + wave : (blockIdx.x * 2u + (wave >> 1)) * 4u + (wave & 1u) + 2u * i;
+        tile_of[i] = TPW == 1 ? blockIdx.x * (uint32_t)WPS + wave : (blockIdx.x * 2u + (wave >> 1)) * 4u + (wave & 1u) + 2u * i;
         nt[i] = tile_of[i] < n_tiles ? tile_of[i] : n_tiles - 1;
     }
 
@@ -116,30 +125,36 @@ __global__ __launch_bounds__(256 * KS) void k_batch(const uint4v *__restrict__ q
 #pragma unroll
         for (int i = 0; i < TPW; i++) acc[mt][i] = float4v{0.f, 0.f, 0.f, 0.f};
 
-    // ---- A tile: load j of wave w covers rows 16 j + 4 w .. + 3 of the tile; lane L takes row 4 w + L / 16 and the
-    // row's vector (L % 16) ^ (row % 16) (8 halves) and writes it to slot L % 16 of that row, so that slot s of row r
-    // holds vector s ^ (r % 16).  Rows past m_rows replay the last row (never stored); vectors past K replay the
-    // chunk's first vector of the row (the padded weights there are zero).
-    const uint32_t a_vec = (lane & 15u) ^ ((4u * wave + (lane >> 4)) & 15u);
-    uint32_t a_off[MT];
+    // ---- A tile: the tile's 4 MT row quads (four rows each) go to the slice's waves in turn, load j of wave w takes
+    // quad w + j WPS; lane L takes row L / 16 of the quad and the row's vector (L % 16) ^ (row % 16) (8 halves) and
+    // writes it to slot L % 16 of that row, so that slot s of row r holds vector s ^ (r % 16).  Rows past m_rows replay
+    // the last row (never stored); vectors past K replay the chunk's first vector of the row (the padded weights
+    // there are zero).  A load past the last quad reads one 16-byte address with all lanes and lands in the spare row.
+    uint32_t a_vec[NVW], a_off[NVW], a_dst[NVW];
 #pragma unroll
-    for (int j = 0; j < MT; j++) {
-        uint32_t row = 16u * j + 4u * wave + (lane >> 4);
+    for (int j = 0; j < NVW; j++) {
+        const uint32_t quad = wave + (uint32_t)j * WPS;
+        const bool real = quad < 4u * MT;
+        uint32_t row = real ? 4u * quad + (lane >> 4) : 0u;
+        a_vec[j] = real ? (lane & 15u) ^ (row & 15u) : 0u;
         row = row < m_rows ? row : m_rows - 1;
-        a_off[j] = (row * k + a_vec * 8u) * 2u;
+        a_off[j] = (row * k + a_vec[j] * 8u) * 2u;
+        a_dst[j] = real ? 4u * quad * kBtRow + lane * 8u : 2u * kBuf + (lane & 63u) * 8u;  // halves, inside a buffer / the spare row
     }
-    uint4v ar[S][TERMS][MT];
+    uint4v ar[S][TERMS][NVW];
     uint4v wq[S][TPW];
     uint2v ws[S][TPW];
     const uint32_t q_off = lane * 16u, s_off = c * 8u;
     auto load_chunk = [&](int slot, uint32_t kc) {  // kc relative to kc0; the same loads in every call
         const uint32_t kg = kc0 + kc;
-        const uint32_t back = kg * 128u + a_vec * 8u < k ? 0u : a_vec * 16u;
 #pragma unroll
         for (int t = 0; t < TERMS; t++) {
             const TWM_GLOBAL char *src = bt_scalar_base(a_any, (size_t)t * lo_offset + (size_t)kg * 256u);
 #pragma unroll
-            for (int j = 0; j < MT; j++) ar[slot][t][j] = *(const TWM_GLOBAL uint4v *)(src + (a_off[j] - back));
+            for (int j = 0; j < NVW; j++) {
+                const uint32_t back = kg * 128u + a_vec[j] * 8u < k ? 0u : a_vec[j] * 16u;
+                ar[slot][t][j] = *(const TWM_GLOBAL uint4v *)(src + (a_off[j] - back));
+            }
         }
 #pragma unroll
         for (int i = 0; i < TPW; i++) {
@@ -149,12 +164,15 @@ __global__ __launch_bounds__(256 * KS) void k_batch(const uint4v *__restrict__ q
             ws[slot][i] = __builtin_nontemporal_load((const TWM_GLOBAL uint2v *)(bt_scalar_base(sc, tile * 128u) + s_off));
         }
     };
-    auto stage_a = [&](int slot, int buf) {  // this wave's quarter of a tile: registers -> LDS
+    auto stage_a = [&](int slot, int buf) {  // this wave's part of a tile: registers -> LDS
 #pragma unroll
         for (int t = 0; t < TERMS; t++)
 #pragma unroll
-            for (int j = 0; j < MT; j++)
-                *(uint4v *)(a_lds + buf * kBuf + t * kTile + (16 * j + 4 * wave) * kBtRow + lane * 8u) = ar[slot][t][j];
+            for (int j = 0; j < NVW; j++) {
+                // (the spare row lies behind both buffers: its offset takes neither the buffer nor the term)
+                const uint32_t at = a_dst[j] < 2u * kBuf ? buf * kBuf + t * kTile + a_dst[j] : a_dst[j];
+                *(uint4v *)(a_lds + at) = ar[slot][t][j];
+            }
     };
 
     uint32_t rd_off[4];  // row c of a row block, vector 4 g + kb of the chunk -> slot (4 g + kb) ^ c
@@ -236,7 +254,7 @@ __global__ __launch_bounds__(256 * KS) void k_batch(const uint4v *__restrict__ q
         // the slices' sums, added in slice order through LDS (the staging buffers are idle: the last step ended with
         // a barrier); slice 0 stores
         constexpr int kRegs = MT * TPW * 4;
-        float *red = (float *)lds_all;  // [KS - 1][4 waves][kRegs][64 lanes]
+        float *red = (float *)lds_all;  // [KS - 1][WPS waves][kRegs][64 lanes]
         if (slice > 0) {
 #pragma unroll
             for (int mt = 0; mt < MT; mt++)
@@ -244,7 +262,7 @@ __global__ __launch_bounds__(256 * KS) void k_batch(const uint4v *__restrict__ q
                 for (int t = 0; t < TPW; t++)
 #pragma unroll
                     for (int r = 0; r < 4; r++)
-                        red[(((slice - 1u) * 4u + wave) * kRegs + (mt * TPW + t) * 4 + r) * 64u + lane] = acc[mt][t][r];
+                        red[(((slice - 1u) * WPS + wave) * kRegs + (mt * TPW + t) * 4 + r) * 64u + lane] = acc[mt][t][r];
         }
         __syncthreads();
         if (slice > 0) return;
@@ -256,7 +274,7 @@ __global__ __launch_bounds__(256 * KS) void k_batch(const uint4v *__restrict__ q
                 for (int t = 0; t < TPW; t++)
 #pragma unroll
                     for (int r = 0; r < 4; r++)
-                        acc[mt][t][r] += red[(((sl - 1) * 4 + wave) * kRegs + (mt * TPW + t) * 4 + r) * 64u + lane];
+                        acc[mt][t][r] += red[(((sl - 1) * WPS + wave) * kRegs + (mt * TPW + t) * 4 + r) * 64u + lane];
     }
 
     // ---- store: lane (c, kb) holds rows 16 mt + 4 kb + r of column 16 tile + c
@@ -316,15 +334,16 @@ __global__ __launch_bounds__(256 * KS) void k_batch(const uint4v *__restrict__ q
     }
 }
 
-template <int MT, int TERMS, int TPW, int KS>
+template <int MT, int TERMS, int TPW, int KS, int WPS = 4>
 static hipError_t launch_batch_t(hipStream_t s, const WeightView &w, const void *a, uint32_t m, const OutSpec &out,
                                  uint32_t splits, float *partials, uint32_t lo_offset)
 {
     uint32_t cps = (w.k_chunks + splits - 1) / splits;
     splits = (w.k_chunks + cps - 1) / cps;  // no empty split
     const uint32_t quads = w.n_tiles / 4;   // n_tiles is a multiple of 4
-    dim3 grid((quads + TPW - 1) / TPW, splits);
-    hipLaunchKernelGGL((k_batch<MT, TERMS, TPW, KS>), grid, dim3(256 * KS), 0, s, (const uint4v *)w.qw, (const uint2v *)w.sc, a, out,
+    constexpr uint32_t kQuadsPerGroup = WPS * TPW / 4;
+    dim3 grid((quads + kQuadsPerGroup - 1) / kQuadsPerGroup, splits);
+    hipLaunchKernelGGL((k_batch<MT, TERMS, TPW, KS, WPS>), grid, dim3(64 * WPS * KS), 0, s, (const uint4v *)w.qw, (const uint2v *)w.sc, a, out,
                        splits > 1 ? partials : nullptr, m, w.k, w.n, w.n_tiles, w.k_chunks, cps, lo_offset);
     if (splits > 1) {
         hipError_t e = launch_splitk_reduce(s, partials, out, m, w.n, w.n_tiles * 16, splits);
@@ -337,8 +356,19 @@ static hipError_t launch_batch_t(hipStream_t s, const WeightView &w, const void 
 // (its staging buffers would need 128 KB of LDS); otherwise two.
 template <int MT, int TERMS, int TPW>
 static hipError_t launch_batch_slices(hipStream_t s, const WeightView &w, const void *a, uint32_t m, const OutSpec &out,
-                                      uint32_t splits, uint32_t k_slices, float *partials, uint32_t lo_offset)
+                                      uint32_t splits, uint32_t k_slices, uint32_t quads_per_group, float *partials,
+                                      uint32_t lo_offset)
 {
+    if constexpr (TPW == 1) {
+        // two or three quads per workgroup (eight or twelve waves per slice; two slices only with eight)
+        if (quads_per_group == 3) return launch_batch_t<MT, TERMS, 1, 1, 12>(s, w, a, m, out, splits, partials, lo_offset);
+        if (quads_per_group == 2) {
+            if constexpr (!(MT == 2 && TERMS == 2)) {
+                if (k_slices >= 2) return launch_batch_t<MT, TERMS, 1, 2, 8>(s, w, a, m, out, splits, partials, lo_offset);
+            }
+            return launch_batch_t<MT, TERMS, 1, 1, 8>(s, w, a, m, out, splits, partials, lo_offset);
+        }
+    }
     if constexpr (TPW == 1 && !(MT == 2 && TERMS == 2)) {
         if (k_slices == 4) return launch_batch_t<MT, TERMS, TPW, 4>(s, w, a, m, out, splits, partials, lo_offset);
     }
@@ -346,17 +376,19 @@ static hipError_t launch_batch_slices(hipStream_t s, const WeightView &w, const 
     return launch_batch_t<MT, TERMS, TPW, 1>(s, w, a, m, out, splits, partials, lo_offset);
 }
 
-// M <= 32.  two_row_blocks: take the 32-row variant (f16-rounded weights) also for 16 rows or fewer -- the last rows
+// M <= 32.  quads_per_group: 1, 2 or 3 column quads per workgroup sharing one activation tile (one tile per wave; with
+// two tiles per wave the workgroup owns two quads anyway).  two_row_blocks: take the 32-row variant (f16-rounded weights) also for 16 rows or fewer -- the last rows
 // of a larger M, so that one call runs one arithmetic.  tiles_per_wave: 1 or 2 (a gated store without split-K needs 2).  `scratch` holds, for f32 activations,
 // their two f16 terms (2 x M x K halves) and after them the split-K partials (splits x M x (n_tiles * 16) floats);
 // the split factor is cut to what fits.
 hipError_t launch_batch(hipStream_t s, const WeightView &w, const void *a, bool a_f32, uint32_t m, const OutSpec &out,
-                        uint32_t splits, uint32_t tiles_per_wave, uint32_t k_slices, bool two_row_blocks, float *scratch,
-                        size_t scratch_bytes)
+                        uint32_t splits, uint32_t tiles_per_wave, uint32_t k_slices, uint32_t quads_per_group,
+                        bool two_row_blocks, float *scratch, size_t scratch_bytes)
 {
     if (m == 0 || w.n == 0) return hipSuccess;
     if (m > 32 || w.k_chunks == 0 || w.n_tiles % 4 != 0) return hipErrorInvalidValue;
     if (tiles_per_wave != 1 && tiles_per_wave != 2) return hipErrorInvalidValue;
+    if (quads_per_group < 1 || quads_per_group > 3) return hipErrorInvalidValue;
     if (k_slices != 1 && k_slices != 2 && k_slices != 4) return hipErrorInvalidValue;
     float *partials = scratch;
     size_t partial_bytes = scratch ? scratch_bytes : 0;
@@ -379,7 +411,7 @@ hipError_t launch_batch(hipStream_t s, const WeightView &w, const void *a, bool 
     if (splits < 1) splits = 1;
     if (w.k_chunks < splits) splits = w.k_chunks;
     if (out.swiglu && splits == 1) tiles_per_wave = 2;
-#define TWM_BATCH_CASE(MT, T, P) return launch_batch_slices<MT, T, P>(s, w, a, m, out, splits, k_slices, partials, lo_offset)
+#define TWM_BATCH_CASE(MT, T, P) return launch_batch_slices<MT, T, P>(s, w, a, m, out, splits, k_slices, quads_per_group, partials, lo_offset)
     if (m <= 16 && !two_row_blocks) {
         if (tiles_per_wave == 2) { if (a_f32) TWM_BATCH_CASE(1, 2, 2); TWM_BATCH_CASE(1, 1, 2); }
         if (a_f32) TWM_BATCH_CASE(1, 2, 1);

@@ -123,8 +123,8 @@ hipError_t launch_stream(hipStream_t s, const WeightView &w, const void *a, bool
 hipError_t launch_split_hi_lo(hipStream_t s, const float *a, _Float16 *hi, _Float16 *lo, size_t count);
 // batched decode with the activations shared through LDS (M <= 32); tiles_per_wave 1 or 2, k_slices 1, 2 or 4
 hipError_t launch_batch(hipStream_t s, const WeightView &w, const void *a, bool a_f32, uint32_t m, const OutSpec &out,
-                        uint32_t splits, uint32_t tiles_per_wave, uint32_t k_slices, bool two_row_blocks, float *scratch,
-                        size_t scratch_bytes);
+                        uint32_t splits, uint32_t tiles_per_wave, uint32_t k_slices, uint32_t quads_per_group,
+                        bool two_row_blocks, float *scratch, size_t scratch_bytes);
 hipError_t launch_geglu_rows(hipStream_t s, const float *gu, float *out, uint32_t dim, uint32_t batch, bool paired);
 // act: 0 out[slot][n]; 1 gelu_tanh(gate) * up, 2 silu(gate) * up into out[slot][n/2] (paired bank)
 hipError_t launch_bank_gemv(hipStream_t s, const BankView &b, const void *a, bool a_f32, uint32_t a_slot_stride,

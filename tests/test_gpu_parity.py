@@ -706,9 +706,10 @@ def test_five_to_eight_rows_on_wide_matrices(dev):
 
 
 def test_lds_shared_batched_decode_kernel(dev):
-    # option "kernel" = 4: one or two tiles per wave ("nt"), one / two / four k-slices per workgroup ("waves" 0 / 8 /
-    # 16), split-K over workgroups; ragged N and K (K not a multiple of 128), f16 and f32 rows, up to 16 rows against
-    # the exact-weight truth, 17 .. 32 rows against the f16-weight truth
+    # option "kernel" = 4: one or two tiles per wave ("nt" 1 / 2), two or three column quads per workgroup on one
+    # activation tile ("nt" 4 / 3), one / two / four k-slices per workgroup ("waves" 0 / 8 / 16), split-K over
+    # workgroups; ragged N and K (K not a multiple of 128), f16 and f32 rows, up to 16 rows against the exact-weight
+    # truth, 17 .. 32 rows against the f16-weight truth
     for k, n in ((160, 33), (416, 9000), (3584, 512)):
         packed, scales, a16 = synth(k, n, 32, 5200 + n)
         w = T.MarlinWeight.upload(dev, packed, scales, k, n)
@@ -717,7 +718,7 @@ def test_lds_shared_batched_decode_kernel(dev):
             for m in (5, 9, 16, 17, 31, 32):
                 truth = gemm_truth(a16[:m], packed, scales, m, k, n)
                 bar = TIGHT if m <= 16 else 1e-3
-                for nt in (1, 2):
+                for nt in (1, 2, 3, 4):
                     dev.set_option("nt", nt)
                     for waves in (0, 8, 16):
                         dev.set_option("waves", waves)
