@@ -1,4 +1,5 @@
-// Batched-decode kernel with the activations shared through LDS (M = 9 .. 32, and wide matrices from M = 5).
+// Batched-decode kernel with the activations shared through LDS (M = 17 .. 32; M = 9 .. 16 on wide matrices and with
+// f32 rows; M = 5 .. 8 with f32 rows on shallow K).
 //
 // Semantics, up to 16 rows: as the streaming kernel (reference order, crates/kernels/src/quantize.rs:1219-1238; M > 1
 // has the meaning of gemm_q4_0, quantize.rs:1825-1858): per 32-deep group the products a * (q - 8) are summed in f32
@@ -6,24 +7,26 @@
 // group sum is scaled once by f32(scale) and added to the running f32 sum, groups in ascending order.
 // 17 .. 32 rows: the reference's own M > 1 arithmetic, Q4 unpack to FP16 then FP16 GEMM with f32 accumulation
 // (quantize.rs:534-571, :1825-1858), as the prefill kernel: the B operand is f16_rne(f32(scale) * (q - 8)), made by one
-// packed f16 multiply, and the MFMAs accumulate over K directly (f32 activations still as two f16 terms).  (With two
-// row blocks the exact form costs eight f32 multiply-adds per tile and group after the MFMAs, and the kernel is bound
-// by the vector ALU: 3584 -> 37888 at M = 32 took 26.6 us that way.)
+// packed f16 multiply, and the MFMAs accumulate over K directly (f32 activations still as two f16 terms): with two
+// row blocks the exact form costs eight f32 multiply-adds per tile and group after the MFMAs.
 //
 // Why a second kernel: the streaming kernel keeps a whole chunk of activations (32 rows x 128 k) per wave in
 // registers, twice, so only two waves fit a SIMD and each has one chunk of weights in flight; at 32 rows it is
-// bound by the memory latency, not by HBM.  Here the four waves of a workgroup advance through K together and
-// share the activations through LDS:
-//   A : each wave loads a quarter of the chunk's 16 MT x 128 f16 tile (16 bytes per lane and row block), three
-//       chunks ahead in four register slots, and writes it to LDS one chunk ahead of its use (two LDS buffers,
-//       256-byte rows with XOR-swizzled 16-byte slots: conflict-free writes and operand reads); f32 activations
-//       are split beforehand into two f16 arrays (hi, lo) and both tiles are staged;
+// bound by the memory latency, not by HBM.  Here the waves of a slice (4, 8 or 12: one, two or three 64-column
+// quads) advance through K together and share the activations through LDS:
+//   A : the first 4 MT waves load four rows each of the chunk's 16 MT x 128 f16 tile (with four waves: MT times four
+//       rows), three chunks ahead in four register slots, and write them to LDS one chunk ahead of their use (two
+//       LDS buffers, 256-byte rows with XOR-swizzled 16-byte slots: conflict-free writes and operand reads); f32
+//       activations are split beforehand into two f16 arrays (hi, lo) and both tiles are staged;
 //   B : a wave owns TPW 16-column tiles; per chunk and tile 16 bytes of nibbles + 8 bytes of scales per lane,
 //       three chunks ahead in four register slots (6 TPW registers each);
 //   one barrier per chunk.
-// A wave then needs about 100 registers with three chunks of loads in flight (the streaming kernel: 170 with
-// one).  No reduction at the end: a wave holds complete sums of its tiles (or a K-split's partial sums).
-// Bound: HBM (weights are read once, the activations come from L2 once per workgroup and chunk).
+// A wave then needs 70 to 100 registers with three chunks of loads in flight (the streaming kernel: 170 with
+// one).  A wave holds complete sums of its tiles (or a K-split's partial sums; k-slices of one workgroup add theirs
+// through LDS at the end).
+// Bound: HBM for the weights, read once; the activation tile comes from L2 once per workgroup and chunk and its
+// requests share the CU's memory requests in flight with the weight stream, which is why more columns per
+// workgroup pay where they do not unbalance the CUs (the host's cost model chooses).
 #include "twm_device.h"
 
 namespace twm {
