@@ -149,6 +149,9 @@ def main():
     ap.add_argument("--no-vendor-gemm", action="store_true",
                     help="skip timing rocBLAS' dense FP16 GEMM beside the prefill kernel")
     ap.add_argument("--no-batched", action="store_true", help="skip the batched-decode layer (M = 4 .. 32)")
+    ap.add_argument("--batched-eager", action="store_true",
+                    help="batched-decode layer without graph capture (rocprofv3 has crashed in hipGraphLaunch of graphs this long)")
+    ap.add_argument("--no-small", action="store_true", help="skip the small configurations (Qwen-0.5B layer, 4096 x 4096)")
     ap.add_argument("--sweep-splits", action="store_true",
                     help="also time every projection at M=1,4,8,16,32 with forced split-K factors next to the library's "
                          "own choice (batched decode configuration)")
@@ -297,9 +300,12 @@ def main():
                         T.gemm(dev, layers[li][name][0], bufs[name][0], m, bufs[name][1])
             run_rows()
             dev.synchronize()
-            g_rows = T.GraphCapture.record_with_device(dev, run_rows)
-            ms = time_launches(dev, lambda i: g_rows.replay(), max(4, steps // L // 4)) / L
-            graphs_done.append(g_rows)
+            if args.batched_eager:      # for a kernel trace: launches issued one by one (the host then sets the pace)
+                ms = time_launches(dev, lambda i: run_rows(), max(4, steps // L // 4)) / L
+            else:
+                g_rows = T.GraphCapture.record_with_device(dev, run_rows)
+                ms = time_launches(dev, lambda i: g_rows.replay(), max(4, steps // L // 4)) / L
+                graphs_done.append(g_rows)
             lb = sum(algo_bytes(k, n, m) for _, k, n in LAYER_7B)
             extra["layer_M%d" % m] = {"us": round(ms * 1e3, 2), "GBps": round(lb / (ms * 1e-3) / 1e9, 1),
                                       "frac_hbm": round(lb / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
@@ -307,7 +313,7 @@ def main():
     log("small configurations")
     # the small configurations: launch- and latency-bound, reported per projection and as one graph per layer
     small = {}
-    for label, shapes in (("qwen05b", LAYER_05B), ("cfg0", CFG0)):
+    for label, shapes in (() if args.no_small else (("qwen05b", LAYER_05B), ("cfg0", CFG0))):
         sets = []
         for _ in range(8):                                   # 8 x 9.4 MB: still inside the 256 MB cache, as in a real
             host = make_layer(rng, shapes)                   # 0.5B model (all weights 250 MB) these shapes would be
