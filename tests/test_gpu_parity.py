@@ -48,12 +48,15 @@ def f16_as_f32(bits):
     return bits.view(np.float16).astype(np.float32)
 
 
-def gemm_truth(a16, packed, scales, m, k, n):
+EXACT_MAX_M = 32   # the decode kernels (M <= 32) use exact weights; the prefill GEMM above that the FP16 Q4 unpack
+
+
+def gemm_truth(a16, packed, scales, m, k, n, rounded=False):
     """f64 dequant-then-matmul the library's default path is held to: exact weights f32(scale)*(q-8) up to
-    M = 16; from M = 17 on the FP16 Q4 unpack f16(scale*(q-8)) (the 32-row batched-decode kernel and the
-    prefill GEMM), which is the reference's M > 1 route (quantize.rs:534-571 then an FP16 GEMM)."""
+    M = 32 (every decode kernel); above that, or with rounded=True, the FP16 Q4 unpack f16(scale*(q-8)) of the
+    prefill GEMM, which is the reference's dequant-then-FP16-GEMM route (quantize.rs:534-571)."""
     a = f16_as_f32(a16).reshape(m, k)
-    if m <= 16:
+    if m <= EXACT_MAX_M and not rounded:
         return O.gemm_f64(a, packed, scales, m, k, n)
     w16 = O.dequant_f16(packed, scales, k, n).view(np.float16).astype(np.float64).reshape(k, n)
     return a.astype(np.float64) @ w16
@@ -244,7 +247,7 @@ def test_gemm_swiglu_batched_and_prefill_rows(dev, m, splits):
     t = gemm_truth(a16, fp, fs, m, h, 2 * ffn)
     tg, tu = t[:, :ffn], t[:, ffn:]
     truth = tg / (1.0 + np.exp(-tg)) * tu
-    bar = TIGHT if m <= 16 else 1e-3
+    bar = TIGHT if m <= EXACT_MAX_M else 1e-3
     assert rel_err(out.to_host(), truth) < bar
     j = np.arange(ffn)
     col = (j // 32) * 64 + j % 32
@@ -282,7 +285,7 @@ def test_gemm_geglu_gate(dev, m, splits):
     t = gemm_truth(a16, fp, fs, m, h, 2 * ffn)
     tg, tu = t[:, :ffn], t[:, ffn:]
     truth = 0.5 * tg * (1.0 + np.tanh(0.7978845608 * (tg + 0.044715 * tg ** 3))) * tu
-    assert rel_err(out.to_host(), truth) < (TIGHT if m <= 16 else 1e-3)
+    assert rel_err(out.to_host(), truth) < (TIGHT if m <= EXACT_MAX_M else 1e-3)
     w.free()
 
 
@@ -416,6 +419,20 @@ def test_gemm_tw_marlin_m1_from_buffer_and_errors(dev):
     finally:
         dev.set_option("m1_exact", 0)
     assert np.array_equal(c.to_host(), O.gemv_ref_order(a, packed, scales, 1, k, n, 1)[0])
+    # an offset that keeps only the 4-byte alignment the reference's own kernel needs (it reads a record as four
+    # 32-bit words, quantize.rs:1227-1228), with and without the reference's split-K: the f32 kernel takes over
+    for kk, nn in ((128, 64), (2048, 96)):
+        pk, sc_, a16b = synth(kk, nn, 1, 10 + kk)
+        ab = f16_as_f32(a16b)
+        slab = np.concatenate([np.zeros(36, np.uint8), pk])
+        cb = T.GpuTensor.from_host(dev, np.full(nn, np.nan, np.float32))
+        T.gemm_tw_marlin_m1_from_buffer(dev, T.GpuTensor.from_host(dev, ab), T.GpuTensor.from_host(dev, slab), 36,
+                                        T.GpuTensor.from_host(dev, sc_, "f16"), 0, cb, nn, kk)
+        assert rel_err(cb.to_host(), O.gemm_f64(ab, pk, sc_, 1, kk, nn)[0]) < TIGHT
+        with pytest.raises(T.DeviceError) as e2:         # not even 4-byte aligned: a fault in the reference
+            T.gemm_tw_marlin_m1_from_buffer(dev, T.GpuTensor.from_host(dev, ab), T.GpuTensor.from_host(dev, slab), 35,
+                                            T.GpuTensor.from_host(dev, sc_, "f16"), 0, cb, nn, kk)
+        assert e2.value.code == T._lib.SHAPE_ERROR
     with pytest.raises(T.DeviceError) as e:              # the reference asserts k % 32 == 0 (quantize.rs:1311)
         T.gemm_tw_marlin_m1(dev, c, c, c, c, n, 100)
     assert e.value.code == T._lib.SHAPE_ERROR
@@ -443,10 +460,18 @@ def test_gemm_matches_golden(dev, name):
     w = T.MarlinWeight.upload(dev, d["packed"], d["scales"], k, n)
     for a_f32 in (False, True):
         got = run_gemm(dev, w, d["a_f16"], m, n, a_f32=a_f32)
-        if m <= 16:
+        if m <= EXACT_MAX_M:
             assert rel_err(got, d["c_f64"]) < TIGHT, (name, a_f32)
+            if m > 16:   # option: the 32-row batched-decode kernel on the FP16 Q4 unpack (the fixture's dequant_f16)
+                w16 = d["dequant_f16"].view(np.float16).astype(np.float64).reshape(k, n)
+                exact = f16_as_f32(d["a_f16"]).astype(np.float64).reshape(m, k) @ w16
+                dev.set_option("batch_rounded", 1)
+                try:
+                    assert rel_err(run_gemm(dev, w, d["a_f16"], m, n, a_f32=a_f32), exact) < TIGHT, (name, a_f32)
+                finally:
+                    dev.set_option("batch_rounded", 0)
         else:
-            # M > 16 runs the MFMAs on the FP16 Q4 unpack (the fixture's dequant_f16), like the reference's
+            # M > 32 runs the MFMAs on the FP16 Q4 unpack (the fixture's dequant_f16), like the reference's
             # dequant-then-matmul; against the f32-weight result the weight rounding (2^-12 each) shows
             w16 = d["dequant_f16"].view(np.float16).astype(np.float64).reshape(k, n)
             exact = f16_as_f32(d["a_f16"]).astype(np.float64).reshape(m, k) @ w16
@@ -473,9 +498,9 @@ def test_reference_gemm_q4_0_correctness_case(dev, m):
     full = a.astype(np.float64) @ b.astype(np.float64)
     nrmse = np.sqrt(((got - full) ** 2).sum() / max((full ** 2).sum(), 1e-10))
     assert nrmse < 0.15
-    if m <= 16:
+    if m <= EXACT_MAX_M:
         assert rel_err(got, O.gemm_f64(a, ph, sh, m, k, n)) < TIGHT
-    else:   # M > 16: f16 activations and the FP16 Q4 unpack
+    else:   # the prefill GEMM: f16 activations and the FP16 Q4 unpack
         w16 = O.dequant_f16(ph, sh, k, n).view(np.float16).astype(np.float64).reshape(k, n)
         assert rel_err(got, a.astype(np.float16).astype(np.float64) @ w16) < TIGHT
     if m == 1:
@@ -545,15 +570,11 @@ def test_batched_decode_7b_shapes(dev, m, k, n):
     w = T.MarlinWeight.upload(dev, packed, scales, k, n)
     truth = gemm_truth(a16, packed, scales, m, k, n)
     got = run_gemm(dev, w, a16, m, n)
-    assert rel_err(got, truth) < (TIGHT if m <= 16 else 1e-3)
+    assert rel_err(got, truth) < TIGHT
     # every row of the batch agrees with the same row run alone (another kernel variant and
-    # summation order, so agreement is to f32 rounding, not bitwise; M = 32 also differs by the
-    # FP16 rounding of the weights, 2^-12 each, which shows relative to the largest output)
+    # summation order, so agreement is to f32 rounding, not bitwise)
     alone = run_gemm(dev, w, a16[m - 1:m], 1, n)
-    if m <= 16:
-        assert rel_err(alone[0], got[m - 1]) < TIGHT
-    else:
-        assert np.abs(alone[0] - got[m - 1]).max() / np.abs(alone[0]).max() < 1e-3
+    assert rel_err(alone[0], got[m - 1]) < TIGHT
     w.free()
 
 
@@ -708,16 +729,17 @@ def test_five_to_eight_rows_on_wide_matrices(dev):
 def test_lds_shared_batched_decode_kernel(dev):
     # option "kernel" = 4: one or two tiles per wave ("nt" 1 / 2), two or three column quads per workgroup on one
     # activation tile ("nt" 4 / 3), one / two / four k-slices per workgroup ("waves" 0 / 8 / 16), split-K over
-    # workgroups; ragged N and K (K not a multiple of 128), f16 and f32 rows, up to 16 rows against the exact-weight
-    # truth, 17 .. 32 rows against the f16-weight truth
+    # workgroups; ragged N and K (K not a multiple of 128), f16 and f32 rows, against the exact-weight truth; 17 .. 32
+    # rows also with option "batch_rounded" against the f16-weight truth
     for k, n in ((160, 33), (416, 9000), (3584, 512)):
         packed, scales, a16 = synth(k, n, 32, 5200 + n)
         w = T.MarlinWeight.upload(dev, packed, scales, k, n)
         try:
             dev.set_option("kernel", 4)
-            for m in (5, 9, 16, 17, 31, 32):
-                truth = gemm_truth(a16[:m], packed, scales, m, k, n)
-                bar = TIGHT if m <= 16 else 1e-3
+            for m, rounded in ((5, 0), (9, 0), (16, 0), (17, 0), (31, 0), (32, 0), (17, 1), (32, 1)):
+                dev.set_option("batch_rounded", rounded)
+                truth = gemm_truth(a16[:m], packed, scales, m, k, n, rounded=bool(rounded))
+                bar = 1e-3 if rounded else TIGHT
                 for nt in (1, 2, 3, 4):
                     dev.set_option("nt", nt)
                     for waves in (0, 8, 16):
@@ -733,12 +755,12 @@ def test_lds_shared_batched_decode_kernel(dev):
                 assert np.array_equal(run_gemm(dev, w, a16[:m], m, n, 3), run_gemm(dev, w, a16[:m], m, n, 3))
                 dev.set_option("waves", 0)
         finally:
-            for key in ("kernel", "nt", "waves"):
+            for key in ("kernel", "nt", "waves", "batch_rounded"):
                 dev.set_option(key, 0)
         # the library's own plan takes this kernel from 17 rows on (and from 9 on wide matrices): same bits as forced
         for m in ((12, 20, 32) if n > 8192 else (20, 32)):
             auto = run_gemm(dev, w, a16[:m], m, n)
-            assert rel_err(auto, gemm_truth(a16[:m], packed, scales, m, k, n)) < (TIGHT if m <= 16 else 1e-3), (k, n, m)
+            assert rel_err(auto, gemm_truth(a16[:m], packed, scales, m, k, n)) < TIGHT, (k, n, m)
         w.free()
     # the gated store (two tiles per wave: a gate tile and the up tile of the same features in one lane), unsplit and
     # through the split-K partial sums
@@ -755,7 +777,7 @@ def test_lds_shared_batched_decode_kernel(dev):
         for splits in (0, 2):
             out = T.GpuTensor.from_host(dev, np.full((m, ffn), np.nan, np.float32))
             T.gemm_swiglu(dev, wp, T.GpuTensor.from_host(dev, a16, "f16"), m, out, splits)
-            assert rel_err(out.to_host(), want) < (TIGHT if m <= 16 else 1e-3), (m, splits)
+            assert rel_err(out.to_host(), want) < TIGHT, (m, splits)
     wp.free()
 
 
@@ -808,9 +830,6 @@ def test_f32_activations_keep_their_precision(dev, m):
     w = T.MarlinWeight.upload(dev, packed, scales, k, n)
     truth = O.gemm_f64(a_raw, packed, scales, m, k, n)
     held_to, bar = truth, TIGHT
-    if m > 16:   # from 17 rows on the weights are the FP16 Q4 unpack; the activations keep both terms all the same
-        w16 = O.dequant_f16(packed, scales, k, n).view(np.float16).astype(np.float64).reshape(k, n)
-        held_to, bar = a_raw.astype(np.float64) @ w16, 1e-3
     for splits in (0, 1, 3):
         c = T.GpuTensor.from_host(dev, np.full((m, n), np.nan, np.float32))
         T.gemm(dev, w, T.GpuTensor.from_host(dev, a_raw), m, c, splits)
@@ -835,7 +854,7 @@ def test_random_shapes_against_the_oracle(dev):
         w = T.MarlinWeight.upload(dev, packed, scales, k, n)
         got = run_gemm(dev, w, a16, m, n, splits, a_f32)
         truth = gemm_truth(a16, packed, scales, m, k, n)
-        assert rel_err(got, truth) < (TIGHT if m <= 16 else 1e-3), (case, k, n, m, splits, a_f32)
+        assert rel_err(got, truth) < (TIGHT if m <= EXACT_MAX_M else 1e-3), (case, k, n, m, splits, a_f32)
         assert np.array_equal(w.dequant_f16().to_host().reshape(-1), O.dequant_f16(packed, scales, k, n).reshape(-1)), case
         if m == 1:
             c = T.GpuTensor.from_host(dev, np.full(n, np.nan, np.float32))
@@ -868,21 +887,33 @@ def test_random_deep_shapes_against_the_oracle(dev):
 
 
 def test_m_larger_than_32_is_tiled_by_the_decode_kernels(dev):
-    # with the prefill kernel switched off, any M runs as 32-row blocks of the batched-decode kernel (FP16 Q4 unpack,
-    # the last 6 rows included: one call, one arithmetic), or as 32-row blocks of the exact-weight streaming kernel
+    # with the prefill kernel switched off, any M runs as 32-row blocks of the batched-decode kernel (exact weights;
+    # with option "batch_rounded" the FP16 Q4 unpack, the last 6 rows included: one call, one arithmetic), or as
+    # 32-row blocks of the streaming kernel
     m, k, n = 70, 256, 128
     packed, scales, a16 = synth(k, n, m, 33)
     w = T.MarlinWeight.upload(dev, packed, scales, k, n)
     try:
         dev.set_option("prefill_min_m", 1 << 30)
+        exact = O.gemm_f64(f16_as_f32(a16), packed, scales, m, k, n)
         got = run_gemm(dev, w, a16, m, n)
-        assert rel_err(got, gemm_truth(a16, packed, scales, m, k, n)) < 1e-3
+        assert rel_err(got, exact) < TIGHT
         for lo, hi in ((0, 32), (32, 64), (64, 70)):
-            assert np.array_equal(got[lo:hi], run_gemm(dev, w, a16[lo:hi], hi - lo, n) if hi - lo > 16 else got[lo:hi])
+            block = run_gemm(dev, w, a16[lo:hi], hi - lo, n)
+            if hi - lo > 16:
+                assert np.array_equal(got[lo:hi], block)
+            else:       # six rows alone take another kernel: the same sums in another order
+                assert rel_err(block, got[lo:hi]) < TIGHT
+        dev.set_option("batch_rounded", 1)
+        got = run_gemm(dev, w, a16, m, n)
+        assert rel_err(got, gemm_truth(a16, packed, scales, m, k, n, rounded=True)) < 1e-3
+        assert np.abs(got - exact).max() / np.abs(exact).max() < 1e-3
+        dev.set_option("batch_rounded", 0)
         dev.set_option("kernel", 3)
         assert rel_err(run_gemm(dev, w, a16, m, n), O.gemm_f64(f16_as_f32(a16), packed, scales, m, k, n)) < TIGHT
     finally:
         dev.set_option("kernel", 0)
+        dev.set_option("batch_rounded", 0)
         dev.set_option("prefill_min_m", 33)
     w.free()
 
@@ -913,15 +944,20 @@ def test_prefill_kernel_matches_oracle(dev, m, k, n):
     finally:
         dev.set_option("prefill_bm", 0)
         dev.set_option("prefill_min_m", 33)
-    # with the prefill kernel off: the batched-decode kernel runs the same arithmetic in 32-row blocks, and the
-    # exact-weight streaming kernel agrees with both to the weight rounding
+    # with the prefill kernel off: the batched-decode kernel runs the same arithmetic in 32-row blocks under option
+    # "batch_rounded"; by default it and the streaming kernel use the exact weights
     try:
         dev.set_option("prefill_min_m", 1 << 30)
-        assert rel_err(run_gemm(dev, w, a16, m, n), exact) < 1e-3
+        assert rel_err(run_gemm(dev, w, a16, m, n), truth) < TIGHT
+        dev.set_option("batch_rounded", 1)
+        if m > 16:
+            assert rel_err(run_gemm(dev, w, a16, m, n), exact) < 1e-3
+        dev.set_option("batch_rounded", 0)
         dev.set_option("kernel", 3)
         assert rel_err(run_gemm(dev, w, a16, m, n), truth) < TIGHT
     finally:
         dev.set_option("kernel", 0)
+        dev.set_option("batch_rounded", 0)
         dev.set_option("prefill_min_m", 33)
     w.free()
 
