@@ -100,6 +100,8 @@ int twm_ctx_info(twm_ctx *ctx, char *buf, size_t buf_len);
  *                   the reference's split-K rule and float atomics (bit-equal to the reference order when that
  *                   rule yields one split); 0 (default) = the MFMA kernel
  *   "m1_splits"     twm_gemm_tw_marlin_m1: split-K factor of the MFMA kernel (0 .. 64)
+ *   "batch_rounded" twm_gemm at M = 17 .. 32: 1 = weights rounded to f16 and summed over K by the MFMAs, the arithmetic
+ *                   of the prefill GEMM; 0 (default) = exact weights with f32 group scales as for M <= 16
  * Values outside these sets return TWM_SHAPE_ERROR, unknown keys TWM_UNSUPPORTED_OP. */
 int twm_ctx_set_option(twm_ctx *ctx, const char *key, int value);
 
@@ -180,11 +182,12 @@ int twm_argmax_f32(twm_ctx *ctx, const float *input_dev, uint32_t rows, uint32_t
 /* ---- the quantized-GEMM entry point, reference layout in, no repack ------------------ */
 
 /* gemm_tw_marlin_m1 (quantize.rs:1301-1360): C[1,N] = A[1,K] * dequant(packed, scales),
- * f32 activations and output, arrays exactly as the reference holds them (packed 16-byte aligned).
+ * f32 activations and output, arrays exactly as the reference holds them (packed at least 4-byte aligned, the
+ * alignment the reference's own kernel needs; 16-byte aligned for the fast kernel).
  * Runs the M <= 4 MFMA kernel straight on those arrays: weights (q - 8) exact, every f32 activation
  * enters as two f16 terms a = f16(a) + f16(a - f16(a)) (about 22 bits; |a| must stay inside the f16
  * range), f32 sum per group times f32(scale), deterministic split-K.  Option "m1_exact" selects the
- * plain f32 kernel in the reference's order instead (also taken when a_dev is not 16-byte aligned).
+ * plain f32 kernel in the reference's order instead (also taken when a_dev or packed_dev is not 16-byte aligned).
  * K % 32 != 0 returns TWM_SHAPE_ERROR where the reference asserts (quantize.rs:1311).
  * Uses the context's scratch like twm_gemm. */
 int twm_gemm_tw_marlin_m1(twm_ctx *ctx, const float *a_dev, const uint8_t *packed_dev,
@@ -228,10 +231,9 @@ int twm_weight_dequant_f16(twm_ctx *ctx, const twm_weight *w, uint16_t *out_kn_d
 /* C[M,N] (f32, row-major) = A[M,K] (f16 or f32, row-major) * dequant(W), f32 accumulation.
  * M = 1 is gemm_tw_marlin_m1 (quantize.rs:1301); M > 1 has the semantics of gemm_q4_0
  * (quantize.rs:1825-1858).  splits = 0 lets the library choose (twm_pick_splits).
- * M <= 16: decode kernels (M <= 4 one lane per column, above that 16-column tiles), weights exact,
- *          each group's f32 sum scaled by f32(scale).
- * M = 17 .. 32: batched-decode kernel on the reference's FP16 Q4 unpack, f16(scale * (q - 8)), as in
- *          its dequant-then-matmul route for M > 1.
+ * M <= 32: decode kernels (M <= 4 one lane per column, above that 16-column tiles), weights exact,
+ *          each group's f32 sum scaled by f32(scale): a row's result does not depend on the batch it is in
+ *          beyond f32 summation order.  (Option "batch_rounded": M = 17 .. 32 on the FP16 Q4 unpack.)
  * Up to M = 32 f32 activations enter as two f16 terms, f16(a) + f16(a - f16(a)), about 22 bits (|a|
  * inside the f16 range).
  * M  > 32: prefill GEMM on the same FP16 unpack; f32 activations are rounded to f16 first.  Uses the

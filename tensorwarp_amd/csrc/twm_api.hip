@@ -16,7 +16,7 @@ using namespace twm;
 
 static thread_local std::string g_err;
 
-static int fail(int code, const char *fmt, ...)
+int twm::api_fail(int code, const char *fmt, ...)
 {
     char buf[512];
     va_list ap;
@@ -30,7 +30,7 @@ static int fail(int code, const char *fmt, ...)
 #define HIP_TRY(expr, code, what)                                                      \
     do {                                                                               \
         hipError_t e__ = (expr);                                                       \
-        if (e__ != hipSuccess) return fail(code, "%s: %s", what, hipGetErrorString(e__)); \
+        if (e__ != hipSuccess) return api_fail(code, "%s: %s", what, hipGetErrorString(e__)); \
     } while (0)
 
 struct twm_ctx {
@@ -52,6 +52,7 @@ struct twm_ctx {
     int dequant_src;      // which copy twm_weight_dequant_f16 unpacks: 0 = 16-column tiles, 1 = column-lane
     int m1_exact;         // twm_gemm_tw_marlin_m1: 1 = f32 activations and f32 FMAs in the reference's order
     int m1_splits;        // twm_gemm_tw_marlin_m1: split-K factor of the MFMA kernel, 0 = heuristic
+    int batch_rounded;    // M = 17 .. 32: 1 = weights rounded to f16 (the reference's dequant-then-FP16-GEMM arithmetic), 0 = exact
     hipDeviceProp_t prop;
 };
 
@@ -99,12 +100,12 @@ twm_ctx *twm_ctx_create(int ordinal)
     int count = 0;
     hipError_t e = hipGetDeviceCount(&count);
     if (e != hipSuccess || ordinal < 0 || ordinal >= count) {
-        fail(TWM_DEVICE_ERROR, "twm_ctx_create: no HIP device %d (%s)", ordinal,
+        api_fail(TWM_DEVICE_ERROR, "twm_ctx_create: no HIP device %d (%s)", ordinal,
              e != hipSuccess ? hipGetErrorString(e) : "ordinal out of range");
         return nullptr;
     }
     twm_ctx *c = new (std::nothrow) twm_ctx();
-    if (!c) { fail(TWM_MEMORY_ERROR, "twm_ctx_create: out of host memory"); return nullptr; }
+    if (!c) { api_fail(TWM_MEMORY_ERROR, "twm_ctx_create: out of host memory"); return nullptr; }
     c->ordinal = ordinal;
     c->capturing = false;
     c->force_nt = 0;
@@ -114,6 +115,7 @@ twm_ctx *twm_ctx_create(int ordinal)
     c->dequant_src = 0;
     c->m1_exact = 0;
     c->m1_splits = 0;
+    c->batch_rounded = 0;
     c->prefill_bm = 0;
     c->prefill_min_m = 33;  // M <= 32 is batched decode (exact f32 scales, weights streamed once)
     c->ws = nullptr;
@@ -121,7 +123,7 @@ twm_ctx *twm_ctx_create(int ordinal)
     c->own_stream = nullptr;
     bool ok = hipSetDevice(ordinal) == hipSuccess && hipGetDeviceProperties(&c->prop, ordinal) == hipSuccess;
     if (ok && strncmp(c->prop.gcnArchName, "gfx950", 6) != 0) {
-        fail(TWM_DEVICE_ERROR, "twm_ctx_create: device %d is %s; this library holds gfx950 code only", ordinal,
+        api_fail(TWM_DEVICE_ERROR, "twm_ctx_create: device %d is %s; this library holds gfx950 code only", ordinal,
              c->prop.gcnArchName);
         delete c;
         return nullptr;
@@ -136,7 +138,7 @@ twm_ctx *twm_ctx_create(int ordinal)
     ok = ok && hipMemset(c->counters, 0, c->n_counters * sizeof(unsigned)) == hipSuccess;
     ok = ok && hipDeviceSynchronize() == hipSuccess;
     if (!ok) {
-        fail(TWM_DEVICE_ERROR, "twm_ctx_create: %s", hipGetErrorString(hipGetLastError()));
+        api_fail(TWM_DEVICE_ERROR, "twm_ctx_create: %s", hipGetErrorString(hipGetLastError()));
         if (c->ws) (void)hipFree(c->ws);
         if (c->counters) (void)hipFree(c->counters);
         if (c->own_stream) (void)hipStreamDestroy(c->own_stream);
@@ -159,15 +161,15 @@ void twm_ctx_destroy(twm_ctx *ctx)
 
 int twm_ctx_sync(twm_ctx *ctx)
 {
-    if (!ctx) return fail(TWM_INVALID_HANDLE, "twm_ctx_sync: null context");
+    if (!ctx) return api_fail(TWM_INVALID_HANDLE, "twm_ctx_sync: null context");
     HIP_TRY(hipStreamSynchronize(ctx->stream), TWM_DEVICE_ERROR, "stream synchronize");
     return TWM_OK;
 }
 
 int twm_ctx_set_stream(twm_ctx *ctx, void *hip_stream)
 {
-    if (!ctx) return fail(TWM_INVALID_HANDLE, "twm_ctx_set_stream: null context");
-    if (ctx->capturing) return fail(TWM_UNSUPPORTED_OP, "twm_ctx_set_stream: a graph capture is open");
+    if (!ctx) return api_fail(TWM_INVALID_HANDLE, "twm_ctx_set_stream: null context");
+    if (ctx->capturing) return api_fail(TWM_UNSUPPORTED_OP, "twm_ctx_set_stream: a graph capture is open");
     ctx->stream = hip_stream ? (hipStream_t)hip_stream : ctx->own_stream;
     return TWM_OK;
 }
@@ -176,7 +178,7 @@ void *twm_ctx_stream(twm_ctx *ctx) { return ctx ? (void *)ctx->stream : nullptr;
 
 int twm_ctx_info(twm_ctx *ctx, char *buf, size_t buf_len)
 {
-    if (!ctx || !buf || buf_len == 0) return fail(TWM_INVALID_HANDLE, "twm_ctx_info: null argument");
+    if (!ctx || !buf || buf_len == 0) return api_fail(TWM_INVALID_HANDLE, "twm_ctx_info: null argument");
     snprintf(buf, buf_len, "%s (%s) | %d CUs | %.1f GiB", ctx->prop.name, ctx->prop.gcnArchName,
              ctx->prop.multiProcessorCount, (double)ctx->prop.totalGlobalMem / (1024.0 * 1024.0 * 1024.0));
     return TWM_OK;
@@ -189,72 +191,77 @@ int twm_ctx_info(twm_ctx *ctx, char *buf, size_t buf_len)
  * runs the prefill kernel. */
 int twm_ctx_set_option(twm_ctx *ctx, const char *key, int value)
 {
-    if (!ctx || !key) return fail(TWM_INVALID_HANDLE, "twm_ctx_set_option: null argument");
+    if (!ctx || !key) return api_fail(TWM_INVALID_HANDLE, "twm_ctx_set_option: null argument");
     if (strcmp(key, "nt") == 0) {
-        if (value < 0 || value > 4) return fail(TWM_SHAPE_ERROR, "twm_ctx_set_option: nt must be 0 .. 4");
+        if (value < 0 || value > 4) return api_fail(TWM_SHAPE_ERROR, "twm_ctx_set_option: nt must be 0 .. 4");
         ctx->force_nt = value;
         return TWM_OK;
     }
     if (strcmp(key, "waves") == 0) {
         if (value != 0 && value != 1 && value != 2 && value != 4 && value != 8 && value != 16)
-            return fail(TWM_SHAPE_ERROR, "twm_ctx_set_option: waves must be 0, 1, 2, 4, 8 or 16");
+            return api_fail(TWM_SHAPE_ERROR, "twm_ctx_set_option: waves must be 0, 1, 2, 4, 8 or 16");
         ctx->force_waves = value;
         return TWM_OK;
     }
     if (strcmp(key, "sub") == 0) {
         if (value != 0 && value != 1 && value != 16 && value != 32)
-            return fail(TWM_SHAPE_ERROR, "twm_ctx_set_option: sub must be 0, 1, 16 or 32");
+            return api_fail(TWM_SHAPE_ERROR, "twm_ctx_set_option: sub must be 0, 1, 16 or 32");
         ctx->force_sub = value;
         return TWM_OK;
     }
     if (strcmp(key, "prefill_bm") == 0) {
-        if (value != 0 && value != 64 && value != 128) return fail(TWM_SHAPE_ERROR, "twm_ctx_set_option: prefill_bm must be 0, 64 or 128");
+        if (value != 0 && value != 64 && value != 128) return api_fail(TWM_SHAPE_ERROR, "twm_ctx_set_option: prefill_bm must be 0, 64 or 128");
         ctx->prefill_bm = value;
         return TWM_OK;
     }
     if (strcmp(key, "prefill_min_m") == 0) {
-        if (value < 1) return fail(TWM_SHAPE_ERROR, "twm_ctx_set_option: prefill_min_m must be >= 1");
+        if (value < 1) return api_fail(TWM_SHAPE_ERROR, "twm_ctx_set_option: prefill_min_m must be >= 1");
         ctx->prefill_min_m = value;
         return TWM_OK;
     }
     if (strcmp(key, "dequant_src") == 0) {
-        if (value != 0 && value != 1) return fail(TWM_SHAPE_ERROR, "twm_ctx_set_option: dequant_src must be 0 or 1");
+        if (value != 0 && value != 1) return api_fail(TWM_SHAPE_ERROR, "twm_ctx_set_option: dequant_src must be 0 or 1");
         ctx->dequant_src = value;
         return TWM_OK;
     }
     if (strcmp(key, "m1_exact") == 0) {
-        if (value != 0 && value != 1) return fail(TWM_SHAPE_ERROR, "twm_ctx_set_option: m1_exact must be 0 or 1");
+        if (value != 0 && value != 1) return api_fail(TWM_SHAPE_ERROR, "twm_ctx_set_option: m1_exact must be 0 or 1");
         ctx->m1_exact = value;
         return TWM_OK;
     }
     if (strcmp(key, "m1_splits") == 0) {
-        if (value < 0 || value > 64) return fail(TWM_SHAPE_ERROR, "twm_ctx_set_option: m1_splits must be 0 .. 64");
+        if (value < 0 || value > 64) return api_fail(TWM_SHAPE_ERROR, "twm_ctx_set_option: m1_splits must be 0 .. 64");
         ctx->m1_splits = value;
         return TWM_OK;
     }
+    if (strcmp(key, "batch_rounded") == 0) {
+        if (value != 0 && value != 1) return api_fail(TWM_SHAPE_ERROR, "twm_ctx_set_option: batch_rounded must be 0 or 1");
+        ctx->batch_rounded = value;
+        return TWM_OK;
+    }
     if (strcmp(key, "kernel") == 0) {
-        if (value < 0 || value > 4) return fail(TWM_SHAPE_ERROR, "twm_ctx_set_option: kernel must be 0 .. 4");
+        if (value < 0 || value > 4) return api_fail(TWM_SHAPE_ERROR, "twm_ctx_set_option: kernel must be 0 .. 4");
         ctx->force_kernel = value;
         return TWM_OK;
     }
-    return fail(TWM_UNSUPPORTED_OP, "twm_ctx_set_option: unknown key %s", key);
+    return api_fail(TWM_UNSUPPORTED_OP, "twm_ctx_set_option: unknown key %s", key);
 }
 
 /* ---- memory ---------------------------------------------------------------------------- */
 
 void *twm_malloc(twm_ctx *ctx, size_t bytes)
 {
-    if (!ctx) { fail(TWM_INVALID_HANDLE, "twm_malloc: null context"); return nullptr; }
-    if (ctx->capturing) { fail(TWM_UNSUPPORTED_OP, "twm_malloc: not allowed inside a graph capture"); return nullptr; }
+    if (!ctx) { api_fail(TWM_INVALID_HANDLE, "twm_malloc: null context"); return nullptr; }
+    if (ctx->capturing) { api_fail(TWM_UNSUPPORTED_OP, "twm_malloc: not allowed inside a graph capture"); return nullptr; }
     void *p = nullptr;
     hipError_t e = hipMalloc(&p, bytes ? bytes : 4);
-    if (e != hipSuccess) { fail(TWM_MEMORY_ERROR, "hipMalloc(%zu): %s", bytes, hipGetErrorString(e)); return nullptr; }
+    if (e != hipSuccess) { api_fail(TWM_MEMORY_ERROR, "hipMalloc(%zu): %s", bytes, hipGetErrorString(e)); return nullptr; }
     return p;
 }
 
 int twm_free(twm_ctx *ctx, void *ptr_dev)
 {
-    if (!ctx) return fail(TWM_INVALID_HANDLE, "twm_free: null context");
+    if (!ctx) return api_fail(TWM_INVALID_HANDLE, "twm_free: null context");
     if (!ptr_dev) return TWM_OK;
     HIP_TRY(hipFree(ptr_dev), TWM_MEMORY_ERROR, "hipFree");
     return TWM_OK;
@@ -262,10 +269,10 @@ int twm_free(twm_ctx *ctx, void *ptr_dev)
 
 int twm_memcpy_h2d(twm_ctx *ctx, void *dst_dev, const void *src_host, size_t bytes)
 {
-    if (!ctx) return fail(TWM_INVALID_HANDLE, "twm_memcpy_h2d: null context");
+    if (!ctx) return api_fail(TWM_INVALID_HANDLE, "twm_memcpy_h2d: null context");
     if (bytes == 0) return TWM_OK;
-    if (!dst_dev || !src_host) return fail(TWM_INVALID_HANDLE, "twm_memcpy_h2d: null pointer");
-    if (ctx->capturing) return fail(TWM_UNSUPPORTED_OP, "twm_memcpy_h2d: not allowed inside a graph capture");
+    if (!dst_dev || !src_host) return api_fail(TWM_INVALID_HANDLE, "twm_memcpy_h2d: null pointer");
+    if (ctx->capturing) return api_fail(TWM_UNSUPPORTED_OP, "twm_memcpy_h2d: not allowed inside a graph capture");
     HIP_TRY(hipMemcpyAsync(dst_dev, src_host, bytes, hipMemcpyHostToDevice, ctx->stream), TWM_MEMORY_ERROR, "memcpy h2d");
     HIP_TRY(hipStreamSynchronize(ctx->stream), TWM_DEVICE_ERROR, "memcpy h2d sync");
     return TWM_OK;
@@ -273,10 +280,10 @@ int twm_memcpy_h2d(twm_ctx *ctx, void *dst_dev, const void *src_host, size_t byt
 
 int twm_memcpy_d2h(twm_ctx *ctx, void *dst_host, const void *src_dev, size_t bytes)
 {
-    if (!ctx) return fail(TWM_INVALID_HANDLE, "twm_memcpy_d2h: null context");
+    if (!ctx) return api_fail(TWM_INVALID_HANDLE, "twm_memcpy_d2h: null context");
     if (bytes == 0) return TWM_OK;
-    if (!dst_host || !src_dev) return fail(TWM_INVALID_HANDLE, "twm_memcpy_d2h: null pointer");
-    if (ctx->capturing) return fail(TWM_UNSUPPORTED_OP, "twm_memcpy_d2h: not allowed inside a graph capture");
+    if (!dst_host || !src_dev) return api_fail(TWM_INVALID_HANDLE, "twm_memcpy_d2h: null pointer");
+    if (ctx->capturing) return api_fail(TWM_UNSUPPORTED_OP, "twm_memcpy_d2h: not allowed inside a graph capture");
     HIP_TRY(hipMemcpyAsync(dst_host, src_dev, bytes, hipMemcpyDeviceToHost, ctx->stream), TWM_MEMORY_ERROR, "memcpy d2h");
     HIP_TRY(hipStreamSynchronize(ctx->stream), TWM_DEVICE_ERROR, "memcpy d2h sync");
     return TWM_OK;
@@ -284,20 +291,20 @@ int twm_memcpy_d2h(twm_ctx *ctx, void *dst_host, const void *src_dev, size_t byt
 
 int twm_memcpy_d2d(twm_ctx *ctx, void *dst_dev, const void *src_dev, size_t bytes)
 {
-    if (!ctx) return fail(TWM_INVALID_HANDLE, "twm_memcpy_d2d: null context");
+    if (!ctx) return api_fail(TWM_INVALID_HANDLE, "twm_memcpy_d2d: null context");
     if (bytes == 0) return TWM_OK;
-    if (!dst_dev || !src_dev) return fail(TWM_INVALID_HANDLE, "twm_memcpy_d2d: null pointer");
+    if (!dst_dev || !src_dev) return api_fail(TWM_INVALID_HANDLE, "twm_memcpy_d2d: null pointer");
     HIP_TRY(hipMemcpyAsync(dst_dev, src_dev, bytes, hipMemcpyDeviceToDevice, ctx->stream), TWM_MEMORY_ERROR, "memcpy d2d");
     return TWM_OK;
 }
 
 int twm_memset_zero(twm_ctx *ctx, void *ptr_dev, size_t bytes)
 {
-    if (!ctx) return fail(TWM_INVALID_HANDLE, "twm_memset_zero: null context");
+    if (!ctx) return api_fail(TWM_INVALID_HANDLE, "twm_memset_zero: null context");
     if (bytes == 0) return TWM_OK;
-    if (!ptr_dev) return fail(TWM_INVALID_HANDLE, "twm_memset_zero: null pointer");
+    if (!ptr_dev) return api_fail(TWM_INVALID_HANDLE, "twm_memset_zero: null pointer");
     if (bytes % 4 != 0 || ((uintptr_t)ptr_dev & 3) != 0)
-        return fail(TWM_SHAPE_ERROR, "twm_memset_zero: pointer and size must be multiples of 4 bytes");
+        return api_fail(TWM_SHAPE_ERROR, "twm_memset_zero: pointer and size must be multiples of 4 bytes");
     HIP_TRY(launch_fill_zero(ctx->stream, ptr_dev, bytes), TWM_DEVICE_ERROR, "fill kernel launch");
     return TWM_OK;
 }
@@ -306,30 +313,30 @@ int twm_memset_zero(twm_ctx *ctx, void *ptr_dev, size_t bytes)
 
 void *twm_event_create(twm_ctx *ctx)
 {
-    if (!ctx) { fail(TWM_INVALID_HANDLE, "twm_event_create: null context"); return nullptr; }
+    if (!ctx) { api_fail(TWM_INVALID_HANDLE, "twm_event_create: null context"); return nullptr; }
     hipEvent_t ev = nullptr;
     hipError_t e = hipEventCreate(&ev);
-    if (e != hipSuccess) { fail(TWM_DEVICE_ERROR, "hipEventCreate: %s", hipGetErrorString(e)); return nullptr; }
+    if (e != hipSuccess) { api_fail(TWM_DEVICE_ERROR, "hipEventCreate: %s", hipGetErrorString(e)); return nullptr; }
     return (void *)ev;
 }
 
 int twm_event_destroy(twm_ctx *ctx, void *event)
 {
-    if (!ctx || !event) return fail(TWM_INVALID_HANDLE, "twm_event_destroy: null argument");
+    if (!ctx || !event) return api_fail(TWM_INVALID_HANDLE, "twm_event_destroy: null argument");
     HIP_TRY(hipEventDestroy((hipEvent_t)event), TWM_DEVICE_ERROR, "hipEventDestroy");
     return TWM_OK;
 }
 
 int twm_event_record(twm_ctx *ctx, void *event)
 {
-    if (!ctx || !event) return fail(TWM_INVALID_HANDLE, "twm_event_record: null argument");
+    if (!ctx || !event) return api_fail(TWM_INVALID_HANDLE, "twm_event_record: null argument");
     HIP_TRY(hipEventRecord((hipEvent_t)event, ctx->stream), TWM_DEVICE_ERROR, "hipEventRecord");
     return TWM_OK;
 }
 
 int twm_event_elapsed_ms(twm_ctx *ctx, void *start, void *stop, float *ms_out)
 {
-    if (!ctx || !start || !stop || !ms_out) return fail(TWM_INVALID_HANDLE, "twm_event_elapsed_ms: null argument");
+    if (!ctx || !start || !stop || !ms_out) return api_fail(TWM_INVALID_HANDLE, "twm_event_elapsed_ms: null argument");
     HIP_TRY(hipEventSynchronize((hipEvent_t)stop), TWM_DEVICE_ERROR, "hipEventSynchronize");
     HIP_TRY(hipEventElapsedTime(ms_out, (hipEvent_t)start, (hipEvent_t)stop), TWM_DEVICE_ERROR, "hipEventElapsedTime");
     return TWM_OK;
@@ -337,19 +344,19 @@ int twm_event_elapsed_ms(twm_ctx *ctx, void *start, void *stop, float *ms_out)
 
 /* ---- format operations -------------------------------------------------------------------- */
 
-static int check_kn(const char *who, uint32_t k, uint32_t n)
+extern "C++" int twm::check_kn(const char *who, uint32_t k, uint32_t n)
 {
-    if (k % 32 != 0) return fail(TWM_SHAPE_ERROR, "%s: K (%u) must be divisible by 32", who, k);
-    if ((uint64_t)(k / 32) * n * 16 > (1ull << 40)) return fail(TWM_SHAPE_ERROR, "%s: K x N too large", who);
+    if (k % 32 != 0) return api_fail(TWM_SHAPE_ERROR, "%s: K (%u) must be divisible by 32", who, k);
+    if ((uint64_t)(k / 32) * n * 16 > (1ull << 40)) return api_fail(TWM_SHAPE_ERROR, "%s: K x N too large", who);
     return TWM_OK;
 }
 
 int twm_quantize_weights_q4_0(twm_ctx *ctx, const float *w_kn_dev, uint32_t k, uint32_t n, uint8_t *q4_dev)
 {
-    if (!ctx) return fail(TWM_INVALID_HANDLE, "twm_quantize_weights_q4_0: null context");
+    if (!ctx) return api_fail(TWM_INVALID_HANDLE, "twm_quantize_weights_q4_0: null context");
     if (int rc = check_kn("twm_quantize_weights_q4_0", k, n)) return rc;
     if (k == 0 || n == 0) return TWM_OK;
-    if (!w_kn_dev || !q4_dev) return fail(TWM_INVALID_HANDLE, "twm_quantize_weights_q4_0: null pointer");
+    if (!w_kn_dev || !q4_dev) return api_fail(TWM_INVALID_HANDLE, "twm_quantize_weights_q4_0: null pointer");
     HIP_TRY(launch_quantize_q4_0(ctx->stream, w_kn_dev, k, n, q4_dev), TWM_DEVICE_ERROR, "quantize launch");
     return TWM_OK;
 }
@@ -357,10 +364,10 @@ int twm_quantize_weights_q4_0(twm_ctx *ctx, const float *w_kn_dev, uint32_t k, u
 int twm_reorder_to_tw_marlin(twm_ctx *ctx, const uint8_t *q4_dev, uint32_t k, uint32_t n, uint8_t *packed_dev,
                              uint16_t *scales_dev)
 {
-    if (!ctx) return fail(TWM_INVALID_HANDLE, "twm_reorder_to_tw_marlin: null context");
+    if (!ctx) return api_fail(TWM_INVALID_HANDLE, "twm_reorder_to_tw_marlin: null context");
     if (int rc = check_kn("twm_reorder_to_tw_marlin", k, n)) return rc;
     if (k == 0 || n == 0) return TWM_OK;
-    if (!q4_dev || !packed_dev || !scales_dev) return fail(TWM_INVALID_HANDLE, "twm_reorder_to_tw_marlin: null pointer");
+    if (!q4_dev || !packed_dev || !scales_dev) return api_fail(TWM_INVALID_HANDLE, "twm_reorder_to_tw_marlin: null pointer");
     HIP_TRY(launch_reorder(ctx->stream, q4_dev, k, n, packed_dev, scales_dev), TWM_DEVICE_ERROR, "reorder launch");
     return TWM_OK;
 }
@@ -368,11 +375,11 @@ int twm_reorder_to_tw_marlin(twm_ctx *ctx, const uint8_t *q4_dev, uint32_t k, ui
 int twm_quantize_f32_to_tw_marlin(twm_ctx *ctx, const float *w_dev, int w_is_nk, uint32_t k, uint32_t n,
                                   uint8_t *packed_dev, uint16_t *scales_dev)
 {
-    if (!ctx) return fail(TWM_INVALID_HANDLE, "twm_quantize_f32_to_tw_marlin: null context");
+    if (!ctx) return api_fail(TWM_INVALID_HANDLE, "twm_quantize_f32_to_tw_marlin: null context");
     if (int rc = check_kn("twm_quantize_f32_to_tw_marlin", k, n)) return rc;
     if (k == 0 || n == 0) return TWM_OK;
     if (!w_dev || !packed_dev || !scales_dev)
-        return fail(TWM_INVALID_HANDLE, "twm_quantize_f32_to_tw_marlin: null pointer");
+        return api_fail(TWM_INVALID_HANDLE, "twm_quantize_f32_to_tw_marlin: null pointer");
     HIP_TRY(launch_quantize_twm(ctx->stream, w_dev, w_is_nk, k, n, packed_dev, scales_dev), TWM_DEVICE_ERROR,
             "quantize launch");
     return TWM_OK;
@@ -381,18 +388,18 @@ int twm_quantize_f32_to_tw_marlin(twm_ctx *ctx, const float *w_dev, int w_is_nk,
 int twm_fuse_tw_marlin_n(twm_ctx *ctx, const uint8_t *const *packed_devs, const uint16_t *const *scales_devs, uint32_t k,
                          const uint32_t *ns, uint32_t count, uint8_t *packed_out_dev, uint16_t *scales_out_dev)
 {
-    if (!ctx) return fail(TWM_INVALID_HANDLE, "twm_fuse_tw_marlin_n: null context");
-    if (!packed_devs || !scales_devs || !ns) return fail(TWM_INVALID_HANDLE, "twm_fuse_tw_marlin_n: null array");
+    if (!ctx) return api_fail(TWM_INVALID_HANDLE, "twm_fuse_tw_marlin_n: null context");
+    if (!packed_devs || !scales_devs || !ns) return api_fail(TWM_INVALID_HANDLE, "twm_fuse_tw_marlin_n: null array");
     uint64_t total = 0;
     for (uint32_t i = 0; i < count; i++) total += ns[i];
-    if (total > 0xFFFFFFFFull) return fail(TWM_SHAPE_ERROR, "twm_fuse_tw_marlin_n: fused N overflows u32");
+    if (total > 0xFFFFFFFFull) return api_fail(TWM_SHAPE_ERROR, "twm_fuse_tw_marlin_n: fused N overflows u32");
     if (int rc = check_kn("twm_fuse_tw_marlin_n", k, (uint32_t)total)) return rc;
     if (total == 0 || k == 0) return TWM_OK;
-    if (!packed_out_dev || !scales_out_dev) return fail(TWM_INVALID_HANDLE, "twm_fuse_tw_marlin_n: null output");
+    if (!packed_out_dev || !scales_out_dev) return api_fail(TWM_INVALID_HANDLE, "twm_fuse_tw_marlin_n: null output");
     uint32_t off = 0;
     for (uint32_t i = 0; i < count; i++) {
         if (ns[i] == 0) continue;
-        if (!packed_devs[i] || !scales_devs[i]) return fail(TWM_INVALID_HANDLE, "twm_fuse_tw_marlin_n: null input %u", i);
+        if (!packed_devs[i] || !scales_devs[i]) return api_fail(TWM_INVALID_HANDLE, "twm_fuse_tw_marlin_n: null input %u", i);
         HIP_TRY(launch_fuse_one(ctx->stream, packed_devs[i], scales_devs[i], k / 32, ns[i], (uint32_t)total, off,
                                 packed_out_dev, scales_out_dev),
                 TWM_DEVICE_ERROR, "fuse launch");
@@ -404,10 +411,10 @@ int twm_fuse_tw_marlin_n(twm_ctx *ctx, const uint8_t *const *packed_devs, const 
 static int dequant_common(twm_ctx *ctx, const uint8_t *packed_dev, const uint16_t *scales_dev, uint32_t k, uint32_t n,
                           void *out, bool f16)
 {
-    if (!ctx) return fail(TWM_INVALID_HANDLE, "twm_dequant: null context");
+    if (!ctx) return api_fail(TWM_INVALID_HANDLE, "twm_dequant: null context");
     if (int rc = check_kn("twm_dequant", k, n)) return rc;
     if (k == 0 || n == 0) return TWM_OK;
-    if (!packed_dev || !scales_dev || !out) return fail(TWM_INVALID_HANDLE, "twm_dequant: null pointer");
+    if (!packed_dev || !scales_dev || !out) return api_fail(TWM_INVALID_HANDLE, "twm_dequant: null pointer");
     HIP_TRY(launch_dequant(ctx->stream, packed_dev, scales_dev, k, n, out, f16), TWM_DEVICE_ERROR, "dequant launch");
     return TWM_OK;
 }
@@ -427,9 +434,9 @@ int twm_dequant_to_f32(twm_ctx *ctx, const uint8_t *packed_dev, const uint16_t *
 int twm_split_qkv(twm_ctx *ctx, const float *qkv_dev, float *q_dev, float *k_dev, float *v_dev, uint32_t h,
                   uint32_t kv_dim, uint32_t batch)
 {
-    if (!ctx) return fail(TWM_INVALID_HANDLE, "twm_split_qkv: null context");
+    if (!ctx) return api_fail(TWM_INVALID_HANDLE, "twm_split_qkv: null context");
     if ((uint64_t)batch * ((uint64_t)h + 2ull * kv_dim) == 0) return TWM_OK;
-    if (!qkv_dev || !q_dev || !k_dev || !v_dev) return fail(TWM_INVALID_HANDLE, "twm_split_qkv: null pointer");
+    if (!qkv_dev || !q_dev || !k_dev || !v_dev) return api_fail(TWM_INVALID_HANDLE, "twm_split_qkv: null pointer");
     HIP_TRY(launch_split_qkv(ctx->stream, qkv_dev, q_dev, k_dev, v_dev, h, kv_dim, batch), TWM_DEVICE_ERROR,
             "split_qkv launch");
     return TWM_OK;
@@ -437,9 +444,9 @@ int twm_split_qkv(twm_ctx *ctx, const float *qkv_dev, float *q_dev, float *k_dev
 
 int twm_argmax_f32(twm_ctx *ctx, const float *input_dev, uint32_t rows, uint32_t cols, int32_t *out_dev)
 {
-    if (!ctx) return fail(TWM_INVALID_HANDLE, "twm_argmax_f32: null context");
+    if (!ctx) return api_fail(TWM_INVALID_HANDLE, "twm_argmax_f32: null context");
     if (rows == 0) return TWM_OK;
-    if (!out_dev || (cols != 0 && !input_dev)) return fail(TWM_INVALID_HANDLE, "twm_argmax_f32: null pointer");
+    if (!out_dev || (cols != 0 && !input_dev)) return api_fail(TWM_INVALID_HANDLE, "twm_argmax_f32: null pointer");
     HIP_TRY(launch_argmax(ctx->stream, input_dev, rows, cols, out_dev, ctx->ws, ctx->ws_bytes), TWM_DEVICE_ERROR, "argmax launch");
     return TWM_OK;
 }
@@ -447,9 +454,9 @@ int twm_argmax_f32(twm_ctx *ctx, const float *input_dev, uint32_t rows, uint32_t
 int twm_split_gate_up(twm_ctx *ctx, const float *gate_up_dev, float *gate_dev, float *up_dev, uint32_t ffn_dim,
                       uint32_t batch)
 {
-    if (!ctx) return fail(TWM_INVALID_HANDLE, "twm_split_gate_up: null context");
+    if (!ctx) return api_fail(TWM_INVALID_HANDLE, "twm_split_gate_up: null context");
     if ((uint64_t)batch * ffn_dim == 0) return TWM_OK;
-    if (!gate_up_dev || !gate_dev || !up_dev) return fail(TWM_INVALID_HANDLE, "twm_split_gate_up: null pointer");
+    if (!gate_up_dev || !gate_dev || !up_dev) return api_fail(TWM_INVALID_HANDLE, "twm_split_gate_up: null pointer");
     HIP_TRY(launch_split_gate_up(ctx->stream, gate_up_dev, gate_dev, up_dev, ffn_dim, batch), TWM_DEVICE_ERROR,
             "split_gate_up launch");
     return TWM_OK;
@@ -457,21 +464,21 @@ int twm_split_gate_up(twm_ctx *ctx, const float *gate_up_dev, float *gate_dev, f
 
 int twm_silu_mul(twm_ctx *ctx, const float *gate_dev, const float *up_dev, float *out_dev, size_t count)
 {
-    if (!ctx) return fail(TWM_INVALID_HANDLE, "twm_silu_mul: null context");
+    if (!ctx) return api_fail(TWM_INVALID_HANDLE, "twm_silu_mul: null context");
     if (count == 0) return TWM_OK;
-    if (!gate_dev || !up_dev || !out_dev) return fail(TWM_INVALID_HANDLE, "twm_silu_mul: null pointer");
+    if (!gate_dev || !up_dev || !out_dev) return api_fail(TWM_INVALID_HANDLE, "twm_silu_mul: null pointer");
     HIP_TRY(launch_silu_mul(ctx->stream, gate_dev, up_dev, out_dev, count), TWM_DEVICE_ERROR, "silu_mul launch");
     return TWM_OK;
 }
 
 int twm_swiglu_rows(twm_ctx *ctx, const float *gate_up_dev, uint32_t batch, uint32_t ffn_dim, int paired, float *out_dev)
 {
-    if (!ctx) return fail(TWM_INVALID_HANDLE, "twm_swiglu_rows: null context");
+    if (!ctx) return api_fail(TWM_INVALID_HANDLE, "twm_swiglu_rows: null context");
     if (paired && ffn_dim % kPairWidth != 0)
-        return fail(TWM_SHAPE_ERROR, "twm_swiglu_rows: the paired order needs ffn_dim %% %u == 0, got %u", kPairWidth, ffn_dim);
-    if ((uint64_t)ffn_dim * 2 > 0xFFFFFFFFull) return fail(TWM_SHAPE_ERROR, "twm_swiglu_rows: 2 * ffn_dim overflows u32");
+        return api_fail(TWM_SHAPE_ERROR, "twm_swiglu_rows: the paired order needs ffn_dim %% %u == 0, got %u", kPairWidth, ffn_dim);
+    if ((uint64_t)ffn_dim * 2 > 0xFFFFFFFFull) return api_fail(TWM_SHAPE_ERROR, "twm_swiglu_rows: 2 * ffn_dim overflows u32");
     if ((uint64_t)batch * ffn_dim == 0) return TWM_OK;
-    if (!gate_up_dev || !out_dev) return fail(TWM_INVALID_HANDLE, "twm_swiglu_rows: null pointer");
+    if (!gate_up_dev || !out_dev) return api_fail(TWM_INVALID_HANDLE, "twm_swiglu_rows: null pointer");
     HIP_TRY(launch_swiglu_rows(ctx->stream, gate_up_dev, out_dev, ffn_dim, batch, paired != 0), TWM_DEVICE_ERROR,
             "swiglu_rows launch");
     return TWM_OK;
@@ -479,8 +486,8 @@ int twm_swiglu_rows(twm_ctx *ctx, const float *gate_up_dev, uint32_t batch, uint
 
 static int check_pair_args(const char *who, uint32_t k, uint32_t ffn_dim)
 {
-    if (ffn_dim % kPairWidth != 0) return fail(TWM_SHAPE_ERROR, "%s: ffn_dim must be a multiple of %u, got %u", who, kPairWidth, ffn_dim);
-    if ((uint64_t)ffn_dim * 2 > 0xFFFFFFFFull) return fail(TWM_SHAPE_ERROR, "%s: 2 * ffn_dim overflows u32", who);
+    if (ffn_dim % kPairWidth != 0) return api_fail(TWM_SHAPE_ERROR, "%s: ffn_dim must be a multiple of %u, got %u", who, kPairWidth, ffn_dim);
+    if ((uint64_t)ffn_dim * 2 > 0xFFFFFFFFull) return api_fail(TWM_SHAPE_ERROR, "%s: 2 * ffn_dim overflows u32", who);
     return check_kn(who, k, ffn_dim * 2);
 }
 
@@ -488,11 +495,11 @@ int twm_pair_gate_up(twm_ctx *ctx, const uint8_t *gate_packed_dev, const uint16_
                      const uint8_t *up_packed_dev, const uint16_t *up_scales_dev, uint32_t k, uint32_t ffn_dim,
                      uint8_t *packed_out_dev, uint16_t *scales_out_dev)
 {
-    if (!ctx) return fail(TWM_INVALID_HANDLE, "twm_pair_gate_up: null context");
+    if (!ctx) return api_fail(TWM_INVALID_HANDLE, "twm_pair_gate_up: null context");
     if (int rc = check_pair_args("twm_pair_gate_up", k, ffn_dim)) return rc;
     if (k == 0 || ffn_dim == 0) return TWM_OK;
     if (!gate_packed_dev || !gate_scales_dev || !up_packed_dev || !up_scales_dev || !packed_out_dev || !scales_out_dev)
-        return fail(TWM_INVALID_HANDLE, "twm_pair_gate_up: null pointer");
+        return api_fail(TWM_INVALID_HANDLE, "twm_pair_gate_up: null pointer");
     HIP_TRY(launch_pair_gate_up(ctx->stream, gate_packed_dev, gate_scales_dev, up_packed_dev, up_scales_dev, k / 32,
                                 ffn_dim, packed_out_dev, scales_out_dev),
             TWM_DEVICE_ERROR, "pair_gate_up launch");
@@ -520,22 +527,24 @@ void twm_pick_splits_reference(uint32_t k, uint32_t n, uint32_t *n_blocks, uint3
     if (groups_per_split) *groups_per_split = (groups + sp - 1u) / sp;
 }
 
-int twm_gemm_tw_marlin_m1(twm_ctx *ctx, const float *a_dev, const uint8_t *packed_dev, const uint16_t *scales_dev,
-                          float *c_dev, uint32_t n, uint32_t k)
+extern "C++" int twm::m1_dispatch(const M1Env &env, const char *who, const float *a_dev, const uint8_t *packed_dev,
+                       const uint16_t *scales_dev, float *c_dev, uint32_t n, uint32_t k)
 {
-    if (!ctx) return fail(TWM_INVALID_HANDLE, "twm_gemm_tw_marlin_m1: null context");
-    if (int rc = check_kn("twm_gemm_tw_marlin_m1", k, n)) return rc;
+    if (int rc = check_kn(who, k, n)) return rc;
     if (n == 0) return TWM_OK;
-    if (!c_dev) return fail(TWM_INVALID_HANDLE, "twm_gemm_tw_marlin_m1: null output");
-    if (k == 0) return twm_memset_zero(ctx, c_dev, (size_t)n * 4);
-    if (!a_dev || !packed_dev || !scales_dev) return fail(TWM_INVALID_HANDLE, "twm_gemm_tw_marlin_m1: null input");
-    if (((uintptr_t)packed_dev & 15) != 0) return fail(TWM_SHAPE_ERROR, "twm_gemm_tw_marlin_m1: packed must be 16-byte aligned");
-    if (ctx->m1_exact || ((uintptr_t)a_dev & 15) != 0) {
+    if (!c_dev) return api_fail(TWM_INVALID_HANDLE, "%s: null output", who);
+    if (k == 0) {
+        HIP_TRY(launch_fill_zero(env.stream, c_dev, (size_t)n * 4), TWM_DEVICE_ERROR, "fill kernel launch");
+        return TWM_OK;
+    }
+    if (!a_dev || !packed_dev || !scales_dev) return api_fail(TWM_INVALID_HANDLE, "%s: null input", who);
+    // the reference kernel reads a record as four 32-bit words (quantize.rs:1227-1228): 4-byte alignment is its own limit
+    if (((uintptr_t)packed_dev & 3) != 0) return api_fail(TWM_SHAPE_ERROR, "%s: packed must be 4-byte aligned", who);
+    if (env.exact || ((uintptr_t)a_dev & 15) != 0 || ((uintptr_t)packed_dev & 15) != 0) {
         // f32 activations, f32 FMAs, the reference kernel's order and its own split-K rule (float atomics)
         uint32_t nb, sp, gps;
         twm_pick_splits_reference(k, n, &nb, &sp, &gps);
-        HIP_TRY(launch_ref_gemv(ctx->stream, a_dev, packed_dev, scales_dev, c_dev, n, k, sp, gps), TWM_DEVICE_ERROR,
-                "gemv launch");
+        HIP_TRY(launch_ref_gemv(env.stream, a_dev, packed_dev, scales_dev, c_dev, n, k, sp, gps), TWM_DEVICE_ERROR, "gemv launch");
         return TWM_OK;
     }
     // the M <= 4 MFMA kernels reading the reference's arrays as they are (f32 activations as two f16 terms)
@@ -548,19 +557,21 @@ int twm_gemm_tw_marlin_m1(twm_ctx *ctx, const float *a_dev, const uint8_t *packe
     // Qwen2.5-7B, Llama-3-8B, 13B and 70B projections; option "sub" = 1 keeps the 64-column kernel.
     const uint32_t tiles64 = n_pad / 64, passes16 = (k_chunks + 3) / 4, passes32 = (k_chunks + 1) / 2;
     uint32_t sub = tiles64 <= 64 ? 16 : 32, sub_waves = (sub == 16 && passes16 <= 8) ? 8 : 16;
-    bool use_sub = ctx->force_sub != 1 && (sub == 16 ? passes16 : passes32) <= 16;
-    if (ctx->force_sub >= 16) {
-        sub = (uint32_t)ctx->force_sub;
+    bool use_sub = env.force_sub != 1 && (sub == 16 ? passes16 : passes32) <= 16;
+    if (env.force_sub >= 16) {
+        sub = (uint32_t)env.force_sub;
         sub_waves = 8;
         use_sub = true;
     }
     if (use_sub) {
-        uint32_t sp = ctx->m1_splits ? (uint32_t)ctx->m1_splits : 1;
-        if (ctx->force_waves) sub_waves = (uint32_t)ctx->force_waves;
+        uint32_t sp = env.splits ? (uint32_t)env.splits : 1;
+        if (env.force_waves) sub_waves = (uint32_t)env.force_waves;
         if (sp > k_chunks) sp = k_chunks;
-        while (sp > 1 && (size_t)sp * n_pad * 4 > ctx->ws_bytes) sp--;
-        if (n_pad / sub > ctx->n_counters) sp = 1;
-        HIP_TRY(launch_gemv4s_ref(ctx->stream, packed_dev, scales_dev, k, n, a_dev, c_dev, ctx->ws, ctx->counters, sub, sub_waves, sp),
+        while (sp > 1 && (size_t)sp * n_pad * 4 > env.ws_bytes) sp--;
+        if (n_pad / sub > env.n_counters) sp = 1;
+        if (sp > 1 && env.clear_counters)
+            HIP_TRY(launch_fill_zero(env.stream, env.counters, (size_t)(n_pad / sub) * 4), TWM_DEVICE_ERROR, "fill kernel launch");
+        HIP_TRY(launch_gemv4s_ref(env.stream, packed_dev, scales_dev, k, n, a_dev, c_dev, env.ws, env.counters, sub, sub_waves, sp),
                 TWM_DEVICE_ERROR, "sub-tile gemv launch");
         return TWM_OK;
     }
@@ -573,15 +584,26 @@ int twm_gemm_tw_marlin_m1(twm_ctx *ctx, const float *a_dev, const uint8_t *packe
         plan.waves = 16;
         while (tiles64 * plan.splits * 2 <= 256 && k_chunks >= plan.splits * 2 * 8) plan.splits *= 2;
     }
-    if (ctx->force_waves) plan.waves = (uint32_t)ctx->force_waves;
-    if (ctx->m1_splits) plan.splits = (uint32_t)ctx->m1_splits;
+    if (env.force_waves) plan.waves = (uint32_t)env.force_waves;
+    if (env.splits) plan.splits = (uint32_t)env.splits;
     if (plan.splits > k_chunks) plan.splits = k_chunks;
-    while (plan.splits > 1 && (size_t)plan.splits * n_pad * 4 > ctx->ws_bytes) plan.splits--;
-    if (tiles64 > ctx->n_counters) plan.splits = 1;
-    HIP_TRY(launch_gemv4_ref(ctx->stream, packed_dev, scales_dev, k, n, a_dev, c_dev, ctx->ws, ctx->counters, plan.waves,
+    while (plan.splits > 1 && (size_t)plan.splits * n_pad * 4 > env.ws_bytes) plan.splits--;
+    if (tiles64 > env.n_counters) plan.splits = 1;
+    if (plan.splits > 1 && env.clear_counters)
+        HIP_TRY(launch_fill_zero(env.stream, env.counters, (size_t)tiles64 * 4), TWM_DEVICE_ERROR, "fill kernel launch");
+    HIP_TRY(launch_gemv4_ref(env.stream, packed_dev, scales_dev, k, n, a_dev, c_dev, env.ws, env.counters, plan.waves,
                              plan.splits),
             TWM_DEVICE_ERROR, "gemv launch");
     return TWM_OK;
+}
+
+int twm_gemm_tw_marlin_m1(twm_ctx *ctx, const float *a_dev, const uint8_t *packed_dev, const uint16_t *scales_dev,
+                          float *c_dev, uint32_t n, uint32_t k)
+{
+    if (!ctx) return api_fail(TWM_INVALID_HANDLE, "twm_gemm_tw_marlin_m1: null context");
+    const M1Env env = {ctx->stream, ctx->m1_exact, ctx->m1_splits, ctx->force_sub, ctx->force_waves,
+                       ctx->ws, ctx->ws_bytes, ctx->counters, ctx->n_counters, false};
+    return m1_dispatch(env, "twm_gemm_tw_marlin_m1", a_dev, packed_dev, scales_dev, c_dev, n, k);
 }
 
 int twm_gemm_tw_marlin_m1_from_buffer(twm_ctx *ctx, const float *a_dev, const uint8_t *packed_buf_dev,
@@ -589,7 +611,7 @@ int twm_gemm_tw_marlin_m1_from_buffer(twm_ctx *ctx, const float *a_dev, const ui
                                       float *c_dev, uint32_t n, uint32_t k)
 {
     if (!packed_buf_dev || !scales_buf_dev)
-        return fail(TWM_INVALID_HANDLE, "twm_gemm_tw_marlin_m1_from_buffer: null slab");
+        return api_fail(TWM_INVALID_HANDLE, "twm_gemm_tw_marlin_m1_from_buffer: null slab");
     return twm_gemm_tw_marlin_m1(ctx, a_dev, packed_buf_dev + packed_offset, scales_buf_dev + scales_offset, c_dev, n, k);
 }
 
@@ -598,7 +620,7 @@ int twm_gemm_tw_marlin_m1_from_buffer(twm_ctx *ctx, const float *a_dev, const ui
 static twm_weight *weight_alloc(twm_ctx *ctx, uint32_t k, uint32_t n)
 {
     twm_weight *w = new (std::nothrow) twm_weight();
-    if (!w) { fail(TWM_MEMORY_ERROR, "twm_weight: out of host memory"); return nullptr; }
+    if (!w) { api_fail(TWM_MEMORY_ERROR, "twm_weight: out of host memory"); return nullptr; }
     w->ctx = ctx;
     w->k = k;
     w->n = n;
@@ -617,7 +639,7 @@ static twm_weight *weight_alloc(twm_ctx *ctx, uint32_t k, uint32_t n)
     if (tiles == 0) return w;
     hipError_t e = hipMalloc(&w->qw, w->bytes);
     if (e != hipSuccess) {
-        fail(TWM_MEMORY_ERROR, "twm_weight: hipMalloc(%zu): %s", w->bytes, hipGetErrorString(e));
+        api_fail(TWM_MEMORY_ERROR, "twm_weight: hipMalloc(%zu): %s", w->bytes, hipGetErrorString(e));
         delete w;
         return nullptr;
     }
@@ -629,14 +651,14 @@ static twm_weight *weight_alloc(twm_ctx *ctx, uint32_t k, uint32_t n)
 twm_weight *twm_weight_from_device(twm_ctx *ctx, const uint8_t *packed_dev, const uint16_t *scales_dev, uint32_t k,
                                    uint32_t n)
 {
-    if (!ctx) { fail(TWM_INVALID_HANDLE, "twm_weight_from_device: null context"); return nullptr; }
-    if (ctx->capturing) { fail(TWM_UNSUPPORTED_OP, "twm_weight_from_device: not allowed inside a graph capture"); return nullptr; }
+    if (!ctx) { api_fail(TWM_INVALID_HANDLE, "twm_weight_from_device: null context"); return nullptr; }
+    if (ctx->capturing) { api_fail(TWM_UNSUPPORTED_OP, "twm_weight_from_device: not allowed inside a graph capture"); return nullptr; }
     if (check_kn("twm_weight_from_device", k, n)) return nullptr;
     if ((uint64_t)k * n != 0 && (!packed_dev || !scales_dev)) {
-        fail(TWM_INVALID_HANDLE, "twm_weight_from_device: null pointer");
+        api_fail(TWM_INVALID_HANDLE, "twm_weight_from_device: null pointer");
         return nullptr;
     }
-    if (((uintptr_t)packed_dev & 3) != 0) { fail(TWM_SHAPE_ERROR, "twm_weight_from_device: packed must be 4-byte aligned"); return nullptr; }
+    if (((uintptr_t)packed_dev & 3) != 0) { api_fail(TWM_SHAPE_ERROR, "twm_weight_from_device: packed must be 4-byte aligned"); return nullptr; }
     twm_weight *w = weight_alloc(ctx, k, n);
     if (!w) return nullptr;
     if (w->qw) {
@@ -645,7 +667,7 @@ twm_weight *twm_weight_from_device(twm_ctx *ctx, const uint8_t *packed_dev, cons
             e = launch_repack_col(ctx->stream, packed_dev, scales_dev, k, n, w->cq, w->n_tiles * kTileN, w->k_chunks);
         if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
         if (e != hipSuccess) {
-            fail(TWM_DEVICE_ERROR, "twm_weight_from_device: repack: %s", hipGetErrorString(e));
+            api_fail(TWM_DEVICE_ERROR, "twm_weight_from_device: repack: %s", hipGetErrorString(e));
             (void)hipFree(w->qw);
             delete w;
             return nullptr;
@@ -657,15 +679,15 @@ twm_weight *twm_weight_from_device(twm_ctx *ctx, const uint8_t *packed_dev, cons
 twm_weight *twm_weight_upload(twm_ctx *ctx, const uint8_t *packed_host, const uint16_t *scales_host, uint32_t k,
                               uint32_t n)
 {
-    if (!ctx) { fail(TWM_INVALID_HANDLE, "twm_weight_upload: null context"); return nullptr; }
-    if (ctx->capturing) { fail(TWM_UNSUPPORTED_OP, "twm_weight_upload: not allowed inside a graph capture"); return nullptr; }
+    if (!ctx) { api_fail(TWM_INVALID_HANDLE, "twm_weight_upload: null context"); return nullptr; }
+    if (ctx->capturing) { api_fail(TWM_UNSUPPORTED_OP, "twm_weight_upload: not allowed inside a graph capture"); return nullptr; }
     if (check_kn("twm_weight_upload", k, n)) return nullptr;
     size_t pbytes = (size_t)(k / 32) * n * 16, sbytes = (size_t)(k / 32) * n * 2;
     if (pbytes == 0) return twm_weight_from_device(ctx, nullptr, nullptr, k, n);
-    if (!packed_host || !scales_host) { fail(TWM_INVALID_HANDLE, "twm_weight_upload: null pointer"); return nullptr; }
+    if (!packed_host || !scales_host) { api_fail(TWM_INVALID_HANDLE, "twm_weight_upload: null pointer"); return nullptr; }
     void *stage = nullptr;
     hipError_t e = hipMalloc(&stage, pbytes + sbytes);
-    if (e != hipSuccess) { fail(TWM_MEMORY_ERROR, "twm_weight_upload: staging hipMalloc: %s", hipGetErrorString(e)); return nullptr; }
+    if (e != hipSuccess) { api_fail(TWM_MEMORY_ERROR, "twm_weight_upload: staging hipMalloc: %s", hipGetErrorString(e)); return nullptr; }
     uint8_t *p = (uint8_t *)stage;
     uint16_t *s = (uint16_t *)(p + pbytes);
     twm_weight *w = nullptr;
@@ -678,8 +700,8 @@ twm_weight *twm_weight_upload(twm_ctx *ctx, const uint8_t *packed_host, const ui
 twm_weight *twm_weight_gate_up(twm_ctx *ctx, const uint8_t *gate_packed_dev, const uint16_t *gate_scales_dev,
                                const uint8_t *up_packed_dev, const uint16_t *up_scales_dev, uint32_t k, uint32_t ffn_dim)
 {
-    if (!ctx) { fail(TWM_INVALID_HANDLE, "twm_weight_gate_up: null context"); return nullptr; }
-    if (ctx->capturing) { fail(TWM_UNSUPPORTED_OP, "twm_weight_gate_up: not allowed inside a graph capture"); return nullptr; }
+    if (!ctx) { api_fail(TWM_INVALID_HANDLE, "twm_weight_gate_up: null context"); return nullptr; }
+    if (ctx->capturing) { api_fail(TWM_UNSUPPORTED_OP, "twm_weight_gate_up: not allowed inside a graph capture"); return nullptr; }
     if (check_pair_args("twm_weight_gate_up", k, ffn_dim)) return nullptr;
     uint32_t n = ffn_dim * 2;
     size_t pbytes = (size_t)(k / 32) * n * 16, sbytes = (size_t)(k / 32) * n * 2;
@@ -689,7 +711,7 @@ twm_weight *twm_weight_gate_up(twm_ctx *ctx, const uint8_t *gate_packed_dev, con
     } else {
         void *stage = nullptr;
         hipError_t e = hipMalloc(&stage, pbytes + sbytes);
-        if (e != hipSuccess) { fail(TWM_MEMORY_ERROR, "twm_weight_gate_up: staging hipMalloc: %s", hipGetErrorString(e)); return nullptr; }
+        if (e != hipSuccess) { api_fail(TWM_MEMORY_ERROR, "twm_weight_gate_up: staging hipMalloc: %s", hipGetErrorString(e)); return nullptr; }
         uint8_t *p = (uint8_t *)stage;
         uint16_t *sc = (uint16_t *)(p + pbytes);
         if (twm_pair_gate_up(ctx, gate_packed_dev, gate_scales_dev, up_packed_dev, up_scales_dev, k, ffn_dim, p, sc) == TWM_OK)
@@ -716,7 +738,7 @@ void twm_weight_destroy(twm_weight *w)
 
 int twm_weight_dims(const twm_weight *w, uint32_t *k, uint32_t *n)
 {
-    if (!w) return fail(TWM_INVALID_HANDLE, "twm_weight_dims: null weight");
+    if (!w) return api_fail(TWM_INVALID_HANDLE, "twm_weight_dims: null weight");
     if (k) *k = w->k;
     if (n) *n = w->n;
     return TWM_OK;
@@ -764,12 +786,12 @@ size_t twm_weight_blob_bytes(const twm_weight *w) { return w ? sizeof(WeightBlob
 
 int twm_weight_export(twm_ctx *ctx, const twm_weight *w, void *blob_host, size_t blob_bytes)
 {
-    if (!ctx || !w) return fail(TWM_INVALID_HANDLE, "twm_weight_export: null handle");
-    if (w->ctx != ctx) return fail(TWM_INVALID_HANDLE, "twm_weight_export: weight belongs to another context");
-    if (ctx->capturing) return fail(TWM_UNSUPPORTED_OP, "twm_weight_export: not allowed inside a graph capture");
-    if (!blob_host) return fail(TWM_INVALID_HANDLE, "twm_weight_export: null buffer");
+    if (!ctx || !w) return api_fail(TWM_INVALID_HANDLE, "twm_weight_export: null handle");
+    if (w->ctx != ctx) return api_fail(TWM_INVALID_HANDLE, "twm_weight_export: weight belongs to another context");
+    if (ctx->capturing) return api_fail(TWM_UNSUPPORTED_OP, "twm_weight_export: not allowed inside a graph capture");
+    if (!blob_host) return api_fail(TWM_INVALID_HANDLE, "twm_weight_export: null buffer");
     if (blob_bytes != twm_weight_blob_bytes(w))
-        return fail(TWM_SHAPE_ERROR, "twm_weight_export: the buffer must hold %zu bytes, got %zu", twm_weight_blob_bytes(w), blob_bytes);
+        return api_fail(TWM_SHAPE_ERROR, "twm_weight_export: the buffer must hold %zu bytes, got %zu", twm_weight_blob_bytes(w), blob_bytes);
     uint8_t *payload = (uint8_t *)blob_host + sizeof(WeightBlobHeader);
     size_t payload_bytes = (w->qw != nullptr) ? w->bytes : 0;
     if (payload_bytes)
@@ -791,14 +813,14 @@ int twm_weight_export(twm_ctx *ctx, const twm_weight *w, void *blob_host, size_t
 
 twm_weight *twm_weight_import(twm_ctx *ctx, const void *blob_host, size_t blob_bytes)
 {
-    if (!ctx) { fail(TWM_INVALID_HANDLE, "twm_weight_import: null context"); return nullptr; }
-    if (ctx->capturing) { fail(TWM_UNSUPPORTED_OP, "twm_weight_import: not allowed inside a graph capture"); return nullptr; }
-    if (!blob_host || blob_bytes < sizeof(WeightBlobHeader)) { fail(TWM_SHAPE_ERROR, "twm_weight_import: blob shorter than its header"); return nullptr; }
+    if (!ctx) { api_fail(TWM_INVALID_HANDLE, "twm_weight_import: null context"); return nullptr; }
+    if (ctx->capturing) { api_fail(TWM_UNSUPPORTED_OP, "twm_weight_import: not allowed inside a graph capture"); return nullptr; }
+    if (!blob_host || blob_bytes < sizeof(WeightBlobHeader)) { api_fail(TWM_SHAPE_ERROR, "twm_weight_import: blob shorter than its header"); return nullptr; }
     WeightBlobHeader hd;
     memcpy(&hd, blob_host, sizeof hd);
-    if (memcmp(hd.magic, kBlobMagic, 8) != 0) { fail(TWM_SHAPE_ERROR, "twm_weight_import: not a repacked-weight blob (bad magic)"); return nullptr; }
+    if (memcmp(hd.magic, kBlobMagic, 8) != 0) { api_fail(TWM_SHAPE_ERROR, "twm_weight_import: not a repacked-weight blob (bad magic)"); return nullptr; }
     if (hd.layout != kBlobLayout) {
-        fail(TWM_UNSUPPORTED_OP, "twm_weight_import: blob has layout %u, this library writes %u: repack from the TW-Marlin arrays", hd.layout, kBlobLayout);
+        api_fail(TWM_UNSUPPORTED_OP, "twm_weight_import: blob has layout %u, this library writes %u: repack from the TW-Marlin arrays", hd.layout, kBlobLayout);
         return nullptr;
     }
     if (check_kn("twm_weight_import", hd.k, hd.n)) return nullptr;
@@ -808,11 +830,11 @@ twm_weight *twm_weight_import(twm_ctx *ctx, const void *blob_host, size_t blob_b
     bool ok = w->n_tiles == hd.n_tiles && w->k_chunks == hd.k_chunks && w->bytes == hd.payload_bytes &&
               blob_bytes == sizeof(WeightBlobHeader) + hd.payload_bytes && hd.paired <= 1 &&
               (!hd.paired || hd.n % (2 * kPairWidth) == 0);
-    if (!ok) fail(TWM_SHAPE_ERROR, "twm_weight_import: header does not describe a %u x %u weight of %zu bytes", hd.k, hd.n, blob_bytes);
+    if (!ok) api_fail(TWM_SHAPE_ERROR, "twm_weight_import: header does not describe a %u x %u weight of %zu bytes", hd.k, hd.n, blob_bytes);
     size_t payload_bytes = w->qw ? w->bytes : 0;
     if (ok && blob_checksum(payload, payload_bytes) != hd.checksum) {
         ok = false;
-        fail(TWM_SHAPE_ERROR, "twm_weight_import: checksum mismatch (corrupt or truncated blob)");
+        api_fail(TWM_SHAPE_ERROR, "twm_weight_import: checksum mismatch (corrupt or truncated blob)");
     }
     if (ok && payload_bytes) ok = twm_memcpy_h2d(ctx, w->qw, payload, payload_bytes) == TWM_OK;
     if (!ok) {
@@ -840,9 +862,9 @@ static WeightView view_of(const twm_weight *w)
 
 int twm_weight_dequant_f16(twm_ctx *ctx, const twm_weight *w, uint16_t *out_kn_dev)
 {
-    if (!ctx || !w) return fail(TWM_INVALID_HANDLE, "twm_weight_dequant_f16: null handle");
+    if (!ctx || !w) return api_fail(TWM_INVALID_HANDLE, "twm_weight_dequant_f16: null handle");
     if ((uint64_t)w->k * w->n == 0) return TWM_OK;
-    if (!out_kn_dev) return fail(TWM_INVALID_HANDLE, "twm_weight_dequant_f16: null output");
+    if (!out_kn_dev) return api_fail(TWM_INVALID_HANDLE, "twm_weight_dequant_f16: null output");
     // "dequant_src" = 1 reads the column-lane copy instead of the 16-column tile order
     if (ctx->dequant_src == 1)
         HIP_TRY(launch_weight_dequant_f16_col(ctx->stream, view_of(w), out_kn_dev), TWM_DEVICE_ERROR, "dequant launch");
@@ -1063,7 +1085,7 @@ uint32_t twm_pick_splits(uint32_t k, uint32_t n, uint32_t m)
 static int gemm_common(twm_ctx *ctx, const twm_weight *w, const void *a_dev, int a_dtype, uint32_t m, const OutSpec &out,
                        uint32_t splits, const char *who, float *swiglu_out = nullptr, uint32_t gate_act = 2)
 {
-    if (a_dtype != TWM_F16 && a_dtype != TWM_F32) return fail(TWM_UNSUPPORTED_OP, "%s: activations must be f16 or f32", who);
+    if (a_dtype != TWM_F16 && a_dtype != TWM_F32) return api_fail(TWM_UNSUPPORTED_OP, "%s: activations must be f16 or f32", who);
     if (m == 0 || w->n == 0) return TWM_OK;
     if (w->k == 0) {
         for (uint32_t s = 0; s < out.count; s++) {
@@ -1078,8 +1100,8 @@ static int gemm_common(twm_ctx *ctx, const twm_weight *w, const void *a_dev, int
         }
         return TWM_OK;
     }
-    if (!a_dev) return fail(TWM_INVALID_HANDLE, "%s: null activations", who);
-    if (((uintptr_t)a_dev & 15) != 0) return fail(TWM_SHAPE_ERROR, "%s: activations must be 16-byte aligned", who);
+    if (!a_dev) return api_fail(TWM_INVALID_HANDLE, "%s: null activations", who);
+    if (((uintptr_t)a_dev & 15) != 0) return api_fail(TWM_SHAPE_ERROR, "%s: activations must be 16-byte aligned", who);
     WeightView v = view_of(w);
     size_t a_row_bytes = (size_t)w->k * (a_dtype == TWM_F16 ? 2 : 4);
     uint32_t n_ld = w->n_tiles * kTileN;
@@ -1123,8 +1145,9 @@ static int gemm_common(twm_ctx *ctx, const twm_weight *w, const void *a_dev, int
                             (m > 16 || (!splits && ((m > 8 && (n_ld / 64 > 128 || rows_f32)) ||
                                                     (rows_f32 && m > 4 && w->k_chunks <= 64))));
     if (ctx->force_kernel == 4 || batch_auto) {
-        // batched decode with the activations shared through LDS, in 32-row blocks: from 17 rows on (there it runs the
-        // reference's M > 1 arithmetic on f16-rounded weights, like the prefill kernel), and from 9 rows on wide
+        // batched decode with the activations shared through LDS, in 32-row blocks: from 17 rows on (the same exact
+        // arithmetic as below 17 rows; option "batch_rounded" runs the f16-rounded weights of the prefill kernel
+        // there), and from 9 rows on wide
         // matrices (3584 -> 37888: M = 16 19.8 against 22.8 us of the streaming kernel, M = 32 26.7 against
         // 33.3; 18944 -> 3584 at M = 32 17.3 against 21.8; at M = 9 .. 16 on narrow matrices the two are within 3 %
         // with f16 rows).  f32 rows, which the streaming kernel holds twice in registers: from 9 rows on everywhere
@@ -1139,9 +1162,10 @@ static int gemm_common(twm_ctx *ctx, const twm_weight *w, const void *a_dev, int
             // forced: "nt" 2 = two tiles per wave, 4 = two quads per workgroup, 3 = three; "waves" 8 / 16 = 2 / 4 k-slices
             BatchPlan bp = {splits ? splits : 1, ctx->force_waves == 8 ? 2u : ctx->force_waves == 16 ? 4u : 1u,
                             ctx->force_nt == 2 ? 2u : 1u, ctx->force_nt == 4 ? 2u : ctx->force_nt == 3 ? 3u : 1u};
-            if (batch_auto) bp = plan_batch(w->n_tiles, w->k_chunks, m > 16 ? 32 : mb, rows_f32, splits);
+            const bool rounded = ctx->batch_rounded && m > 16;
+            if (batch_auto) bp = plan_batch(w->n_tiles, w->k_chunks, rounded ? 32 : mb, rows_f32, splits);
             HIP_TRY(launch_batch(ctx->stream, v, a_blk, a_dtype == TWM_F32, mb, o, bp.splits, bp.tiles_per_wave, bp.slices,
-                                 bp.quads_per_group, m > 16, ctx->ws, ctx->ws_bytes),
+                                 bp.quads_per_group, rounded, ctx->ws, ctx->ws_bytes),
                     TWM_DEVICE_ERROR, "batched decode launch");
         }
         return TWM_OK;
@@ -1164,8 +1188,8 @@ static int gemm_common(twm_ctx *ctx, const twm_weight *w, const void *a_dev, int
         uint32_t mb = m - m0 < (uint32_t)kMaxDecodeM ? m - m0 : (uint32_t)kMaxDecodeM;
         DecodePlan plan;
         bool lane_col = mb <= 4 && ctx->force_kernel != 1;
-        if (swiglu_out && !lane_col) return fail(TWM_UNSUPPORTED_OP, "%s: the 16-column tile kernel has no gated store", who);
-        if (ctx->force_kernel == 2 && !lane_col) return fail(TWM_UNSUPPORTED_OP, "%s: the one-lane-per-column kernel takes M <= 4", who);
+        if (swiglu_out && !lane_col) return api_fail(TWM_UNSUPPORTED_OP, "%s: the 16-column tile kernel has no gated store", who);
+        if (ctx->force_kernel == 2 && !lane_col) return api_fail(TWM_UNSUPPORTED_OP, "%s: the one-lane-per-column kernel takes M <= 4", who);
         if (lane_col) plan = plan_gemv4(w->n_tiles, w->k_chunks, ctx->force_nt, ctx->force_waves, splits);
         else plan = plan_decode(w->n_tiles, w->k_chunks, mb, ctx->force_nt, ctx->force_waves == 1 || ctx->force_waves == 2 ? 0 : ctx->force_waves, splits);
         // the scratch must hold splits x mb x n_ld partials and one counter per tile group
@@ -1206,9 +1230,9 @@ static int gemm_common(twm_ctx *ctx, const twm_weight *w, const void *a_dev, int
 
 int twm_gemm(twm_ctx *ctx, const twm_weight *w, const void *a_dev, int a_dtype, uint32_t m, float *c_dev, uint32_t splits)
 {
-    if (!ctx || !w) return fail(TWM_INVALID_HANDLE, "twm_gemm: null handle");
-    if (w->ctx != ctx) return fail(TWM_INVALID_HANDLE, "twm_gemm: weight belongs to another context");
-    if (m != 0 && w->n != 0 && !c_dev) return fail(TWM_INVALID_HANDLE, "twm_gemm: null output");
+    if (!ctx || !w) return api_fail(TWM_INVALID_HANDLE, "twm_gemm: null handle");
+    if (w->ctx != ctx) return api_fail(TWM_INVALID_HANDLE, "twm_gemm: weight belongs to another context");
+    if (m != 0 && w->n != 0 && !c_dev) return api_fail(TWM_INVALID_HANDLE, "twm_gemm: null output");
     OutSpec out;
     memset(&out, 0, sizeof out);
     out.count = 1;
@@ -1222,18 +1246,18 @@ int twm_gemm_split_bias(twm_ctx *ctx, const twm_weight *w, const void *a_dev, in
                         float *const *outs_dev, const float *const *biases_dev, const uint32_t *ns, uint32_t count,
                         uint32_t splits)
 {
-    if (!ctx || !w) return fail(TWM_INVALID_HANDLE, "twm_gemm_split_bias: null handle");
-    if (w->ctx != ctx) return fail(TWM_INVALID_HANDLE, "twm_gemm_split_bias: weight belongs to another context");
-    if (!outs_dev || !ns) return fail(TWM_INVALID_HANDLE, "twm_gemm_split_bias: null array");
+    if (!ctx || !w) return api_fail(TWM_INVALID_HANDLE, "twm_gemm_split_bias: null handle");
+    if (w->ctx != ctx) return api_fail(TWM_INVALID_HANDLE, "twm_gemm_split_bias: weight belongs to another context");
+    if (!outs_dev || !ns) return api_fail(TWM_INVALID_HANDLE, "twm_gemm_split_bias: null array");
     if (count == 0 || count > (uint32_t)kMaxSegs)
-        return fail(TWM_SHAPE_ERROR, "twm_gemm_split_bias: between 1 and %d outputs are supported", kMaxSegs);
+        return api_fail(TWM_SHAPE_ERROR, "twm_gemm_split_bias: between 1 and %d outputs are supported", kMaxSegs);
     OutSpec out;
     memset(&out, 0, sizeof out);
     uint64_t total = 0;
     uint32_t used = 0;
     for (uint32_t i = 0; i < count; i++) {
         if (ns[i] == 0) continue;
-        if (m != 0 && !outs_dev[i]) return fail(TWM_INVALID_HANDLE, "twm_gemm_split_bias: null output %u", i);
+        if (m != 0 && !outs_dev[i]) return api_fail(TWM_INVALID_HANDLE, "twm_gemm_split_bias: null output %u", i);
         out.seg[used].ptr = outs_dev[i];
         out.seg[used].start = (uint32_t)total;
         out.seg[used].width = ns[i];
@@ -1242,7 +1266,7 @@ int twm_gemm_split_bias(twm_ctx *ctx, const twm_weight *w, const void *a_dev, in
         total += ns[i];
     }
     out.count = used;
-    if (total != w->n) return fail(TWM_SHAPE_ERROR, "twm_gemm_split_bias: outputs cover %llu columns, weight has %u",
+    if (total != w->n) return api_fail(TWM_SHAPE_ERROR, "twm_gemm_split_bias: outputs cover %llu columns, weight has %u",
                                    (unsigned long long)total, w->n);
     return gemm_common(ctx, w, a_dev, a_dtype, m, out, splits, "twm_gemm_split_bias");
 }
@@ -1256,13 +1280,13 @@ int twm_gemm_split(twm_ctx *ctx, const twm_weight *w, const void *a_dev, int a_d
 static int gemm_gated(twm_ctx *ctx, const twm_weight *w, const void *a_dev, int a_dtype, uint32_t m, float *out_dev,
                       uint32_t splits, uint32_t act, const char *who)
 {
-    if (!ctx || !w) return fail(TWM_INVALID_HANDLE, "%s: null handle", who);
-    if (w->ctx != ctx) return fail(TWM_INVALID_HANDLE, "%s: weight belongs to another context", who);
-    if (!w->paired) return fail(TWM_UNSUPPORTED_OP, "%s: the weight was not built by twm_weight_gate_up", who);
+    if (!ctx || !w) return api_fail(TWM_INVALID_HANDLE, "%s: null handle", who);
+    if (w->ctx != ctx) return api_fail(TWM_INVALID_HANDLE, "%s: weight belongs to another context", who);
+    if (!w->paired) return api_fail(TWM_UNSUPPORTED_OP, "%s: the weight was not built by twm_weight_gate_up", who);
     uint32_t ffn = w->n / 2;
     if (m == 0 || ffn == 0) return TWM_OK;
-    if (!out_dev) return fail(TWM_INVALID_HANDLE, "%s: null output", who);
-    if (((uintptr_t)out_dev & 15) != 0) return fail(TWM_SHAPE_ERROR, "%s: the output must be 16-byte aligned", who);
+    if (!out_dev) return api_fail(TWM_INVALID_HANDLE, "%s: null output", who);
+    if (((uintptr_t)out_dev & 15) != 0) return api_fail(TWM_SHAPE_ERROR, "%s: the output must be 16-byte aligned", who);
     if (w->k == 0) return twm_memset_zero(ctx, out_dev, (size_t)m * ffn * 4);  // gate(0) * 0
     OutSpec out;
     memset(&out, 0, sizeof out);
@@ -1287,24 +1311,24 @@ twm_bank *twm_bank_from_device(twm_ctx *ctx, const uint8_t *packed_base_dev, con
                                size_t packed_bytes_per_expert, size_t scales_per_expert, uint32_t k, uint32_t n,
                                uint32_t num_experts, int pair_gate_up)
 {
-    if (!ctx) { fail(TWM_INVALID_HANDLE, "twm_bank_from_device: null context"); return nullptr; }
-    if (ctx->capturing) { fail(TWM_UNSUPPORTED_OP, "twm_bank_from_device: not allowed inside a graph capture"); return nullptr; }
+    if (!ctx) { api_fail(TWM_INVALID_HANDLE, "twm_bank_from_device: null context"); return nullptr; }
+    if (ctx->capturing) { api_fail(TWM_UNSUPPORTED_OP, "twm_bank_from_device: not allowed inside a graph capture"); return nullptr; }
     if (check_kn("twm_bank_from_device", k, n)) return nullptr;
     if (pair_gate_up && n % (2 * kPairWidth) != 0) {
-        fail(TWM_SHAPE_ERROR, "twm_bank_from_device: a paired gate/up bank needs N %% %u == 0, got %u", 2 * kPairWidth, n);
+        api_fail(TWM_SHAPE_ERROR, "twm_bank_from_device: a paired gate/up bank needs N %% %u == 0, got %u", 2 * kPairWidth, n);
         return nullptr;
     }
     size_t groups = k / 32;
     if (packed_bytes_per_expert < groups * n * 16 || scales_per_expert < groups * n || packed_bytes_per_expert % 4 != 0) {
-        fail(TWM_SHAPE_ERROR, "twm_bank_from_device: per-expert strides (%zu bytes, %zu scales) do not hold a %u x %u matrix",
+        api_fail(TWM_SHAPE_ERROR, "twm_bank_from_device: per-expert strides (%zu bytes, %zu scales) do not hold a %u x %u matrix",
              packed_bytes_per_expert, scales_per_expert, k, n);
         return nullptr;
     }
     bool empty = (uint64_t)k * n * num_experts == 0;
-    if (!empty && (!packed_base_dev || !scales_base_dev)) { fail(TWM_INVALID_HANDLE, "twm_bank_from_device: null pointer"); return nullptr; }
-    if (((uintptr_t)packed_base_dev & 3) != 0) { fail(TWM_SHAPE_ERROR, "twm_bank_from_device: packed must be 4-byte aligned"); return nullptr; }
+    if (!empty && (!packed_base_dev || !scales_base_dev)) { api_fail(TWM_INVALID_HANDLE, "twm_bank_from_device: null pointer"); return nullptr; }
+    if (((uintptr_t)packed_base_dev & 3) != 0) { api_fail(TWM_SHAPE_ERROR, "twm_bank_from_device: packed must be 4-byte aligned"); return nullptr; }
     twm_bank *b = new (std::nothrow) twm_bank();
-    if (!b) { fail(TWM_MEMORY_ERROR, "twm_bank: out of host memory"); return nullptr; }
+    if (!b) { api_fail(TWM_MEMORY_ERROR, "twm_bank: out of host memory"); return nullptr; }
     b->ctx = ctx;
     b->k = k;
     b->n = n;
@@ -1318,7 +1342,7 @@ twm_bank *twm_bank_from_device(twm_ctx *ctx, const uint8_t *packed_base_dev, con
     if (empty || b->bytes == 0) return b;
     hipError_t e = hipMalloc(&b->cq, b->bytes);
     if (e != hipSuccess) {
-        fail(TWM_MEMORY_ERROR, "twm_bank: hipMalloc(%zu): %s", b->bytes, hipGetErrorString(e));
+        api_fail(TWM_MEMORY_ERROR, "twm_bank: hipMalloc(%zu): %s", b->bytes, hipGetErrorString(e));
         delete b;
         return nullptr;
     }
@@ -1328,7 +1352,7 @@ twm_bank *twm_bank_from_device(twm_ctx *ctx, const uint8_t *packed_base_dev, con
                               b->n_pad, b->k_chunks, pair_gate_up ? n / 2 : 0);
     if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
     if (e != hipSuccess) {
-        fail(TWM_DEVICE_ERROR, "twm_bank_from_device: repack: %s", hipGetErrorString(e));
+        api_fail(TWM_DEVICE_ERROR, "twm_bank_from_device: repack: %s", hipGetErrorString(e));
         (void)hipFree(b->cq);
         delete b;
         return nullptr;
@@ -1363,12 +1387,12 @@ static BankView bank_view(const twm_bank *b)
 
 static int bank_common_checks(const char *who, twm_ctx *ctx, const twm_bank *b, const void *a_dev, int a_dtype)
 {
-    if (!ctx || !b) return fail(TWM_INVALID_HANDLE, "%s: null handle", who);
-    if (b->ctx != ctx) return fail(TWM_INVALID_HANDLE, "%s: bank belongs to another context", who);
-    if (a_dtype != TWM_F16 && a_dtype != TWM_F32) return fail(TWM_UNSUPPORTED_OP, "%s: activations must be f16 or f32", who);
+    if (!ctx || !b) return api_fail(TWM_INVALID_HANDLE, "%s: null handle", who);
+    if (b->ctx != ctx) return api_fail(TWM_INVALID_HANDLE, "%s: bank belongs to another context", who);
+    if (a_dtype != TWM_F16 && a_dtype != TWM_F32) return api_fail(TWM_UNSUPPORTED_OP, "%s: activations must be f16 or f32", who);
     if (b->k != 0 && b->n != 0) {
-        if (!a_dev) return fail(TWM_INVALID_HANDLE, "%s: null activations", who);
-        if (((uintptr_t)a_dev & 15) != 0) return fail(TWM_SHAPE_ERROR, "%s: activations must be 16-byte aligned", who);
+        if (!a_dev) return api_fail(TWM_INVALID_HANDLE, "%s: null activations", who);
+        if (((uintptr_t)a_dev & 15) != 0) return api_fail(TWM_SHAPE_ERROR, "%s: activations must be 16-byte aligned", who);
     }
     return TWM_OK;
 }
@@ -1377,16 +1401,16 @@ int twm_bank_gemv(twm_ctx *ctx, const twm_bank *b, const void *a_dev, int a_dtyp
                   const float *topk_ids_dev, uint32_t top_k, int act, float *out_dev)
 {
     if (int rc = bank_common_checks("twm_bank_gemv", ctx, b, a_dev, a_dtype)) return rc;
-    if (act < 0 || act > 2) return fail(TWM_UNSUPPORTED_OP, "twm_bank_gemv: act must be 0 (none), 1 (GEGLU) or 2 (SwiGLU)");
-    if (act != 0 && !b->paired) return fail(TWM_UNSUPPORTED_OP, "twm_bank_gemv: a fused gate needs a bank built with pair_gate_up");
+    if (act < 0 || act > 2) return api_fail(TWM_UNSUPPORTED_OP, "twm_bank_gemv: act must be 0 (none), 1 (GEGLU) or 2 (SwiGLU)");
+    if (act != 0 && !b->paired) return api_fail(TWM_UNSUPPORTED_OP, "twm_bank_gemv: a fused gate needs a bank built with pair_gate_up");
     if (top_k == 0 || b->n == 0) return TWM_OK;
-    if (top_k > 65535u) return fail(TWM_SHAPE_ERROR, "twm_bank_gemv: at most 65535 slots per call");
-    if (!topk_ids_dev || !out_dev) return fail(TWM_INVALID_HANDLE, "twm_bank_gemv: null pointer");
+    if (top_k > 65535u) return api_fail(TWM_SHAPE_ERROR, "twm_bank_gemv: at most 65535 slots per call");
+    if (!topk_ids_dev || !out_dev) return api_fail(TWM_INVALID_HANDLE, "twm_bank_gemv: null pointer");
     uint32_t width = act ? b->n / 2 : b->n;
     if (b->k == 0 || b->experts == 0) return twm_memset_zero(ctx, out_dev, (size_t)top_k * width * 4);  // gate(0) * 0 = 0
     // every slot's row must keep the 16-byte alignment of the loads
     if ((a_slot_stride * (a_dtype == TWM_F32 ? 4u : 2u)) % 16u != 0)
-        return fail(TWM_SHAPE_ERROR, "twm_bank_gemv: the activation stride must keep rows 16-byte aligned");
+        return api_fail(TWM_SHAPE_ERROR, "twm_bank_gemv: the activation stride must keep rows 16-byte aligned");
     HIP_TRY(launch_bank_gemv(ctx->stream, bank_view(b), a_dev, a_dtype == TWM_F32, a_slot_stride, topk_ids_dev, top_k, act, out_dev,
                              ctx->force_sub, ctx->force_waves),
             TWM_DEVICE_ERROR, "bank gemv launch");
@@ -1398,10 +1422,10 @@ int twm_bank_down_axpy(twm_ctx *ctx, const twm_bank *b, const void *a_all_dev, i
 {
     if (int rc = bank_common_checks("twm_bank_down_axpy", ctx, b, a_all_dev, a_dtype)) return rc;
     if (top_k == 0 || b->n == 0 || b->k == 0 || b->experts == 0) return TWM_OK;  // nothing is added
-    if (top_k > (uint32_t)kMaxBankSlots) return fail(TWM_SHAPE_ERROR, "twm_bank_down_axpy: at most %d slots per call, got %u", kMaxBankSlots, top_k);
-    if (!topk_ids_dev || !topk_weights_dev || !acc_dev) return fail(TWM_INVALID_HANDLE, "twm_bank_down_axpy: null pointer");
+    if (top_k > (uint32_t)kMaxBankSlots) return api_fail(TWM_SHAPE_ERROR, "twm_bank_down_axpy: at most %d slots per call, got %u", kMaxBankSlots, top_k);
+    if (!topk_ids_dev || !topk_weights_dev || !acc_dev) return api_fail(TWM_INVALID_HANDLE, "twm_bank_down_axpy: null pointer");
     if ((b->k * (a_dtype == TWM_F32 ? 4u : 2u)) % 16u != 0)
-        return fail(TWM_SHAPE_ERROR, "twm_bank_down_axpy: K must keep the activation rows 16-byte aligned");
+        return api_fail(TWM_SHAPE_ERROR, "twm_bank_down_axpy: K must keep the activation rows 16-byte aligned");
     HIP_TRY(launch_bank_down_axpy(ctx->stream, bank_view(b), a_all_dev, a_dtype == TWM_F32, topk_ids_dev, topk_weights_dev, top_k, acc_dev,
                                   ctx->force_sub, ctx->force_waves),
             TWM_DEVICE_ERROR, "bank down_axpy launch");
@@ -1410,12 +1434,12 @@ int twm_bank_down_axpy(twm_ctx *ctx, const twm_bank *b, const void *a_all_dev, i
 
 int twm_geglu_rows(twm_ctx *ctx, const float *gate_up_dev, uint32_t batch, uint32_t dim, int paired, float *out_dev)
 {
-    if (!ctx) return fail(TWM_INVALID_HANDLE, "twm_geglu_rows: null context");
+    if (!ctx) return api_fail(TWM_INVALID_HANDLE, "twm_geglu_rows: null context");
     if (paired && dim % kPairWidth != 0)
-        return fail(TWM_SHAPE_ERROR, "twm_geglu_rows: the paired order needs dim %% %u == 0, got %u", kPairWidth, dim);
-    if ((uint64_t)dim * 2 > 0xFFFFFFFFull) return fail(TWM_SHAPE_ERROR, "twm_geglu_rows: 2 * dim overflows u32");
+        return api_fail(TWM_SHAPE_ERROR, "twm_geglu_rows: the paired order needs dim %% %u == 0, got %u", kPairWidth, dim);
+    if ((uint64_t)dim * 2 > 0xFFFFFFFFull) return api_fail(TWM_SHAPE_ERROR, "twm_geglu_rows: 2 * dim overflows u32");
     if ((uint64_t)batch * dim == 0) return TWM_OK;
-    if (!gate_up_dev || !out_dev) return fail(TWM_INVALID_HANDLE, "twm_geglu_rows: null pointer");
+    if (!gate_up_dev || !out_dev) return api_fail(TWM_INVALID_HANDLE, "twm_geglu_rows: null pointer");
     HIP_TRY(launch_geglu_rows(ctx->stream, gate_up_dev, out_dev, dim, batch, paired != 0), TWM_DEVICE_ERROR, "geglu_rows launch");
     return TWM_OK;
 }
@@ -1424,9 +1448,9 @@ int twm_geglu_rows(twm_ctx *ctx, const float *gate_up_dev, uint32_t batch, uint3
 
 int twm_graph_begin(twm_ctx *ctx)
 {
-    if (!ctx) return fail(TWM_INVALID_HANDLE, "twm_graph_begin: null context");
-    if (ctx->capturing) return fail(TWM_UNSUPPORTED_OP, "twm_graph_begin: a capture is already open");
-    if (ctx->stream == nullptr) return fail(TWM_UNSUPPORTED_OP, "twm_graph_begin: cannot capture the null stream");
+    if (!ctx) return api_fail(TWM_INVALID_HANDLE, "twm_graph_begin: null context");
+    if (ctx->capturing) return api_fail(TWM_UNSUPPORTED_OP, "twm_graph_begin: a capture is already open");
+    if (ctx->stream == nullptr) return api_fail(TWM_UNSUPPORTED_OP, "twm_graph_begin: cannot capture the null stream");
     HIP_TRY(hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeRelaxed), TWM_DEVICE_ERROR, "hipStreamBeginCapture");
     ctx->capturing = true;
     return TWM_OK;
@@ -1434,25 +1458,25 @@ int twm_graph_begin(twm_ctx *ctx)
 
 twm_graph *twm_graph_end(twm_ctx *ctx)
 {
-    if (!ctx) { fail(TWM_INVALID_HANDLE, "twm_graph_end: null context"); return nullptr; }
-    if (!ctx->capturing) { fail(TWM_UNSUPPORTED_OP, "twm_graph_end: no capture is open"); return nullptr; }
+    if (!ctx) { api_fail(TWM_INVALID_HANDLE, "twm_graph_end: null context"); return nullptr; }
+    if (!ctx->capturing) { api_fail(TWM_UNSUPPORTED_OP, "twm_graph_end: no capture is open"); return nullptr; }
     ctx->capturing = false;
     hipGraph_t graph = nullptr;
     hipError_t e = hipStreamEndCapture(ctx->stream, &graph);
     if (e != hipSuccess || !graph) {
-        fail(TWM_DEVICE_ERROR, "hipStreamEndCapture: %s", hipGetErrorString(e));
+        api_fail(TWM_DEVICE_ERROR, "hipStreamEndCapture: %s", hipGetErrorString(e));
         return nullptr;
     }
     hipGraphExec_t exec = nullptr;
     e = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
     if (e != hipSuccess) {
-        fail(TWM_DEVICE_ERROR, "hipGraphInstantiate: %s", hipGetErrorString(e));
+        api_fail(TWM_DEVICE_ERROR, "hipGraphInstantiate: %s", hipGetErrorString(e));
         (void)hipGraphDestroy(graph);
         return nullptr;
     }
     twm_graph *g = new (std::nothrow) twm_graph();
     if (!g) {
-        fail(TWM_MEMORY_ERROR, "twm_graph_end: out of host memory");
+        api_fail(TWM_MEMORY_ERROR, "twm_graph_end: out of host memory");
         (void)hipGraphExecDestroy(exec);
         (void)hipGraphDestroy(graph);
         return nullptr;
@@ -1464,8 +1488,8 @@ twm_graph *twm_graph_end(twm_ctx *ctx)
 
 int twm_graph_launch(twm_ctx *ctx, twm_graph *g)
 {
-    if (!ctx || !g) return fail(TWM_INVALID_HANDLE, "twm_graph_launch: null handle");
-    if (ctx->capturing) return fail(TWM_UNSUPPORTED_OP, "twm_graph_launch: a capture is open");
+    if (!ctx || !g) return api_fail(TWM_INVALID_HANDLE, "twm_graph_launch: null handle");
+    if (ctx->capturing) return api_fail(TWM_UNSUPPORTED_OP, "twm_graph_launch: a capture is open");
     HIP_TRY(hipGraphLaunch(g->exec, ctx->stream), TWM_DEVICE_ERROR, "hipGraphLaunch");
     return TWM_OK;
 }

@@ -5,10 +5,11 @@
 // has the meaning of gemm_q4_0, quantize.rs:1825-1858): per 32-deep group the products a * (q - 8) are summed in f32
 // by one v_mfma_f32_16x16x32_f16 with a zero accumulator ((q - 8) and the f16 activations are exact operands), the
 // group sum is scaled once by f32(scale) and added to the running f32 sum, groups in ascending order.
-// 17 .. 32 rows: the reference's own M > 1 arithmetic, Q4 unpack to FP16 then FP16 GEMM with f32 accumulation
-// (quantize.rs:534-571, :1825-1858), as the prefill kernel: the B operand is f16_rne(f32(scale) * (q - 8)), made by one
-// packed f16 multiply, and the MFMAs accumulate over K directly (f32 activations still as two f16 terms): with two
-// row blocks the exact form costs eight f32 multiply-adds per tile and group after the MFMAs.
+// 17 .. 32 rows: the same arithmetic on two 16-row blocks (eight f32 multiply-adds per tile and group after the
+// MFMAs), so that a row's result does not depend on how many rows are batched with it.
+// Option (RND): the reference's dequant-then-FP16-GEMM arithmetic (quantize.rs:534-571, :1825-1858), as the prefill
+// kernel: the B operand is f16_rne(f32(scale) * (q - 8)), made by one packed f16 multiply, and the MFMAs accumulate
+// over K directly (f32 activations still as two f16 terms).
 //
 // Why a second kernel: the streaming kernel keeps a whole chunk of activations (32 rows x 128 k) per wave in
 // registers, twice, so only two waves fit a SIMD and each has one chunk of weights in flight; at 32 rows it is
@@ -81,13 +82,13 @@ constexpr int kBtRow = 128;  // halves per LDS row (256 bytes)
 // memory requests in flight.  The first 4 MT waves of a slice stage the tile (four rows each, or MT times four with
 // WPS = 4); the others issue the same load on one 16-byte address and write a spare LDS row, which keeps every
 // wave's count of loads in flight the same.
-template <int MT, int TERMS, int TPW, int KS, int WPS>
+template <int MT, bool RND, int TERMS, int TPW, int KS, int WPS>
 __global__ __launch_bounds__(64 * WPS * KS) void k_batch(const uint4v *__restrict__ qw, const uint2v *__restrict__ sc,
                                                 const void *__restrict__ a_any, OutSpec out, float *__restrict__ partials,
                                                 uint32_t m_rows, uint32_t k, uint32_t n, uint32_t n_tiles,
                                                 uint32_t k_chunks, uint32_t chunks_per_split, uint32_t lo_offset)
 {
-    constexpr bool kRounded = MT == 2;       // 17 .. 32 rows: weights rounded to f16 as in the reference's M > 1 route
+    constexpr bool kRounded = RND;           // weights rounded to f16 as in the reference's dequant-then-FP16-GEMM route (option)
     constexpr int S = 4;                     // register slots: chunk kc lives in slot kc % S, three chunks are in flight
     constexpr int kTile = 16 * MT * kBtRow;  // halves of one term's tile
     constexpr int kBuf = TERMS * kTile;      // halves of one LDS buffer
@@ -337,7 +338,7 @@ __global__ __launch_bounds__(64 * WPS * KS) void k_batch(const uint4v *__restric
     }
 }
 
-template <int MT, int TERMS, int TPW, int KS, int WPS = 4>
+template <int MT, bool RND, int TERMS, int TPW, int KS, int WPS = 4>
 static hipError_t launch_batch_t(hipStream_t s, const WeightView &w, const void *a, uint32_t m, const OutSpec &out,
                                  uint32_t splits, float *partials, uint32_t lo_offset)
 {
@@ -346,7 +347,7 @@ static hipError_t launch_batch_t(hipStream_t s, const WeightView &w, const void 
     const uint32_t quads = w.n_tiles / 4;   // n_tiles is a multiple of 4
     constexpr uint32_t kQuadsPerGroup = WPS * TPW / 4;
     dim3 grid((quads + kQuadsPerGroup - 1) / kQuadsPerGroup, splits);
-    hipLaunchKernelGGL((k_batch<MT, TERMS, TPW, KS, WPS>), grid, dim3(64 * WPS * KS), 0, s, (const uint4v *)w.qw, (const uint2v *)w.sc, a, out,
+    hipLaunchKernelGGL((k_batch<MT, RND, TERMS, TPW, KS, WPS>), grid, dim3(64 * WPS * KS), 0, s, (const uint4v *)w.qw, (const uint2v *)w.sc, a, out,
                        splits > 1 ? partials : nullptr, m, w.k, w.n, w.n_tiles, w.k_chunks, cps, lo_offset);
     if (splits > 1) {
         hipError_t e = launch_splitk_reduce(s, partials, out, m, w.n, w.n_tiles * 16, splits);
@@ -357,36 +358,37 @@ static hipError_t launch_batch_t(hipStream_t s, const WeightView &w, const void 
 
 // Four k-slices (sixteen waves) only with one tile per wave (register file) and not for the 32-row two-term variant
 // (its staging buffers would need 128 KB of LDS); otherwise two.
-template <int MT, int TERMS, int TPW>
+template <int MT, bool RND, int TERMS, int TPW>
 static hipError_t launch_batch_slices(hipStream_t s, const WeightView &w, const void *a, uint32_t m, const OutSpec &out,
                                       uint32_t splits, uint32_t k_slices, uint32_t quads_per_group, float *partials,
                                       uint32_t lo_offset)
 {
     if constexpr (TPW == 1) {
         // two or three quads per workgroup (eight or twelve waves per slice; two slices only with eight)
-        if (quads_per_group == 3) return launch_batch_t<MT, TERMS, 1, 1, 12>(s, w, a, m, out, splits, partials, lo_offset);
+        if (quads_per_group == 3) return launch_batch_t<MT, RND, TERMS, 1, 1, 12>(s, w, a, m, out, splits, partials, lo_offset);
         if (quads_per_group == 2) {
             if constexpr (!(MT == 2 && TERMS == 2)) {
-                if (k_slices >= 2) return launch_batch_t<MT, TERMS, 1, 2, 8>(s, w, a, m, out, splits, partials, lo_offset);
+                if (k_slices >= 2) return launch_batch_t<MT, RND, TERMS, 1, 2, 8>(s, w, a, m, out, splits, partials, lo_offset);
             }
-            return launch_batch_t<MT, TERMS, 1, 1, 8>(s, w, a, m, out, splits, partials, lo_offset);
+            return launch_batch_t<MT, RND, TERMS, 1, 1, 8>(s, w, a, m, out, splits, partials, lo_offset);
         }
     }
     if constexpr (TPW == 1 && !(MT == 2 && TERMS == 2)) {
-        if (k_slices == 4) return launch_batch_t<MT, TERMS, TPW, 4>(s, w, a, m, out, splits, partials, lo_offset);
+        if (k_slices == 4) return launch_batch_t<MT, RND, TERMS, TPW, 4>(s, w, a, m, out, splits, partials, lo_offset);
     }
-    if (k_slices >= 2) return launch_batch_t<MT, TERMS, TPW, 2>(s, w, a, m, out, splits, partials, lo_offset);
-    return launch_batch_t<MT, TERMS, TPW, 1>(s, w, a, m, out, splits, partials, lo_offset);
+    if (k_slices >= 2) return launch_batch_t<MT, RND, TERMS, TPW, 2>(s, w, a, m, out, splits, partials, lo_offset);
+    return launch_batch_t<MT, RND, TERMS, TPW, 1>(s, w, a, m, out, splits, partials, lo_offset);
 }
 
 // M <= 32.  quads_per_group: 1, 2 or 3 column quads per workgroup sharing one activation tile (one tile per wave; with
-// two tiles per wave the workgroup owns two quads anyway).  two_row_blocks: take the 32-row variant (f16-rounded weights) also for 16 rows or fewer -- the last rows
-// of a larger M, so that one call runs one arithmetic.  tiles_per_wave: 1 or 2 (a gated store without split-K needs 2).  `scratch` holds, for f32 activations,
+// two tiles per wave the workgroup owns two quads anyway).  rounded: weights rounded to f16 and accumulated over K by
+// the MFMAs (always on the 32-row variant, so that one call runs one arithmetic whatever its last block's height);
+// otherwise the exact per-group f32 scaling.  tiles_per_wave: 1 or 2 (a gated store without split-K needs 2).  `scratch` holds, for f32 activations,
 // their two f16 terms (2 x M x K halves) and after them the split-K partials (splits x M x (n_tiles * 16) floats);
 // the split factor is cut to what fits.
 hipError_t launch_batch(hipStream_t s, const WeightView &w, const void *a, bool a_f32, uint32_t m, const OutSpec &out,
                         uint32_t splits, uint32_t tiles_per_wave, uint32_t k_slices, uint32_t quads_per_group,
-                        bool two_row_blocks, float *scratch, size_t scratch_bytes)
+                        bool rounded, float *scratch, size_t scratch_bytes)
 {
     if (m == 0 || w.n == 0) return hipSuccess;
     if (m > 32 || w.k_chunks == 0 || w.n_tiles % 4 != 0) return hipErrorInvalidValue;
@@ -414,15 +416,20 @@ hipError_t launch_batch(hipStream_t s, const WeightView &w, const void *a, bool 
     if (splits < 1) splits = 1;
     if (w.k_chunks < splits) splits = w.k_chunks;
     if (out.swiglu && splits == 1) tiles_per_wave = 2;
-#define TWM_BATCH_CASE(MT, T, P) return launch_batch_slices<MT, T, P>(s, w, a, m, out, splits, k_slices, quads_per_group, partials, lo_offset)
-    if (m <= 16 && !two_row_blocks) {
-        if (tiles_per_wave == 2) { if (a_f32) TWM_BATCH_CASE(1, 2, 2); TWM_BATCH_CASE(1, 1, 2); }
-        if (a_f32) TWM_BATCH_CASE(1, 2, 1);
-        TWM_BATCH_CASE(1, 1, 1);
+#define TWM_BATCH_CASE(MT, R, T, P) return launch_batch_slices<MT, R, T, P>(s, w, a, m, out, splits, k_slices, quads_per_group, partials, lo_offset)
+    if (rounded) {
+        if (tiles_per_wave == 2) { if (a_f32) TWM_BATCH_CASE(2, true, 2, 2); TWM_BATCH_CASE(2, true, 1, 2); }
+        if (a_f32) TWM_BATCH_CASE(2, true, 2, 1);
+        TWM_BATCH_CASE(2, true, 1, 1);
     }
-    if (tiles_per_wave == 2) { if (a_f32) TWM_BATCH_CASE(2, 2, 2); TWM_BATCH_CASE(2, 1, 2); }
-    if (a_f32) TWM_BATCH_CASE(2, 2, 1);
-    TWM_BATCH_CASE(2, 1, 1);
+    if (m <= 16) {
+        if (tiles_per_wave == 2) { if (a_f32) TWM_BATCH_CASE(1, false, 2, 2); TWM_BATCH_CASE(1, false, 1, 2); }
+        if (a_f32) TWM_BATCH_CASE(1, false, 2, 1);
+        TWM_BATCH_CASE(1, false, 1, 1);
+    }
+    if (tiles_per_wave == 2) { if (a_f32) TWM_BATCH_CASE(2, false, 2, 2); TWM_BATCH_CASE(2, false, 1, 2); }
+    if (a_f32) TWM_BATCH_CASE(2, false, 2, 1);
+    TWM_BATCH_CASE(2, false, 1, 1);
 #undef TWM_BATCH_CASE
 }
 

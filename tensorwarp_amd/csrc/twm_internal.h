@@ -69,6 +69,25 @@ struct DecodePlan {
     uint32_t lane_col;  // 1: M <= 4 kernel, one lane per column (nt = 64-column tiles per workgroup)
 };
 
+// ---- host-side helpers shared by the files that hold C-ABI entry points ---------------
+// records the message for twm_last_error() on the calling thread and returns `code`
+int api_fail(int code, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
+// K % 32 == 0 and K x N within the ABI's limit, else TWM_SHAPE_ERROR with the message set
+int check_kn(const char *who, uint32_t k, uint32_t n);
+// What the dispatch of the GEMV on the reference's arrays needs from its caller: the stream, the knobs, and the
+// split-K scratch (f32 partial sums and one arrival counter per column tile, zero between launches).
+struct M1Env {
+    hipStream_t stream;
+    int exact, splits, force_sub, force_waves;
+    float *ws;
+    size_t ws_bytes;
+    unsigned *counters;
+    uint32_t n_counters;
+    bool clear_counters;  // zero the counters a split launch uses first (a scratch shared with unknown earlier calls)
+};
+int m1_dispatch(const M1Env &env, const char *who, const float *a_dev, const uint8_t *packed_dev,
+                const uint16_t *scales_dev, float *c_dev, uint32_t n, uint32_t k);
+
 // ---- launchers (all asynchronous on `s`, return the launch status) ---------------
 hipError_t launch_fill_zero(hipStream_t s, void *ptr, size_t bytes);
 hipError_t launch_quantize_q4_0(hipStream_t s, const float *w_kn, uint32_t k, uint32_t n, uint8_t *q4);
@@ -124,7 +143,7 @@ hipError_t launch_split_hi_lo(hipStream_t s, const float *a, _Float16 *hi, _Floa
 // batched decode with the activations shared through LDS (M <= 32); tiles_per_wave 1 or 2, k_slices 1, 2 or 4
 hipError_t launch_batch(hipStream_t s, const WeightView &w, const void *a, bool a_f32, uint32_t m, const OutSpec &out,
                         uint32_t splits, uint32_t tiles_per_wave, uint32_t k_slices, uint32_t quads_per_group,
-                        bool two_row_blocks, float *scratch, size_t scratch_bytes);
+                        bool rounded, float *scratch, size_t scratch_bytes);
 hipError_t launch_geglu_rows(hipStream_t s, const float *gu, float *out, uint32_t dim, uint32_t batch, bool paired);
 // act: 0 out[slot][n]; 1 gelu_tanh(gate) * up, 2 silu(gate) * up into out[slot][n/2] (paired bank)
 hipError_t launch_bank_gemv(hipStream_t s, const BankView &b, const void *a, bool a_f32, uint32_t a_slot_stride,

@@ -494,9 +494,11 @@ hipError_t launch_pair_gate_up(hipStream_t s, const uint8_t *gate_packed, const 
 // One lane per output column: a wave reads 64 x 16 B = 1 KiB contiguous per group.
 // The activation index is wave-uniform, so A comes in through scalar loads.
 // ---------------------------------------------------------------------------------
-template <bool ATOMIC>
+// ALIGN16: the records are 16-byte aligned (one 128-bit load); otherwise four 32-bit loads, the alignment the
+// reference's own kernel needs (quantize.rs:1227-1228).
+template <bool ATOMIC, bool ALIGN16>
 __global__ __launch_bounds__(256) void k_ref_gemv(float *__restrict__ c, const float *__restrict__ a,
-                                                   const uint4v *__restrict__ packed,
+                                                   const uint32_t *__restrict__ packed,
                                                    const uint16_t *__restrict__ scales, uint32_t n, uint32_t groups,
                                                    uint32_t gps)
 {
@@ -507,7 +509,10 @@ __global__ __launch_bounds__(256) void k_ref_gemv(float *__restrict__ c, const f
     float dot = 0.0f;
     for (uint32_t g = g0; g < g1; g++) {
         float s = f16_bits_to_f32(scales[(size_t)g * n + col]);
-        uint4v v = packed[(size_t)g * n + col];
+        const uint32_t *rec = packed + ((size_t)g * n + col) * 4u;
+        uint4v v;
+        if (ALIGN16) v = *(const uint4v *)rec;
+        else v = uint4v{rec[0], rec[1], rec[2], rec[3]};
         const float *ab = a + g * 32;
         float gdot = 0.0f;
 #pragma unroll
@@ -530,15 +535,21 @@ hipError_t launch_ref_gemv(hipStream_t s, const float *a, const uint8_t *packed,
 {
     if (n == 0) return hipSuccess;
     dim3 grid((n + 255) / 256, splits);
+    const bool align16 = ((uintptr_t)packed & 15) == 0;
     if (splits > 1) {
         hipError_t e = launch_fill_zero(s, c, (size_t)n * 4);
         if (e != hipSuccess) return e;
-        hipLaunchKernelGGL(k_ref_gemv<true>, grid, dim3(256), 0, s, c, a, (const uint4v *)packed, scales, n, k / 32,
-                           groups_per_split);
-    } else {
-        hipLaunchKernelGGL(k_ref_gemv<false>, grid, dim3(256), 0, s, c, a, (const uint4v *)packed, scales, n, k / 32,
-                           groups_per_split);
     }
+#define TWM_REF_GEMV(AT, AL) \
+    hipLaunchKernelGGL((k_ref_gemv<AT, AL>), grid, dim3(256), 0, s, c, a, (const uint32_t *)packed, scales, n, k / 32, groups_per_split)
+    if (splits > 1) {
+        if (align16) TWM_REF_GEMV(true, true);
+        else TWM_REF_GEMV(true, false);
+    } else {
+        if (align16) TWM_REF_GEMV(false, true);
+        else TWM_REF_GEMV(false, false);
+    }
+#undef TWM_REF_GEMV
     return hipGetLastError();
 }
 
