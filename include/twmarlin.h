@@ -197,6 +197,16 @@ int twm_gemm_tw_marlin_m1(twm_ctx *ctx, const float *a_dev, const uint8_t *packe
 int twm_gemm_tw_marlin_m1_from_buffer(twm_ctx *ctx, const float *a_dev, const uint8_t *packed_buf_dev,
                                       size_t packed_offset, const uint16_t *scales_buf_dev,
                                       size_t scales_offset, float *c_dev, uint32_t n, uint32_t k);
+/* twm_gemm_tw_marlin_m1 for callers that cannot allocate: code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc.  No counterpart in the reference.  It takes no context: work is issued on
+ * hip_stream (a hipStream_t, NULL = the null stream) of the current device, with the library's default plan, and
+ * the split-K scratch is a static device array inside the library (64 KiB of partial sums + 256 counters per GPU,
+ * held until the process ends).  The call itself allocates and frees nothing and never synchronises.  Results are
+ * bit-identical to twm_gemm_tw_marlin_m1 with default options.  Limits: N <= 2^20 and K <= 2^20, beyond which
+ * TWM_SHAPE_ERROR is returned; alignment rules as twm_gemm_tw_marlin_m1.  All calls on one GPU share that GPU's
+ * array: two calls that overlap in time on one GPU (two streams, two threads) race; calls on one stream do not. */
+int twm_gemm_tw_marlin_m1_noalloc(void *hip_stream, const float *a_dev, const uint8_t *packed_dev,
+                                  const uint16_t *scales_dev, float *c_dev, uint32_t n, uint32_t k);
 /* The reference's adaptive split-K rule, bit for bit (quantize.rs:1314-1325). */
 void twm_pick_splits_reference(uint32_t k, uint32_t n, uint32_t *n_blocks, uint32_t *splits,
                                uint32_t *groups_per_split);

@@ -130,6 +130,7 @@ twm_ctx *twm_ctx_create(int ordinal)
     }
     ok = ok && hipStreamCreateWithFlags(&c->own_stream, hipStreamNonBlocking) == hipSuccess;
     ok = ok && init_prefill() == hipSuccess;
+    ok = ok && noalloc_scratch_for_current_device("twm_ctx_create") != nullptr;
     c->stream = c->own_stream;
     c->ws_bytes = kWsBytes;
     c->n_counters = kCounters;

@@ -88,6 +88,10 @@ struct M1Env {
 int m1_dispatch(const M1Env &env, const char *who, const float *a_dev, const uint8_t *packed_dev,
                 const uint16_t *scales_dev, float *c_dev, uint32_t n, uint32_t k);
 
+// twm_noalloc.hip: device address of the no-allocation entry point's static scratch on the current device (looked
+// up once per device; twm_ctx_create calls it so that the lookup has happened before any capture); nullptr on failure
+void *noalloc_scratch_for_current_device(const char *who);
+
 // ---- launchers (all asynchronous on `s`, return the launch status) ---------------
 hipError_t launch_fill_zero(hipStream_t s, void *ptr, size_t bytes);
 hipError_t launch_quantize_q4_0(hipStream_t s, const float *w_kn, uint32_t k, uint32_t n, uint8_t *q4);
