@@ -15,6 +15,7 @@
 using namespace twm;
 
 static thread_local std::string g_err;
+twm::TraceBuf twm::g_trace = {nullptr, 0};
 
 int twm::api_fail(int code, const char *fmt, ...)
 {
@@ -39,11 +40,15 @@ struct twm_ctx {
     hipStream_t stream;
     float *ws;            // split-K partial tiles
     size_t ws_bytes;
+    float *sk_ws;         // parked partial tiles of the stream-K prefill GEMM
+    size_t sk_ws_bytes;
+    int prefill_sk;       // stream-K prefill: 0 = the planner's choice, 1 = off, 128 / 256 = on with that block height
     unsigned *counters;   // one arrival counter per tile group, zero between launches
     uint32_t n_counters;
     bool capturing;
     int force_nt;         // 0 = heuristic
     int force_waves;      // 0 = heuristic
+    int force_sub_waves;  // sub-tile kernels with a forced width: waves per workgroup (1 .. 16), 0 = "waves" or eight
     int force_sub;        // M <= 4: 0 = heuristic, 1 = whole 64-column tiles per workgroup, 32 or 16 = the sub-tile kernel
     int force_kernel;     // 0 = heuristic, 1 = 16-column tile kernel, 2 = one-lane-per-column kernel (M <= 4), 3 = streaming kernel (M <= 32),
                           // 4 = batched-decode kernel with LDS-shared activations (M <= 32; "nt" = tiles per wave, "waves" 8 / 16 = 2 / 4 k-slices)
@@ -111,6 +116,7 @@ twm_ctx *twm_ctx_create(int ordinal)
     c->force_nt = 0;
     c->force_waves = 0;
     c->force_sub = 0;
+    c->force_sub_waves = 0;
     c->force_kernel = 0;
     c->dequant_src = 0;
     c->m1_exact = 0;
@@ -119,6 +125,9 @@ twm_ctx *twm_ctx_create(int ordinal)
     c->prefill_bm = 0;
     c->prefill_min_m = 33;  // M <= 32 is batched decode (exact f32 scales, weights streamed once)
     c->ws = nullptr;
+    c->sk_ws = nullptr;
+    c->sk_ws_bytes = 0;
+    c->prefill_sk = 0;
     c->counters = nullptr;
     c->own_stream = nullptr;
     bool ok = hipSetDevice(ordinal) == hipSuccess && hipGetDeviceProperties(&c->prop, ordinal) == hipSuccess;
@@ -129,18 +138,23 @@ twm_ctx *twm_ctx_create(int ordinal)
         return nullptr;
     }
     ok = ok && hipStreamCreateWithFlags(&c->own_stream, hipStreamNonBlocking) == hipSuccess;
-    ok = ok && init_prefill() == hipSuccess;
+    ok = ok && init_prefill() == hipSuccess && init_prefill_sk() == hipSuccess;
     ok = ok && noalloc_scratch_for_current_device("twm_ctx_create") != nullptr;
     c->stream = c->own_stream;
     c->ws_bytes = kWsBytes;
     c->n_counters = kCounters;
     ok = ok && hipMalloc((void **)&c->ws, c->ws_bytes) == hipSuccess;
     ok = ok && hipMalloc((void **)&c->counters, c->n_counters * sizeof(unsigned)) == hipSuccess;
+    if (ok) {  // two 256-row partial tiles per CU
+        c->sk_ws_bytes = prefill_sk_scratch_bytes(256, (uint32_t)c->prop.multiProcessorCount);
+        ok = hipMalloc((void **)&c->sk_ws, c->sk_ws_bytes) == hipSuccess;
+    }
     ok = ok && hipMemset(c->counters, 0, c->n_counters * sizeof(unsigned)) == hipSuccess;
     ok = ok && hipDeviceSynchronize() == hipSuccess;
     if (!ok) {
         api_fail(TWM_DEVICE_ERROR, "twm_ctx_create: %s", hipGetErrorString(hipGetLastError()));
         if (c->ws) (void)hipFree(c->ws);
+        if (c->sk_ws) (void)hipFree(c->sk_ws);
         if (c->counters) (void)hipFree(c->counters);
         if (c->own_stream) (void)hipStreamDestroy(c->own_stream);
         delete c;
@@ -155,6 +169,7 @@ void twm_ctx_destroy(twm_ctx *ctx)
     (void)hipSetDevice(ctx->ordinal);
     (void)hipStreamSynchronize(ctx->stream);
     (void)hipFree(ctx->ws);
+    (void)hipFree(ctx->sk_ws);
     (void)hipFree(ctx->counters);
     (void)hipStreamDestroy(ctx->own_stream);
     delete ctx;
@@ -164,6 +179,15 @@ int twm_ctx_sync(twm_ctx *ctx)
 {
     if (!ctx) return api_fail(TWM_INVALID_HANDLE, "twm_ctx_sync: null context");
     HIP_TRY(hipStreamSynchronize(ctx->stream), TWM_DEVICE_ERROR, "stream synchronize");
+    return TWM_OK;
+}
+
+int twm_debug_trace(twm_ctx *ctx, uint32_t *trace_dev, uint32_t capacity_workgroups)
+{
+    if (!ctx) return api_fail(TWM_INVALID_HANDLE, "twm_debug_trace: null context");
+    if (ctx->capturing) return api_fail(TWM_UNSUPPORTED_OP, "twm_debug_trace: a graph capture is open");
+    g_trace.ptr = capacity_workgroups ? trace_dev : nullptr;
+    g_trace.capacity = trace_dev ? capacity_workgroups : 0;
     return TWM_OK;
 }
 
@@ -204,6 +228,11 @@ int twm_ctx_set_option(twm_ctx *ctx, const char *key, int value)
         ctx->force_waves = value;
         return TWM_OK;
     }
+    if (strcmp(key, "sub_waves") == 0) {
+        if (value < 0 || value > 16) return api_fail(TWM_SHAPE_ERROR, "twm_ctx_set_option: sub_waves must be 0 .. 16");
+        ctx->force_sub_waves = value;
+        return TWM_OK;
+    }
     if (strcmp(key, "sub") == 0) {
         if (value != 0 && value != 1 && value != 16 && value != 32)
             return api_fail(TWM_SHAPE_ERROR, "twm_ctx_set_option: sub must be 0, 1, 16 or 32");
@@ -213,6 +242,12 @@ int twm_ctx_set_option(twm_ctx *ctx, const char *key, int value)
     if (strcmp(key, "prefill_bm") == 0) {
         if (value != 0 && value != 64 && value != 128) return api_fail(TWM_SHAPE_ERROR, "twm_ctx_set_option: prefill_bm must be 0, 64 or 128");
         ctx->prefill_bm = value;
+        return TWM_OK;
+    }
+    if (strcmp(key, "prefill_sk") == 0) {
+        if (value != 0 && value != 1 && value != 128 && value != 256)
+            return api_fail(TWM_SHAPE_ERROR, "twm_ctx_set_option: prefill_sk must be 0, 1, 128 or 256");
+        ctx->prefill_sk = value;
         return TWM_OK;
     }
     if (strcmp(key, "prefill_min_m") == 0) {
@@ -1111,13 +1146,16 @@ static int gemm_common(twm_ctx *ctx, const twm_weight *w, const void *a_dev, int
     gated.swiglu = swiglu_out;
     gated.gate_act = gate_act;
     if (m >= (uint32_t)ctx->prefill_min_m) {
-        HIP_TRY(launch_prefill(ctx->stream, v, a_dev, a_dtype == TWM_F32, m, gated, (uint32_t)ctx->prefill_bm, splits, ctx->ws, ctx->ws_bytes), TWM_DEVICE_ERROR, "prefill launch");
+        const PrefillSk sk = {ctx->sk_ws, ctx->sk_ws_bytes, ctx->counters, ctx->n_counters, (uint32_t)ctx->prop.multiProcessorCount,
+                              ctx->prefill_sk};
+        HIP_TRY(launch_prefill(ctx->stream, v, a_dev, a_dtype == TWM_F32, m, gated, (uint32_t)ctx->prefill_bm, splits, ctx->ws, ctx->ws_bytes, &sk),
+                TWM_DEVICE_ERROR, "prefill launch");
         return TWM_OK;
     }
     if (ctx->force_kernel == 0 && m > 4 && m <= 16 && a_dtype == TWM_F16 && ctx->force_sub != 1) {
         // M = 5 .. 16 on narrow matrices: the lane-per-column sub-tile kernel with two to four row groups
         SubPlan sub = {0, 0};
-        if (ctx->force_sub >= 16) sub = SubPlan{(uint32_t)ctx->force_sub, ctx->force_waves ? (uint32_t)ctx->force_waves : 8};
+        if (ctx->force_sub >= 16) sub = SubPlan{(uint32_t)ctx->force_sub, ctx->force_sub_waves ? (uint32_t)ctx->force_sub_waves : ctx->force_waves ? (uint32_t)ctx->force_waves : 8};
         else if (!ctx->force_nt && !ctx->force_waves && !splits) sub = plan_gemv4_sub_rows(n_ld / 64, w->k_chunks);
         if (sub.sub) {
             uint32_t ssp = splits ? splits : 1;
@@ -1202,7 +1240,7 @@ static int gemm_common(twm_ctx *ctx, const twm_weight *w, const void *a_dev, int
         SubPlan sub = {0, 0};
         if (lane_col && ctx->force_sub >= 16) {
             sub.sub = (uint32_t)ctx->force_sub;
-            sub.waves = ctx->force_waves ? (uint32_t)ctx->force_waves : 8;
+            sub.waves = ctx->force_sub_waves ? (uint32_t)ctx->force_sub_waves : ctx->force_waves ? (uint32_t)ctx->force_waves : 8;
         } else if (lane_col && ctx->force_sub == 0 && !ctx->force_nt && !ctx->force_waves && !splits) {
             // (an explicit nt, waves or split factor asks for the 64-column kernel's plan)
             sub = plan_gemv4_sub(n_ld / 64, w->k_chunks, mb, a_dtype == TWM_F32);

@@ -40,12 +40,12 @@ __device__ __forceinline__ void gemv4s_store_out(const OutSpec &out, uint32_t m,
 // take the passes (64 / SUB chunks each) of the k-range in turn.
 // REFL: cw is the reference's packed array u8 [G][N][16] and ref_scales its f16 [G][N] (no repack; one row of f32
 // activations): a sub-tile's records of one group are still SUB * 16 contiguous bytes.
-template <int SUB, int RL, bool AF32, bool ONE, bool REFL = false>
-__global__ __launch_bounds__(1024) void k_gemv4s(const char *__restrict__ cw, const void *__restrict__ a_any, OutSpec out,
-                                                  float *__restrict__ ws, unsigned *__restrict__ counters, uint32_t m_rows,
-                                                  uint32_t k, uint32_t n, uint32_t n_pad, uint32_t k_chunks,
-                                                  uint32_t sub_tiles, uint32_t splits, uint32_t cps,
-                                                  const uint16_t *__restrict__ ref_scales = nullptr)
+template <int SUB, int RL, bool AF32, bool ONE, bool REFL>
+__device__ __forceinline__ void gemv4s_body(const char *__restrict__ cw, const void *__restrict__ a_any, const OutSpec &out,
+                                            float *__restrict__ ws, unsigned *__restrict__ counters, uint32_t m_rows,
+                                            uint32_t k, uint32_t n, uint32_t n_pad, uint32_t k_chunks,
+                                            uint32_t sub_tiles, uint32_t splits, uint32_t cps,
+                                            const uint16_t *__restrict__ ref_scales, uint32_t *trace_loaded)
 {
     static_assert(!REFL || (AF32 && RL == 1), "the reference-layout variant is the M = 1, f32-activation entry point");
     constexpr int CPP = 64 / SUB;     // chunks per pass
@@ -119,6 +119,7 @@ __global__ __launch_bounds__(1024) void k_gemv4s(const char *__restrict__ cw, co
     auto compute_pass = [&](const ChunkS<SUB, RG> &r) { gemv4s_compute<SUB, RL, TERMS>(r, dq, acc); };
     // (ONE: the launcher saw that no wave has a second pass: one register set, no loop)
     gemv4s_run_passes<SUB, ONE, RG>(wave, waves, passes, load_pass, compute_pass);
+    if (trace_loaded && threadIdx.x == 0) *trace_loaded = (uint32_t)__builtin_amdgcn_s_memrealtime();  // data arrived and unpacked
 
     // ---- sum over the waves and over the chunks of a pass (lane groups) through LDS ----
 #pragma unroll
@@ -186,6 +187,28 @@ __global__ __launch_bounds__(1024) void k_gemv4s(const char *__restrict__ cw, co
     if (threadIdx.x == 0) __hip_atomic_store(&counters[st], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
+// trace (a profiling aid, nullptr in normal use): workgroup b writes four words at trace[4 b]: the 100 MHz clock
+// at its start, after wave 0 has unpacked its pass, and at its end, and the hardware id of the CU it ran on.
+template <int SUB, int RL, bool AF32, bool ONE, bool REFL = false>
+__global__ __launch_bounds__(1024) void k_gemv4s(const char *__restrict__ cw, const void *__restrict__ a_any, OutSpec out,
+                                                  float *__restrict__ ws, unsigned *__restrict__ counters, uint32_t m_rows,
+                                                  uint32_t k, uint32_t n, uint32_t n_pad, uint32_t k_chunks,
+                                                  uint32_t sub_tiles, uint32_t splits, uint32_t cps,
+                                                  const uint16_t *__restrict__ ref_scales = nullptr,
+                                                  uint32_t *__restrict__ trace = nullptr)
+{
+    uint32_t *tr = trace ? trace + 4u * blockIdx.x : nullptr;
+    if (tr && threadIdx.x == 0) {
+        tr[0] = (uint32_t)__builtin_amdgcn_s_memrealtime();
+        tr[1] = 0u;
+        // HW_ID (register 4): wave, SIMD, CU, SH, SE ids; XCC_ID (register 20): the XCD
+        tr[3] = (__builtin_amdgcn_s_getreg((31 << 11) | 4) & 0xFFFFu) | (__builtin_amdgcn_s_getreg((3 << 11) | 20) << 16);
+    }
+    gemv4s_body<SUB, RL, AF32, ONE, REFL>(cw, a_any, out, ws, counters, m_rows, k, n, n_pad, k_chunks, sub_tiles, splits, cps,
+                                          ref_scales, tr ? tr + 1 : nullptr);
+    if (tr && threadIdx.x == 0) tr[2] = (uint32_t)__builtin_amdgcn_s_memrealtime();
+}
+
 template <int SUB, int RL>
 static hipError_t launch_gemv4s_t(hipStream_t s, const WeightView &w, const void *a, bool a_f32, uint32_t m,
                                   const OutSpec &out, float *ws, unsigned *counters, uint32_t waves, uint32_t splits)
@@ -199,7 +222,8 @@ static hipError_t launch_gemv4s_t(hipStream_t s, const WeightView &w, const void
     const bool one = (cps + 64 / SUB - 1) / (64 / SUB) <= waves;
 #define TWM_S_LAUNCH(AF, ONEV)                                                                                          \
     hipLaunchKernelGGL((k_gemv4s<SUB, RL, AF, ONEV>), dim3(blocks), dim3(waves * 64), lds, s, (const char *)w.cq, a, out, \
-                       ws, counters, m, w.k, w.n, n_pad, w.k_chunks, sub_tiles, splits, cps)
+                       ws, counters, m, w.k, w.n, n_pad, w.k_chunks, sub_tiles, splits, cps, (const uint16_t *)nullptr,     \
+                       g_trace.ptr && blocks <= g_trace.capacity ? g_trace.ptr : (uint32_t *)nullptr)
     if (a_f32) {
         if constexpr (RL <= 4) {
             if (one) TWM_S_LAUNCH(true, true);

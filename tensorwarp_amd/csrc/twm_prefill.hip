@@ -16,68 +16,11 @@
 //   16*MT v_mfma_f32_16x16x32_f16 (MT row blocks x 4 column tiles x 4 groups), 16*MT accumulator registers.
 // One v_mfma issue slot hides about two other vector instructions, so the unpack (14 instructions per
 // tile and group, shared by MT row blocks) is only free from MT = 8 on.
-#include "twm_device.h"
+#include "twm_prefill_core.h"
 
 #include <type_traits>
 
 namespace twm {
-
-constexpr int kPfRowStride = 128;  // halves per LDS row (256 bytes, unpadded: the 16-byte slots of a row are XOR-swizzled)
-
-struct PfConsts {
-    uint32_t mask_lo, mask_hi, magic_lo, magic_hi;
-};
-
-__device__ __forceinline__ PfConsts make_pf_consts()
-{
-    PfConsts c = {0x000F000Fu, 0x00F000F0u, 0x64006400u, 0x54005400u};
-    asm volatile("" : "+s"(c.mask_lo), "+s"(c.mask_hi), "+v"(c.magic_lo), "+v"(c.magic_hi));
-    return c;
-}
-
-// Pins a uniform address in a scalar register pair so that the load takes it as its scalar base with the
-// per-lane part as a 32-bit offset (otherwise the loop-invariant per-lane part is folded into a 64-bit
-// vector base and every load costs a 64-bit vector add).
-#define TWM_GLOBAL __attribute__((address_space(1)))
-__device__ __forceinline__ const TWM_GLOBAL char *scalar_base(const void *p, size_t byte_offset)
-{
-    uint64_t v = (uint64_t)p + byte_offset;
-    asm("" : "+s"(v));  // not volatile: a volatile asm would cut the scheduling region in two
-    return (const TWM_GLOBAL char *)v;
-}
-
-// MFMA B operand of one tile and group: eight FP16 weights per lane
-union PfFrag {
-    uint32_t u[4];
-    half2v h2[4];
-    half8 h;
-};
-
-// Half of a fragment: nibbles 0..3 (half 0) or 4..7 (half 1) of word `w` -> f16(scale * (q - 8)).
-// 1024 + q and 64 + q are built by OR-ing the nibble into an f16 mantissa; the subtraction is exact.
-__device__ __forceinline__ void pf_unpack_half(PfFrag &r, int half, uint32_t w, uint32_t scale16, const PfConsts &c)
-{
-    union { uint32_t u; half2v h; } s2;
-    s2.u = scale16 | (scale16 << 16);
-    const half2v b_lo = {(_Float16)-1032.0f, (_Float16)-1032.0f};
-    const half2v b_hi = {(_Float16)-72.0f, (_Float16)-72.0f};
-    if (half) w >>= 8;
-    r.u[2 * half] = (w & c.mask_lo) | c.magic_lo;
-    r.u[2 * half + 1] = (w & c.mask_hi) | c.magic_hi;
-    r.h2[2 * half] = (r.h2[2 * half] + b_lo) * s2.h;
-    r.h2[2 * half + 1] = (r.h2[2 * half + 1] + b_hi) * s2.h;
-}
-
-__device__ __forceinline__ void pf_store_out(const OutSpec &out, uint32_t m, uint32_t col, float v)
-{
-#pragma unroll
-    for (uint32_t s = 0; s < kMaxSegs; s++) {
-        if (s < out.count) {
-            uint32_t rel = col - out.seg[s].start;
-            if (rel < out.seg[s].width) out.seg[s].ptr[(size_t)m * out.seg[s].width + rel] = out.seg[s].bias ? v + out.seg[s].bias[rel] : v;
-        }
-    }
-}
 
 template <int MT>  // MT = 16-row blocks per workgroup tile (BM = 16 * MT rows)
 __global__ __launch_bounds__(256) void k_prefill(const uint4v *__restrict__ qw, const uint2v *__restrict__ sc,
@@ -223,37 +166,37 @@ __global__ __launch_bounds__(256) void k_prefill(const uint4v *__restrict__ qw, 
     };
 
     // One k-chunk (B slot S = kc & 1, LDS buffer kc & 1).  On entry af0 / bf0 hold group 0 of this chunk.
-    //   step 0   : load B (nibbles, scales) of chunk kc+1 into the other slot
-    //   step 1, 2: no loads; at the end of step 2 wait for this wave's loads, then the chunk's only barrier:
-    //              A tile kc+1 is complete, and every wave is done reading buffer kc & 1 (tile kc: its reads
-    //              were issued up to step 2 and are waited for by the barrier)
-    //   step 3   : A tile kc+2 -> buffer kc & 1; the step's own reads and unpack are already those of chunk
-    //              kc+1, group 0
+    //   step 0 .. 2: no loads; at the end of step 2 wait for this wave's loads, then the chunk's only barrier:
+    //              A tile kc+1 and B of chunk kc+1 are complete (both requested a whole chunk ago, nothing newer
+    //              is in flight), and every wave is done reading buffer kc & 1 (tile kc: its reads were issued
+    //              up to step 2 and are waited for by the barrier)
+    //   step 3   : A tile kc+2 -> buffer kc & 1 and B of chunk kc+2 -> slot S (its last group was unpacked in
+    //              step 2); the step's own reads and unpack are already those of chunk kc+1, group 0
     // Past the end the last chunk is loaded again and never used.
     auto chunk = [&](auto slot_c, uint32_t kc) {
         constexpr int S = decltype(slot_c)::value, S1 = S ^ 1;
         const uint32_t buf = kc & 1u;
-        const uint32_t kc1 = kc + 1 < last ? kc + 1 : last, kc2 = kc + 2 < last ? kc + 2 : last;
-        step(af0, bf0, af1, bf1, buf, 1, S, 1, [&](int u) {
-#pragma unroll
-            for (int t = 0; t < 4; t++) {
-                if (t * MT / 4 == u) load_bq(S1, kc1, t);
-                if (t * MT / 4 + (MT >= 8 ? 1 : 0) == u) load_bs(S1, kc1, t);
-            }
-        });
+        const uint32_t kc2 = kc + 2 < last ? kc + 2 : last;
+        step(af0, bf0, af1, bf1, buf, 1, S, 1, [&](int) {});
         step(af1, bf1, af0, bf0, buf, 2, S, 2, [&](int) {});
         step(af0, bf0, af1, bf1, buf, 3, S, 3, [&](int) {});
         wait_loads();
         __syncthreads();
         step(af1, bf1, af0, bf0, buf ^ 1u, 0, S1, 0, [&](int u) {
             if (u < NV) load_a(buf, kc2, u);
+            // B of chunk kc + 2 into this chunk's own slot, whose last group was unpacked in step 2
+#pragma unroll
+            for (int t = 0; t < 4; t++) {
+                if (t * MT / 4 == u) load_bq(S, kc2, t);
+                if (t * MT / 4 + (MT >= 8 ? 1 : 0) == u) load_bs(S, kc2, t);
+            }
         });
         pin_acc();
     };
     using S0 = std::integral_constant<int, 0>;
     using S1 = std::integral_constant<int, 1>;
 
-    // prologue: tiles 0 and 1 -> LDS, B chunk 0 -> slot 0
+    // prologue: tiles 0 and 1 -> LDS, B chunks 0 and 1 -> slots 0 and 1
     const uint32_t kc1p = 1 < last ? 1 : last;
 #pragma unroll
     for (int j = 0; j < NV; j++) load_a(0, 0, j);
@@ -261,6 +204,8 @@ __global__ __launch_bounds__(256) void k_prefill(const uint4v *__restrict__ qw, 
     for (int t = 0; t < 4; t++) {
         load_bq(0, 0, t);
         load_bs(0, 0, t);
+        load_bq(1, kc1p, t);
+        load_bs(1, kc1p, t);
     }
 #pragma unroll
     for (int j = 0; j < NV; j++) load_a(1, kc1p, j);
@@ -524,12 +469,20 @@ hipError_t init_prefill()
 // `scratch` (scratch_bytes) holds the f16 copy of f32 activations and / or the split-K partials; when it
 // cannot hold all M rows the rows are processed in slabs.
 hipError_t launch_prefill(hipStream_t s, const WeightView &w, const void *a, bool a_f32, uint32_t m, const OutSpec &out,
-                          uint32_t block_rows, uint32_t splits, void *scratch, size_t scratch_bytes)
+                          uint32_t block_rows, uint32_t splits, void *scratch, size_t scratch_bytes, const PrefillSk *sk)
 {
     if (m == 0 || w.n == 0) return hipSuccess;
     if (block_rows != 0 && block_rows != 64 && block_rows != 128) return hipErrorInvalidValue;
     const size_t n_ld = (size_t)w.n_tiles * 16;
     auto run = [&](const _Float16 *a16, uint32_t rows, const OutSpec &o, void *ws, size_t ws_bytes) {
+        // Option prefill_sk: the tiles dealt out by stream-K (twm_prefill_sk.hip); the gated store stays with the plain kernel.
+        if (sk && sk->mode >= 128 && !o.swiglu && sk->partials) {
+            const uint32_t sk_rows = 128u;
+            hipError_t e = launch_prefill_sk(s, w, a16, rows, o, sk_rows, sk->workers, sk->partials, sk->partial_bytes, sk->counters,
+                                             sk->n_counters);
+            if (e != hipErrorInvalidValue) return e;  // (a shape it does not take: the plain kernel below)
+            (void)hipGetLastError();
+        }
         PrefillPlan plan = plan_prefill(rows, block_rows, splits, (w.n_tiles + 15) / 16, w.k_chunks, n_ld);
         size_t per_split = (size_t)rows * n_ld * 4;
         if (plan.splits > 1 && (!ws || per_split == 0 || plan.splits > ws_bytes / per_split)) {
