@@ -996,7 +996,9 @@ static SubPlan plan_gemv4_sub(uint32_t tiles64, uint32_t k_chunks, uint32_t m, b
         // rounds: 49.3 against 47.8)
         const uint32_t rounds = (tiles64 + 255) / 256;
         const bool poor_fill = tiles64 * 5 < rounds * 256 * 4;
-        if (!a_f32 && m <= 2 && passes16 <= 8 && poor_fill) return narrow16;
+        // (several workgroups per CU: no idle eighth wave, 3584 -> 37888 at M = 1 14.8 against 15.3 us; with one workgroup
+        // per CU the eight-wave form is the faster one, 3584 -> 3584 3.9 against 4.05)
+        if (!a_f32 && m <= 2 && passes16 <= 8 && poor_fill) return SubPlan{16, passes16};
         if (a_f32 && m <= 2 && tiles64 < 256 && k_chunks <= 32) return SubPlan{32, 16};
         return none;
     }

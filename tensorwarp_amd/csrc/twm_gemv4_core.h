@@ -83,7 +83,10 @@ __device__ __forceinline__ float4v mfma_piece(half4v a, half4v b, float4v c)
 // Term modes of the activations: one f16 term; two terms as two MFMA passes (a_lo holds the second); or, for
 // at most two rows, two terms packed into the four MFMA rows (lane l: row (l % 4) / 2, term l % 2), which
 // costs no extra MFMA: the 4x4x4 instruction computes four rows anyway.
-enum { kTermsOne = 0, kTermsTwoPasses = 1, kTermsRowPacked = 2 };
+enum { kTermsOne = 0, kTermsTwoPasses = 1, kTermsRowPacked = 2, kTermsOneRow = 3 };
+// kTermsOneRow (sub-tile kernels, one row of f16 activations): a lane loads ONE 8-wide piece of its chunk instead of the
+// 64 / SUB pieces its MFMA block supplies, and the unpack hands the pieces round inside each quad of lanes
+// (gemv4s_load_a, gemv4s_compute).
 template <bool AF32, int RL>
 constexpr int gemv4_terms() { return AF32 ? (RL <= 2 ? kTermsRowPacked : kTermsTwoPasses) : kTermsOne; }
 
@@ -218,6 +221,7 @@ struct ChunkS {
     uint2v sc;                    // four f16 scales
     uint4v a[RG][64 / SUB];       // activations: row 4*rg + (lane % SUB) % 4, piece (lane % SUB) / 4 of every 2*SUB-wide slice
     uint4v a_lo[64 / SUB];        // f32 activations as two passes: the residual terms
+    bool live;                    // false: a chunk past the k-range, replayed from a valid one; its scales count as 0
 };
 
 template <int SUB, int P>
@@ -237,6 +241,17 @@ __device__ __forceinline__ void gemv4s_load_a(ChunkS<SUB, RG> &r, const void *a_
                                               uint32_t k, bool lane_is_lo, uint32_t m_rows = 0)
 {
     static_assert(RG == 1 || !AF32, "more than four rows: f16 activations only");
+    if (TERMS == kTermsOneRow) {
+        // One row: only row 0 of an MFMA block's A operand counts, so the 16 pieces of a chunk need 16 lanes, once.
+        // 16 columns: lane cl holds piece cl (the chunk's 256 bytes, contiguous over the lane group); 32 columns: the
+        // lanes of MFMA block b (cl / 4) hold pieces 2 b and 2 b + 1 in turn.
+        static_assert(TERMS != kTermsOneRow || (!AF32 && RG == 1), "one row of f16 activations");
+        const uint32_t piece = SUB == 16 ? cl : (cl >> 2) * 2u + (cl & 1u);
+        uint32_t k0 = kc * 128u + piece * 8u;
+        if (k0 > k - 8u) k0 = k - 8u;  // only the zero-padded groups of a last partial chunk get here
+        r.a[0][0] = *(const uint4v *)((const _Float16 *)a_any + (size_t)arow * k + k0);
+        return;
+    }
 #pragma unroll
     for (int j = 0; j < 64 / SUB; j++) {
         uint32_t k0 = kc * 128u + j * (2u * SUB) + (cl >> 2) * 8u;
@@ -263,14 +278,36 @@ __device__ __forceinline__ void gemv4s_load_a(ChunkS<SUB, RG> &r, const void *a_
 }
 
 // The lane's weights from the column-lane copy: blk = the block of the lane's chunk, col = column in the
-// 64-column tile; live = false zeroes the scales (a chunk past the k-range replays a valid one as zeros).
-template <int SUB, int RG>
+// 64-column tile; live = false: a chunk past the k-range replays a valid one, gemv4s_compute takes its scales as 0.
+// (Nothing here may touch a loaded value: any use makes the compiler wait for the load where it is issued, and
+// the next pass's loads would no longer be in flight while this pass is unpacked.)
+template <int SUB, int RG, bool DEFER = false>
 __device__ __forceinline__ void gemv4s_load_w(ChunkS<SUB, RG> &r, const char *blk, uint32_t col, bool live)
 {
+    if (DEFER) {
+        r.sc = ld_once((const uint2v *)(blk + 4096u + col * 8u));
+        __builtin_amdgcn_sched_barrier(0);  // (the scheduler would put it last, and the first group's sum waits for it)
 #pragma unroll
-    for (int g = 0; g < 4; g++) r.wq[g] = ld_once((const uint4v *)(blk + g * 1024u + col * 16u));
-    uint2v s = ld_once((const uint2v *)(blk + 4096u + col * 8u));
-    r.sc = live ? s : uint2v{0u, 0u};
+        for (int g = 0; g < 4; g++) r.wq[g] = ld_once((const uint4v *)(blk + g * 1024u + col * 16u));  // (in the order of their use)
+        r.live = live;
+    } else {
+        // a single pass per wave: nothing is in flight behind these loads, the scales may be masked right here
+#pragma unroll
+        for (int g = 0; g < 4; g++) r.wq[g] = ld_once((const uint4v *)(blk + g * 1024u + col * 16u));
+        uint2v s = ld_once((const uint2v *)(blk + 4096u + col * 8u));
+        r.sc = live ? s : uint2v{0u, 0u};
+        r.live = true;
+    }
+}
+
+// lane I of every quad of lanes, in all four lanes of the quad
+template <int I>
+__device__ __forceinline__ uint4v quad_bcast(uint4v v)
+{
+    uint4v o;
+#pragma unroll
+    for (int w = 0; w < 4; w++) o[w] = (uint32_t)__builtin_amdgcn_mov_dpp((int)v[w], I * 0x55, 0xF, 0xF, true);  // quad_perm [I,I,I,I]
+    return o;
 }
 
 // acc[row] += f32(scale) * (sum over the group of A * (q - 8)) for the four groups of the lane's chunk
@@ -281,8 +318,20 @@ __device__ __forceinline__ void gemv4s_compute(const ChunkS<SUB, (RL + 3) / 4> &
     constexpr int RG = (RL + 3) / 4;
     static_assert(TERMS != kTermsRowPacked || RL <= 2, "row-packed terms hold at most two rows");
     static_assert(RG == 1 || TERMS == kTermsOne, "more than four rows: one f16 term");
+    static_assert(TERMS != kTermsOneRow || RL == 1, "the shared-piece form holds one row");
     union { uint2v u; _Float16 h[4]; } sv;
     sv.u = r.sc;
+    // kTermsOneRow: the piece held by lane i of every quad, in all four lanes of the quad (row 0 is the one that counts)
+    constexpr int QN = TERMS == kTermsOneRow ? (SUB == 16 ? 4 : 2) : 1;
+    uint4v quad[QN];
+    if (TERMS == kTermsOneRow) {
+        quad[0] = r.a[0][0];
+        if (QN > 1) quad[1 % QN] = quad_bcast<1>(r.a[0][0]);
+        if (QN > 2) {
+            quad[2 % QN] = quad_bcast<2>(r.a[0][0]);
+            quad[3 % QN] = quad_bcast<3>(r.a[0][0]);
+        }
+    }
 #pragma unroll
     for (int g = 0; g < 4; g++) {
         float4v d[RG];
@@ -293,11 +342,15 @@ __device__ __forceinline__ void gemv4s_compute(const ChunkS<SUB, (RL + 3) / 4> &
         // (4g + W) % PIECES of the lane group
 #define TWM_SUB_PIECE(W)                                                                   \
     {                                                                                      \
-        constexpr int PG = 4 * G + W, J = PG / PIECES, ABID = PG % PIECES;                 \
+        constexpr int PG = 4 * G + W, ONE_ROW = TERMS == kTermsOneRow;                     \
+        constexpr int J = ONE_ROW ? 0 : PG / PIECES;                                       \
+        /* one row: piece PG sits in MFMA block PG / 4, lane PG % 4 (16 columns) or block PG / 2, lane PG % 2 */ \
+        constexpr int ABID = ONE_ROW ? (SUB == 16 ? PG / 4 : PG / 2) : PG % PIECES;        \
+        constexpr int QI = ONE_ROW ? (SUB == 16 ? PG % 4 : PG % 2) : 0;                    \
         union { uint4v u; half4v h[2]; } av, al;                                           \
         gemv4_dequant_word(r.wq[G][W], dq, lo4, hi4);                                      \
         _Pragma("unroll") for (int rg = 0; rg < RG; rg++) {                                \
-            av.u = r.a[rg][J];                                                             \
+            av.u = ONE_ROW ? quad[QI] : r.a[rg][J];                                        \
             d[rg] = mfma_sub<SUB, ABID>(av.h[0], lo4, d[rg]);                              \
             d[rg] = mfma_sub<SUB, ABID>(av.h[1], hi4, d[rg]);                              \
         }                                                                                  \
@@ -315,7 +368,7 @@ __device__ __forceinline__ void gemv4s_compute(const ChunkS<SUB, (RL + 3) / 4> &
         TWM_SUB_GROUP(0) TWM_SUB_GROUP(1) TWM_SUB_GROUP(2) TWM_SUB_GROUP(3)
 #undef TWM_SUB_GROUP
 #undef TWM_SUB_PIECE
-        const float s = (float)sv.h[g];
+        const float s = r.live ? (float)sv.h[g] : 0.f;
 #pragma unroll
         for (int rr = 0; rr < RL; rr++) {
             if (TERMS == kTermsRowPacked) acc[rr] = fmaf(d[0][2 * rr] + d[0][2 * rr + 1], s, acc[rr]);
@@ -324,9 +377,16 @@ __device__ __forceinline__ void gemv4s_compute(const ChunkS<SUB, (RL + 3) / 4> &
     }
 }
 
-// The passes first, first + stride, ... < passes with two register sets: the next pass's loads are in flight
-// while this one is unpacked.  ONE: the caller knows that no wave has a second pass.
-template <int SUB, bool ONE, int RG = 1, class Load, class Compute>
+// The passes first, first + stride, ... < passes with two register sets.  ONE: the caller knows that no wave has a
+// second pass.
+// PIPE: the next pass's loads are in flight while this one is unpacked.  The loop body is one basic block - prefetch,
+// unpack, prefetch, unpack - and a prefetch past the wave's last pass is issued all the same (load() replays the
+// k-range's last chunk for it, marked dead, and nobody unpacks it): with a prefetch under a condition of its own the
+// compiler either moves the loads down into the block that uses them, or assumes at the join that they were not issued
+// and waits for the newest loads before the unpack may read the older ones - which is what the plain form below
+// does: its second register set only saves the address arithmetic.  The pipelined form needs both sets live through
+// the unpack; the variants with more rows or f32 activations would spill, and stay with the plain form.
+template <int SUB, bool ONE, int RG = 1, bool PIPE = false, class Load, class Compute>
 __device__ __forceinline__ void gemv4s_run_passes(uint32_t first, uint32_t stride, uint32_t passes, Load load, Compute compute)
 {
     if (ONE) {
@@ -337,10 +397,25 @@ __device__ __forceinline__ void gemv4s_run_passes(uint32_t first, uint32_t strid
         }
         return;
     }
+    if (first >= passes) return;
     ChunkS<SUB, RG> r0, r1;
     uint32_t p = first;
-    if (p >= passes) return;
     load(r0, p);
+    if (PIPE) {
+        const uint32_t mine = (passes - first + stride - 1u) / stride;  // this wave's passes
+        for (uint32_t i = 1; i < mine; i += 2) {
+            load(r1, p + stride);
+            __builtin_amdgcn_sched_barrier(0);  // (the scheduler would sink the prefetch below the unpack)
+            compute(r0);
+            __builtin_amdgcn_sched_barrier(0);
+            load(r0, p + 2u * stride);
+            __builtin_amdgcn_sched_barrier(0);
+            compute(r1);
+            p += 2u * stride;
+        }
+        if (mine & 1u) compute(r0);
+        return;
+    }
     while (true) {
         uint32_t pn = p + stride;
         if (pn < passes) load(r1, pn);

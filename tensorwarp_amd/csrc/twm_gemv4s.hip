@@ -49,7 +49,11 @@ __device__ __forceinline__ void gemv4s_body(const char *__restrict__ cw, const v
 {
     static_assert(!REFL || (AF32 && RL == 1), "the reference-layout variant is the M = 1, f32-activation entry point");
     constexpr int CPP = 64 / SUB;     // chunks per pass
-    constexpr int TERMS = gemv4_terms<AF32, RL>();
+    // One row of f16 activations on 16 columns, several passes per wave (deep K): the pipelined pass loop with the
+    // shared-piece form of the activations (18944 -> 3584 at M = 1: 9.2 against 10.0 us).  A wave that makes a single
+    // pass gains nothing from either, and the other variants run out of registers with both sets live.
+    constexpr bool PIPE = !ONE && !AF32 && RL == 1 && SUB == 16 && !REFL;
+    constexpr int TERMS = PIPE ? kTermsOneRow : gemv4_terms<AF32, RL>();
     extern __shared__ float red[];    // [waves][RL][64]
     __shared__ int s_last;
 
@@ -111,14 +115,22 @@ __device__ __forceinline__ void gemv4s_body(const char *__restrict__ cw, const v
                 sb[g] = ok[g] ? sb[g] : 0u;
             }
             r.sc = uint2v{sb[0] | (sb[1] << 16), sb[2] | (sb[3] << 16)};
+            r.live = true;  // (masked group by group above)
+            gemv4s_load_a<SUB, AF32, TERMS, REFL, RG>(r, a_any, arow, kc, cl, k, lane_is_lo, m_rows);
         } else {
-            gemv4s_load_w<SUB>(r, tbase + (size_t)kc * kColBlockBytes, col_in_tile(cl), live);
+            if (PIPE) {
+                // activations first: loads complete in the order of their issue, and these come from the cache
+                gemv4s_load_a<SUB, AF32, TERMS, REFL, RG>(r, a_any, arow, kc, cl, k, lane_is_lo, m_rows);
+                gemv4s_load_w<SUB, RG, true>(r, tbase + (size_t)kc * kColBlockBytes, col_in_tile(cl), live);
+            } else {
+                gemv4s_load_w<SUB, RG, false>(r, tbase + (size_t)kc * kColBlockBytes, col_in_tile(cl), live);
+                gemv4s_load_a<SUB, AF32, TERMS, REFL, RG>(r, a_any, arow, kc, cl, k, lane_is_lo, m_rows);
+            }
         }
-        gemv4s_load_a<SUB, AF32, TERMS, REFL, RG>(r, a_any, arow, kc, cl, k, lane_is_lo, m_rows);
     };
     auto compute_pass = [&](const ChunkS<SUB, RG> &r) { gemv4s_compute<SUB, RL, TERMS>(r, dq, acc); };
     // (ONE: the launcher saw that no wave has a second pass: one register set, no loop)
-    gemv4s_run_passes<SUB, ONE, RG>(wave, waves, passes, load_pass, compute_pass);
+    gemv4s_run_passes<SUB, ONE, RG, PIPE>(wave, waves, passes, load_pass, compute_pass);
     if (trace_loaded && threadIdx.x == 0) *trace_loaded = (uint32_t)__builtin_amdgcn_s_memrealtime();  // data arrived and unpacked
 
     // ---- sum over the waves and over the chunks of a pass (lane groups) through LDS ----
