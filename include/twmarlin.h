@@ -105,11 +105,11 @@ int twm_ctx_info(twm_ctx *ctx, char *buf, size_t buf_len);
  * Values outside these sets return TWM_SHAPE_ERROR, unknown keys TWM_UNSUPPORTED_OP. */
 int twm_ctx_set_option(twm_ctx *ctx, const char *key, int value);
 
-/* Profiling aid, no counterpart in the reference: while trace_dev is set (process-wide), every launch of the M <= 4
- * sub-tile GEMV kernel with at most capacity_workgroups workgroups has workgroup b write four 32-bit words at
- * trace_dev[4 b]: the GPU's 100 MHz clock at its start, after its first wave has unpacked its weights, and at its end,
- * and the hardware id of the CU it ran on (bits 0-15 HW_ID, bits 16-19 the XCD).  NULL or 0 switches it off.  The
- * kernels test one pointer for NULL when it is off. */
+/* Profiling aid, no counterpart in the reference: while trace_dev is set (process-wide), every launch of the M = 1
+ * sub-tile GEMV kernel (f16 activations) with at most capacity_workgroups workgroups runs a traced twin of the kernel,
+ * in which workgroup b writes four 32-bit words at trace_dev[4 b]: the GPU's 100 MHz clock at its start, after its
+ * first wave has unpacked its weights, and at its end, and the hardware id of the CU it ran on (bits 0-15 HW_ID, bits
+ * 16-19 the XCD).  NULL or 0 switches it off; the product kernels carry no trace code. */
 int twm_debug_trace(twm_ctx *ctx, uint32_t *trace_dev, uint32_t capacity_workgroups);
 
 /* ---- device memory (GpuTensor::{zeros,from_host,to_host}, tensor.rs:9-104) ------ */

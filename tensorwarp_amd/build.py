@@ -10,7 +10,9 @@ LIB = os.path.join(HERE, "libtwmarlin_hip.so")
 SOURCES = ["twm_kernels.hip", "twm_decode.hip", "twm_gemv4.hip", "twm_gemv4s.hip", "twm_moe.hip", "twm_stream.hip", "twm_batch.hip", "twm_prefill.hip", "twm_prefill_sk.hip", "twm_noalloc.hip", "twm_api.hip"]
 # The batched-decode kernels read every MFMA result with vector instructions right away (scale, add):
 # with the default choice the results land in AGPRs and each costs a v_accvgpr_read first.
-PER_FILE_FLAGS = {"twm_stream.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"], "twm_batch.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"]}
+# The decode kernels' first sixteen argument words arrive preloaded in scalar registers (see k_gemv4s).
+PRELOAD = ["-mllvm", "-amdgpu-kernarg-preload-count=16"]
+PER_FILE_FLAGS = {"twm_gemv4s.hip": PRELOAD, "twm_stream.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"], "twm_batch.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"]}
 # -packed-fp32-ops off: v_pk_{add,mul,fma}_f32 are not to be generated on this hardware pool.
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fno-gpu-rdc",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",

@@ -44,7 +44,7 @@ template <int SUB, int RL, bool AF32, bool ONE, bool REFL>
 __device__ __forceinline__ void gemv4s_body(const char *__restrict__ cw, const void *__restrict__ a_any, const OutSpec &out,
                                             float *__restrict__ ws, unsigned *__restrict__ counters, uint32_t m_rows,
                                             uint32_t k, uint32_t n, uint32_t n_pad, uint32_t k_chunks,
-                                            uint32_t sub_tiles, uint32_t splits, uint32_t cps,
+                                            uint32_t sub_tiles, uint32_t splits, uint32_t cps, bool gated_store,
                                             const uint16_t *__restrict__ ref_scales, uint32_t *trace_loaded)
 {
     static_assert(!REFL || (AF32 && RL == 1), "the reference-layout variant is the M = 1, f32-activation entry point");
@@ -74,7 +74,7 @@ __device__ __forceinline__ void gemv4s_body(const char *__restrict__ cw, const v
 
     // Gated store (paired gate_up weight: each 64-column tile is 32 gate columns, then the up columns of the same
     // features): the workgroup takes SUB / 2 gate columns and their up columns, so that it can write the products.
-    const bool gated = !REFL && out.swiglu != nullptr;
+    const bool gated = !REFL && gated_store;  // (= out.swiglu != nullptr, as an argument of its own: see k_gemv4s)
     auto col_in_tile = [&](uint32_t c) {
         return gated ? (c / (SUB / 2)) * 32u + part * (SUB / 2) + c % (SUB / 2) : part * SUB + c;
     };
@@ -199,26 +199,42 @@ __device__ __forceinline__ void gemv4s_body(const char *__restrict__ cw, const v
     if (threadIdx.x == 0) __hip_atomic_store(&counters[st], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-// trace (a profiling aid, nullptr in normal use): workgroup b writes four words at trace[4 b]: the 100 MHz clock
-// at its start, after wave 0 has unpacked its pass, and at its end, and the hardware id of the CU it ran on.
+// Argument order: what the address arithmetic of the first loads needs comes first, sixteen 32-bit words in all, which
+// the build has the hardware preload into scalar registers at wave start (-amdgpu-kernarg-preload-count); the output
+// description, a few hundred bytes that only the store needs, comes last.  A wave that has to fetch its arguments first
+// starts its weight loads one memory round trip later, and with one workgroup per CU nothing hides that.
 template <int SUB, int RL, bool AF32, bool ONE, bool REFL = false>
-__global__ __launch_bounds__(1024) void k_gemv4s(const char *__restrict__ cw, const void *__restrict__ a_any, OutSpec out,
-                                                  float *__restrict__ ws, unsigned *__restrict__ counters, uint32_t m_rows,
+__global__ __launch_bounds__(1024) void k_gemv4s(const char *__restrict__ cw, const void *__restrict__ a_any, uint32_t m_rows,
                                                   uint32_t k, uint32_t n, uint32_t n_pad, uint32_t k_chunks,
-                                                  uint32_t sub_tiles, uint32_t splits, uint32_t cps,
-                                                  const uint16_t *__restrict__ ref_scales = nullptr,
-                                                  uint32_t *__restrict__ trace = nullptr)
+                                                  uint32_t sub_tiles, uint32_t splits, uint32_t cps, uint32_t gated_store,
+                                                  const uint16_t *__restrict__ ref_scales, float *__restrict__ ws,
+                                                  unsigned *__restrict__ counters, OutSpec out)
 {
-    uint32_t *tr = trace ? trace + 4u * blockIdx.x : nullptr;
-    if (tr && threadIdx.x == 0) {
+    gemv4s_body<SUB, RL, AF32, ONE, REFL>(cw, a_any, out, ws, counters, m_rows, k, n, n_pad, k_chunks, sub_tiles, splits, cps,
+                                          gated_store != 0, ref_scales, nullptr);
+}
+
+// The same kernel with a trace (twm_debug_trace; one row of f16 activations only): workgroup b writes four words at
+// trace[4 b]: the 100 MHz clock at its start, after wave 0 has unpacked its passes, and at its end, and the hardware
+// id of the CU it ran on.  A kernel of its own: reading the trace pointer first would put a second, dependent kernel
+// argument fetch in front of every wave of the product kernel.
+template <int SUB, bool ONE>
+__global__ __launch_bounds__(1024) void k_gemv4s_traced(const char *__restrict__ cw, const void *__restrict__ a_any, OutSpec out,
+                                                         float *__restrict__ ws, unsigned *__restrict__ counters,
+                                                         uint32_t m_rows, uint32_t k, uint32_t n, uint32_t n_pad,
+                                                         uint32_t k_chunks, uint32_t sub_tiles, uint32_t splits, uint32_t cps,
+                                                         uint32_t *__restrict__ trace)
+{
+    uint32_t *tr = trace + 4u * blockIdx.x;
+    if (threadIdx.x == 0) {
         tr[0] = (uint32_t)__builtin_amdgcn_s_memrealtime();
         tr[1] = 0u;
         // HW_ID (register 4): wave, SIMD, CU, SH, SE ids; XCC_ID (register 20): the XCD
         tr[3] = (__builtin_amdgcn_s_getreg((31 << 11) | 4) & 0xFFFFu) | (__builtin_amdgcn_s_getreg((3 << 11) | 20) << 16);
     }
-    gemv4s_body<SUB, RL, AF32, ONE, REFL>(cw, a_any, out, ws, counters, m_rows, k, n, n_pad, k_chunks, sub_tiles, splits, cps,
-                                          ref_scales, tr ? tr + 1 : nullptr);
-    if (tr && threadIdx.x == 0) tr[2] = (uint32_t)__builtin_amdgcn_s_memrealtime();
+    gemv4s_body<SUB, 1, false, ONE, false>(cw, a_any, out, ws, counters, m_rows, k, n, n_pad, k_chunks, sub_tiles, splits, cps,
+                                           out.swiglu != nullptr, nullptr, tr + 1);
+    if (threadIdx.x == 0) tr[2] = (uint32_t)__builtin_amdgcn_s_memrealtime();
 }
 
 template <int SUB, int RL>
@@ -233,9 +249,20 @@ static hipError_t launch_gemv4s_t(hipStream_t s, const WeightView &w, const void
     size_t lds = (size_t)waves * RL * 64 * sizeof(float);
     const bool one = (cps + 64 / SUB - 1) / (64 / SUB) <= waves;
 #define TWM_S_LAUNCH(AF, ONEV)                                                                                          \
-    hipLaunchKernelGGL((k_gemv4s<SUB, RL, AF, ONEV>), dim3(blocks), dim3(waves * 64), lds, s, (const char *)w.cq, a, out, \
-                       ws, counters, m, w.k, w.n, n_pad, w.k_chunks, sub_tiles, splits, cps, (const uint16_t *)nullptr,     \
-                       g_trace.ptr && blocks <= g_trace.capacity ? g_trace.ptr : (uint32_t *)nullptr)
+    hipLaunchKernelGGL((k_gemv4s<SUB, RL, AF, ONEV>), dim3(blocks), dim3(waves * 64), lds, s, (const char *)w.cq, a, m, w.k, \
+                       w.n, n_pad, w.k_chunks, sub_tiles, splits, cps, out.swiglu ? 1u : 0u, (const uint16_t *)nullptr, ws,  \
+                       counters, out)
+    if constexpr (RL == 1) {
+        if (!a_f32 && g_trace.ptr && blocks <= g_trace.capacity) {
+            if (one)
+                hipLaunchKernelGGL((k_gemv4s_traced<SUB, true>), dim3(blocks), dim3(waves * 64), lds, s, (const char *)w.cq, a, out,
+                                   ws, counters, m, w.k, w.n, n_pad, w.k_chunks, sub_tiles, splits, cps, g_trace.ptr);
+            else
+                hipLaunchKernelGGL((k_gemv4s_traced<SUB, false>), dim3(blocks), dim3(waves * 64), lds, s, (const char *)w.cq, a, out,
+                                   ws, counters, m, w.k, w.n, n_pad, w.k_chunks, sub_tiles, splits, cps, g_trace.ptr);
+            return hipGetLastError();
+        }
+    }
     if (a_f32) {
         if constexpr (RL <= 4) {
             if (one) TWM_S_LAUNCH(true, true);
@@ -298,7 +325,7 @@ hipError_t launch_gemv4s_ref(hipStream_t s, const uint8_t *packed, const uint16_
     out.seg[0].width = n;
 #define TWM_S_REF(SUBV, ONEV)                                                                                          \
     hipLaunchKernelGGL((k_gemv4s<SUBV, 1, true, ONEV, true>), dim3(blocks), dim3(waves * 64), lds, s, (const char *)packed, \
-                       (const void *)a, out, ws, counters, 1u, k, n, n_pad, k_chunks, sub_tiles, splits, cps, scales)
+                       (const void *)a, 1u, k, n, n_pad, k_chunks, sub_tiles, splits, cps, 0u, scales, ws, counters, out)
     if (sub == 32) {
         if (one) TWM_S_REF(32, true);
         else TWM_S_REF(32, false);
