@@ -89,11 +89,15 @@ int twm_ctx_info(twm_ctx *ctx, char *buf, size_t buf_len);
  *   "waves"         waves per workgroup of the decode kernels (1, 2, 4, 8, 16; streaming kernel 4 or 8)
  *   "sub"           M <= 4 and expert-bank kernels: 1 = whole 64-column tiles per workgroup, 16 or 32 = sub-tiles
  *                   of that many columns (with "waves" waves, default 8), 0 = the planner's choice per shape
- *   "kernel"        decode kernel: 1 = 16x16x32 tile kernel (16-row blocks), 2 = one-lane-per-column kernel
+ *   "kernel"        decode kernel: 2 = one-lane-per-column kernel on whole 64-column tiles
  *                   (M <= 4 only), 3 = batched-decode streaming kernel (32-row blocks), 4 = batched-decode kernel
  *                   with the activations shared through LDS (32-row blocks; "nt" 1 / 2 = tiles per wave, 4 / 3 =
  *                   two / three column quads per workgroup, "waves" 8 / 16 = two / four k-slices per workgroup)
  *   "dequant_src"   which repacked copy twm_weight_dequant_f16 unpacks: 0 = 16-column tiles, 1 = column lanes
+ *   "weight_copies" the repacked orders a new weight handle is given: 0 or 3 = both, 1 = 16-column tiles only,
+ *                   2 = column lanes only (twm_weight_ensure)
+ *   "sub_waves"     waves per workgroup of the sub-tile kernels when "sub" forces their width (1 .. 16)
+ *   "prefill_sk"    prefill GEMM: 128 = tiles dealt out by stream-K over one workgroup per CU, 0 / 1 = off
  *   "prefill_min_m" smallest M that runs the prefill GEMM (default 33; below it the decode kernels run)
  *   "prefill_bm"    rows of A per prefill workgroup (64 or 128)
  *   "m1_exact"      twm_gemm_tw_marlin_m1: 1 = f32 activations and f32 FMAs in the reference kernel's order with
@@ -232,6 +236,16 @@ void twm_weight_destroy(twm_weight *w);
 int twm_weight_dims(const twm_weight *w, uint32_t *k, uint32_t *n);
 /* device bytes held by the repacked weight */
 size_t twm_weight_bytes(const twm_weight *w);
+/* The handle holds the weight in up to two orders: the 16-column tile order (copy 1: the kernels for M >= 5 and the
+ * prefill GEMM) and the column-lane order (copy 2: M <= 4, and M = 5 .. 16 on narrow matrices), 4.5 bits per weight
+ * each.  Option "weight_copies" says which ones a new handle gets (0 or 3 = both, the default; 1; 2); a call that needs
+ * a copy the handle does not hold builds it from the other one on the spot -- which allocates, so inside a graph
+ * capture such a call fails with TWM_UNSUPPORTED_OP: ask for the copy beforehand with twm_weight_ensure.
+ * twm_weight_drop frees one of two copies (synchronises the stream); twm_weight_copies returns the mask held.
+ * No counterpart in the reference, whose kernels read the one TW-Marlin order. */
+int twm_weight_ensure(twm_ctx *ctx, twm_weight *w, int copies);
+int twm_weight_drop(twm_ctx *ctx, twm_weight *w, int copies);
+int twm_weight_copies(const twm_weight *w);
 /* The repacked weight as a self-describing byte blob, for an on-disk cache of the internal order
  * beside the reference's pre-quantized `.warp` cache (crates/loader/src/warp_cache.rs:1-21: store
  * it there as one U8 tensor per projection).  Import skips quantize / reorder / fuse / repack: it
@@ -303,6 +317,13 @@ typedef struct twm_bank twm_bank;
 twm_bank *twm_bank_from_device(twm_ctx *ctx, const uint8_t *packed_base_dev, const uint16_t *scales_base_dev,
                                size_t packed_bytes_per_expert, size_t scales_per_expert, uint32_t k,
                                uint32_t n, uint32_t num_experts, int pair_gate_up);
+/* The same bank from per-expert offset tables: expert e lies at packed_base + packed_offsets[e] (bytes, a multiple of
+ * 4) and scales_base + scales_offsets[e] (f16 elements), both tables u32 arrays of num_experts entries in device
+ * memory -- the arguments of gemm_tw_marlin_m1_indirect (crates/kernels/src/quantize_indirect.rs:228-253), whose
+ * experts need not be equally spaced.  The tables are read once, here (a synchronous copy); the inputs are not retained. */
+twm_bank *twm_bank_from_device_offsets(twm_ctx *ctx, const uint8_t *packed_base_dev, const uint16_t *scales_base_dev,
+                                       const uint32_t *packed_offsets_dev, const uint32_t *scales_offsets_dev, uint32_t k,
+                                       uint32_t n, uint32_t num_experts, int pair_gate_up);
 void twm_bank_destroy(twm_bank *b);
 size_t twm_bank_bytes(const twm_bank *b);
 /* All top_k expert GEMVs in one launch, the expert of slot s being (int)topk_ids_dev[s], read on the

@@ -58,6 +58,9 @@ SIGNATURES = {
     "twm_weight_destroy": (None, [_vp]),
     "twm_weight_dims": (_int, [_vp, C.POINTER(_u32), C.POINTER(_u32)]),
     "twm_weight_bytes": (_sz, [_vp]),
+    "twm_weight_ensure": (_int, [_vp, _vp, _int]),
+    "twm_weight_drop": (_int, [_vp, _vp, _int]),
+    "twm_weight_copies": (_int, [_vp]),
     "twm_weight_blob_bytes": (_sz, [_vp]),
     "twm_weight_export": (_int, [_vp, _vp, _vp, _sz]),
     "twm_weight_import": (_vp, [_vp, _vp, _sz]),
@@ -70,6 +73,7 @@ SIGNATURES = {
     "twm_gemm_geglu": (_int, [_vp, _vp, _vp, _int, _u32, _vp, _u32]),
     "twm_gemm_split_bias": (_int, [_vp, _vp, _vp, _int, _u32, C.POINTER(_vp), C.POINTER(_vp), C.POINTER(_u32), _u32, _u32]),
     "twm_bank_from_device": (_vp, [_vp, _vp, _vp, _sz, _sz, _u32, _u32, _u32, _int]),
+    "twm_bank_from_device_offsets": (_vp, [_vp, _vp, _vp, _vp, _vp, _u32, _u32, _u32, _int]),
     "twm_bank_destroy": (None, [_vp]),
     "twm_bank_bytes": (_sz, [_vp]),
     "twm_bank_gemv": (_int, [_vp, _vp, _vp, _int, _u32, _vp, _u32, _int, _vp]),

@@ -50,24 +50,30 @@ struct twm_ctx {
     int force_waves;      // 0 = heuristic
     int force_sub_waves;  // sub-tile kernels with a forced width: waves per workgroup (1 .. 16), 0 = "waves" or eight
     int force_sub;        // M <= 4: 0 = heuristic, 1 = whole 64-column tiles per workgroup, 32 or 16 = the sub-tile kernel
-    int force_kernel;     // 0 = heuristic, 1 = 16-column tile kernel, 2 = one-lane-per-column kernel (M <= 4), 3 = streaming kernel (M <= 32),
+    int force_kernel;     // 0 = heuristic, 2 = one-lane-per-column kernel on whole tiles (M <= 4), 3 = streaming kernel (M <= 32),
                           // 4 = batched-decode kernel with LDS-shared activations (M <= 32; "nt" = tiles per wave, "waves" 8 / 16 = 2 / 4 k-slices)
     int prefill_bm;       // rows of A per prefill workgroup: 0 = choose, 64 or 128
     int prefill_min_m;    // M from which the LDS/MFMA prefill kernel runs instead of 16-row decode blocks
     int dequant_src;      // which copy twm_weight_dequant_f16 unpacks: 0 = 16-column tiles, 1 = column-lane
+    int weight_copies;    // copies a new weight handle is given: 0 or 3 = both, 1 = 16-column tiles only, 2 = column-lane only
     int m1_exact;         // twm_gemm_tw_marlin_m1: 1 = f32 activations and f32 FMAs in the reference's order
     int m1_splits;        // twm_gemm_tw_marlin_m1: split-K factor of the MFMA kernel, 0 = heuristic
     int batch_rounded;    // M = 17 .. 32: 1 = weights rounded to f16 (the reference's dequant-then-FP16-GEMM arithmetic), 0 = exact
     hipDeviceProp_t prop;
 };
 
+// The two repacked copies are allocations of their own, each made when the handle is created (option
+// "weight_copies") or at the first call that needs it (weight_ensure): a decode-only or prefill-only deployment holds
+// one copy, 4.5 bits per weight.
+enum { kCopyTile = 1, kCopyCol = 2 };
 struct twm_weight {
     twm_ctx *ctx;
-    void *qw;   // one allocation: 16-column tile order (qw, sc) then the column-lane copy (cq, cs)
+    void *qw;   // 16-column tile order: nibbles (qw) and scales (sc) in one allocation; nullptr while not built
     void *sc;
-    void *cq;   // column-lane copy: 4608-byte blocks (nibbles + scales together)
+    void *cq;   // column-lane copy: 4608-byte blocks (nibbles + scales together); nullptr while not built
     uint32_t k, n, groups, n_tiles, k_chunks;
-    size_t bytes;
+    size_t copy_bytes;  // one copy
+    size_t bytes;       // device memory held now
     bool paired;  // gate_up weight whose columns are in the paired order (32 gate, 32 up, ...)
 };
 
@@ -119,6 +125,7 @@ twm_ctx *twm_ctx_create(int ordinal)
     c->force_sub_waves = 0;
     c->force_kernel = 0;
     c->dequant_src = 0;
+    c->weight_copies = 0;
     c->m1_exact = 0;
     c->m1_splits = 0;
     c->batch_rounded = 0;
@@ -210,7 +217,7 @@ int twm_ctx_info(twm_ctx *ctx, char *buf, size_t buf_len)
 }
 
 /* Tuning knobs for sweeps (0 = heuristic): "nt" = tiles per workgroup (1, 2, 4); "waves" = waves per
- * workgroup; "kernel" = 1 the 16-column tile kernel, 2 the one-lane-per-column kernel (M <= 4), 3 the
+ * workgroup; "kernel" = 2 the one-lane-per-column kernel (M <= 4), 3 the
  * streaming kernel, 4 the batched-decode kernel with LDS-shared activations;
  * "dequant_src" = which weight copy twm_weight_dequant_f16 unpacks; "prefill_min_m" = smallest M that
  * runs the prefill kernel. */
@@ -255,6 +262,11 @@ int twm_ctx_set_option(twm_ctx *ctx, const char *key, int value)
         ctx->prefill_min_m = value;
         return TWM_OK;
     }
+    if (strcmp(key, "weight_copies") == 0) {
+        if (value < 0 || value > 3) return api_fail(TWM_SHAPE_ERROR, "twm_ctx_set_option: weight_copies must be 0 .. 3");
+        ctx->weight_copies = value;
+        return TWM_OK;
+    }
     if (strcmp(key, "dequant_src") == 0) {
         if (value != 0 && value != 1) return api_fail(TWM_SHAPE_ERROR, "twm_ctx_set_option: dequant_src must be 0 or 1");
         ctx->dequant_src = value;
@@ -276,7 +288,7 @@ int twm_ctx_set_option(twm_ctx *ctx, const char *key, int value)
         return TWM_OK;
     }
     if (strcmp(key, "kernel") == 0) {
-        if (value < 0 || value > 4) return api_fail(TWM_SHAPE_ERROR, "twm_ctx_set_option: kernel must be 0 .. 4");
+        if (value < 0 || value > 4 || value == 1) return api_fail(TWM_SHAPE_ERROR, "twm_ctx_set_option: kernel must be 0, 2, 3 or 4");
         ctx->force_kernel = value;
         return TWM_OK;
     }
@@ -665,24 +677,83 @@ static twm_weight *weight_alloc(twm_ctx *ctx, uint32_t k, uint32_t n)
     w->n_tiles = n_pad / kTileN;
     w->k_chunks = (w->groups + kChunkGroups - 1) / kChunkGroups;
     size_t tiles = (size_t)w->n_tiles * w->k_chunks;
-    // Both copies hold the same K x N weights (16-column tiles for M > 4, one lane per column for
-    // M <= 4); with 288 GB of HBM the second copy of a 4-bit model is cheap and each kernel streams
-    // the order that suits it.
-    size_t qbytes = tiles * 1024, sbytes = tiles * 128;
-    w->bytes = 2 * (qbytes + sbytes);
+    w->copy_bytes = tiles * (1024 + 128);  // nibbles + scales: the same in either order
+    w->bytes = 0;
     w->qw = w->sc = w->cq = nullptr;
     w->paired = false;
-    if (tiles == 0) return w;
-    hipError_t e = hipMalloc(&w->qw, w->bytes);
-    if (e != hipSuccess) {
-        api_fail(TWM_MEMORY_ERROR, "twm_weight: hipMalloc(%zu): %s", w->bytes, hipGetErrorString(e));
-        delete w;
-        return nullptr;
-    }
-    w->sc = (char *)w->qw + qbytes;
-    w->cq = (char *)w->sc + sbytes;
     return w;
 }
+
+// device memory for the copies in `mask` that the handle does not hold yet (contents undefined)
+static int weight_alloc_copies(twm_weight *w, int mask, const char *who)
+{
+    if (w->copy_bytes == 0) return TWM_OK;
+    if ((mask & kCopyTile) && !w->qw) {
+        hipError_t e = hipMalloc(&w->qw, w->copy_bytes);
+        if (e != hipSuccess) { w->qw = nullptr; return api_fail(TWM_MEMORY_ERROR, "%s: hipMalloc(%zu): %s", who, w->copy_bytes, hipGetErrorString(e)); }
+        w->sc = (char *)w->qw + (size_t)w->n_tiles * w->k_chunks * 1024;
+        w->bytes += w->copy_bytes;
+    }
+    if ((mask & kCopyCol) && !w->cq) {
+        hipError_t e = hipMalloc(&w->cq, w->copy_bytes);
+        if (e != hipSuccess) { w->cq = nullptr; return api_fail(TWM_MEMORY_ERROR, "%s: hipMalloc(%zu): %s", who, w->copy_bytes, hipGetErrorString(e)); }
+        w->bytes += w->copy_bytes;
+    }
+    return TWM_OK;
+}
+
+static void weight_release(twm_weight *w)
+{
+    if (w->qw) (void)hipFree(w->qw);
+    if (w->cq) (void)hipFree(w->cq);
+    delete w;
+}
+
+static int copies_of(const twm_weight *w) { return (w->qw ? kCopyTile : 0) | (w->cq ? kCopyCol : 0); }
+
+// Makes sure the handle holds the copies in `mask`, building a missing one from the other on the context's stream.
+// Allocates, so not inside a graph capture: a caller that captures its launches asks for the copies before
+// (twm_weight_ensure, or option "weight_copies" when the handle is made).
+static int weight_ensure(twm_ctx *ctx, const twm_weight *cw, int mask, const char *who)
+{
+    twm_weight *w = const_cast<twm_weight *>(cw);  // (the handle is the library's own object; callers see it opaque)
+    const int have = copies_of(w), missing = mask & ~have;
+    if (!missing || w->copy_bytes == 0) return TWM_OK;
+    if (ctx->capturing)
+        return api_fail(TWM_UNSUPPORTED_OP, "%s: this call needs the weight's %s copy, which the handle does not hold, and building it "
+                        "allocates: call twm_weight_ensure before the capture", who, (missing & kCopyTile) ? "16-column tile" : "column-lane");
+    if (!have) return api_fail(TWM_INVALID_HANDLE, "%s: the weight holds no copy at all", who);
+    if (int rc = weight_alloc_copies(w, missing, who)) return rc;
+    hipError_t e = (missing & kCopyTile) ? launch_col_to_tile(ctx->stream, w->cq, w->n_tiles, w->k_chunks, w->qw, w->sc)
+                                         : launch_tile_to_col(ctx->stream, w->qw, w->sc, w->n_tiles, w->k_chunks, w->cq);
+    if (e != hipSuccess) return api_fail(TWM_DEVICE_ERROR, "%s: building the second weight copy: %s", who, hipGetErrorString(e));
+    return TWM_OK;
+}
+
+int twm_weight_ensure(twm_ctx *ctx, twm_weight *w, int copies)
+{
+    if (!ctx || !w) return api_fail(TWM_INVALID_HANDLE, "twm_weight_ensure: null handle");
+    if (w->ctx != ctx) return api_fail(TWM_INVALID_HANDLE, "twm_weight_ensure: weight belongs to another context");
+    if (copies < 1 || copies > 3) return api_fail(TWM_SHAPE_ERROR, "twm_weight_ensure: copies is 1 (16-column tiles), 2 (column-lane) or 3 (both)");
+    return weight_ensure(ctx, w, copies, "twm_weight_ensure");
+}
+
+int twm_weight_drop(twm_ctx *ctx, twm_weight *w, int copies)
+{
+    if (!ctx || !w) return api_fail(TWM_INVALID_HANDLE, "twm_weight_drop: null handle");
+    if (w->ctx != ctx) return api_fail(TWM_INVALID_HANDLE, "twm_weight_drop: weight belongs to another context");
+    if (ctx->capturing) return api_fail(TWM_UNSUPPORTED_OP, "twm_weight_drop: not allowed inside a graph capture");
+    if (copies != kCopyTile && copies != kCopyCol) return api_fail(TWM_SHAPE_ERROR, "twm_weight_drop: copies is 1 (16-column tiles) or 2 (column-lane)");
+    if (w->copy_bytes == 0 || !(copies_of(w) & copies)) return TWM_OK;
+    if (copies_of(w) == copies) return api_fail(TWM_SHAPE_ERROR, "twm_weight_drop: that is the only copy the handle holds");
+    HIP_TRY(hipStreamSynchronize(ctx->stream), TWM_DEVICE_ERROR, "twm_weight_drop: sync");
+    if (copies == kCopyTile) { (void)hipFree(w->qw); w->qw = w->sc = nullptr; }
+    else { (void)hipFree(w->cq); w->cq = nullptr; }
+    w->bytes -= w->copy_bytes;
+    return TWM_OK;
+}
+
+int twm_weight_copies(const twm_weight *w) { return w ? copies_of(w) : 0; }
 
 twm_weight *twm_weight_from_device(twm_ctx *ctx, const uint8_t *packed_dev, const uint16_t *scales_dev, uint32_t k,
                                    uint32_t n)
@@ -697,15 +768,17 @@ twm_weight *twm_weight_from_device(twm_ctx *ctx, const uint8_t *packed_dev, cons
     if (((uintptr_t)packed_dev & 3) != 0) { api_fail(TWM_SHAPE_ERROR, "twm_weight_from_device: packed must be 4-byte aligned"); return nullptr; }
     twm_weight *w = weight_alloc(ctx, k, n);
     if (!w) return nullptr;
-    if (w->qw) {
-        hipError_t e = launch_repack(ctx->stream, packed_dev, scales_dev, k, n, w->qw, w->sc, w->n_tiles, w->k_chunks);
-        if (e == hipSuccess)
+    const int mask = ctx->weight_copies ? ctx->weight_copies : (kCopyTile | kCopyCol);
+    if (weight_alloc_copies(w, mask, "twm_weight_from_device")) { weight_release(w); return nullptr; }
+    if (w->copy_bytes) {
+        hipError_t e = hipSuccess;
+        if (w->qw) e = launch_repack(ctx->stream, packed_dev, scales_dev, k, n, w->qw, w->sc, w->n_tiles, w->k_chunks);
+        if (e == hipSuccess && w->cq)
             e = launch_repack_col(ctx->stream, packed_dev, scales_dev, k, n, w->cq, w->n_tiles * kTileN, w->k_chunks);
         if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
         if (e != hipSuccess) {
             api_fail(TWM_DEVICE_ERROR, "twm_weight_from_device: repack: %s", hipGetErrorString(e));
-            (void)hipFree(w->qw);
-            delete w;
+            weight_release(w);
             return nullptr;
         }
     }
@@ -765,11 +838,8 @@ int twm_weight_is_paired(const twm_weight *w) { return w && w->paired ? 1 : 0; }
 void twm_weight_destroy(twm_weight *w)
 {
     if (!w) return;
-    if (w->qw) {
-        (void)hipStreamSynchronize(w->ctx->stream);
-        (void)hipFree(w->qw);
-    }
-    delete w;
+    if (w->qw || w->cq) (void)hipStreamSynchronize(w->ctx->stream);
+    weight_release(w);
 }
 
 int twm_weight_dims(const twm_weight *w, uint32_t *k, uint32_t *n)
@@ -792,11 +862,12 @@ struct WeightBlobHeader {
     uint32_t paired;
     uint64_t payload_bytes;
     uint64_t checksum;      // of the payload
-    uint8_t reserved[16];
+    uint8_t copies;         // payload: the 16-column tile copy (bit 0) and / or the column-lane copy (bit 1), in this order
+    uint8_t reserved[15];
 };
 static_assert(sizeof(WeightBlobHeader) == 64, "blob header is 64 bytes");
 static const char kBlobMagic[8] = {'T', 'W', 'M', 'W', 'G', 'T', '0', '1'};
-static const uint32_t kBlobLayout = 3;
+static const uint32_t kBlobLayout = 4;
 
 // Four independent multiply-rotate lanes over 64-bit words (memory-bound on the host), folded at the end.
 static uint64_t blob_checksum(const uint8_t *p, size_t bytes)
@@ -829,9 +900,15 @@ int twm_weight_export(twm_ctx *ctx, const twm_weight *w, void *blob_host, size_t
     if (blob_bytes != twm_weight_blob_bytes(w))
         return api_fail(TWM_SHAPE_ERROR, "twm_weight_export: the buffer must hold %zu bytes, got %zu", twm_weight_blob_bytes(w), blob_bytes);
     uint8_t *payload = (uint8_t *)blob_host + sizeof(WeightBlobHeader);
-    size_t payload_bytes = (w->qw != nullptr) ? w->bytes : 0;
-    if (payload_bytes)
-        if (int rc = twm_memcpy_d2h(ctx, payload, w->qw, payload_bytes)) return rc;
+    size_t at = 0;
+    if (w->qw) {
+        if (int rc = twm_memcpy_d2h(ctx, payload + at, w->qw, w->copy_bytes)) return rc;
+        at += w->copy_bytes;
+    }
+    if (w->cq) {
+        if (int rc = twm_memcpy_d2h(ctx, payload + at, w->cq, w->copy_bytes)) return rc;
+        at += w->copy_bytes;
+    }
     WeightBlobHeader hd;
     memset(&hd, 0, sizeof hd);
     memcpy(hd.magic, kBlobMagic, 8);
@@ -841,8 +918,9 @@ int twm_weight_export(twm_ctx *ctx, const twm_weight *w, void *blob_host, size_t
     hd.n_tiles = w->n_tiles;
     hd.k_chunks = w->k_chunks;
     hd.paired = w->paired ? 1u : 0u;
-    hd.payload_bytes = w->bytes;
-    hd.checksum = blob_checksum(payload, payload_bytes);
+    hd.payload_bytes = at;
+    hd.checksum = blob_checksum(payload, at);
+    hd.copies = (uint8_t)copies_of(w);
     memcpy(blob_host, &hd, sizeof hd);
     return TWM_OK;
 }
@@ -863,19 +941,24 @@ twm_weight *twm_weight_import(twm_ctx *ctx, const void *blob_host, size_t blob_b
     twm_weight *w = weight_alloc(ctx, hd.k, hd.n);
     if (!w) return nullptr;
     const uint8_t *payload = (const uint8_t *)blob_host + sizeof(WeightBlobHeader);
-    bool ok = w->n_tiles == hd.n_tiles && w->k_chunks == hd.k_chunks && w->bytes == hd.payload_bytes &&
+    const int held = hd.copies & 3, n_held = (held & 1) + (held >> 1);
+    bool ok = w->n_tiles == hd.n_tiles && w->k_chunks == hd.k_chunks && hd.copies <= 3 &&
+              (w->copy_bytes == 0 ? hd.payload_bytes == 0 : (n_held >= 1 && hd.payload_bytes == (uint64_t)n_held * w->copy_bytes)) &&
               blob_bytes == sizeof(WeightBlobHeader) + hd.payload_bytes && hd.paired <= 1 &&
               (!hd.paired || hd.n % (2 * kPairWidth) == 0);
     if (!ok) api_fail(TWM_SHAPE_ERROR, "twm_weight_import: header does not describe a %u x %u weight of %zu bytes", hd.k, hd.n, blob_bytes);
-    size_t payload_bytes = w->qw ? w->bytes : 0;
-    if (ok && blob_checksum(payload, payload_bytes) != hd.checksum) {
+    if (ok && blob_checksum(payload, (size_t)hd.payload_bytes) != hd.checksum) {
         ok = false;
         api_fail(TWM_SHAPE_ERROR, "twm_weight_import: checksum mismatch (corrupt or truncated blob)");
     }
-    if (ok && payload_bytes) ok = twm_memcpy_h2d(ctx, w->qw, payload, payload_bytes) == TWM_OK;
+    if (ok && w->copy_bytes) {
+        ok = weight_alloc_copies(w, held, "twm_weight_import") == TWM_OK;
+        size_t at = 0;
+        if (ok && w->qw) { ok = twm_memcpy_h2d(ctx, w->qw, payload + at, w->copy_bytes) == TWM_OK; at += w->copy_bytes; }
+        if (ok && w->cq) ok = twm_memcpy_h2d(ctx, w->cq, payload + at, w->copy_bytes) == TWM_OK;
+    }
     if (!ok) {
-        if (w->qw) (void)hipFree(w->qw);
-        delete w;
+        weight_release(w);
         return nullptr;
     }
     w->paired = hd.paired != 0;
@@ -901,7 +984,8 @@ int twm_weight_dequant_f16(twm_ctx *ctx, const twm_weight *w, uint16_t *out_kn_d
     if (!ctx || !w) return api_fail(TWM_INVALID_HANDLE, "twm_weight_dequant_f16: null handle");
     if ((uint64_t)w->k * w->n == 0) return TWM_OK;
     if (!out_kn_dev) return api_fail(TWM_INVALID_HANDLE, "twm_weight_dequant_f16: null output");
-    // "dequant_src" = 1 reads the column-lane copy instead of the 16-column tile order
+    // "dequant_src" = 1 reads the column-lane copy instead of the 16-column tile order (each builds its copy if need be)
+    if (int rc = weight_ensure(ctx, w, ctx->dequant_src == 1 ? kCopyCol : kCopyTile, "twm_weight_dequant_f16")) return rc;
     if (ctx->dequant_src == 1)
         HIP_TRY(launch_weight_dequant_f16_col(ctx->stream, view_of(w), out_kn_dev), TWM_DEVICE_ERROR, "dequant launch");
     else
@@ -910,37 +994,6 @@ int twm_weight_dequant_f16(twm_ctx *ctx, const twm_weight *w, uint16_t *out_kn_d
 }
 
 /* ---- dispatcher --------------------------------------------------------------------------- */
-
-// Tile / wave / split-K choice for 256 CUs x 4 SIMDs.  Work comes in units of one n-tile x one
-// k-chunk (1 KiB of nibbles).  Aim for about 4096 waves (16 per CU), each with at least two units
-// when the matrix is big enough; split K inside the workgroup first (LDS reduction), across
-// workgroups only when there are too few n-tiles to occupy the CUs.
-static DecodePlan plan_decode(uint32_t n_tiles, uint32_t k_chunks, uint32_t m, int force_nt, int force_waves,
-                              uint32_t force_splits)
-{
-    DecodePlan p;
-    p.lane_col = 0;
-    p.nt = 1;
-    if (n_tiles >= 2048) p.nt = 2;
-    if (force_nt && force_nt != 3) p.nt = (uint32_t)force_nt;  // (3 is a choice of the batched-decode kernel only)
-    uint32_t tg = n_tiles / p.nt;
-    if (tg == 0) tg = 1;
-    // waves per workgroup: enough that tg * waves reaches ~4096, bounded by the chunks available
-    p.waves = 4;
-    while (p.waves < 16 && tg * p.waves < 3072 && k_chunks >= p.waves * 2) p.waves *= 2;
-    if (force_waves) p.waves = (uint32_t)force_waves;
-    while (p.waves > 4 && p.waves * p.nt > 64) p.waves /= 2;
-    // cross-workgroup splits: the partial tiles of this kernel are 16 rows deep, so parking and re-reading them
-    // costs more than idle CUs unless fewer than 128 workgroups exist (per-shape sweep: 224 tile groups of the
-    // 7B `down` run 15 us unsplit, 24 us with 4 splits)
-    uint32_t sp = 1;
-    uint32_t per_wg = p.waves * 2;  // keep >= 2 chunks per wave
-    while (tg * sp < 128 && (k_chunks / (sp * 2)) >= per_wg) sp *= 2;
-    if (force_splits) sp = force_splits;
-    if (sp > k_chunks) sp = k_chunks ? k_chunks : 1;
-    p.splits = sp;
-    return p;
-}
 
 // M <= 4 kernel (one lane per column): a workgroup of `waves` waves shares nt tiles of 64 columns
 // and splits its k-chunks among the waves; workgroups split K further when 64-column tiles alone
@@ -1143,11 +1196,17 @@ static int gemm_common(twm_ctx *ctx, const twm_weight *w, const void *a_dev, int
     WeightView v = view_of(w);
     size_t a_row_bytes = (size_t)w->k * (a_dtype == TWM_F16 ? 2 : 4);
     uint32_t n_ld = w->n_tiles * kTileN;
-    // the paired store: every kernel but the 16-column tile kernel of option "kernel" = 1 has it
     OutSpec gated = out;
     gated.swiglu = swiglu_out;
     gated.gate_act = gate_act;
+    // the copy a launch reads is built here if the handle does not hold it yet (weight_ensure)
+#define TWM_NEED(COPY)                                                 \
+    do {                                                               \
+        if (int rc_ = weight_ensure(ctx, w, COPY, who)) return rc_;    \
+        v = view_of(w);                                                \
+    } while (0)
     if (m >= (uint32_t)ctx->prefill_min_m) {
+        TWM_NEED(kCopyTile);
         const PrefillSk sk = {ctx->sk_ws, ctx->sk_ws_bytes, ctx->counters, ctx->n_counters, (uint32_t)ctx->prop.multiProcessorCount,
                               ctx->prefill_sk};
         HIP_TRY(launch_prefill(ctx->stream, v, a_dev, a_dtype == TWM_F32, m, gated, (uint32_t)ctx->prefill_bm, splits, ctx->ws, ctx->ws_bytes, &sk),
@@ -1164,6 +1223,7 @@ static int gemm_common(twm_ctx *ctx, const twm_weight *w, const void *a_dev, int
             if (ssp > w->k_chunks) ssp = w->k_chunks;
             while (ssp > 1 && (size_t)ssp * m * n_ld * 4 > ctx->ws_bytes) ssp--;
             if (n_ld / sub.sub > ctx->n_counters) ssp = 1;
+            TWM_NEED(kCopyCol);
             HIP_TRY(launch_gemv4s(ctx->stream, v, a_dev, false, m, gated, ctx->ws, ctx->counters, sub.sub, sub.waves, ssp),
                     TWM_DEVICE_ERROR, "sub-tile gemv launch");
             return TWM_OK;
@@ -1176,6 +1236,7 @@ static int gemm_common(twm_ctx *ctx, const twm_weight *w, const void *a_dev, int
             DecodePlan plan = plan_gemv4(w->n_tiles, w->k_chunks, 1, ctx->force_waves, 0);
             while (plan.splits > 1 && (size_t)plan.splits * m * n_ld * 4 > ctx->ws_bytes) plan.splits--;
             if (w->n_tiles / plan.nt > ctx->n_counters) plan.splits = 1;
+            TWM_NEED(kCopyCol);
             HIP_TRY(launch_gemv4(ctx->stream, v, a_dev, false, m, gated, ctx->ws, ctx->counters, 1, plan.waves, plan.splits, swiglu_out),
                     TWM_DEVICE_ERROR, "gemv launch");
             return TWM_OK;
@@ -1186,6 +1247,7 @@ static int gemm_common(twm_ctx *ctx, const twm_weight *w, const void *a_dev, int
                             (m > 16 || (!splits && ((m > 8 && (n_ld / 64 > 128 || rows_f32)) ||
                                                     (rows_f32 && m > 4 && w->k_chunks <= 64))));
     if (ctx->force_kernel == 4 || batch_auto) {
+        TWM_NEED(kCopyTile);
         // batched decode with the activations shared through LDS, in 32-row blocks: from 17 rows on (the same exact
         // arithmetic as below 17 rows; option "batch_rounded" runs the f16-rounded weights of the prefill kernel
         // there), and from 9 rows on wide
@@ -1212,6 +1274,7 @@ static int gemm_common(twm_ctx *ctx, const twm_weight *w, const void *a_dev, int
         return TWM_OK;
     }
     if (ctx->force_kernel == 3 || (ctx->force_kernel == 0 && m > 4)) {
+        TWM_NEED(kCopyTile);
         // batched decode: 32-row blocks of the streaming kernel
         for (uint32_t m0 = 0; m0 < m; m0 += kMaxStreamM) {
             uint32_t mb = m - m0 < (uint32_t)kMaxStreamM ? m - m0 : (uint32_t)kMaxStreamM;
@@ -1225,25 +1288,21 @@ static int gemm_common(twm_ctx *ctx, const twm_weight *w, const void *a_dev, int
         }
         return TWM_OK;
     }
-    for (uint32_t m0 = 0; m0 < m; m0 += kMaxDecodeM) {
-        uint32_t mb = m - m0 < (uint32_t)kMaxDecodeM ? m - m0 : (uint32_t)kMaxDecodeM;
-        DecodePlan plan;
-        bool lane_col = mb <= 4 && ctx->force_kernel != 1;
-        if (swiglu_out && !lane_col) return api_fail(TWM_UNSUPPORTED_OP, "%s: the 16-column tile kernel has no gated store", who);
-        if (ctx->force_kernel == 2 && !lane_col) return api_fail(TWM_UNSUPPORTED_OP, "%s: the one-lane-per-column kernel takes M <= 4", who);
-        if (lane_col) plan = plan_gemv4(w->n_tiles, w->k_chunks, ctx->force_nt, ctx->force_waves, splits);
-        else plan = plan_decode(w->n_tiles, w->k_chunks, mb, ctx->force_nt, ctx->force_waves == 1 || ctx->force_waves == 2 ? 0 : ctx->force_waves, splits);
+    // M <= 4: one lane per column (whole 64-column tiles, or the sub-tile kernel where the planner takes it)
+    if (m > 4) return api_fail(TWM_UNSUPPORTED_OP, "%s: the one-lane-per-column kernel takes M <= 4", who);
+    {
+        const uint32_t mb = m;
+        TWM_NEED(kCopyCol);
+        DecodePlan plan = plan_gemv4(w->n_tiles, w->k_chunks, ctx->force_nt, ctx->force_waves, splits);
         // the scratch must hold splits x mb x n_ld partials and one counter per tile group
         while (plan.splits > 1 && (size_t)plan.splits * mb * n_ld * 4 > ctx->ws_bytes) plan.splits--;
         if (w->n_tiles / plan.nt > ctx->n_counters) plan.splits = 1;
-        OutSpec o = gated;   // (the one-lane-per-column kernel takes the gated output as its own argument)
-        for (uint32_t s = 0; s < o.count; s++) o.seg[s].ptr += (size_t)m0 * o.seg[s].width;
-        const char *a_blk = (const char *)a_dev + (size_t)m0 * a_row_bytes;
+        OutSpec o = gated;
         SubPlan sub = {0, 0};
-        if (lane_col && ctx->force_sub >= 16) {
+        if (ctx->force_sub >= 16) {
             sub.sub = (uint32_t)ctx->force_sub;
             sub.waves = ctx->force_sub_waves ? (uint32_t)ctx->force_sub_waves : ctx->force_waves ? (uint32_t)ctx->force_waves : 8;
-        } else if (lane_col && ctx->force_sub == 0 && !ctx->force_nt && !ctx->force_waves && !splits) {
+        } else if (ctx->force_sub == 0 && !ctx->force_nt && !ctx->force_waves && !splits) {
             // (an explicit nt, waves or split factor asks for the 64-column kernel's plan)
             sub = plan_gemv4_sub(n_ld / 64, w->k_chunks, mb, a_dtype == TWM_F32);
             // the gated store splits a sub-tile into a gate and an up half: 16 columns would read 128-byte runs
@@ -1255,17 +1314,14 @@ static int gemm_common(twm_ctx *ctx, const twm_weight *w, const void *a_dev, int
             if (ssp > w->k_chunks) ssp = w->k_chunks;
             while (ssp > 1 && (size_t)ssp * mb * n_ld * 4 > ctx->ws_bytes) ssp--;
             if (n_ld / sub.sub > ctx->n_counters) ssp = 1;
-            if (swiglu_out) o.swiglu = swiglu_out + (size_t)m0 * (w->n / 2);
-            HIP_TRY(launch_gemv4s(ctx->stream, v, a_blk, a_dtype == TWM_F32, mb, o, ctx->ws, ctx->counters, sub.sub, sub.waves, ssp),
+            HIP_TRY(launch_gemv4s(ctx->stream, v, a_dev, a_dtype == TWM_F32, mb, o, ctx->ws, ctx->counters, sub.sub, sub.waves, ssp),
                     TWM_DEVICE_ERROR, "sub-tile gemv launch");
-        } else if (lane_col)
-            HIP_TRY(launch_gemv4(ctx->stream, v, a_blk, a_dtype == TWM_F32, mb, o, ctx->ws, ctx->counters, plan.nt,
-                                 plan.waves, plan.splits, swiglu_out ? swiglu_out + (size_t)m0 * (w->n / 2) : nullptr),
+        } else
+            HIP_TRY(launch_gemv4(ctx->stream, v, a_dev, a_dtype == TWM_F32, mb, o, ctx->ws, ctx->counters, plan.nt,
+                                 plan.waves, plan.splits, swiglu_out),
                     TWM_DEVICE_ERROR, "gemv launch");
-        else
-            HIP_TRY(launch_decode(ctx->stream, v, a_blk, a_dtype == TWM_F32, mb, o, ctx->ws, ctx->counters, plan),
-                    TWM_DEVICE_ERROR, "gemm launch");
     }
+#undef TWM_NEED
     return TWM_OK;
 }
 
@@ -1348,26 +1404,13 @@ int twm_gemm_geglu(twm_ctx *ctx, const twm_weight *w, const void *a_dev, int a_d
 
 /* ---- expert banks (mixture-of-experts decode) ------------------------------------------------ */
 
-twm_bank *twm_bank_from_device(twm_ctx *ctx, const uint8_t *packed_base_dev, const uint16_t *scales_base_dev,
-                               size_t packed_bytes_per_expert, size_t scales_per_expert, uint32_t k, uint32_t n,
-                               uint32_t num_experts, int pair_gate_up)
+// The bank of both constructors: expert x lies at packed_base + packed_off[x] (bytes) and scales_base + scales_off[x]
+// (f16 elements); the offsets have been checked by the caller.
+static twm_bank *bank_build(twm_ctx *ctx, const char *who, const uint8_t *packed_base_dev, const uint16_t *scales_base_dev,
+                            const std::vector<size_t> &packed_off, const std::vector<size_t> &scales_off, uint32_t k, uint32_t n,
+                            uint32_t num_experts, int pair_gate_up)
 {
-    if (!ctx) { api_fail(TWM_INVALID_HANDLE, "twm_bank_from_device: null context"); return nullptr; }
-    if (ctx->capturing) { api_fail(TWM_UNSUPPORTED_OP, "twm_bank_from_device: not allowed inside a graph capture"); return nullptr; }
-    if (check_kn("twm_bank_from_device", k, n)) return nullptr;
-    if (pair_gate_up && n % (2 * kPairWidth) != 0) {
-        api_fail(TWM_SHAPE_ERROR, "twm_bank_from_device: a paired gate/up bank needs N %% %u == 0, got %u", 2 * kPairWidth, n);
-        return nullptr;
-    }
-    size_t groups = k / 32;
-    if (packed_bytes_per_expert < groups * n * 16 || scales_per_expert < groups * n || packed_bytes_per_expert % 4 != 0) {
-        api_fail(TWM_SHAPE_ERROR, "twm_bank_from_device: per-expert strides (%zu bytes, %zu scales) do not hold a %u x %u matrix",
-             packed_bytes_per_expert, scales_per_expert, k, n);
-        return nullptr;
-    }
-    bool empty = (uint64_t)k * n * num_experts == 0;
-    if (!empty && (!packed_base_dev || !scales_base_dev)) { api_fail(TWM_INVALID_HANDLE, "twm_bank_from_device: null pointer"); return nullptr; }
-    if (((uintptr_t)packed_base_dev & 3) != 0) { api_fail(TWM_SHAPE_ERROR, "twm_bank_from_device: packed must be 4-byte aligned"); return nullptr; }
+    const size_t groups = k / 32;
     twm_bank *b = new (std::nothrow) twm_bank();
     if (!b) { api_fail(TWM_MEMORY_ERROR, "twm_bank: out of host memory"); return nullptr; }
     b->ctx = ctx;
@@ -1380,7 +1423,7 @@ twm_bank *twm_bank_from_device(twm_ctx *ctx, const uint8_t *packed_base_dev, con
     b->expert_bytes = (size_t)(b->n_pad / 64) * b->k_chunks * kColBlockBytes;
     b->bytes = b->expert_bytes * num_experts;
     b->cq = nullptr;
-    if (empty || b->bytes == 0) return b;
+    if ((uint64_t)k * n * num_experts == 0 || b->bytes == 0) return b;
     hipError_t e = hipMalloc(&b->cq, b->bytes);
     if (e != hipSuccess) {
         api_fail(TWM_MEMORY_ERROR, "twm_bank: hipMalloc(%zu): %s", b->bytes, hipGetErrorString(e));
@@ -1388,17 +1431,76 @@ twm_bank *twm_bank_from_device(twm_ctx *ctx, const uint8_t *packed_base_dev, con
         return nullptr;
     }
     for (uint32_t x = 0; x < num_experts && e == hipSuccess; x++)
-        e = launch_repack_col(ctx->stream, packed_base_dev + (size_t)x * packed_bytes_per_expert,
-                              scales_base_dev + (size_t)x * scales_per_expert, k, n, (char *)b->cq + (size_t)x * b->expert_bytes,
-                              b->n_pad, b->k_chunks, pair_gate_up ? n / 2 : 0);
+        e = launch_repack_col(ctx->stream, packed_base_dev + packed_off[x], scales_base_dev + scales_off[x], k, n,
+                              (char *)b->cq + (size_t)x * b->expert_bytes, b->n_pad, b->k_chunks, pair_gate_up ? n / 2 : 0);
     if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
     if (e != hipSuccess) {
-        api_fail(TWM_DEVICE_ERROR, "twm_bank_from_device: repack: %s", hipGetErrorString(e));
+        api_fail(TWM_DEVICE_ERROR, "%s: repack: %s", who, hipGetErrorString(e));
         (void)hipFree(b->cq);
         delete b;
         return nullptr;
     }
     return b;
+}
+
+static bool bank_args_ok(twm_ctx *ctx, const char *who, const uint8_t *packed_base_dev, const uint16_t *scales_base_dev, uint32_t k,
+                         uint32_t n, uint32_t num_experts, int pair_gate_up)
+{
+    if (!ctx) { api_fail(TWM_INVALID_HANDLE, "%s: null context", who); return false; }
+    if (ctx->capturing) { api_fail(TWM_UNSUPPORTED_OP, "%s: not allowed inside a graph capture", who); return false; }
+    if (check_kn(who, k, n)) return false;
+    if (pair_gate_up && n % (2 * kPairWidth) != 0) {
+        api_fail(TWM_SHAPE_ERROR, "%s: a paired gate/up bank needs N %% %u == 0, got %u", who, 2 * kPairWidth, n);
+        return false;
+    }
+    const bool empty = (uint64_t)k * n * num_experts == 0;
+    if (!empty && (!packed_base_dev || !scales_base_dev)) { api_fail(TWM_INVALID_HANDLE, "%s: null pointer", who); return false; }
+    if (((uintptr_t)packed_base_dev & 3) != 0) { api_fail(TWM_SHAPE_ERROR, "%s: packed must be 4-byte aligned", who); return false; }
+    return true;
+}
+
+twm_bank *twm_bank_from_device(twm_ctx *ctx, const uint8_t *packed_base_dev, const uint16_t *scales_base_dev,
+                               size_t packed_bytes_per_expert, size_t scales_per_expert, uint32_t k, uint32_t n,
+                               uint32_t num_experts, int pair_gate_up)
+{
+    if (!bank_args_ok(ctx, "twm_bank_from_device", packed_base_dev, scales_base_dev, k, n, num_experts, pair_gate_up)) return nullptr;
+    size_t groups = k / 32;
+    if (packed_bytes_per_expert < groups * n * 16 || scales_per_expert < groups * n || packed_bytes_per_expert % 4 != 0) {
+        api_fail(TWM_SHAPE_ERROR, "twm_bank_from_device: per-expert strides (%zu bytes, %zu scales) do not hold a %u x %u matrix",
+             packed_bytes_per_expert, scales_per_expert, k, n);
+        return nullptr;
+    }
+    std::vector<size_t> po(num_experts), so(num_experts);
+    for (uint32_t x = 0; x < num_experts; x++) {
+        po[x] = (size_t)x * packed_bytes_per_expert;
+        so[x] = (size_t)x * scales_per_expert;
+    }
+    return bank_build(ctx, "twm_bank_from_device", packed_base_dev, scales_base_dev, po, so, k, n, num_experts, pair_gate_up);
+}
+
+twm_bank *twm_bank_from_device_offsets(twm_ctx *ctx, const uint8_t *packed_base_dev, const uint16_t *scales_base_dev,
+                                       const uint32_t *packed_offsets_dev, const uint32_t *scales_offsets_dev, uint32_t k,
+                                       uint32_t n, uint32_t num_experts, int pair_gate_up)
+{
+    const char *who = "twm_bank_from_device_offsets";
+    if (!bank_args_ok(ctx, who, packed_base_dev, scales_base_dev, k, n, num_experts, pair_gate_up)) return nullptr;
+    if (num_experts != 0 && (!packed_offsets_dev || !scales_offsets_dev)) { api_fail(TWM_INVALID_HANDLE, "%s: null offset table", who); return nullptr; }
+    // the tables are read once, here: the bank holds its own copy of every expert
+    std::vector<uint32_t> po32(num_experts), so32(num_experts);
+    if (num_experts != 0) {
+        hipError_t e = hipStreamSynchronize(ctx->stream);
+        if (e == hipSuccess) e = hipMemcpy(po32.data(), packed_offsets_dev, (size_t)num_experts * 4, hipMemcpyDeviceToHost);
+        if (e == hipSuccess) e = hipMemcpy(so32.data(), scales_offsets_dev, (size_t)num_experts * 4, hipMemcpyDeviceToHost);
+        if (e != hipSuccess) { api_fail(TWM_DEVICE_ERROR, "%s: reading the offset tables: %s", who, hipGetErrorString(e)); return nullptr; }
+    }
+    std::vector<size_t> po(num_experts), so(num_experts);
+    for (uint32_t x = 0; x < num_experts; x++) {
+        // the reference's kernel reads a record as four 32-bit words (quantize_indirect.rs:216-218): 4-byte alignment
+        if (po32[x] % 4 != 0) { api_fail(TWM_SHAPE_ERROR, "%s: packed offset of expert %u (%u) is not 4-byte aligned", who, x, po32[x]); return nullptr; }
+        po[x] = po32[x];
+        so[x] = so32[x];
+    }
+    return bank_build(ctx, who, packed_base_dev, scales_base_dev, po, so, k, n, num_experts, pair_gate_up);
 }
 
 void twm_bank_destroy(twm_bank *b)

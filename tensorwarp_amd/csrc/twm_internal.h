@@ -19,7 +19,6 @@ constexpr int kTileN = 16;
 constexpr int kChunkGroups = 4;
 constexpr int kNPadTo = 64;      // N is padded to a multiple of this, so 1, 2 or 4 tiles per block divide
 constexpr int kMaxSegs = 4;
-constexpr int kMaxDecodeM = 16;     // rows per launch of the tile kernel (one 16-row MFMA block)
 constexpr int kMaxStreamM = 32;     // rows per launch of the batched-decode streaming kernel
 constexpr uint32_t kColBlockBytes = 4608;  // column-lane copy: 4 x 1024 B of nibbles + 512 B of scales per (tile, chunk)
 
@@ -127,6 +126,9 @@ hipError_t launch_repack(hipStream_t s, const uint8_t *packed, const uint16_t *s
 hipError_t launch_weight_dequant_f16(hipStream_t s, const WeightView &w, uint16_t *out_kn);
 // pair_ffn != 0: the source columns are [gate | up] halves of width pair_ffn and the copy is written in the
 // paired order (32 gate, 32 up, ...)
+// one repacked copy from the other (n_tiles is a multiple of 4)
+hipError_t launch_col_to_tile(hipStream_t s, const void *cq, uint32_t n_tiles, uint32_t k_chunks, void *qw, void *sc);
+hipError_t launch_tile_to_col(hipStream_t s, const void *qw, const void *sc, uint32_t n_tiles, uint32_t k_chunks, void *cq);
 hipError_t launch_repack_col(hipStream_t s, const uint8_t *packed, const uint16_t *scales, uint32_t k, uint32_t n,
                              void *cq, uint32_t n_pad, uint32_t k_chunks, uint32_t pair_ffn = 0);
 hipError_t launch_weight_dequant_f16_col(hipStream_t s, const WeightView &w, uint16_t *out_kn);
@@ -177,7 +179,5 @@ hipError_t launch_bank_gemv(hipStream_t s, const BankView &b, const void *a, boo
                             const float *ids, uint32_t slots, int act, float *out, int force_sub = 0, int force_waves = 0);
 hipError_t launch_bank_down_axpy(hipStream_t s, const BankView &b, const void *a_all, bool a_f32, const float *ids,
                                  const float *weights, uint32_t slots, float *accum, int force_sub = 0, int force_waves = 0);
-hipError_t launch_decode(hipStream_t s, const WeightView &w, const void *a, bool a_f32, uint32_t m, const OutSpec &out,
-                         float *ws, unsigned *counters, DecodePlan plan);
 
 }  // namespace twm

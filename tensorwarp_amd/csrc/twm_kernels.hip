@@ -6,9 +6,9 @@
 //   quantizer .................. :414-474, crates/loader/src/gemma_moe_q4.rs:218-254
 //   reorder / fuse ............. :912-956, :1018-1063
 //   split_qkv / split_gate_up .. crates/kernels/src/ops.rs:2255-2297
-// This file holds the format operations, the GEMV on the reference layout and the repack into
-// the wave tile order; the MFMA decode kernel that streams the repacked weights is in
-// twm_decode.hip.
+// This file holds the format operations, the GEMV on the reference layout and the repacks into
+// the two streaming orders; the MFMA kernels that stream the repacked weights are in twm_gemv4*.hip,
+// twm_stream.hip, twm_batch.hip and twm_prefill.hip.
 #include "twm_device.h"
 
 namespace twm {
@@ -705,6 +705,64 @@ hipError_t launch_weight_dequant_f16_col(hipStream_t s, const WeightView &w, uin
     if (total == 0) return hipSuccess;
     hipLaunchKernelGGL(k_weight_dequant_f16_col, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s,
                        (const char *)w.cq, w.k, w.n, w.k_chunks, out_kn);
+    return hipGetLastError();
+}
+
+// ---------------------------------------------------------------------------------
+// One repacked copy from the other.  Both hold every 32-bit word of the reference's records with the same nibble
+// permutation, so the conversion moves words: word kb of column c's record of group g is
+//   tile copy:        qw[(kc * n_tiles + c / 16) * 64 + kb * 16 + c % 16][g % 4]
+//   column-lane copy: block (c / 64, kc), group row g % 4, lane c % 64, word kb
+// ---------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void k_col_to_tile(const char *__restrict__ cw, uint32_t n_tiles, uint32_t k_chunks,
+                                                      uint4v *__restrict__ qw, uint2v *__restrict__ sc)
+{
+    size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;  // (kc * n_tiles + nt) * 64 + lane
+    if (idx >= (size_t)n_tiles * k_chunks * 64) return;
+    const uint32_t lane = (uint32_t)(idx & 63), c = lane & 15, kb = lane >> 4;
+    const size_t tile = idx >> 6;
+    const uint32_t nt = (uint32_t)(tile % n_tiles), kc = (uint32_t)(tile / n_tiles);
+    const char *blk = cw + ((size_t)(nt / 4) * k_chunks + kc) * kColBlockBytes;
+    const uint32_t col = (nt % 4) * 16 + c;
+    uint4v o;
+#pragma unroll
+    for (int i = 0; i < 4; i++) o[i] = *(const uint32_t *)(blk + i * 1024u + col * 16u + kb * 4u);
+    qw[idx] = o;
+    if (kb == 0) sc[tile * 16 + c] = *(const uint2v *)(blk + 4096u + col * 8u);
+}
+
+__global__ __launch_bounds__(256) void k_tile_to_col(const uint32_t *__restrict__ qw, const uint2v *__restrict__ sc,
+                                                      uint32_t n_tiles, uint32_t k_chunks, char *__restrict__ cw)
+{
+    size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;  // ((tile64 * k_chunks + kc) * 4 + g) * 64 + lane
+    if (idx >= (size_t)(n_tiles / 4) * k_chunks * 256) return;
+    const uint32_t lane = (uint32_t)(idx & 63), gi = (uint32_t)((idx >> 6) & 3);
+    const size_t blk = idx >> 8;
+    const uint32_t kc = (uint32_t)(blk % k_chunks), tile64 = (uint32_t)(blk / k_chunks);
+    const size_t tile = (size_t)kc * n_tiles + tile64 * 4 + lane / 16;
+    uint4v o;
+#pragma unroll
+    for (int kb = 0; kb < 4; kb++) o[kb] = qw[(tile * 64 + kb * 16 + lane % 16) * 4 + gi];
+    char *base = cw + blk * kColBlockBytes;
+    *(uint4v *)(base + gi * 1024u + lane * 16u) = o;
+    if (gi == 0) *(uint2v *)(base + 4096u + lane * 8u) = sc[tile * 16 + lane % 16];
+}
+
+hipError_t launch_col_to_tile(hipStream_t s, const void *cq, uint32_t n_tiles, uint32_t k_chunks, void *qw, void *sc)
+{
+    size_t total = (size_t)n_tiles * k_chunks * 64;
+    if (total == 0) return hipSuccess;
+    hipLaunchKernelGGL(k_col_to_tile, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, (const char *)cq, n_tiles,
+                       k_chunks, (uint4v *)qw, (uint2v *)sc);
+    return hipGetLastError();
+}
+
+hipError_t launch_tile_to_col(hipStream_t s, const void *qw, const void *sc, uint32_t n_tiles, uint32_t k_chunks, void *cq)
+{
+    size_t total = (size_t)(n_tiles / 4) * k_chunks * 256;
+    if (total == 0) return hipSuccess;
+    hipLaunchKernelGGL(k_tile_to_col, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, (const uint32_t *)qw,
+                       (const uint2v *)sc, n_tiles, k_chunks, (char *)cq);
     return hipGetLastError();
 }
 

@@ -296,6 +296,19 @@ class MarlinWeight:
     def nbytes(self):
         return self.device._l.twm_weight_bytes(self.handle)
 
+    COPY_TILES, COPY_COLUMN_LANE = 1, 2
+
+    @property
+    def copies(self):
+        """Mask of the repacked orders the handle holds now (COPY_TILES | COPY_COLUMN_LANE)."""
+        return self.device._l.twm_weight_copies(self.handle)
+
+    def ensure(self, copies):
+        _check(self.device._l.twm_weight_ensure(self.device.handle, self.handle, copies))
+
+    def drop(self, copies):
+        _check(self.device._l.twm_weight_drop(self.device.handle, self.handle, copies))
+
     def export_blob(self):
         """The repacked weight as a uint8 array (header + device bytes) for an on-disk cache."""
         size = self.device._l.twm_weight_blob_bytes(self.handle)
@@ -407,6 +420,17 @@ class ExpertBank:
                     pair_gate_up=False):
         h = device._l.twm_bank_from_device(device.handle, packed_buf.ptr, scales_buf.ptr, packed_bytes_per_expert,
                                            scales_per_expert, k, n, num_experts, int(pair_gate_up))
+        if not h:
+            raise DeviceError(_lib.SHAPE_ERROR, device._l.twm_last_error().decode())
+        return cls(device, h, k, n, num_experts, bool(pair_gate_up))
+
+    @classmethod
+    def from_device_offsets(cls, device, packed_buf, packed_offsets, scales_buf, scales_offsets, k, n, num_experts,
+                            pair_gate_up=False):
+        """Experts at packed_buf + packed_offsets[e] (bytes) and scales_buf + scales_offsets[e] (elements), u32 device
+        tables: the arguments of gemm_tw_marlin_m1_indirect (quantize_indirect.rs:228-253)."""
+        h = device._l.twm_bank_from_device_offsets(device.handle, packed_buf.ptr, scales_buf.ptr, packed_offsets.ptr,
+                                                   scales_offsets.ptr, k, n, num_experts, int(pair_gate_up))
         if not h:
             raise DeviceError(_lib.SHAPE_ERROR, device._l.twm_last_error().decode())
         return cls(device, h, k, n, num_experts, bool(pair_gate_up))

@@ -253,13 +253,6 @@ def test_gemm_swiglu_batched_and_prefill_rows(dev, m, splits):
     col = (j // 32) * 64 + j % 32
     got = tmp.to_host().reshape(m, 2 * ffn)
     assert rel_err(got[:, col], tg) < bar and rel_err(got[:, col + 32], tu) < bar
-    try:
-        dev.set_option("kernel", 1)                      # the 16-column tile kernel has no gated store
-        if m < 33:
-            with pytest.raises(T.DeviceError):
-                T.gemm_swiglu(dev, w, ad, m, out, splits)
-    finally:
-        dev.set_option("kernel", 0)
     w.free()
 
 
@@ -579,15 +572,15 @@ def test_batched_decode_7b_shapes(dev, m, k, n):
 
 
 def test_split_k_choice_does_not_change_the_result(dev):
-    # both decode kernels (1 = 16-column tiles, 2 = one lane per column), every tile width, many split factors
+    # the one-lane-per-column kernel on whole tiles, every tile width, many split factors
     k, n = 4096, 4096
     packed, scales, a16 = synth(k, n, 1, 31)
     w = T.MarlinWeight.upload(dev, packed, scales, k, n)
     truth = O.gemm_f64(f16_as_f32(a16), packed, scales, 1, k, n)
     try:
-        for kernel in (1, 2):
+        for kernel in (2,):
             dev.set_option("kernel", kernel)
-            for nt in ((1, 2) if kernel == 2 else (1, 2, 4)):
+            for nt in (1, 2):
                 dev.set_option("nt", nt)
                 for splits in (1, 2, 5, 8, 32):
                     got = run_gemm(dev, w, a16, 1, n, splits)
@@ -789,7 +782,7 @@ def test_split_factors_that_do_not_divide_the_k_chunks(dev):
     w = T.MarlinWeight.upload(dev, packed, scales, k, n)
     truth = O.gemm_f64(f16_as_f32(a16), packed, scales, 2, k, n)
     try:
-        for kernel in (1, 2):
+        for kernel in (2,):
             dev.set_option("kernel", kernel)
             for splits in (5, 8, 9, 11, 12, 13, 15, 20, 27, 28):
                 assert rel_err(run_gemm(dev, w, a16, 2, n, splits), truth) < TIGHT, (kernel, splits)
@@ -807,8 +800,8 @@ def test_decode_kernels_rows_and_f32_activations(dev, m):
     truth = O.gemm_f64(f16_as_f32(a16), packed, scales, m, k, n)
     try:
         dev.set_option("prefill_min_m", 1 << 30)
-        # 1 = 16-column tile kernel (16-row blocks), 2 = one lane per column (M <= 4), 3 = streaming kernel (32-row blocks)
-        for kernel in ((1, 2, 3) if m <= 4 else (1, 3)):
+        # 2 = one lane per column (M <= 4), 3 = streaming kernel (32-row blocks)
+        for kernel in ((2, 3) if m <= 4 else (3,)):
             dev.set_option("kernel", kernel)
             for splits in (0, 1, 2, 3):
                 for a_f32 in (False, True):
@@ -1001,6 +994,64 @@ def test_empty_inputs(dev):
     T.gemm(dev, w0, a, 1, c8)        # K == 0: the empty sum
     assert np.all(c8.to_host() == 0)
     w0.free()
+
+
+def test_weight_handle_with_one_copy_builds_the_other_on_demand(dev):
+    # A decode-only or prefill-only handle holds 4.5 bits per weight; the other order is built from it, word for word,
+    # at the first call that needs it: results and Q4 unpack equal those of a handle made with both copies.
+    k, n = 640, 200
+    packed, scales = O.synth_packed(k, n, 990), O.synth_scales(k, n, 991)
+    both = T.MarlinWeight.upload(dev, packed, scales, k, n)
+    assert both.copies == 3
+    one_copy = both.nbytes // 2
+    a1 = T.GpuTensor.from_host(dev, O.synth_act_f16(1, k, 992), "f16")
+    a8 = T.GpuTensor.from_host(dev, O.synth_act_f16(8, k, 993), "f16")
+    a40 = T.GpuTensor.from_host(dev, O.synth_act_f16(40, k, 994), "f16")
+    def run(w):
+        outs = []
+        for a, m in ((a1, 1), (a8, 8), (a40, 40)):
+            c = T.GpuTensor.zeros(dev, (m, n), "f32")
+            T.gemm(dev, w, a, m, c)
+            outs.append(c.to_host())
+        return outs
+    want = run(both)
+    want_deq = both.dequant_f16().to_host()
+    for first, label in ((T.MarlinWeight.COPY_COLUMN_LANE, "column-lane first"), (T.MarlinWeight.COPY_TILES, "tiles first")):
+        dev.set_option("weight_copies", first)
+        w = T.MarlinWeight.upload(dev, packed, scales, k, n)
+        dev.set_option("weight_copies", 0)
+        assert w.copies == first and w.nbytes == one_copy, label
+        # a capture may not allocate: the call that needs the missing copy is refused, and says what to do
+        m_other, a_other = (40, a40) if first == T.MarlinWeight.COPY_COLUMN_LANE else (1, a1)
+        c = T.GpuTensor.zeros(dev, (m_other, n), "f32")
+        with pytest.raises(T.DeviceError, match="twm_weight_ensure"):
+            T.GraphCapture.record_with_device(dev, lambda: T.gemm(dev, w, a_other, m_other, c))
+        assert w.copies == first
+        # the export of a one-copy handle is half as long and comes back as it was
+        blob = w.export_blob()
+        assert blob.size == 64 + one_copy
+        w_back = T.MarlinWeight.import_blob(dev, blob)
+        assert w_back.copies == first
+        got = run(w)
+        assert w.copies == 3 and w.nbytes == 2 * one_copy, label
+        for g, t in zip(got, want):
+            assert np.array_equal(g, t), label
+        for src in (0, 1):
+            dev.set_option("dequant_src", src)
+            assert np.array_equal(w.dequant_f16().to_host(), want_deq), label
+            assert np.array_equal(w_back.dequant_f16().to_host(), want_deq), label
+        dev.set_option("dequant_src", 0)
+        for g, t in zip(run(w_back), want):
+            assert np.array_equal(g, t), label
+        # drop one again: the handle is back to one copy, and the last copy cannot be dropped
+        w.drop(first)
+        assert w.copies == 3 - first and w.nbytes == one_copy
+        with pytest.raises(T.DeviceError):
+            w.drop(3 - first)
+        for g, t in zip(run(w), want):
+            assert np.array_equal(g, t), label
+        w.free(); w_back.free()
+    both.free()
 
 
 def test_repacked_weight_blob_round_trip_through_a_warp_file(dev, tmp_path):
@@ -1216,6 +1267,45 @@ def test_bank_ignores_ids_outside_the_bank(dev):
     assert not got[1].any() and not got[2].any() and not got[4].any()
     assert rel_err(got[[0, 3]], O.bank_gemv_f64(a32, packed, scales, [1, 2], k, n)) < TIGHT
     bank.free()
+
+
+def test_bank_from_offset_tables_with_unequal_spacing(dev):
+    # gemm_tw_marlin_m1_indirect's addressing (quantize_indirect.rs:196-197): expert e at packed_base + packed_offsets[e]
+    # bytes and scales_base + scales_offsets[e] elements, the experts in any order and with gaps of any size
+    k, n, experts = 256, 96, 4
+    G = k // 32
+    packed = [O.synth_packed(k, n, 1080 + 2 * e) for e in range(experts)]
+    scales = [O.synth_scales(k, n, 1081 + 2 * e) for e in range(experts)]
+    order, gaps_p, gaps_s = [2, 0, 3, 1], [4, 260, 0, 12], [1, 0, 7, 33]
+    pbuf, sbuf = np.full(4 * (G * n * 16 + 300), 0xEE, np.uint8), np.full(4 * (G * n + 50), 0x7BFF, np.uint16)
+    poff, soff = np.zeros(experts, np.uint32), np.zeros(experts, np.uint32)
+    pp = ss = 0
+    for e, gp, gs in zip(order, gaps_p, gaps_s):
+        pp, ss = pp + gp, ss + gs
+        poff[e], soff[e] = pp, ss
+        pbuf[pp:pp + G * n * 16] = packed[e]
+        sbuf[ss:ss + G * n] = scales[e]
+        pp, ss = pp + G * n * 16, ss + G * n
+    pd, sd = T.GpuTensor.from_host(dev, pbuf), T.GpuTensor.from_host(dev, sbuf, "f16")
+    pod, sod = T.GpuTensor.from_host(dev, poff.view(np.int32), "i32"), T.GpuTensor.from_host(dev, soff.view(np.int32), "i32")
+    bank = T.ExpertBank.from_device_offsets(dev, pd, pod, sd, sod, k, n, experts)
+    ids = [3, 0, 2, 1, 3]
+    a32 = f16_as_f32(O.synth_act_f16(1, k, 1090)).reshape(1, k)
+    out = T.GpuTensor.zeros(dev, (len(ids), n), "f32")
+    T.batched_marlin_gate_up(dev, T.GpuTensor.from_host(dev, a32), bank, T.GpuTensor.from_host(dev, np.array(ids, np.float32)), out, len(ids))
+    assert rel_err(out.to_host().reshape(len(ids), n), O.bank_gemv_f64(a32, packed, scales, ids, k, n)) < TIGHT
+    # the bank equals the one built from equal strides, byte for byte in its results
+    bank2, _, _ = make_bank(dev, k, n, 1, 1080)
+    o1, o2 = T.GpuTensor.zeros(dev, (1, n), "f32"), T.GpuTensor.zeros(dev, (1, n), "f32")
+    zero = T.GpuTensor.from_host(dev, np.zeros(1, np.float32))
+    T.batched_marlin_gate_up(dev, T.GpuTensor.from_host(dev, a32), bank, zero, o1, 1)
+    T.batched_marlin_gate_up(dev, T.GpuTensor.from_host(dev, a32), bank2, zero, o2, 1)
+    assert np.array_equal(o1.to_host(), o2.to_host())
+    # a record offset that is not a multiple of four bytes is the reference kernel's own limit (it reads 32-bit words)
+    poff_bad = poff.copy(); poff_bad[1] += 2
+    with pytest.raises(T.DeviceError):
+        T.ExpertBank.from_device_offsets(dev, pd, T.GpuTensor.from_host(dev, poff_bad.view(np.int32), "i32"), sd, sod, k, n, experts)
+    bank.free(); bank2.free()
 
 
 # ---------------------------------------------------------------- fused projections
