@@ -54,11 +54,12 @@ struct Chunk4 {
     uint2v sc[NT];     // four f16 scales
     uint4v a[RG];      // activations: row 4*rg + lane%4, k-piece lane/4 (8 halves)
     uint4v a_lo;       // f32 activations only: the f16 residuals a - f16(a) of the same eight values
+    float a_inv[4];    // f32 activations only: what the sums of the four A rows are multiplied by (f32_terms_range)
 };
 
 // f32 activations enter the f16 MFMA as two terms, a = f16(a) + f16(a - f16(a)) (about 22 significant bits;
 // the subtraction is exact), so that a caller's f32 values are not silently cut to 11 bits.  Values beyond the
-// f16 range (|a| > 65504) are not supported by this path.
+// f16 range are scaled into it first, a chunk of a wave at a time (f32_terms_range).
 __device__ __forceinline__ void split_f32x8(const float (&v)[8], uint4v &hi, uint4v &lo)
 {
     union { half8 h; uint4v u; } ch, cl;
@@ -70,6 +71,37 @@ __device__ __forceinline__ void split_f32x8(const float (&v)[8], uint4v &hi, uin
     }
     hi = ch.u;
     lo = cl.u;
+}
+
+// f32 activations beyond the f16 range.  The wave's values of one chunk (or pass) are about to be taken as f16 terms.
+// Lanes with the same lane % 4 hold the same activation row (one row of the MFMA's A operand); when any value of
+// the wave exceeds the largest f16, every such row scales its values by a power of two of its own that brings its
+// largest below 2^15 (exact), and inv[i] is what the sums of A row i are multiplied by afterwards (exact as well): the
+// results come out as with unbounded terms.  In range every factor is 1 and nothing is touched, at the price of a
+// maximum over the lane's values and one vote per call.  (Infinities and NaNs stay what they are.)
+template <int NV>
+__device__ __forceinline__ void f32_terms_range(float (&v)[NV], float (&inv)[4])
+{
+    float m = 0.f;
+#pragma unroll
+    for (int i = 0; i < NV; i++) m = fmaxf(m, fabsf(v[i]));
+#pragma unroll
+    for (int i = 0; i < 4; i++) inv[i] = 1.f;
+    if (__builtin_amdgcn_ballot_w64(!(m <= 65000.f)) == 0) return;
+    if (!(m == m)) m = __builtin_inff();  // (fmaxf drops a NaN; the vote saw it through the negated comparison)
+#pragma unroll
+    for (int off = 32; off >= 4; off >>= 1) m = fmaxf(m, __shfl_xor(m, off, 64));   // over the lanes of this row
+    float mine = 1.f;
+    if (m > 16384.f) {
+        const uint32_t e = (__float_as_uint(m) >> 23) & 0xFFu;       // biased exponent of the row's largest value, >= 141
+        const float down = __uint_as_float((254u + 14u - e) << 23);   // 2^(14 - (e - 127))
+#pragma unroll
+        for (int i = 0; i < NV; i++) v[i] *= down;
+        mine = __uint_as_float((e - 14u) << 23);                     // 2^((e - 127) - 14)
+    }
+    const int quad = (int)(__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u)) & ~3u);
+#pragma unroll
+    for (int i = 0; i < 4; i++) inv[i] = __shfl(mine, quad + i, 64);
 }
 
 template <int P>
@@ -110,7 +142,8 @@ __device__ __forceinline__ void gemv4_load_chunk(Chunk4<NT, RG> &r, const char *
     if (AF32) {
         const float4 *p = (const float4 *)((const float *)a_any + (size_t)arow * k + k0);
         float4 x = p[0], y = p[1];
-        const float v[8] = {x.x, x.y, x.z, x.w, y.x, y.y, y.z, y.w};
+        float v[8] = {x.x, x.y, x.z, x.w, y.x, y.y, y.z, y.w};
+        f32_terms_range(v, r.a_inv);
         split_f32x8(v, r.a[0], r.a_lo);
         if (TERMS == kTermsRowPacked) {
 #pragma unroll
@@ -141,23 +174,25 @@ __device__ __forceinline__ void gemv4_load_chunk_ref(Chunk4<NT, 1> &r, const cha
     for (int t = 0; t < NT; t++) {
         const uint32_t col = (tile0 + t) * 64u + lane;
         const uint32_t colc = col < n ? col : n - 1u;
-        uint32_t sb[4];
+        uint32_t sb[4], keep[4];
 #pragma unroll
         for (int g = 0; g < 4; g++) {
             const uint32_t gg = kc * 4u + g;
             const uint32_t ggc = gg < groups ? gg : groups - 1u;
             const size_t idx = (size_t)ggc * n + colc;
             r.wq[t][g] = ld_once((const uint4v *)(packed + idx * 16u));
-            const uint32_t sbits = ld_once(scales + idx);
-            sb[g] = (gg < groups && col < n) ? sbits : 0u;
+            sb[g] = ld_once(scales + idx);
+            keep[g] = (gg < groups && col < n) ? 0xFFFFu : 0u;
         }
-        r.sc[t] = uint2v{sb[0] | (sb[1] << 16), sb[2] | (sb[3] << 16)};
+        // (dead groups masked after the packing: a select on a freshly loaded value becomes a branch around the load)
+        r.sc[t] = uint2v{(sb[0] | (sb[1] << 16)) & (keep[0] | (keep[1] << 16)), (sb[2] | (sb[3] << 16)) & (keep[2] | (keep[3] << 16))};
     }
     uint32_t k0 = kc * 128u + apiece;
     if (k0 > k - 8u) k0 = k - 8u;
     const float4 *p = (const float4 *)(a + k0);
     float4 x = p[0], y = p[1];
-    const float v[8] = {x.x, y.x, x.y, y.y, x.z, y.z, x.w, y.w};
+    float v[8] = {x.x, y.x, x.y, y.y, x.z, y.z, x.w, y.w};
+    f32_terms_range(v, r.a_inv);
     split_f32x8(v, r.a[0], r.a_lo);
 #pragma unroll
     for (int i = 0; i < 4; i++) r.a[0][i] = lane_is_lo ? r.a_lo[i] : r.a[0][i];  // one row: row-packed terms
@@ -200,10 +235,12 @@ __device__ __forceinline__ void gemv4_compute_chunk(const Chunk4<NT, (RL + 3) / 
             if (g == 2) { TWM_PIECE(0, 8) TWM_PIECE(1, 9) TWM_PIECE(2, 10) TWM_PIECE(3, 11) }
             if (g == 3) { TWM_PIECE(0, 12) TWM_PIECE(1, 13) TWM_PIECE(2, 14) TWM_PIECE(3, 15) }
 #undef TWM_PIECE
-            float s = (float)sv.h[g];
+            const float s = (float)sv.h[g];
 #pragma unroll
             for (int rr = 0; rr < RL; rr++) {
-                if (TERMS == kTermsRowPacked) acc[t][rr] = fmaf(d[0][2 * rr] + d[0][2 * rr + 1], s, acc[t][rr]);
+                // (a_inv: 1 unless the f32 activations of that row were scaled into the f16 range)
+                if (TERMS == kTermsRowPacked) acc[t][rr] = fmaf(d[0][2 * rr] + d[0][2 * rr + 1], s * r.a_inv[2 * rr], acc[t][rr]);
+                else if (TERMS == kTermsTwoPasses) acc[t][rr] = fmaf(d[0][rr], s * r.a_inv[rr], acc[t][rr]);
                 else acc[t][rr] = fmaf(d[rr / 4][rr % 4], s, acc[t][rr]);
             }
         }
@@ -221,6 +258,7 @@ struct ChunkS {
     uint2v sc;                    // four f16 scales
     uint4v a[RG][64 / SUB];       // activations: row 4*rg + (lane % SUB) % 4, piece (lane % SUB) / 4 of every 2*SUB-wide slice
     uint4v a_lo[64 / SUB];        // f32 activations as two passes: the residual terms
+    float a_inv[4];               // f32 activations: what the sums of the four A rows are multiplied by (f32_terms_range)
     bool live;                    // false: a chunk past the k-range, replayed from a valid one; its scales count as 0
 };
 
@@ -230,6 +268,43 @@ __device__ __forceinline__ float4v mfma_sub(half4v a, half4v b, float4v c)
     static_assert(SUB == 32 || SUB == 16, "sub-tiles are 32 or 16 columns wide");
     constexpr int CBSZ = SUB == 32 ? 3 : 2;
     return __builtin_amdgcn_mfma_f32_4x4x4f16(a, b, c, CBSZ, P, 0);
+}
+
+// f32 activations in two steps, so that a caller can issue its weight loads between them: the loads of the lane's
+// 64 / SUB pieces of eight (ref_order: in the k order (0,4,1,5 | 2,6,3,7) the unpack of the reference's nibble order
+// yields), then the range check and the split into f16 terms, which wait for the values.
+template <int SUB, bool REF_ORDER>
+__device__ __forceinline__ void gemv4s_load_a_f32(float (&v)[64 / SUB * 8], const void *a_any, uint32_t arow, uint32_t kc,
+                                                  uint32_t cl, uint32_t k)
+{
+#pragma unroll
+    for (int j = 0; j < 64 / SUB; j++) {
+        uint32_t k0 = kc * 128u + j * (2u * SUB) + (cl >> 2) * 8u;
+        if (k0 > k - 8u) k0 = k - 8u;  // only the zero-padded groups of a last partial chunk get here
+        const float4 *p = (const float4 *)((const float *)a_any + (size_t)arow * k + k0);
+        float4 x = p[0], y = p[1];
+        const float w[8] = {x.x, REF_ORDER ? y.x : x.y, REF_ORDER ? x.y : x.z, REF_ORDER ? y.y : x.w,
+                            REF_ORDER ? x.z : y.x, REF_ORDER ? y.z : y.y, REF_ORDER ? x.w : y.z, y.w};
+#pragma unroll
+        for (int i = 0; i < 8; i++) v[8 * j + i] = w[i];
+    }
+}
+
+template <int SUB, int TERMS, int RG>
+__device__ __forceinline__ void gemv4s_split_a_f32(ChunkS<SUB, RG> &r, float (&v)[64 / SUB * 8], bool lane_is_lo)
+{
+    f32_terms_range(v, r.a_inv);
+#pragma unroll
+    for (int j = 0; j < 64 / SUB; j++) {
+        float w[8];
+#pragma unroll
+        for (int i = 0; i < 8; i++) w[i] = v[8 * j + i];
+        split_f32x8(w, r.a[0][j], r.a_lo[j]);
+        if (TERMS == kTermsRowPacked) {
+#pragma unroll
+            for (int i = 0; i < 4; i++) r.a[0][j][i] = lane_is_lo ? r.a_lo[j][i] : r.a[0][j][i];
+        }
+    }
 }
 
 // The lane's activations of chunk kc: 64 / SUB pieces of eight, row arow (term modes as gemv4_load_chunk).
@@ -252,27 +327,21 @@ __device__ __forceinline__ void gemv4s_load_a(ChunkS<SUB, RG> &r, const void *a_
         r.a[0][0] = *(const uint4v *)((const _Float16 *)a_any + (size_t)arow * k + k0);
         return;
     }
+    if (AF32) {
+        float v[64 / SUB * 8];
+        gemv4s_load_a_f32<SUB, REF_ORDER>(v, a_any, arow, kc, cl, k);
+        gemv4s_split_a_f32<SUB, TERMS, RG>(r, v, lane_is_lo);
+        return;
+    }
 #pragma unroll
     for (int j = 0; j < 64 / SUB; j++) {
         uint32_t k0 = kc * 128u + j * (2u * SUB) + (cl >> 2) * 8u;
         if (k0 > k - 8u) k0 = k - 8u;  // only the zero-padded groups of a last partial chunk get here
-        if (AF32) {
-            const float4 *p = (const float4 *)((const float *)a_any + (size_t)arow * k + k0);
-            float4 x = p[0], y = p[1];
-            const float v[8] = {x.x, REF_ORDER ? y.x : x.y, REF_ORDER ? x.y : x.z, REF_ORDER ? y.y : x.w,
-                                REF_ORDER ? x.z : y.x, REF_ORDER ? y.z : y.y, REF_ORDER ? x.w : y.z, y.w};
-            split_f32x8(v, r.a[0][j], r.a_lo[j]);
-            if (TERMS == kTermsRowPacked) {
 #pragma unroll
-                for (int i = 0; i < 4; i++) r.a[0][j][i] = lane_is_lo ? r.a_lo[j][i] : r.a[0][j][i];
-            }
-        } else {
-#pragma unroll
-            for (int rg = 0; rg < RG; rg++) {
-                uint32_t row = arow + 4u * rg;
-                if (RG > 1 && row > m_rows - 1u) row = m_rows - 1u;
-                r.a[rg][j] = *(const uint4v *)((const _Float16 *)a_any + (size_t)row * k + k0);
-            }
+        for (int rg = 0; rg < RG; rg++) {
+            uint32_t row = arow + 4u * rg;
+            if (RG > 1 && row > m_rows - 1u) row = m_rows - 1u;
+            r.a[rg][j] = *(const uint4v *)((const _Float16 *)a_any + (size_t)row * k + k0);
         }
     }
 }
@@ -371,7 +440,9 @@ __device__ __forceinline__ void gemv4s_compute(const ChunkS<SUB, (RL + 3) / 4> &
         const float s = r.live ? (float)sv.h[g] : 0.f;
 #pragma unroll
         for (int rr = 0; rr < RL; rr++) {
-            if (TERMS == kTermsRowPacked) acc[rr] = fmaf(d[0][2 * rr] + d[0][2 * rr + 1], s, acc[rr]);
+            // (a_inv: 1 unless the f32 activations of that row were scaled into the f16 range)
+            if (TERMS == kTermsRowPacked) acc[rr] = fmaf(d[0][2 * rr] + d[0][2 * rr + 1], s * r.a_inv[2 * rr], acc[rr]);
+            else if (TERMS == kTermsTwoPasses) acc[rr] = fmaf(d[0][rr], s * r.a_inv[rr], acc[rr]);
             else acc[rr] = fmaf(d[rr / 4][rr % 4], s, acc[rr]);
         }
     }

@@ -395,6 +395,46 @@ def test_gemm_tw_marlin_m1_reference_layout(dev, k, n):
         dev.set_option("m1_exact", 0)
 
 
+@pytest.mark.parametrize("k,n", [(3584, 608), (896, 1152), (18944, 192), (1184, 200)])
+def test_f32_activations_beyond_the_f16_range(dev, k, n):
+    # The reference's GEMV takes any f32 row (quantize.rs:1188, 1219-1238).  Here the activations reach the MFMA as f16
+    # terms; a wave whose chunk holds a value past the f16 range scales the chunk by a power of two first.  Rows whose
+    # entries reach 1e6, a single huge entry among ordinary ones, and the largest finite f32 magnitudes that keep the
+    # f32 result finite: the drop-in entry on both its kernels (K up to 4096 and beyond) and twm_gemm at M <= 4.
+    packed, scales, _ = synth(k, n, 1, 8800 + k)
+    pd, sd = T.GpuTensor.from_host(dev, packed), T.GpuTensor.from_host(dev, scales, "f16")
+    base = O.synth_normal_f32(4 * k, 8900 + k).reshape(4, k)
+    rows = base.copy()
+    rows[0] *= np.float32(2.5e5)                       # |a| up to about 1e6 everywhere
+    rows[1, 5::97] *= np.float32(3.0e5)                # a few huge entries among ordinary ones
+    rows[2] *= np.float32(1.0e30)                      # far beyond: sums near 1e33 still fit f32
+    rows[3, k // 2] = np.float32(70000.0)              # just past the largest f16
+    c = T.GpuTensor.zeros(dev, (n,), "f32")
+    for r in range(4):
+        a = np.ascontiguousarray(rows[r])
+        truth = O.gemm_f64(a.reshape(1, k), packed, scales, 1, k, n)[0]
+        T.gemm_tw_marlin_m1(dev, T.GpuTensor.from_host(dev, a), pd, sd, c, n, k)
+        got = c.to_host()
+        assert np.isfinite(got).all(), r
+        assert rel_err(got, truth) < TIGHT, r
+    w = T.MarlinWeight.from_device(dev, pd, sd, k, n)
+    for m in (1, 2, 4):
+        truth = O.gemm_f64(rows[:m], packed, scales, m, k, n)
+        cm = T.GpuTensor.zeros(dev, (m, n), "f32")
+        T.gemm(dev, w, T.GpuTensor.from_host(dev, np.ascontiguousarray(rows[:m])), m, cm)
+        for r in range(m):   # (row by row: the rows differ by 30 orders of magnitude)
+            assert rel_err(cm.to_host()[r], truth[r]) < TIGHT, (m, r)
+    # in range nothing changes: the same bits as before the guard, i.e. as with the values given as exact f16 pairs
+    a_in = np.ascontiguousarray(base[0])
+    T.gemm_tw_marlin_m1(dev, T.GpuTensor.from_host(dev, a_in), pd, sd, c, n, k)
+    first = c.to_host()
+    a_in[7] = np.float32(64999.0)
+    T.gemm_tw_marlin_m1(dev, T.GpuTensor.from_host(dev, a_in), pd, sd, c, n, k)
+    assert rel_err(c.to_host(), O.gemm_f64(a_in.reshape(1, k), packed, scales, 1, k, n)[0]) < TIGHT
+    assert np.isfinite(first).all()
+    w.free()
+
+
 def test_gemm_tw_marlin_m1_from_buffer_and_errors(dev):
     k, n = 128, 64
     packed, scales, a16 = synth(k, n, 1, 9)
