@@ -117,6 +117,69 @@ def time_launches(dev, fn, reps, settle_ms=25.0):
     return run(reps) / reps
 
 
+def trace_decode(T, dev, layers):
+    """The layer's four GEMVs at M = 1, launched one after the other as in the layer, with every workgroup writing
+    the GPU's 100 MHz clock at its start, when its first wave has its weights unpacked, and at its end
+    (twm_debug_trace).  Prints, per projection: the gap since the previous kernel's last workgroup ended, when the
+    first data was there, the span from first start to last end, and the bytes of finished workgroups per microsecond."""
+    cap, slots = 4096, 48
+    trace = T.GpuTensor.zeros(dev, (slots * cap * 4,), "i32")
+    order = [name for name, _, _ in LAYER_7B]
+    shape = {name: (k, n) for name, k, n in LAYER_7B}
+
+    def launch(i, traced):
+        name = order[i % 4]
+        w, a, c = layers[(i // 4) % len(layers)][name]
+        if traced:
+            dev._l.twm_debug_trace(dev.handle, trace.ptr + (i % slots) * cap * 16, cap)
+        T.gemm(dev, w, a, 1, c)
+    for i in range(4000):
+        launch(i, False)
+    dev.synchronize()
+    for i in range(slots):
+        launch(i, True)
+    dev.synchronize()
+    dev._l.twm_debug_trace(dev.handle, None, 0)
+    t = trace.to_host().view(np.uint32).reshape(slots, cap, 4)
+    rows = {name: [] for name in order}
+    prev_end = None
+    for i in range(slots):
+        x = t[i][t[i][:, 2] != 0]
+        st, ld, en = x[:, 0].astype(np.int64), x[:, 1].astype(np.int64), x[:, 2].astype(np.int64)
+        s0 = st.min()
+        hw = x[:, 3]
+        cus = len(np.unique(((hw >> 16) & 0xF) * 4096 + ((hw >> 8) & 0xFF)))   # XCD, then SE / SH / CU bits of HW_ID
+        k, n = shape[order[i % 4]]
+        per_wg = algo_bytes(k, n) / len(x)
+        ends = np.sort((en - s0) / 100.0)
+        span = ends[-1]
+        # steady rate: between the moment 10 % and the moment 90 % of the workgroups have ended
+        lo, hi = ends[int(0.1 * len(x))], ends[int(0.9 * len(x)) - 1]
+        steady = 0.8 * len(x) * per_wg / max(hi - lo, 1e-9) / 1e6 if len(x) >= 512 else float("nan")
+        if i >= 8:   # (the first launches after the switch to the traced kernels are left out)
+            rows[order[i % 4]].append((len(x), cus, (s0 - prev_end) / 100.0 if prev_end is not None else float("nan"),
+                                       (st.max() - s0) / 100.0, (ld[ld > 0].min() - s0) / 100.0, (ld[ld > 0] - st[ld > 0]).mean() / 100.0,
+                                       ends[0], span, (en - st).mean() / 100.0, steady))
+        prev_end = en.max()
+    print("| projection | workgroups | CUs used | gap since the previous kernel's last end | last workgroup starts | first wave unpacked | "
+          "start to unpacked (mean) | first workgroup ends | span (first start to last end) | workgroup lifetime (mean) | "
+          "rate between 10 % and 90 % of the workgroups done |")
+    print("|---|---|---|---|---|---|---|---|---|---|---|")
+    for name in order:
+        r = np.array(rows[name], dtype=np.float64)
+        m = np.array([np.nanmean(r[:, j]) if np.isfinite(r[:, j]).any() else float("nan") for j in range(r.shape[1])])
+        k, n = shape[name]
+        print("| %s %d -> %d | %d | %d | %.2f us | %.2f us | %.2f us | %.2f us | %.2f us | %.2f us | %.2f us | %s |" % (
+            name, k, n, m[0], m[1], m[2], m[3], m[4], m[5], m[6], m[7], m[8],
+            ("%.2f TB/s" % m[9]) if np.isfinite(m[9]) else "-"))
+    tot = sum(np.nanmean(np.array(rows[nm])[:, 2]) + np.nanmean(np.array(rows[nm])[:, 7]) for nm in order)
+    print("\nsum of gaps and spans: %.2f us per layer (traced kernels, eager launches)" % tot)
+    for name in order:
+        k, n = shape[name]
+        m = np.array(rows[name], dtype=np.float64).mean(axis=0)
+        print("%s: %.1f MB in a span of %.2f us = %.2f TB/s inside the kernel" % (name, algo_bytes(k, n) / 1e6, m[7], algo_bytes(k, n) / m[7] / 1e6))
+
+
 def profiler_attached():
     """True when a rocprofiler tool library is preloaded into this process (rocprofv3 does that).  Under it the
     bench issues every launch eagerly: rocprofv3 has crashed on the host inside hipGraphLaunch on this bench's
@@ -208,6 +271,9 @@ def main():
     ap.add_argument("--pmc-copy", action="store_true",
                     help="also run four 64 MiB device-to-device copies: a kernel of known traffic to scale rocprofv3 "
                          "FETCH_SIZE / WRITE_SIZE readings by")
+    ap.add_argument("--trace-decode", action="store_true",
+                    help="instead of the timings: run the four M = 1 GEMVs of the layer with the library's per-workgroup "
+                         "clock trace (twm_debug_trace) and print where each launch's time goes, as a markdown table")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU; --gpus %d is not supported (no collectives, no sharding)" % args.gpus)
@@ -245,6 +311,10 @@ def main():
         for name, k, n in LAYER_7B:
             w, a, c = entry[name]
             T.gemm(dev, w, a, 1, c)
+
+    if args.trace_decode:
+        trace_decode(T, dev, layers)
+        return
 
     if args.pmc_copy:
         src = T.GpuTensor.zeros(dev, (64 << 20,), "u8")
