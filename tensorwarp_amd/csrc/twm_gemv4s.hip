@@ -49,11 +49,12 @@ __device__ __forceinline__ void gemv4s_body(const char *__restrict__ cw, const v
 {
     static_assert(!REFL || (AF32 && RL == 1), "the reference-layout variant is the M = 1, f32-activation entry point");
     constexpr int CPP = 64 / SUB;     // chunks per pass
-    // One row of f16 activations on 16 columns, several passes per wave (deep K): the pipelined pass loop with the
-    // shared-piece form of the activations (18944 -> 3584 at M = 1: 9.2 against 10.0 us).  A wave that makes a single
-    // pass gains nothing from either, and the other variants run out of registers with both sets live.
-    constexpr bool PIPE = !ONE && !AF32 && RL == 1 && SUB == 16 && !REFL;
-    constexpr int TERMS = PIPE ? kTermsOneRow : gemv4_terms<AF32, RL>();
+    // f16 activations on 16 columns, several passes per wave (deep K), up to four rows: the pipelined pass loop, and for
+    // one row the shared-piece form of the activations (18944 -> 3584: 8.9 against 10.0 us at M = 1, 9.95 against 10.35
+    // at M = 2, level at M = 4).  A wave that makes a single pass gains nothing from either, and the other variants
+    // run out of registers with both sets live.
+    constexpr bool PIPE = !ONE && !AF32 && RL <= 4 && SUB == 16 && !REFL;
+    constexpr int TERMS = (PIPE && RL == 1) ? kTermsOneRow : gemv4_terms<AF32, RL>();
     extern __shared__ float red[];    // [waves][RL][64]
     __shared__ int s_last;
 
