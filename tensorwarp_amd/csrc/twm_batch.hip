@@ -84,9 +84,9 @@ constexpr int kBtRow = 128;  // halves per LDS row (256 bytes)
 // wave's count of loads in flight the same.
 template <int MT, bool RND, int TERMS, int TPW, int KS, int WPS>
 __global__ __launch_bounds__(64 * WPS * KS) void k_batch(const uint4v *__restrict__ qw, const uint2v *__restrict__ sc,
-                                                const void *__restrict__ a_any, OutSpec out, float *__restrict__ partials,
-                                                uint32_t m_rows, uint32_t k, uint32_t n, uint32_t n_tiles,
-                                                uint32_t k_chunks, uint32_t chunks_per_split, uint32_t lo_offset)
+                                                const void *__restrict__ a_any, uint32_t m_rows, uint32_t k, uint32_t n,
+                                                uint32_t n_tiles, uint32_t k_chunks, uint32_t chunks_per_split,
+                                                uint32_t lo_offset, float *__restrict__ partials, OutSpec out)
 {
     constexpr bool kRounded = RND;           // weights rounded to f16 as in the reference's dequant-then-FP16-GEMM route (option)
     constexpr int S = 4;                     // register slots: chunk kc lives in slot kc % S, three chunks are in flight
@@ -347,8 +347,8 @@ static hipError_t launch_batch_t(hipStream_t s, const WeightView &w, const void 
     const uint32_t quads = w.n_tiles / 4;   // n_tiles is a multiple of 4
     constexpr uint32_t kQuadsPerGroup = WPS * TPW / 4;
     dim3 grid((quads + kQuadsPerGroup - 1) / kQuadsPerGroup, splits);
-    hipLaunchKernelGGL((k_batch<MT, RND, TERMS, TPW, KS, WPS>), grid, dim3(64 * WPS * KS), 0, s, (const uint4v *)w.qw, (const uint2v *)w.sc, a, out,
-                       splits > 1 ? partials : nullptr, m, w.k, w.n, w.n_tiles, w.k_chunks, cps, lo_offset);
+    hipLaunchKernelGGL((k_batch<MT, RND, TERMS, TPW, KS, WPS>), grid, dim3(64 * WPS * KS), 0, s, (const uint4v *)w.qw, (const uint2v *)w.sc, a,
+                       m, w.k, w.n, w.n_tiles, w.k_chunks, cps, lo_offset, splits > 1 ? partials : nullptr, out);
     if (splits > 1) {
         hipError_t e = launch_splitk_reduce(s, partials, out, m, w.n, w.n_tiles * 16, splits);
         if (e != hipSuccess) return e;

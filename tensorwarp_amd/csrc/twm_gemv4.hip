@@ -38,10 +38,10 @@ __device__ __forceinline__ void gemv4_store_out(const OutSpec &out, uint32_t m, 
 // REFL: cw is the reference's packed array and ref_scales its scales (no repack; M = 1, f32 activations).
 template <int NT, int RL, bool AF32, bool REFL = false>
 __global__ __launch_bounds__(1024) void k_gemv4(const char *__restrict__ cw, const void *__restrict__ a_any,
-                                                 OutSpec out, float *__restrict__ ws, unsigned *__restrict__ counters, uint32_t m_rows, uint32_t k,
-                                                 uint32_t n, uint32_t n_pad, uint32_t k_chunks, uint32_t tile_groups,
-                                                 uint32_t splits, uint32_t cps, float *__restrict__ swiglu_out,
-                                                 const uint16_t *__restrict__ ref_scales = nullptr)
+                                                 uint32_t m_rows, uint32_t k, uint32_t n, uint32_t n_pad, uint32_t k_chunks,
+                                                 uint32_t tile_groups, uint32_t splits, uint32_t cps,
+                                                 const uint16_t *__restrict__ ref_scales, float *__restrict__ ws,
+                                                 unsigned *__restrict__ counters, float *__restrict__ swiglu_out, OutSpec out)
 {
     extern __shared__ float red[];  // [waves][NT][RL][64]
     __shared__ int s_last;
@@ -214,15 +214,13 @@ static hipError_t launch_gemv4_t(hipStream_t s, const WeightView &w, const void 
     size_t lds = (size_t)waves * NT * RL * 64 * sizeof(float);
     if (a_f32) {
         if constexpr (RL <= 4)
-            hipLaunchKernelGGL((k_gemv4<NT, RL, true>), dim3(blocks), dim3(waves * 64), lds, s, (const char *)w.cq, a, out, ws,
-                               counters, m, w.k, w.n, n_pad, w.k_chunks, tile_groups,
-                               splits, cps, swiglu_out);
+            hipLaunchKernelGGL((k_gemv4<NT, RL, true>), dim3(blocks), dim3(waves * 64), lds, s, (const char *)w.cq, a, m, w.k, w.n,
+                               n_pad, w.k_chunks, tile_groups, splits, cps, (const uint16_t *)nullptr, ws, counters, swiglu_out, out);
         else
             return hipErrorInvalidValue;  // more than four rows: f16 activations only
     } else
-        hipLaunchKernelGGL((k_gemv4<NT, RL, false>), dim3(blocks), dim3(waves * 64), lds, s, (const char *)w.cq, a, out, ws,
-                           counters, m, w.k, w.n, n_pad, w.k_chunks, tile_groups,
-                           splits, cps, swiglu_out);
+        hipLaunchKernelGGL((k_gemv4<NT, RL, false>), dim3(blocks), dim3(waves * 64), lds, s, (const char *)w.cq, a, m, w.k, w.n,
+                           n_pad, w.k_chunks, tile_groups, splits, cps, (const uint16_t *)nullptr, ws, counters, swiglu_out, out);
     return hipGetLastError();
 }
 
@@ -246,8 +244,7 @@ hipError_t launch_gemv4_ref(hipStream_t s, const uint8_t *packed, const uint16_t
     out.seg[0].start = 0;
     out.seg[0].width = n;
     hipLaunchKernelGGL((k_gemv4<1, 1, true, true>), dim3(blocks), dim3(waves * 64), lds, s, (const char *)packed,
-                       (const void *)a, out, ws, counters, 1u, k, n, n_pad, k_chunks, tiles64, splits, cps,
-                       (float *)nullptr, scales);
+                       (const void *)a, 1u, k, n, n_pad, k_chunks, tiles64, splits, cps, scales, ws, counters, (float *)nullptr, out);
     return hipGetLastError();
 }
 

@@ -99,9 +99,9 @@ struct ChunkRegs {
 
 template <int MT, bool AF32, int WAVES>
 __global__ __launch_bounds__(WAVES * 64) void k_stream(const uint4v *__restrict__ qw, const uint2v *__restrict__ sc,
-                                                 const void *__restrict__ a_any, OutSpec out, float *__restrict__ partials,
-                                                 uint32_t m_rows, uint32_t k, uint32_t n, uint32_t n_tiles,
-                                                 uint32_t k_chunks, uint32_t chunks_per_split, uint32_t lo_offset)
+                                                 const void *__restrict__ a_any, uint32_t m_rows, uint32_t k, uint32_t n,
+                                                 uint32_t n_tiles, uint32_t k_chunks, uint32_t chunks_per_split,
+                                                 uint32_t lo_offset, float *__restrict__ partials, OutSpec out)
 {
     constexpr uint32_t kABytes = 2u;  // f16 rows; with AF32 a_any holds the hi rows and, lo_offset bytes on, the lo rows
     __shared__ float red[WAVES][16 * MT][64];
@@ -267,8 +267,8 @@ static hipError_t launch_stream_t(hipStream_t s, const WeightView &w, const void
     uint32_t cps = (w.k_chunks + splits - 1) / splits;
     splits = (w.k_chunks + cps - 1) / cps;  // no empty split
     dim3 grid(w.n_tiles / 4, splits);
-    hipLaunchKernelGGL((k_stream<MT, AF32, WAVES>), grid, dim3(WAVES * 64), 0, s, (const uint4v *)w.qw, (const uint2v *)w.sc, a, out,
-                       splits > 1 ? partials : nullptr, m, w.k, w.n, w.n_tiles, w.k_chunks, cps, lo_offset);
+    hipLaunchKernelGGL((k_stream<MT, AF32, WAVES>), grid, dim3(WAVES * 64), 0, s, (const uint4v *)w.qw, (const uint2v *)w.sc, a,
+                       m, w.k, w.n, w.n_tiles, w.k_chunks, cps, lo_offset, splits > 1 ? partials : nullptr, out);
     if (splits > 1) {
         hipError_t e = launch_splitk_reduce(s, partials, out, m, w.n, w.n_tiles * 16, splits);
         if (e != hipSuccess) return e;
