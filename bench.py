@@ -254,6 +254,7 @@ def main():
     ap.add_argument("--no-vendor-gemm", action="store_true",
                     help="skip timing rocBLAS' dense FP16 GEMM beside the prefill kernel")
     ap.add_argument("--no-batched", action="store_true", help="skip the batched-decode layer (M = 4 .. 32)")
+    ap.add_argument("--no-tune", action="store_true", help="skip the layer with measured plans (twm_weight_tune)")
     ap.add_argument("--batched-eager", action="store_true",
                     help="batched-decode layer without graph capture (rocprofv3 has crashed in hipGraphLaunch of graphs this long)")
     ap.add_argument("--eager", action="store_true",
@@ -460,6 +461,34 @@ def main():
                 graphs_done.append(g_rows)
             lb = sum(algo_bytes(k, n, m) for _, k, n in LAYER_7B)
             extra["layer_M%d" % m] = {"us": round(ms * 1e3, 2), "GBps": round(lb / (ms * 1e-3) / 1e9, 1),
+                                      "frac_hbm": round(lb / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
+
+    # the same layer once more with measured plans: twm_weight_tune times the launch forms per weight and row count and
+    # keeps what beats the planners' choice by more than 2 % (the role of the reference's autotune table)
+    tuned = None
+    if not args.no_batched and not args.no_tune:
+        log("decode layer with measured plans")
+        t0 = time.time()
+        for li in range(L):
+            for name, k, n in LAYER_7B:
+                layers[li][name][0].tune([1, 4, 8, 16, 32])
+        tuned = {"tune_seconds": round(time.time() - t0, 2),
+                 "plans_layer0": {name: {"M%d" % m: layers[0][name][0].tuned_plan(m) for m in (1, 4, 8, 16, 32)} for name, _, _ in LAYER_7B}}
+        for m in (1, 4, 8, 16, 32):
+            bufs = {name: (T.GpuTensor.from_host(dev, rng.standard_normal((m, k), dtype=np.float32).astype(np.float16).view(np.uint16), "f16"),
+                           T.GpuTensor.zeros(dev, (m, n), "f32")) for name, k, n in LAYER_7B}
+
+            def run_rows(m=m, bufs=bufs):
+                for li in range(L):
+                    for name, k, n in LAYER_7B:
+                        T.gemm(dev, layers[li][name][0], bufs[name][0], m, bufs[name][1])
+            run_rows()
+            dev.synchronize()
+            g_rows = capture(run_rows)
+            ms = time_launches(dev, lambda i: g_rows.replay(), max(4, steps // L // 4)) / L
+            graphs_done.append(g_rows)
+            lb = sum(algo_bytes(k, n, m) for _, k, n in LAYER_7B)
+            tuned["layer_M%d" % m] = {"us": round(ms * 1e3, 2), "GBps": round(lb / (ms * 1e-3) / 1e9, 1),
                                       "frac_hbm": round(lb / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
 
     log("small configurations")
@@ -896,6 +925,8 @@ def main():
                                    "all_m2048_shapes": {key: v["frac_mfma_f16_peak"] for key, v in m2048.items()}}
     if extra:
         out["batched_decode"] = extra
+    if tuned is not None:
+        out["decode_with_measured_plans"] = tuned
     if sweep:
         out["split_sweep"] = sweep
     if prefill_sweep is not None:

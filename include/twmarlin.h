@@ -244,6 +244,18 @@ size_t twm_weight_bytes(const twm_weight *w);
  * capture such a call fails with TWM_UNSUPPORTED_OP: ask for the copy beforehand with twm_weight_ensure.
  * twm_weight_drop frees one of two copies (synchronises the stream); twm_weight_copies returns the mask held.
  * No counterpart in the reference, whose kernels read the one TW-Marlin order. */
+/* Measured plans, the role of AutoTuner::tune_gemm and its per-shape table (crates/kernels/src/autotune.rs:254-396):
+ * for each of the `count` row counts in ms[], times this weight's GEMM in the launch forms that the option knobs can
+ * ask for (sub-tile widths and waves, whole tiles with K-splits, streaming and LDS-shared batched-decode forms, prefill
+ * block heights and K-splits) on synthetic f16 activations -- as captured graphs replayed over copies of the weight that
+ * together exceed the 256 MB cache -- and keeps the fastest for that bucket of row counts (1, 2, 3-4, 5-8, ...
+ * 513-1024, above) when it beats the planners' own choice by more than 2 %.  Later calls with f16
+ * activations, splits = 0 and no knob set run the kept form; the table travels with twm_weight_export / _import.
+ * Allocates trial buffers and synchronises: a load-time call, not for a graph capture.
+ * twm_weight_tuned_plan returns the bucket's entry as eight ints: valid, kernel, nt, waves, sub, sub_waves, splits,
+ * prefill_bm (valid = 0: the planners' choice runs). */
+int twm_weight_tune(twm_ctx *ctx, twm_weight *w, const uint32_t *ms, uint32_t count);
+int twm_weight_tuned_plan(const twm_weight *w, uint32_t m, int *knobs8);
 int twm_weight_ensure(twm_ctx *ctx, twm_weight *w, int copies);
 int twm_weight_drop(twm_ctx *ctx, twm_weight *w, int copies);
 int twm_weight_copies(const twm_weight *w);

@@ -58,6 +58,8 @@ SIGNATURES = {
     "twm_weight_destroy": (None, [_vp]),
     "twm_weight_dims": (_int, [_vp, C.POINTER(_u32), C.POINTER(_u32)]),
     "twm_weight_bytes": (_sz, [_vp]),
+    "twm_weight_tune": (_int, [_vp, _vp, _vp, _u32]),
+    "twm_weight_tuned_plan": (_int, [_vp, _u32, _vp]),
     "twm_weight_ensure": (_int, [_vp, _vp, _int]),
     "twm_weight_drop": (_int, [_vp, _vp, _int]),
     "twm_weight_copies": (_int, [_vp]),

@@ -62,6 +62,22 @@ struct twm_ctx {
     hipDeviceProp_t prop;
 };
 
+// A launch form as the option knobs name it (twm_ctx_set_option), measured to be the fastest for one weight and one
+// bucket of row counts by twm_weight_tune: the role of the per-shape table of crates/kernels/src/autotune.rs:254-396.
+struct TunedPlan {
+    uint8_t valid, kernel, nt, waves, sub, sub_waves, splits, prefill_bm;
+};
+static_assert(sizeof(TunedPlan) == 8, "a tuned plan is eight bytes of the weight blob");
+constexpr int kTuneBuckets = 12;
+// row counts 1, 2, 3-4, 5-8, 9-16, 17-32, 33-64, 65-128, 129-256, 257-512, 513-1024, above
+static int tune_bucket(uint32_t m)
+{
+    if (m <= 2) return (int)m - 1;
+    int b = 2;
+    for (uint32_t top = 4; m > top && b < kTuneBuckets - 1; top *= 2) b++;
+    return b;
+}
+
 // The two repacked copies are allocations of their own, each made when the handle is created (option
 // "weight_copies") or at the first call that needs it (weight_ensure): a decode-only or prefill-only deployment holds
 // one copy, 4.5 bits per weight.
@@ -75,6 +91,7 @@ struct twm_weight {
     size_t copy_bytes;  // one copy
     size_t bytes;       // device memory held now
     bool paired;  // gate_up weight whose columns are in the paired order (32 gate, 32 up, ...)
+    TunedPlan tuned[kTuneBuckets];  // measured plans per row-count bucket (twm_weight_tune); valid = 0: the planners' choice
 };
 
 struct twm_bank {
@@ -681,6 +698,7 @@ static twm_weight *weight_alloc(twm_ctx *ctx, uint32_t k, uint32_t n)
     w->bytes = 0;
     w->qw = w->sc = w->cq = nullptr;
     w->paired = false;
+    memset(w->tuned, 0, sizeof w->tuned);
     return w;
 }
 
@@ -867,7 +885,8 @@ struct WeightBlobHeader {
 };
 static_assert(sizeof(WeightBlobHeader) == 64, "blob header is 64 bytes");
 static const char kBlobMagic[8] = {'T', 'W', 'M', 'W', 'G', 'T', '0', '1'};
-static const uint32_t kBlobLayout = 4;
+static const uint32_t kBlobLayout = 5;
+static const size_t kBlobTrailer = sizeof(TunedPlan) * kTuneBuckets;  // the measured plans (twm_weight_tune), after the payload
 
 // Four independent multiply-rotate lanes over 64-bit words (memory-bound on the host), folded at the end.
 static uint64_t blob_checksum(const uint8_t *p, size_t bytes)
@@ -889,7 +908,7 @@ static uint64_t blob_checksum(const uint8_t *p, size_t bytes)
     return r;
 }
 
-size_t twm_weight_blob_bytes(const twm_weight *w) { return w ? sizeof(WeightBlobHeader) + w->bytes : 0; }
+size_t twm_weight_blob_bytes(const twm_weight *w) { return w ? sizeof(WeightBlobHeader) + w->bytes + kBlobTrailer : 0; }
 
 int twm_weight_export(twm_ctx *ctx, const twm_weight *w, void *blob_host, size_t blob_bytes)
 {
@@ -922,6 +941,7 @@ int twm_weight_export(twm_ctx *ctx, const twm_weight *w, void *blob_host, size_t
     hd.checksum = blob_checksum(payload, at);
     hd.copies = (uint8_t)copies_of(w);
     memcpy(blob_host, &hd, sizeof hd);
+    memcpy(payload + at, w->tuned, kBlobTrailer);
     return TWM_OK;
 }
 
@@ -944,7 +964,7 @@ twm_weight *twm_weight_import(twm_ctx *ctx, const void *blob_host, size_t blob_b
     const int held = hd.copies & 3, n_held = (held & 1) + (held >> 1);
     bool ok = w->n_tiles == hd.n_tiles && w->k_chunks == hd.k_chunks && hd.copies <= 3 &&
               (w->copy_bytes == 0 ? hd.payload_bytes == 0 : (n_held >= 1 && hd.payload_bytes == (uint64_t)n_held * w->copy_bytes)) &&
-              blob_bytes == sizeof(WeightBlobHeader) + hd.payload_bytes && hd.paired <= 1 &&
+              blob_bytes == sizeof(WeightBlobHeader) + hd.payload_bytes + kBlobTrailer && hd.paired <= 1 &&
               (!hd.paired || hd.n % (2 * kPairWidth) == 0);
     if (!ok) api_fail(TWM_SHAPE_ERROR, "twm_weight_import: header does not describe a %u x %u weight of %zu bytes", hd.k, hd.n, blob_bytes);
     if (ok && blob_checksum(payload, (size_t)hd.payload_bytes) != hd.checksum) {
@@ -962,6 +982,11 @@ twm_weight *twm_weight_import(twm_ctx *ctx, const void *blob_host, size_t blob_b
         return nullptr;
     }
     w->paired = hd.paired != 0;
+    memcpy(w->tuned, payload + hd.payload_bytes, kBlobTrailer);
+    for (TunedPlan &p : w->tuned)   // (a plan is a set of option values: anything outside their ranges is dropped)
+        if (p.valid > 1 || p.kernel > 4 || p.kernel == 1 || p.nt > 4 || p.waves > 16 || p.sub_waves > 16 ||
+            (p.sub != 0 && p.sub != 1 && p.sub != 16 && p.sub != 32) || (p.prefill_bm != 0 && p.prefill_bm != 64 && p.prefill_bm != 128))
+            memset(&p, 0, sizeof p);
     return w;
 }
 
@@ -1173,8 +1198,8 @@ uint32_t twm_pick_splits(uint32_t k, uint32_t n, uint32_t m)
 
 // swiglu_out (paired weight): the launch writes silu(gate) * up to swiglu_out[m][n/2] instead of the columns
 // to `out`.
-static int gemm_common(twm_ctx *ctx, const twm_weight *w, const void *a_dev, int a_dtype, uint32_t m, const OutSpec &out,
-                       uint32_t splits, const char *who, float *swiglu_out = nullptr, uint32_t gate_act = 2)
+static int gemm_dispatch(twm_ctx *ctx, const twm_weight *w, const void *a_dev, int a_dtype, uint32_t m, const OutSpec &out,
+                         uint32_t splits, const char *who, float *swiglu_out = nullptr, uint32_t gate_act = 2)
 {
     if (a_dtype != TWM_F16 && a_dtype != TWM_F32) return api_fail(TWM_UNSUPPORTED_OP, "%s: activations must be f16 or f32", who);
     if (m == 0 || w->n == 0) return TWM_OK;
@@ -1322,6 +1347,208 @@ static int gemm_common(twm_ctx *ctx, const twm_weight *w, const void *a_dev, int
                     TWM_DEVICE_ERROR, "gemv launch");
     }
 #undef TWM_NEED
+    return TWM_OK;
+}
+
+// The knobs of a launch form, saved and set as one
+struct Knobs {
+    int kernel, nt, waves, sub, sub_waves, prefill_bm;
+};
+static Knobs knobs_of(const twm_ctx *c) { return Knobs{c->force_kernel, c->force_nt, c->force_waves, c->force_sub, c->force_sub_waves, c->prefill_bm}; }
+static void set_knobs(twm_ctx *c, const Knobs &k)
+{
+    c->force_kernel = k.kernel;
+    c->force_nt = k.nt;
+    c->force_waves = k.waves;
+    c->force_sub = k.sub;
+    c->force_sub_waves = k.sub_waves;
+    c->prefill_bm = k.prefill_bm;
+}
+
+// With nothing forced by the caller, a plan that twm_weight_tune measured for this weight and row count is what runs.
+static int gemm_common(twm_ctx *ctx, const twm_weight *w, const void *a_dev, int a_dtype, uint32_t m, const OutSpec &out,
+                       uint32_t splits, const char *who, float *swiglu_out = nullptr, uint32_t gate_act = 2)
+{
+    const Knobs user = knobs_of(ctx);
+    const bool free_choice = !splits && !user.kernel && !user.nt && !user.waves && !user.sub && !user.sub_waves && !user.prefill_bm;
+    const TunedPlan *tp = (m >= 1 && free_choice && !swiglu_out && a_dtype == TWM_F16) ? &w->tuned[tune_bucket(m)] : nullptr;
+    if (!tp || !tp->valid) return gemm_dispatch(ctx, w, a_dev, a_dtype, m, out, splits, who, swiglu_out, gate_act);
+    set_knobs(ctx, Knobs{tp->kernel, tp->nt, tp->waves, tp->sub, tp->sub_waves, tp->prefill_bm});
+    const int rc = gemm_dispatch(ctx, w, a_dev, a_dtype, m, out, tp->splits, who, swiglu_out, gate_act);
+    set_knobs(ctx, user);
+    return rc;
+}
+
+// Candidate launch forms for `m` rows: what the option knobs can ask for.  The first entry is the planners' own choice.
+static void tune_candidates(uint32_t m, uint32_t k_chunks, std::vector<TunedPlan> &out)
+{
+    auto add = [&](int kernel, int nt, int waves, int sub, int sub_waves, int splits, int bm) {
+        out.push_back(TunedPlan{1, (uint8_t)kernel, (uint8_t)nt, (uint8_t)waves, (uint8_t)sub, (uint8_t)sub_waves, (uint8_t)splits, (uint8_t)bm});
+    };
+    add(0, 0, 0, 0, 0, 0, 0);
+    const uint32_t passes16 = (k_chunks + 3) / 4, passes32 = (k_chunks + 1) / 2;
+    if (m <= 16) {
+        // sub-tile kernel: one pass per wave where sixteen waves cover K, else the pass loop on 4, 8 or 16 waves
+        for (int sub : {16, 32}) {
+            const uint32_t passes = sub == 16 ? passes16 : passes32;
+            if (passes <= 16) add(0, 0, 0, sub, (int)passes, 0, 0);
+            for (int wv : {4, 8, 16})
+                if ((uint32_t)wv < passes || (passes <= 16 && (uint32_t)wv != passes)) add(0, 0, 0, sub, wv, 0, 0);
+        }
+    }
+    if (m <= 4) {
+        for (int wv : {8, 16})
+            for (int sp : {1, 2, 4, 8}) add(2, 1, wv, 0, 0, sp, 0);   // whole 64-column tiles, K split over workgroups
+        add(2, 2, 8, 0, 0, 1, 0);
+    } else if (m <= 32) {
+        for (int sp : {1, 2, 3, 4, 6, 8}) add(3, 0, 0, 0, 0, sp, 0);  // streaming kernel
+        for (int nt : {1, 2, 3, 4})                                     // LDS-shared kernel: tiles per wave / quads per workgroup
+            for (int wv : {0, 8, 16})                                   // k-slices
+                for (int sp : {1, 2, 3, 4, 6})
+                    if (!(wv == 16 && nt != 1) && !(wv == 8 && nt == 3)) add(4, nt, wv, 0, 0, sp, 0);
+    } else {
+        for (int bm : {64, 128})
+            for (int sp : {1, 2, 3, 4, 6, 8}) add(0, 0, 0, 0, 0, sp, bm);
+    }
+}
+
+int twm_weight_tune(twm_ctx *ctx, twm_weight *w, const uint32_t *ms, uint32_t count)
+{
+    if (!ctx || !w) return api_fail(TWM_INVALID_HANDLE, "twm_weight_tune: null handle");
+    if (w->ctx != ctx) return api_fail(TWM_INVALID_HANDLE, "twm_weight_tune: weight belongs to another context");
+    if (ctx->capturing) return api_fail(TWM_UNSUPPORTED_OP, "twm_weight_tune: not allowed inside a graph capture");
+    if (count != 0 && !ms) return api_fail(TWM_INVALID_HANDLE, "twm_weight_tune: null row counts");
+    if (w->copy_bytes == 0 || w->k == 0 || w->n == 0) return TWM_OK;
+    uint32_t m_max = 0;
+    for (uint32_t i = 0; i < count; i++) {
+        if (ms[i] == 0 || ms[i] > 65536u) return api_fail(TWM_SHAPE_ERROR, "twm_weight_tune: row counts are 1 .. 65536");
+        if (ms[i] > m_max) m_max = ms[i];
+    }
+    if (m_max == 0) return TWM_OK;
+    // synthetic f16 activations (a fixed pattern of small values) and an output, both released at the end
+    void *a_dev = nullptr, *c_dev = nullptr;
+    const size_t a_bytes = (size_t)m_max * w->k * 2, c_bytes = (size_t)m_max * w->n * 4;
+    if (hipMalloc(&a_dev, a_bytes) != hipSuccess || hipMalloc(&c_dev, c_bytes) != hipSuccess) {
+        if (a_dev) (void)hipFree(a_dev);
+        return api_fail(TWM_MEMORY_ERROR, "twm_weight_tune: hipMalloc of the trial buffers");
+    }
+    int rc = TWM_OK;
+    {
+        std::vector<uint16_t> host(a_bytes / 2);
+        uint32_t x = 2463534242u;
+        for (auto &h : host) {
+            x ^= x << 13; x ^= x >> 17; x ^= x << 5;
+            h = (uint16_t)(0x3000u + (x & 0x0FFFu)) | (uint16_t)((x >> 16) & 0x8000u);  // +-[0.125, 0.5)
+        }
+        rc = twm_memcpy_h2d(ctx, a_dev, host.data(), a_bytes);
+    }
+    hipEvent_t e0 = nullptr, e1 = nullptr;
+    if (rc == TWM_OK && (hipEventCreate(&e0) != hipSuccess || hipEventCreate(&e1) != hipSuccess))
+        rc = api_fail(TWM_DEVICE_ERROR, "twm_weight_tune: hipEventCreate");
+    // The trials rotate over copies of the weight that together exceed the 256 MB cache in front of HBM, as the layers
+    // of a model do: timed on one resident copy, the forms that are best from the caches would win.
+    if (rc == TWM_OK) rc = weight_ensure(ctx, w, kCopyTile | kCopyCol, "twm_weight_tune");
+    std::vector<twm_weight> clones;
+    if (rc == TWM_OK) {
+        size_t want = ((size_t)320 << 20) / (2 * w->copy_bytes) + 1;
+        if (want > 32) want = 32;
+        for (size_t c = 0; c + 1 < want && rc == TWM_OK; c++) {
+            twm_weight cl = *w;
+            cl.qw = cl.sc = cl.cq = nullptr;
+            if (hipMalloc(&cl.qw, w->copy_bytes) != hipSuccess || hipMalloc(&cl.cq, w->copy_bytes) != hipSuccess) {
+                if (cl.qw) (void)hipFree(cl.qw);
+                (void)hipGetLastError();
+                break;   // (fewer copies: the trials are warmer than a model's layers would be, but still fair among themselves)
+            }
+            cl.sc = (char *)cl.qw + (size_t)w->n_tiles * w->k_chunks * 1024;
+            if (hipMemcpyAsync(cl.qw, w->qw, w->copy_bytes, hipMemcpyDeviceToDevice, ctx->stream) != hipSuccess ||
+                hipMemcpyAsync(cl.cq, w->cq, w->copy_bytes, hipMemcpyDeviceToDevice, ctx->stream) != hipSuccess)
+                rc = api_fail(TWM_DEVICE_ERROR, "twm_weight_tune: copying the weight");
+            clones.push_back(cl);
+        }
+    }
+    uint32_t turn = 0;
+    auto next_weight = [&]() -> const twm_weight * {
+        const size_t n = clones.size() + 1;
+        const size_t at = turn++ % n;
+        return at == 0 ? w : &clones[at - 1];
+    };
+    const Knobs user = knobs_of(ctx);
+    OutSpec out;
+    memset(&out, 0, sizeof out);
+    out.count = 1;
+    out.seg[0].ptr = (float *)c_dev;
+    out.seg[0].width = w->n;
+    for (uint32_t i = 0; i < count && rc == TWM_OK; i++) {
+        const uint32_t m = ms[i];
+        std::vector<TunedPlan> cands;
+        tune_candidates(m, w->k_chunks, cands);
+        const int reps = m <= 32 ? 24 : 6;
+        float best_ms = 0.f, own_ms = 0.f;
+        TunedPlan best = cands[0];
+        for (size_t c = 0; c < cands.size(); c++) {
+            const TunedPlan &p = cands[c];
+            set_knobs(ctx, Knobs{p.kernel, p.nt, p.waves, p.sub, p.sub_waves, p.prefill_bm});
+            bool ok = true;
+            for (int r = 0; r < 2 && ok; r++) ok = gemm_dispatch(ctx, next_weight(), a_dev, TWM_F16, m, out, p.splits, "twm_weight_tune") == TWM_OK;
+            float ms_taken = 0.f;
+            // timed as the decode loop runs it: a captured graph of `reps` launches over the rotating copies, replayed
+            hipGraph_t graph = nullptr;
+            hipGraphExec_t exec = nullptr;
+            if (ok) {
+                ok = hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeRelaxed) == hipSuccess;
+                bool launched = ok;
+                for (int r = 0; r < reps && launched; r++)
+                    launched = gemm_dispatch(ctx, next_weight(), a_dev, TWM_F16, m, out, p.splits, "twm_weight_tune") == TWM_OK;
+                if (ok) ok = hipStreamEndCapture(ctx->stream, &graph) == hipSuccess && launched;
+                ok = ok && graph && hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0) == hipSuccess;
+            }
+            for (int run = 0; run < 3 && ok; run++) {   // one untimed replay, then the faster of two timed ones
+                float t = 0.f;
+                (void)hipEventRecord(e0, ctx->stream);
+                ok = hipGraphLaunch(exec, ctx->stream) == hipSuccess;
+                (void)hipEventRecord(e1, ctx->stream);
+                ok = ok && hipEventSynchronize(e1) == hipSuccess && hipEventElapsedTime(&t, e0, e1) == hipSuccess;
+                if (run == 1 || (run == 2 && t < ms_taken)) ms_taken = t;
+            }
+            if (exec) (void)hipGraphExecDestroy(exec);
+            if (graph) (void)hipGraphDestroy(graph);
+            if (!ok) {   // a form this shape does not take: skipped
+                (void)hipGetLastError();
+                continue;
+            }
+            if (c == 0) own_ms = ms_taken;
+            if (best_ms == 0.f || ms_taken < best_ms) {
+                best_ms = ms_taken;
+                best = p;
+            }
+        }
+        // the planners' choice stays unless a forced form beats it by more than 2 % (timing noise)
+        TunedPlan &slot = w->tuned[tune_bucket(m)];
+        if (own_ms > 0.f && best_ms < 0.98f * own_ms && (best.kernel || best.nt || best.waves || best.sub || best.sub_waves || best.splits || best.prefill_bm))
+            slot = best;
+        else
+            memset(&slot, 0, sizeof slot);
+    }
+    set_knobs(ctx, user);
+    (void)hipStreamSynchronize(ctx->stream);
+    for (twm_weight &cl : clones) {
+        (void)hipFree(cl.qw);
+        (void)hipFree(cl.cq);
+    }
+    if (e0) (void)hipEventDestroy(e0);
+    if (e1) (void)hipEventDestroy(e1);
+    (void)hipFree(a_dev);
+    (void)hipFree(c_dev);
+    return rc;
+}
+
+int twm_weight_tuned_plan(const twm_weight *w, uint32_t m, int *knobs8)
+{
+    if (!w || !knobs8 || m == 0) return api_fail(TWM_INVALID_HANDLE, "twm_weight_tuned_plan: null argument");
+    const TunedPlan &p = w->tuned[tune_bucket(m)];
+    const int v[8] = {p.valid, p.kernel, p.nt, p.waves, p.sub, p.sub_waves, p.splits, p.prefill_bm};
+    for (int i = 0; i < 8; i++) knobs8[i] = v[i];
     return TWM_OK;
 }
 

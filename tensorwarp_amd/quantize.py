@@ -303,6 +303,18 @@ class MarlinWeight:
         """Mask of the repacked orders the handle holds now (COPY_TILES | COPY_COLUMN_LANE)."""
         return self.device._l.twm_weight_copies(self.handle)
 
+    def tune(self, ms):
+        """autotune.rs:254-396 — measure the launch forms for these row counts and keep the fastest per bucket."""
+        arr = (C.c_uint32 * len(ms))(*ms)
+        _check(self.device._l.twm_weight_tune(self.device.handle, self.handle, arr, len(ms)))
+
+    def tuned_plan(self, m):
+        """The kept plan for m rows: dict of the option values, or None when the planners' choice runs."""
+        v = (C.c_int * 8)()
+        _check(self.device._l.twm_weight_tuned_plan(self.handle, m, v))
+        keys = ("valid", "kernel", "nt", "waves", "sub", "sub_waves", "splits", "prefill_bm")
+        return dict(zip(keys[1:], list(v)[1:])) if v[0] else None
+
     def ensure(self, copies):
         _check(self.device._l.twm_weight_ensure(self.device.handle, self.handle, copies))
 

@@ -1069,7 +1069,7 @@ def test_weight_handle_with_one_copy_builds_the_other_on_demand(dev):
         assert w.copies == first
         # the export of a one-copy handle is half as long and comes back as it was
         blob = w.export_blob()
-        assert blob.size == 64 + one_copy
+        assert blob.size == 64 + one_copy + 96          # header, one copy, the table of measured plans
         w_back = T.MarlinWeight.import_blob(dev, blob)
         assert w_back.copies == first
         got = run(w)
@@ -1094,6 +1094,47 @@ def test_weight_handle_with_one_copy_builds_the_other_on_demand(dev):
     both.free()
 
 
+def test_weight_tune_keeps_results_and_travels_with_the_blob(dev):
+    # twm_weight_tune (the role of autotune.rs:254-396) times the launch forms and keeps the fastest per bucket of row
+    # counts.  Whatever it keeps, results stay inside the same bar against the oracle, a call with an explicit split
+    # factor or a knob set is not touched, and the table comes back from an exported blob.
+    k, n = 2048, 768
+    packed, scales = O.synth_packed(k, n, 1500), O.synth_scales(k, n, 1501)
+    w = T.MarlinWeight.upload(dev, packed, scales, k, n)
+    ms = [1, 4, 8, 32, 80]
+    acts = {m: O.synth_act_f16(m, k, 1510 + m) for m in ms}
+    before = {m: run_gemm(dev, w, acts[m], m, n, 0) for m in ms}
+    w.tune(ms)
+    plans = {m: w.tuned_plan(m) for m in ms}
+    print("kept plans:", plans)
+    assert w.tuned_plan(2) is None and w.tuned_plan(16) is None       # buckets that were not asked for
+    for m in ms:
+        got = run_gemm(dev, w, acts[m], m, n, 0)
+        if m <= 32:
+            truth = O.gemm_f64(f16_as_f32(acts[m]), packed, scales, m, k, n)
+            assert rel_err(got, truth) < TIGHT, (m, plans[m])
+        else:   # the prefill GEMM: weights of the FP16 Q4 unpack, f32 accumulation in whatever K-split order
+            w16 = O.dequant_f16(packed, scales, k, n).view(np.float16).astype(np.float64).reshape(k, n)
+            truth = acts[m].view(np.float16).astype(np.float64).reshape(m, k) @ w16
+            assert rel_err(got, truth) < 1e-3 and rel_err(before[m], truth) < 1e-3, (m, plans[m])
+        # forced calls do not look at the table
+        assert np.array_equal(run_gemm(dev, w, acts[m], m, n, 1), run_gemm(dev, w, acts[m], m, n, 1))
+    blob = w.export_blob()
+    w2 = T.MarlinWeight.import_blob(dev, blob)
+    for m in ms:
+        assert w2.tuned_plan(m) == plans[m]
+        assert np.array_equal(run_gemm(dev, w2, acts[m], m, n, 0), run_gemm(dev, w, acts[m], m, n, 0))
+    # tuning again with no row counts changes nothing; an entry outside the option ranges is dropped at import
+    w.tune([])
+    assert {m: w.tuned_plan(m) for m in ms} == plans
+    bad = blob.copy()
+    bad[-96:-88] = np.array([1, 9, 0, 0, 0, 0, 0, 0], np.uint8)         # bucket 0: kernel 9 does not exist
+    w3 = T.MarlinWeight.import_blob(dev, bad)
+    assert w3.tuned_plan(1) is None
+    for x in (w, w2, w3):
+        x.free()
+
+
 def test_repacked_weight_blob_round_trip_through_a_warp_file(dev, tmp_path):
     from tensorwarp_amd import warp_cache as W
     k, n, ffn = 640, 200, 96
@@ -1104,7 +1145,7 @@ def test_repacked_weight_blob_round_trip_through_a_warp_file(dev, tmp_path):
     wp = T.MarlinWeight.gate_up(dev, (T.GpuTensor.from_host(dev, gp), T.GpuTensor.from_host(dev, gs, "f16")),
                                 (T.GpuTensor.from_host(dev, up), T.GpuTensor.from_host(dev, us, "f16")), k, ffn)
     blob, blob_p = w.export_blob(), wp.export_blob()
-    assert blob.size == 64 + w.nbytes and bytes(blob[:8]) == b"TWMWGT01"
+    assert blob.size == 64 + w.nbytes + 96 and bytes(blob[:8]) == b"TWMWGT01"
     path = tmp_path / "model.warp"
     W.save_warp_cache(path, '{"layout": "gfx950"}', [("l0.w", W.DTYPE_U8, blob.shape, blob),
                                                     ("l0.gate_up", W.DTYPE_U8, blob_p.shape, blob_p)])
