@@ -202,7 +202,16 @@ void twm_ctx_destroy(twm_ctx *ctx)
 int twm_ctx_sync(twm_ctx *ctx)
 {
     if (!ctx) return api_fail(TWM_INVALID_HANDLE, "twm_ctx_sync: null context");
-    HIP_TRY(hipStreamSynchronize(ctx->stream), TWM_DEVICE_ERROR, "stream synchronize");
+    hipError_t e = hipStreamSynchronize(ctx->stream);
+    if (e != hipSuccess) {
+        // A launch that died may have left arrival counters of the in-launch split-K above zero, which would make
+        // every later split-K launch of this context finish its tiles early: put them back to zero if the device
+        // still takes a call.
+        (void)hipGetLastError();
+        (void)hipMemset(ctx->counters, 0, ctx->n_counters * sizeof(unsigned));
+        (void)hipGetLastError();
+        return api_fail(TWM_DEVICE_ERROR, "twm_ctx_sync: %s", hipGetErrorString(e));
+    }
     return TWM_OK;
 }
 

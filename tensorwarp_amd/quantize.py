@@ -388,14 +388,24 @@ class TWMarlinWeights:
 
     NAMES = ("wq", "wk", "wv", "wo", "wg", "wu", "wd")
 
-    def __init__(self, device, hidden_size, kv_dim, ffn_dim, pairs):
+    def __init__(self, device, hidden_size, kv_dim, ffn_dim, pairs, attn_norm=None, ffn_norm=None, bq=None, bk=None, bv=None):
         self.device, self.h, self.kv, self.ffn = device, hidden_size, kv_dim, ffn_dim
         for name in self.NAMES:
             p, s = pairs[name]
             setattr(self, name + "_packed", p)
             setattr(self, name + "_scales", s)
+        # the rest of the reference's struct (quantize.rs:1068-1080): the two norm vectors, which this path only
+        # carries, and the optional Q/K/V biases, which qkv() adds in the GEMV's store
+        self.attn_norm, self.ffn_norm = attn_norm, ffn_norm
+        self.bq, self.bk, self.bv = bq, bk, bv
         self.wqkv_packed = self.wqkv_scales = self.wgu_packed = self.wgu_scales = None
         self.repacked = {}
+
+    def qkv(self, a, m, q, k, v, splits=0):
+        """The fused QKV projection of the decode step (generate.rs:2152-2165): one GEMV whose store writes q, k and v
+        and adds bq / bk / bv where the layer has them (repack_for_decode first)."""
+        biases = [self.bq, self.bk, self.bv] if (self.bq is not None or self.bk is not None or self.bv is not None) else None
+        gemm_split(self.device, self.repacked["qkv"], a, m, [q, k, v], [self.h, self.kv, self.kv], splits, biases=biases)
 
     def fuse_projections(self):
         """quantize.rs:1138"""

@@ -1439,6 +1439,34 @@ def test_fused_qkv_and_gate_up_equal_separate_projections(dev):
         T.gemm_split(dev, rp["gate_up"], a3d, 3, [g, u], [ffn, ffn - 1])
 
 
+def test_layer_container_carries_norms_and_adds_biases(dev):
+    # TWMarlinWeights (quantize.rs:1067-1086) with its norm vectors and optional Q/K/V biases: qkv() is the fused GEMV of
+    # the decode step with the biases of generate.rs:2162-2165 added in the store; a layer without biases gives the plain sums
+    h, kv, ffn = 640, 128, 1280
+    names = {"wq": (h, h), "wk": (h, kv), "wv": (h, kv), "wo": (h, h), "wg": (h, ffn), "wu": (h, ffn), "wd": (ffn, h)}
+    host = {nm: (O.synth_packed(k, n, 1600 + i), O.synth_scales(k, n, 1700 + i)) for i, (nm, (k, n)) in enumerate(names.items())}
+    pairs = {nm: (T.GpuTensor.from_host(dev, p), T.GpuTensor.from_host(dev, s_, "f16")) for nm, (p, s_) in host.items()}
+    bq, bk, bv = (O.synth_normal_f32(x, 1800 + j) for j, x in enumerate((h, kv, kv)))
+    norm = T.GpuTensor.from_host(dev, np.ones(h, np.float32))
+    layer = T.TWMarlinWeights(dev, h, kv, ffn, pairs, attn_norm=norm, ffn_norm=norm,
+                              bq=T.GpuTensor.from_host(dev, bq), bk=T.GpuTensor.from_host(dev, bk), bv=T.GpuTensor.from_host(dev, bv))
+    plain = T.TWMarlinWeights(dev, h, kv, ffn, pairs)
+    assert layer.attn_norm is norm and plain.bq is None
+    a16 = O.synth_act_f16(1, h, 1900)
+    ad = T.GpuTensor.from_host(dev, a16, "f16")
+    outs = {}
+    for label, lw in (("biased", layer), ("plain", plain)):
+        lw.repack_for_decode()
+        q, kk, v = (T.GpuTensor.zeros(dev, (x,), "f32") for x in (h, kv, kv))
+        lw.qkv(ad, 1, q, kk, v)
+        outs[label] = [t.to_host() for t in (q, kk, v)]
+    for got_b, got_p, nm, b in zip(outs["biased"], outs["plain"], ("wq", "wk", "wv"), (bq, bk, bv)):
+        k_, n_ = names[nm]
+        truth = O.gemm_f64(f16_as_f32(a16), host[nm][0], host[nm][1], 1, k_, n_)[0]
+        assert rel_err(got_p, truth) < TIGHT
+        assert np.array_equal(got_b, got_p + b)      # one f32 add on top of the unbiased result
+
+
 @pytest.mark.parametrize("m,splits", [(1, 0), (1, 4), (3, 0), (12, 0), (12, 2), (40, 0), (70, 2)])
 def test_gemm_split_bias_adds_bq_bk_bv_in_the_store(dev, m, splits):
     # q = gemv + bq etc. (the add the reference makes in its bias + RoPE kernel): one f32 add per element on
