@@ -1071,7 +1071,10 @@ static SubPlan plan_gemv4_sub(uint32_t tiles64, uint32_t k_chunks, uint32_t m, b
     if (k_chunks < 16) return none;  // shallow K: nothing to gain over one chunk per wave of the 64-column plan
     const bool two_pass = a_f32 && m > 2;
     const uint32_t passes16 = (k_chunks + 3) / 4;
-    const SubPlan narrow16 = {16, passes16 <= 8 ? 8u : 16u};
+    // waves per workgroup on 16 columns: one pass each while eight or sixteen cover K; deeper, the pipelined pass loop
+    // on eight waves for one row and on four from two rows on (18944 -> 3584: M = 1 8.96 / 9.01 / 9.05 us on 8 / 4 / 16
+    // waves, M = 2 9.5 / 9.2 / 9.7, M = 4 11.2 / 10.75 / 11.75)
+    const SubPlan narrow16 = {16, passes16 <= 8 ? 8u : passes16 <= 16 ? 16u : (m >= 2 && !a_f32) ? 4u : 8u};
     if (tiles64 > 128) {
         // wide matrices: only the cheapest activations (f16, up to two rows) leave the sub-tiles ahead
         // (3584 -> 37888: 15.8 against 17.0 us at M = 1, 18.3 against 17.3 at M = 4, 19.9 against 17.9 with f32 rows)
@@ -1090,7 +1093,9 @@ static SubPlan plan_gemv4_sub(uint32_t tiles64, uint32_t k_chunks, uint32_t m, b
         return none;
     }
     if (two_pass && passes16 > 16) return k_chunks <= 100 ? SubPlan{32, 8} : none;  // (the looping 16-column variant spills)
-    if (m > 2 && passes16 > 32) return none;   // very deep K, four rows: the 64-column split-K plan is level or ahead
+    // very deep K, three or four rows: with f32 rows the 64-column split-K plan is level or ahead; with f16 rows the
+    // pipelined pass loop is (18944 -> 3584 at M = 3 / 4: 9.96 / 10.75 against 11.75 / 11.84 us)
+    if (m > 2 && passes16 > 32 && a_f32) return none;
     if (tiles64 > 64) return SubPlan{32, 16};  // 16 columns would leave a second, quarter-full round of workgroups
     return narrow16;
 }
