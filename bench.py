@@ -36,7 +36,7 @@ LAYER_05B = [("qkv", 896, 1152), ("o", 896, 896), ("gate_up", 896, 9728), ("down
 CFG0 = [("cfg0", 4096, 4096)]                                                                     # the single-GEMV configuration
 # HBM bytes per gate_up launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, each scaled by
 # what the same counter reads for a 64 MiB copy (profiles/k_gemv4s_gate_up_m1_hbm_traffic.md).
-GATE_UP_TRAFFIC_BYTES = 76664500
+GATE_UP_TRAFFIC_BYTES = 76679700
 
 
 def algo_bytes(k, n, m=1):
@@ -318,10 +318,17 @@ def main():
         return
 
     if args.pmc_copy:
+        # kernels of known traffic to scale counter readings by: a device-to-device copy of 64 MiB (a kernel only when
+        # the runtime does not hand it to a copy engine), a fill kernel that writes 64 MiB, and an argmax over one row of
+        # 16 Mi floats, which reads 64 MiB
         src = T.GpuTensor.zeros(dev, (64 << 20,), "u8")
         dst = T.GpuTensor.zeros(dev, (64 << 20,), "u8")
+        row = T.GpuTensor.zeros(dev, (1, 16 << 20), "f32")
+        idx = T.GpuTensor.zeros(dev, (1,), "i32")
         for _ in range(4):
             dev._l.twm_memcpy_d2d(dev.handle, dst.ptr, src.ptr, 64 << 20)
+            dev._l.twm_memset_zero(dev.handle, dst.ptr, 64 << 20)
+            T.argmax(dev, row, idx, 1, 16 << 20)
         dev.synchronize()
 
     log("decode layer: warm-up and graphs")

@@ -12,7 +12,7 @@ SOURCES = ["twm_kernels.hip", "twm_gemv4.hip", "twm_gemv4s.hip", "twm_moe.hip", 
 # with the default choice the results land in AGPRs and each costs a v_accvgpr_read first.
 # The decode kernels' first sixteen argument words arrive preloaded in scalar registers (see k_gemv4s).
 PRELOAD = ["-mllvm", "-amdgpu-kernarg-preload-count=16"]
-PER_FILE_FLAGS = {"twm_gemv4s.hip": PRELOAD, "twm_gemv4.hip": PRELOAD, "twm_stream.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"] + PRELOAD,
+PER_FILE_FLAGS = {"twm_gemv4s.hip": PRELOAD, "twm_gemv4.hip": PRELOAD, "twm_moe.hip": PRELOAD, "twm_stream.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"] + PRELOAD,
                   "twm_batch.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"] + PRELOAD}
 # -packed-fp32-ops off: v_pk_{add,mul,fma}_f32 are not to be generated on this hardware pool.
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fno-gpu-rdc",
