@@ -641,8 +641,6 @@ def main():
         bank_gu = T.ExpertBank.from_device(dev, gu_p, gu_s, g_gu * 2 * dim * 16, g_gu * 2 * dim, k, 2 * dim, experts)
         bank_gu_paired = T.ExpertBank.from_device(dev, gu_p, gu_s, g_gu * 2 * dim * 16, g_gu * 2 * dim, k, 2 * dim, experts, pair_gate_up=True)
         bank_d = T.ExpertBank.from_device(dev, d_p, d_s, g_d * k * 16, g_d * k, dim, k, experts)
-        for t in (gu_p, gu_s, d_p, d_s):
-            t.free()
         id_sets = [T.GpuTensor.from_host(dev, ((np.arange(top_k) * 16 + r) % experts).astype(np.float32)) for r in range(16)]
         wts = T.GpuTensor.from_host(dev, np.full(top_k, 0.125, np.float32))
         x = T.GpuTensor.from_host(dev, rng.standard_normal(k, dtype=np.float32))
@@ -660,9 +658,16 @@ def main():
             for ids in id_sets:
                 T.batched_marlin_gate_up(dev, x, bank_gu_paired, ids, geglu_b, top_k, act=T.ACT_GEGLU)
                 T.batched_marlin_down_axpy(dev, geglu_b, bank_d, ids, wts, acc_b, top_k)
+        acc_c = T.GpuTensor.zeros(dev, (k,), "f32")
+
+        def slabs():   # the reference's own arguments: raw slabs, nothing repacked
+            for ids in id_sets:
+                T.batched_marlin_gate_up_slabs(dev, x, gu_p, gu_s, ids, gate_up_all, g_gu * 2 * dim * 16, g_gu * 2 * dim, 2 * dim, k, top_k)
+                T.batched_marlin_split_geglu(dev, gate_up_all, geglu_a, dim, top_k)
+                T.batched_marlin_down_axpy_slabs(dev, geglu_a, d_p, d_s, ids, wts, acc_c, g_d * k * 16, g_d * k, k, dim, top_k)
         moe_bytes = top_k * (algo_bytes(k, 2 * dim) + algo_bytes(dim, k))
         moe = {"hidden": k, "expert_dim": dim, "experts": experts, "top_k": top_k, "bytes": moe_bytes}
-        for label, fn in (("gate_up_geglu_down_us", three), ("fused_geglu_then_down_us", two)):
+        for label, fn in (("gate_up_geglu_down_us", three), ("fused_geglu_then_down_us", two), ("reference_slabs_us", slabs)):
             fn()
             dev.synchronize()
             gr = capture(fn)

@@ -363,6 +363,36 @@ int twm_bank_down_axpy(twm_ctx *ctx, const twm_bank *b, const void *a_all_dev, i
 int twm_geglu_rows(twm_ctx *ctx, const float *gate_up_dev, uint32_t batch, uint32_t dim, int paired,
                    float *out_dev);
 
+/* ---- the reference's MoE launches with its own arguments: raw slabs, nothing repacked, no bank ---- */
+
+/* batched_marlin_gate_up (crates/kernels/src/moe_batched_marlin.rs:153-182): output[s][n] = input[1, K] x W[id_s] for
+ * s < top_k in one launch, id_s = (int)topk_ids_dev[s] read on the device; expert x's TW-Marlin arrays lie at
+ * packed_buf_dev + x * packed_bytes_per_expert (u8 [K/32][N][16]) and scales_buf_dev + x * scales_per_expert
+ * (f16 [K/32][N]).  Arguments in the reference's order.  f32 activations enter as two f16 terms (any finite value,
+ * as in twm_gemm_tw_marlin_m1); an id below zero or NaN gives a row of zeros where the reference reads out of bounds.
+ * Slower than a bank (twm_bank_gemv) by what the [G][N] order costs: a wave's four group rows are N * 16 bytes apart. */
+int twm_batched_marlin_gate_up(twm_ctx *ctx, const float *input_dev, const uint8_t *packed_buf_dev,
+                               const uint16_t *scales_buf_dev, const float *topk_ids_dev, float *output_dev,
+                               uint32_t packed_bytes_per_expert, uint32_t scales_per_expert, uint32_t n, uint32_t k,
+                               uint32_t top_k);
+/* batched_marlin_down_axpy (moe_batched_marlin.rs:184-213): acc[n] += sum over s < top_k of topk_weights[s] *
+ * (geglu_all[s][K] x W[id_s]).  The reference adds with float atomics in no fixed order; here slot by slot, in order,
+ * deterministic (sixteen slots per launch, further launches for more). */
+int twm_batched_marlin_down_axpy(twm_ctx *ctx, const float *geglu_all_dev, const uint8_t *packed_buf_dev,
+                                 const uint16_t *scales_buf_dev, const float *topk_ids_dev, const float *topk_weights_dev,
+                                 float *acc_dev, uint32_t packed_bytes_per_expert, uint32_t scales_per_expert, uint32_t n,
+                                 uint32_t k, uint32_t top_k);
+/* batched_marlin_split_geglu (moe_batched_marlin.rs:215-232): output[s][j] = gelu_tanh(gate_up[s][j]) *
+ * gate_up[s][moe_dim + j]; = twm_geglu_rows with the plain column order. */
+int twm_batched_marlin_split_geglu(twm_ctx *ctx, const float *gate_up_dev, float *output_dev, uint32_t moe_dim,
+                                   uint32_t top_k);
+/* gemm_tw_marlin_m1_indirect (crates/kernels/src/quantize_indirect.rs:228-253): C[1, N] = A[1, K] x W[expert_idx] with
+ * the expert's arrays at packed_buf_dev + packed_offsets_dev[expert_idx] (bytes, a multiple of 4) and scales_buf_dev +
+ * scales_offsets_dev[expert_idx] (f16 elements); both tables u32 arrays in device memory, read by the kernel. */
+int twm_gemm_tw_marlin_m1_indirect(twm_ctx *ctx, const float *a_dev, const uint8_t *packed_buf_dev,
+                                   const uint32_t *packed_offsets_dev, const uint16_t *scales_buf_dev,
+                                   const uint32_t *scales_offsets_dev, int expert_idx, float *c_dev, uint32_t n, uint32_t k);
+
 /* The library's split-K choice for MI355X (256 CUs) with f16 activations; same role as quantize.rs:1317-1325.
  * 1 where the plan needs no split (among others wherever M <= 16 runs on column sub-tiles). */
 uint32_t twm_pick_splits(uint32_t k, uint32_t n, uint32_t m);

@@ -81,6 +81,10 @@ SIGNATURES = {
     "twm_bank_gemv": (_int, [_vp, _vp, _vp, _int, _u32, _vp, _u32, _int, _vp]),
     "twm_bank_down_axpy": (_int, [_vp, _vp, _vp, _int, _vp, _vp, _u32, _vp]),
     "twm_geglu_rows": (_int, [_vp, _vp, _u32, _u32, _int, _vp]),
+    "twm_batched_marlin_gate_up": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _u32, _u32, _u32, _u32, _u32]),
+    "twm_batched_marlin_down_axpy": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _u32, _u32, _u32, _u32, _u32]),
+    "twm_batched_marlin_split_geglu": (_int, [_vp, _vp, _vp, _u32, _u32]),
+    "twm_gemm_tw_marlin_m1_indirect": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _int, _vp, _u32, _u32]),
     "twm_pick_splits": (_u32, [_u32, _u32, _u32]),
     "twm_graph_begin": (_int, [_vp]),
     "twm_graph_end": (_vp, [_vp]),

@@ -1816,6 +1816,85 @@ int twm_bank_down_axpy(twm_ctx *ctx, const twm_bank *b, const void *a_all_dev, i
     return TWM_OK;
 }
 
+/* ---- the reference's MoE launches on its own slabs (no bank) ------------------------------------ */
+
+static int raw_checks(const char *who, twm_ctx *ctx, const float *a_dev, const uint8_t *packed_buf_dev,
+                      const uint16_t *scales_buf_dev, uint32_t n, uint32_t k)
+{
+    if (!ctx) return api_fail(TWM_INVALID_HANDLE, "%s: null context", who);
+    if (int rc = check_kn(who, k, n)) return rc;
+    if (!a_dev || !packed_buf_dev || !scales_buf_dev) return api_fail(TWM_INVALID_HANDLE, "%s: null input", who);
+    // the reference kernels read a record as four 32-bit words: 4-byte alignment is their own limit
+    if (((uintptr_t)packed_buf_dev & 3) != 0) return api_fail(TWM_SHAPE_ERROR, "%s: packed must be 4-byte aligned", who);
+    if (((uintptr_t)a_dev & 15) != 0 || (k * 4u) % 16u != 0)
+        return api_fail(TWM_SHAPE_ERROR, "%s: activation rows must be 16-byte aligned", who);
+    return TWM_OK;
+}
+
+int twm_batched_marlin_gate_up(twm_ctx *ctx, const float *input_dev, const uint8_t *packed_buf_dev,
+                               const uint16_t *scales_buf_dev, const float *topk_ids_dev, float *output_dev,
+                               uint32_t packed_bytes_per_expert, uint32_t scales_per_expert, uint32_t n, uint32_t k,
+                               uint32_t top_k)
+{
+    const char *who = "twm_batched_marlin_gate_up";
+    if (!ctx) return api_fail(TWM_INVALID_HANDLE, "%s: null context", who);
+    if (int rc = check_kn(who, k, n)) return rc;
+    if (top_k == 0 || n == 0) return TWM_OK;
+    if (top_k > 65535u) return api_fail(TWM_SHAPE_ERROR, "%s: at most 65535 slots per call", who);
+    if (!output_dev) return api_fail(TWM_INVALID_HANDLE, "%s: null output", who);
+    if (k == 0) return twm_memset_zero(ctx, output_dev, (size_t)top_k * n * 4);
+    if (int rc = raw_checks(who, ctx, input_dev, packed_buf_dev, scales_buf_dev, n, k)) return rc;
+    if (!topk_ids_dev) return api_fail(TWM_INVALID_HANDLE, "%s: null ids", who);
+    if (packed_bytes_per_expert % 4u != 0) return api_fail(TWM_SHAPE_ERROR, "%s: the packed stride must be a multiple of 4", who);
+    const RawView v = {packed_buf_dev, scales_buf_dev, packed_bytes_per_expert, scales_per_expert, nullptr, nullptr, 0, k, n};
+    HIP_TRY(launch_raw_gemv(ctx->stream, v, input_dev, 0, topk_ids_dev, top_k, output_dev, ctx->force_sub, ctx->force_waves),
+            TWM_DEVICE_ERROR, "expert gemv launch");
+    return TWM_OK;
+}
+
+int twm_batched_marlin_down_axpy(twm_ctx *ctx, const float *geglu_all_dev, const uint8_t *packed_buf_dev,
+                                 const uint16_t *scales_buf_dev, const float *topk_ids_dev, const float *topk_weights_dev,
+                                 float *acc_dev, uint32_t packed_bytes_per_expert, uint32_t scales_per_expert, uint32_t n,
+                                 uint32_t k, uint32_t top_k)
+{
+    const char *who = "twm_batched_marlin_down_axpy";
+    if (!ctx) return api_fail(TWM_INVALID_HANDLE, "%s: null context", who);
+    if (int rc = check_kn(who, k, n)) return rc;
+    if (top_k == 0 || n == 0 || k == 0) return TWM_OK;  // nothing is added
+    if (int rc = raw_checks(who, ctx, geglu_all_dev, packed_buf_dev, scales_buf_dev, n, k)) return rc;
+    if (!topk_ids_dev || !topk_weights_dev || !acc_dev) return api_fail(TWM_INVALID_HANDLE, "%s: null pointer", who);
+    if (packed_bytes_per_expert % 4u != 0) return api_fail(TWM_SHAPE_ERROR, "%s: the packed stride must be a multiple of 4", who);
+    const RawView v = {packed_buf_dev, scales_buf_dev, packed_bytes_per_expert, scales_per_expert, nullptr, nullptr, 0, k, n};
+    HIP_TRY(launch_raw_down_axpy(ctx->stream, v, geglu_all_dev, topk_ids_dev, topk_weights_dev, top_k, acc_dev, ctx->force_sub,
+                                 ctx->force_waves),
+            TWM_DEVICE_ERROR, "expert down_axpy launch");
+    return TWM_OK;
+}
+
+int twm_batched_marlin_split_geglu(twm_ctx *ctx, const float *gate_up_dev, float *output_dev, uint32_t moe_dim, uint32_t top_k)
+{
+    return twm_geglu_rows(ctx, gate_up_dev, top_k, moe_dim, 0, output_dev);
+}
+
+int twm_gemm_tw_marlin_m1_indirect(twm_ctx *ctx, const float *a_dev, const uint8_t *packed_buf_dev,
+                                   const uint32_t *packed_offsets_dev, const uint16_t *scales_buf_dev,
+                                   const uint32_t *scales_offsets_dev, int expert_idx, float *c_dev, uint32_t n, uint32_t k)
+{
+    const char *who = "twm_gemm_tw_marlin_m1_indirect";
+    if (!ctx) return api_fail(TWM_INVALID_HANDLE, "%s: null context", who);
+    if (int rc = check_kn(who, k, n)) return rc;
+    if (n == 0) return TWM_OK;
+    if (!c_dev) return api_fail(TWM_INVALID_HANDLE, "%s: null output", who);
+    if (k == 0) return twm_memset_zero(ctx, c_dev, (size_t)n * 4);
+    if (int rc = raw_checks(who, ctx, a_dev, packed_buf_dev, scales_buf_dev, n, k)) return rc;
+    if (!packed_offsets_dev || !scales_offsets_dev) return api_fail(TWM_INVALID_HANDLE, "%s: null offset table", who);
+    if (expert_idx < 0) return api_fail(TWM_SHAPE_ERROR, "%s: negative expert index %d", who, expert_idx);
+    const RawView v = {packed_buf_dev, scales_buf_dev, 0, 0, packed_offsets_dev, scales_offsets_dev, expert_idx, k, n};
+    HIP_TRY(launch_raw_gemv(ctx->stream, v, a_dev, 0, nullptr, 1, c_dev, ctx->force_sub, ctx->force_waves), TWM_DEVICE_ERROR,
+            "expert gemv launch");
+    return TWM_OK;
+}
+
 int twm_geglu_rows(twm_ctx *ctx, const float *gate_up_dev, uint32_t batch, uint32_t dim, int paired, float *out_dev)
 {
     if (!ctx) return api_fail(TWM_INVALID_HANDLE, "twm_geglu_rows: null context");

@@ -369,6 +369,46 @@ __device__ __forceinline__ void gemv4s_load_w(ChunkS<SUB, RG> &r, const char *bl
     }
 }
 
+// The lane's weights and f32 activations of chunk kc from the reference's own arrays (packed u8 [G][N][16], scales f16
+// [G][N]; crates/kernels/src/quantize.rs:1219-1238): a sub-tile's records of one group are SUB * 16 contiguous bytes.
+// col = the lane's column, already clamped to n - 1; col_ok = false gives the lane weight 0, as do live = false (a chunk
+// past the k-range, replayed) and the groups past K / 32 of a last partial chunk.
+// Order of issue: the activations first (their range check, f32_terms_range, needs them all, loads complete in the order
+// of their issue, and these come from the cache); all eight weight loads into locals before anything is written to r
+// (written straight into r, each pair was followed by a full wait); the four scales before the records (the first
+// group's sum needs them); the scales of dead groups masked after the four have been packed (a select on a freshly
+// loaded value is turned into a branch around the load, with a full wait behind it).
+template <int SUB, int TERMS, int RG>
+__device__ __forceinline__ void gemv4s_load_pass_ref(ChunkS<SUB, RG> &r, const char *packed, const uint16_t *scales,
+                                                     const void *a_any, uint32_t arow, uint32_t kc, bool live, uint32_t col,
+                                                     bool col_ok, uint32_t n, uint32_t groups, uint32_t cl, uint32_t k,
+                                                     bool lane_is_lo)
+{
+    float av[64 / SUB * 8];
+    gemv4s_load_a_f32<SUB, true>(av, a_any, arow, kc, cl, k);
+    __builtin_amdgcn_sched_barrier(0);
+    uint4v wq[4];
+    uint32_t sb[4];
+    uint32_t keep[4];
+    size_t idx[4];
+#pragma unroll
+    for (int g = 0; g < 4; g++) {
+        const uint32_t gg = kc * 4u + g;
+        idx[g] = (size_t)(gg < groups ? gg : groups - 1u) * n + col;
+        keep[g] = (live && gg < groups && col_ok) ? 0xFFFFu : 0u;  // weight exactly 0 otherwise
+        sb[g] = ld_once(scales + idx[g]);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int g = 0; g < 4; g++) wq[g] = ld_once((const uint4v *)(packed + idx[g] * 16u));
+#pragma unroll
+    for (int g = 0; g < 4; g++) r.wq[g] = wq[g];
+    r.sc = uint2v{(sb[0] | (sb[1] << 16)) & (keep[0] | (keep[1] << 16)), (sb[2] | (sb[3] << 16)) & (keep[2] | (keep[3] << 16))};
+    r.live = true;  // (masked group by group above)
+    __builtin_amdgcn_sched_barrier(0);
+    gemv4s_split_a_f32<SUB, TERMS, RG>(r, av, lane_is_lo);
+}
+
 // lane I of every quad of lanes, in all four lanes of the quad
 template <int I>
 __device__ __forceinline__ uint4v quad_bcast(uint4v v)

@@ -98,34 +98,8 @@ __device__ __forceinline__ void gemv4s_body(const char *__restrict__ cw, const v
         const bool live = kc < kc1;
         kc = live ? kc : kc1 - 1u;  // a chunk past the k-range replays the last one with scale 0
         if (REFL) {
-            // the activations first: their range check (f32_terms_range) needs them all, loads complete in the order of
-            // their issue, and these come from the cache
-            float av[64 / SUB * 8];
-            gemv4s_load_a_f32<SUB, true>(av, a_any, arow, kc, cl, k);
-            __builtin_amdgcn_sched_barrier(0);
-            // (all eight loads into locals first: written straight into r, each pair was followed by a full wait; and the
-            // scales of dead groups are masked after the four have been packed: a select on a freshly loaded value is
-            // turned into a branch around the load, with a full wait behind it)
-            uint4v wq[4];
-            uint32_t sb[4];
-            uint32_t keep[4];
-            size_t idx[4];
-#pragma unroll
-            for (int g = 0; g < 4; g++) {
-                const uint32_t gg = kc * 4u + g;
-                idx[g] = (size_t)(gg < ref_groups ? gg : ref_groups - 1u) * n + ref_col;
-                keep[g] = (live && gg < ref_groups && st * SUB + cl < n) ? 0xFFFFu : 0u;  // weight exactly 0 otherwise
-                sb[g] = ld_once(ref_scales + idx[g]);   // (the four scales before the records: the first group's sum needs them all)
-            }
-            __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-            for (int g = 0; g < 4; g++) wq[g] = ld_once((const uint4v *)(cw + idx[g] * 16u));
-#pragma unroll
-            for (int g = 0; g < 4; g++) r.wq[g] = wq[g];
-            r.sc = uint2v{(sb[0] | (sb[1] << 16)) & (keep[0] | (keep[1] << 16)), (sb[2] | (sb[3] << 16)) & (keep[2] | (keep[3] << 16))};
-            r.live = true;  // (masked group by group above)
-            __builtin_amdgcn_sched_barrier(0);
-            gemv4s_split_a_f32<SUB, TERMS, RG>(r, av, lane_is_lo);
+            gemv4s_load_pass_ref<SUB, TERMS, RG>(r, cw, ref_scales, a_any, arow, kc, live, ref_col, st * SUB + cl < n, n, ref_groups,
+                                                 cl, k, lane_is_lo);
         } else {
             if (PIPE) {
                 // activations first: loads complete in the order of their issue, and these come from the cache

@@ -59,6 +59,17 @@ struct BankView {
     size_t expert_bytes;
     uint32_t experts, k, n, n_pad, k_chunks;
 };
+// The reference's own expert slabs (nothing repacked): packed u8 [G][N][16] and scales f16 [G][N] per expert, expert x at
+// packed + x * packed_stride / scales + x * scales_stride, or -- offset tables set -- the one expert `index` at
+// packed + packed_offs[index] (bytes) / scales + scales_offs[index] (f16 elements), the tables read on the device.
+struct RawView {
+    const uint8_t *packed;
+    const uint16_t *scales;
+    uint32_t packed_stride, scales_stride;
+    const uint32_t *packed_offs, *scales_offs;
+    int index;
+    uint32_t k, n;
+};
 constexpr int kMaxBankSlots = 16;   // top-k of the fused down + axpy launch (one wave or more per slot)
 
 struct DecodePlan {
@@ -179,5 +190,11 @@ hipError_t launch_bank_gemv(hipStream_t s, const BankView &b, const void *a, boo
                             const float *ids, uint32_t slots, int act, float *out, int force_sub = 0, int force_waves = 0);
 hipError_t launch_bank_down_axpy(hipStream_t s, const BankView &b, const void *a_all, bool a_f32, const float *ids,
                                  const float *weights, uint32_t slots, float *accum, int force_sub = 0, int force_waves = 0);
+
+// the same two launches on the reference's slabs, f32 activations (moe_batched_marlin.rs:153-214, quantize_indirect.rs:228-253)
+hipError_t launch_raw_gemv(hipStream_t s, const RawView &v, const float *a, uint32_t a_slot_stride, const float *ids,
+                           uint32_t slots, float *out, int force_sub = 0, int force_waves = 0);
+hipError_t launch_raw_down_axpy(hipStream_t s, const RawView &v, const float *a_all, const float *ids, const float *weights,
+                                uint32_t slots, float *accum, int force_sub = 0, int force_waves = 0);
 
 }  // namespace twm

@@ -149,6 +149,139 @@ __global__ __launch_bounds__(1024) void k_bank_down_axpy(const char *__restrict_
     }
 }
 
+// ---- the same two launches on the reference's own slabs (no bank, nothing repacked) --------------------------
+// batched_marlin_gate_up / batched_marlin_down_axpy (moe_batched_marlin.rs:20-74, 78-134) take the slab of all experts'
+// packed arrays u8 [G][N][16], the slab of their scales f16 [G][N], and per-expert strides; the expert of a slot is
+// (int)ids[slot].  gemm_tw_marlin_m1_indirect (quantize_indirect.rs:185-253) takes two u32 offset tables on the device
+// and a fixed expert index instead.  Both forms come down to two base addresses per slot.  An id below zero (or NaN),
+// where the reference would read before the slab, contributes zeros.  f32 activations as two f16 terms, like the
+// dense entry point on the reference's arrays.
+struct RawSlab {
+    const char *packed;
+    const uint16_t *scales;
+    uint32_t packed_stride, scales_stride;        // bytes, f16 elements per expert (strided form)
+    const uint32_t *packed_offs, *scales_offs;     // device tables: bytes, f16 elements (offset form; null otherwise)
+    int index;                                     // offset form: the expert
+};
+
+__device__ __forceinline__ bool raw_expert(const RawSlab &e, const float *ids, uint32_t slot, const char *&packed,
+                                           const uint16_t *&scales)
+{
+    if (e.packed_offs) {
+        packed = e.packed + e.packed_offs[e.index];
+        scales = e.scales + e.scales_offs[e.index];
+        return true;
+    }
+    const float id = ids[slot];
+    const bool ok = id >= 0.f;
+    const uint64_t x = ok ? (uint64_t)id : 0u;
+    packed = e.packed + x * e.packed_stride;
+    scales = e.scales + x * e.scales_stride;
+    return ok;
+}
+
+// grid = (sub-tiles, slots); workgroup = `waves` waves on SUB columns of one slot's expert, wave w takes passes
+// w, w + waves, ...; out[slot][n] = A[slot * a_slot_stride ...] x W[expert]
+template <int SUB, bool ONE>
+__global__ __launch_bounds__(1024) void k_raw_gemv(RawSlab e, const float *__restrict__ a, uint32_t a_slot_stride,
+                                                    const float *__restrict__ ids, float *__restrict__ out, uint32_t k,
+                                                    uint32_t n, uint32_t k_chunks)
+{
+    constexpr int CPP = 64 / SUB;
+    constexpr int TERMS = gemv4_terms<true, 1>();
+    extern __shared__ float red[];  // [waves][64]
+    const uint32_t st = blockIdx.x, slot = blockIdx.y;
+    const uint32_t waves = blockDim.x >> 6;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const uint32_t lane = threadIdx.x & 63u, cl = lane % SUB, cg = lane / SUB;
+    const uint32_t passes = (k_chunks + CPP - 1) / CPP;
+    const uint32_t on = st * SUB + cl, col = on < n ? on : n - 1u;
+    const char *packed;
+    const uint16_t *scales;
+    const bool have = raw_expert(e, ids, slot, packed, scales);
+
+    float acc[1] = {0.f};
+    if (have) {
+        const float *a_row = a + (size_t)slot * a_slot_stride;
+        const Gemv4Consts dq = make_gemv4_consts();
+        const bool is_lo = (cl & 1u) != 0;
+        gemv4s_run_passes<SUB, ONE>(
+            wave, waves, passes,
+            [&](ChunkS<SUB> &r, uint32_t pass) {
+                uint32_t kc = pass * CPP + cg;
+                const bool live = kc < k_chunks;
+                kc = live ? kc : k_chunks - 1u;
+                gemv4s_load_pass_ref<SUB, TERMS, 1>(r, packed, scales, a_row, 0, kc, live, col, on < n, n, k / 32u, cl, k, is_lo);
+            },
+            [&](const ChunkS<SUB> &r) { gemv4s_compute<SUB, 1, TERMS>(r, dq, acc); });
+    }
+    red[wave * 64 + lane] = acc[0];
+    __syncthreads();
+    if (threadIdx.x < SUB) {
+        const uint32_t o = st * SUB + threadIdx.x;
+        if (o < n) {
+            float v = 0.f;
+            for (uint32_t w = 0; w < waves; w++)
+#pragma unroll
+                for (int q = 0; q < CPP; q++) v += red[w * 64 + q * SUB + threadIdx.x];
+            out[(size_t)slot * n + o] = v;
+        }
+    }
+}
+
+// grid = sub-tiles; workgroup = slots * wps waves: wave (slot, j) takes passes j, j + wps, ... of its slot's expert on
+// row slot0 + slot of a_all; one thread per column then adds weight * dot to the accumulator slot by slot.
+template <int SUB, bool ONE>
+__global__ __launch_bounds__(1024) void k_raw_down_axpy(RawSlab e, const float *__restrict__ a_all, const float *__restrict__ ids,
+                                                         const float *__restrict__ weights, float *__restrict__ accum, uint32_t k,
+                                                         uint32_t n, uint32_t k_chunks, uint32_t slots, uint32_t wps)
+{
+    constexpr int CPP = 64 / SUB;
+    constexpr int TERMS = gemv4_terms<true, 1>();
+    extern __shared__ float red[];  // [slots * wps][64]
+    const uint32_t st = blockIdx.x;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const uint32_t lane = threadIdx.x & 63u, cl = lane % SUB, cg = lane / SUB;
+    const uint32_t slot = wave / wps, j = wave % wps;
+    const uint32_t passes = (k_chunks + CPP - 1) / CPP;
+    const uint32_t on = st * SUB + cl, col = on < n ? on : n - 1u;
+    const char *packed;
+    const uint16_t *scales;
+    const bool have = raw_expert(e, ids, slot, packed, scales);
+
+    float acc[1] = {0.f};
+    if (have) {
+        const float *a_row = a_all + (size_t)slot * k;
+        const Gemv4Consts dq = make_gemv4_consts();
+        const bool is_lo = (cl & 1u) != 0;
+        gemv4s_run_passes<SUB, ONE>(
+            j, wps, passes,
+            [&](ChunkS<SUB> &r, uint32_t pass) {
+                uint32_t kc = pass * CPP + cg;
+                const bool live = kc < k_chunks;
+                kc = live ? kc : k_chunks - 1u;
+                gemv4s_load_pass_ref<SUB, TERMS, 1>(r, packed, scales, a_row, 0, kc, live, col, on < n, n, k / 32u, cl, k, is_lo);
+            },
+            [&](const ChunkS<SUB> &r) { gemv4s_compute<SUB, 1, TERMS>(r, dq, acc); });
+    }
+    red[wave * 64 + lane] = acc[0];
+    __syncthreads();
+    if (threadIdx.x < SUB) {
+        const uint32_t o = st * SUB + threadIdx.x;
+        if (o < n) {
+            float total = accum[o];
+            for (uint32_t s = 0; s < slots; s++) {
+                float dot = 0.f;
+                for (uint32_t q = 0; q < wps; q++)
+#pragma unroll
+                    for (int c = 0; c < CPP; c++) dot += red[(s * wps + q) * 64 + c * SUB + threadIdx.x];
+                total += weights[s] * dot;
+            }
+            accum[o] = total;
+        }
+    }
+}
+
 template <bool PAIRED, int ACT>
 __global__ __launch_bounds__(256) void k_gate_rows(const float *__restrict__ gu, float *__restrict__ out, uint32_t dim,
                                                     uint32_t batch)
@@ -243,6 +376,82 @@ hipError_t launch_bank_down_axpy(hipStream_t s, const BankView &b, const void *a
 #undef TWM_DOWN_ONE
 #undef TWM_DOWN_LAUNCH
     return hipGetLastError();
+}
+
+static RawSlab raw_slab(const RawView &v)
+{
+    RawSlab e;
+    e.packed = (const char *)v.packed;
+    e.scales = v.scales;
+    e.packed_stride = v.packed_stride;
+    e.scales_stride = v.scales_stride;
+    e.packed_offs = v.packed_offs;
+    e.scales_offs = v.scales_offs;
+    e.index = v.index;
+    return e;
+}
+
+hipError_t launch_raw_gemv(hipStream_t s, const RawView &v, const float *a, uint32_t a_slot_stride, const float *ids,
+                           uint32_t slots, float *out, int force_sub, int force_waves)
+{
+    if (slots == 0 || v.n == 0) return hipSuccess;
+    if (v.k == 0 || v.k % 32 != 0 || slots > 65535u) return hipErrorInvalidValue;
+    const uint32_t n_pad = ((v.n + 63) / 64) * 64, k_chunks = (v.k / 32 + 3) / 4;
+    const uint32_t sub = bank_sub(n_pad, slots, true, force_sub), sub_tiles = (v.n + sub - 1) / sub;
+    const uint32_t passes = (k_chunks + 64 / sub - 1) / (64 / sub);
+    uint32_t waves = passes < 16 ? passes : 16;
+    if (force_waves >= 1 && force_waves <= 16) waves = (uint32_t)force_waves;
+    const bool one = passes <= waves;
+    dim3 grid(sub_tiles, slots), block(waves * 64);
+    const size_t lds = (size_t)waves * 64 * sizeof(float);
+    const RawSlab e = raw_slab(v);
+#define TWM_RAW_LAUNCH(SUBV, ONEV) \
+    hipLaunchKernelGGL((k_raw_gemv<SUBV, ONEV>), grid, block, lds, s, e, a, a_slot_stride, ids, out, v.k, v.n, k_chunks)
+    if (sub == 16) {
+        if (one) TWM_RAW_LAUNCH(16, true);
+        else TWM_RAW_LAUNCH(16, false);
+    } else {
+        if (one) TWM_RAW_LAUNCH(32, true);
+        else TWM_RAW_LAUNCH(32, false);
+    }
+#undef TWM_RAW_LAUNCH
+    return hipGetLastError();
+}
+
+// slots beyond kMaxBankSlots: one launch per sixteen, in slot order on the stream, so the sum keeps its order
+hipError_t launch_raw_down_axpy(hipStream_t s, const RawView &v, const float *a_all, const float *ids, const float *weights,
+                                uint32_t slots, float *accum, int force_sub, int force_waves)
+{
+    if (slots == 0 || v.n == 0) return hipSuccess;
+    if (v.k == 0 || v.k % 32 != 0) return hipErrorInvalidValue;
+    const uint32_t n_pad = ((v.n + 63) / 64) * 64, k_chunks = (v.k / 32 + 3) / 4;
+    const RawSlab e = raw_slab(v);
+    for (uint32_t s0 = 0; s0 < slots; s0 += kMaxBankSlots) {
+        const uint32_t now = slots - s0 < (uint32_t)kMaxBankSlots ? slots - s0 : (uint32_t)kMaxBankSlots;
+        const uint32_t sub = bank_sub(n_pad, now, false, force_sub), sub_tiles = (v.n + sub - 1) / sub;
+        const uint32_t passes = (k_chunks + 64 / sub - 1) / (64 / sub);
+        uint32_t wps = 16 / now;
+        if (wps > passes) wps = passes;
+        if (force_waves >= 1 && (uint32_t)force_waves * now <= 16) wps = (uint32_t)force_waves;
+        if (wps == 0) wps = 1;
+        const bool one = passes <= wps;
+        const uint32_t waves = now * wps;
+        const size_t lds = (size_t)waves * 64 * sizeof(float);
+#define TWM_RAW_DOWN(SUBV, ONEV)                                                                                           \
+    hipLaunchKernelGGL((k_raw_down_axpy<SUBV, ONEV>), dim3(sub_tiles), dim3(waves * 64), lds, s, e, a_all + (size_t)s0 * v.k, \
+                       ids + s0, weights + s0, accum, v.k, v.n, k_chunks, now, wps)
+        if (sub == 16) {
+            if (one) TWM_RAW_DOWN(16, true);
+            else TWM_RAW_DOWN(16, false);
+        } else {
+            if (one) TWM_RAW_DOWN(32, true);
+            else TWM_RAW_DOWN(32, false);
+        }
+#undef TWM_RAW_DOWN
+        hipError_t err = hipGetLastError();
+        if (err != hipSuccess) return err;
+    }
+    return hipSuccess;
 }
 
 }  // namespace twm

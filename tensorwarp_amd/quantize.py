@@ -478,6 +478,28 @@ def batched_marlin_gate_up(device, input, bank, topk_ids, output, top_k, act=ACT
                                    topk_ids.ptr, top_k, act, output.ptr))
 
 
+def batched_marlin_gate_up_slabs(device, input, packed_buf, scales_buf, topk_ids, output, packed_bytes_per_expert,
+                                 scales_per_expert, n, k, top_k):
+    """moe_batched_marlin.rs:153 with the reference's own arguments: the experts' TW-Marlin arrays as they lie in the
+    two slabs, expert x at x * packed_bytes_per_expert / x * scales_per_expert; nothing is repacked."""
+    _check(device._l.twm_batched_marlin_gate_up(device.handle, input.ptr, packed_buf.ptr, scales_buf.ptr, topk_ids.ptr,
+                                                output.ptr, packed_bytes_per_expert, scales_per_expert, n, k, top_k))
+
+
+def batched_marlin_down_axpy_slabs(device, geglu_all, packed_buf, scales_buf, topk_ids, topk_weights, acc,
+                                   packed_bytes_per_expert, scales_per_expert, n, k, top_k):
+    """moe_batched_marlin.rs:184 with the reference's own arguments (slot order instead of float atomics)."""
+    _check(device._l.twm_batched_marlin_down_axpy(device.handle, geglu_all.ptr, packed_buf.ptr, scales_buf.ptr, topk_ids.ptr,
+                                                  topk_weights.ptr, acc.ptr, packed_bytes_per_expert, scales_per_expert,
+                                                  n, k, top_k))
+
+
+def gemm_tw_marlin_m1_indirect(device, a, packed_buf, packed_offsets, scales_buf, scales_offsets, expert_idx, c, n, k):
+    """quantize_indirect.rs:228 — C = A x W[expert_idx], the expert found through the two u32 device tables."""
+    _check(device._l.twm_gemm_tw_marlin_m1_indirect(device.handle, a.ptr, packed_buf.ptr, packed_offsets.ptr, scales_buf.ptr,
+                                                    scales_offsets.ptr, int(expert_idx), c.ptr, n, k))
+
+
 def batched_marlin_split_geglu(device, gate_up, output, moe_dim, top_k, paired=False):
     """moe_batched_marlin.rs:215"""
     _check(device._l.twm_geglu_rows(device.handle, gate_up.ptr, top_k, moe_dim, int(paired), output.ptr))

@@ -66,6 +66,10 @@ def test_null_handles_are_rejected_not_crashed():
     assert lib.twm_bank_gemv(None, None, None, _lib.F32, 0, None, 1, 0, None) == _lib.INVALID_HANDLE
     assert lib.twm_bank_down_axpy(None, None, None, _lib.F32, None, None, 1, None) == _lib.INVALID_HANDLE
     assert lib.twm_geglu_rows(None, None, 1, 32, 0, None) == _lib.INVALID_HANDLE
+    assert lib.twm_batched_marlin_gate_up(None, None, None, None, None, None, 0, 0, 64, 64, 1) == _lib.INVALID_HANDLE
+    assert lib.twm_batched_marlin_down_axpy(None, None, None, None, None, None, None, 0, 0, 64, 64, 1) == _lib.INVALID_HANDLE
+    assert lib.twm_batched_marlin_split_geglu(None, None, None, 32, 1) == _lib.INVALID_HANDLE
+    assert lib.twm_gemm_tw_marlin_m1_indirect(None, None, None, None, None, None, 0, None, 64, 64) == _lib.INVALID_HANDLE
     assert lib.twm_argmax_f32(None, None, 1, 1, None) == _lib.INVALID_HANDLE
     lib.twm_ctx_destroy(None)
     lib.twm_weight_destroy(None)

@@ -1389,6 +1389,97 @@ def test_bank_from_offset_tables_with_unequal_spacing(dev):
     bank.free(); bank2.free()
 
 
+@pytest.mark.parametrize("k,dim,experts,top_k", [(2816, 704, 12, 8), (96, 20, 3, 3), (1184, 100, 4, 20), (4096, 64, 2, 1)])
+def test_expert_launches_on_the_reference_slabs(dev, k, dim, experts, top_k):
+    # The reference's three MoE launches with its own arguments (moe_batched_marlin.rs:153-232): all experts' TW-Marlin
+    # arrays in two slabs, per-expert strides, ids and weights on the device; nothing is repacked.  The strides are
+    # larger than the arrays (a gap of junk between experts), f32 activations that are not f16 values.
+    n, G = 2 * dim, k // 32
+    gap_p, gap_s = 48, 5
+    pbe, spe = G * n * 16 + gap_p, G * n + gap_s
+    packed = [O.synth_packed(k, n, 5100 + 2 * e) for e in range(experts)]
+    scales = [O.synth_scales(k, n, 5101 + 2 * e) for e in range(experts)]
+    pbuf, sbuf = np.full(experts * pbe, 0xEE, np.uint8), np.full(experts * spe, 0x7BFF, np.uint16)
+    for e in range(experts):
+        pbuf[e * pbe:e * pbe + G * n * 16] = packed[e]
+        sbuf[e * spe:e * spe + G * n] = scales[e]
+    pd, sd = T.GpuTensor.from_host(dev, pbuf), T.GpuTensor.from_host(dev, sbuf, "f16")
+    ids_h = np.array([(5 * s + 1) % experts for s in range(top_k)], np.float32)
+    wts_h = (np.abs(O.synth_normal_f32(top_k, 5150)) * np.float32(0.3) + np.float32(0.01)).astype(np.float32)
+    ids, wts = T.GpuTensor.from_host(dev, ids_h), T.GpuTensor.from_host(dev, wts_h)
+    a32 = O.synth_normal_f32(k, 5151).reshape(1, k)
+    # gate + up
+    gu = T.GpuTensor.zeros(dev, (top_k, n), "f32")
+    T.batched_marlin_gate_up_slabs(dev, T.GpuTensor.from_host(dev, a32), pd, sd, ids, gu, pbe, spe, n, k, top_k)
+    rows = O.bank_gemv_f64(a32, packed, scales, ids_h, k, n)
+    guh = gu.to_host().reshape(top_k, n)
+    assert rel_err(guh, rows) < TIGHT
+    # split + GEGLU, the plain [gate | up] order
+    act = T.GpuTensor.zeros(dev, (top_k, dim), "f32")
+    T.batched_marlin_split_geglu(dev, gu, act, dim, top_k)
+    g64, u64 = guh[:, :dim].astype(np.float64), guh[:, dim:].astype(np.float64)
+    want = 0.5 * g64 * (1.0 + np.tanh(0.7978845608 * (g64 + 0.044715 * g64 ** 3))) * u64
+    assert rel_err(act.to_host().reshape(top_k, dim), want) < 1e-5
+    # down + weighted sum on a [dim -> hidden] slab: the roles of K and N swap, so build a second pair of slabs
+    kd, nd = (dim + 31) // 32 * 32, 72
+    Gd = kd // 32
+    pbe_d, spe_d = Gd * nd * 16 + 16, Gd * nd + 3
+    packed_d = [O.synth_packed(kd, nd, 5200 + 2 * e) for e in range(experts)]
+    scales_d = [O.synth_scales(kd, nd, 5201 + 2 * e) for e in range(experts)]
+    pbuf_d, sbuf_d = np.full(experts * pbe_d, 0xEE, np.uint8), np.full(experts * spe_d, 0x7BFF, np.uint16)
+    for e in range(experts):
+        pbuf_d[e * pbe_d:e * pbe_d + Gd * nd * 16] = packed_d[e]
+        sbuf_d[e * spe_d:e * spe_d + Gd * nd] = scales_d[e]
+    ad = O.synth_normal_f32(top_k * kd, 5250).reshape(top_k, kd)
+    acc0 = O.synth_normal_f32(nd, 5251)
+    acc = T.GpuTensor.from_host(dev, acc0)
+    pdd, sdd = T.GpuTensor.from_host(dev, pbuf_d), T.GpuTensor.from_host(dev, sbuf_d, "f16")
+    T.batched_marlin_down_axpy_slabs(dev, T.GpuTensor.from_host(dev, ad), pdd, sdd, ids, wts, acc, pbe_d, spe_d, nd, kd, top_k)
+    rows_d = O.bank_gemv_f64(ad, packed_d, scales_d, ids_h, kd, nd)
+    truth = acc0.astype(np.float64) + (wts_h.astype(np.float64)[:, None] * rows_d).sum(axis=0)
+    assert rel_err(acc.to_host(), truth) < TIGHT
+    acc2 = T.GpuTensor.from_host(dev, acc0)
+    T.batched_marlin_down_axpy_slabs(dev, T.GpuTensor.from_host(dev, ad), pdd, sdd, ids, wts, acc2, pbe_d, spe_d, nd, kd, top_k)
+    assert np.array_equal(acc2.to_host(), acc.to_host())          # slot order: run to run identical
+    # the same numbers as a bank built from the same slabs (other kernels, other order of the f32 sum)
+    bank = T.ExpertBank.from_device(dev, pdd, sdd, pbe_d, spe_d, kd, nd, experts)
+    acc3 = T.GpuTensor.from_host(dev, acc0)
+    for s0 in range(0, top_k, 16):
+        cnt = min(16, top_k - s0)
+        T.batched_marlin_down_axpy(dev, T.GpuTensor.from_host(dev, ad[s0:s0 + cnt]), bank,
+                                   T.GpuTensor.from_host(dev, ids_h[s0:s0 + cnt]), T.GpuTensor.from_host(dev, wts_h[s0:s0 + cnt]), acc3, cnt)
+    assert rel_err(acc3.to_host(), truth) < TIGHT
+    bank.free()
+
+
+def test_indirect_gemv_reads_the_offset_tables_on_the_device(dev):
+    # gemm_tw_marlin_m1_indirect (quantize_indirect.rs:228-253): the expert through packed_offsets[idx] / scales_offsets[idx]
+    k, n, experts = 256, 96, 4
+    G = k // 32
+    packed = [O.synth_packed(k, n, 5300 + 2 * e) for e in range(experts)]
+    scales = [O.synth_scales(k, n, 5301 + 2 * e) for e in range(experts)]
+    order, gaps_p, gaps_s = [2, 0, 3, 1], [4, 260, 0, 12], [1, 0, 7, 33]
+    pbuf, sbuf = np.full(4 * (G * n * 16 + 300), 0xEE, np.uint8), np.full(4 * (G * n + 50), 0x7BFF, np.uint16)
+    poff, soff = np.zeros(experts, np.uint32), np.zeros(experts, np.uint32)
+    pp = ss = 0
+    for e, gp, gs in zip(order, gaps_p, gaps_s):
+        pp, ss = pp + gp, ss + gs
+        poff[e], soff[e] = pp, ss
+        pbuf[pp:pp + G * n * 16] = packed[e]
+        sbuf[ss:ss + G * n] = scales[e]
+        pp, ss = pp + G * n * 16, ss + G * n
+    pd, sd = T.GpuTensor.from_host(dev, pbuf), T.GpuTensor.from_host(dev, sbuf, "f16")
+    pod, sod = T.GpuTensor.from_host(dev, poff.view(np.int32), "i32"), T.GpuTensor.from_host(dev, soff.view(np.int32), "i32")
+    a32 = O.synth_normal_f32(k, 5350).reshape(1, k)
+    ad = T.GpuTensor.from_host(dev, a32)
+    c = T.GpuTensor.zeros(dev, (n,), "f32")
+    for e in range(experts):
+        T.gemm_tw_marlin_m1_indirect(dev, ad, pd, pod, sd, sod, e, c, n, k)
+        assert rel_err(c.to_host(), O.gemm_f64(a32, packed[e], scales[e], 1, k, n)[0]) < TIGHT, e
+    with pytest.raises(T.DeviceError):
+        T.gemm_tw_marlin_m1_indirect(dev, ad, pd, pod, sd, sod, -1, c, n, k)
+
+
 # ---------------------------------------------------------------- fused projections
 
 def test_fused_qkv_and_gate_up_equal_separate_projections(dev):
