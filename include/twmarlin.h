@@ -233,6 +233,12 @@ twm_weight *twm_weight_upload(twm_ctx *ctx, const uint8_t *packed_host, const ui
 /* Same from device arrays (e.g. the output of twm_fuse_tw_marlin_n). The inputs are not retained. */
 twm_weight *twm_weight_from_device(twm_ctx *ctx, const uint8_t *packed_dev, const uint16_t *scales_dev,
                                    uint32_t k, uint32_t n);
+/* fuse_tw_marlin_n on handles (crates/kernels/src/quantize.rs:1018-1063: QKV = [h | kv | kv], gate+up = [ffn | ffn]):
+ * a new handle whose columns are those of parts[0], parts[1], ... in turn; the parts stay valid and unchanged.  Works on
+ * the repacked copies (block copies, no unpacking), so every part but the last must be a multiple of 64 columns wide --
+ * which the reference's head and ffn dimensions are; otherwise fuse the arrays (twm_fuse_tw_marlin_n) and upload.
+ * Results are bit-identical to a handle made from the fused arrays.  All parts share K and the context. */
+twm_weight *twm_weight_fuse_n(twm_ctx *ctx, const twm_weight *const *parts, uint32_t count);
 void twm_weight_destroy(twm_weight *w);
 int twm_weight_dims(const twm_weight *w, uint32_t *k, uint32_t *n);
 /* device bytes held by the repacked weight */

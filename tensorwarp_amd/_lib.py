@@ -56,6 +56,7 @@ SIGNATURES = {
     "twm_weight_upload": (_vp, [_vp, _vp, _vp, _u32, _u32]),
     "twm_weight_from_device": (_vp, [_vp, _vp, _vp, _u32, _u32]),
     "twm_weight_destroy": (None, [_vp]),
+    "twm_weight_fuse_n": (_vp, [_vp, _vp, _u32]),
     "twm_weight_dims": (_int, [_vp, C.POINTER(_u32), C.POINTER(_u32)]),
     "twm_weight_bytes": (_sz, [_vp]),
     "twm_weight_tune": (_int, [_vp, _vp, _vp, _u32]),

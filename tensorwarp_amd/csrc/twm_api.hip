@@ -812,6 +812,60 @@ twm_weight *twm_weight_from_device(twm_ctx *ctx, const uint8_t *packed_dev, cons
     return w;
 }
 
+// Fusing along N on the repacked copies is block copying: the column-lane copy is tile-major (one contiguous run per
+// input), the 16-column tile copy chunk-major (one 2-D copy per input: k_chunks rows of the input's tiles).
+twm_weight *twm_weight_fuse_n(twm_ctx *ctx, const twm_weight *const *parts, uint32_t count)
+{
+    const char *who = "twm_weight_fuse_n";
+    if (!ctx || !parts || count == 0) { api_fail(TWM_INVALID_HANDLE, "%s: null argument", who); return nullptr; }
+    if (ctx->capturing) { api_fail(TWM_UNSUPPORTED_OP, "%s: not allowed inside a graph capture", who); return nullptr; }
+    uint64_t total = 0;
+    for (uint32_t i = 0; i < count; i++) {
+        const twm_weight *p = parts[i];
+        if (!p) { api_fail(TWM_INVALID_HANDLE, "%s: part %u is null", who, i); return nullptr; }
+        if (p->ctx != ctx) { api_fail(TWM_INVALID_HANDLE, "%s: part %u belongs to another context", who, i); return nullptr; }
+        if (p->k != parts[0]->k) { api_fail(TWM_SHAPE_ERROR, "%s: part %u has K = %u, part 0 has %u", who, i, p->k, parts[0]->k); return nullptr; }
+        if (p->paired) { api_fail(TWM_UNSUPPORTED_OP, "%s: part %u is a paired gate/up weight", who, i); return nullptr; }
+        if (i + 1 < count && p->n % kNPadTo != 0) {
+            api_fail(TWM_SHAPE_ERROR, "%s: part %u has N = %u; every part but the last must be a multiple of %u columns "
+                     "(fuse the arrays with twm_fuse_tw_marlin_n instead)", who, i, p->n, kNPadTo);
+            return nullptr;
+        }
+        total += p->n;
+    }
+    if (total > 0xFFFFFFFFull) { api_fail(TWM_SHAPE_ERROR, "%s: fused N overflows u32", who); return nullptr; }
+    if (check_kn(who, parts[0]->k, (uint32_t)total)) return nullptr;
+    twm_weight *w = weight_alloc(ctx, parts[0]->k, (uint32_t)total);
+    if (!w) return nullptr;
+    const int mask = ctx->weight_copies ? ctx->weight_copies : (kCopyTile | kCopyCol);
+    for (uint32_t i = 0; i < count; i++)
+        if (weight_ensure(ctx, parts[i], mask, who)) { weight_release(w); return nullptr; }
+    if (weight_alloc_copies(w, mask, who)) { weight_release(w); return nullptr; }
+    hipError_t e = hipSuccess;
+    uint32_t t16 = 0;  // 16-column tiles before this part
+    for (uint32_t i = 0; i < count && e == hipSuccess && w->copy_bytes; i++) {
+        const twm_weight *p = parts[i];
+        if (p->n_tiles == 0) continue;
+        if (w->cq)
+            e = hipMemcpyAsync((char *)w->cq + (size_t)(t16 / 4) * w->k_chunks * kColBlockBytes, p->cq,
+                               (size_t)(p->n_tiles / 4) * p->k_chunks * kColBlockBytes, hipMemcpyDeviceToDevice, ctx->stream);
+        if (e == hipSuccess && w->qw)
+            e = hipMemcpy2DAsync((char *)w->qw + (size_t)t16 * 1024, (size_t)w->n_tiles * 1024, p->qw, (size_t)p->n_tiles * 1024,
+                                 (size_t)p->n_tiles * 1024, w->k_chunks, hipMemcpyDeviceToDevice, ctx->stream);
+        if (e == hipSuccess && w->qw)
+            e = hipMemcpy2DAsync((char *)w->sc + (size_t)t16 * 128, (size_t)w->n_tiles * 128, p->sc, (size_t)p->n_tiles * 128,
+                                 (size_t)p->n_tiles * 128, w->k_chunks, hipMemcpyDeviceToDevice, ctx->stream);
+        t16 += p->n_tiles;
+    }
+    if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
+    if (e != hipSuccess) {
+        api_fail(TWM_DEVICE_ERROR, "%s: copy: %s", who, hipGetErrorString(e));
+        weight_release(w);
+        return nullptr;
+    }
+    return w;
+}
+
 twm_weight *twm_weight_upload(twm_ctx *ctx, const uint8_t *packed_host, const uint16_t *scales_host, uint32_t k,
                               uint32_t n)
 {

@@ -280,6 +280,16 @@ class MarlinWeight:
         return cls(device, h, k, n)
 
     @classmethod
+    def fuse_n(cls, device, parts):
+        """fuse_tw_marlin_n (quantize.rs:1018) on handles: the parts' columns side by side in a new handle."""
+        import ctypes
+        arr = (ctypes.c_void_p * len(parts))(*[p.handle for p in parts])
+        h = device._l.twm_weight_fuse_n(device.handle, arr, len(parts))
+        if not h:
+            raise DeviceError(_lib.SHAPE_ERROR, device._l.twm_last_error().decode())
+        return cls(device, h, parts[0].k, sum(p.n for p in parts))
+
+    @classmethod
     def gate_up(cls, device, gate, up, k, ffn_dim):
         """Paired gate/up weight for gemm_swiglu; gate and up are (packed, scales) device pairs."""
         h = device._l.twm_weight_gate_up(device.handle, gate[0].ptr, gate[1].ptr, up[0].ptr, up[1].ptr, k, ffn_dim)

@@ -58,6 +58,7 @@ def test_null_handles_are_rejected_not_crashed():
     assert lib.twm_pair_gate_up(None, None, None, None, None, 64, 64, None, None) == _lib.INVALID_HANDLE
     assert lib.twm_weight_gate_up(None, None, None, None, None, 64, 64) is None
     assert lib.twm_weight_is_paired(None) == 0
+    assert lib.twm_weight_fuse_n(None, None, 0) is None
     assert lib.twm_weight_blob_bytes(None) == 0
     assert lib.twm_weight_export(None, None, None, 0) == _lib.INVALID_HANDLE
     assert lib.twm_weight_import(None, None, 0) is None

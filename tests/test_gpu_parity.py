@@ -1482,6 +1482,43 @@ def test_indirect_gemv_reads_the_offset_tables_on_the_device(dev):
 
 # ---------------------------------------------------------------- fused projections
 
+def test_fusing_handles_equals_fusing_the_arrays(dev):
+    # fuse_tw_marlin_n (quantize.rs:1018-1063) on repacked handles: block copies of both copies; the results of every
+    # kernel family are bit-identical to those of a handle made from the fused arrays
+    k, ns = 1184, [128, 64, 200]      # K not a multiple of 128; the last part is ragged
+    host = [(O.synth_packed(k, n, 5400 + i), O.synth_scales(k, n, 5450 + i)) for i, n in enumerate(ns)]
+    devp = [(T.GpuTensor.from_host(dev, p), T.GpuTensor.from_host(dev, s, "f16")) for p, s in host]
+    parts = [T.MarlinWeight.from_device(dev, p, s, k, n) for (p, s), n in zip(devp, ns)]
+    fused = T.MarlinWeight.fuse_n(dev, parts)
+    fp, fs = O.fuse_tw_marlin_n(host, k, ns)
+    ref = T.MarlinWeight.upload(dev, fp, fs, k, sum(ns))
+    assert fused.n == sum(ns) and fused.copies == 3
+    for m in (1, 4, 8, 32, 96):
+        a16 = O.synth_act_f16(m, k, 5500 + m)
+        a_dev = T.GpuTensor.from_host(dev, a16, "f16")
+        c1, c2 = T.GpuTensor.zeros(dev, (m, sum(ns)), "f32"), T.GpuTensor.zeros(dev, (m, sum(ns)), "f32")
+        T.gemm(dev, fused, a_dev, m, c1)
+        T.gemm(dev, ref, a_dev, m, c2)
+        assert np.array_equal(c1.to_host(), c2.to_host()), m
+    truth = O.gemm_f64(f16_as_f32(O.synth_act_f16(1, k, 5501)), fp, fs, 1, k, sum(ns))
+    c = T.GpuTensor.zeros(dev, (1, sum(ns)), "f32")
+    T.gemm(dev, fused, T.GpuTensor.from_host(dev, O.synth_act_f16(1, k, 5501), "f16"), 1, c)
+    assert rel_err(c.to_host().reshape(1, -1), truth) < TIGHT
+    # a part in the middle that is not a multiple of 64 columns wide cannot be block-copied
+    with pytest.raises(T.DeviceError):
+        T.MarlinWeight.fuse_n(dev, [parts[2], parts[0]])
+    # handles with one copy: the fused handle follows the option, missing copies of the parts are built
+    dev.set_option("weight_copies", 2)
+    one = T.MarlinWeight.fuse_n(dev, parts)
+    dev.set_option("weight_copies", 0)
+    assert one.copies == 2
+    c3 = T.GpuTensor.zeros(dev, (1, sum(ns)), "f32")
+    T.gemm(dev, one, T.GpuTensor.from_host(dev, O.synth_act_f16(1, k, 5501), "f16"), 1, c3)
+    assert np.array_equal(c3.to_host(), c.to_host())
+    for w in parts + [fused, ref, one]:
+        w.free()
+
+
 def test_fused_qkv_and_gate_up_equal_separate_projections(dev):
     # fused-vs-unfused equality, the check the reference makes for F32 weights only
     # (transformer.rs:2230-2287), here on TW-Marlin weights and bit for bit
