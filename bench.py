@@ -436,6 +436,36 @@ def main():
     drop_in["layer_us"] = round(sum(v["us"] for v in drop_in.values()), 2)
 
 
+    log("f32 activations on the repacked handles")
+    # what a caller gets that keeps the reference's f32 activation buffers (twm_gemm with TWM_F32): per projection, and the
+    # layer as one graph over the rotating layers
+    f32_rows = {}
+    a32s = {name: T.GpuTensor.from_host(dev, layers_host[0][name][2].view(np.float16).astype(np.float32)) for name, k, n in LAYER_7B}
+    for name, k, n in LAYER_7B:
+        def one(i, name=name):
+            w, _, c = layers[i % args.layers][name]
+            T.gemm(dev, w, a32s[name], 1, c)
+        for i in range(8):
+            one(i)
+        dev.synchronize()
+        ms, how = time_short_launches(dev, T_graphs, one, 104, graphs_done)
+        b = k * n // 2 + (k // 32) * n * 2 + k * 4 + n * 4
+        f32_rows[name] = {"us": round(ms * 1e3, 2), "GBps": round(b / (ms * 1e-3) / 1e9, 1), "timed": how}
+
+    def run_all_f32():
+        for li in range(L):
+            for name, k, n in LAYER_7B:
+                T.gemm(dev, layers[li][name][0], a32s[name], 1, layers[li][name][2])
+    if not graphs_off:
+        g32 = capture(run_all_f32)
+        for _ in range(3):
+            g32.replay()
+        dev.synchronize()
+        f32_rows["layer_us"] = round(time_launches(dev, lambda i: g32.replay(), max(8, steps // L)) / L * 1e3, 2)
+        graphs_done.append(g32)
+    else:
+        f32_rows["layer_us"] = round(sum(v["us"] for v in f32_rows.values()), 2)
+
     gu = per_shape["gate_up"]
     gu_bytes = algo_bytes(3584, 37888)
     roofline = {"bound": "hbm", "kernel": "k_gemv4s (gate_up 3584->37888, M=1)",
@@ -916,6 +946,7 @@ def main():
         "cpu_baseline": cpu,
         "per_projection": per_shape,
         "drop_in_reference_layout_m1": drop_in,
+        "f32_activations_m1": f32_rows,
     }
     out["small_shapes_m1"] = small
     if lm:

@@ -625,13 +625,15 @@ extern "C++" int twm::m1_dispatch(const M1Env &env, const char *who, const float
     uint32_t n_pad = ((n + 63) / 64) * 64, k_chunks = (k / 32 + kChunkGroups - 1) / kChunkGroups;
     // On the reference's arrays a wave's four group rows of a chunk are N x 16 bytes apart, and many waves in flight
     // with one pass each pay better than on the contiguous copy: the sub-tile kernel with sixteen waves on 32
-    // columns, or with 16 columns when 64-column tiles number no more than 64 -- as long as every wave gets a
-    // single pass (K <= 4096, or 8192 on 16 columns).  Deeper matrices keep the 64-column kernel and its split-K
-    // (8192 -> 57344: 46.6 against 63.7 us; 14336 -> 4096: 11.0 against 12.5).  Fitted to sweeps over the
+    // columns as long as every wave gets a single pass (K <= 4096), or with 16 columns when 64-column tiles number no
+    // more than 64.  Deeper wide matrices keep the 64-column kernel and its split-K (8192 -> 57344: 46.6 against
+    // 63.7 us).  Fitted to sweeps over the
     // Qwen2.5-7B, Llama-3-8B, 13B and 70B projections; option "sub" = 1 keeps the 64-column kernel.
     const uint32_t tiles64 = n_pad / 64, passes16 = (k_chunks + 3) / 4, passes32 = (k_chunks + 1) / 2;
     uint32_t sub = tiles64 <= 64 ? 16 : 32, sub_waves = (sub == 16 && passes16 <= 8) ? 8 : 16;
-    bool use_sub = env.force_sub != 1 && (sub == 16 ? passes16 : passes32) <= 16;
+    // (on 16 columns a deeper K runs the pipelined pass loop on sixteen waves: 18944 -> 3584 12.5 against 12.8 us,
+    // 14336 -> 4096 10.8 against 11.7)
+    bool use_sub = env.force_sub != 1 && (sub == 16 || passes32 <= 16);
     if (env.force_sub >= 16) {
         sub = (uint32_t)env.force_sub;
         sub_waves = 8;
@@ -1128,7 +1130,8 @@ static SubPlan plan_gemv4_sub(uint32_t tiles64, uint32_t k_chunks, uint32_t m, b
     // waves per workgroup on 16 columns: one pass each while eight or sixteen cover K; deeper, the pipelined pass loop
     // on eight waves for one row and on four from two rows on (18944 -> 3584: M = 1 8.96 / 9.01 / 9.05 us on 8 / 4 / 16
     // waves, M = 2 9.5 / 9.2 / 9.7, M = 4 11.2 / 10.75 / 11.75)
-    const SubPlan narrow16 = {16, passes16 <= 8 ? 8u : passes16 <= 16 ? 16u : (m >= 2 && !a_f32) ? 4u : 8u};
+    // (one row of f32 activations, which a lane takes as one shared piece: 9.3 / 9.6 us on 4 / 8 waves)
+    const SubPlan narrow16 = {16, passes16 <= 8 ? 8u : passes16 <= 16 ? 16u : ((m >= 2 && !a_f32) || (m == 1 && a_f32)) ? 4u : 8u};
     if (tiles64 > 128) {
         // wide matrices: only the cheapest activations (f16, up to two rows) leave the sub-tiles ahead
         // (3584 -> 37888: 15.8 against 17.0 us at M = 1, 18.3 against 17.3 at M = 4, 19.9 against 17.9 with f32 rows)
@@ -1143,6 +1146,9 @@ static SubPlan plan_gemv4_sub(uint32_t tiles64, uint32_t k_chunks, uint32_t m, b
         // (several workgroups per CU: no idle eighth wave, 3584 -> 37888 at M = 1 14.8 against 15.3 us; with one workgroup
         // per CU the eight-wave form is the faster one, 3584 -> 3584 3.9 against 4.05)
         if (!a_f32 && m <= 2 && passes16 <= 8 && poor_fill) return SubPlan{16, passes16};
+        // one row of f32 activations: the shared-piece form in the pipelined loop on four waves (3584 -> 37888: 15.75 us
+        // against 17.0 with one pass per wave and 16.8 on whole tiles)
+        if (a_f32 && m == 1 && passes16 <= 8 && poor_fill) return SubPlan{16, 4};
         if (a_f32 && m <= 2 && tiles64 < 256 && k_chunks <= 32) return SubPlan{32, 16};
         return none;
     }

@@ -79,7 +79,8 @@ __device__ __forceinline__ void split_f32x8(const float (&v)[8], uint4v &hi, uin
 // largest below 2^15 (exact), and inv[i] is what the sums of A row i are multiplied by afterwards (exact as well): the
 // results come out as with unbounded terms.  In range every factor is 1 and nothing is touched, at the price of a
 // maximum over the lane's values and one vote per call.  (Infinities and NaNs stay what they are.)
-template <int NV>
+// ONE_ROW: every lane of the wave holds values of the same activation row: one factor for the wave.
+template <int NV, bool ONE_ROW = false>
 __device__ __forceinline__ void f32_terms_range(float (&v)[NV], float (&inv)[4])
 {
     float m = 0.f;
@@ -90,7 +91,7 @@ __device__ __forceinline__ void f32_terms_range(float (&v)[NV], float (&inv)[4])
     if (__builtin_amdgcn_ballot_w64(!(m <= 65000.f)) == 0) return;
     if (!(m == m)) m = __builtin_inff();  // (fmaxf drops a NaN; the vote saw it through the negated comparison)
 #pragma unroll
-    for (int off = 32; off >= 4; off >>= 1) m = fmaxf(m, __shfl_xor(m, off, 64));   // over the lanes of this row
+    for (int off = 32; off >= (ONE_ROW ? 1 : 4); off >>= 1) m = fmaxf(m, __shfl_xor(m, off, 64));   // over the lanes of this row
     float mine = 1.f;
     if (m > 16384.f) {
         const uint32_t e = (__float_as_uint(m) >> 23) & 0xFFu;       // biased exponent of the row's largest value, >= 141
@@ -98,6 +99,11 @@ __device__ __forceinline__ void f32_terms_range(float (&v)[NV], float (&inv)[4])
 #pragma unroll
         for (int i = 0; i < NV; i++) v[i] *= down;
         mine = __uint_as_float((e - 14u) << 23);                     // 2^((e - 127) - 14)
+    }
+    if (ONE_ROW) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) inv[i] = mine;
+        return;
     }
     const int quad = (int)(__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u)) & ~3u);
 #pragma unroll
@@ -115,10 +121,13 @@ __device__ __forceinline__ float4v mfma_piece(half4v a, half4v b, float4v c)
 // Term modes of the activations: one f16 term; two terms as two MFMA passes (a_lo holds the second); or, for
 // at most two rows, two terms packed into the four MFMA rows (lane l: row (l % 4) / 2, term l % 2), which
 // costs no extra MFMA: the 4x4x4 instruction computes four rows anyway.
-enum { kTermsOne = 0, kTermsTwoPasses = 1, kTermsRowPacked = 2, kTermsOneRow = 3 };
+enum { kTermsOne = 0, kTermsTwoPasses = 1, kTermsRowPacked = 2, kTermsOneRow = 3, kTermsOneRowF32 = 4 };
 // kTermsOneRow (sub-tile kernels, one row of f16 activations): a lane loads ONE 8-wide piece of its chunk instead of the
 // 64 / SUB pieces its MFMA block supplies, and the unpack hands the pieces round inside each quad of lanes
 // (gemv4s_load_a, gemv4s_compute).
+// kTermsOneRowF32: the same for one row of f32 activations: a lane loads and splits ONE piece (a and a_lo hold its two
+// f16 terms), and the unpack hands both terms round the quad: lanes 0 and 2 of a quad take the first term, lanes 1 and 3
+// the residual, so that rows 0 and 1 of the MFMA's A block are the two terms (rows 2 and 3 repeat them, unused).
 template <bool AF32, int RL>
 constexpr int gemv4_terms() { return AF32 ? (RL <= 2 ? kTermsRowPacked : kTermsTwoPasses) : kTermsOne; }
 
@@ -290,6 +299,43 @@ __device__ __forceinline__ void gemv4s_load_a_f32(float (&v)[64 / SUB * 8], cons
     }
 }
 
+// The lane's one piece of a row of f32 activations (kTermsOneRowF32): piece cl on 16 columns; on 32 columns the lanes
+// of MFMA block b (cl / 4) hold pieces 2 b and 2 b + 1 in turn.  The eight values stay as they were loaded, in a[0][0]
+// and a_lo[0] (nothing here waits for them); gemv4s_compute checks their range and splits them.
+template <int SUB, bool REF_ORDER, int RG>
+__device__ __forceinline__ void gemv4s_load_a_f32_piece(ChunkS<SUB, RG> &r, const void *a_any, uint32_t arow, uint32_t kc,
+                                                        uint32_t cl, uint32_t k)
+{
+    const uint32_t piece = SUB == 16 ? cl : (cl >> 2) * 2u + (cl & 1u);
+    uint32_t k0 = kc * 128u + piece * 8u;
+    if (k0 > k - 8u) k0 = k - 8u;  // only the zero-padded groups of a last partial chunk get here
+    const uint4v *p = (const uint4v *)((const float *)a_any + (size_t)arow * k + k0);
+    r.a[0][0] = p[0];
+    r.a_lo[0] = p[1];
+}
+
+// ... and the split, when the values are needed: two f16 terms of the eight values in the k order of the unpack
+template <bool REF_ORDER>
+__device__ __forceinline__ void gemv4s_split_a_f32_piece(uint4v x, uint4v y, uint4v &hi, uint4v &lo, float (&inv)[4])
+{
+    float v[8] = {__uint_as_float(x[0]), __uint_as_float(REF_ORDER ? y[0] : x[1]), __uint_as_float(REF_ORDER ? x[1] : x[2]),
+                  __uint_as_float(REF_ORDER ? y[1] : x[3]), __uint_as_float(REF_ORDER ? x[2] : y[0]),
+                  __uint_as_float(REF_ORDER ? y[2] : y[1]), __uint_as_float(REF_ORDER ? x[3] : y[2]), __uint_as_float(y[3])};
+    f32_terms_range<8, true>(v, inv);
+    // Both terms rounded toward zero, two values per instruction: the first term need not be the nearest f16, only
+    // near enough for the residual a - hi to be exact in f32 (it is: below one f16 step of a), and a residual cut by
+    // one of its own steps is 2^-21 of a.  A value that is an f16 gets hi = a, lo = 0 either way.
+    typedef __fp16 pk2 __attribute__((ext_vector_type(2)));
+    union { pk2 p[4]; uint4v u; } ch, cl;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        ch.p[i] = __builtin_amdgcn_cvt_pkrtz(v[2 * i], v[2 * i + 1]);
+        cl.p[i] = __builtin_amdgcn_cvt_pkrtz(v[2 * i] - (float)ch.p[i][0], v[2 * i + 1] - (float)ch.p[i][1]);
+    }
+    hi = ch.u;
+    lo = cl.u;
+}
+
 template <int SUB, int TERMS, int RG>
 __device__ __forceinline__ void gemv4s_split_a_f32(ChunkS<SUB, RG> &r, float (&v)[64 / SUB * 8], bool lane_is_lo)
 {
@@ -325,6 +371,11 @@ __device__ __forceinline__ void gemv4s_load_a(ChunkS<SUB, RG> &r, const void *a_
         uint32_t k0 = kc * 128u + piece * 8u;
         if (k0 > k - 8u) k0 = k - 8u;  // only the zero-padded groups of a last partial chunk get here
         r.a[0][0] = *(const uint4v *)((const _Float16 *)a_any + (size_t)arow * k + k0);
+        return;
+    }
+    if (TERMS == kTermsOneRowF32) {
+        static_assert(TERMS != kTermsOneRowF32 || (AF32 && RG == 1), "one row of f32 activations");
+        gemv4s_load_a_f32_piece<SUB, REF_ORDER, RG>(r, a_any, arow, kc, cl, k);
         return;
     }
     if (AF32) {
@@ -384,8 +435,10 @@ __device__ __forceinline__ void gemv4s_load_pass_ref(ChunkS<SUB, RG> &r, const c
                                                      bool col_ok, uint32_t n, uint32_t groups, uint32_t cl, uint32_t k,
                                                      bool lane_is_lo)
 {
+    constexpr bool PIECE = TERMS == kTermsOneRowF32;
     float av[64 / SUB * 8];
-    gemv4s_load_a_f32<SUB, true>(av, a_any, arow, kc, cl, k);
+    if constexpr (PIECE) gemv4s_load_a_f32_piece<SUB, true, RG>(r, a_any, arow, kc, cl, k);
+    else gemv4s_load_a_f32<SUB, true>(av, a_any, arow, kc, cl, k);
     __builtin_amdgcn_sched_barrier(0);
     uint4v wq[4];
     uint32_t sb[4];
@@ -406,32 +459,40 @@ __device__ __forceinline__ void gemv4s_load_pass_ref(ChunkS<SUB, RG> &r, const c
     r.sc = uint2v{(sb[0] | (sb[1] << 16)) & (keep[0] | (keep[1] << 16)), (sb[2] | (sb[3] << 16)) & (keep[2] | (keep[3] << 16))};
     r.live = true;  // (masked group by group above)
     __builtin_amdgcn_sched_barrier(0);
-    gemv4s_split_a_f32<SUB, TERMS, RG>(r, av, lane_is_lo);
+    if constexpr (!PIECE) gemv4s_split_a_f32<SUB, TERMS, RG>(r, av, lane_is_lo);
 }
 
+// lanes (A, B, C, D) of every quad of lanes, in its lanes 0 .. 3
+template <int A, int B, int C, int D>
+__device__ __forceinline__ uint4v quad_perm(uint4v v)
+{
+    uint4v o;
+#pragma unroll
+    for (int w = 0; w < 4; w++) o[w] = (uint32_t)__builtin_amdgcn_mov_dpp((int)v[w], A | (B << 2) | (C << 4) | (D << 6), 0xF, 0xF, true);
+    return o;
+}
 // lane I of every quad of lanes, in all four lanes of the quad
 template <int I>
 __device__ __forceinline__ uint4v quad_bcast(uint4v v)
 {
-    uint4v o;
-#pragma unroll
-    for (int w = 0; w < 4; w++) o[w] = (uint32_t)__builtin_amdgcn_mov_dpp((int)v[w], I * 0x55, 0xF, 0xF, true);  // quad_perm [I,I,I,I]
-    return o;
+    return quad_perm<I, I, I, I>(v);
 }
 
 // acc[row] += f32(scale) * (sum over the group of A * (q - 8)) for the four groups of the lane's chunk
-template <int SUB, int RL, int TERMS>
+// (REF_ORDER: kTermsOneRowF32 on the reference's nibble order, whose unpack yields k (0,4,1,5 | 2,6,3,7) per eight)
+template <int SUB, int RL, int TERMS, bool REF_ORDER = false>
 __device__ __forceinline__ void gemv4s_compute(const ChunkS<SUB, (RL + 3) / 4> &r, const Gemv4Consts &dq, float (&acc)[RL])
 {
     constexpr int PIECES = SUB / 4;  // 8-wide k pieces per A register
     constexpr int RG = (RL + 3) / 4;
     static_assert(TERMS != kTermsRowPacked || RL <= 2, "row-packed terms hold at most two rows");
     static_assert(RG == 1 || TERMS == kTermsOne, "more than four rows: one f16 term");
-    static_assert(TERMS != kTermsOneRow || RL == 1, "the shared-piece form holds one row");
+    static_assert((TERMS != kTermsOneRow && TERMS != kTermsOneRowF32) || RL == 1, "the shared-piece forms hold one row");
     union { uint2v u; _Float16 h[4]; } sv;
     sv.u = r.sc;
     // kTermsOneRow: the piece held by lane i of every quad, in all four lanes of the quad (row 0 is the one that counts)
-    constexpr int QN = TERMS == kTermsOneRow ? (SUB == 16 ? 4 : 2) : 1;
+    constexpr bool SHARED = TERMS == kTermsOneRow || TERMS == kTermsOneRowF32;
+    constexpr int QN = SHARED ? (SUB == 16 ? 4 : 2) : 1;
     uint4v quad[QN];
     if (TERMS == kTermsOneRow) {
         quad[0] = r.a[0][0];
@@ -439,6 +500,29 @@ __device__ __forceinline__ void gemv4s_compute(const ChunkS<SUB, (RL + 3) / 4> &
         if (QN > 2) {
             quad[2 % QN] = quad_bcast<2>(r.a[0][0]);
             quad[3 % QN] = quad_bcast<3>(r.a[0][0]);
+        }
+    }
+    float inv1[4] = {1.f, 1.f, 1.f, 1.f};
+    if (TERMS == kTermsOneRowF32) {
+        uint4v hi, lo;
+        gemv4s_split_a_f32_piece<REF_ORDER>(r.a[0][0], r.a_lo[0], hi, lo, inv1);
+        // Rows 0 and 1 of an A block (lanes 0 and 1 of a quad) must be the two terms of one piece; rows 2 and 3 do not
+        // count.  Lanes (0, 1) and (2, 3) swap one term each: z holds (first, residual) of the even lanes' pieces in
+        // lanes (0, 1) and (2, 3), z2 those of the odd lanes' pieces.  On 16 columns a quad holds four pieces (lane i
+        // piece i of its block's four); on 32 columns two (lanes 0, 2 and 1, 3 hold the same).
+        const bool odd = (threadIdx.x & 1u) != 0;
+        const uint4v hs = quad_perm<1, 0, 3, 2>(hi), ls = quad_perm<1, 0, 3, 2>(lo);
+        uint4v z, z2;
+#pragma unroll
+        for (int w = 0; w < 4; w++) {
+            z[w] = odd ? ls[w] : hi[w];
+            z2[w] = odd ? lo[w] : hs[w];
+        }
+        quad[0] = z;
+        if (QN > 1) quad[1 % QN] = z2;
+        if (QN > 2) {
+            quad[2 % QN] = quad_perm<2, 3, 2, 3>(z);
+            quad[3 % QN] = quad_perm<2, 3, 2, 3>(z2);
         }
     }
 #pragma unroll
@@ -451,7 +535,7 @@ __device__ __forceinline__ void gemv4s_compute(const ChunkS<SUB, (RL + 3) / 4> &
         // (4g + W) % PIECES of the lane group
 #define TWM_SUB_PIECE(W)                                                                   \
     {                                                                                      \
-        constexpr int PG = 4 * G + W, ONE_ROW = TERMS == kTermsOneRow;                     \
+        constexpr int PG = 4 * G + W, ONE_ROW = SHARED;                                    \
         constexpr int J = ONE_ROW ? 0 : PG / PIECES;                                       \
         /* one row: piece PG sits in MFMA block PG / 4, lane PG % 4 (16 columns) or block PG / 2, lane PG % 2 */ \
         constexpr int ABID = ONE_ROW ? (SUB == 16 ? PG / 4 : PG / 2) : PG % PIECES;        \
@@ -481,7 +565,8 @@ __device__ __forceinline__ void gemv4s_compute(const ChunkS<SUB, (RL + 3) / 4> &
 #pragma unroll
         for (int rr = 0; rr < RL; rr++) {
             // (a_inv: 1 unless the f32 activations of that row were scaled into the f16 range)
-            if (TERMS == kTermsRowPacked) acc[rr] = fmaf(d[0][2 * rr] + d[0][2 * rr + 1], s * r.a_inv[2 * rr], acc[rr]);
+            if (TERMS == kTermsOneRowF32) acc[rr] = fmaf(d[0][0] + d[0][1], s * inv1[0], acc[rr]);
+            else if (TERMS == kTermsRowPacked) acc[rr] = fmaf(d[0][2 * rr] + d[0][2 * rr + 1], s * r.a_inv[2 * rr], acc[rr]);
             else if (TERMS == kTermsTwoPasses) acc[rr] = fmaf(d[0][rr], s * r.a_inv[rr], acc[rr]);
             else acc[rr] = fmaf(d[rr / 4][rr % 4], s, acc[rr]);
         }

@@ -53,8 +53,11 @@ __device__ __forceinline__ void gemv4s_body(const char *__restrict__ cw, const v
     // one row the shared-piece form of the activations (18944 -> 3584: 8.9 against 10.0 us at M = 1, 9.95 against 10.35
     // at M = 2, level at M = 4).  A wave that makes a single pass gains nothing from either, and the other variants
     // run out of registers with both sets live.
-    constexpr bool PIPE = !ONE && !AF32 && RL <= 4 && SUB == 16 && !REFL;
-    constexpr int TERMS = (PIPE && RL == 1) ? kTermsOneRow : gemv4_terms<AF32, RL>();
+    // One row of f32 activations: the shared-piece form as well (a lane splits one piece instead of two or four),
+    // which on 16 columns also leaves room for the pipelined loop.
+    constexpr bool F32_PIECE = AF32 && RL == 1;
+    constexpr bool PIPE = !ONE && (!AF32 || F32_PIECE) && RL <= 4 && SUB == 16;
+    constexpr int TERMS = F32_PIECE ? kTermsOneRowF32 : (PIPE && RL == 1) ? kTermsOneRow : gemv4_terms<AF32, RL>();
     extern __shared__ float red[];    // [waves][RL][64]
     __shared__ int s_last;
 
@@ -84,7 +87,7 @@ __device__ __forceinline__ void gemv4s_body(const char *__restrict__ cw, const v
     const uint32_t ref_groups = k / 32u;
     const Gemv4Consts dq = make_gemv4_consts();
 
-    uint32_t arow = TERMS == kTermsRowPacked ? (cl & 3u) >> 1 : cl & 3u;
+    uint32_t arow = (TERMS == kTermsOneRow || TERMS == kTermsOneRowF32) ? 0u : TERMS == kTermsRowPacked ? (cl & 3u) >> 1 : cl & 3u;
     if (arow > m_rows - 1) arow = m_rows - 1;
     const bool lane_is_lo = TERMS == kTermsRowPacked && (cl & 1u) != 0;
 
@@ -105,13 +108,17 @@ __device__ __forceinline__ void gemv4s_body(const char *__restrict__ cw, const v
                 // activations first: loads complete in the order of their issue, and these come from the cache
                 gemv4s_load_a<SUB, AF32, TERMS, REFL, RG>(r, a_any, arow, kc, cl, k, lane_is_lo, m_rows);
                 gemv4s_load_w<SUB, RG, true>(r, tbase + (size_t)kc * kColBlockBytes, col_in_tile(cl), live);
+            } else if (F32_PIECE) {
+                // (the same order: the split of the f32 piece can then run while the weights are on their way)
+                gemv4s_load_a<SUB, AF32, TERMS, REFL, RG>(r, a_any, arow, kc, cl, k, lane_is_lo, m_rows);
+                gemv4s_load_w<SUB, RG, false>(r, tbase + (size_t)kc * kColBlockBytes, col_in_tile(cl), live);
             } else {
                 gemv4s_load_w<SUB, RG, false>(r, tbase + (size_t)kc * kColBlockBytes, col_in_tile(cl), live);
                 gemv4s_load_a<SUB, AF32, TERMS, REFL, RG>(r, a_any, arow, kc, cl, k, lane_is_lo, m_rows);
             }
         }
     };
-    auto compute_pass = [&](const ChunkS<SUB, RG> &r) { gemv4s_compute<SUB, RL, TERMS>(r, dq, acc); };
+    auto compute_pass = [&](const ChunkS<SUB, RG> &r) { gemv4s_compute<SUB, RL, TERMS, REFL>(r, dq, acc); };
     // (ONE: the launcher saw that no wave has a second pass: one register set, no loop)
     gemv4s_run_passes<SUB, ONE, RG, PIPE>(wave, waves, passes, load_pass, compute_pass);
     if (trace_loaded && threadIdx.x == 0) *trace_loaded = (uint32_t)__builtin_amdgcn_s_memrealtime();  // data arrived and unpacked

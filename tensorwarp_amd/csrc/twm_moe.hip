@@ -43,7 +43,7 @@ __global__ __launch_bounds__(1024) void k_bank_gemv(const char *__restrict__ ban
                                                      uint32_t k, uint32_t n, uint32_t k_chunks, uint32_t sub_tiles)
 {
     constexpr int CPP = 64 / SUB;
-    constexpr int TERMS = gemv4_terms<AF32, 1>();   // one row: f32 activations as two row-packed terms
+    constexpr int TERMS = AF32 ? kTermsOneRowF32 : kTermsOne;   // one row: f32 activations as two f16 terms of one shared piece per lane
     extern __shared__ float red[];  // [waves][64]
     const uint32_t st = blockIdx.x, slot = blockIdx.y;
     if (st >= sub_tiles) return;
@@ -103,7 +103,7 @@ __global__ __launch_bounds__(1024) void k_bank_down_axpy(const char *__restrict_
                                                           uint32_t slots, uint32_t wps)
 {
     constexpr int CPP = 64 / SUB;
-    constexpr int TERMS = gemv4_terms<AF32, 1>();
+    constexpr int TERMS = AF32 ? kTermsOneRowF32 : kTermsOne;
     extern __shared__ float red[];  // [slots * wps][64]
     const uint32_t st = blockIdx.x;
     if (st >= sub_tiles) return;
@@ -188,7 +188,7 @@ __global__ __launch_bounds__(1024) void k_raw_gemv(RawSlab e, const float *__res
                                                     uint32_t n, uint32_t k_chunks)
 {
     constexpr int CPP = 64 / SUB;
-    constexpr int TERMS = gemv4_terms<true, 1>();
+    constexpr int TERMS = kTermsOneRowF32;
     extern __shared__ float red[];  // [waves][64]
     const uint32_t st = blockIdx.x, slot = blockIdx.y;
     const uint32_t waves = blockDim.x >> 6;
@@ -213,7 +213,7 @@ __global__ __launch_bounds__(1024) void k_raw_gemv(RawSlab e, const float *__res
                 kc = live ? kc : k_chunks - 1u;
                 gemv4s_load_pass_ref<SUB, TERMS, 1>(r, packed, scales, a_row, 0, kc, live, col, on < n, n, k / 32u, cl, k, is_lo);
             },
-            [&](const ChunkS<SUB> &r) { gemv4s_compute<SUB, 1, TERMS>(r, dq, acc); });
+            [&](const ChunkS<SUB> &r) { gemv4s_compute<SUB, 1, TERMS, true>(r, dq, acc); });
     }
     red[wave * 64 + lane] = acc[0];
     __syncthreads();
@@ -237,7 +237,7 @@ __global__ __launch_bounds__(1024) void k_raw_down_axpy(RawSlab e, const float *
                                                          uint32_t n, uint32_t k_chunks, uint32_t slots, uint32_t wps)
 {
     constexpr int CPP = 64 / SUB;
-    constexpr int TERMS = gemv4_terms<true, 1>();
+    constexpr int TERMS = kTermsOneRowF32;
     extern __shared__ float red[];  // [slots * wps][64]
     const uint32_t st = blockIdx.x;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -262,7 +262,7 @@ __global__ __launch_bounds__(1024) void k_raw_down_axpy(RawSlab e, const float *
                 kc = live ? kc : k_chunks - 1u;
                 gemv4s_load_pass_ref<SUB, TERMS, 1>(r, packed, scales, a_row, 0, kc, live, col, on < n, n, k / 32u, cl, k, is_lo);
             },
-            [&](const ChunkS<SUB> &r) { gemv4s_compute<SUB, 1, TERMS>(r, dq, acc); });
+            [&](const ChunkS<SUB> &r) { gemv4s_compute<SUB, 1, TERMS, true>(r, dq, acc); });
     }
     red[wave * 64 + lane] = acc[0];
     __syncthreads();

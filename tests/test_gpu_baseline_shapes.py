@@ -144,6 +144,29 @@ def test_batched_decode_qwen7b_all_projections(dev, m, name):
     w.free()
 
 
+@pytest.mark.parametrize("name", list(SHAPES_7B))
+def test_f32_rows_qwen7b_all_projections(dev, name):
+    # The reference's decode loop holds f32 activations (generate.rs:2153): one and two rows of f32 values that are not
+    # f16 values, on the repacked handle (each lane splits one shared piece of the row; deep K in the pipelined pass
+    # loop) and, for one row, on the reference's arrays as they are.
+    k, n = SHAPES_7B[name]
+    packed, scales, _ = synth(k, n, 1, 7400 + k % 89 + n % 83)
+    a_raw = (O.synth_normal_f32(2 * k, 7450 + n % 71) * np.float32(1.37)).reshape(2, k)
+    truth = O.gemm_f64(a_raw, packed, scales, 2, k, n)
+    w = T.MarlinWeight.upload(dev, packed, scales, k, n)
+    for m in (1, 2):
+        c = T.GpuTensor.from_host(dev, np.full((m, n), np.nan, np.float32))
+        T.gemm(dev, w, T.GpuTensor.from_host(dev, np.ascontiguousarray(a_raw[:m])), m, c)
+        err = rel_err(c.to_host().reshape(m, n), truth[:m])
+        print("f32 rows M=%d %s rel err %.2e" % (m, name, err), flush=True)
+        assert err < TIGHT
+    pd, sd = T.GpuTensor.from_host(dev, packed), T.GpuTensor.from_host(dev, scales, "f16")
+    c1 = T.GpuTensor.from_host(dev, np.full((n,), np.nan, np.float32))
+    T.gemm_tw_marlin_m1(dev, T.GpuTensor.from_host(dev, np.ascontiguousarray(a_raw[0])), pd, sd, c1, n, k)
+    assert rel_err(c1.to_host(), truth[0]) < TIGHT
+    w.free()
+
+
 # ---------------------------------------------------------------- LM head 3584 -> 152064 + argmax
 
 def test_lm_head_gemv_and_argmax_at_vocabulary_width(dev):
