@@ -403,6 +403,13 @@ int twm_gemm_tw_marlin_m1_indirect(twm_ctx *ctx, const float *a_dev, const uint8
  * 1 where the plan needs no split (among others wherever M <= 16 runs on column sub-tiles). */
 uint32_t twm_pick_splits(uint32_t k, uint32_t n, uint32_t m);
 
+/* What twm_gemm would launch for a K x N weight, m rows of f16 / f32 activations and (gated != 0) the gated store of a
+ * paired weight, as one line of text: the kernel, its workgroup shape, the K-split and the repacked copy it reads.
+ * ctx = NULL: a fresh context's defaults; otherwise the context's options count.  Touches no device: usable to
+ * see what the planners decide -- the counterpart of AutoTuner::heuristic_variant and ::report
+ * (crates/kernels/src/autotune.rs:505-515, 648-668) -- and to test them without a GPU. */
+int twm_plan_describe(const twm_ctx *ctx, uint32_t k, uint32_t n, uint32_t m, int a_dtype, int gated, char *text, size_t bytes);
+
 /* ---- graph capture / replay (GraphCapture::{record_with_device, replay}, cuda_graph.rs:85-117) */
 
 /* Starts capturing the work issued on the context's stream. */

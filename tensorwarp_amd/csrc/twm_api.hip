@@ -1259,15 +1259,212 @@ static BatchPlan plan_batch(uint32_t n_tiles, uint32_t k_chunks, uint32_t m, boo
     return best;
 }
 
+// ---- the launch form of a GEMM: chosen in one place, launched in another ---------------------------------
+// What twm_gemm will run for a weight's shape, a row count and the context's knobs.  Nothing here touches the device.
+enum FormKind { kFormPrefill = 0, kFormSubTile = 1, kFormWholeTile = 2, kFormBatch = 3, kFormStream = 4, kFormNone = 5 };
+struct LaunchForm {
+    int kind;
+    int copy;                 // the repacked order it reads (kCopyTile / kCopyCol)
+    uint32_t sub, waves;      // sub-tile kernel: columns per workgroup, waves; whole tiles / streaming: waves
+    uint32_t nt;              // whole tiles: 64-column tiles per workgroup
+    uint32_t splits;          // K-splits over workgroups (prefill: the forced factor, 0 = plan_prefill's choice)
+    bool batch_auto;          // LDS-shared batched decode: plan_batch per 32-row block, else `batch` as forced
+    bool rounded;             //   ... on f16-rounded weights (option "batch_rounded")
+    BatchPlan batch;
+};
+struct FormEnv {              // the knobs and limits of a context
+    int kernel, nt, waves, sub, sub_waves, prefill_min_m, batch_rounded;
+    size_t ws_bytes;          // split-K scratch
+    uint32_t n_counters;      // arrival counters
+};
+static FormEnv form_env(const twm_ctx *c)
+{
+    return FormEnv{c->force_kernel, c->force_nt, c->force_waves, c->force_sub, c->force_sub_waves, c->prefill_min_m,
+                   c->batch_rounded, c->ws_bytes, c->n_counters};
+}
+
+// n_tiles: 16-column tiles of the padded weight; gated: the gated store of a paired weight
+static LaunchForm choose_form(const FormEnv &e, uint32_t n_tiles, uint32_t k_chunks, uint32_t m, bool a_f32, uint32_t splits, bool gated)
+{
+    LaunchForm f = {};
+    const uint32_t n_ld = n_tiles * kTileN, tiles64 = n_ld / 64;
+    f.splits = splits;
+    if (m >= (uint32_t)e.prefill_min_m) {
+        f.kind = kFormPrefill;
+        f.copy = kCopyTile;
+        return f;
+    }
+    // the sub-tile kernel's K-split fits the scratch and the counters
+    auto fit_sub_splits = [&](uint32_t sub) {
+        uint32_t ssp = splits ? splits : 1;
+        if (ssp > k_chunks) ssp = k_chunks;
+        while (ssp > 1 && (size_t)ssp * m * n_ld * 4 > e.ws_bytes) ssp--;
+        if (n_ld / sub > e.n_counters) ssp = 1;
+        return ssp;
+    };
+    auto fit_whole_splits = [&](DecodePlan &plan) {
+        while (plan.splits > 1 && (size_t)plan.splits * m * n_ld * 4 > e.ws_bytes) plan.splits--;
+        if (n_tiles / plan.nt > e.n_counters) plan.splits = 1;
+    };
+    if (e.kernel == 0 && m > 4 && m <= 16 && !a_f32 && e.sub != 1) {
+        // M = 5 .. 16 on narrow matrices: the lane-per-column sub-tile kernel with two to four row groups
+        SubPlan sub = {0, 0};
+        if (e.sub >= 16) sub = SubPlan{(uint32_t)e.sub, e.sub_waves ? (uint32_t)e.sub_waves : e.waves ? (uint32_t)e.waves : 8};
+        else if (!e.nt && !e.waves && !splits) sub = plan_gemv4_sub_rows(tiles64, k_chunks);
+        if (sub.sub) {
+            f.kind = kFormSubTile;
+            f.copy = kCopyCol;
+            f.sub = sub.sub;
+            f.waves = sub.waves;
+            f.splits = fit_sub_splits(sub.sub);
+            return f;
+        }
+        if (m <= 8 && tiles64 > 128 && !e.nt && !splits) {
+            // M = 5 .. 8 on wide matrices: the 64-column lane-per-column kernel with two row groups, which unpacks with
+            // fewer vector instructions than the streaming kernel (3584 -> 37888 at M = 8: 18.0 against 19.2 us,
+            // 3584 -> 152064: 54.8 against 60.0; with four row groups, M = 9 .. 16, it needs 127 registers and loses;
+            // on 128 tiles or fewer the streaming kernel's split-K is ahead: 14336 -> 4096 11.4 against 19.8 us)
+            DecodePlan plan = plan_gemv4(n_tiles, k_chunks, 1, e.waves, 0);
+            fit_whole_splits(plan);
+            f.kind = kFormWholeTile;
+            f.copy = kCopyCol;
+            f.nt = 1;
+            f.waves = plan.waves;
+            f.splits = plan.splits;
+            return f;
+        }
+    }
+    const bool batch_auto = e.kernel == 0 && !e.nt && !e.waves &&
+                            (m > 16 || (!splits && ((m > 8 && (tiles64 > 128 || a_f32)) || (a_f32 && m > 4 && k_chunks <= 64))));
+    if (e.kernel == 4 || batch_auto) {
+        // batched decode with the activations shared through LDS, in 32-row blocks: from 17 rows on (the same exact
+        // arithmetic as below 17 rows; option "batch_rounded" runs the f16-rounded weights of the prefill kernel
+        // there), and from 9 rows on wide
+        // matrices (3584 -> 37888: M = 16 19.8 against 22.8 us of the streaming kernel, M = 32 26.7 against
+        // 33.3; 18944 -> 3584 at M = 32 17.3 against 21.8; at M = 9 .. 16 on narrow matrices the two are within 3 %
+        // with f16 rows).  f32 rows, which the streaming kernel holds twice in registers: from 9 rows on everywhere
+        // (3584 -> 4608 at M = 16 10.9 against 15.1 us, 18944 -> 3584 20.6 against 23.3), from 5 rows on up to 64
+        // chunks deep (3584 -> 4608 at M = 8 10.5 against 11.4; 13824 -> 5120 would lose 18.6 against 18.5)
+        f.kind = kFormBatch;
+        f.copy = kCopyTile;
+        f.batch_auto = batch_auto;
+        f.rounded = e.batch_rounded && m > 16;
+        // forced: "nt" 2 = two tiles per wave, 4 = two quads per workgroup, 3 = three; "waves" 8 / 16 = 2 / 4 k-slices
+        f.batch = BatchPlan{splits ? splits : 1, e.waves == 8 ? 2u : e.waves == 16 ? 4u : 1u, e.nt == 2 ? 2u : 1u,
+                            e.nt == 4 ? 2u : e.nt == 3 ? 3u : 1u};
+        return f;
+    }
+    if (e.kernel == 3 || (e.kernel == 0 && m > 4)) {
+        f.kind = kFormStream;   // batched decode: 32-row blocks of the streaming kernel
+        f.copy = kCopyTile;
+        return f;
+    }
+    // M <= 4: one lane per column (whole 64-column tiles, or the sub-tile kernel where the planner takes it)
+    if (m > 4) {
+        f.kind = kFormNone;
+        return f;
+    }
+    f.copy = kCopyCol;
+    SubPlan sub = {0, 0};
+    if (e.sub >= 16) {
+        sub.sub = (uint32_t)e.sub;
+        sub.waves = e.sub_waves ? (uint32_t)e.sub_waves : e.waves ? (uint32_t)e.waves : 8;
+    } else if (e.sub == 0 && !e.nt && !e.waves && !splits) {
+        // (an explicit nt, waves or split factor asks for the 64-column kernel's plan)
+        sub = plan_gemv4_sub(tiles64, k_chunks, m, a_f32);
+        // the gated store splits a sub-tile into a gate and an up half: 16 columns would read 128-byte runs
+        // (3584 -> 2 x 18944 at M = 1: 17.0 us on 16 columns, 16.3 on 32, 17.1 on whole tiles)
+        if (gated && sub.sub == 16) sub = SubPlan{32, 8};
+    }
+    if (sub.sub) {
+        f.kind = kFormSubTile;
+        f.sub = sub.sub;
+        f.waves = sub.waves;
+        f.splits = fit_sub_splits(sub.sub);
+        return f;
+    }
+    DecodePlan plan = plan_gemv4(n_tiles, k_chunks, e.nt, e.waves, splits);
+    fit_whole_splits(plan);  // the scratch must hold splits x m x n_ld partials and one counter per tile group
+    f.kind = kFormWholeTile;
+    f.nt = plan.nt;
+    f.waves = plan.waves;
+    f.splits = plan.splits;
+    return f;
+}
+
+static void tiles_of(uint32_t k, uint32_t n, uint32_t &n_tiles, uint32_t &k_chunks)
+{
+    n_tiles = ((n + kNPadTo - 1) / kNPadTo) * kNPadTo / kTileN;
+    k_chunks = (k / 32 + kChunkGroups - 1) / kChunkGroups;
+}
+static FormEnv default_env()
+{
+    return FormEnv{0, 0, 0, 0, 0, 33, 0, kWsBytes, kCounters};
+}
+
 uint32_t twm_pick_splits(uint32_t k, uint32_t n, uint32_t m)
 {
-    uint32_t n_tiles = ((n + kNPadTo - 1) / kNPadTo) * kNPadTo / kTileN;
-    uint32_t k_chunks = (k / 32 + kChunkGroups - 1) / kChunkGroups;
-    // (f16 activations assumed; where the planner takes the sub-tile kernel, K is not split at all)
-    if (m <= 4) return plan_gemv4_sub(n_tiles * kTileN / 64, k_chunks, m, false).sub ? 1 : plan_gemv4(n_tiles, k_chunks, 0, 0, 0).splits;
-    if (m <= 16 && plan_gemv4_sub_rows(n_tiles * kTileN / 64, k_chunks).sub) return 1;
-    if (m > 16 || (m > 8 && n_tiles * kTileN / 64 > 128)) return plan_batch(n_tiles, k_chunks, m, false).splits;
-    return plan_stream(n_tiles, k_chunks, m);
+    uint32_t n_tiles, k_chunks;
+    tiles_of(k, n, n_tiles, k_chunks);
+    if (m == 0 || n_tiles == 0 || k_chunks == 0) return 1;
+    // (f16 activations, nothing forced, the default scratch)
+    const LaunchForm f = choose_form(default_env(), n_tiles, k_chunks, m, false, 0, false);
+    switch (f.kind) {
+    case kFormSubTile:
+    case kFormWholeTile: return f.splits;
+    case kFormBatch: return plan_batch(n_tiles, k_chunks, m < 32 ? m : 32, false).splits;
+    case kFormStream: return plan_stream(n_tiles, k_chunks, m < 32 ? m : 32);
+    default: return 1;  // prefill: see twm_plan_describe
+    }
+}
+
+int twm_plan_describe(const twm_ctx *ctx, uint32_t k, uint32_t n, uint32_t m, int a_dtype, int gated, char *text, size_t bytes)
+{
+    if (!text || bytes == 0) return api_fail(TWM_INVALID_HANDLE, "twm_plan_describe: null buffer");
+    if (a_dtype != TWM_F16 && a_dtype != TWM_F32) return api_fail(TWM_UNSUPPORTED_OP, "twm_plan_describe: activations must be f16 or f32");
+    if (int rc = check_kn("twm_plan_describe", k, n)) return rc;
+    uint32_t n_tiles, k_chunks;
+    tiles_of(k, n, n_tiles, k_chunks);
+    if (m == 0 || n == 0 || k == 0) {
+        snprintf(text, bytes, "nothing to launch");
+        return TWM_OK;
+    }
+    const bool a_f32 = a_dtype == TWM_F32;
+    const FormEnv e = ctx ? form_env(ctx) : default_env();
+    const LaunchForm f = choose_form(e, n_tiles, k_chunks, m, a_f32, 0, gated != 0);
+    const uint32_t mb = m < (uint32_t)kMaxStreamM ? m : (uint32_t)kMaxStreamM;
+    switch (f.kind) {
+    case kFormPrefill: {
+        uint32_t bm = 0, sp = 0;
+        prefill_plan_of(m, 0, 0, n_tiles, k_chunks, e.ws_bytes, &bm, &sp);
+        snprintf(text, bytes, "k_prefill: %u-row x 256-column blocks, %u K-split%s%s; 16-column tile copy", bm, sp, sp == 1 ? "" : "s",
+                 sp > 1 ? " + k_splitk_reduce" : "");
+        break;
+    }
+    case kFormSubTile:
+        snprintf(text, bytes, "k_gemv4s: %u-column sub-tiles, %u waves, %u K-split%s; column-lane copy", f.sub, f.waves, f.splits,
+                 f.splits == 1 ? "" : "s");
+        break;
+    case kFormWholeTile:
+        snprintf(text, bytes, "k_gemv4: %u x 64-column tiles per workgroup, %u waves, %u K-split%s; column-lane copy", f.nt, f.waves,
+                 f.splits, f.splits == 1 ? "" : "s");
+        break;
+    case kFormBatch: {
+        const BatchPlan bp = f.batch_auto ? plan_batch(n_tiles, k_chunks, f.rounded ? 32 : mb, a_f32, 0) : f.batch;
+        snprintf(text, bytes, "k_batch: %u quad%s per workgroup, %u tile%s per wave, %u k-slice%s, %u K-split%s%s; 16-column tile copy",
+                 bp.quads_per_group, bp.quads_per_group == 1 ? "" : "s", bp.tiles_per_wave, bp.tiles_per_wave == 1 ? "" : "s", bp.slices,
+                 bp.slices == 1 ? "" : "s", bp.splits, bp.splits == 1 ? "" : "s", bp.splits > 1 ? " + k_splitk_reduce" : "");
+        break;
+    }
+    case kFormStream: {
+        const uint32_t sp = plan_stream(n_tiles, k_chunks, mb);
+        snprintf(text, bytes, "k_stream: %u waves, %u K-split%s%s; 16-column tile copy", stream_waves(n_tiles, mb, e.waves), sp,
+                 sp == 1 ? "" : "s", sp > 1 ? " + k_splitk_reduce" : "");
+        break;
+    }
+    default: snprintf(text, bytes, "no kernel takes this case with the knobs set"); break;
+    }
+    return TWM_OK;
 }
 
 // swiglu_out (paired weight): the launch writes silu(gate) * up to swiglu_out[m][n/2] instead of the columns
@@ -1292,136 +1489,59 @@ static int gemm_dispatch(twm_ctx *ctx, const twm_weight *w, const void *a_dev, i
     }
     if (!a_dev) return api_fail(TWM_INVALID_HANDLE, "%s: null activations", who);
     if (((uintptr_t)a_dev & 15) != 0) return api_fail(TWM_SHAPE_ERROR, "%s: activations must be 16-byte aligned", who);
-    WeightView v = view_of(w);
-    size_t a_row_bytes = (size_t)w->k * (a_dtype == TWM_F16 ? 2 : 4);
-    uint32_t n_ld = w->n_tiles * kTileN;
+    const bool a_f32 = a_dtype == TWM_F32;
+    const size_t a_row_bytes = (size_t)w->k * (a_f32 ? 4 : 2);
     OutSpec gated = out;
     gated.swiglu = swiglu_out;
     gated.gate_act = gate_act;
-    // the copy a launch reads is built here if the handle does not hold it yet (weight_ensure)
-#define TWM_NEED(COPY)                                                 \
-    do {                                                               \
-        if (int rc_ = weight_ensure(ctx, w, COPY, who)) return rc_;    \
-        v = view_of(w);                                                \
-    } while (0)
-    if (m >= (uint32_t)ctx->prefill_min_m) {
-        TWM_NEED(kCopyTile);
+    const LaunchForm f = choose_form(form_env(ctx), w->n_tiles, w->k_chunks, m, a_f32, splits, swiglu_out != nullptr);
+    if (f.kind == kFormNone) return api_fail(TWM_UNSUPPORTED_OP, "%s: the one-lane-per-column kernel takes M <= 4", who);
+    // the copy the launch reads is built here if the handle does not hold it yet
+    if (int rc = weight_ensure(ctx, w, f.copy, who)) return rc;
+    const WeightView v = view_of(w);
+    // rows beyond 32: blocks of 32 rows, each a launch of its own
+    auto row_blocks = [&](auto &&launch_block) -> int {
+        for (uint32_t m0 = 0; m0 < m; m0 += kMaxStreamM) {
+            const uint32_t mb = m - m0 < (uint32_t)kMaxStreamM ? m - m0 : (uint32_t)kMaxStreamM;
+            OutSpec o = gated;
+            for (uint32_t s = 0; s < o.count; s++) o.seg[s].ptr += (size_t)m0 * o.seg[s].width;
+            if (o.swiglu) o.swiglu += (size_t)m0 * (w->n / 2);
+            if (int rc = launch_block((const char *)a_dev + (size_t)m0 * a_row_bytes, mb, o)) return rc;
+        }
+        return TWM_OK;
+    };
+    switch (f.kind) {
+    case kFormPrefill: {
         const PrefillSk sk = {ctx->sk_ws, ctx->sk_ws_bytes, ctx->counters, ctx->n_counters, (uint32_t)ctx->prop.multiProcessorCount,
                               ctx->prefill_sk};
-        HIP_TRY(launch_prefill(ctx->stream, v, a_dev, a_dtype == TWM_F32, m, gated, (uint32_t)ctx->prefill_bm, splits, ctx->ws, ctx->ws_bytes, &sk),
+        HIP_TRY(launch_prefill(ctx->stream, v, a_dev, a_f32, m, gated, (uint32_t)ctx->prefill_bm, splits, ctx->ws, ctx->ws_bytes, &sk),
                 TWM_DEVICE_ERROR, "prefill launch");
         return TWM_OK;
     }
-    if (ctx->force_kernel == 0 && m > 4 && m <= 16 && a_dtype == TWM_F16 && ctx->force_sub != 1) {
-        // M = 5 .. 16 on narrow matrices: the lane-per-column sub-tile kernel with two to four row groups
-        SubPlan sub = {0, 0};
-        if (ctx->force_sub >= 16) sub = SubPlan{(uint32_t)ctx->force_sub, ctx->force_sub_waves ? (uint32_t)ctx->force_sub_waves : ctx->force_waves ? (uint32_t)ctx->force_waves : 8};
-        else if (!ctx->force_nt && !ctx->force_waves && !splits) sub = plan_gemv4_sub_rows(n_ld / 64, w->k_chunks);
-        if (sub.sub) {
-            uint32_t ssp = splits ? splits : 1;
-            if (ssp > w->k_chunks) ssp = w->k_chunks;
-            while (ssp > 1 && (size_t)ssp * m * n_ld * 4 > ctx->ws_bytes) ssp--;
-            if (n_ld / sub.sub > ctx->n_counters) ssp = 1;
-            TWM_NEED(kCopyCol);
-            HIP_TRY(launch_gemv4s(ctx->stream, v, a_dev, false, m, gated, ctx->ws, ctx->counters, sub.sub, sub.waves, ssp),
-                    TWM_DEVICE_ERROR, "sub-tile gemv launch");
-            return TWM_OK;
-        }
-        if (m <= 8 && n_ld / 64 > 128 && !ctx->force_nt && !splits) {
-            // M = 5 .. 8 on wide matrices: the 64-column lane-per-column kernel with two row groups, which unpacks with
-            // fewer vector instructions than the streaming kernel (3584 -> 37888 at M = 8: 18.0 against 19.2 us,
-            // 3584 -> 152064: 54.8 against 60.0; with four row groups, M = 9 .. 16, it needs 127 registers and loses;
-            // on 128 tiles or fewer the streaming kernel's split-K is ahead: 14336 -> 4096 11.4 against 19.8 us)
-            DecodePlan plan = plan_gemv4(w->n_tiles, w->k_chunks, 1, ctx->force_waves, 0);
-            while (plan.splits > 1 && (size_t)plan.splits * m * n_ld * 4 > ctx->ws_bytes) plan.splits--;
-            if (w->n_tiles / plan.nt > ctx->n_counters) plan.splits = 1;
-            TWM_NEED(kCopyCol);
-            HIP_TRY(launch_gemv4(ctx->stream, v, a_dev, false, m, gated, ctx->ws, ctx->counters, 1, plan.waves, plan.splits, swiglu_out),
-                    TWM_DEVICE_ERROR, "gemv launch");
-            return TWM_OK;
-        }
-    }
-    const bool rows_f32 = a_dtype == TWM_F32;
-    const bool batch_auto = ctx->force_kernel == 0 && !ctx->force_nt && !ctx->force_waves &&
-                            (m > 16 || (!splits && ((m > 8 && (n_ld / 64 > 128 || rows_f32)) ||
-                                                    (rows_f32 && m > 4 && w->k_chunks <= 64))));
-    if (ctx->force_kernel == 4 || batch_auto) {
-        TWM_NEED(kCopyTile);
-        // batched decode with the activations shared through LDS, in 32-row blocks: from 17 rows on (the same exact
-        // arithmetic as below 17 rows; option "batch_rounded" runs the f16-rounded weights of the prefill kernel
-        // there), and from 9 rows on wide
-        // matrices (3584 -> 37888: M = 16 19.8 against 22.8 us of the streaming kernel, M = 32 26.7 against
-        // 33.3; 18944 -> 3584 at M = 32 17.3 against 21.8; at M = 9 .. 16 on narrow matrices the two are within 3 %
-        // with f16 rows).  f32 rows, which the streaming kernel holds twice in registers: from 9 rows on everywhere
-        // (3584 -> 4608 at M = 16 10.9 against 15.1 us, 18944 -> 3584 20.6 against 23.3), from 5 rows on up to 64
-        // chunks deep (3584 -> 4608 at M = 8 10.5 against 11.4; 13824 -> 5120 would lose 18.6 against 18.5)
-        for (uint32_t m0 = 0; m0 < m; m0 += kMaxStreamM) {
-            uint32_t mb = m - m0 < (uint32_t)kMaxStreamM ? m - m0 : (uint32_t)kMaxStreamM;
-            OutSpec o = gated;
-            for (uint32_t s = 0; s < o.count; s++) o.seg[s].ptr += (size_t)m0 * o.seg[s].width;
-            if (o.swiglu) o.swiglu += (size_t)m0 * (w->n / 2);
-            const char *a_blk = (const char *)a_dev + (size_t)m0 * a_row_bytes;
-            // forced: "nt" 2 = two tiles per wave, 4 = two quads per workgroup, 3 = three; "waves" 8 / 16 = 2 / 4 k-slices
-            BatchPlan bp = {splits ? splits : 1, ctx->force_waves == 8 ? 2u : ctx->force_waves == 16 ? 4u : 1u,
-                            ctx->force_nt == 2 ? 2u : 1u, ctx->force_nt == 4 ? 2u : ctx->force_nt == 3 ? 3u : 1u};
-            const bool rounded = ctx->batch_rounded && m > 16;
-            if (batch_auto) bp = plan_batch(w->n_tiles, w->k_chunks, rounded ? 32 : mb, rows_f32, splits);
-            HIP_TRY(launch_batch(ctx->stream, v, a_blk, a_dtype == TWM_F32, mb, o, bp.splits, bp.tiles_per_wave, bp.slices,
-                                 bp.quads_per_group, rounded, ctx->ws, ctx->ws_bytes),
-                    TWM_DEVICE_ERROR, "batched decode launch");
-        }
+    case kFormSubTile:
+        HIP_TRY(launch_gemv4s(ctx->stream, v, a_dev, a_f32, m, gated, ctx->ws, ctx->counters, f.sub, f.waves, f.splits), TWM_DEVICE_ERROR,
+                "sub-tile gemv launch");
         return TWM_OK;
-    }
-    if (ctx->force_kernel == 3 || (ctx->force_kernel == 0 && m > 4)) {
-        TWM_NEED(kCopyTile);
-        // batched decode: 32-row blocks of the streaming kernel
-        for (uint32_t m0 = 0; m0 < m; m0 += kMaxStreamM) {
-            uint32_t mb = m - m0 < (uint32_t)kMaxStreamM ? m - m0 : (uint32_t)kMaxStreamM;
-            OutSpec o = gated;
-            for (uint32_t s = 0; s < o.count; s++) o.seg[s].ptr += (size_t)m0 * o.seg[s].width;
-            if (o.swiglu) o.swiglu += (size_t)m0 * (w->n / 2);
-            const char *a_blk = (const char *)a_dev + (size_t)m0 * a_row_bytes;
-            HIP_TRY(launch_stream(ctx->stream, v, a_blk, a_dtype == TWM_F32, mb, o, splits ? splits : plan_stream(w->n_tiles, w->k_chunks, mb),
+    case kFormWholeTile:
+        HIP_TRY(launch_gemv4(ctx->stream, v, a_dev, a_f32, m, gated, ctx->ws, ctx->counters, f.nt, f.waves, f.splits, swiglu_out),
+                TWM_DEVICE_ERROR, "gemv launch");
+        return TWM_OK;
+    case kFormBatch:
+        return row_blocks([&](const char *a_blk, uint32_t mb, const OutSpec &o) -> int {
+            const BatchPlan bp = f.batch_auto ? plan_batch(w->n_tiles, w->k_chunks, f.rounded ? 32 : mb, a_f32, splits) : f.batch;
+            HIP_TRY(launch_batch(ctx->stream, v, a_blk, a_f32, mb, o, bp.splits, bp.tiles_per_wave, bp.slices, bp.quads_per_group, f.rounded,
+                                 ctx->ws, ctx->ws_bytes),
+                    TWM_DEVICE_ERROR, "batched decode launch");
+            return TWM_OK;
+        });
+    default:  // kFormStream
+        return row_blocks([&](const char *a_blk, uint32_t mb, const OutSpec &o) -> int {
+            HIP_TRY(launch_stream(ctx->stream, v, a_blk, a_f32, mb, o, splits ? splits : plan_stream(w->n_tiles, w->k_chunks, mb),
                                   stream_waves(w->n_tiles, mb, ctx->force_waves), ctx->ws, ctx->ws_bytes),
                     TWM_DEVICE_ERROR, "batched decode launch");
-        }
-        return TWM_OK;
+            return TWM_OK;
+        });
     }
-    // M <= 4: one lane per column (whole 64-column tiles, or the sub-tile kernel where the planner takes it)
-    if (m > 4) return api_fail(TWM_UNSUPPORTED_OP, "%s: the one-lane-per-column kernel takes M <= 4", who);
-    {
-        const uint32_t mb = m;
-        TWM_NEED(kCopyCol);
-        DecodePlan plan = plan_gemv4(w->n_tiles, w->k_chunks, ctx->force_nt, ctx->force_waves, splits);
-        // the scratch must hold splits x mb x n_ld partials and one counter per tile group
-        while (plan.splits > 1 && (size_t)plan.splits * mb * n_ld * 4 > ctx->ws_bytes) plan.splits--;
-        if (w->n_tiles / plan.nt > ctx->n_counters) plan.splits = 1;
-        OutSpec o = gated;
-        SubPlan sub = {0, 0};
-        if (ctx->force_sub >= 16) {
-            sub.sub = (uint32_t)ctx->force_sub;
-            sub.waves = ctx->force_sub_waves ? (uint32_t)ctx->force_sub_waves : ctx->force_waves ? (uint32_t)ctx->force_waves : 8;
-        } else if (ctx->force_sub == 0 && !ctx->force_nt && !ctx->force_waves && !splits) {
-            // (an explicit nt, waves or split factor asks for the 64-column kernel's plan)
-            sub = plan_gemv4_sub(n_ld / 64, w->k_chunks, mb, a_dtype == TWM_F32);
-            // the gated store splits a sub-tile into a gate and an up half: 16 columns would read 128-byte runs
-            // (3584 -> 2 x 18944 at M = 1: 17.0 us on 16 columns, 16.3 on 32, 17.1 on whole tiles)
-            if (swiglu_out && sub.sub == 16) sub = SubPlan{32, 8};
-        }
-        if (sub.sub) {
-            uint32_t ssp = splits ? splits : 1;
-            if (ssp > w->k_chunks) ssp = w->k_chunks;
-            while (ssp > 1 && (size_t)ssp * mb * n_ld * 4 > ctx->ws_bytes) ssp--;
-            if (n_ld / sub.sub > ctx->n_counters) ssp = 1;
-            HIP_TRY(launch_gemv4s(ctx->stream, v, a_dev, a_dtype == TWM_F32, mb, o, ctx->ws, ctx->counters, sub.sub, sub.waves, ssp),
-                    TWM_DEVICE_ERROR, "sub-tile gemv launch");
-        } else
-            HIP_TRY(launch_gemv4(ctx->stream, v, a_dev, a_dtype == TWM_F32, mb, o, ctx->ws, ctx->counters, plan.nt,
-                                 plan.waves, plan.splits, swiglu_out),
-                    TWM_DEVICE_ERROR, "gemv launch");
-    }
-#undef TWM_NEED
-    return TWM_OK;
 }
 
 // The knobs of a launch form, saved and set as one

@@ -436,6 +436,38 @@ static PrefillPlan plan_prefill(uint32_t rows, uint32_t force_rows, uint32_t for
     return best;
 }
 
+// The plan within what the scratch can hold of partial sums (ws_bytes = 0: no scratch, unsplit).
+static PrefillPlan plan_prefill_within(uint32_t rows, uint32_t block_rows, uint32_t splits, uint32_t n_tiles, uint32_t k_chunks,
+                                       size_t ws_bytes)
+{
+    const size_t n_ld = (size_t)n_tiles * 16;
+    PrefillPlan plan = plan_prefill(rows, block_rows, splits, (n_tiles + 15) / 16, k_chunks, n_ld);
+    const size_t per_split = (size_t)rows * n_ld * 4;
+    if (plan.splits > 1 && (ws_bytes == 0 || per_split == 0 || plan.splits > ws_bytes / per_split)) {
+        // the scratch cannot hold that many partial sums: plan again within what it holds (at least unsplit)
+        uint32_t cap = (ws_bytes == 0 || per_split == 0) ? 1u : (uint32_t)(ws_bytes / per_split);
+        if (cap < 2) cap = 1;
+        if (splits) plan.splits = cap;  // a forced factor is cut, the forced height kept
+        else {
+            PrefillPlan capped = {0, 0, 1e30};
+            for (uint32_t sp = 1; sp <= cap; sp++) {
+                PrefillPlan c = plan_prefill(rows, block_rows, sp, (n_tiles + 15) / 16, k_chunks, n_ld);
+                if (c.us < capped.us) capped = c;
+            }
+            plan = capped;
+        }
+    }
+    return plan;
+}
+
+void prefill_plan_of(uint32_t rows, uint32_t block_rows, uint32_t splits, uint32_t n_tiles, uint32_t k_chunks, size_t ws_bytes,
+                     uint32_t *block_rows_out, uint32_t *splits_out)
+{
+    const PrefillPlan plan = plan_prefill_within(rows, block_rows, splits, n_tiles, k_chunks, ws_bytes);
+    *block_rows_out = plan.block_rows;
+    *splits_out = plan.splits;
+}
+
 template <int MT>
 static hipError_t launch_prefill_t(hipStream_t s, const WeightView &w, const _Float16 *a, uint32_t m, const OutSpec &out,
                                    uint32_t splits, float *partials)
@@ -473,7 +505,6 @@ hipError_t launch_prefill(hipStream_t s, const WeightView &w, const void *a, boo
 {
     if (m == 0 || w.n == 0) return hipSuccess;
     if (block_rows != 0 && block_rows != 64 && block_rows != 128) return hipErrorInvalidValue;
-    const size_t n_ld = (size_t)w.n_tiles * 16;
     auto run = [&](const _Float16 *a16, uint32_t rows, const OutSpec &o, void *ws, size_t ws_bytes) {
         // Option prefill_sk: the tiles dealt out by stream-K (twm_prefill_sk.hip); the gated store stays with the plain kernel.
         if (sk && sk->mode >= 128 && !o.swiglu && sk->partials) {
@@ -483,22 +514,7 @@ hipError_t launch_prefill(hipStream_t s, const WeightView &w, const void *a, boo
             if (e != hipErrorInvalidValue) return e;  // (a shape it does not take: the plain kernel below)
             (void)hipGetLastError();
         }
-        PrefillPlan plan = plan_prefill(rows, block_rows, splits, (w.n_tiles + 15) / 16, w.k_chunks, n_ld);
-        size_t per_split = (size_t)rows * n_ld * 4;
-        if (plan.splits > 1 && (!ws || per_split == 0 || plan.splits > ws_bytes / per_split)) {
-            // the scratch cannot hold that many partial sums: plan again within what it holds (at least unsplit)
-            uint32_t cap = (!ws || per_split == 0) ? 1u : (uint32_t)(ws_bytes / per_split);
-            if (cap < 2) cap = 1;
-            if (splits) plan.splits = cap;  // a forced factor is cut, the forced height kept
-            else {
-                PrefillPlan capped = {0, 0, 1e30};
-                for (uint32_t sp = 1; sp <= cap; sp++) {
-                    PrefillPlan c = plan_prefill(rows, block_rows, sp, (w.n_tiles + 15) / 16, w.k_chunks, n_ld);
-                    if (c.us < capped.us) capped = c;
-                }
-                plan = capped;
-            }
-        }
+        const PrefillPlan plan = plan_prefill_within(rows, block_rows, splits, w.n_tiles, w.k_chunks, ws ? ws_bytes : 0);
         return plan.block_rows == 64 ? launch_prefill_t<4>(s, w, a16, rows, o, plan.splits, (float *)ws)
                                      : launch_prefill_t<8>(s, w, a16, rows, o, plan.splits, (float *)ws);
     };
