@@ -860,7 +860,7 @@ def main():
 
     prefill_sweep = None
     if args.sweep_prefill:
-        # block height (64 / 128 rows per workgroup) x split-K forced against the library's plan; the plan is timed
+        # block form (64 x 256, 128 x 256, 128 rows x 192 columns per workgroup) x split-K forced against the library's plan; the plan is timed
         # after the forced cases, every case after ~200 untimed launches
         prefill_sweep = {}
         for k, n in ((4096, 11008), (11008, 4096), (3584, 37888), (18944, 3584), (3584, 4608)):
@@ -871,7 +871,7 @@ def main():
                 a_m = T.GpuTensor.from_host(dev, rng.standard_normal((m, k), dtype=np.float32).astype(np.float16).view(np.uint16), "f16")
                 c_m = T.GpuTensor.zeros(dev, (m, n), "f32")
                 row = {}
-                for bm, sp in ((64, 1), (64, 2), (64, 4), (128, 1), (128, 2), (128, 4), (0, 0)):
+                for bm, sp in ((64, 1), (64, 2), (64, 4), (128, 1), (128, 2), (128, 4), (192, 1), (192, 2), (192, 4), (0, 0)):
                     dev.set_option("prefill_bm", bm)
                     for _ in range(200):
                         T.gemm(dev, w, a_m, m, c_m, sp)

@@ -99,7 +99,7 @@ int twm_ctx_info(twm_ctx *ctx, char *buf, size_t buf_len);
  *   "sub_waves"     waves per workgroup of the sub-tile kernels when "sub" forces their width (1 .. 16)
  *   "prefill_sk"    prefill GEMM: 128 = tiles dealt out by stream-K over one workgroup per CU, 0 / 1 = off
  *   "prefill_min_m" smallest M that runs the prefill GEMM (default 33; below it the decode kernels run)
- *   "prefill_bm"    rows of A per prefill workgroup (64 or 128)
+ *   "prefill_bm"    prefill block form: 64 = 64 rows x 256 columns, 128 = 128 x 256, 192 = 128 rows x 192 columns
  *   "m1_exact"      twm_gemm_tw_marlin_m1: 1 = f32 activations and f32 FMAs in the reference kernel's order with
  *                   the reference's split-K rule and float atomics (bit-equal to the reference order when that
  *                   rule yields one split); 0 (default) = the MFMA kernel

@@ -52,7 +52,7 @@ struct twm_ctx {
     int force_sub;        // M <= 4: 0 = heuristic, 1 = whole 64-column tiles per workgroup, 32 or 16 = the sub-tile kernel
     int force_kernel;     // 0 = heuristic, 2 = one-lane-per-column kernel on whole tiles (M <= 4), 3 = streaming kernel (M <= 32),
                           // 4 = batched-decode kernel with LDS-shared activations (M <= 32; "nt" = tiles per wave, "waves" 8 / 16 = 2 / 4 k-slices)
-    int prefill_bm;       // rows of A per prefill workgroup: 0 = choose, 64 or 128
+    int prefill_bm;       // prefill block form: 0 = choose, 64 = 64 rows x 256 columns, 128 = 128 x 256, 192 = 128 rows x 192 columns
     int prefill_min_m;    // M from which the LDS/MFMA prefill kernel runs instead of 16-row decode blocks
     int dequant_src;      // which copy twm_weight_dequant_f16 unpacks: 0 = 16-column tiles, 1 = column-lane
     int weight_copies;    // copies a new weight handle is given: 0 or 3 = both, 1 = 16-column tiles only, 2 = column-lane only
@@ -273,7 +273,8 @@ int twm_ctx_set_option(twm_ctx *ctx, const char *key, int value)
         return TWM_OK;
     }
     if (strcmp(key, "prefill_bm") == 0) {
-        if (value != 0 && value != 64 && value != 128) return api_fail(TWM_SHAPE_ERROR, "twm_ctx_set_option: prefill_bm must be 0, 64 or 128");
+        if (value != 0 && value != 64 && value != 128 && value != 192)
+            return api_fail(TWM_SHAPE_ERROR, "twm_ctx_set_option: prefill_bm must be 0, 64, 128 or 192");
         ctx->prefill_bm = value;
         return TWM_OK;
     }
@@ -1050,7 +1051,7 @@ twm_weight *twm_weight_import(twm_ctx *ctx, const void *blob_host, size_t blob_b
     memcpy(w->tuned, payload + hd.payload_bytes, kBlobTrailer);
     for (TunedPlan &p : w->tuned)   // (a plan is a set of option values: anything outside their ranges is dropped)
         if (p.valid > 1 || p.kernel > 4 || p.kernel == 1 || p.nt > 4 || p.waves > 16 || p.sub_waves > 16 ||
-            (p.sub != 0 && p.sub != 1 && p.sub != 16 && p.sub != 32) || (p.prefill_bm != 0 && p.prefill_bm != 64 && p.prefill_bm != 128))
+            (p.sub != 0 && p.sub != 1 && p.sub != 16 && p.sub != 32) || (p.prefill_bm != 0 && p.prefill_bm != 64 && p.prefill_bm != 128 && p.prefill_bm != 192))
             memset(&p, 0, sizeof p);
     return w;
 }
@@ -1436,9 +1437,9 @@ int twm_plan_describe(const twm_ctx *ctx, uint32_t k, uint32_t n, uint32_t m, in
     switch (f.kind) {
     case kFormPrefill: {
         uint32_t bm = 0, sp = 0;
-        prefill_plan_of(m, 0, 0, n_tiles, k_chunks, e.ws_bytes, &bm, &sp);
-        snprintf(text, bytes, "k_prefill: %u-row x 256-column blocks, %u K-split%s%s; 16-column tile copy", bm, sp, sp == 1 ? "" : "s",
-                 sp > 1 ? " + k_splitk_reduce" : "");
+        prefill_plan_of(m, 0, 0, n_tiles, k_chunks, e.ws_bytes, gated != 0, &bm, &sp);
+        snprintf(text, bytes, "k_prefill: %u-row x %u-column blocks, %u K-split%s%s; 16-column tile copy", bm == 64 ? 64u : 128u,
+                 bm == 192 ? 192u : 256u, sp, sp == 1 ? "" : "s", sp > 1 ? " + k_splitk_reduce" : "");
         break;
     }
     case kFormSubTile:
@@ -1601,7 +1602,7 @@ static void tune_candidates(uint32_t m, uint32_t k_chunks, std::vector<TunedPlan
                 for (int sp : {1, 2, 3, 4, 6})
                     if (!(wv == 16 && nt != 1) && !(wv == 8 && nt == 3)) add(4, nt, wv, 0, 0, sp, 0);
     } else {
-        for (int bm : {64, 128})
+        for (int bm : {64, 128, 192})
             for (int sp : {1, 2, 3, 4, 6, 8}) add(0, 0, 0, 0, 0, sp, bm);
     }
 }

@@ -184,9 +184,9 @@ hipError_t launch_split_hi_lo(hipStream_t s, const float *a, _Float16 *hi, _Floa
 hipError_t launch_batch(hipStream_t s, const WeightView &w, const void *a, bool a_f32, uint32_t m, const OutSpec &out,
                         uint32_t splits, uint32_t tiles_per_wave, uint32_t k_slices, uint32_t quads_per_group,
                         bool rounded, float *scratch, size_t scratch_bytes);
-// the block height (64 / 128 rows) and K-split launch_prefill takes for `rows` rows of f16 activations with that much scratch
+// the block form (64, 128, or 192 = 128 rows x 192 columns) and K-split launch_prefill takes for `rows` rows of f16 activations with that much scratch
 void prefill_plan_of(uint32_t rows, uint32_t block_rows, uint32_t splits, uint32_t n_tiles, uint32_t k_chunks, size_t ws_bytes,
-                     uint32_t *block_rows_out, uint32_t *splits_out);
+                     bool gated, uint32_t *block_rows_out, uint32_t *splits_out);
 hipError_t launch_geglu_rows(hipStream_t s, const float *gu, float *out, uint32_t dim, uint32_t batch, bool paired);
 // act: 0 out[slot][n]; 1 gelu_tanh(gate) * up, 2 silu(gate) * up into out[slot][n/2] (paired bank)
 hipError_t launch_bank_gemv(hipStream_t s, const BankView &b, const void *a, bool a_f32, uint32_t a_slot_stride,

@@ -22,7 +22,9 @@
 
 namespace twm {
 
-template <int MT>  // MT = 16-row blocks per workgroup tile (BM = 16 * MT rows)
+// MT = 16-row blocks per workgroup tile (BM = 16 * MT rows); NTW = 16-column tiles per wave: 4 (256-column blocks) or
+// 3 (192-column blocks, for shapes whose 256-column blocks leave a round of workgroups mostly empty)
+template <int MT, int NTW = 4>
 __global__ __launch_bounds__(256) void k_prefill(const uint4v *__restrict__ qw, const uint2v *__restrict__ sc,
                                                   const _Float16 *__restrict__ a_any, OutSpec out, uint32_t m_rows,
                                                   uint32_t k, uint32_t n, uint32_t n_tiles, uint32_t k_chunks,
@@ -31,7 +33,7 @@ __global__ __launch_bounds__(256) void k_prefill(const uint4v *__restrict__ qw, 
 {
     constexpr int kPfTileHalves = 16 * MT * kPfRowStride;
     constexpr int NV = MT;       // direct-to-LDS load instructions per wave and A tile (16 MT rows / 16)
-    constexpr int PPU = 8 / MT;  // half fragments unpacked per unit (a unit = one row block's four MFMAs)
+    constexpr int HP = 2 * NTW;  // half fragments of B operands per 32-deep group
     extern __shared__ _Float16 a_lds[];  // two tiles of kPfTileHalves (64 KB at MT = 8)
 
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -62,7 +64,7 @@ __global__ __launch_bounds__(256) void k_prefill(const uint4v *__restrict__ qw, 
         by = band * kBand + u % hb;
     }
     const uint32_t m0 = by * (16u * MT);
-    const uint32_t nt0 = (bx * 4u + wave) * 4u;  // first of this wave's four 16-column tiles
+    const uint32_t nt0 = (bx * 4u + wave) * NTW;  // first of this wave's NTW 16-column tiles
     // split-K: blockIdx.z takes chunks [kc0, kc0 + nchunks); chunk indices below are relative to kc0
     const uint32_t kc0 = blockIdx.z * chunks_per_split;
     const uint32_t nchunks = k_chunks - kc0 < chunks_per_split ? k_chunks - kc0 : chunks_per_split;
@@ -71,22 +73,22 @@ __global__ __launch_bounds__(256) void k_prefill(const uint4v *__restrict__ qw, 
     const PfConsts dq = make_pf_consts();
 
     // this wave's tiles; tiles past the end replay the last tile and are never stored
-    uint32_t nt[4];
+    uint32_t nt[NTW];
 #pragma unroll
-    for (int t = 0; t < 4; t++) nt[t] = nt0 + t < n_tiles ? nt0 + t : n_tiles - 1;
+    for (int t = 0; t < NTW; t++) nt[t] = nt0 + t < n_tiles ? nt0 + t : n_tiles - 1;
 
     // Accumulators live in AGPRs.  The empty asm pins them there across the loop back edge; without it the
     // compiler carries them in VGPRs and copies all of them to AGPRs and back every iteration.
-    float4v acc[MT][4];
+    float4v acc[MT][NTW];
 #pragma unroll
     for (int mt = 0; mt < MT; mt++)
 #pragma unroll
-        for (int t = 0; t < 4; t++) acc[mt][t] = float4v{0.f, 0.f, 0.f, 0.f};
+        for (int t = 0; t < NTW; t++) acc[mt][t] = float4v{0.f, 0.f, 0.f, 0.f};
     auto pin_acc = [&]() {
 #pragma unroll
         for (int mt = 0; mt < MT; mt++)
 #pragma unroll
-            for (int t = 0; t < 4; t++) asm volatile("" : "+a"(acc[mt][t]));
+            for (int t = 0; t < NTW; t++) asm volatile("" : "+a"(acc[mt][t]));
     };
     pin_acc();
 
@@ -118,8 +120,8 @@ __global__ __launch_bounds__(256) void k_prefill(const uint4v *__restrict__ qw, 
     auto wait_loads = [&]() { __builtin_amdgcn_s_waitcnt(0x0F70); };  // vmcnt(0), other counters untouched
 
     // ---- B: chunk kc lives in register slot kc % 2
-    uint4v bq[2][4];
-    uint2v bs[2][4];
+    uint4v bq[2][NTW];
+    uint2v bs[2][NTW];
     const uint32_t q_off = lane * 16u, s_off = c * 8u;
     auto load_bq = [&](int slot, uint32_t kc, int t) {
         bq[slot][t] = *(const TWM_GLOBAL uint4v *)(scalar_base(qw, (size_t)((kc0 + kc) * n_tiles + nt[t]) * 1024u) + q_off);
@@ -128,7 +130,7 @@ __global__ __launch_bounds__(256) void k_prefill(const uint4v *__restrict__ qw, 
         bs[slot][t] = *(const TWM_GLOBAL uint2v *)(scalar_base(sc, (size_t)((kc0 + kc) * n_tiles + nt[t]) * 128u) + s_off);
     };
     // half fragment hp (tile hp / 2, half hp % 2) of group g
-    auto unpack = [&](int slot, int g, PfFrag (&bf)[4], int hp) {
+    auto unpack = [&](int slot, int g, PfFrag (&bf)[NTW], int hp) {
         const int t = hp >> 1;
         uint32_t pair = bs[slot][t][g >> 1];
         uint32_t s16 = (g & 1) ? (pair >> 16) : (pair & 0xFFFFu);
@@ -143,23 +145,24 @@ __global__ __launch_bounds__(256) void k_prefill(const uint4v *__restrict__ qw, 
     };
 
     half8 af0[MT], af1[MT];
-    PfFrag bf0[4], bf1[4];
+    PfFrag bf0[NTW], bf1[NTW];
 
     // One step = the MFMAs of one 32-deep group, in MT units of four (one row block x four tiles).  Unit mt
     // also fetches the next group's A operand for its row block, unpacks its share of the next group's B
     // operands and issues `extra(mt)`, its share of the traffic for later chunks.  The scheduling barrier
     // after each unit keeps this interleaving: one MFMA issue slot hides about two other instructions,
     // but only if they sit next to it.
-    auto step = [&](const half8 (&af_cur)[MT], const PfFrag (&bf_cur)[4], half8 (&af_nxt)[MT], PfFrag (&bf_nxt)[4],
+    auto step = [&](const half8 (&af_cur)[MT], const PfFrag (&bf_cur)[NTW], half8 (&af_nxt)[MT], PfFrag (&bf_nxt)[NTW],
                     uint32_t rd_buf, int rd_g, int uq_slot, int uq_g, auto extra) {
 #pragma unroll
         for (int mt = 0; mt < MT; mt++) {
             af_nxt[mt] = read_a(rd_buf, rd_g, mt);
             extra(mt);
+            // the 2 NTW half fragments of the next group, dealt over the MT units
 #pragma unroll
-            for (int p = 0; p < PPU; p++) unpack(uq_slot, uq_g, bf_nxt, mt * PPU + p);
+            for (int hp = mt * HP / MT; hp < (mt + 1) * HP / MT; hp++) unpack(uq_slot, uq_g, bf_nxt, hp);
 #pragma unroll
-            for (int t = 0; t < 4; t++)
+            for (int t = 0; t < NTW; t++)
                 acc[mt][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(af_cur[mt], bf_cur[t].h, acc[mt][t], 0, 0, 0);
             __builtin_amdgcn_sched_barrier(0);
         }
@@ -186,7 +189,7 @@ __global__ __launch_bounds__(256) void k_prefill(const uint4v *__restrict__ qw, 
             if (u < NV) load_a(buf, kc2, u);
             // B of chunk kc + 2 into this chunk's own slot, whose last group was unpacked in step 2
 #pragma unroll
-            for (int t = 0; t < 4; t++) {
+            for (int t = 0; t < NTW; t++) {
                 if (t * MT / 4 == u) load_bq(S, kc2, t);
                 if (t * MT / 4 + (MT >= 8 ? 1 : 0) == u) load_bs(S, kc2, t);
             }
@@ -201,7 +204,7 @@ __global__ __launch_bounds__(256) void k_prefill(const uint4v *__restrict__ qw, 
 #pragma unroll
     for (int j = 0; j < NV; j++) load_a(0, 0, j);
 #pragma unroll
-    for (int t = 0; t < 4; t++) {
+    for (int t = 0; t < NTW; t++) {
         load_bq(0, 0, t);
         load_bs(0, 0, t);
         load_bq(1, kc1p, t);
@@ -214,7 +217,7 @@ __global__ __launch_bounds__(256) void k_prefill(const uint4v *__restrict__ qw, 
 #pragma unroll
     for (int mt = 0; mt < MT; mt++) af0[mt] = read_a(0, 0, mt);
 #pragma unroll
-    for (int hp = 0; hp < 8; hp++) unpack(0, 0, bf0, hp);
+    for (int hp = 0; hp < HP; hp++) unpack(0, 0, bf0, hp);
     __builtin_amdgcn_sched_barrier(0);
 
     uint32_t kc = 0;
@@ -239,7 +242,7 @@ __global__ __launch_bounds__(256) void k_prefill(const uint4v *__restrict__ qw, 
 #pragma unroll
         for (int mt = 0; mt < MT; mt++) {
 #pragma unroll
-            for (int t = 0; t < 4; t++)
+            for (int t = 0; t < NTW; t++)
 #pragma unroll
                 for (int r = 0; r < 4; r++) stage[(kb * 4 + r) * 68 + t * 16 + c] = acc[mt][t][r];
 #pragma unroll
@@ -247,7 +250,8 @@ __global__ __launch_bounds__(256) void k_prefill(const uint4v *__restrict__ qw, 
                 const uint32_t row = (lane >> 4) + 4u * i;
                 const float4v v = *(const float4v *)(stage + row * 68 + (lane & 15u) * 4u);
                 const uint32_t om = m0 + mt * 16u + row;
-                if (om < m_rows && col < n_lim) __builtin_nontemporal_store(v, (float4v *)(dst + (size_t)om * ld + col));
+                if (om < m_rows && col < n_lim && (lane & 15u) * 4u < 16u * NTW)
+                    __builtin_nontemporal_store(v, (float4v *)(dst + (size_t)om * ld + col));
             }
         }
         return;
@@ -257,7 +261,7 @@ __global__ __launch_bounds__(256) void k_prefill(const uint4v *__restrict__ qw, 
         const uint32_t n_ld = n_tiles * 16u;
         float *dst = partials + ((size_t)blockIdx.z * m_rows) * n_ld;
 #pragma unroll
-        for (int t = 0; t < 4; t++) {
+        for (int t = 0; t < NTW; t++) {
             if (nt0 + t >= n_tiles) continue;
             uint32_t on = (nt0 + t) * 16u + c;
 #pragma unroll
@@ -270,7 +274,7 @@ __global__ __launch_bounds__(256) void k_prefill(const uint4v *__restrict__ qw, 
         }
         return;
     }
-    if (out.swiglu) {
+    if (NTW == 4 && out.swiglu) {
         // paired gate/up weight: this wave's tiles 0, 1 are 32 gate columns and tiles 2, 3 the up columns of the
         // same features, in the same lanes and registers.  The 16 x 32 gated block of a row block goes through
         // LDS like the plain store: a lane stores 16 bytes, eight lanes cover the wave's 128 bytes of a row.
@@ -285,7 +289,7 @@ __global__ __launch_bounds__(256) void k_prefill(const uint4v *__restrict__ qw, 
             for (int t = 0; t < 2; t++)
 #pragma unroll
                 for (int r = 0; r < 4; r++)
-                    stage[(kb * 4 + r) * 36 + t * 16 + c] = gated_mul(out.gate_act, acc[mt][t][r], acc[mt][t + 2][r]);
+                    stage[(kb * 4 + r) * 36 + t * 16 + c] = gated_mul(out.gate_act, acc[mt][t][r], acc[mt][(t + 2) % NTW][r]);
 #pragma unroll
             for (int i = 0; i < 2; i++) {
                 const uint32_t row = (lane >> 3) + 8u * i;
@@ -304,7 +308,7 @@ __global__ __launch_bounds__(256) void k_prefill(const uint4v *__restrict__ qw, 
         return;
     }
 #pragma unroll
-    for (int t = 0; t < 4; t++) {
+    for (int t = 0; t < NTW; t++) {
         if (nt0 + t >= n_tiles) continue;
         uint32_t on = (nt0 + t) * 16u + c;
         if (on >= n) continue;
@@ -391,34 +395,44 @@ hipError_t launch_splitk_reduce(hipStream_t s, const float *partials, const OutS
     return hipGetLastError();
 }
 
-// Block height and split-K factor by a small cost model fitted to per-shape sweeps on MI355X (microseconds per
+// Block form and split-K factor by a small cost model fitted to per-shape sweeps on MI355X (microseconds per
 // 128-deep chunk and workgroup): a 64-row block alone on a CU 1.1, two sharing a CU 2.0 each, a 128-row block 1.5
 // with few workgroups in flight up to 1.8 with all 256 CUs busy; 3 per round of workgroups for the start and the
 // store; a split costs the second kernel, 2.5 + its read of the partial sums at 4 TB/s.  (128-row blocks unpack
 // every weight for twice the rows: per row they are the cheapest form as soon as there is a workgroup for most
 // CUs, and K 4096 -> N 11008 at M = 512 runs in 50 us on 172 of them against 61 us on 344 64-row blocks.)
+// Forms: 64 = 64 rows x 256 columns, 128 = 128 x 256, 192 = 128 rows x 192 columns (three tiles per wave; it pays where
+// it fills a round of workgroups that 256-column blocks leave mostly empty: 4096 -> 11008 at M = 1024 90.5 against
+// 95.9 us, 3584 -> 4608 at M = 2048 76.7 against 82.6; on full rounds a chunk of it takes 0.95 of a 256-column
+// block's chunk for 0.75 of the columns, 4096 -> 11008 at M = 2048 179 against 161 us.  kPf192 is the weight that
+// reproduces the best form on the 25 cases of the sweep, not that ratio.  Not with the gated store, whose waves hold
+// gate and up tiles in pairs).
+constexpr double kPf192 = 0.80;
 struct PrefillPlan {
-    uint32_t block_rows, splits;
+    uint32_t block_rows, splits;   // block_rows: the form (64, 128, 192)
     double us;
 };
-static PrefillPlan plan_prefill(uint32_t rows, uint32_t force_rows, uint32_t force_splits, uint32_t col_blocks,
-                                uint32_t k_chunks, size_t n_ld)
+static PrefillPlan plan_prefill(uint32_t rows, uint32_t force_rows, uint32_t force_splits, uint32_t n_tiles, uint32_t k_chunks,
+                                bool gated)
 {
     PrefillPlan best = {force_rows ? force_rows : 64u, force_splits ? force_splits : 1u, 1e30};
+    const size_t n_ld = (size_t)n_tiles * 16;
     const double partial_us = (double)rows * (double)n_ld * 4.0 / 4.0e6;  // the reduce kernel's read of one split
-    for (uint32_t bm = 64; bm <= 128; bm += 64) {
+    for (uint32_t bm = 64; bm <= 192; bm += 64) {
         if (force_rows && bm != force_rows) continue;
-        const double wgs = (double)((rows + bm - 1) / bm) * col_blocks;
+        if (bm == 192 && gated) continue;
+        const uint32_t col_blocks = bm == 192 ? (n_tiles + 11) / 12 : (n_tiles + 15) / 16, height = bm == 64 ? 64u : 128u;
+        const double wgs = (double)((rows + height - 1) / height) * col_blocks;
         for (uint32_t sp = 1; sp <= 64; sp++) {
             if (force_splits ? sp != force_splits : sp * 2 > (k_chunks > 1 ? k_chunks : 2) && sp > 1) continue;
             const uint32_t cps = (k_chunks + sp - 1) / sp;
             if (!force_splits && (k_chunks + cps - 1) / cps != sp) continue;  // same work as a smaller factor
             const double total = wgs * sp;
             double t;
-            if (bm == 128) {
+            if (bm >= 128) {
                 const double rounds = (double)(uint64_t)((total + 255.0) / 256.0);
                 const double load = total >= 256.0 ? 1.0 : total / 256.0;
-                t = rounds * (cps * (1.5 + 0.3 * load) + 3.0);
+                t = rounds * (cps * (1.5 + 0.3 * load) * (bm == 192 ? kPf192 : 1.0) + 3.0);
             } else if (total <= 256.0) {
                 t = cps * 1.1 + 3.0;
             } else {
@@ -426,7 +440,9 @@ static PrefillPlan plan_prefill(uint32_t rows, uint32_t force_rows, uint32_t for
                 t = full * (cps * 2.0 + 3.0) + (rem == 0.0 ? 0.0 : (rem <= 256.0 ? cps * 1.1 : cps * 2.0) + 3.0);
             }
             if (sp > 1) t += 2.5 + sp * partial_us;
-            if (t < best.us * (sp > best.splits && bm == best.block_rows ? 0.97 : 1.0)) {  // a larger factor has to pay for itself
+            // a larger factor, and the narrower block, have to pay for themselves
+            const double margin = (sp > best.splits && bm == best.block_rows) || bm == 192 ? 0.97 : 1.0;
+            if (t < best.us * margin) {
                 best.block_rows = bm;
                 best.splits = sp;
                 best.us = t;
@@ -438,10 +454,10 @@ static PrefillPlan plan_prefill(uint32_t rows, uint32_t force_rows, uint32_t for
 
 // The plan within what the scratch can hold of partial sums (ws_bytes = 0: no scratch, unsplit).
 static PrefillPlan plan_prefill_within(uint32_t rows, uint32_t block_rows, uint32_t splits, uint32_t n_tiles, uint32_t k_chunks,
-                                       size_t ws_bytes)
+                                       size_t ws_bytes, bool gated)
 {
     const size_t n_ld = (size_t)n_tiles * 16;
-    PrefillPlan plan = plan_prefill(rows, block_rows, splits, (n_tiles + 15) / 16, k_chunks, n_ld);
+    PrefillPlan plan = plan_prefill(rows, block_rows, splits, n_tiles, k_chunks, gated);
     const size_t per_split = (size_t)rows * n_ld * 4;
     if (plan.splits > 1 && (ws_bytes == 0 || per_split == 0 || plan.splits > ws_bytes / per_split)) {
         // the scratch cannot hold that many partial sums: plan again within what it holds (at least unsplit)
@@ -451,7 +467,7 @@ static PrefillPlan plan_prefill_within(uint32_t rows, uint32_t block_rows, uint3
         else {
             PrefillPlan capped = {0, 0, 1e30};
             for (uint32_t sp = 1; sp <= cap; sp++) {
-                PrefillPlan c = plan_prefill(rows, block_rows, sp, (n_tiles + 15) / 16, k_chunks, n_ld);
+                PrefillPlan c = plan_prefill(rows, block_rows, sp, n_tiles, k_chunks, gated);
                 if (c.us < capped.us) capped = c;
             }
             plan = capped;
@@ -461,21 +477,21 @@ static PrefillPlan plan_prefill_within(uint32_t rows, uint32_t block_rows, uint3
 }
 
 void prefill_plan_of(uint32_t rows, uint32_t block_rows, uint32_t splits, uint32_t n_tiles, uint32_t k_chunks, size_t ws_bytes,
-                     uint32_t *block_rows_out, uint32_t *splits_out)
+                     bool gated, uint32_t *block_rows_out, uint32_t *splits_out)
 {
-    const PrefillPlan plan = plan_prefill_within(rows, block_rows, splits, n_tiles, k_chunks, ws_bytes);
+    const PrefillPlan plan = plan_prefill_within(rows, block_rows, splits, n_tiles, k_chunks, ws_bytes, gated);
     *block_rows_out = plan.block_rows;
     *splits_out = plan.splits;
 }
 
-template <int MT>
+template <int MT, int NTW = 4>
 static hipError_t launch_prefill_t(hipStream_t s, const WeightView &w, const _Float16 *a, uint32_t m, const OutSpec &out,
                                    uint32_t splits, float *partials)
 {
     size_t lds = (size_t)2 * 16 * MT * kPfRowStride * sizeof(_Float16);
     uint32_t cps = (w.k_chunks + splits - 1) / splits;
     splits = (w.k_chunks + cps - 1) / cps;  // no empty split
-    const uint32_t col_blocks = (w.n_tiles + 15) / 16, row_blocks = (m + 16 * MT - 1) / (16 * MT);
+    const uint32_t col_blocks = (w.n_tiles + 4 * NTW - 1) / (4 * NTW), row_blocks = (m + 16 * MT - 1) / (16 * MT);
     dim3 grid(col_blocks * row_blocks, 1, splits);  // the kernel turns the linear id into an XCD-aware tile
     // 16-byte row stores: into the partial sums always (padded width, a multiple of 64); into the output when it
     // is one plain [M, N] matrix with N a multiple of 4 at a 16-byte aligned address
@@ -483,7 +499,8 @@ static hipError_t launch_prefill_t(hipStream_t s, const WeightView &w, const _Fl
     if (splits == 1)
         row_store = !out.swiglu && out.count == 1 && out.seg[0].start == 0 && out.seg[0].width == w.n && !out.seg[0].bias &&
                     w.n % 4 == 0 && ((uintptr_t)out.seg[0].ptr & 15) == 0;
-    hipLaunchKernelGGL((k_prefill<MT>), grid, dim3(256), lds, s, (const uint4v *)w.qw, (const uint2v *)w.sc, a, out, m, w.k,
+    if (NTW != 4 && out.swiglu) return hipErrorInvalidValue;
+    hipLaunchKernelGGL((k_prefill<MT, NTW>), grid, dim3(256), lds, s, (const uint4v *)w.qw, (const uint2v *)w.sc, a, out, m, w.k,
                        w.n, w.n_tiles, w.k_chunks, cps, splits > 1 ? partials : nullptr, row_store, col_blocks, row_blocks);
     if (splits > 1) return launch_splitk_reduce(s, partials, out, m, w.n, w.n_tiles * 16, splits);
     return hipGetLastError();
@@ -492,19 +509,22 @@ static hipError_t launch_prefill_t(hipStream_t s, const WeightView &w, const _Fl
 // Once per device, outside any stream capture: the 128-row variant asks for all 64 KB of dynamic LDS.
 hipError_t init_prefill()
 {
-    return hipFuncSetAttribute((const void *)k_prefill<8>, hipFuncAttributeMaxDynamicSharedMemorySize,
+    hipError_t e = hipFuncSetAttribute((const void *)k_prefill<8>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                       2 * 16 * 8 * kPfRowStride * (int)sizeof(_Float16));
+    if (e != hipSuccess) return e;
+    return hipFuncSetAttribute((const void *)k_prefill<8, 3>, hipFuncAttributeMaxDynamicSharedMemorySize,
                                2 * 16 * 8 * kPfRowStride * (int)sizeof(_Float16));
 }
 
-// block_rows: 64 or 128 rows of A per workgroup, splits: k-split factor; 0 = choose (plan_prefill), within what
-// `scratch` can hold as f32 partial sums.
+// block_rows: the block form (64 = 64 rows x 256 columns, 128 = 128 x 256, 192 = 128 rows x 192 columns), splits: k-split
+// factor; 0 = choose (plan_prefill), within what `scratch` can hold as f32 partial sums.
 // `scratch` (scratch_bytes) holds the f16 copy of f32 activations and / or the split-K partials; when it
 // cannot hold all M rows the rows are processed in slabs.
 hipError_t launch_prefill(hipStream_t s, const WeightView &w, const void *a, bool a_f32, uint32_t m, const OutSpec &out,
                           uint32_t block_rows, uint32_t splits, void *scratch, size_t scratch_bytes, const PrefillSk *sk)
 {
     if (m == 0 || w.n == 0) return hipSuccess;
-    if (block_rows != 0 && block_rows != 64 && block_rows != 128) return hipErrorInvalidValue;
+    if (block_rows != 0 && block_rows != 64 && block_rows != 128 && block_rows != 192) return hipErrorInvalidValue;
     auto run = [&](const _Float16 *a16, uint32_t rows, const OutSpec &o, void *ws, size_t ws_bytes) {
         // Option prefill_sk: the tiles dealt out by stream-K (twm_prefill_sk.hip); the gated store stays with the plain kernel.
         if (sk && sk->mode >= 128 && !o.swiglu && sk->partials) {
@@ -514,9 +534,12 @@ hipError_t launch_prefill(hipStream_t s, const WeightView &w, const void *a, boo
             if (e != hipErrorInvalidValue) return e;  // (a shape it does not take: the plain kernel below)
             (void)hipGetLastError();
         }
-        const PrefillPlan plan = plan_prefill_within(rows, block_rows, splits, w.n_tiles, w.k_chunks, ws ? ws_bytes : 0);
-        return plan.block_rows == 64 ? launch_prefill_t<4>(s, w, a16, rows, o, plan.splits, (float *)ws)
-                                     : launch_prefill_t<8>(s, w, a16, rows, o, plan.splits, (float *)ws);
+        // (a forced 192-column form with the gated store: the 256-column one)
+        const uint32_t form = block_rows == 192 && o.swiglu ? 128u : block_rows;
+        const PrefillPlan plan = plan_prefill_within(rows, form, splits, w.n_tiles, w.k_chunks, ws ? ws_bytes : 0, o.swiglu != nullptr);
+        if (plan.block_rows == 64) return launch_prefill_t<4>(s, w, a16, rows, o, plan.splits, (float *)ws);
+        if (plan.block_rows == 192) return launch_prefill_t<8, 3>(s, w, a16, rows, o, plan.splits, (float *)ws);
+        return launch_prefill_t<8>(s, w, a16, rows, o, plan.splits, (float *)ws);
     };
     if (!a_f32) return run((const _Float16 *)a, m, out, scratch, scratch_bytes);
     // f16 copy of the activations at the front of the scratch, partials behind it

@@ -101,12 +101,12 @@ def test_prefill_llama7b_mlp_shapes(dev, m, k, n):
     w.free()
 
 
-@pytest.mark.parametrize("bm,m,n", [(128, 680, 5848), (64, 680, 5848), (128, 1024, 8192)])
+@pytest.mark.parametrize("bm,m,n", [(128, 680, 5848), (64, 680, 5848), (128, 1024, 8192), (192, 680, 5848), (192, 1024, 11008)])
 def test_prefill_xcd_tile_order_with_ragged_bands(dev, bm, m, n):
     # The tile order that keeps an XCD's workgroups on a patch of the output is taken from 128 tiles on.  680 rows x
     # 5848 columns: 6 x 23 = 138 tiles of 128 x 256 (not a multiple of 8, last band two row blocks high, last row and
     # column blocks ragged) and 11 x 23 = 253 tiles of 64 x 256 (bands of eight, the last three high); 1024 x 8192
-    # is the even case.  Every output is compared (K is shallow), and a NaN canary catches a tile nobody wrote.
+    # is the even case; 192-column blocks make 6 x 31 (ragged last block) and 8 x 58 tiles.  Every output is compared (K is shallow), and a NaN canary catches a tile nobody wrote.
     k = 256
     packed, scales, a16 = synth(k, n, m, 7100 + bm + n)
     w = T.MarlinWeight.upload(dev, packed, scales, k, n)

@@ -959,7 +959,7 @@ def test_prefill_kernel_matches_oracle(dev, m, k, n):
     # Against the f32-weight matmul the FP16 rounding of the weights (2^-12 relative each) shows on
     # near-cancelling outputs, so that comparison is made relative to the largest output.
     # Ragged M (33, 200), K not a multiple of 128 (1184), N not a multiple of 256 / 64 (200, 704); 1 to 5
-    # k-chunks (the k loop is unrolled by three with a remainder); both workgroup heights.
+    # k-chunks (the k loop is unrolled by three with a remainder); every block form.
     packed, scales, a16 = synth(k, n, m, 4000 + m)
     w = T.MarlinWeight.upload(dev, packed, scales, k, n)
     a = f16_as_f32(a16)
@@ -968,7 +968,7 @@ def test_prefill_kernel_matches_oracle(dev, m, k, n):
     truth = O.gemm_f64(a, packed, scales, m, k, n)
     try:
         dev.set_option("prefill_min_m", 1)
-        for bm in (64, 128):
+        for bm in (64, 128, 192):   # 192: 128 rows x 192 columns, three tiles per wave
             dev.set_option("prefill_bm", bm)
             for a_f32 in (False, True):
                 got = run_gemm(dev, w, a16, m, n, a_f32=a_f32)
@@ -1006,7 +1006,7 @@ def test_prefill_split_k(dev, m, k, n):
     w16 = O.dequant_f16(packed, scales, k, n).view(np.float16).astype(np.float64)
     exact = a.astype(np.float64) @ w16
     try:
-        for bm in (64, 128):
+        for bm in (64, 128, 192):   # 192: 128 rows x 192 columns, three tiles per wave
             dev.set_option("prefill_bm", bm)
             base = run_gemm(dev, w, a16, m, n, splits=1)
             assert rel_err(base, exact) < 1e-3
