@@ -20,12 +20,18 @@
 
 #include <type_traits>
 
+// (two workgroups of four waves per CU: the compiler keeps the kernel within 256 registers)
+#define TWM_PF_OCC(HALF) __attribute__((amdgpu_waves_per_eu((HALF) ? 2 : 1)))
+
 namespace twm {
 
 // MT = 16-row blocks per workgroup tile (BM = 16 * MT rows); NTW = 16-column tiles per wave: 4 (256-column blocks) or
 // 3 (192-column blocks, for shapes whose 256-column blocks leave a round of workgroups mostly empty)
-template <int MT, int NTW = 4>
-__global__ __launch_bounds__(256) void k_prefill(const uint4v *__restrict__ qw, const uint2v *__restrict__ sc,
+// HALF: the MFMAs of a 32-deep group run as two half steps of MT / 2 row blocks, and the A operands are read half a step
+// ahead instead of a whole one: MT / 2 x 2 operand registers less, which with NTW = 3 brings the kernel under 256
+// registers, so that two workgroups share a CU and one's MFMAs fill the issue gaps of the other.
+template <int MT, int NTW = 4, bool HALF = false>
+__global__ __launch_bounds__(256) TWM_PF_OCC(HALF) void k_prefill(const uint4v *__restrict__ qw, const uint2v *__restrict__ sc,
                                                   const _Float16 *__restrict__ a_any, OutSpec out, uint32_t m_rows,
                                                   uint32_t k, uint32_t n, uint32_t n_tiles, uint32_t k_chunks,
                                                   uint32_t chunks_per_split, float *__restrict__ partials,
@@ -144,26 +150,44 @@ __global__ __launch_bounds__(256) void k_prefill(const uint4v *__restrict__ qw, 
         return *(const half8 *)(a_lds + buf * kPfTileHalves + rd_off[g] + mt * 16 * kPfRowStride);
     };
 
-    half8 af0[MT], af1[MT];
+    constexpr int AF = HALF ? MT / 2 : MT;   // row blocks whose A operands are held at a time
+    half8 af0[AF], af1[AF];
     PfFrag bf0[NTW], bf1[NTW];
 
-    // One step = the MFMAs of one 32-deep group, in MT units of four (one row block x four tiles).  Unit mt
+    // One step = the MFMAs of one 32-deep group, in MT units of NTW (one row block x NTW tiles).  Unit mt
     // also fetches the next group's A operand for its row block, unpacks its share of the next group's B
     // operands and issues `extra(mt)`, its share of the traffic for later chunks.  The scheduling barrier
     // after each unit keeps this interleaving: one MFMA issue slot hides about two other instructions,
     // but only if they sit next to it.
-    auto step = [&](const half8 (&af_cur)[MT], const PfFrag (&bf_cur)[NTW], half8 (&af_nxt)[MT], PfFrag (&bf_nxt)[NTW],
+    auto step = [&](const half8 (&af_cur)[AF], const PfFrag (&bf_cur)[NTW], half8 (&af_nxt)[AF], PfFrag (&bf_nxt)[NTW],
                     uint32_t rd_buf, int rd_g, int uq_slot, int uq_g, auto extra) {
 #pragma unroll
         for (int mt = 0; mt < MT; mt++) {
-            af_nxt[mt] = read_a(rd_buf, rd_g, mt);
+            af_nxt[mt % AF] = read_a(rd_buf, rd_g, mt);
             extra(mt);
             // the 2 NTW half fragments of the next group, dealt over the MT units
 #pragma unroll
             for (int hp = mt * HP / MT; hp < (mt + 1) * HP / MT; hp++) unpack(uq_slot, uq_g, bf_nxt, hp);
 #pragma unroll
             for (int t = 0; t < NTW; t++)
-                acc[mt][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(af_cur[mt], bf_cur[t].h, acc[mt][t], 0, 0, 0);
+                acc[mt][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(af_cur[mt % AF], bf_cur[t].h, acc[mt][t], 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+    // Half step h of group g: the MFMAs of row blocks h MT/2 .. with the operands in af_cur; unit u reads the operand of
+    // row block (1 - h) MT/2 + u of group rd_g for the next half step, and unpacks its share (part h) of the next group.
+    auto half_step = [&](int h, const half8 (&af_cur)[AF], const PfFrag (&bf_cur)[NTW], half8 (&af_nxt)[AF], PfFrag (&bf_nxt)[NTW],
+                         uint32_t rd_buf, int rd_g, int uq_slot, int uq_g, auto extra) {
+#pragma unroll
+        for (int u = 0; u < AF; u++) {
+            const int mt = h * AF + u;
+            af_nxt[u] = read_a(rd_buf, rd_g, (1 - h) * AF + u);
+            extra(u);
+#pragma unroll
+            for (int hp = mt * HP / MT; hp < (mt + 1) * HP / MT; hp++) unpack(uq_slot, uq_g, bf_nxt, hp);
+#pragma unroll
+            for (int t = 0; t < NTW; t++)
+                acc[mt][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(af_cur[u], bf_cur[t].h, acc[mt][t], 0, 0, 0);
             __builtin_amdgcn_sched_barrier(0);
         }
     };
@@ -176,24 +200,43 @@ __global__ __launch_bounds__(256) void k_prefill(const uint4v *__restrict__ qw, 
     //   step 3   : A tile kc+2 -> buffer kc & 1 and B of chunk kc+2 -> slot S (its last group was unpacked in
     //              step 2); the step's own reads and unpack are already those of chunk kc+1, group 0
     // Past the end the last chunk is loaded again and never used.
+    // HALF: eight half steps; the last reads of tile kc are those of half step 6 (group 3, second half), so the wait
+    // for the loads stands before half step 6 (which already unpacks chunk kc+1), the barrier behind it, and half step 7
+    // issues the loads of chunk kc+2.  On entry af0 holds the first half of group 0.
     auto chunk = [&](auto slot_c, uint32_t kc) {
         constexpr int S = decltype(slot_c)::value, S1 = S ^ 1;
         const uint32_t buf = kc & 1u;
         const uint32_t kc2 = kc + 2 < last ? kc + 2 : last;
-        step(af0, bf0, af1, bf1, buf, 1, S, 1, [&](int) {});
-        step(af1, bf1, af0, bf0, buf, 2, S, 2, [&](int) {});
-        step(af0, bf0, af1, bf1, buf, 3, S, 3, [&](int) {});
-        wait_loads();
-        __syncthreads();
-        step(af1, bf1, af0, bf0, buf ^ 1u, 0, S1, 0, [&](int u) {
-            if (u < NV) load_a(buf, kc2, u);
-            // B of chunk kc + 2 into this chunk's own slot, whose last group was unpacked in step 2
+        auto later_loads = [&](int u, int units) {
+            // (the A parts and the B tiles of chunk kc + 2, dealt over `units` units)
+#pragma unroll
+            for (int j = 0; j < NV; j++)
+                if (j * units / NV == u) load_a(buf, kc2, j);
 #pragma unroll
             for (int t = 0; t < NTW; t++) {
-                if (t * MT / 4 == u) load_bq(S, kc2, t);
-                if (t * MT / 4 + (MT >= 8 ? 1 : 0) == u) load_bs(S, kc2, t);
+                if (t * units / 4 == u) load_bq(S, kc2, t);
+                if (t * units / 4 + (units >= 8 ? 1 : 0) == u) load_bs(S, kc2, t);
             }
-        });
+        };
+        if constexpr (HALF) {
+            half_step(0, af0, bf0, af1, bf1, buf, 0, S, 1, [&](int) {});
+            half_step(1, af1, bf0, af0, bf1, buf, 1, S, 1, [&](int) {});
+            half_step(0, af0, bf1, af1, bf0, buf, 1, S, 2, [&](int) {});
+            half_step(1, af1, bf1, af0, bf0, buf, 2, S, 2, [&](int) {});
+            half_step(0, af0, bf0, af1, bf1, buf, 2, S, 3, [&](int) {});
+            half_step(1, af1, bf0, af0, bf1, buf, 3, S, 3, [&](int) {});
+            wait_loads();
+            half_step(0, af0, bf1, af1, bf0, buf, 3, S1, 0, [&](int) {});
+            __syncthreads();
+            half_step(1, af1, bf1, af0, bf0, buf ^ 1u, 0, S1, 0, [&](int u) { later_loads(u, AF); });
+        } else {
+            step(af0, bf0, af1, bf1, buf, 1, S, 1, [&](int) {});
+            step(af1, bf1, af0, bf0, buf, 2, S, 2, [&](int) {});
+            step(af0, bf0, af1, bf1, buf, 3, S, 3, [&](int) {});
+            wait_loads();
+            __syncthreads();
+            step(af1, bf1, af0, bf0, buf ^ 1u, 0, S1, 0, [&](int u) { later_loads(u, MT); });
+        }
         pin_acc();
     };
     using S0 = std::integral_constant<int, 0>;
@@ -215,7 +258,7 @@ __global__ __launch_bounds__(256) void k_prefill(const uint4v *__restrict__ qw, 
     wait_loads();
     __syncthreads();
 #pragma unroll
-    for (int mt = 0; mt < MT; mt++) af0[mt] = read_a(0, 0, mt);
+    for (int mt = 0; mt < AF; mt++) af0[mt] = read_a(0, 0, mt);
 #pragma unroll
     for (int hp = 0; hp < HP; hp++) unpack(0, 0, bf0, hp);
     __builtin_amdgcn_sched_barrier(0);
@@ -401,12 +444,14 @@ hipError_t launch_splitk_reduce(hipStream_t s, const float *partials, const OutS
 // store; a split costs the second kernel, 2.5 + its read of the partial sums at 4 TB/s.  (128-row blocks unpack
 // every weight for twice the rows: per row they are the cheapest form as soon as there is a workgroup for most
 // CUs, and K 4096 -> N 11008 at M = 512 runs in 50 us on 172 of them against 61 us on 344 64-row blocks.)
-// Forms: 64 = 64 rows x 256 columns, 128 = 128 x 256, 192 = 128 rows x 192 columns (three tiles per wave; it pays where
-// it fills a round of workgroups that 256-column blocks leave mostly empty: 4096 -> 11008 at M = 1024 90.5 against
-// 95.9 us, 3584 -> 4608 at M = 2048 76.7 against 82.6; on full rounds a chunk of it takes 0.95 of a 256-column
-// block's chunk for 0.75 of the columns, 4096 -> 11008 at M = 2048 179 against 161 us.  kPf192 is the weight that
-// reproduces the best form on the 25 cases of the sweep, not that ratio.  Not with the gated store, whose waves hold
-// gate and up tiles in pairs).
+// Forms: 64 = 64 rows x 256 columns, 128 = 128 x 256, 192 = 128 rows x 192 columns (three tiles per wave).  Alone on a
+// CU a chunk of the 192-column form takes 0.95 of a 256-column block's chunk for 0.75 of the columns; it pays where
+// it fills a round of workgroups that 256-column blocks leave mostly empty (4096 -> 11008 at M = 512: 232 workgroups
+// instead of 172, 46.1 against 47.8 us; kPf192 is the weight that reproduces the best form on the sweep's cases with
+// up to 256 workgroups, not that ratio).  With more workgroups than CUs its two-per-CU variant runs (the kernel's HALF
+// form, under 256 registers): 4096 -> 11008 at M = 1024 81.6 us against 102.5 on 256-column blocks, 3584 -> 4608 at
+// M = 2048 66.9 against 90.7, 3584 -> 37888 at M = 2048 462 against 476; level at 4096 -> 11008, M = 2048 (158.7 / 158.0).
+// Not with the gated store, whose waves hold gate and up tiles in pairs.
 constexpr double kPf192 = 0.80;
 struct PrefillPlan {
     uint32_t block_rows, splits;   // block_rows: the form (64, 128, 192)
@@ -429,7 +474,11 @@ static PrefillPlan plan_prefill(uint32_t rows, uint32_t force_rows, uint32_t for
             if (!force_splits && (k_chunks + cps - 1) / cps != sp) continue;  // same work as a smaller factor
             const double total = wgs * sp;
             double t;
-            if (bm >= 128) {
+            if (bm == 192 && total > 256.0) {
+                // two workgroups share a CU: 2.45 per chunk each; a last round of up to one per CU runs at 1.45
+                const double full = (double)(uint64_t)(total / 512.0), rem = total - 512.0 * full;
+                t = full * (cps * 2.45 + 3.0) + (rem == 0.0 ? 0.0 : (rem <= 256.0 ? cps * 1.45 : cps * 2.45) + 3.0);
+            } else if (bm >= 128) {
                 const double rounds = (double)(uint64_t)((total + 255.0) / 256.0);
                 const double load = total >= 256.0 ? 1.0 : total / 256.0;
                 t = rounds * (cps * (1.5 + 0.3 * load) * (bm == 192 ? kPf192 : 1.0) + 3.0);
@@ -484,7 +533,7 @@ void prefill_plan_of(uint32_t rows, uint32_t block_rows, uint32_t splits, uint32
     *splits_out = plan.splits;
 }
 
-template <int MT, int NTW = 4>
+template <int MT, int NTW = 4, bool HALF = false>
 static hipError_t launch_prefill_t(hipStream_t s, const WeightView &w, const _Float16 *a, uint32_t m, const OutSpec &out,
                                    uint32_t splits, float *partials)
 {
@@ -500,7 +549,7 @@ static hipError_t launch_prefill_t(hipStream_t s, const WeightView &w, const _Fl
         row_store = !out.swiglu && out.count == 1 && out.seg[0].start == 0 && out.seg[0].width == w.n && !out.seg[0].bias &&
                     w.n % 4 == 0 && ((uintptr_t)out.seg[0].ptr & 15) == 0;
     if (NTW != 4 && out.swiglu) return hipErrorInvalidValue;
-    hipLaunchKernelGGL((k_prefill<MT, NTW>), grid, dim3(256), lds, s, (const uint4v *)w.qw, (const uint2v *)w.sc, a, out, m, w.k,
+    hipLaunchKernelGGL((k_prefill<MT, NTW, HALF>), grid, dim3(256), lds, s, (const uint4v *)w.qw, (const uint2v *)w.sc, a, out, m, w.k,
                        w.n, w.n_tiles, w.k_chunks, cps, splits > 1 ? partials : nullptr, row_store, col_blocks, row_blocks);
     if (splits > 1) return launch_splitk_reduce(s, partials, out, m, w.n, w.n_tiles * 16, splits);
     return hipGetLastError();
@@ -512,7 +561,10 @@ hipError_t init_prefill()
     hipError_t e = hipFuncSetAttribute((const void *)k_prefill<8>, hipFuncAttributeMaxDynamicSharedMemorySize,
                                        2 * 16 * 8 * kPfRowStride * (int)sizeof(_Float16));
     if (e != hipSuccess) return e;
-    return hipFuncSetAttribute((const void *)k_prefill<8, 3>, hipFuncAttributeMaxDynamicSharedMemorySize,
+    e = hipFuncSetAttribute((const void *)k_prefill<8, 3>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                            2 * 16 * 8 * kPfRowStride * (int)sizeof(_Float16));
+    if (e != hipSuccess) return e;
+    return hipFuncSetAttribute((const void *)k_prefill<8, 3, true>, hipFuncAttributeMaxDynamicSharedMemorySize,
                                2 * 16 * 8 * kPfRowStride * (int)sizeof(_Float16));
 }
 
@@ -538,7 +590,13 @@ hipError_t launch_prefill(hipStream_t s, const WeightView &w, const void *a, boo
         const uint32_t form = block_rows == 192 && o.swiglu ? 128u : block_rows;
         const PrefillPlan plan = plan_prefill_within(rows, form, splits, w.n_tiles, w.k_chunks, ws ? ws_bytes : 0, o.swiglu != nullptr);
         if (plan.block_rows == 64) return launch_prefill_t<4>(s, w, a16, rows, o, plan.splits, (float *)ws);
-        if (plan.block_rows == 192) return launch_prefill_t<8, 3>(s, w, a16, rows, o, plan.splits, (float *)ws);
+        if (plan.block_rows == 192) {
+            // more workgroups than CUs: the variant of which two share a CU (4096 -> 11008 at M = 1024, 464 workgroups:
+            // 81.6 against 89.5 us; at M = 512, 232 workgroups, 49.0 against 46.4)
+            const uint64_t wgs = (uint64_t)((w.n_tiles + 11) / 12) * ((rows + 127) / 128) * plan.splits;
+            return wgs > 256 ? launch_prefill_t<8, 3, true>(s, w, a16, rows, o, plan.splits, (float *)ws)
+                             : launch_prefill_t<8, 3>(s, w, a16, rows, o, plan.splits, (float *)ws);
+        }
         return launch_prefill_t<8>(s, w, a16, rows, o, plan.splits, (float *)ws);
     };
     if (!a_f32) return run((const _Float16 *)a, m, out, scratch, scratch_bytes);

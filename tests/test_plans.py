@@ -51,7 +51,7 @@ def test_plans_of_the_qwen7b_projections(lib, name, m, dtype, want):
 
 
 @pytest.mark.parametrize("k,n,m,want", [
-    (4096, 11008, 2048, "k_prefill: 128-row x 256-column blocks, 1 K-split; 16-column tile copy"),
+    (4096, 11008, 2048, "k_prefill: 128-row x 192-column blocks, 1 K-split; 16-column tile copy"),   # 928 workgroups, two per CU
     (11008, 4096, 2048, "k_prefill: 128-row x 256-column blocks, 1 K-split; 16-column tile copy"),
     (4096, 11008, 512, "k_prefill: 128-row x 192-column blocks, 1 K-split; 16-column tile copy"),   # 232 workgroups instead of 172
     (11008, 4096, 512, "k_prefill: 128-row x 256-column blocks, 4 K-splits + k_splitk_reduce; 16-column tile copy"),
