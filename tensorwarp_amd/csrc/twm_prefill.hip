@@ -138,9 +138,7 @@ __global__ __launch_bounds__(256) TWM_PF_OCC(HALF) void k_prefill(const uint4v *
     // half fragment hp (tile hp / 2, half hp % 2) of group g
     auto unpack = [&](int slot, int g, PfFrag (&bf)[NTW], int hp) {
         const int t = hp >> 1;
-        uint32_t pair = bs[slot][t][g >> 1];
-        uint32_t s16 = (g & 1) ? (pair >> 16) : (pair & 0xFFFFu);
-        pf_unpack_half(bf[t], hp & 1, bq[slot][t][g], s16, dq);
+        pf_unpack_half(bf[t], hp & 1, bq[slot][t][g], bs[slot][t][g >> 1], g & 1, dq);
     };
 
     uint32_t rd_off[4];  // row c of a row block, vector 4 g + kb of the chunk -> slot (4 g + kb) ^ c

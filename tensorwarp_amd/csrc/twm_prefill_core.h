@@ -38,10 +38,13 @@ union PfFrag {
 
 // Half of a fragment: nibbles 0..3 (half 0) or 4..7 (half 1) of word `w` -> f16(scale * (q - 8)).
 // 1024 + q and 64 + q are built by OR-ing the nibble into an f16 mantissa; the subtraction is exact.
-__device__ __forceinline__ void pf_unpack_half(PfFrag &r, int half, uint32_t w, uint32_t scale16, const PfConsts &c)
+// scale_pair holds two groups' f16 scales; `odd` says which one counts (a splat of one half of a register is free: the
+// packed multiply selects the half for both of its lanes).
+__device__ __forceinline__ void pf_unpack_half(PfFrag &r, int half, uint32_t w, uint32_t scale_pair, int odd, const PfConsts &c)
 {
-    union { uint32_t u; half2v h; } s2;
-    s2.u = scale16 | (scale16 << 16);
+    union { uint32_t u; half2v h; } sp, s2;
+    sp.u = scale_pair;
+    s2.h = odd ? half2v{sp.h[1], sp.h[1]} : half2v{sp.h[0], sp.h[0]};
     const half2v b_lo = {(_Float16)-1032.0f, (_Float16)-1032.0f};
     const half2v b_hi = {(_Float16)-72.0f, (_Float16)-72.0f};
     if (half) w >>= 8;

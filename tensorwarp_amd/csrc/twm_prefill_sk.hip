@@ -140,9 +140,7 @@ __global__ __launch_bounds__(256) void k_prefill_sk(const uint4v *__restrict__ q
         };
         auto unpack = [&](int slot, int g, PfFrag (&bf)[4], int hp) {  // half fragment hp (tile hp / 2, half hp % 2) of group g
             const int t = hp >> 1;
-            uint32_t pair = bs[slot][t][g >> 1];
-            uint32_t s16 = (g & 1) ? (pair >> 16) : (pair & 0xFFFFu);
-            pf_unpack_half(bf[t], hp & 1, bq[slot][t][g], s16, dq);
+            pf_unpack_half(bf[t], hp & 1, bq[slot][t][g], bs[slot][t][g >> 1], g & 1, dq);
         };
         auto read_a = [&](uint32_t buf, int g, int mt) {
             return *(const half8 *)(a_lds + buf * kTileHalves + rd_off[g] + mt * 16 * kPfRowStride);
