@@ -21,7 +21,7 @@
 #include <type_traits>
 
 // (two workgroups of four waves per CU: the compiler keeps the kernel within 256 registers)
-#define TWM_PF_OCC(HALF) __attribute__((amdgpu_waves_per_eu((HALF) ? 2 : 1)))
+#define TWM_PF_OCC(TWO) __attribute__((amdgpu_waves_per_eu((TWO) ? 2 : 1)))
 
 namespace twm {
 
