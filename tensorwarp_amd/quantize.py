@@ -62,6 +62,12 @@ class WarpDevice:
     def set_option(self, key, value):
         _check(self._l.twm_ctx_set_option(self.handle, key.encode(), int(value)))
 
+    def plan(self, k, n, m, dtype="f16", gated=False):
+        """What gemm() would launch for a K x N weight and m rows under this context's options, as a line of text."""
+        buf = C.create_string_buffer(256)
+        _check(self._l.twm_plan_describe(self.handle, k, n, m, _lib.F32 if dtype == "f32" else _lib.F16, int(gated), buf, 256))
+        return buf.value.decode()
+
     # timing
     def event(self):
         ev = self._l.twm_event_create(self.handle)

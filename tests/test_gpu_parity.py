@@ -1482,6 +1482,32 @@ def test_indirect_gemv_reads_the_offset_tables_on_the_device(dev):
 
 # ---------------------------------------------------------------- fused projections
 
+def test_plan_description_follows_the_context_options(dev):
+    # twm_plan_describe with a context: the options that force a launch form show in the description, and the
+    # described form is the one that runs (same result bits as forcing it by hand is not observable from outside;
+    # the split factor is: it changes the summation order)
+    k, n = 3584, 3584
+    assert dev.plan(k, n, 1).startswith("k_gemv4s: 16-column sub-tiles, 8 waves")
+    dev.set_option("sub", 1)
+    try:
+        assert dev.plan(k, n, 1).startswith("k_gemv4: 1 x 64-column tiles per workgroup")
+    finally:
+        dev.set_option("sub", 0)
+    dev.set_option("kernel", 3)
+    try:
+        assert dev.plan(k, n, 16).startswith("k_stream:")
+    finally:
+        dev.set_option("kernel", 0)
+    dev.set_option("prefill_min_m", 8)
+    try:
+        assert dev.plan(k, n, 16).startswith("k_prefill:")
+    finally:
+        dev.set_option("prefill_min_m", 33)
+    assert dev.plan(k, n, 16).startswith("k_gemv4s:")
+    assert dev.plan(3584, 37888, 1, gated=True).startswith("k_gemv4s: 32-column sub-tiles")
+    assert dev.plan(18944, 3584, 1, dtype="f32") == "k_gemv4s: 16-column sub-tiles, 4 waves, 1 K-split; column-lane copy"
+
+
 def test_fusing_handles_equals_fusing_the_arrays(dev):
     # fuse_tw_marlin_n (quantize.rs:1018-1063) on repacked handles: block copies of both copies; the results of every
     # kernel family are bit-identical to those of a handle made from the fused arrays
