@@ -66,6 +66,9 @@ __device__ __forceinline__ half8 bt_unpack(uint32_t w, const BtConsts &c)
 }
 
 constexpr int kBtRow = 128;  // halves per LDS row (256 bytes)
+// register slots of a wave's loads (even: the LDS buffer of a chunk is slot & 1).  Three chunks in flight are enough:
+// with six or eight slots 3584 -> 37888 at M = 32 read 23.5 / 24.9 us against 23.5 - 24.1, narrower matrices 4 - 8 % more
+constexpr int kBtSlots = 4;
 
 }  // namespace
 
@@ -89,7 +92,7 @@ __global__ __launch_bounds__(64 * WPS * KS) void k_batch(const uint4v *__restric
                                                 uint32_t lo_offset, float *__restrict__ partials, OutSpec out)
 {
     constexpr bool kRounded = RND;           // weights rounded to f16 as in the reference's dequant-then-FP16-GEMM route (option)
-    constexpr int S = 4;                     // register slots: chunk kc lives in slot kc % S, three chunks are in flight
+    constexpr int S = kBtSlots;              // register slots: chunk kc lives in slot kc % S, S - 1 chunks are in flight
     constexpr int kTile = 16 * MT * kBtRow;  // halves of one term's tile
     constexpr int kBuf = TERMS * kTile;      // halves of one LDS buffer
     static_assert(TPW == 1 || WPS == 4, "two tiles per wave: four waves per slice");
@@ -225,7 +228,7 @@ __global__ __launch_bounds__(64 * WPS * KS) void k_batch(const uint4v *__restric
         }
     };
 
-    // One chunk (slot = kc % 4, LDS buffer kc % 2): loads of chunk kc + 3 go out first; the chunk is computed from its
+    // One chunk (slot = kc % S, LDS buffer kc % 2): loads of chunk kc + S - 1 go out first; the chunk is computed from its
     // LDS buffer and its weight slot; then this wave's part of A tile kc + 1 goes from its registers to the other
     // buffer (every wave finished reading that buffer before the previous barrier); the barrier makes the tile
     // complete.  Past the end the last chunk is loaded again and never used, so that every step issues the same loads
@@ -235,14 +238,14 @@ __global__ __launch_bounds__(64 * WPS * KS) void k_batch(const uint4v *__restric
         return rel < my_last ? rel : my_last;
     };
     auto step = [&](int slot, uint32_t i) {
-        load_chunk((slot + 3) % S, chunk_of(i + 3u));
+        load_chunk((slot + S - 1) % S, chunk_of(i + (uint32_t)(S - 1)));
         if (KS == 1 || i < my_count) compute(slot, slot & 1);  // (uniform over the wave)
         stage_a((slot + 1) % S, (slot + 1) & 1);
         __syncthreads();
     };
 
 #pragma unroll
-    for (int s = 0; s < 3; s++) load_chunk(s, chunk_of((uint32_t)s));
+    for (int s = 0; s < S - 1; s++) load_chunk(s, chunk_of((uint32_t)s));
     stage_a(0, 0);
     __syncthreads();
     uint32_t i0 = 0;
