@@ -196,7 +196,7 @@ int twm_argmax_f32(twm_ctx *ctx, const float *input_dev, uint32_t rows, uint32_t
  * f32 activations and output, arrays exactly as the reference holds them (packed at least 4-byte aligned, the
  * alignment the reference's own kernel needs; 16-byte aligned for the fast kernel).
  * Runs the M <= 4 MFMA kernel straight on those arrays: weights (q - 8) exact, every f32 activation
- * enters as two f16 terms a = f16(a) + f16(a - f16(a)) (about 22 bits; any finite f32: where a value lies
+ * enters as two f16 terms, a first term and the residual a - first (about 21 bits; any finite f32: where a value lies
  * beyond the f16 range, the kernel first scales that stretch of the row by a power of two and the sums back, both
  * exact), f32 sum per group times f32(scale), deterministic split-K.  Option "m1_exact" selects the
  * plain f32 kernel in the reference's order instead (also taken when a_dev or packed_dev is not 16-byte aligned).
@@ -284,7 +284,7 @@ int twm_weight_dequant_f16(twm_ctx *ctx, const twm_weight *w, uint16_t *out_kn_d
  * M <= 32: decode kernels (M <= 4 one lane per column, above that 16-column tiles), weights exact,
  *          each group's f32 sum scaled by f32(scale): a row's result does not depend on the batch it is in
  *          beyond f32 summation order.  (Option "batch_rounded": M = 17 .. 32 on the FP16 Q4 unpack.)
- * Up to M = 32 f32 activations enter as two f16 terms, f16(a) + f16(a - f16(a)), about 22 bits.  M <= 4 takes any
+ * Up to M = 32 f32 activations enter as two f16 terms, a first term and the residual, about 21 bits.  M <= 4 takes any
  * finite f32 (values beyond the f16 range are scaled into it by a power of two per row, and the sums back); from
  * M = 5 on |a| must stay inside the f16 range, as in the reference's FP16 route for M > 1.
  * M  > 32: prefill GEMM on the same FP16 unpack; f32 activations are rounded to f16 first.  Uses the

@@ -13,6 +13,9 @@
 // workgroup of eight waves makes exactly one pass: every load of the launch is issued at once, the kernel has
 // no loop and needs about 50 registers, and 3584 -> 37888 becomes 2368 short-lived workgroups.
 // Rows five to sixteen (f16) repeat the MFMA chain on the unpacked weights per group of four rows.
+// One row of activations, f16 in the pipelined loop or f32 anywhere, is loaded a piece per lane and handed round the
+// quads of lanes by DPP (the term modes kTermsOneRow / kTermsOneRowF32 of twm_gemv4_core.h); f32 values are taken as
+// two f16 terms, first term and residual, which ride in rows 0 and 1 of the MFMA's A block.
 //
 // Arithmetic and output as k_gemv4 (crates/kernels/src/quantize.rs:1186-1298).
 #include "twm_gemv4_core.h"
