@@ -542,15 +542,17 @@ extern "C++" int twm::m1_dispatch(const M1Env &env, const char *who, const float
     // the M <= 4 MFMA kernels reading the reference's arrays as they are (f32 activations as two f16 terms)
     uint32_t n_pad = ((n + 63) / 64) * 64, k_chunks = (k / 32 + kChunkGroups - 1) / kChunkGroups;
     // On the reference's arrays a wave's four group rows of a chunk are N x 16 bytes apart, and many waves in flight
-    // with one pass each pay better than on the contiguous copy: the sub-tile kernel with sixteen waves on 32
-    // columns as long as every wave gets a single pass (K <= 4096), or with 16 columns when 64-column tiles number no
-    // more than 64.  Deeper wide matrices keep the 64-column kernel and its split-K (8192 -> 57344: 46.6 against
-    // 63.7 us).  Fitted to sweeps over the
-    // Qwen2.5-7B, Llama-3-8B, 13B and 70B projections; option "sub" = 1 keeps the 64-column kernel.
+    // with one pass each pay better than on the contiguous copy.  The sub-tile kernel on 16 columns when 64-column tiles
+    // number no more than 64 (any K: deeper ones in the pipelined pass loop on sixteen waves: 18944 -> 3584 10.8 us,
+    // 14336 -> 4096 9.7) and, eight waves of one pass each, on wide matrices up to K = 4096 (3584 -> 37888 16.3 against
+    // 18.1 us on 32 columns, 4096 -> 22016 11.8 against 12.5, 4096 -> 28672 14.6 against 15.8); in between sixteen waves
+    // on 32 columns as long as every wave gets a single pass (3584 -> 4608 4.7 against 4.9, 4096 -> 6144 5.1 against
+    // 5.5).  Deeper wide matrices keep the 64-column kernel and its split-K (8192 -> 57344: 46.6 against 63.7 us).
+    // Fitted to sweeps over the Qwen2.5-7B, Llama-2-7B, Llama-3-8B, 13B and 70B projections; option "sub" = 1 keeps the
+    // 64-column kernel.
     const uint32_t tiles64 = n_pad / 64, passes16 = (k_chunks + 3) / 4, passes32 = (k_chunks + 1) / 2;
-    uint32_t sub = tiles64 <= 64 ? 16 : 32, sub_waves = (sub == 16 && passes16 <= 8) ? 8 : 16;
-    // (on 16 columns a deeper K runs the pipelined pass loop on sixteen waves: 18944 -> 3584 12.5 against 12.8 us,
-    // 14336 -> 4096 10.8 against 11.7)
+    const bool narrow16 = tiles64 <= 64, wide16 = tiles64 >= 256 && passes16 <= 8;
+    uint32_t sub = narrow16 || wide16 ? 16 : 32, sub_waves = (sub == 16 && passes16 <= 8) ? 8 : 16;
     bool use_sub = env.force_sub != 1 && (sub == 16 || passes32 <= 16);
     if (env.force_sub >= 16) {
         sub = (uint32_t)env.force_sub;

@@ -449,7 +449,7 @@ __device__ __forceinline__ void gemv4s_load_pass_ref(ChunkS<SUB, RG> &r, const c
         const uint32_t gg = kc * 4u + g;
         idx[g] = (size_t)(gg < groups ? gg : groups - 1u) * n + col;
         keep[g] = (live && gg < groups && col_ok) ? 0xFFFFu : 0u;  // weight exactly 0 otherwise
-        sb[g] = ld_once(scales + idx[g]);
+        sb[g] = scales[idx[g]];  // (cached: the line holds the scales of the neighbouring sub-tiles, which run on the same XCD)
     }
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll

@@ -26,6 +26,17 @@ namespace twm {
 
 namespace {
 
+// the launch's small numbers in one argument word: K-splits (bits 0-11; the launchers cap the factor at 4095), gated
+// store (12), waves per workgroup (13-17), rows (18-22)
+__host__ __device__ __forceinline__ uint32_t gemv4s_cfg(uint32_t splits, bool gated, uint32_t waves, uint32_t rows)
+{
+    return splits | (gated ? 0x1000u : 0u) | (waves << 13) | (rows << 18);
+}
+__device__ __forceinline__ uint32_t cfg_splits(uint32_t cfg) { return cfg & 0xFFFu; }
+__device__ __forceinline__ bool cfg_gated(uint32_t cfg) { return (cfg & 0x1000u) != 0; }
+__device__ __forceinline__ uint32_t cfg_waves(uint32_t cfg) { return (cfg >> 13) & 0x1Fu; }
+__device__ __forceinline__ uint32_t cfg_rows(uint32_t cfg) { return (cfg >> 18) & 0x1Fu; }
+
 __device__ __forceinline__ void gemv4s_store_out(const OutSpec &out, uint32_t m, uint32_t col, float v)
 {
 #pragma unroll
@@ -45,11 +56,13 @@ __device__ __forceinline__ void gemv4s_store_out(const OutSpec &out, uint32_t m,
 // activations): a sub-tile's records of one group are still SUB * 16 contiguous bytes.
 template <int SUB, int RL, bool AF32, bool ONE, bool REFL>
 __device__ __forceinline__ void gemv4s_body(const char *__restrict__ cw, const void *__restrict__ a_any, const OutSpec &out,
-                                            float *__restrict__ ws, unsigned *__restrict__ counters, uint32_t m_rows,
+                                            float *__restrict__ ws, unsigned *__restrict__ counters, uint32_t cfg,
                                             uint32_t k, uint32_t n, uint32_t n_pad, uint32_t k_chunks,
-                                            uint32_t sub_tiles, uint32_t splits, uint32_t cps, bool gated_store,
+                                            uint32_t sub_tiles, uint32_t cps,
                                             const uint16_t *__restrict__ ref_scales, uint32_t *trace_loaded)
 {
+    const uint32_t splits = cfg_splits(cfg), waves = cfg_waves(cfg), m_rows = cfg_rows(cfg);
+    const bool gated_store = cfg_gated(cfg);
     static_assert(!REFL || (AF32 && RL == 1), "the reference-layout variant is the M = 1, f32-activation entry point");
     constexpr int CPP = 64 / SUB;     // chunks per pass
     // f16 activations on 16 columns, several passes per wave (deep K), up to four rows: the pipelined pass loop, and for
@@ -66,11 +79,14 @@ __device__ __forceinline__ void gemv4s_body(const char *__restrict__ cw, const v
 
     const uint32_t b = blockIdx.x;
     const uint32_t xcd = b & 7u, jj = b >> 3;
-    const uint32_t sp = jj % splits;
-    const uint32_t st = (jj / splits) * 8u + xcd;
+    // (unsplit, as the planner's sub-tile forms are: no division in front of the first loads)
+    const uint32_t sp = splits == 1 ? 0u : jj % splits, jt = splits == 1 ? jj : jj / splits;
+    // Workgroups reach the eight XCDs in turn by linear id.  Repacked copy: sub-tile = id (every block of the copy belongs
+    // to one workgroup).  The reference's arrays: neighbouring sub-tiles share the 128-byte lines of the scale rows (32 or
+    // 64 bytes per sub-tile and group), so each XCD takes a contiguous run of sub-tiles and the shared lines meet in its L2.
+    const uint32_t st = REFL ? xcd * ((sub_tiles + 7u) >> 3) + jt : jt * 8u + xcd;
     if (st >= sub_tiles) return;
 
-    const uint32_t waves = blockDim.x >> 6;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const uint32_t lane = threadIdx.x & 63u;
     const uint32_t cl = lane % SUB, cg = lane / SUB;          // column in the sub-tile, chunk of the pass
@@ -131,7 +147,7 @@ __device__ __forceinline__ void gemv4s_body(const char *__restrict__ cw, const v
     for (int r = 0; r < RL; r++) red[(wave * RL + r) * 64 + lane] = acc[r];
     __syncthreads();
 
-    const uint32_t threads = blockDim.x;
+    const uint32_t threads = waves * 64u;
     const uint32_t entries = RL * SUB;  // entry e = r * SUB + column
     const uint32_t pair_entries = RL * (SUB / 2), ffn = n >> 1;  // gated: entry e = r * SUB/2 + feature
     auto summed = [&](uint32_t r, uint32_t c) {
@@ -192,19 +208,22 @@ __device__ __forceinline__ void gemv4s_body(const char *__restrict__ cw, const v
     if (threadIdx.x == 0) __hip_atomic_store(&counters[st], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-// Argument order: what the address arithmetic of the first loads needs comes first, sixteen 32-bit words in all, which
-// the build has the hardware preload into scalar registers at wave start (-amdgpu-kernarg-preload-count); the output
-// description, a few hundred bytes that only the store needs, comes last.  A wave that has to fetch its arguments first
-// starts its weight loads one memory round trip later, and with one workgroup per CU nothing hides that.
+// Argument order: what the address arithmetic of the first loads needs comes first, thirteen 32-bit words in all, which
+// the build has the hardware preload into scalar registers at wave start (-amdgpu-kernarg-preload-count; thirteen is what
+// the user scalar registers hold beside the argument pointer); the scratch pointers and the output description, a few
+// hundred bytes that only the store needs, come last.  A wave that has to fetch an argument first starts its weight loads
+// one round trip to the scalar cache later, and with one workgroup per CU nothing hides that -- hence also the packed
+// word `cfg` (gemv4s_cfg: split factor, gated store, waves per workgroup, rows), which keeps the workgroup size out of
+// the dispatch packet's hidden arguments, where a read of blockDim would fetch it from.
 template <int SUB, int RL, bool AF32, bool ONE, bool REFL = false>
-__global__ __launch_bounds__(1024) void k_gemv4s(const char *__restrict__ cw, const void *__restrict__ a_any, uint32_t m_rows,
-                                                  uint32_t k, uint32_t n, uint32_t n_pad, uint32_t k_chunks,
-                                                  uint32_t sub_tiles, uint32_t splits, uint32_t cps, uint32_t gated_store,
-                                                  const uint16_t *__restrict__ ref_scales, float *__restrict__ ws,
-                                                  unsigned *__restrict__ counters, OutSpec out)
+__global__ __launch_bounds__(1024) void k_gemv4s(const char *__restrict__ cw, const void *__restrict__ a_any,
+                                                  const uint16_t *__restrict__ ref_scales, uint32_t cfg, uint32_t k,
+                                                  uint32_t k_chunks, uint32_t sub_tiles, uint32_t cps, uint32_t n,
+                                                  uint32_t n_pad, float *__restrict__ ws, unsigned *__restrict__ counters,
+                                                  OutSpec out)
 {
-    gemv4s_body<SUB, RL, AF32, ONE, REFL>(cw, a_any, out, ws, counters, m_rows, k, n, n_pad, k_chunks, sub_tiles, splits, cps,
-                                          gated_store != 0, ref_scales, nullptr);
+    gemv4s_body<SUB, RL, AF32, ONE, REFL>(cw, a_any, out, ws, counters, cfg, k, n, n_pad, k_chunks, sub_tiles, cps, ref_scales,
+                                          nullptr);
 }
 
 // The same kernel with a trace (twm_debug_trace; one row of f16 activations only): workgroup b writes four words at
@@ -225,8 +244,8 @@ __global__ __launch_bounds__(1024) void k_gemv4s_traced(const char *__restrict__
         // HW_ID (register 4): wave, SIMD, CU, SH, SE ids; XCC_ID (register 20): the XCD
         tr[3] = (__builtin_amdgcn_s_getreg((31 << 11) | 4) & 0xFFFFu) | (__builtin_amdgcn_s_getreg((3 << 11) | 20) << 16);
     }
-    gemv4s_body<SUB, 1, false, ONE, false>(cw, a_any, out, ws, counters, m_rows, k, n, n_pad, k_chunks, sub_tiles, splits, cps,
-                                           out.swiglu != nullptr, nullptr, tr + 1);
+    gemv4s_body<SUB, 1, false, ONE, false>(cw, a_any, out, ws, counters, gemv4s_cfg(splits, out.swiglu != nullptr, blockDim.x >> 6, m_rows),
+                                           k, n, n_pad, k_chunks, sub_tiles, cps, nullptr, tr + 1);
     if (threadIdx.x == 0) tr[2] = (uint32_t)__builtin_amdgcn_s_memrealtime();
 }
 
@@ -236,15 +255,16 @@ static hipError_t launch_gemv4s_t(hipStream_t s, const WeightView &w, const void
 {
     uint32_t n_pad = w.n_tiles * kTileN;  // whole 64-column tiles
     uint32_t sub_tiles = n_pad / SUB;
+    if (splits > 4095) splits = 4095;
     uint32_t cps = (w.k_chunks + splits - 1) / splits;
     splits = (w.k_chunks + cps - 1) / cps;
     uint32_t blocks = ((sub_tiles + 7) / 8) * 8 * splits;
     size_t lds = (size_t)waves * RL * 64 * sizeof(float);
     const bool one = (cps + 64 / SUB - 1) / (64 / SUB) <= waves;
 #define TWM_S_LAUNCH(AF, ONEV)                                                                                          \
-    hipLaunchKernelGGL((k_gemv4s<SUB, RL, AF, ONEV>), dim3(blocks), dim3(waves * 64), lds, s, (const char *)w.cq, a, m, w.k, \
-                       w.n, n_pad, w.k_chunks, sub_tiles, splits, cps, out.swiglu ? 1u : 0u, (const uint16_t *)nullptr, ws,  \
-                       counters, out)
+    hipLaunchKernelGGL((k_gemv4s<SUB, RL, AF, ONEV>), dim3(blocks), dim3(waves * 64), lds, s, (const char *)w.cq, a,         \
+                       (const uint16_t *)nullptr, gemv4s_cfg(splits, out.swiglu != nullptr, waves, m), w.k, w.k_chunks,       \
+                       sub_tiles, cps, w.n, n_pad, ws, counters, out)
     if constexpr (RL == 1) {
         if (!a_f32 && g_trace.ptr && blocks <= g_trace.capacity) {
             if (one)
@@ -305,6 +325,7 @@ hipError_t launch_gemv4s_ref(hipStream_t s, const uint8_t *packed, const uint16_
     if (waves < 1 || waves > 16 || (sub != 32 && sub != 16)) return hipErrorInvalidValue;
     const uint32_t n_pad = ((n + 63) / 64) * 64, sub_tiles = n_pad / sub;
     const uint32_t k_chunks = (k / 32 + 3) / 4;
+    if (splits > 4095) splits = 4095;
     const uint32_t cps = (k_chunks + splits - 1) / splits;
     splits = (k_chunks + cps - 1) / cps;
     const uint32_t blocks = ((sub_tiles + 7) / 8) * 8 * splits;
@@ -318,7 +339,8 @@ hipError_t launch_gemv4s_ref(hipStream_t s, const uint8_t *packed, const uint16_
     out.seg[0].width = n;
 #define TWM_S_REF(SUBV, ONEV)                                                                                          \
     hipLaunchKernelGGL((k_gemv4s<SUBV, 1, true, ONEV, true>), dim3(blocks), dim3(waves * 64), lds, s, (const char *)packed, \
-                       (const void *)a, 1u, k, n, n_pad, k_chunks, sub_tiles, splits, cps, 0u, scales, ws, counters, out)
+                       (const void *)a, scales, gemv4s_cfg(splits, false, waves, 1u), k, k_chunks, sub_tiles, cps, n, n_pad, ws,  \
+                       counters, out)
     if (sub == 32) {
         if (one) TWM_S_REF(32, true);
         else TWM_S_REF(32, false);
