@@ -11,7 +11,7 @@ SOURCES = ["twm_kernels.hip", "twm_gemv4.hip", "twm_gemv4s.hip", "twm_moe.hip", 
            "twm_api_weights.hip", "twm_api_gemm.hip", "twm_api_moe.hip"]
 # The batched-decode kernels read every MFMA result with vector instructions right away (scale, add):
 # with the default choice the results land in AGPRs and each costs a v_accvgpr_read first.
-# The decode kernels' first sixteen argument words arrive preloaded in scalar registers (see k_gemv4s).
+# The decode kernels' first argument words (thirteen fit the user scalar registers) arrive preloaded (see k_gemv4s).
 PRELOAD = ["-mllvm", "-amdgpu-kernarg-preload-count=16"]
 PER_FILE_FLAGS = {"twm_gemv4s.hip": PRELOAD, "twm_gemv4.hip": PRELOAD, "twm_moe.hip": PRELOAD, "twm_stream.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"] + PRELOAD,
                   "twm_batch.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"] + PRELOAD}
