@@ -190,7 +190,10 @@ __global__ __launch_bounds__(1024) void k_raw_gemv(RawSlab e, const float *__res
     constexpr int CPP = 64 / SUB;
     constexpr int TERMS = kTermsOneRowF32;
     extern __shared__ float red[];  // [waves][64]
-    const uint32_t st = blockIdx.x, slot = blockIdx.y;
+    // gridDim.x is a multiple of 8 and workgroups reach the eight XCDs in turn: each XCD takes a contiguous run of
+    // sub-tiles, so that the 128-byte lines of the scale rows, which neighbouring sub-tiles share, meet in one L2
+    const uint32_t st = (blockIdx.x & 7u) * (gridDim.x >> 3) + (blockIdx.x >> 3), slot = blockIdx.y;
+    if (st * SUB >= n) return;
     const uint32_t waves = blockDim.x >> 6;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const uint32_t lane = threadIdx.x & 63u, cl = lane % SUB, cg = lane / SUB;
@@ -239,7 +242,8 @@ __global__ __launch_bounds__(1024) void k_raw_down_axpy(RawSlab e, const float *
     constexpr int CPP = 64 / SUB;
     constexpr int TERMS = kTermsOneRowF32;
     extern __shared__ float red[];  // [slots * wps][64]
-    const uint32_t st = blockIdx.x;
+    const uint32_t st = (blockIdx.x & 7u) * (gridDim.x >> 3) + (blockIdx.x >> 3);  // (a contiguous run per XCD, as in k_raw_gemv)
+    if (st * SUB >= n) return;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const uint32_t lane = threadIdx.x & 63u, cl = lane % SUB, cg = lane / SUB;
     const uint32_t slot = wave / wps, j = wave % wps;
@@ -402,7 +406,7 @@ hipError_t launch_raw_gemv(hipStream_t s, const RawView &v, const float *a, uint
     uint32_t waves = passes < 16 ? passes : 16;
     if (force_waves >= 1 && force_waves <= 16) waves = (uint32_t)force_waves;
     const bool one = passes <= waves;
-    dim3 grid(sub_tiles, slots), block(waves * 64);
+    dim3 grid(((sub_tiles + 7) / 8) * 8, slots), block(waves * 64);  // (whole rounds of the eight XCDs: see k_raw_gemv)
     const size_t lds = (size_t)waves * 64 * sizeof(float);
     const RawSlab e = raw_slab(v);
 #define TWM_RAW_LAUNCH(SUBV, ONEV) \
@@ -438,7 +442,7 @@ hipError_t launch_raw_down_axpy(hipStream_t s, const RawView &v, const float *a_
         const uint32_t waves = now * wps;
         const size_t lds = (size_t)waves * 64 * sizeof(float);
 #define TWM_RAW_DOWN(SUBV, ONEV)                                                                                           \
-    hipLaunchKernelGGL((k_raw_down_axpy<SUBV, ONEV>), dim3(sub_tiles), dim3(waves * 64), lds, s, e, a_all + (size_t)s0 * v.k, \
+    hipLaunchKernelGGL((k_raw_down_axpy<SUBV, ONEV>), dim3(((sub_tiles + 7) / 8) * 8), dim3(waves * 64), lds, s, e, a_all + (size_t)s0 * v.k, \
                        ids + s0, weights + s0, accum, v.k, v.n, k_chunks, now, wps)
         if (sub == 16) {
             if (one) TWM_RAW_DOWN(16, true);
