@@ -547,13 +547,19 @@ extern "C++" int twm::m1_dispatch(const M1Env &env, const char *who, const float
     // 14336 -> 4096 9.7) and, eight waves of one pass each, on wide matrices up to K = 4096 (3584 -> 37888 16.3 against
     // 18.1 us on 32 columns, 4096 -> 22016 11.8 against 12.5, 4096 -> 28672 14.6 against 15.8); in between sixteen waves
     // on 32 columns as long as every wave gets a single pass (3584 -> 4608 4.7 against 4.9, 4096 -> 6144 5.1 against
-    // 5.5).  Deeper wide matrices keep the 64-column kernel and its split-K (8192 -> 57344: 46.6 against 63.7 us).
+    // 5.5).  Deeper matrices of 256 tiles or more keep the 64-column kernel and its split-K (8192 -> 57344: 46.6 against
+    // 63.7 us).
     // Fitted to sweeps over the Qwen2.5-7B, Llama-2-7B, Llama-3-8B, 13B and 70B projections; option "sub" = 1 keeps the
     // 64-column kernel.
     const uint32_t tiles64 = n_pad / 64, passes16 = (k_chunks + 3) / 4, passes32 = (k_chunks + 1) / 2;
     const bool narrow16 = tiles64 <= 64, wide16 = tiles64 >= 256 && passes16 <= 8;
     uint32_t sub = narrow16 || wide16 ? 16 : 32, sub_waves = (sub == 16 && passes16 <= 8) ? 8 : 16;
-    bool use_sub = env.force_sub != 1 && (sub == 16 || passes32 <= 16);
+    // 65 .. 255 tiles on a deeper K: still 32 columns, the waves looping over their passes -- sixteen of them up to 128
+    // tiles and 160 chunks, eight beyond (13824 -> 5120 12.2 against 14.6 us on whole tiles with a K-split, 8192 -> 8192
+    // 9.4 / 12.4, 18944 -> 4608 15.3 / 17.1, 28672 -> 8192 24.2 / 27.5, 8192 -> 10240 14.2 / 15.1, 5120 -> 15360 10.5 / 11.0)
+    const bool mid32 = !narrow16 && tiles64 < 256 && passes32 > 16;
+    if (mid32 && !(tiles64 <= 128 && k_chunks <= 160)) sub_waves = 8;
+    bool use_sub = env.force_sub != 1 && (sub == 16 || passes32 <= 16 || mid32);
     if (env.force_sub >= 16) {
         sub = (uint32_t)env.force_sub;
         sub_waves = 8;

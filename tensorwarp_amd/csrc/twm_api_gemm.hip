@@ -79,7 +79,12 @@ static SubPlan plan_gemv4_sub(uint32_t tiles64, uint32_t k_chunks, uint32_t m, b
     // very deep K, three or four rows: with f32 rows the 64-column split-K plan is level or ahead; with f16 rows the
     // pipelined pass loop is (18944 -> 3584 at M = 3 / 4: 9.96 / 10.75 against 11.75 / 11.84 us)
     if (m > 2 && passes16 > 32 && a_f32) return none;
-    if (tiles64 > 64) return SubPlan{32, 16};  // 16 columns would leave a second, quarter-full round of workgroups
+    // 65 .. 128 tiles: 16 columns would leave a second, part-full round of workgroups, and 32 columns on sixteen waves are
+    // ahead -- except for one row on a deep K, where eight waves in the pipelined pass loop on 16 columns win (13824 ->
+    // 5120: 10.6 against 11.2 us with f16, 11.5 against 12.4 with f32 activations; 14336 -> 6144 11.2 / 11.9; 18944 -> 4608
+    // 13.2 / 13.8; 13824 -> 7168 11.4 / 12.6; two rows level, four rows 32 columns again: 14.6 against 12.2)
+    if (tiles64 > 64 && m == 1 && passes16 > 16) return SubPlan{16, 8};
+    if (tiles64 > 64) return SubPlan{32, 16};
     return narrow16;
 }
 
