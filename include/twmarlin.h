@@ -409,6 +409,11 @@ uint32_t twm_pick_splits(uint32_t k, uint32_t n, uint32_t m);
  * see what the planners decide -- the counterpart of AutoTuner::heuristic_variant and ::report
  * (crates/kernels/src/autotune.rs:505-515, 648-668) -- and to test them without a GPU. */
 int twm_plan_describe(const twm_ctx *ctx, uint32_t k, uint32_t n, uint32_t m, int a_dtype, int gated, char *text, size_t bytes);
+/* The same for twm_gemm_tw_marlin_m1 on the reference's arrays (16-byte aligned activations and records assumed; others
+ * run the reference-order kernel): which kernel reads them, with how many columns and waves per workgroup and which
+ * K-split.  The reference's own choice for this call is pick_splits (quantize.rs:1317-1325), mirrored by
+ * twm_pick_splits_reference. */
+int twm_plan_describe_m1(const twm_ctx *ctx, uint32_t k, uint32_t n, char *text, size_t bytes);
 
 /* ---- graph capture / replay (GraphCapture::{record_with_device, replay}, cuda_graph.rs:85-117) */
 

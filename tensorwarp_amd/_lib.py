@@ -83,6 +83,7 @@ SIGNATURES = {
     "twm_bank_down_axpy": (_int, [_vp, _vp, _vp, _int, _vp, _vp, _u32, _vp]),
     "twm_geglu_rows": (_int, [_vp, _vp, _u32, _u32, _int, _vp]),
     "twm_plan_describe": (_int, [_vp, _u32, _u32, _u32, _int, _int, _vp, _sz]),
+    "twm_plan_describe_m1": (_int, [_vp, _u32, _u32, _vp, _sz]),
     "twm_batched_marlin_gate_up": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _u32, _u32, _u32, _u32, _u32]),
     "twm_batched_marlin_down_axpy": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _u32, _u32, _u32, _u32, _u32]),
     "twm_batched_marlin_split_geglu": (_int, [_vp, _vp, _vp, _u32, _u32]),

@@ -519,28 +519,22 @@ void twm_pick_splits_reference(uint32_t k, uint32_t n, uint32_t *n_blocks, uint3
     if (groups_per_split) *groups_per_split = (groups + sp - 1u) / sp;
 }
 
-extern "C++" int twm::m1_dispatch(const M1Env &env, const char *who, const float *a_dev, const uint8_t *packed_dev,
-                       const uint16_t *scales_dev, float *c_dev, uint32_t n, uint32_t k)
+// The launch form of the GEMV on the reference's arrays: chosen here, launched by m1_dispatch, described by
+// twm_plan_describe_m1.  Nothing here touches the device.
+enum M1Kind { kM1RefOrder = 0, kM1SubTile = 1, kM1WholeTile = 2 };
+struct M1Form {
+    int kind;
+    uint32_t sub, waves, splits;  // sub-tile width (sub-tile form), waves per workgroup, K-splits over workgroups
+};
+// aligned16: activations and packed records at 16-byte addresses (the MFMA kernels' loads); ws_bytes / n_counters: the
+// split-K scratch at hand
+static M1Form choose_m1_form(int exact, int force_sub, int force_waves, int force_splits, size_t ws_bytes, uint32_t n_counters,
+                             bool aligned16, uint32_t n, uint32_t k)
 {
-    if (int rc = check_kn(who, k, n)) return rc;
-    if (n == 0) return TWM_OK;
-    if (!c_dev) return api_fail(TWM_INVALID_HANDLE, "%s: null output", who);
-    if (k == 0) {
-        HIP_TRY(launch_fill_zero(env.stream, c_dev, (size_t)n * 4), TWM_DEVICE_ERROR, "fill kernel launch");
-        return TWM_OK;
-    }
-    if (!a_dev || !packed_dev || !scales_dev) return api_fail(TWM_INVALID_HANDLE, "%s: null input", who);
-    // the reference kernel reads a record as four 32-bit words (quantize.rs:1227-1228): 4-byte alignment is its own limit
-    if (((uintptr_t)packed_dev & 3) != 0) return api_fail(TWM_SHAPE_ERROR, "%s: packed must be 4-byte aligned", who);
-    if (env.exact || ((uintptr_t)a_dev & 15) != 0 || ((uintptr_t)packed_dev & 15) != 0) {
-        // f32 activations, f32 FMAs, the reference kernel's order and its own split-K rule (float atomics)
-        uint32_t nb, sp, gps;
-        twm_pick_splits_reference(k, n, &nb, &sp, &gps);
-        HIP_TRY(launch_ref_gemv(env.stream, a_dev, packed_dev, scales_dev, c_dev, n, k, sp, gps), TWM_DEVICE_ERROR, "gemv launch");
-        return TWM_OK;
-    }
+    M1Form f = {kM1RefOrder, 0, 0, 1};
+    if (exact || !aligned16) return f;  // f32 activations, f32 FMAs, the reference kernel's order and its own split-K rule
     // the M <= 4 MFMA kernels reading the reference's arrays as they are (f32 activations as two f16 terms)
-    uint32_t n_pad = ((n + 63) / 64) * 64, k_chunks = (k / 32 + kChunkGroups - 1) / kChunkGroups;
+    const uint32_t n_pad = ((n + 63) / 64) * 64, k_chunks = (k / 32 + kChunkGroups - 1) / kChunkGroups;
     // On the reference's arrays a wave's four group rows of a chunk are N x 16 bytes apart, and many waves in flight
     // with one pass each pay better than on the contiguous copy.  The sub-tile kernel on 16 columns when 64-column tiles
     // number no more than 64 (any K: deeper ones in the pipelined pass loop on sixteen waves: 18944 -> 3584 10.8 us,
@@ -559,43 +553,98 @@ extern "C++" int twm::m1_dispatch(const M1Env &env, const char *who, const float
     // 9.4 / 12.4, 18944 -> 4608 15.3 / 17.1, 28672 -> 8192 24.2 / 27.5, 8192 -> 10240 14.2 / 15.1, 5120 -> 15360 10.5 / 11.0)
     const bool mid32 = !narrow16 && tiles64 < 256 && passes32 > 16;
     if (mid32 && !(tiles64 <= 128 && k_chunks <= 160)) sub_waves = 8;
-    bool use_sub = env.force_sub != 1 && (sub == 16 || passes32 <= 16 || mid32);
-    if (env.force_sub >= 16) {
-        sub = (uint32_t)env.force_sub;
+    bool use_sub = force_sub != 1 && (sub == 16 || passes32 <= 16 || mid32);
+    if (force_sub >= 16) {
+        sub = (uint32_t)force_sub;
         sub_waves = 8;
         use_sub = true;
     }
     if (use_sub) {
-        uint32_t sp = env.splits ? (uint32_t)env.splits : 1;
-        if (env.force_waves) sub_waves = (uint32_t)env.force_waves;
+        uint32_t sp = force_splits ? (uint32_t)force_splits : 1;
+        if (force_waves) sub_waves = (uint32_t)force_waves;
         if (sp > k_chunks) sp = k_chunks;
-        while (sp > 1 && (size_t)sp * n_pad * 4 > env.ws_bytes) sp--;
-        if (n_pad / sub > env.n_counters) sp = 1;
-        if (sp > 1 && env.clear_counters)
-            HIP_TRY(launch_fill_zero(env.stream, env.counters, (size_t)(n_pad / sub) * 4), TWM_DEVICE_ERROR, "fill kernel launch");
-        HIP_TRY(launch_gemv4s_ref(env.stream, packed_dev, scales_dev, k, n, a_dev, c_dev, env.ws, env.counters, sub, sub_waves, sp),
-                TWM_DEVICE_ERROR, "sub-tile gemv launch");
+        while (sp > 1 && (size_t)sp * n_pad * 4 > ws_bytes) sp--;
+        if (n_pad / sub > n_counters) sp = 1;
+        return M1Form{kM1SubTile, sub, sub_waves, sp};
+    }
+    f.kind = kM1WholeTile;
+    f.waves = 8;
+    if (tiles64 < 256) {
+        f.waves = 16;
+        while (tiles64 * f.splits * 2 <= 256 && k_chunks >= f.splits * 2 * 8) f.splits *= 2;
+    }
+    if (force_waves) f.waves = (uint32_t)force_waves;
+    if (force_splits) f.splits = (uint32_t)force_splits;
+    if (f.splits > k_chunks) f.splits = k_chunks;
+    while (f.splits > 1 && (size_t)f.splits * n_pad * 4 > ws_bytes) f.splits--;
+    if (tiles64 > n_counters) f.splits = 1;
+    return f;
+}
+
+extern "C++" int twm::m1_dispatch(const M1Env &env, const char *who, const float *a_dev, const uint8_t *packed_dev,
+                       const uint16_t *scales_dev, float *c_dev, uint32_t n, uint32_t k)
+{
+    if (int rc = check_kn(who, k, n)) return rc;
+    if (n == 0) return TWM_OK;
+    if (!c_dev) return api_fail(TWM_INVALID_HANDLE, "%s: null output", who);
+    if (k == 0) {
+        HIP_TRY(launch_fill_zero(env.stream, c_dev, (size_t)n * 4), TWM_DEVICE_ERROR, "fill kernel launch");
         return TWM_OK;
     }
-    DecodePlan plan;
-    plan.lane_col = 1;
-    plan.nt = 1;
-    plan.waves = 8;
-    plan.splits = 1;
-    if (tiles64 < 256) {
-        plan.waves = 16;
-        while (tiles64 * plan.splits * 2 <= 256 && k_chunks >= plan.splits * 2 * 8) plan.splits *= 2;
+    if (!a_dev || !packed_dev || !scales_dev) return api_fail(TWM_INVALID_HANDLE, "%s: null input", who);
+    // the reference kernel reads a record as four 32-bit words (quantize.rs:1227-1228): 4-byte alignment is its own limit
+    if (((uintptr_t)packed_dev & 3) != 0) return api_fail(TWM_SHAPE_ERROR, "%s: packed must be 4-byte aligned", who);
+    const bool aligned16 = ((uintptr_t)a_dev & 15) == 0 && ((uintptr_t)packed_dev & 15) == 0;
+    const M1Form f = choose_m1_form(env.exact, env.force_sub, env.force_waves, env.splits, env.ws_bytes, env.n_counters, aligned16, n, k);
+    const uint32_t n_pad = ((n + 63) / 64) * 64;
+    switch (f.kind) {
+    case kM1RefOrder: {
+        uint32_t nb, sp, gps;
+        twm_pick_splits_reference(k, n, &nb, &sp, &gps);
+        HIP_TRY(launch_ref_gemv(env.stream, a_dev, packed_dev, scales_dev, c_dev, n, k, sp, gps), TWM_DEVICE_ERROR, "gemv launch");
+        return TWM_OK;
     }
-    if (env.force_waves) plan.waves = (uint32_t)env.force_waves;
-    if (env.splits) plan.splits = (uint32_t)env.splits;
-    if (plan.splits > k_chunks) plan.splits = k_chunks;
-    while (plan.splits > 1 && (size_t)plan.splits * n_pad * 4 > env.ws_bytes) plan.splits--;
-    if (tiles64 > env.n_counters) plan.splits = 1;
-    if (plan.splits > 1 && env.clear_counters)
-        HIP_TRY(launch_fill_zero(env.stream, env.counters, (size_t)tiles64 * 4), TWM_DEVICE_ERROR, "fill kernel launch");
-    HIP_TRY(launch_gemv4_ref(env.stream, packed_dev, scales_dev, k, n, a_dev, c_dev, env.ws, env.counters, plan.waves,
-                             plan.splits),
-            TWM_DEVICE_ERROR, "gemv launch");
+    case kM1SubTile:
+        if (f.splits > 1 && env.clear_counters)
+            HIP_TRY(launch_fill_zero(env.stream, env.counters, (size_t)(n_pad / f.sub) * 4), TWM_DEVICE_ERROR, "fill kernel launch");
+        HIP_TRY(launch_gemv4s_ref(env.stream, packed_dev, scales_dev, k, n, a_dev, c_dev, env.ws, env.counters, f.sub, f.waves, f.splits),
+                TWM_DEVICE_ERROR, "sub-tile gemv launch");
+        return TWM_OK;
+    default:
+        if (f.splits > 1 && env.clear_counters)
+            HIP_TRY(launch_fill_zero(env.stream, env.counters, (size_t)(n_pad / 64) * 4), TWM_DEVICE_ERROR, "fill kernel launch");
+        HIP_TRY(launch_gemv4_ref(env.stream, packed_dev, scales_dev, k, n, a_dev, c_dev, env.ws, env.counters, f.waves, f.splits),
+                TWM_DEVICE_ERROR, "gemv launch");
+        return TWM_OK;
+    }
+}
+
+int twm_plan_describe_m1(const twm_ctx *ctx, uint32_t k, uint32_t n, char *text, size_t bytes)
+{
+    if (!text || bytes == 0) return api_fail(TWM_INVALID_HANDLE, "twm_plan_describe_m1: null buffer");
+    if (int rc = check_kn("twm_plan_describe_m1", k, n)) return rc;
+    if (n == 0 || k == 0) {
+        snprintf(text, bytes, n == 0 ? "nothing to launch" : "k_fill_zero");
+        return TWM_OK;
+    }
+    const M1Form f = ctx ? choose_m1_form(ctx->m1_exact, ctx->force_sub, ctx->force_waves, ctx->m1_splits, ctx->ws_bytes, ctx->n_counters, true, n, k)
+                         : choose_m1_form(0, 0, 0, 0, kWsBytes, kCounters, true, n, k);
+    switch (f.kind) {
+    case kM1RefOrder: {
+        uint32_t nb, sp, gps;
+        twm_pick_splits_reference(k, n, &nb, &sp, &gps);
+        snprintf(text, bytes, "k_ref_gemv: one thread per column, %u K-split%s (the reference's rule); reference arrays", sp, sp == 1 ? "" : "s");
+        break;
+    }
+    case kM1SubTile:
+        snprintf(text, bytes, "k_gemv4s: %u-column sub-tiles, %u waves, %u K-split%s; reference arrays", f.sub, f.waves, f.splits,
+                 f.splits == 1 ? "" : "s");
+        break;
+    default:
+        snprintf(text, bytes, "k_gemv4: 1 x 64-column tiles per workgroup, %u waves, %u K-split%s; reference arrays", f.waves, f.splits,
+                 f.splits == 1 ? "" : "s");
+        break;
+    }
     return TWM_OK;
 }
 

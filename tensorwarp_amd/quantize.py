@@ -68,6 +68,12 @@ class WarpDevice:
         _check(self._l.twm_plan_describe(self.handle, k, n, m, _lib.F32 if dtype == "f32" else _lib.F16, int(gated), buf, 256))
         return buf.value.decode()
 
+    def plan_m1(self, k, n):
+        """What gemm_tw_marlin_m1() would launch on the reference's K x N arrays under this context's options."""
+        buf = C.create_string_buffer(256)
+        _check(self._l.twm_plan_describe_m1(self.handle, k, n, buf, 256))
+        return buf.value.decode()
+
     # timing
     def event(self):
         ev = self._l.twm_event_create(self.handle)

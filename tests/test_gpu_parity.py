@@ -1506,6 +1506,20 @@ def test_plan_description_follows_the_context_options(dev):
     assert dev.plan(k, n, 16).startswith("k_gemv4s:")
     assert dev.plan(3584, 37888, 1, gated=True).startswith("k_gemv4s: 32-column sub-tiles")
     assert dev.plan(18944, 3584, 1, dtype="f32") == "k_gemv4s: 16-column sub-tiles, 4 waves, 1 K-split; column-lane copy"
+    # the drop-in on the reference's arrays: its own planner and options
+    assert dev.plan_m1(3584, 37888) == "k_gemv4s: 16-column sub-tiles, 8 waves, 1 K-split; reference arrays"
+    dev.set_option("m1_exact", 1)
+    try:
+        assert dev.plan_m1(3584, 37888).startswith("k_ref_gemv: one thread per column")
+    finally:
+        dev.set_option("m1_exact", 0)
+    dev.set_option("sub", 1)
+    dev.set_option("m1_splits", 2)
+    try:
+        assert dev.plan_m1(18944, 3584) == "k_gemv4: 1 x 64-column tiles per workgroup, 16 waves, 2 K-splits; reference arrays"
+    finally:
+        dev.set_option("sub", 0)
+        dev.set_option("m1_splits", 0)
 
 
 def test_fusing_handles_equals_fusing_the_arrays(dev):

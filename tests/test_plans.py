@@ -100,3 +100,54 @@ def test_describe_rejects_what_twm_gemm_rejects(lib):
     assert lib.twm_plan_describe(None, 128, 64, 1, 7, 0, buf, 64) == _lib.UNSUPPORTED_OP           # dtype
     assert lib.twm_plan_describe(None, 128, 64, 1, _lib.F16, 0, None, 0) == _lib.INVALID_HANDLE
     assert lib.twm_plan_describe(None, 128, 64, 0, _lib.F16, 0, buf, 64) == 0 and buf.value == b"nothing to launch"
+
+
+# ---------------------------------------------------------------- the drop-in on the reference's arrays
+
+def describe_m1(lib, k, n):
+    buf = ctypes.create_string_buffer(256)
+    rc = lib.twm_plan_describe_m1(None, k, n, buf, 256)
+    assert rc == 0, lib.twm_last_error().decode()
+    return buf.value.decode()
+
+
+@pytest.mark.parametrize("k,n,want", [
+    # the Qwen-7B layer: 32 columns x 16 waves of one pass on qkv, 16 columns elsewhere (one pass per wave on o and on
+    # the wide gate_up, the pass loop on sixteen waves on the deep down)
+    (3584, 4608, "k_gemv4s: 32-column sub-tiles, 16 waves, 1 K-split; reference arrays"),
+    (3584, 3584, "k_gemv4s: 16-column sub-tiles, 8 waves, 1 K-split; reference arrays"),
+    (3584, 37888, "k_gemv4s: 16-column sub-tiles, 8 waves, 1 K-split; reference arrays"),
+    (18944, 3584, "k_gemv4s: 16-column sub-tiles, 16 waves, 1 K-split; reference arrays"),
+    # 65 .. 255 tiles on a deeper K: 32 columns, waves looping; sixteen up to 128 tiles and 160 chunks, else eight
+    (13824, 5120, "k_gemv4s: 32-column sub-tiles, 16 waves, 1 K-split; reference arrays"),
+    (28672, 8192, "k_gemv4s: 32-column sub-tiles, 8 waves, 1 K-split; reference arrays"),
+    (8192, 10240, "k_gemv4s: 32-column sub-tiles, 8 waves, 1 K-split; reference arrays"),
+    # 256 tiles or more beyond K = 4096: whole 64-column tiles
+    (8192, 57344, "k_gemv4: 1 x 64-column tiles per workgroup, 8 waves, 1 K-split; reference arrays"),
+    # the LM head
+    (3584, 152064, "k_gemv4s: 16-column sub-tiles, 8 waves, 1 K-split; reference arrays"),
+])
+def test_known_drop_in_plans(lib, k, n, want):
+    assert describe_m1(lib, k, n) == want
+
+
+def test_drop_in_plan_invariants(lib):
+    for k in (32, 64, 896, 2048, 3584, 4096, 5120, 8192, 11008, 18944, 28672):
+        for n in (8, 64, 300, 1152, 4096, 4608, 6144, 8192, 16384, 22016, 57344):
+            text = describe_m1(lib, k, n)
+            kernel = text.split(":")[0]
+            assert kernel in ("k_gemv4s", "k_gemv4"), text
+            waves = int(re.search(r"(\d+) waves", text).group(1))
+            splits = int(re.search(r"(\d+) K-split", text).group(1))
+            k_chunks = (k // 32 + 3) // 4
+            assert 1 <= waves <= 16 and 1 <= splits <= k_chunks, (k, n, text)
+            if kernel == "k_gemv4s":
+                assert int(re.search(r"(\d+)-column sub-tiles", text).group(1)) in (16, 32)
+
+
+def test_describe_m1_edges(lib):
+    buf = ctypes.create_string_buffer(64)
+    assert lib.twm_plan_describe_m1(None, 100, 64, buf, 64) == _lib.SHAPE_ERROR      # K % 32, as the call itself
+    assert lib.twm_plan_describe_m1(None, 128, 64, None, 0) == _lib.INVALID_HANDLE
+    assert lib.twm_plan_describe_m1(None, 128, 0, buf, 64) == 0 and buf.value == b"nothing to launch"
+    assert lib.twm_plan_describe_m1(None, 0, 64, buf, 64) == 0 and buf.value == b"k_fill_zero"
