@@ -54,7 +54,10 @@ static SubPlan plan_gemv4_sub(uint32_t tiles64, uint32_t k_chunks, uint32_t m, b
     // on eight waves for one row and on four from two rows on (18944 -> 3584: M = 1 8.96 / 9.01 / 9.05 us on 8 / 4 / 16
     // waves, M = 2 9.5 / 9.2 / 9.7, M = 4 11.2 / 10.75 / 11.75)
     // (one row of f32 activations, which a lane takes as one shared piece: 9.3 / 9.6 us on 4 / 8 waves)
-    const SubPlan narrow16 = {16, passes16 <= 8 ? 8u : passes16 <= 16 ? 16u : ((m >= 2 && !a_f32) || (m == 1 && a_f32)) ? 4u : 8u};
+    // (one f16 row after the kernel's arguments all came preloaded: four waves ahead from 28 passes on -- 18944 -> 3584
+    // 8.58 against 8.74 us on eight, 14336 -> 4096 7.48 / 7.64 -- and level or behind below: 11008 -> 4096 6.60 / 6.62,
+    // 11008 -> 2048 5.75 / 5.63, 8960 -> 1536 5.01 / 4.87)
+    const SubPlan narrow16 = {16, passes16 <= 8 ? 8u : passes16 <= 16 ? 16u : ((m >= 2 && !a_f32) || (m == 1 && (a_f32 || passes16 >= 28))) ? 4u : 8u};
     if (tiles64 > 128) {
         // wide matrices: only the cheapest activations (f16, up to two rows) leave the sub-tiles ahead
         // (3584 -> 37888: 15.8 against 17.0 us at M = 1, 18.3 against 17.3 at M = 4, 19.9 against 17.9 with f32 rows)

@@ -31,7 +31,7 @@ QWEN7B = {"qkv": (3584, 4608), "o": (3584, 3584), "gate_up": (3584, 37888), "dow
     ("qkv", 1, "f16", "k_gemv4s: 32-column sub-tiles, 16 waves, 1 K-split; column-lane copy"),
     ("o", 1, "f16", "k_gemv4s: 16-column sub-tiles, 8 waves, 1 K-split; column-lane copy"),
     ("gate_up", 1, "f16", "k_gemv4s: 16-column sub-tiles, 7 waves, 1 K-split; column-lane copy"),
-    ("down", 1, "f16", "k_gemv4s: 16-column sub-tiles, 8 waves, 1 K-split; column-lane copy"),
+    ("down", 1, "f16", "k_gemv4s: 16-column sub-tiles, 4 waves, 1 K-split; column-lane copy"),
     # one row of f32 activations: the pass loop on four waves where K is deep or the matrix wide
     ("gate_up", 1, "f32", "k_gemv4s: 16-column sub-tiles, 4 waves, 1 K-split; column-lane copy"),
     ("down", 1, "f32", "k_gemv4s: 16-column sub-tiles, 4 waves, 1 K-split; column-lane copy"),
