@@ -27,11 +27,12 @@ namespace twm {
 namespace {
 
 // the launch's small numbers in one argument word: K-splits (bits 0-11; the launchers cap the factor at 4095), gated
-// store (12), waves per workgroup (13-17), rows (18-22)
-__host__ __device__ __forceinline__ uint32_t gemv4s_cfg(uint32_t splits, bool gated, uint32_t waves, uint32_t rows)
+// store (12), waves per workgroup (13-17), rows (18-22), a contiguous run of sub-tiles per XCD (23)
+__host__ __device__ __forceinline__ uint32_t gemv4s_cfg(uint32_t splits, bool gated, uint32_t waves, uint32_t rows, bool runs = false)
 {
-    return splits | (gated ? 0x1000u : 0u) | (waves << 13) | (rows << 18);
+    return splits | (gated ? 0x1000u : 0u) | (waves << 13) | (rows << 18) | (runs ? 0x800000u : 0u);
 }
+__device__ __forceinline__ bool cfg_runs(uint32_t cfg) { return (cfg & 0x800000u) != 0; }
 __device__ __forceinline__ uint32_t cfg_splits(uint32_t cfg) { return cfg & 0xFFFu; }
 __device__ __forceinline__ bool cfg_gated(uint32_t cfg) { return (cfg & 0x1000u) != 0; }
 __device__ __forceinline__ uint32_t cfg_waves(uint32_t cfg) { return (cfg >> 13) & 0x1Fu; }
@@ -84,7 +85,7 @@ __device__ __forceinline__ void gemv4s_body(const char *__restrict__ cw, const v
     // Workgroups reach the eight XCDs in turn by linear id.  Repacked copy: sub-tile = id (every block of the copy belongs
     // to one workgroup).  The reference's arrays: neighbouring sub-tiles share the 128-byte lines of the scale rows (32 or
     // 64 bytes per sub-tile and group), so each XCD takes a contiguous run of sub-tiles and the shared lines meet in its L2.
-    const uint32_t st = REFL ? xcd * ((sub_tiles + 7u) >> 3) + jt : jt * 8u + xcd;
+    const uint32_t st = (REFL || cfg_runs(cfg)) ? xcd * ((sub_tiles + 7u) >> 3) + jt : jt * 8u + xcd;
     if (st >= sub_tiles) return;
 
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -261,9 +262,10 @@ static hipError_t launch_gemv4s_t(hipStream_t s, const WeightView &w, const void
     uint32_t blocks = ((sub_tiles + 7) / 8) * 8 * splits;
     size_t lds = (size_t)waves * RL * 64 * sizeof(float);
     const bool one = (cps + 64 / SUB - 1) / (64 / SUB) <= waves;
+    const bool runs = blocks <= 512;  // few workgroups per CU: a contiguous run of sub-tiles per XCD
 #define TWM_S_LAUNCH(AF, ONEV)                                                                                          \
     hipLaunchKernelGGL((k_gemv4s<SUB, RL, AF, ONEV>), dim3(blocks), dim3(waves * 64), lds, s, (const char *)w.cq, a,         \
-                       (const uint16_t *)nullptr, gemv4s_cfg(splits, out.swiglu != nullptr, waves, m), w.k, w.k_chunks,       \
+                       (const uint16_t *)nullptr, gemv4s_cfg(splits, out.swiglu != nullptr, waves, m, runs), w.k, w.k_chunks, \
                        sub_tiles, cps, w.n, n_pad, ws, counters, out)
     if constexpr (RL == 1) {
         if (!a_f32 && g_trace.ptr && blocks <= g_trace.capacity) {
