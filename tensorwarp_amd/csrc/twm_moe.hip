@@ -45,7 +45,9 @@ __global__ __launch_bounds__(1024) void k_bank_gemv(const char *__restrict__ ban
     constexpr int CPP = 64 / SUB;
     constexpr int TERMS = AF32 ? kTermsOneRowF32 : kTermsOne;   // one row: f32 activations as two f16 terms of one shared piece per lane
     extern __shared__ float red[];  // [waves][64]
-    const uint32_t st = blockIdx.x, slot = blockIdx.y;
+    // (gridDim.x is a multiple of 8, workgroups reach the eight XCDs in turn: a contiguous run of sub-tiles per XCD, so
+    // that the sub-tiles of a 64-column tile, whose pieces interleave inside the copy's blocks, stream through one L2)
+    const uint32_t st = (blockIdx.x & 7u) * (gridDim.x >> 3) + (blockIdx.x >> 3), slot = blockIdx.y;
     if (st >= sub_tiles) return;
     const uint32_t waves = blockDim.x >> 6;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -105,7 +107,7 @@ __global__ __launch_bounds__(1024) void k_bank_down_axpy(const char *__restrict_
     constexpr int CPP = 64 / SUB;
     constexpr int TERMS = AF32 ? kTermsOneRowF32 : kTermsOne;
     extern __shared__ float red[];  // [slots * wps][64]
-    const uint32_t st = blockIdx.x;
+    const uint32_t st = (blockIdx.x & 7u) * (gridDim.x >> 3) + (blockIdx.x >> 3);  // (a contiguous run per XCD, as in k_bank_gemv)
     if (st >= sub_tiles) return;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const uint32_t lane = threadIdx.x & 63u, cl = lane % SUB, cg = lane / SUB;
@@ -329,7 +331,7 @@ hipError_t launch_bank_gemv(hipStream_t s, const BankView &b, const void *a, boo
     uint32_t waves = passes < 16 ? passes : 16;
     if (force_waves >= 1 && force_waves <= 16) waves = (uint32_t)force_waves;
     const bool one = passes <= waves;
-    dim3 grid(sub_tiles, slots), block(waves * 64);
+    dim3 grid(((sub_tiles + 7) / 8) * 8, slots), block(waves * 64);  // (whole rounds of the eight XCDs: see k_bank_gemv)
     size_t lds = (size_t)waves * 64 * sizeof(float);
 #define TWM_BANK_LAUNCH(SUBV, F32, A, ONEV)                                                                            \
     hipLaunchKernelGGL((k_bank_gemv<SUBV, F32, A, ONEV>), grid, block, lds, s, (const char *)b.cq, b.expert_bytes,      \
@@ -367,7 +369,7 @@ hipError_t launch_bank_down_axpy(hipStream_t s, const BankView &b, const void *a
     const uint32_t waves = slots * wps;
     size_t lds = (size_t)waves * 64 * sizeof(float);
 #define TWM_DOWN_LAUNCH(SUBV, F32, ONEV)                                                                               \
-    hipLaunchKernelGGL((k_bank_down_axpy<SUBV, F32, ONEV>), dim3(sub_tiles), dim3(waves * 64), lds, s, (const char *)b.cq, \
+    hipLaunchKernelGGL((k_bank_down_axpy<SUBV, F32, ONEV>), dim3(((sub_tiles + 7) / 8) * 8), dim3(waves * 64), lds, s, (const char *)b.cq, \
                        b.expert_bytes, b.experts, a_all, ids, weights, accum, b.k, b.n, b.k_chunks, sub_tiles, slots, wps)
 #define TWM_DOWN_ONE(SUBV, F32)                  \
     if (one) TWM_DOWN_LAUNCH(SUBV, F32, true);   \
