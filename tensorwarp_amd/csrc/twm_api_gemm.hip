@@ -72,6 +72,9 @@ static SubPlan plan_gemv4_sub(uint32_t tiles64, uint32_t k_chunks, uint32_t m, b
         // (several workgroups per CU: no idle eighth wave, 3584 -> 37888 at M = 1 14.8 against 15.3 us; with one workgroup
         // per CU the eight-wave form is the faster one, 3584 -> 3584 3.9 against 4.05)
         if (!a_f32 && m <= 2 && passes16 <= 8 && poor_fill) return SubPlan{16, passes16};
+        // (three and four rows: only where the last round is under 70 % full -- 4096 -> 22016, 67 %: 11.6 / 12.4 against
+        // 12.8 / 12.9 us on whole tiles; 3584 -> 37888, 77 %: 16.3 / 17.5 against 16.0 / 16.1)
+        if (!a_f32 && m <= 4 && passes16 <= 8 && tiles64 * 10 < rounds * 256 * 7) return SubPlan{16, passes16};
         // one row of f32 activations: the shared-piece form in the pipelined loop on four waves (3584 -> 37888: 15.75 us
         // against 17.0 with one pass per wave and 16.8 on whole tiles)
         if (a_f32 && m == 1 && passes16 <= 8 && poor_fill) return SubPlan{16, 4};
