@@ -362,7 +362,10 @@ def test_repack_is_lossless_at_7b_shape(dev):
 
 # ---------------------------------------------------------------- GEMV on the reference layout
 
-@pytest.mark.parametrize("k,n", [(64, 8), (128, 64), (896, 1152), (4096, 4096), (4864, 896), (3584, 300)])
+# (the last two: 65 .. 255 column tiles on a K past one pass per wave -- 32-column sub-tiles with sixteen, then eight
+# waves looping over their passes)
+@pytest.mark.parametrize("k,n", [(64, 8), (128, 64), (896, 1152), (4096, 4096), (4864, 896), (3584, 300), (4608, 4200),
+                                 (6144, 8300)])
 def test_gemm_tw_marlin_m1_reference_layout(dev, k, n):
     packed, scales, a16 = synth(k, n, 1, k + n)
     a = f16_as_f32(a16)
