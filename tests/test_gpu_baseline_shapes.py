@@ -167,6 +167,27 @@ def test_f32_rows_qwen7b_all_projections(dev, name):
     w.free()
 
 
+# ---------------------------------------------------------------- planner branches away from the benchmark shapes
+
+@pytest.mark.parametrize("k,n,ms,want", [
+    # 65 .. 128 column tiles on a deep K: one row runs 16-column sub-tiles in the pipelined pass loop (f16 and f32 rows)
+    (13824, 5120, (1,), "k_gemv4s: 16-column sub-tiles, 8 waves"),
+    # a wide matrix whose last round of whole tiles is under 70 % full: the sub-tiles up to four f16 rows
+    (4096, 22016, (3, 4), "k_gemv4s: 16-column sub-tiles, 8 waves"),
+])
+def test_planner_branches_on_other_model_shapes(dev, k, n, ms, want):
+    packed, scales, a16 = synth(k, n, max(ms), 7700 + k % 97 + n % 89)
+    w = T.MarlinWeight.upload(dev, packed, scales, k, n)
+    for m in ms:
+        assert dev.plan(k, n, m).startswith(want), dev.plan(k, n, m)
+        truth = O.gemm_f64(f16_as_f32(a16[:m]).reshape(m, k), packed, scales, m, k, n)
+        assert rel_err(run_gemm(dev, w, a16[:m], m, n), truth) < TIGHT, m
+        if m == 1:
+            assert dev.plan(k, n, m, dtype="f32").startswith(want)
+            assert rel_err(run_gemm(dev, w, a16[:m], m, n, a_f32=True), truth) < TIGHT
+    w.free()
+
+
 # ---------------------------------------------------------------- LM head 3584 -> 152064 + argmax
 
 def test_lm_head_gemv_and_argmax_at_vocabulary_width(dev):
