@@ -410,7 +410,7 @@ def main():
         per_shape[name] = {"k": k, "n": n, "us": round(ms * 1e3, 3), "GBps": round(b / (ms * 1e-3) / 1e9, 1),
                            "frac_hbm": round(b / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4), "timed": how,
                            "timed_windows": len(windows), "us_min": round(min(windows) * 1e3, 3),
-                           "us_max": round(max(windows) * 1e3, 3)}
+                           "us_max": round(max(windows) * 1e3, 3), "plan": dev.plan(k, n, 1)}
 
     log("drop-in on the reference layout")
     # the literal drop-in: gemm_tw_marlin_m1 on the reference's arrays (no repack), f32 activations
@@ -431,7 +431,7 @@ def main():
         dev.synchronize()
         ms, how = time_short_launches(dev, T_graphs, one, 104, graphs_done)
         b = k * n // 2 + (k // 32) * n * 2 + k * 4 + n * 4
-        drop_in[name] = {"us": round(ms * 1e3, 2), "GBps": round(b / (ms * 1e-3) / 1e9, 1), "timed": how}
+        drop_in[name] = {"us": round(ms * 1e3, 2), "GBps": round(b / (ms * 1e-3) / 1e9, 1), "timed": how, "plan": dev.plan_m1(k, n)}
         one(0)                                             # layer 0 again, for the comparison
         w, a, c = layers[0][name]
         T.gemm(dev, w, a, 1, c)
