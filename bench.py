@@ -745,12 +745,17 @@ def main():
                 for i in range(3):
                     one(i)
                 dev.synchronize()
-                ms = time_launches(dev, one, 20)
+                # five timed windows of 20 launches each, the median one counts (as for the decode kernels)
+                pf_windows = [time_launches(dev, one, 20)] + [time_launches(dev, one, 20, settle_ms=0.0) for _ in range(4)]
+                ms = sorted(pf_windows)[len(pf_windows) // 2]
                 tf = 2.0 * m * n * k / (ms * 1e-3) / 1e12
                 err, ncols = sampled_prefill_rel_err(c_m.to_host(), packed, scales.view(np.uint16), a_host, m, k, n, rng)
                 assert err < 1e-2, "prefill result outside the tolerance: %g" % err
                 prefill["M%d_K%d_N%d" % (m, k, n)] = {"us": round(ms * 1e3, 1), "TFLOPs": round(tf, 1),
                                                       "frac_mfma_f16_peak": round(tf / MFMA_F16_PEAK_TFLOPS, 4),
+                                                      "timed_windows": len(pf_windows),
+                                                      "us_min": round(min(pf_windows) * 1e3, 1), "us_max": round(max(pf_windows) * 1e3, 1),
+                                                      "plan": dev.plan(k, n, m),
                                                       "max_rel_err": err,
                                                       "max_rel_err_over": "all %d rows x %d sampled columns, f64 product on the FP16 Q4 unpack" % (m, ncols)}
                 if vendor is not None and vendor.ok:
@@ -974,6 +979,8 @@ def main():
         out["roofline_prefill"] = {"bound": "mfma", "kernel": "k_prefill (%s, the slower M = 2048 shape)" % worst[0],
                                    "achieved": worst[1]["TFLOPs"], "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
                                    "frac": worst[1]["frac_mfma_f16_peak"], "us_per_launch": worst[1]["us"],
+                                   "us_min": worst[1]["us_min"], "us_max": worst[1]["us_max"],
+                                   "timed_windows": worst[1]["timed_windows"],
                                    "all_m2048_shapes": {key: v["frac_mfma_f16_peak"] for key, v in m2048.items()}}
     if extra:
         out["batched_decode"] = extra
