@@ -10,6 +10,8 @@ typedef float float4v __attribute__((ext_vector_type(4)));
 typedef unsigned int uint4v __attribute__((ext_vector_type(4)));
 typedef unsigned int uint2v __attribute__((ext_vector_type(2)));
 
+#define TWM_GLOBAL __attribute__((address_space(1)))   // a pointer into device memory, for the builtins that ask for one
+
 // SwiGLU gate of the reference (warp_fused_silu_mul, crates/kernels/src/ops.rs:966-976):
 // silu(g) * u with silu(g) = g / (1 + exp(-g)), every step in f32.  One definition for the
 // elementwise kernels and for the GEMV epilogue, so that both give the same bits.

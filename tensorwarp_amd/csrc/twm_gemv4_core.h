@@ -573,6 +573,24 @@ __device__ __forceinline__ void gemv4s_compute(const ChunkS<SUB, (RL + 3) / 4> &
     }
 }
 
+// The sum of v over the lanes l, l + W, l + 2 W, ... of the wave (W = 16, 32; 64: v itself), returned in every one of
+// them: v_permlane32_swap puts the lower half's values beside the upper half's, v_permlane16_swap the even rows of 16
+// lanes beside the odd ones; an add after each.  The order of the additions is fixed: (g0 + g2) + (g1 + g3).
+template <int W>
+__device__ __forceinline__ float sum_lane_groups(float v)
+{
+    static_assert(W == 16 || W == 32 || W == 64, "lane groups of 16, 32 or 64");
+    if (W <= 32) {
+        auto h = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+        v = __uint_as_float(h[0]) + __uint_as_float(h[1]);
+    }
+    if (W == 16) {
+        auto q = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+        v = __uint_as_float(q[0]) + __uint_as_float(q[1]);
+    }
+    return v;
+}
+
 // The passes first, first + stride, ... < passes with two register sets.  ONE: the caller knows that no wave has a
 // second pass.
 // PIPE: the next pass's loads are in flight while this one is unpacked.  The loop body is one basic block - prefetch,

@@ -75,7 +75,7 @@ __device__ __forceinline__ void gemv4s_body(const char *__restrict__ cw, const v
     constexpr bool F32_PIECE = AF32 && RL == 1;
     constexpr bool PIPE = !ONE && (!AF32 || F32_PIECE) && RL <= 4 && SUB == 16;
     constexpr int TERMS = F32_PIECE ? kTermsOneRowF32 : (PIPE && RL == 1) ? kTermsOneRow : gemv4_terms<AF32, RL>();
-    extern __shared__ float red[];    // [waves][RL][64]
+    extern __shared__ float red[];    // [waves][RL][SUB]
     __shared__ int s_last;
 
     const uint32_t b = blockIdx.x;
@@ -143,70 +143,121 @@ __device__ __forceinline__ void gemv4s_body(const char *__restrict__ cw, const v
     gemv4s_run_passes<SUB, ONE, RG, PIPE>(wave, waves, passes, load_pass, compute_pass);
     if (trace_loaded && threadIdx.x == 0) *trace_loaded = (uint32_t)__builtin_amdgcn_s_memrealtime();  // data arrived and unpacked
 
-    // ---- sum over the waves and over the chunks of a pass (lane groups) through LDS ----
+    // ---- sum over the chunks of a pass (lane groups) inside the wave, over the waves through LDS ----
+    // In the wave: lanes l, l + SUB, ... hold the same column; two lane swaps (v_permlane32_swap, v_permlane16_swap)
+    // and two adds leave the wave's total of a column in every lane that holds it - no LDS, no wait.  Across the waves:
+    // one LDS hop of waves * RL * SUB floats.  Where the RL * SUB entries of the workgroup fit one wave (one or two
+    // rows, four on 16 columns), wave 0 alone finishes: 64 / E lanes per entry each add every (64 / E)-th wave's value,
+    // four independent reads at a time, and the same lane swaps add those - against one thread walking waves * 64 / SUB
+    // values one dependent read after the other, which took longer than the unpack of a pass.
+    constexpr int E = RL * SUB;       // entries of the workgroup: e = r * SUB + column
 #pragma unroll
-    for (int r = 0; r < RL; r++) red[(wave * RL + r) * 64 + lane] = acc[r];
+    for (int r = 0; r < RL; r++) acc[r] = sum_lane_groups<SUB>(acc[r]);
+    if (cg == 0) {
+#pragma unroll
+        for (int r = 0; r < RL; r++) red[wave * E + r * SUB + cl] = acc[r];
+    }
     __syncthreads();
 
-    const uint32_t threads = waves * 64u;
-    const uint32_t entries = RL * SUB;  // entry e = r * SUB + column
-    const uint32_t pair_entries = RL * (SUB / 2), ffn = n >> 1;  // gated: entry e = r * SUB/2 + feature
-    auto summed = [&](uint32_t r, uint32_t c) {
-        float v = 0.f;
-        for (uint32_t w = 0; w < waves; w++)
-#pragma unroll
-            for (int q = 0; q < CPP; q++) v += red[(w * RL + r) * 64 + q * SUB + c];
-        return v;
-    };
+    const uint32_t ffn = n >> 1;
     auto col_of = [&](uint32_t c) { return REFL ? st * SUB + c : tile * 64u + col_in_tile(c); };
-    if (splits == 1) {
+    // Four values at a time of entry e, waves first, first + step, ...: the reads are independent, the sum is in
+    // wave order.  (A wave past the last one re-reads wave 0's value and counts as zero: no branch round a read.)
+    auto sum_waves = [&](uint32_t e, uint32_t first, uint32_t step) {
+        float t = 0.f;
+        for (uint32_t w0 = first; w0 < waves; w0 += 4u * step) {
+            float x[4];
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const uint32_t w = w0 + j * step;
+                x[j] = red[(w < waves ? w : 0u) * E + e];
+            }
+#pragma unroll
+            for (int j = 0; j < 4; j++) t += (w0 + j * step < waves) ? x[j] : 0.f;
+        }
+        return t;
+    };
+    // `total` of entry (r, c), held by the calling lane: to its destination
+    auto finish = [&](uint32_t r, uint32_t c, float total, float partner, bool owner) {
         if (gated) {
-            for (uint32_t e = threadIdx.x; e < pair_entries; e += threads) {
-                uint32_t i = e % (SUB / 2), r = e / (SUB / 2), feat = tile * 32u + part * (SUB / 2) + i;
-                if (r < m_rows && feat < ffn)
-                    out.swiglu[(size_t)r * ffn + feat] = gated_mul(out.gate_act, summed(r, i), summed(r, SUB / 2 + i));
+            // partner = the total of column c + SUB / 2, the up column of gate column c
+            const uint32_t feat = tile * 32u + part * (SUB / 2) + c;
+            if (owner && c < SUB / 2 && r < m_rows && feat < ffn) out.swiglu[(size_t)r * ffn + feat] = gated_mul(out.gate_act, total, partner);
+        } else {
+            const uint32_t on = col_of(c);
+            if (owner && r < m_rows && on < n) gemv4s_store_out(out, r, on, total);
+        }
+    };
+    if constexpr (E <= 64) {
+        // wave 0 finishes; the other waves are done
+        if (wave != 0) return;
+        constexpr int PARTS = 64 / E;
+        const uint32_t e = lane % E, r = e / SUB, c = e % SUB;
+        float total = sum_lane_groups<E>(sum_waves(e, lane / E, PARTS));   // (every lane of an entry holds it)
+        const bool owner = lane < E;
+        if (splits == 1) {
+            finish(r, c, total, gated ? __shfl_down(total, SUB / 2, 64) : 0.f, owner);
+            return;
+        }
+        // cross-workgroup split-K as in k_gemv4: park the partial, count arrivals, the last one adds in split order
+        const uint32_t on = col_of(c);
+        const bool valid = owner && r < m_rows && on < n;
+        if (valid) __hip_atomic_store(&ws[((size_t)sp * m_rows + r) * n_pad + on], total, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __builtin_amdgcn_s_waitcnt(0);  // vmcnt(0): this wave's scratch stores have completed
+        unsigned prev = 0;
+        if (lane == 0) prev = __hip_atomic_fetch_add(&counters[st], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if ((unsigned)__builtin_amdgcn_readfirstlane((int)prev) != splits - 1) return;
+        total = 0.f;
+        if (valid)
+            for (uint32_t s2 = 0; s2 < splits; s2++)
+                total += __hip_atomic_load(&ws[((size_t)s2 * m_rows + r) * n_pad + on], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        finish(r, c, total, gated ? __shfl_down(total, SUB / 2, 64) : 0.f, owner);
+        if (lane == 0) __hip_atomic_store(&counters[st], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        return;
+    } else {
+        // more entries than a wave has lanes (four rows on 32 columns, five to sixteen rows): a thread per entry
+        const uint32_t threads = waves * 64u;
+        if (splits == 1) {
+            for (uint32_t e = threadIdx.x; e < (uint32_t)E; e += threads) {
+                const uint32_t r = e / SUB, c = e % SUB;
+                if (gated) {
+                    if (c < SUB / 2) finish(r, c, sum_waves(e, 0u, 1u), sum_waves(e + SUB / 2, 0u, 1u), true);
+                } else {
+                    finish(r, c, sum_waves(e, 0u, 1u), 0.f, true);
+                }
             }
             return;
         }
-        for (uint32_t e = threadIdx.x; e < entries; e += threads) {
-            uint32_t c = e % SUB, r = e / SUB, on = col_of(c);
-            if (r < m_rows && on < n) gemv4s_store_out(out, r, on, summed(r, c));
+        for (uint32_t e = threadIdx.x; e < (uint32_t)E; e += threads) {
+            const uint32_t r = e / SUB, on = col_of(e % SUB);
+            if (r < m_rows && on < n)
+                __hip_atomic_store(&ws[((size_t)sp * m_rows + r) * n_pad + on], sum_waves(e, 0u, 1u), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
-        return;
-    }
-    // cross-workgroup split-K as in k_gemv4: park the partial, count arrivals, the last one adds in split order
-    for (uint32_t e = threadIdx.x; e < entries; e += threads) {
-        uint32_t c = e % SUB, r = e / SUB, on = col_of(c);
-        if (r < m_rows && on < n)
-            __hip_atomic_store(&ws[((size_t)sp * m_rows + r) * n_pad + on], summed(r, c), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    }
-    __builtin_amdgcn_s_waitcnt(0);  // vmcnt(0): this wave's scratch stores have completed
-    __syncthreads();
-    if (threadIdx.x == 0) {
-        unsigned prev = __hip_atomic_fetch_add(&counters[st], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        s_last = (prev == splits - 1);
-    }
-    __syncthreads();
-    if (!s_last) return;
-    auto parked = [&](uint32_t r, uint32_t on) {
-        float v = 0.f;
-        for (uint32_t s = 0; s < splits; s++)
-            v += __hip_atomic_load(&ws[((size_t)s * m_rows + r) * n_pad + on], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        return v;
-    };
-    if (gated) {
-        for (uint32_t e = threadIdx.x; e < pair_entries; e += threads) {
-            uint32_t i = e % (SUB / 2), r = e / (SUB / 2), feat = tile * 32u + part * (SUB / 2) + i;
-            if (r < m_rows && feat < ffn)
-                out.swiglu[(size_t)r * ffn + feat] = gated_mul(out.gate_act, parked(r, col_of(i)), parked(r, col_of(SUB / 2 + i)));
+        __builtin_amdgcn_s_waitcnt(0);  // vmcnt(0): this wave's scratch stores have completed
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            unsigned prev = __hip_atomic_fetch_add(&counters[st], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            s_last = (prev == splits - 1);
         }
-    } else {
-        for (uint32_t e = threadIdx.x; e < entries; e += threads) {
-            uint32_t c = e % SUB, r = e / SUB, on = col_of(c);
-            if (r < m_rows && on < n) gemv4s_store_out(out, r, on, parked(r, on));
+        __syncthreads();
+        if (!s_last) return;
+        auto parked = [&](uint32_t r, uint32_t on) {
+            float v = 0.f;
+            if (r < m_rows && on < n)
+                for (uint32_t s2 = 0; s2 < splits; s2++)
+                    v += __hip_atomic_load(&ws[((size_t)s2 * m_rows + r) * n_pad + on], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            return v;
+        };
+        for (uint32_t e = threadIdx.x; e < (uint32_t)E; e += threads) {
+            const uint32_t r = e / SUB, c = e % SUB;
+            if (gated) {
+                if (c < SUB / 2) finish(r, c, parked(r, col_of(c)), parked(r, col_of(c + SUB / 2)), true);
+            } else {
+                finish(r, c, parked(r, col_of(c)), 0.f, true);
+            }
         }
+        if (threadIdx.x == 0) __hip_atomic_store(&counters[st], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
-    if (threadIdx.x == 0) __hip_atomic_store(&counters[st], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 // Argument order: what the address arithmetic of the first loads needs comes first, thirteen 32-bit words in all, which
@@ -260,7 +311,7 @@ static hipError_t launch_gemv4s_t(hipStream_t s, const WeightView &w, const void
     uint32_t cps = (w.k_chunks + splits - 1) / splits;
     splits = (w.k_chunks + cps - 1) / cps;
     uint32_t blocks = ((sub_tiles + 7) / 8) * 8 * splits;
-    size_t lds = (size_t)waves * RL * 64 * sizeof(float);
+    size_t lds = (size_t)waves * RL * SUB * sizeof(float);
     const bool one = (cps + 64 / SUB - 1) / (64 / SUB) <= waves;
     const bool runs = blocks <= 512;  // few workgroups per CU: a contiguous run of sub-tiles per XCD
 #define TWM_S_LAUNCH(AF, ONEV)                                                                                          \
@@ -331,7 +382,7 @@ hipError_t launch_gemv4s_ref(hipStream_t s, const uint8_t *packed, const uint16_
     const uint32_t cps = (k_chunks + splits - 1) / splits;
     splits = (k_chunks + cps - 1) / cps;
     const uint32_t blocks = ((sub_tiles + 7) / 8) * 8 * splits;
-    const size_t lds = (size_t)waves * 64 * sizeof(float);
+    const size_t lds = (size_t)waves * sub * sizeof(float);
     const bool one = (cps + 64 / sub - 1) / (64 / sub) <= waves;
     OutSpec out;
     memset(&out, 0, sizeof out);

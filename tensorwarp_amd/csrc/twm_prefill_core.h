@@ -21,7 +21,6 @@ __device__ __forceinline__ PfConsts make_pf_consts()
 // Pins a uniform address in a scalar register pair so that the load takes it as its scalar base with the
 // per-lane part as a 32-bit offset (otherwise the loop-invariant per-lane part is folded into a 64-bit
 // vector base and every load costs a 64-bit vector add).
-#define TWM_GLOBAL __attribute__((address_space(1)))
 __device__ __forceinline__ const TWM_GLOBAL char *scalar_base(const void *p, size_t byte_offset)
 {
     uint64_t v = (uint64_t)p + byte_offset;
