@@ -47,7 +47,14 @@ struct SubPlan {
 static SubPlan plan_gemv4_sub(uint32_t tiles64, uint32_t k_chunks, uint32_t m, bool a_f32)
 {
     const SubPlan none = {0, 0};
-    if (k_chunks < 16) return none;  // shallow K: nothing to gain over one chunk per wave of the 64-column plan
+    // shallow K, one row: short-lived workgroups on sub-tiles, whose waves sum by lane swaps and one LDS hop, are ahead
+    // of the 64-column plan (896 -> 1152 2.64 against 3.09 us, 1536 -> 2048 2.69 / 3.90, 1536 -> 1536 2.67 / 3.86,
+    // 896 -> 9728 3.34 / 3.59; f32 rows 2.72 / 3.31, 2.91 / 4.06); more rows: nothing measured, the 64-column plan stays
+    if (k_chunks < 16) {
+        if (m != 1) return none;
+        const uint32_t p16 = (k_chunks + 3) / 4;
+        return tiles64 > 128 ? SubPlan{32, 8} : SubPlan{16, p16 < 4 ? 4u : p16};
+    }
     const bool two_pass = a_f32 && m > 2;
     const uint32_t passes16 = (k_chunks + 3) / 4;
     // waves per workgroup on 16 columns: one pass each while eight or sixteen cover K; deeper, the pipelined pass loop
@@ -57,7 +64,11 @@ static SubPlan plan_gemv4_sub(uint32_t tiles64, uint32_t k_chunks, uint32_t m, b
     // (one f16 row after the kernel's arguments all came preloaded: four waves ahead from 28 passes on -- 18944 -> 3584
     // 8.58 against 8.74 us on eight, 14336 -> 4096 7.48 / 7.64 -- and level or behind below: 11008 -> 4096 6.60 / 6.62,
     // 11008 -> 2048 5.75 / 5.63, 8960 -> 1536 5.01 / 4.87)
-    const SubPlan narrow16 = {16, passes16 <= 8 ? 8u : passes16 <= 16 ? 16u : ((m >= 2 && !a_f32) || (m == 1 && (a_f32 || passes16 >= 28))) ? 4u : 8u};
+    // (one row, 17 .. 32 passes: two passes per wave with all their loads issued up front, k_gemv4s_upfront -- 11008 -> 4096
+    // 6.20 against 6.44 us in the loop, f32 row 6.35 / 6.64; 14336 -> 4096 7.28 / 7.64; 8960 -> 1536 4.51 / 4.85; three
+    // passes per wave, 18944 -> 3584, are level with the loop on four waves: 8.35 / 8.27)
+    const SubPlan narrow16 = {16, passes16 <= 8 ? 8u : passes16 <= 16 ? 16u : (m == 1 && passes16 <= 32) ? (passes16 + 1) / 2
+                                  : ((m >= 2 && !a_f32) || (m == 1 && (a_f32 || passes16 >= 28))) ? 4u : 8u};
     if (tiles64 > 128) {
         // wide matrices: only the cheapest activations (f16, up to two rows) leave the sub-tiles ahead
         // (3584 -> 37888: 15.8 against 17.0 us at M = 1, 18.3 against 17.3 at M = 4, 19.9 against 17.9 with f32 rows)

@@ -573,6 +573,25 @@ __device__ __forceinline__ void gemv4s_compute(const ChunkS<SUB, (RL + 3) / 4> &
     }
 }
 
+// NP passes per wave - first, first + stride, ... - with every load of the wave issued before the first unpack: NP
+// register sets, no loop.  The loads are unconditional (a pass past the last one replays the k-range's last chunk and
+// nobody unpacks it), so the wait in front of each unpack is an exact count of the loads issued after its own.
+template <int SUB, int NP, int RG = 1, class Load, class Compute>
+__device__ __forceinline__ void gemv4s_run_upfront(uint32_t first, uint32_t stride, uint32_t passes, Load load, Compute compute)
+{
+    ChunkS<SUB, RG> r[NP];
+#pragma unroll
+    for (int i = 0; i < NP; i++) {
+        load(r[i], first + i * stride);
+        __builtin_amdgcn_sched_barrier(0);
+    }
+#pragma unroll
+    for (int i = 0; i < NP; i++) {
+        if (first + i * stride < passes) compute(r[i]);
+        __builtin_amdgcn_sched_barrier(0);
+    }
+}
+
 // The sum of v over the lanes l, l + W, l + 2 W, ... of the wave (W = 16, 32; 64: v itself), returned in every one of
 // them: v_permlane32_swap puts the lower half's values beside the upper half's, v_permlane16_swap the even rows of 16
 // lanes beside the odd ones; an add after each.  The order of the additions is fixed: (g0 + g2) + (g1 + g3).

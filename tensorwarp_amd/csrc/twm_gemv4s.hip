@@ -55,7 +55,10 @@ __device__ __forceinline__ void gemv4s_store_out(const OutSpec &out, uint32_t m,
 // take the passes (64 / SUB chunks each) of the k-range in turn.
 // REFL: cw is the reference's packed array u8 [G][N][16] and ref_scales its f16 [G][N] (no repack; one row of f32
 // activations): a sub-tile's records of one group are still SUB * 16 contiguous bytes.
-template <int SUB, int RL, bool AF32, bool ONE, bool REFL>
+// NP >= 2 (16 columns, one row): every wave makes up to NP passes and issues all their loads before its first unpack
+// (gemv4s_run_upfront): a workgroup that is alone on its CU has its whole share of the matrix in flight at once, like
+// the one-pass form, where the pass loop keeps two passes per wave in flight and walks K one memory round trip at a time.
+template <int SUB, int RL, bool AF32, bool ONE, bool REFL, int NP = 0>
 __device__ __forceinline__ void gemv4s_body(const char *__restrict__ cw, const void *__restrict__ a_any, const OutSpec &out,
                                             float *__restrict__ ws, unsigned *__restrict__ counters, uint32_t cfg,
                                             uint32_t k, uint32_t n, uint32_t n_pad, uint32_t k_chunks,
@@ -73,8 +76,10 @@ __device__ __forceinline__ void gemv4s_body(const char *__restrict__ cw, const v
     // One row of f32 activations: the shared-piece form as well (a lane splits one piece instead of two or four),
     // which on 16 columns also leaves room for the pipelined loop.
     constexpr bool F32_PIECE = AF32 && RL == 1;
-    constexpr bool PIPE = !ONE && (!AF32 || F32_PIECE) && RL <= 4 && SUB == 16;
-    constexpr int TERMS = F32_PIECE ? kTermsOneRowF32 : (PIPE && RL == 1) ? kTermsOneRow : gemv4_terms<AF32, RL>();
+    constexpr bool UPFRONT = NP >= 2;
+    static_assert(!UPFRONT || (!ONE && RL == 1 && SUB == 16), "several passes up front: one row on 16 columns");
+    constexpr bool PIPE = !ONE && !UPFRONT && (!AF32 || F32_PIECE) && RL <= 4 && SUB == 16;
+    constexpr int TERMS = F32_PIECE ? kTermsOneRowF32 : ((PIPE || UPFRONT) && RL == 1) ? kTermsOneRow : gemv4_terms<AF32, RL>();
     extern __shared__ float red[];    // [waves][RL][SUB]
     __shared__ int s_last;
 
@@ -124,7 +129,7 @@ __device__ __forceinline__ void gemv4s_body(const char *__restrict__ cw, const v
             gemv4s_load_pass_ref<SUB, TERMS, RG>(r, cw, ref_scales, a_any, arow, kc, live, ref_col, st * SUB + cl < n, n, ref_groups,
                                                  cl, k, lane_is_lo);
         } else {
-            if (PIPE) {
+            if (PIPE || UPFRONT) {
                 // activations first: loads complete in the order of their issue, and these come from the cache
                 gemv4s_load_a<SUB, AF32, TERMS, REFL, RG>(r, a_any, arow, kc, cl, k, lane_is_lo, m_rows);
                 gemv4s_load_w<SUB, RG, true>(r, tbase + (size_t)kc * kColBlockBytes, col_in_tile(cl), live);
@@ -140,7 +145,8 @@ __device__ __forceinline__ void gemv4s_body(const char *__restrict__ cw, const v
     };
     auto compute_pass = [&](const ChunkS<SUB, RG> &r) { gemv4s_compute<SUB, RL, TERMS, REFL>(r, dq, acc); };
     // (ONE: the launcher saw that no wave has a second pass: one register set, no loop)
-    gemv4s_run_passes<SUB, ONE, RG, PIPE>(wave, waves, passes, load_pass, compute_pass);
+    if constexpr (UPFRONT) gemv4s_run_upfront<SUB, NP, RG>(wave, waves, passes, load_pass, compute_pass);
+    else gemv4s_run_passes<SUB, ONE, RG, PIPE>(wave, waves, passes, load_pass, compute_pass);
     if (trace_loaded && threadIdx.x == 0) *trace_loaded = (uint32_t)__builtin_amdgcn_s_memrealtime();  // data arrived and unpacked
 
     // ---- sum over the chunks of a pass (lane groups) inside the wave, over the waves through LDS ----
@@ -278,6 +284,18 @@ __global__ __launch_bounds__(1024) void k_gemv4s(const char *__restrict__ cw, co
                                           nullptr);
 }
 
+// 16 columns, one row, up to NP passes per wave with all their loads issued up front.
+template <bool AF32, bool REFL, int NP>
+__global__ __launch_bounds__(1024) void k_gemv4s_upfront(const char *__restrict__ cw, const void *__restrict__ a_any,
+                                                          const uint16_t *__restrict__ ref_scales, uint32_t cfg, uint32_t k,
+                                                          uint32_t k_chunks, uint32_t sub_tiles, uint32_t cps, uint32_t n,
+                                                          uint32_t n_pad, float *__restrict__ ws, unsigned *__restrict__ counters,
+                                                          OutSpec out)
+{
+    gemv4s_body<16, 1, AF32, false, REFL, NP>(cw, a_any, out, ws, counters, cfg, k, n, n_pad, k_chunks, sub_tiles, cps, ref_scales,
+                                              nullptr);
+}
+
 // The same kernel with a trace (twm_debug_trace; one row of f16 activations only): workgroup b writes four words at
 // trace[4 b]: the 100 MHz clock at its start, after wave 0 has unpacked its passes, and at its end, and the hardware
 // id of the CU it ran on.  A kernel of its own: reading the trace pointer first would put a second, dependent kernel
@@ -326,6 +344,19 @@ static hipError_t launch_gemv4s_t(hipStream_t s, const WeightView &w, const void
             else
                 hipLaunchKernelGGL((k_gemv4s_traced<SUB, false>), dim3(blocks), dim3(waves * 64), lds, s, (const char *)w.cq, a, out,
                                    ws, counters, m, w.k, w.n, n_pad, w.k_chunks, sub_tiles, splits, cps, g_trace.ptr);
+            return hipGetLastError();
+        }
+    }
+    if constexpr (SUB == 16 && RL == 1) {
+        const uint32_t np = ((cps + 3) / 4 + waves - 1) / waves;  // passes per wave
+        if ((np == 2 || np == 3) && !out.swiglu) {
+#define TWM_S_UP(AF, NPV)                                                                                               \
+    hipLaunchKernelGGL((k_gemv4s_upfront<AF, false, NPV>), dim3(blocks), dim3(waves * 64), lds, s, (const char *)w.cq, a,    \
+                       (const uint16_t *)nullptr, gemv4s_cfg(splits, false, waves, m, runs), w.k, w.k_chunks, sub_tiles, cps, \
+                       w.n, n_pad, ws, counters, out)
+            if (a_f32) { if (np == 2) TWM_S_UP(true, 2); else TWM_S_UP(true, 3); }
+            else { if (np == 2) TWM_S_UP(false, 2); else TWM_S_UP(false, 3); }
+#undef TWM_S_UP
             return hipGetLastError();
         }
     }
@@ -394,6 +425,16 @@ hipError_t launch_gemv4s_ref(hipStream_t s, const uint8_t *packed, const uint16_
     hipLaunchKernelGGL((k_gemv4s<SUBV, 1, true, ONEV, true>), dim3(blocks), dim3(waves * 64), lds, s, (const char *)packed, \
                        (const void *)a, scales, gemv4s_cfg(splits, false, waves, 1u), k, k_chunks, sub_tiles, cps, n, n_pad, ws,  \
                        counters, out)
+    const uint32_t np = ((cps + 3) / 4 + waves - 1) / waves;  // passes per wave on 16 columns
+    if (sub == 16 && (np == 2 || np == 3)) {
+        if (np == 2)
+            hipLaunchKernelGGL((k_gemv4s_upfront<true, true, 2>), dim3(blocks), dim3(waves * 64), lds, s, (const char *)packed, (const void *)a,
+                               scales, gemv4s_cfg(splits, false, waves, 1u), k, k_chunks, sub_tiles, cps, n, n_pad, ws, counters, out);
+        else
+            hipLaunchKernelGGL((k_gemv4s_upfront<true, true, 3>), dim3(blocks), dim3(waves * 64), lds, s, (const char *)packed, (const void *)a,
+                               scales, gemv4s_cfg(splits, false, waves, 1u), k, k_chunks, sub_tiles, cps, n, n_pad, ws, counters, out);
+        return hipGetLastError();
+    }
     if (sub == 32) {
         if (one) TWM_S_REF(32, true);
         else TWM_S_REF(32, false);

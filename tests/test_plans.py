@@ -57,7 +57,7 @@ def test_plans_of_the_qwen7b_projections(lib, name, m, dtype, want):
     (11008, 4096, 512, "k_prefill: 128-row x 256-column blocks, 4 K-splits + k_splitk_reduce; 16-column tile copy"),
     (3584, 4608, 2048, "k_prefill: 128-row x 192-column blocks, 1 K-split; 16-column tile copy"),
     (3584, 152064, 1, "k_gemv4: 1 x 64-column tiles per workgroup, 8 waves, 1 K-split; column-lane copy"),
-    (896, 1152, 1, "k_gemv4: 1 x 64-column tiles per workgroup, 8 waves, 1 K-split; column-lane copy"),
+    (896, 1152, 1, "k_gemv4s: 16-column sub-tiles, 4 waves, 1 K-split; column-lane copy"),
 ])
 def test_plans_of_prefill_lm_head_and_small_shapes(lib, k, n, m, want):
     assert describe(lib, k, n, m) == want
