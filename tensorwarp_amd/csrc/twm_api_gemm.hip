@@ -80,9 +80,9 @@ static SubPlan plan_gemv4_sub(uint32_t tiles64, uint32_t k_chunks, uint32_t m, b
         // rounds: 49.3 against 47.8)
         const uint32_t rounds = (tiles64 + 255) / 256;
         const bool poor_fill = tiles64 * 5 < rounds * 256 * 4;
-        // (several workgroups per CU: no idle eighth wave, 3584 -> 37888 at M = 1 14.8 against 15.3 us; with one workgroup
-        // per CU the eight-wave form is the faster one, 3584 -> 3584 3.9 against 4.05)
-        if (!a_f32 && m <= 2 && passes16 <= 8 && poor_fill) return SubPlan{16, passes16};
+        // (an even number of waves, so that the workgroups of a CU lie evenly on its four SIMDs and four of them fit:
+        // 3584 -> 37888 at M = 1 13.4 us on eight waves, the eighth idle, against 14.2 on seven)
+        if (!a_f32 && m <= 2 && passes16 <= 8 && poor_fill) return SubPlan{16, (passes16 + 1u) & ~1u};
         // (three and four rows: only where the last round is under 70 % full -- 4096 -> 22016, 67 %: 11.6 / 12.4 against
         // 12.8 / 12.9 us on whole tiles; 3584 -> 37888, 77 %: 16.3 / 17.5 against 16.0 / 16.1)
         if (!a_f32 && m <= 4 && passes16 <= 8 && tiles64 * 10 < rounds * 256 * 7) return SubPlan{16, passes16};

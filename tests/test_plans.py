@@ -27,10 +27,10 @@ QWEN7B = {"qkv": (3584, 4608), "o": (3584, 3584), "gate_up": (3584, 37888), "dow
 
 
 @pytest.mark.parametrize("name,m,dtype,want", [
-    # M = 1, the headline: sub-tiles everywhere; gate_up one pass per wave (28 chunks / 4 = 7 waves), down the pass loop
+    # M = 1, the headline: sub-tiles everywhere; gate_up one pass per wave (28 chunks / 4 = 7 passes on eight waves), down the pass loop
     ("qkv", 1, "f16", "k_gemv4s: 32-column sub-tiles, 16 waves, 1 K-split; column-lane copy"),
     ("o", 1, "f16", "k_gemv4s: 16-column sub-tiles, 8 waves, 1 K-split; column-lane copy"),
-    ("gate_up", 1, "f16", "k_gemv4s: 16-column sub-tiles, 7 waves, 1 K-split; column-lane copy"),
+    ("gate_up", 1, "f16", "k_gemv4s: 16-column sub-tiles, 8 waves, 1 K-split; column-lane copy"),
     ("down", 1, "f16", "k_gemv4s: 16-column sub-tiles, 4 waves, 1 K-split; column-lane copy"),
     # one row of f32 activations: the pass loop on four waves where K is deep or the matrix wide
     ("gate_up", 1, "f32", "k_gemv4s: 16-column sub-tiles, 4 waves, 1 K-split; column-lane copy"),
