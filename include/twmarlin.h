@@ -213,12 +213,17 @@ int twm_gemm_tw_marlin_m1_from_buffer(twm_ctx *ctx, const float *a_dev, const ui
  * harnesses that forbid hipMalloc.  No counterpart in the reference.  It takes no context: work is issued on
  * hip_stream (a hipStream_t, NULL = the null stream) of the current device, with the library's default plan, and
  * the split-K scratch is a static device array inside the library (64 KiB of partial sums + 256 counters per GPU,
- * held until the process ends).  The call itself allocates and frees nothing and never synchronises.  Results are
+ * held until the process ends; the default plan cuts K over workgroups on matrices of at most 1024 columns whose K is
+ * at least 16384 deep, e.g. 16384 -> 256, and those launches park their partial sums there).  The call itself allocates and frees nothing and never synchronises.  Results are
  * bit-identical to twm_gemm_tw_marlin_m1 with default options.  Limits: N <= 2^20 and K <= 2^20, beyond which
  * TWM_SHAPE_ERROR is returned; alignment rules as twm_gemm_tw_marlin_m1.  All calls on one GPU share that GPU's
  * array: two calls that overlap in time on one GPU (two streams, two threads) race; calls on one stream do not. */
 int twm_gemm_tw_marlin_m1_noalloc(void *hip_stream, const float *a_dev, const uint8_t *packed_dev,
                                   const uint16_t *scales_dev, float *c_dev, uint32_t n, uint32_t k);
+/* Testing aid for the entry point above (no counterpart in the reference): sets every byte of the current GPU's static
+ * scratch, partial sums and arrival counters, to `value` on hip_stream.  A test poisons the scratch with it and then
+ * shows that a call's result does not depend on what was there.  Not for use under graph capture. */
+int twm_noalloc_scratch_fill(void *hip_stream, int value);
 /* The reference's adaptive split-K rule, bit for bit (quantize.rs:1314-1325). */
 void twm_pick_splits_reference(uint32_t k, uint32_t n, uint32_t *n_blocks, uint32_t *splits,
                                uint32_t *groups_per_split);

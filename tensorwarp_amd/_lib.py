@@ -51,6 +51,7 @@ SIGNATURES = {
     "twm_pair_gate_up": (_int, [_vp, _vp, _vp, _vp, _vp, _u32, _u32, _vp, _vp]),
     "twm_gemm_tw_marlin_m1": (_int, [_vp, _vp, _vp, _vp, _vp, _u32, _u32]),
     "twm_gemm_tw_marlin_m1_noalloc": (_int, [_vp, _vp, _vp, _vp, _vp, _u32, _u32]),
+    "twm_noalloc_scratch_fill": (_int, [_vp, _int]),
     "twm_gemm_tw_marlin_m1_from_buffer": (_int, [_vp, _vp, _vp, _sz, _vp, _sz, _vp, _u32, _u32]),
     "twm_pick_splits_reference": (None, [_u32, _u32, C.POINTER(_u32), C.POINTER(_u32), C.POINTER(_u32)]),
     "twm_weight_upload": (_vp, [_vp, _vp, _vp, _u32, _u32]),

@@ -541,7 +541,7 @@ static M1Form choose_m1_form(int exact, int force_sub, int force_waves, int forc
     // 14336 -> 4096 9.7) and, eight waves of one pass each, on wide matrices up to K = 4096 (3584 -> 37888 16.3 against
     // 18.1 us on 32 columns, 4096 -> 22016 11.8 against 12.5, 4096 -> 28672 14.6 against 15.8); in between sixteen waves
     // on 32 columns as long as every wave gets a single pass (3584 -> 4608 4.7 against 4.9, 4096 -> 6144 5.1 against
-    // 5.5).  Deeper matrices of 256 tiles or more keep the 64-column kernel and its split-K (8192 -> 57344: 46.6 against
+    // 5.5).  Deeper matrices of 256 tiles or more keep the 64-column kernel (its K-split only by option; 8192 -> 57344: 46.6 against
     // 63.7 us).
     // Fitted to sweeps over the Qwen2.5-7B, Llama-2-7B, Llama-3-8B, 13B and 70B projections; option "sub" = 1 keeps the
     // 64-column kernel.
@@ -561,18 +561,23 @@ static M1Form choose_m1_form(int exact, int force_sub, int force_waves, int forc
     }
     if (use_sub) {
         uint32_t sp = force_splits ? (uint32_t)force_splits : 1;
+        if (!force_splits && sub == 16 && n_pad / 16 <= 64) {
+            // A few sub-tiles on a very deep K (16384 -> 256 is sixteen workgroups): cut K over workgroups while that
+            // leaves each at least 64 chunks and the workgroups within the CU count -- the hand-over between workgroups
+            // (partial sums of a few KB, the last to arrive adds them in split order) costs over a microsecond, and only
+            // such ranges are worth it: 16384 -> 256 5.70 us on two ranges against 6.76 on one (four 5.62, eight 7.02),
+            // 32768 -> 64 6.09 on four against 12.57; but 8192 -> 200 4.30 on one against 4.76 on two, 4096 -> 1000 3.28 / 4.54.
+            while (n_pad / 16 * sp * 2 <= 256 && k_chunks / (sp * 2) >= 64) sp *= 2;
+        }
         if (force_waves) sub_waves = (uint32_t)force_waves;
         if (sp > k_chunks) sp = k_chunks;
         while (sp > 1 && (size_t)sp * n_pad * 4 > ws_bytes) sp--;
         if (n_pad / sub > n_counters) sp = 1;
         return M1Form{kM1SubTile, sub, sub_waves, sp};
     }
+    // (only matrices of 256 tiles or more on a deep K get here, or option "sub" = 1: eight waves, no K-split of its own)
     f.kind = kM1WholeTile;
     f.waves = 8;
-    if (tiles64 < 256) {
-        f.waves = 16;
-        while (tiles64 * f.splits * 2 <= 256 && k_chunks >= f.splits * 2 * 8) f.splits *= 2;
-    }
     if (force_waves) f.waves = (uint32_t)force_waves;
     if (force_splits) f.splits = (uint32_t)force_splits;
     if (f.splits > k_chunks) f.splits = k_chunks;

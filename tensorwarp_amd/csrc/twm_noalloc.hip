@@ -11,9 +11,9 @@ using namespace twm;
 
 namespace {
 
-// f32 partial sums followed by the arrival counters.  The dispatch splits K only below 256 column tiles of 64 and
-// never into more than 256 / tiles ranges, so splits x padded N <= 16384 floats and fewer than 256 counters are
-// ever used, whatever the shape.
+// f32 partial sums followed by the arrival counters.  The default plan splits K only on matrices of at most 64
+// sub-tiles of 16 columns (N <= 1024) and never into more ranges than bring the workgroups to 256, so splits x padded
+// N <= 4096 floats and at most 64 counters are ever used, whatever the shape; a split that would not fit is reduced.
 constexpr size_t kPartialBytes = 64u << 10;
 constexpr uint32_t kCounters = 256;
 // the largest shape the entry point takes
@@ -73,4 +73,16 @@ extern "C" int twm_gemm_tw_marlin_m1_noalloc(void *hip_stream, const float *a_de
     const M1Env env = {(hipStream_t)hip_stream, 0, 0, 0, 0, (float *)base, kPartialBytes,
                        (unsigned *)(base + kPartialBytes), kCounters, true};
     return m1_dispatch(env, who, a_dev, packed_dev, scales_dev, c_dev, n, k);
+}
+
+// Testing aid: every byte of the current GPU's scratch (partial sums and counters) set to `value` on hip_stream, so
+// that a test can show that a call does not depend on what earlier calls left there.  Not for capture (a memset node).
+extern "C" int twm_noalloc_scratch_fill(void *hip_stream, int value)
+{
+    const char *who = "twm_noalloc_scratch_fill";
+    unsigned char *base = (unsigned char *)noalloc_scratch_for_current_device(who);
+    if (!base) return TWM_DEVICE_ERROR;
+    hipError_t e = hipMemsetAsync(base, value & 0xFF, sizeof scratch, (hipStream_t)hip_stream);
+    if (e != hipSuccess) return api_fail(TWM_DEVICE_ERROR, "%s: %s", who, hipGetErrorString(e));
+    return TWM_OK;
 }

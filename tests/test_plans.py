@@ -132,8 +132,8 @@ def test_known_drop_in_plans(lib, k, n, want):
 
 
 def test_drop_in_plan_invariants(lib):
-    for k in (32, 64, 896, 2048, 3584, 4096, 5120, 8192, 11008, 18944, 28672):
-        for n in (8, 64, 300, 1152, 4096, 4608, 6144, 8192, 16384, 22016, 57344):
+    for k in (32, 64, 896, 2048, 3584, 4096, 5120, 8192, 11008, 16384, 18944, 28672, 32768, 65536):
+        for n in (8, 64, 100, 256, 300, 1024, 1152, 4096, 4608, 6144, 8192, 16384, 22016, 57344):
             text = describe_m1(lib, k, n)
             kernel = text.split(":")[0]
             assert kernel in ("k_gemv4s", "k_gemv4"), text
@@ -143,6 +143,14 @@ def test_drop_in_plan_invariants(lib):
             assert 1 <= waves <= 16 and 1 <= splits <= k_chunks, (k, n, text)
             if kernel == "k_gemv4s":
                 assert int(re.search(r"(\d+)-column sub-tiles", text).group(1)) in (16, 32)
+            # K is cut over workgroups only on a few 16-column sub-tiles with a very deep K each, within the CU count;
+            # what the no-allocation entry point's static scratch (16 Ki floats, 256 counters) is sized by
+            sub_tiles = (n + 63) // 64 * 4
+            if splits > 1:
+                assert kernel == "k_gemv4s" and sub_tiles <= 64 and k_chunks // splits >= 64 and sub_tiles * splits <= 256, (k, n, text)
+                assert splits * ((n + 63) // 64 * 64) <= 16384 and sub_tiles <= 256
+    assert "2 K-splits" in describe_m1(lib, 16384, 256) and "4 K-splits" in describe_m1(lib, 32768, 64)
+    assert "1 K-split;" in describe_m1(lib, 8192, 200) and "1 K-split;" in describe_m1(lib, 18944, 3584)
 
 
 def test_describe_m1_edges(lib):
