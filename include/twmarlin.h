@@ -97,7 +97,6 @@ int twm_ctx_info(twm_ctx *ctx, char *buf, size_t buf_len);
  *   "weight_copies" the repacked orders a new weight handle is given: 0 or 3 = both, 1 = 16-column tiles only,
  *                   2 = column lanes only (twm_weight_ensure)
  *   "sub_waves"     waves per workgroup of the sub-tile kernels when "sub" forces their width (1 .. 16)
- *   "prefill_sk"    prefill GEMM: 128 = tiles dealt out by stream-K over one workgroup per CU, 0 / 1 = off
  *   "prefill_min_m" smallest M that runs the prefill GEMM (default 33; below it the decode kernels run)
  *   "prefill_bm"    prefill block form: 64 = 64 rows x 256 columns, 128 = 128 x 256, 192 = 128 rows x 192 columns
  *   "m1_exact"      twm_gemm_tw_marlin_m1: 1 = f32 activations and f32 FMAs in the reference kernel's order with

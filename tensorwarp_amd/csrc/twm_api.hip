@@ -66,9 +66,6 @@ twm_ctx *twm_ctx_create(int ordinal)
     c->prefill_bm = 0;
     c->prefill_min_m = 33;  // M <= 32 is batched decode (exact f32 scales, weights streamed once)
     c->ws = nullptr;
-    c->sk_ws = nullptr;
-    c->sk_ws_bytes = 0;
-    c->prefill_sk = 0;
     c->counters = nullptr;
     c->own_stream = nullptr;
     bool ok = hipSetDevice(ordinal) == hipSuccess && hipGetDeviceProperties(&c->prop, ordinal) == hipSuccess;
@@ -79,23 +76,18 @@ twm_ctx *twm_ctx_create(int ordinal)
         return nullptr;
     }
     ok = ok && hipStreamCreateWithFlags(&c->own_stream, hipStreamNonBlocking) == hipSuccess;
-    ok = ok && init_prefill() == hipSuccess && init_prefill_sk() == hipSuccess;
+    ok = ok && init_prefill() == hipSuccess;
     ok = ok && noalloc_scratch_for_current_device("twm_ctx_create") != nullptr;
     c->stream = c->own_stream;
     c->ws_bytes = kWsBytes;
     c->n_counters = kCounters;
     ok = ok && hipMalloc((void **)&c->ws, c->ws_bytes) == hipSuccess;
     ok = ok && hipMalloc((void **)&c->counters, c->n_counters * sizeof(unsigned)) == hipSuccess;
-    if (ok) {  // two 256-row partial tiles per CU
-        c->sk_ws_bytes = prefill_sk_scratch_bytes(256, (uint32_t)c->prop.multiProcessorCount);
-        ok = hipMalloc((void **)&c->sk_ws, c->sk_ws_bytes) == hipSuccess;
-    }
     ok = ok && hipMemset(c->counters, 0, c->n_counters * sizeof(unsigned)) == hipSuccess;
     ok = ok && hipDeviceSynchronize() == hipSuccess;
     if (!ok) {
         api_fail(TWM_DEVICE_ERROR, "twm_ctx_create: %s", hipGetErrorString(hipGetLastError()));
         if (c->ws) (void)hipFree(c->ws);
-        if (c->sk_ws) (void)hipFree(c->sk_ws);
         if (c->counters) (void)hipFree(c->counters);
         if (c->own_stream) (void)hipStreamDestroy(c->own_stream);
         delete c;
@@ -110,7 +102,6 @@ void twm_ctx_destroy(twm_ctx *ctx)
     (void)hipSetDevice(ctx->ordinal);
     (void)hipStreamSynchronize(ctx->stream);
     (void)hipFree(ctx->ws);
-    (void)hipFree(ctx->sk_ws);
     (void)hipFree(ctx->counters);
     (void)hipStreamDestroy(ctx->own_stream);
     delete ctx;
@@ -193,12 +184,6 @@ int twm_ctx_set_option(twm_ctx *ctx, const char *key, int value)
         if (value != 0 && value != 64 && value != 128 && value != 192)
             return api_fail(TWM_SHAPE_ERROR, "twm_ctx_set_option: prefill_bm must be 0, 64, 128 or 192");
         ctx->prefill_bm = value;
-        return TWM_OK;
-    }
-    if (strcmp(key, "prefill_sk") == 0) {
-        if (value != 0 && value != 1 && value != 128 && value != 256)
-            return api_fail(TWM_SHAPE_ERROR, "twm_ctx_set_option: prefill_sk must be 0, 1, 128 or 256");
-        ctx->prefill_sk = value;
         return TWM_OK;
     }
     if (strcmp(key, "prefill_min_m") == 0) {

@@ -457,9 +457,7 @@ static int gemm_dispatch(twm_ctx *ctx, const twm_weight *w, const void *a_dev, i
     };
     switch (f.kind) {
     case kFormPrefill: {
-        const PrefillSk sk = {ctx->sk_ws, ctx->sk_ws_bytes, ctx->counters, ctx->n_counters, (uint32_t)ctx->prop.multiProcessorCount,
-                              ctx->prefill_sk};
-        HIP_TRY(launch_prefill(ctx->stream, v, a_dev, a_f32, m, gated, (uint32_t)ctx->prefill_bm, splits, ctx->ws, ctx->ws_bytes, &sk),
+        HIP_TRY(launch_prefill(ctx->stream, v, a_dev, a_f32, m, gated, (uint32_t)ctx->prefill_bm, splits, ctx->ws, ctx->ws_bytes),
                 TWM_DEVICE_ERROR, "prefill launch");
         return TWM_OK;
     }

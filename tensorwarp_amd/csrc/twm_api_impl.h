@@ -25,9 +25,6 @@ struct twm_ctx {
     hipStream_t stream;
     float *ws;            // split-K partial tiles
     size_t ws_bytes;
-    float *sk_ws;         // parked partial tiles of the stream-K prefill GEMM
-    size_t sk_ws_bytes;
-    int prefill_sk;       // stream-K prefill: 0 = the planner's choice, 1 = off, 128 / 256 = on with that block height
     unsigned *counters;   // one arrival counter per tile group, zero between launches
     uint32_t n_counters;
     bool capturing;

@@ -156,23 +156,8 @@ hipError_t launch_gemv4(hipStream_t s, const WeightView &w, const void *a, bool 
 hipError_t launch_gemv4_ref(hipStream_t s, const uint8_t *packed, const uint16_t *scales, uint32_t k, uint32_t n,
                             const float *a, float *c, float *ws, unsigned *counters, uint32_t waves, uint32_t splits);
 hipError_t init_prefill();
-// Stream-K scheduling of the prefill GEMM (twm_prefill_sk.hip): what launch_prefill needs to take it
-struct PrefillSk {
-    float *partials;       // parked partial tiles
-    size_t partial_bytes;
-    unsigned *counters;    // one per tile, zero between launches
-    uint32_t n_counters;
-    uint32_t workers;      // workgroups to launch: one per CU
-    int mode;              // 0 = the planner's choice, 1 = off, 128 / 256 = on with blocks of that many rows
-};
 hipError_t launch_prefill(hipStream_t s, const WeightView &w, const void *a, bool a_f32, uint32_t m, const OutSpec &out,
-                          uint32_t block_rows, uint32_t splits, void *scratch, size_t scratch_bytes,
-                          const PrefillSk *sk = nullptr);
-hipError_t init_prefill_sk();
-size_t prefill_sk_scratch_bytes(uint32_t block_rows, uint32_t workers);
-hipError_t launch_prefill_sk(hipStream_t s, const WeightView &w, const _Float16 *a16, uint32_t m, const OutSpec &out,
-                             uint32_t block_rows, uint32_t workers, float *partials, size_t partial_bytes,
-                             unsigned *counters, uint32_t n_counters);
+                          uint32_t block_rows, uint32_t splits, void *scratch, size_t scratch_bytes);
 // out[row][col] = sum over splits (in order) of partials[split][row][col], partials rows n_ld floats wide
 hipError_t launch_splitk_reduce(hipStream_t s, const float *partials, const OutSpec &out, uint32_t m, uint32_t n,
                                 uint32_t n_ld, uint32_t splits);

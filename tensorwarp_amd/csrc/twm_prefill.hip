@@ -571,19 +571,11 @@ hipError_t init_prefill()
 // `scratch` (scratch_bytes) holds the f16 copy of f32 activations and / or the split-K partials; when it
 // cannot hold all M rows the rows are processed in slabs.
 hipError_t launch_prefill(hipStream_t s, const WeightView &w, const void *a, bool a_f32, uint32_t m, const OutSpec &out,
-                          uint32_t block_rows, uint32_t splits, void *scratch, size_t scratch_bytes, const PrefillSk *sk)
+                          uint32_t block_rows, uint32_t splits, void *scratch, size_t scratch_bytes)
 {
     if (m == 0 || w.n == 0) return hipSuccess;
     if (block_rows != 0 && block_rows != 64 && block_rows != 128 && block_rows != 192) return hipErrorInvalidValue;
     auto run = [&](const _Float16 *a16, uint32_t rows, const OutSpec &o, void *ws, size_t ws_bytes) {
-        // Option prefill_sk: the tiles dealt out by stream-K (twm_prefill_sk.hip); the gated store stays with the plain kernel.
-        if (sk && sk->mode >= 128 && !o.swiglu && sk->partials) {
-            const uint32_t sk_rows = 128u;
-            hipError_t e = launch_prefill_sk(s, w, a16, rows, o, sk_rows, sk->workers, sk->partials, sk->partial_bytes, sk->counters,
-                                             sk->n_counters);
-            if (e != hipErrorInvalidValue) return e;  // (a shape it does not take: the plain kernel below)
-            (void)hipGetLastError();
-        }
         // (a forced 192-column form with the gated store: the 256-column one)
         const uint32_t form = block_rows == 192 && o.swiglu ? 128u : block_rows;
         const PrefillPlan plan = plan_prefill_within(rows, form, splits, w.n_tiles, w.k_chunks, ws ? ws_bytes : 0, o.swiglu != nullptr);

@@ -1,4 +1,4 @@
-// Building blocks shared by the prefill GEMM kernels (twm_prefill.hip, twm_prefill_sk.hip): the Q4 unpack to MFMA B
+// Building blocks of the prefill GEMM kernel (twm_prefill.hip): the Q4 unpack to MFMA B
 // operands, the scalar-base load helper, the generic output store.
 #pragma once
 #include "twm_device.h"
