@@ -288,11 +288,16 @@ int twm_weight_dequant_f16(twm_ctx *ctx, const twm_weight *w, uint16_t *out_kn_d
  * M <= 32: decode kernels (M <= 4 one lane per column, above that 16-column tiles), weights exact,
  *          each group's f32 sum scaled by f32(scale): a row's result does not depend on the batch it is in
  *          beyond f32 summation order.  (Option "batch_rounded": M = 17 .. 32 on the FP16 Q4 unpack.)
- * Up to M = 32 f32 activations enter as two f16 terms, a first term and the residual, about 21 bits.  M <= 4 takes any
- * finite f32 (values beyond the f16 range are scaled into it by a power of two per row, and the sums back); from
- * M = 5 on |a| must stay inside the f16 range, as in the reference's FP16 route for M > 1.
- * M  > 32: prefill GEMM on the same FP16 unpack; f32 activations are rounded to f16 first.  Uses the
- * context's scratch: one context must not run two calls at the same time. */
+ * Up to M = 32 f32 activations enter as two f16 terms, a first term and the residual, about 21 bits.  Any finite f32
+ * row is taken, as by the reference's kernels, which multiply in f32 (quantize.rs:1188, 186-246): values beyond the f16
+ * range, and rows too small for it, are scaled by a power of two first and the sums back, both exact -- per stretch of
+ * a row inside the kernels at M <= 4, per row by a conversion kernel ahead of the GEMM from M = 5 on.
+ * M  > 32: prefill GEMM on the FP16 Q4 unpack (the arithmetic of the reference's FP16 route, DequantizedF16Weights +
+ *          HGEMM, quantize.rs:620-670).  f32 activations are scaled per row in the same way and then rounded to ONE f16
+ *          term: a deviation from gemm_q4_0 (quantize.rs:1825-1858), which multiplies f32 A by f32 weights -- about
+ *          11 bits per activation, inside the 1e-2 bar on the sum but not the reference's f32 product; a caller that
+ *          needs the f32 product of many rows calls in blocks of 32 rows ("prefill_min_m").
+ * Uses the context's scratch: one context must not run two calls at the same time. */
 int twm_gemm(twm_ctx *ctx, const twm_weight *w, const void *a_dev, int a_dtype, uint32_t m,
              float *c_dev, uint32_t splits);
 /* Fused projection with the split folded into the store: column ranges of the fused

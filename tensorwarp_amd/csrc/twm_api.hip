@@ -560,9 +560,10 @@ static M1Form choose_m1_form(int exact, int force_sub, int force_waves, int forc
         if (n_pad / sub > n_counters) sp = 1;
         return M1Form{kM1SubTile, sub, sub_waves, sp};
     }
-    // (only matrices of 256 tiles or more on a deep K get here, or option "sub" = 1: eight waves, no K-split of its own)
+    // (only matrices of 256 tiles or more on a deep K get here, or option "sub" = 1: no K-split of its own; sixteen
+    // waves where there are fewer tiles than CUs)
     f.kind = kM1WholeTile;
-    f.waves = 8;
+    f.waves = tiles64 < 256 ? 16 : 8;
     if (force_waves) f.waves = (uint32_t)force_waves;
     if (force_splits) f.splits = (uint32_t)force_splits;
     if (f.splits > k_chunks) f.splits = k_chunks;

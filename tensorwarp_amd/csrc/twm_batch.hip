@@ -313,7 +313,10 @@ __global__ __launch_bounds__(64 * WPS * KS) void k_batch(const uint4v *__restric
 #pragma unroll
                 for (int r = 0; r < 4; r++) {
                     const uint32_t row = 16u * mt + 4u * kb + r;
-                    if (row < m_rows) out.swiglu[(size_t)row * ffn + feat] = gated_mul(out.gate_act, acc[mt][0][r], acc[mt][1][r]);
+                    if (row < m_rows) {
+                        const float rs = out.row_scale ? out.row_scale[row] : 1.f;  // (f32 rows scaled into the f16 range)
+                        out.swiglu[(size_t)row * ffn + feat] = gated_mul(out.gate_act, acc[mt][0][r] * rs, acc[mt][1][r] * rs);
+                    }
                 }
             return;
         }
@@ -335,7 +338,10 @@ __global__ __launch_bounds__(64 * WPS * KS) void k_batch(const uint4v *__restric
 #pragma unroll
                 for (int r = 0; r < 4; r++) {
                     const uint32_t row = 16u * mt + 4u * kb + r;
-                    if (row < m_rows) out.seg[sg].ptr[(size_t)row * out.seg[sg].width + rel] = has_b ? acc[mt][i][r] + b : acc[mt][i][r];
+                    if (row < m_rows) {
+                        const float v = out.row_scale ? acc[mt][i][r] * out.row_scale[row] : acc[mt][i][r];
+                        out.seg[sg].ptr[(size_t)row * out.seg[sg].width + rel] = has_b ? v + b : v;
+                    }
                 }
         }
     }
@@ -389,7 +395,7 @@ static hipError_t launch_batch_slices(hipStream_t s, const WeightView &w, const 
 // otherwise the exact per-group f32 scaling.  tiles_per_wave: 1 or 2 (a gated store without split-K needs 2).  `scratch` holds, for f32 activations,
 // their two f16 terms (2 x M x K halves) and after them the split-K partials (splits x M x (n_tiles * 16) floats);
 // the split factor is cut to what fits.
-hipError_t launch_batch(hipStream_t s, const WeightView &w, const void *a, bool a_f32, uint32_t m, const OutSpec &out,
+hipError_t launch_batch(hipStream_t s, const WeightView &w, const void *a, bool a_f32, uint32_t m, const OutSpec &out_in,
                         uint32_t splits, uint32_t tiles_per_wave, uint32_t k_slices, uint32_t quads_per_group,
                         bool rounded, float *scratch, size_t scratch_bytes)
 {
@@ -401,16 +407,20 @@ hipError_t launch_batch(hipStream_t s, const WeightView &w, const void *a, bool 
     float *partials = scratch;
     size_t partial_bytes = scratch ? scratch_bytes : 0;
     uint32_t lo_offset = 0;
+    OutSpec out = out_in;
     if (a_f32) {
+        // the rows' power-of-two factors (256 bytes), their two f16 terms, then the partial sums
         size_t term_bytes = (((size_t)m * w.k * 2) + 255) & ~(size_t)255;
-        if (!scratch || scratch_bytes < 2 * term_bytes || term_bytes > 0x7FFFFFFFu) return hipErrorInvalidValue;
-        _Float16 *hi = (_Float16 *)scratch, *lo = (_Float16 *)((char *)scratch + term_bytes);
-        hipError_t e = launch_split_hi_lo(s, (const float *)a, hi, lo, (size_t)m * w.k);
+        if (!scratch || scratch_bytes < 256 + 2 * term_bytes || term_bytes > 0x7FFFFFFFu) return hipErrorInvalidValue;
+        float *row_scale = scratch;
+        _Float16 *hi = (_Float16 *)((char *)scratch + 256), *lo = (_Float16 *)((char *)scratch + 256 + term_bytes);
+        hipError_t e = launch_f32_rows_to_f16(s, (const float *)a, hi, lo, row_scale, m, w.k);
         if (e != hipSuccess) return e;
         a = hi;
+        out.row_scale = row_scale;
         lo_offset = (uint32_t)term_bytes;
-        partials = (float *)((char *)scratch + 2 * term_bytes);
-        partial_bytes = scratch_bytes - 2 * term_bytes;
+        partials = (float *)((char *)scratch + 256 + 2 * term_bytes);
+        partial_bytes = scratch_bytes - 256 - 2 * term_bytes;
     }
     if (splits < 1) splits = 1;
     size_t per_split = (size_t)m * w.n_tiles * 16 * 4;

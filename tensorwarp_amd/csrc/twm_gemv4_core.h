@@ -77,8 +77,9 @@ __device__ __forceinline__ void split_f32x8(const float (&v)[8], uint4v &hi, uin
 // Lanes with the same lane % 4 hold the same activation row (one row of the MFMA's A operand); when any value of
 // the wave exceeds the largest f16, every such row scales its values by a power of two of its own that brings its
 // largest below 2^15 (exact), and inv[i] is what the sums of A row i are multiplied by afterwards (exact as well): the
-// results come out as with unbounded terms.  In range every factor is 1 and nothing is touched, at the price of a
-// maximum over the lane's values and one vote per call.  (Infinities and NaNs stay what they are.)
+// results come out as with unbounded terms.  A row whose values in the wave are all below 2^-6 is scaled up the same
+// way, so that its residual terms do not fall into the f16 subnormals.  In range every factor is 1 and nothing is
+// touched, at the price of a maximum over the lane's values and one vote per call.  (Infinities and NaNs stay what they are.)
 // ONE_ROW: every lane of the wave holds values of the same activation row: one factor for the wave.
 template <int NV, bool ONE_ROW = false>
 __device__ __forceinline__ void f32_terms_range(float (&v)[NV], float (&inv)[4])
@@ -88,13 +89,15 @@ __device__ __forceinline__ void f32_terms_range(float (&v)[NV], float (&inv)[4])
     for (int i = 0; i < NV; i++) m = fmaxf(m, fabsf(v[i]));
 #pragma unroll
     for (int i = 0; i < 4; i++) inv[i] = 1.f;
-    if (__builtin_amdgcn_ballot_w64(!(m <= 65000.f)) == 0) return;
+    // (a lane whose values are all small, below 2^-6, votes too: when that holds for the row's whole stretch, the residual
+    // terms, 2^-11 of their values, would fall into the f16 subnormals (below 2^-14), and the stretch is scaled up instead)
+    if (__builtin_amdgcn_ballot_w64(!(m <= 65000.f) || (m < 0.015625f && m > 0.f)) == 0) return;
     if (!(m == m)) m = __builtin_inff();  // (fmaxf drops a NaN; the vote saw it through the negated comparison)
 #pragma unroll
     for (int off = 32; off >= (ONE_ROW ? 1 : 4); off >>= 1) m = fmaxf(m, __shfl_xor(m, off, 64));   // over the lanes of this row
     float mine = 1.f;
-    if (m > 16384.f) {
-        const uint32_t e = (__float_as_uint(m) >> 23) & 0xFFu;       // biased exponent of the row's largest value, >= 141
+    if (m > 16384.f || (m < 0.015625f && m >= 1e-30f)) {
+        const uint32_t e = (__float_as_uint(m) >> 23) & 0xFFu;       // biased exponent of the row's largest value
         const float down = __uint_as_float((254u + 14u - e) << 23);   // 2^(14 - (e - 127))
 #pragma unroll
         for (int i = 0; i < NV; i++) v[i] *= down;

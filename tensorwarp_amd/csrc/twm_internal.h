@@ -41,6 +41,10 @@ struct OutSpec {
     // swiglu[row][n / 2] instead of the n columns to the segments.
     float *swiglu;
     uint32_t gate_act;  // 1 = gelu_tanh(gate) * up (GEGLU), otherwise silu(gate) * up
+    // f32 activations at M >= 5: row r of the activations was scaled by a power of two to sit inside the f16 range
+    // (launch_f32_rows_to_f16), and every sum of row r is multiplied by row_scale[r] before bias, gate and store
+    // (exact; 1 for a row that needed nothing).  Null: no scaling.
+    const float *row_scale;
 };
 
 // feature index of internal column `col` of a paired weight (col % 64 < 32: the gate column; + 32: its up column)
@@ -164,7 +168,11 @@ hipError_t launch_splitk_reduce(hipStream_t s, const float *partials, const OutS
 hipError_t launch_stream(hipStream_t s, const WeightView &w, const void *a, bool a_f32, uint32_t m, const OutSpec &out,
                          uint32_t splits, uint32_t waves, float *partials, size_t partial_bytes);
 // f32 -> two f16 arrays: hi = f16(a), lo = f16(a - hi)
-hipError_t launch_split_hi_lo(hipStream_t s, const float *a, _Float16 *hi, _Float16 *lo, size_t count);
+// f32 activation rows -> f16: hi = f16(a * 2^-s), lo = f16(a * 2^-s - hi) (lo null: the one rounded term only), with a
+// power of two per row that brings the row's largest magnitude to [2^13, 2^14) when it lies outside [2^-2, 2^14], and
+// row_scale[row] = 2^s for the stores (1 otherwise; a row of zeros, infinities or NaNs is left as it is).
+hipError_t launch_f32_rows_to_f16(hipStream_t s, const float *a, _Float16 *hi, _Float16 *lo, float *row_scale, uint32_t rows,
+                                  uint32_t k);
 // batched decode with the activations shared through LDS (M <= 32); tiles_per_wave 1 or 2, k_slices 1, 2 or 4
 hipError_t launch_batch(hipStream_t s, const WeightView &w, const void *a, bool a_f32, uint32_t m, const OutSpec &out,
                         uint32_t splits, uint32_t tiles_per_wave, uint32_t k_slices, uint32_t quads_per_group,

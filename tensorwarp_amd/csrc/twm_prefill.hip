@@ -289,10 +289,12 @@ __global__ __launch_bounds__(256) TWM_PF_OCC(HALF) void k_prefill(const uint4v *
 #pragma unroll
             for (int i = 0; i < 4; i++) {
                 const uint32_t row = (lane >> 4) + 4u * i;
-                const float4v v = *(const float4v *)(stage + row * 68 + (lane & 15u) * 4u);
+                float4v v = *(const float4v *)(stage + row * 68 + (lane & 15u) * 4u);
                 const uint32_t om = m0 + mt * 16u + row;
-                if (om < m_rows && col < n_lim && (lane & 15u) * 4u < 16u * NTW)
+                if (om < m_rows && col < n_lim && (lane & 15u) * 4u < 16u * NTW) {
+                    if (out.row_scale && !partials) v *= out.row_scale[om];  // (f32 rows scaled into the f16 range)
                     __builtin_nontemporal_store(v, (float4v *)(dst + (size_t)om * ld + col));
+                }
             }
         }
         return;
@@ -329,8 +331,11 @@ __global__ __launch_bounds__(256) TWM_PF_OCC(HALF) void k_prefill(const uint4v *
 #pragma unroll
             for (int t = 0; t < 2; t++)
 #pragma unroll
-                for (int r = 0; r < 4; r++)
-                    stage[(kb * 4 + r) * 36 + t * 16 + c] = gated_mul(out.gate_act, acc[mt][t][r], acc[mt][(t + 2) % NTW][r]);
+                for (int r = 0; r < 4; r++) {
+                    const uint32_t om = m0 + mt * 16u + kb * 4u + r;
+                    const float rs = out.row_scale && om < m_rows ? out.row_scale[om] : 1.f;
+                    stage[(kb * 4 + r) * 36 + t * 16 + c] = gated_mul(out.gate_act, acc[mt][t][r] * rs, acc[mt][(t + 2) % NTW][r] * rs);
+                }
 #pragma unroll
             for (int i = 0; i < 2; i++) {
                 const uint32_t row = (lane >> 3) + 8u * i;
@@ -358,7 +363,7 @@ __global__ __launch_bounds__(256) TWM_PF_OCC(HALF) void k_prefill(const uint4v *
 #pragma unroll
             for (int r = 0; r < 4; r++) {
                 uint32_t om = m0 + mt * 16u + kb * 4u + r;
-                if (om < m_rows) pf_store_out(out, om, on, acc[mt][t][r]);
+                if (om < m_rows) pf_store_out(out, om, on, out.row_scale ? acc[mt][t][r] * out.row_scale[om] : acc[mt][t][r]);
             }
     }
 }
@@ -378,6 +383,10 @@ __global__ __launch_bounds__(256) void k_splitk_reduce(const float *__restrict__
         float4 v = src[z * stride4];
         s.x += v.x; s.y += v.y; s.z += v.z; s.w += v.w;
     }
+    if (out.row_scale) {
+        const float rs = out.row_scale[row];  // (f32 rows scaled into the f16 range)
+        s.x *= rs; s.y *= rs; s.z *= rs; s.w *= rs;
+    }
     if (col + 0 < n) pf_store_out(out, row, col + 0, s.x);
     if (col + 1 < n) pf_store_out(out, row, col + 1, s.y);
     if (col + 2 < n) pf_store_out(out, row, col + 2, s.z);
@@ -388,7 +397,7 @@ __global__ __launch_bounds__(256) void k_splitk_reduce(const float *__restrict__
 // (32 columns apart) in split order and stores silu(gate) * up.
 __global__ __launch_bounds__(256) void k_splitk_reduce_swiglu(const float *__restrict__ partials, float *__restrict__ gate_out,
                                                                 uint32_t m_rows, uint32_t ffn, uint32_t n_ld, uint32_t splits,
-                                                                uint32_t act)
+                                                                uint32_t act, const float *__restrict__ row_scale)
 {
     size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
     uint32_t quads = ffn / 4;  // ffn is a multiple of 32
@@ -403,20 +412,10 @@ __global__ __launch_bounds__(256) void k_splitk_reduce_swiglu(const float *__res
         g.x += v.x; g.y += v.y; g.z += v.z; g.w += v.w;
         u.x += w.x; u.y += w.y; u.z += w.z; u.w += w.w;
     }
-    float4 o = {gated_mul(act, g.x, u.x), gated_mul(act, g.y, u.y), gated_mul(act, g.z, u.z), gated_mul(act, g.w, u.w)};
+    const float rs = row_scale ? row_scale[row] : 1.f;  // (f32 rows scaled into the f16 range)
+    float4 o = {gated_mul(act, g.x * rs, u.x * rs), gated_mul(act, g.y * rs, u.y * rs), gated_mul(act, g.z * rs, u.z * rs),
+                gated_mul(act, g.w * rs, u.w * rs)};
     *(float4 *)(gate_out + (size_t)row * ffn + feat) = o;
-}
-
-// f32 activations are rounded to f16 (round-to-nearest-even, as the MFMA operand needs) into scratch first
-__global__ __launch_bounds__(256) void k_cvt_f32_f16(const float4 *__restrict__ src, uint2v *__restrict__ dst, size_t n4)
-{
-    size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
-    if (i >= n4) return;
-    float4 x = src[i];
-    union { half2v h[2]; uint2v u; } cv;
-    cv.h[0] = half2v{(_Float16)x.x, (_Float16)x.y};
-    cv.h[1] = half2v{(_Float16)x.z, (_Float16)x.w};
-    dst[i] = cv.u;
 }
 
 hipError_t launch_splitk_reduce(hipStream_t s, const float *partials, const OutSpec &out, uint32_t m, uint32_t n,
@@ -428,7 +427,7 @@ hipError_t launch_splitk_reduce(hipStream_t s, const float *partials, const OutS
         if (n % (2 * kPairWidth) != 0) return hipErrorInvalidValue;
         size_t fq = (size_t)m * (n / 2) / 4;
         hipLaunchKernelGGL(k_splitk_reduce_swiglu, dim3((unsigned)((fq + 255) / 256)), dim3(256), 0, s, partials, out.swiglu, m,
-                           n / 2, n_ld, splits, out.gate_act);
+                           n / 2, n_ld, splits, out.gate_act, out.row_scale);
         return hipGetLastError();
     }
     hipLaunchKernelGGL(k_splitk_reduce, dim3((unsigned)((quads + 255) / 256)), dim3(256), 0, s, partials, out, m, n, n_ld,
@@ -590,22 +589,25 @@ hipError_t launch_prefill(hipStream_t s, const WeightView &w, const void *a, boo
         return launch_prefill_t<8>(s, w, a16, rows, o, plan.splits, (float *)ws);
     };
     if (!a_f32) return run((const _Float16 *)a, m, out, scratch, scratch_bytes);
-    // f16 copy of the activations at the front of the scratch, partials behind it
-    size_t row_bytes = (size_t)w.k * 2;
-    if (!scratch || scratch_bytes < row_bytes) return hipErrorInvalidValue;
-    uint32_t slab = (uint32_t)(scratch_bytes / 2 / row_bytes < m ? scratch_bytes / 2 / row_bytes : m);
+    // f16 copy of the activations (each row scaled by a power of two where it would leave the f16 range, the factors in
+    // front of the copy) at the front of the scratch, partials behind it
+    size_t row_bytes = (size_t)w.k * 2 + 4;
+    if (!scratch || scratch_bytes < row_bytes + 512) return hipErrorInvalidValue;
+    uint32_t slab = (uint32_t)((scratch_bytes - 512) / 2 / row_bytes < m ? (scratch_bytes - 512) / 2 / row_bytes : m);
     if (slab == 0) slab = 1;
     if (slab >= 128) slab -= slab % 128;
     for (uint32_t r0 = 0; r0 < m; r0 += slab) {
         uint32_t rows = m - r0 < slab ? m - r0 : slab;
-        size_t n4 = (size_t)rows * w.k / 4;  // k is a multiple of 32
-        hipLaunchKernelGGL(k_cvt_f32_f16, dim3((unsigned)((n4 + 255) / 256)), dim3(256), 0, s,
-                           (const float4 *)((const float *)a + (size_t)r0 * w.k), (uint2v *)scratch, n4);
+        float *row_scale = (float *)scratch;
+        _Float16 *a16 = (_Float16 *)((char *)scratch + (((size_t)rows * 4 + 255) & ~(size_t)255));
+        hipError_t ce = launch_f32_rows_to_f16(s, (const float *)a + (size_t)r0 * w.k, a16, nullptr, row_scale, rows, w.k);
+        if (ce != hipSuccess) return ce;
         OutSpec o = out;
+        o.row_scale = row_scale;
         for (uint32_t i = 0; i < o.count; i++) o.seg[i].ptr += (size_t)r0 * o.seg[i].width;
         if (o.swiglu) o.swiglu += (size_t)r0 * (w.n / 2);
-        size_t used = ((size_t)rows * row_bytes + 255) & ~(size_t)255;
-        hipError_t e = run((const _Float16 *)scratch, rows, o, (char *)scratch + used, scratch_bytes - used);
+        size_t used = (size_t)((char *)a16 - (char *)scratch) + (((size_t)rows * w.k * 2 + 255) & ~(size_t)255);
+        hipError_t e = run(a16, rows, o, (char *)scratch + used, scratch_bytes - used);
         if (e != hipSuccess) return e;
     }
     return hipGetLastError();

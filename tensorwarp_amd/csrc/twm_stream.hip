@@ -217,6 +217,8 @@ __global__ __launch_bounds__(WAVES * 64) void k_stream(const uint4v *__restrict_
 #pragma unroll
         for (int w = 1; w < WAVES; w++) s += red[w][reg][src_lane];
         if (row >= m_rows) continue;
+        const float rs = out.row_scale && !partials ? out.row_scale[row] : 1.f;  // (f32 rows scaled into the f16 range)
+        s *= rs;
         if (partials) {
             partials[((size_t)blockIdx.y * m_rows + row) * n_ld + on] = s;
         } else if (out.swiglu) {
@@ -227,7 +229,7 @@ __global__ __launch_bounds__(WAVES * 64) void k_stream(const uint4v *__restrict_
 #pragma unroll
                 for (int w = 1; w < WAVES; w++) u += red[w][reg + 8][src_lane];
                 const uint32_t ffn = n >> 1, feat = paired_feature(on);
-                if (feat < ffn) out.swiglu[(size_t)row * ffn + feat] = gated_mul(out.gate_act, s, u);
+                if (feat < ffn) out.swiglu[(size_t)row * ffn + feat] = gated_mul(out.gate_act, s, u * rs);
             }
         } else if (on < n) {
 #pragma unroll
@@ -241,22 +243,54 @@ __global__ __launch_bounds__(WAVES * 64) void k_stream(const uint4v *__restrict_
     }
 }
 
-// f32 activations -> two f16 arrays: hi = f16(a), lo = f16(a - hi) (the subtraction is exact)
-__global__ __launch_bounds__(256) void k_split_f32_hi_lo(const float *__restrict__ a, _Float16 *__restrict__ hi,
-                                                          _Float16 *__restrict__ lo, size_t count)
+// f32 activations -> f16 terms, a workgroup per row: hi = f16(x), lo = f16(x - hi) (the subtraction is exact) of
+// x = a * 2^-s, where s brings the row's largest magnitude to [2^13, 2^14) when it lies outside [2^-2, 2^14] (any finite
+// f32 row keeps about 21 bits per value relative to the row's largest, as the reference's f32 product would; in range
+// s = 0 and nothing changes), and row_scale[row] = 2^s, which the GEMM's store multiplies the row's sums by (exact).
+// TWO = false: the one rounded term only (the prefill GEMM's operand).
+template <bool TWO>
+__global__ __launch_bounds__(1024) void k_f32_rows_to_f16(const float *__restrict__ a, _Float16 *__restrict__ hi,
+                                                           _Float16 *__restrict__ lo, float *__restrict__ row_scale, uint32_t k)
 {
-    size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
-    if (i >= count) return;
-    float v = a[i];
-    _Float16 h = (_Float16)v;
-    hi[i] = h;
-    lo[i] = (_Float16)(v - (float)h);
+    __shared__ float s_max[16];
+    const float *src = a + (size_t)blockIdx.x * k;
+    float m = 0.f;
+    bool odd = false;  // an infinity or a NaN in the row
+    for (uint32_t i = threadIdx.x; i < k; i += 1024u) {
+        const float v = fabsf(src[i]);
+        odd = odd || !(v <= 3.4028234e38f);
+        m = fmaxf(m, v);
+    }
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) m = fmaxf(m, __shfl_xor(m, off, 64));
+    if (__builtin_amdgcn_ballot_w64(odd) != 0) m = __builtin_inff();
+    if ((threadIdx.x & 63u) == 0) s_max[threadIdx.x >> 6] = m;
+    __syncthreads();
+    m = s_max[0];
+#pragma unroll
+    for (int w = 1; w < 16; w++) m = fmaxf(m, s_max[w]);
+    float down = 1.f, back = 1.f;
+    const uint32_t e = (__float_as_uint(m) >> 23) & 0xFFu;   // biased exponent of the row's largest magnitude
+    if (e != 0xFFu && e >= 16u && (m > 16384.f || m < 0.25f)) {
+        down = __uint_as_float((254u + 13u - e) << 23);       // 2^(13 - (e - 127))
+        back = __uint_as_float((e - 13u) << 23);              // 2^((e - 127) - 13)
+    }
+    if (threadIdx.x == 0) row_scale[blockIdx.x] = back;
+    _Float16 *dh = hi + (size_t)blockIdx.x * k, *dl = TWO ? lo + (size_t)blockIdx.x * k : nullptr;
+    for (uint32_t i = threadIdx.x; i < k; i += 1024u) {
+        const float v = src[i] * down;
+        const _Float16 h = (_Float16)v;
+        dh[i] = h;
+        if (TWO) dl[i] = (_Float16)(v - (float)h);
+    }
 }
 
-hipError_t launch_split_hi_lo(hipStream_t s, const float *a, _Float16 *hi, _Float16 *lo, size_t count)
+hipError_t launch_f32_rows_to_f16(hipStream_t s, const float *a, _Float16 *hi, _Float16 *lo, float *row_scale, uint32_t rows,
+                                  uint32_t k)
 {
-    if (count == 0) return hipSuccess;
-    hipLaunchKernelGGL(k_split_f32_hi_lo, dim3((unsigned)((count + 255) / 256)), dim3(256), 0, s, a, hi, lo, count);
+    if (rows == 0 || k == 0) return hipSuccess;
+    if (lo) hipLaunchKernelGGL(k_f32_rows_to_f16<true>, dim3(rows), dim3(1024), 0, s, a, hi, lo, row_scale, k);
+    else hipLaunchKernelGGL(k_f32_rows_to_f16<false>, dim3(rows), dim3(1024), 0, s, a, hi, lo, row_scale, k);
     return hipGetLastError();
 }
 
@@ -278,7 +312,7 @@ static hipError_t launch_stream_t(hipStream_t s, const WeightView &w, const void
 
 // M <= 32.  `scratch` holds, for f32 activations, their two f16 terms (2 x M x K halves) and after them the
 // split-K partials (splits x M x (n_tiles * 16) floats); the split factor is cut to what fits.
-hipError_t launch_stream(hipStream_t s, const WeightView &w, const void *a, bool a_f32, uint32_t m, const OutSpec &out,
+hipError_t launch_stream(hipStream_t s, const WeightView &w, const void *a, bool a_f32, uint32_t m, const OutSpec &out_in,
                          uint32_t splits, uint32_t waves, float *scratch, size_t scratch_bytes)
 {
     if (m == 0 || w.n == 0) return hipSuccess;
@@ -287,16 +321,20 @@ hipError_t launch_stream(hipStream_t s, const WeightView &w, const void *a, bool
     float *partials = scratch;
     size_t partial_bytes = scratch ? scratch_bytes : 0;
     uint32_t lo_offset = 0;
+    OutSpec out = out_in;
     if (a_f32) {
+        // the rows' power-of-two factors (256 bytes), their two f16 terms, then the partial sums
         size_t term_bytes = (((size_t)m * w.k * 2) + 255) & ~(size_t)255;
-        if (!scratch || scratch_bytes < 2 * term_bytes || term_bytes > 0x7FFFFFFFu) return hipErrorInvalidValue;
-        _Float16 *hi = (_Float16 *)scratch, *lo = (_Float16 *)((char *)scratch + term_bytes);
-        hipError_t e = launch_split_hi_lo(s, (const float *)a, hi, lo, (size_t)m * w.k);
+        if (!scratch || scratch_bytes < 256 + 2 * term_bytes || term_bytes > 0x7FFFFFFFu) return hipErrorInvalidValue;
+        float *row_scale = scratch;
+        _Float16 *hi = (_Float16 *)((char *)scratch + 256), *lo = (_Float16 *)((char *)scratch + 256 + term_bytes);
+        hipError_t e = launch_f32_rows_to_f16(s, (const float *)a, hi, lo, row_scale, m, w.k);
         if (e != hipSuccess) return e;
         a = hi;
+        out.row_scale = row_scale;
         lo_offset = (uint32_t)term_bytes;
-        partials = (float *)((char *)scratch + 2 * term_bytes);
-        partial_bytes = scratch_bytes - 2 * term_bytes;
+        partials = (float *)((char *)scratch + 256 + 2 * term_bytes);
+        partial_bytes = scratch_bytes - 256 - 2 * term_bytes;
     }
     if (splits < 1) splits = 1;
     size_t per_split = (size_t)m * w.n_tiles * 16 * 4;

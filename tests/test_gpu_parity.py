@@ -443,6 +443,104 @@ def test_f32_activations_beyond_the_f16_range(dev, k, n):
     w.free()
 
 
+@pytest.mark.parametrize("k,n", [(3584, 608), (1184, 200)])
+def test_f32_rows_of_any_size_from_five_rows_on(dev, k, n):
+    # The reference's only quantized GEMM for M > 1 takes `const float *A` and multiplies in f32 (quantize.rs:186-246,
+    # 1825-1858), so any finite f32 row is a valid input.  From five rows on the activations are converted once per
+    # launch, a workgroup per row, with a power of two per row that keeps the row inside the f16 range (and a tiny row
+    # out of the subnormals); the store multiplies the row's sums back.  Rows of 1e6, of 1e30, of 1e-6 and of 1e-30 next
+    # to ordinary ones, a single huge entry among ordinary ones, at 8 and 32 rows (both batched-decode kernels, both
+    # row-block heights) against the exact-weight f64 product; and at 64 rows (the prefill GEMM, which rounds the scaled
+    # activations to one f16 term: values that are f16 numbers times a power of two, so that the rounding is exact)
+    # against the f64 product on the FP16 Q4 unpack.  The gated store scales before the gate.
+    packed, scales, _ = synth(k, n, 1, 9800 + k)
+    w = T.MarlinWeight.upload(dev, packed, scales, k, n)
+    factors = [2.5e5, 1.0, 1.0e30, 1.0e-6, 1.0, 1.0e-30, 3.0, 7.0e4]
+    for m in (8, 32):
+        rows = O.synth_normal_f32(m * k, 9900 + m).reshape(m, k).copy()
+        for r in range(m):
+            rows[r] *= np.float32(factors[r % len(factors)])
+        rows[4, 5::97] *= np.float32(3.0e5)              # a few huge entries among ordinary ones
+        truth = O.gemm_f64(rows, packed, scales, m, k, n)
+        for splits in (0, 3):
+            c = T.GpuTensor.from_host(dev, np.full((m, n), np.nan, np.float32))
+            T.gemm(dev, w, T.GpuTensor.from_host(dev, np.ascontiguousarray(rows)), m, c, splits)
+            got = c.to_host()
+            assert np.isfinite(got).all(), (m, splits)
+            for r in range(m):   # (row by row: the rows differ by sixty orders of magnitude)
+                assert rel_err(got[r], truth[r]) < TIGHT, (m, splits, r)
+    m = 64
+    a16 = O.synth_act_f16(m, k, 9950)
+    rows = f16_as_f32(a16).reshape(m, k).copy()
+    pow2 = [2.0 ** 18, 1.0, 2.0 ** 100, 2.0 ** -20, 1.0, 2.0 ** -100, 2.0, 2.0 ** 17]
+    for r in range(m):
+        rows[r] *= np.float32(pow2[r % len(pow2)])
+    w16 = O.dequant_f16(packed, scales, k, n).view(np.float16).astype(np.float64).reshape(k, n)
+    truth = rows.astype(np.float64) @ w16
+    for splits in (0, 2):
+        c = T.GpuTensor.from_host(dev, np.full((m, n), np.nan, np.float32))
+        T.gemm(dev, w, T.GpuTensor.from_host(dev, np.ascontiguousarray(rows)), m, c, splits)
+        got = c.to_host()
+        assert np.isfinite(got).all(), splits
+        for r in range(m):   # (the prefill GEMM's bar: f32 sums over all of K inside the MFMAs)
+            assert rel_err(got[r], truth[r]) < 1e-3, (splits, r)
+    w.free()
+
+
+@pytest.mark.parametrize("m", [8, 32, 64])
+def test_f32_rows_of_any_size_through_the_gated_store(dev, m):
+    h, ffn = 640, 224
+    gp, gs = O.synth_packed(h, ffn, 1300), O.synth_scales(h, ffn, 1301)
+    up, us = O.synth_packed(h, ffn, 1302), O.synth_scales(h, ffn, 1303)
+    gd = (T.GpuTensor.from_host(dev, gp), T.GpuTensor.from_host(dev, gs, "f16"))
+    ud = (T.GpuTensor.from_host(dev, up), T.GpuTensor.from_host(dev, us, "f16"))
+    w = T.MarlinWeight.gate_up(dev, gd, ud, h, ffn)
+    rows = f16_as_f32(O.synth_act_f16(m, h, 1304)).reshape(m, h).copy()
+    for r in range(m):
+        rows[r] *= np.float32([2.0 ** 17, 1.0, 2.0 ** -18, 2.0 ** 16][r % 4]) * np.float32(0.02)
+    ad = T.GpuTensor.from_host(dev, np.ascontiguousarray(rows))
+    for splits in (0, 2):
+        out = T.GpuTensor.from_host(dev, np.full((m, ffn), np.nan, np.float32))
+        T.gemm_swiglu(dev, w, ad, m, out, splits)
+        tmp = T.GpuTensor.zeros(dev, (m, 2 * ffn), "f32")
+        T.gemm(dev, w, ad, m, tmp, splits)
+        seq = T.GpuTensor.zeros(dev, (m, ffn), "f32")
+        T.swiglu_rows(dev, tmp, seq, ffn, m, paired=True)
+        got, want = out.to_host(), seq.to_host()
+        assert np.isfinite(got).all()
+        # (the fused and the two-step launch may run different plans; each row against the other at the bar of one ulp of
+        # exp, relative to the row's largest value)
+        for r in range(m):
+            assert np.abs(got[r] - want[r]).max() <= 1e-5 * np.abs(want[r]).max(), (m, splits, r)
+    w.free()
+
+
+@pytest.mark.parametrize("k,n", [(3584, 608), (18944, 192), (1184, 200)])
+def test_f32_rows_of_tiny_magnitude(dev, k, n):
+    # Rows whose values are all far below the f16 normal range (scaled by 1e-6, 1e-20): the residual term of the two-term
+    # form would fall into the f16 subnormals and the result would keep a few bits; the kernels scale such a stretch up
+    # by a power of two first.  The drop-in entry and twm_gemm at one to four rows.
+    packed, scales, _ = synth(k, n, 1, 8700 + k)
+    pd, sd = T.GpuTensor.from_host(dev, packed), T.GpuTensor.from_host(dev, scales, "f16")
+    w = T.MarlinWeight.from_device(dev, pd, sd, k, n)
+    base = O.synth_normal_f32(4 * k, 8750 + k).reshape(4, k)
+    for scale in (1.0e-6, 1.0e-20):
+        rows = np.ascontiguousarray(base * np.float32(scale))
+        rows[3] = base[3]                                     # an ordinary row beside them
+        rows[2, ::2] = base[2, ::2] * np.float32(1.0e-3)      # tiny and small values mixed
+        truth = O.gemm_f64(rows, packed, scales, 4, k, n)
+        c = T.GpuTensor.zeros(dev, (n,), "f32")
+        for r in range(4):
+            T.gemm_tw_marlin_m1(dev, T.GpuTensor.from_host(dev, np.ascontiguousarray(rows[r])), pd, sd, c, n, k)
+            assert rel_err(c.to_host(), truth[r]) < TIGHT, (scale, r)
+        for m in (1, 2, 4):
+            cm = T.GpuTensor.zeros(dev, (m, n), "f32")
+            T.gemm(dev, w, T.GpuTensor.from_host(dev, np.ascontiguousarray(rows[:m])), m, cm)
+            for r in range(m):
+                assert rel_err(cm.to_host()[r], truth[r]) < TIGHT, (scale, m, r)
+    w.free()
+
+
 def test_gemm_tw_marlin_m1_from_buffer_and_errors(dev):
     k, n = 128, 64
     packed, scales, a16 = synth(k, n, 1, 9)
