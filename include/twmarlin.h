@@ -65,6 +65,21 @@ const char *twm_version(void);
 int twm_device_count(void);
 /* Text of the last failure on the calling thread ("" if none). */
 const char *twm_last_error(void);
+/* Which DeviceError variant of the reference (device.rs:278-292: Init, PtxLoad, FuncNotFound, Sync, Memory, Launch) the
+ * last failure on the calling thread corresponds to, for a wrapper that maps codes back to that enum: a failed
+ * context creation is Init (a device that is not gfx950, for which the library holds no code object, is PtxLoad),
+ * a failed synchronise Sync, a failed allocation or copy Memory, everything else that reached the device Launch;
+ * argument errors (shape, handle, unsupported) never reached the device and are TWM_KIND_NONE. */
+enum {
+    TWM_KIND_NONE = 0,
+    TWM_KIND_INIT = 1,
+    TWM_KIND_CODE_OBJECT = 2,    /* DeviceError::PtxLoad */
+    TWM_KIND_FUNC_NOT_FOUND = 3, /* (never raised: kernels are linked into the library) */
+    TWM_KIND_SYNC = 4,
+    TWM_KIND_MEMORY = 5,
+    TWM_KIND_LAUNCH = 6
+};
+int twm_last_error_kind(void);
 
 /* c_api.rs:52-59 warp_device_create / WarpDevice::new (device.rs) + KernelCache::new.
  * All kernels are precompiled gfx950 code inside the library, so there is no
@@ -81,6 +96,13 @@ int twm_ctx_sync(twm_ctx *ctx);
 int twm_ctx_set_stream(twm_ctx *ctx, void *hip_stream);
 /* The hipStream_t work is currently issued on. */
 void *twm_ctx_stream(twm_ctx *ctx);
+/* Stream objects for a caller that has none of its own (the reference creates its streams through the driver crate,
+ * device.rs:230-265): a non-blocking hipStream_t at the default priority on the context's device, to be handed to
+ * twm_ctx_set_stream; destroy it only after the context has been pointed elsewhere.  twm_stream_sync blocks until the
+ * stream's work is done (a failure reports TWM_KIND_SYNC). */
+void *twm_stream_create(twm_ctx *ctx);
+int twm_stream_destroy(twm_ctx *ctx, void *hip_stream);
+int twm_stream_sync(twm_ctx *ctx, void *hip_stream);
 /* c_api.rs:69-80 warp_device_info: fills buf with "<name> | <CUs> CUs | <GiB> GiB". */
 int twm_ctx_info(twm_ctx *ctx, char *buf, size_t buf_len);
 /* Tuning knobs for per-shape sweeps (the role AutoTuner::tune_gemm plays in
@@ -108,8 +130,9 @@ int twm_ctx_info(twm_ctx *ctx, char *buf, size_t buf_len);
  * Values outside these sets return TWM_SHAPE_ERROR, unknown keys TWM_UNSUPPORTED_OP. */
 int twm_ctx_set_option(twm_ctx *ctx, const char *key, int value);
 
-/* Profiling aid, no counterpart in the reference: while trace_dev is set (process-wide), every launch of the M = 1
- * sub-tile GEMV kernel (f16 activations) with at most capacity_workgroups workgroups runs a traced twin of the kernel,
+/* Profiling aid, no counterpart in the reference: while trace_dev is set on a context, every launch of the M = 1
+ * sub-tile GEMV kernel (f16 activations) that this context issues with at most capacity_workgroups workgroups runs a
+ * traced twin of the kernel (other contexts are not affected),
  * in which workgroup b writes four 32-bit words at trace_dev[4 b]: the GPU's 100 MHz clock at its start, after its
  * first wave has unpacked its weights, and at its end, and the hardware id of the CU it ran on (bits 0-15 HW_ID, bits
  * 16-19 the XCD).  NULL or 0 switches it off; the product kernels carry no trace code. */
@@ -160,6 +183,12 @@ int twm_dequant_to_f16(twm_ctx *ctx, const uint8_t *packed_dev, const uint16_t *
 /* same, f32 output (exact product) */
 int twm_dequant_to_f32(twm_ctx *ctx, const uint8_t *packed_dev, const uint16_t *scales_dev,
                        uint32_t k, uint32_t n, float *out_kn_dev);
+/* fp16::cast_f32_to_f16 / cast_f16_to_f32 (crates/kernels/src/fp16.rs:133-166): elementwise, round to nearest even.
+ * The GEMM entry points write f32 rows, as the reference's decode buffers are (generate.rs:1382-1404); a caller that
+ * keeps f16 rows (the reference's FP16 pipeline) converts with these, and converts its f32 norm output to f16 once
+ * where it wants the faster TWM_F16 input. */
+int twm_cast_f32_to_f16(twm_ctx *ctx, const float *src_dev, uint16_t *dst_dev, size_t count);
+int twm_cast_f16_to_f32(twm_ctx *ctx, const uint16_t *src_dev, float *dst_dev, size_t count);
 /* split_qkv (ops.rs:2300-2321) and split_gate_up (ops.rs:2324-2343) */
 int twm_split_qkv(twm_ctx *ctx, const float *qkv_dev, float *q_dev, float *k_dev, float *v_dev,
                   uint32_t h, uint32_t kv_dim, uint32_t batch);

@@ -19,6 +19,12 @@ SIGNATURES = {
     "twm_version": (C.c_char_p, []),
     "twm_device_count": (_int, []),
     "twm_last_error": (C.c_char_p, []),
+    "twm_last_error_kind": (_int, []),
+    "twm_stream_create": (_vp, [_vp]),
+    "twm_stream_destroy": (_int, [_vp, _vp]),
+    "twm_stream_sync": (_int, [_vp, _vp]),
+    "twm_cast_f32_to_f16": (_int, [_vp, _vp, _vp, _sz]),
+    "twm_cast_f16_to_f32": (_int, [_vp, _vp, _vp, _sz]),
     "twm_ctx_create": (_vp, [_int]),
     "twm_ctx_destroy": (None, [_vp]),
     "twm_ctx_sync": (_int, [_vp]),

@@ -14,7 +14,7 @@
 using namespace twm;
 
 static thread_local std::string g_err;
-twm::TraceBuf twm::g_trace = {nullptr, 0};
+static thread_local int g_err_kind = TWM_KIND_NONE;
 
 int twm::api_fail(int code, const char *fmt, ...)
 {
@@ -24,8 +24,11 @@ int twm::api_fail(int code, const char *fmt, ...)
     vsnprintf(buf, sizeof buf, fmt, ap);
     va_end(ap);
     g_err = buf;
+    g_err_kind = code == TWM_MEMORY_ERROR ? TWM_KIND_MEMORY : code == TWM_DEVICE_ERROR ? TWM_KIND_LAUNCH : TWM_KIND_NONE;
     return code;
 }
+
+void twm::set_error_kind(int kind) { g_err_kind = kind; }
 
 extern "C" {
 
@@ -39,6 +42,7 @@ int twm_device_count(void)
 }
 
 const char *twm_last_error(void) { return g_err.c_str(); }
+int twm_last_error_kind(void) { return g_err_kind; }
 
 twm_ctx *twm_ctx_create(int ordinal)
 {
@@ -47,6 +51,7 @@ twm_ctx *twm_ctx_create(int ordinal)
     if (e != hipSuccess || ordinal < 0 || ordinal >= count) {
         api_fail(TWM_DEVICE_ERROR, "twm_ctx_create: no HIP device %d (%s)", ordinal,
              e != hipSuccess ? hipGetErrorString(e) : "ordinal out of range");
+        set_error_kind(TWM_KIND_INIT);
         return nullptr;
     }
     twm_ctx *c = new (std::nothrow) twm_ctx();
@@ -58,6 +63,7 @@ twm_ctx *twm_ctx_create(int ordinal)
     c->force_sub = 0;
     c->force_sub_waves = 0;
     c->force_kernel = 0;
+    c->trace = TraceBuf{nullptr, 0};
     c->dequant_src = 0;
     c->weight_copies = 0;
     c->m1_exact = 0;
@@ -72,6 +78,7 @@ twm_ctx *twm_ctx_create(int ordinal)
     if (ok && strncmp(c->prop.gcnArchName, "gfx950", 6) != 0) {
         api_fail(TWM_DEVICE_ERROR, "twm_ctx_create: device %d is %s; this library holds gfx950 code only", ordinal,
              c->prop.gcnArchName);
+        set_error_kind(TWM_KIND_CODE_OBJECT);
         delete c;
         return nullptr;
     }
@@ -87,6 +94,7 @@ twm_ctx *twm_ctx_create(int ordinal)
     ok = ok && hipDeviceSynchronize() == hipSuccess;
     if (!ok) {
         api_fail(TWM_DEVICE_ERROR, "twm_ctx_create: %s", hipGetErrorString(hipGetLastError()));
+        set_error_kind(TWM_KIND_INIT);
         if (c->ws) (void)hipFree(c->ws);
         if (c->counters) (void)hipFree(c->counters);
         if (c->own_stream) (void)hipStreamDestroy(c->own_stream);
@@ -118,7 +126,46 @@ int twm_ctx_sync(twm_ctx *ctx)
         (void)hipGetLastError();
         (void)hipMemset(ctx->counters, 0, ctx->n_counters * sizeof(unsigned));
         (void)hipGetLastError();
-        return api_fail(TWM_DEVICE_ERROR, "twm_ctx_sync: %s", hipGetErrorString(e));
+        api_fail(TWM_DEVICE_ERROR, "twm_ctx_sync: %s", hipGetErrorString(e));
+        set_error_kind(TWM_KIND_SYNC);
+        return TWM_DEVICE_ERROR;
+    }
+    return TWM_OK;
+}
+
+void *twm_stream_create(twm_ctx *ctx)
+{
+    if (!ctx) { api_fail(TWM_INVALID_HANDLE, "twm_stream_create: null context"); return nullptr; }
+    hipStream_t s = nullptr;
+    hipError_t e = hipSetDevice(ctx->ordinal);
+    if (e == hipSuccess) e = hipStreamCreateWithFlags(&s, hipStreamNonBlocking);
+    if (e != hipSuccess) {
+        api_fail(TWM_DEVICE_ERROR, "twm_stream_create: %s", hipGetErrorString(e));
+        set_error_kind(TWM_KIND_INIT);
+        return nullptr;
+    }
+    return (void *)s;
+}
+
+int twm_stream_destroy(twm_ctx *ctx, void *hip_stream)
+{
+    if (!ctx) return api_fail(TWM_INVALID_HANDLE, "twm_stream_destroy: null context");
+    if (!hip_stream) return TWM_OK;
+    if ((hipStream_t)hip_stream == ctx->own_stream) return api_fail(TWM_INVALID_HANDLE, "twm_stream_destroy: that is the context's own stream");
+    if ((hipStream_t)hip_stream == ctx->stream) return api_fail(TWM_UNSUPPORTED_OP, "twm_stream_destroy: the context still issues its work on this stream (twm_ctx_set_stream first)");
+    HIP_TRY(hipStreamDestroy((hipStream_t)hip_stream), TWM_DEVICE_ERROR, "twm_stream_destroy");
+    return TWM_OK;
+}
+
+int twm_stream_sync(twm_ctx *ctx, void *hip_stream)
+{
+    if (!ctx) return api_fail(TWM_INVALID_HANDLE, "twm_stream_sync: null context");
+    hipError_t e = hipStreamSynchronize((hipStream_t)hip_stream);
+    if (e != hipSuccess) {
+        (void)hipGetLastError();
+        api_fail(TWM_DEVICE_ERROR, "twm_stream_sync: %s", hipGetErrorString(e));
+        set_error_kind(TWM_KIND_SYNC);
+        return TWM_DEVICE_ERROR;
     }
     return TWM_OK;
 }
@@ -127,8 +174,8 @@ int twm_debug_trace(twm_ctx *ctx, uint32_t *trace_dev, uint32_t capacity_workgro
 {
     if (!ctx) return api_fail(TWM_INVALID_HANDLE, "twm_debug_trace: null context");
     if (ctx->capturing) return api_fail(TWM_UNSUPPORTED_OP, "twm_debug_trace: a graph capture is open");
-    g_trace.ptr = capacity_workgroups ? trace_dev : nullptr;
-    g_trace.capacity = trace_dev ? capacity_workgroups : 0;
+    ctx->trace.ptr = capacity_workgroups ? trace_dev : nullptr;
+    ctx->trace.capacity = trace_dev ? capacity_workgroups : 0;
     return TWM_OK;
 }
 
@@ -232,7 +279,11 @@ void *twm_malloc(twm_ctx *ctx, size_t bytes)
     if (ctx->capturing) { api_fail(TWM_UNSUPPORTED_OP, "twm_malloc: not allowed inside a graph capture"); return nullptr; }
     void *p = nullptr;
     hipError_t e = hipMalloc(&p, bytes ? bytes : 4);
-    if (e != hipSuccess) { api_fail(TWM_MEMORY_ERROR, "hipMalloc(%zu): %s", bytes, hipGetErrorString(e)); return nullptr; }
+    if (e != hipSuccess) {
+        (void)hipGetLastError();  // (the runtime keeps the error for the next caller of hipGetLastError otherwise)
+        api_fail(TWM_MEMORY_ERROR, "hipMalloc(%zu): %s", bytes, hipGetErrorString(e));
+        return nullptr;
+    }
     return p;
 }
 
@@ -406,6 +457,24 @@ int twm_dequant_to_f32(twm_ctx *ctx, const uint8_t *packed_dev, const uint16_t *
                        float *out_kn_dev)
 {
     return dequant_common(ctx, packed_dev, scales_dev, k, n, out_kn_dev, false);
+}
+
+int twm_cast_f32_to_f16(twm_ctx *ctx, const float *src_dev, uint16_t *dst_dev, size_t count)
+{
+    if (!ctx) return api_fail(TWM_INVALID_HANDLE, "twm_cast_f32_to_f16: null context");
+    if (count == 0) return TWM_OK;
+    if (!src_dev || !dst_dev) return api_fail(TWM_INVALID_HANDLE, "twm_cast_f32_to_f16: null buffer");
+    HIP_TRY(launch_cast(ctx->stream, src_dev, dst_dev, count, true), TWM_DEVICE_ERROR, "cast kernel launch");
+    return TWM_OK;
+}
+
+int twm_cast_f16_to_f32(twm_ctx *ctx, const uint16_t *src_dev, float *dst_dev, size_t count)
+{
+    if (!ctx) return api_fail(TWM_INVALID_HANDLE, "twm_cast_f16_to_f32: null context");
+    if (count == 0) return TWM_OK;
+    if (!src_dev || !dst_dev) return api_fail(TWM_INVALID_HANDLE, "twm_cast_f16_to_f32: null buffer");
+    HIP_TRY(launch_cast(ctx->stream, src_dev, dst_dev, count, false), TWM_DEVICE_ERROR, "cast kernel launch");
+    return TWM_OK;
 }
 
 int twm_split_qkv(twm_ctx *ctx, const float *qkv_dev, float *q_dev, float *k_dev, float *v_dev, uint32_t h,

@@ -462,7 +462,7 @@ static int gemm_dispatch(twm_ctx *ctx, const twm_weight *w, const void *a_dev, i
         return TWM_OK;
     }
     case kFormSubTile:
-        HIP_TRY(launch_gemv4s(ctx->stream, v, a_dev, a_f32, m, gated, ctx->ws, ctx->counters, f.sub, f.waves, f.splits), TWM_DEVICE_ERROR,
+        HIP_TRY(launch_gemv4s(ctx->stream, v, a_dev, a_f32, m, gated, ctx->ws, ctx->counters, f.sub, f.waves, f.splits, ctx->trace), TWM_DEVICE_ERROR,
                 "sub-tile gemv launch");
         return TWM_OK;
     case kFormWholeTile:

@@ -16,11 +16,15 @@
 #define HIP_TRY(expr, code, what)                                                      \
     do {                                                                               \
         hipError_t e__ = (expr);                                                       \
-        if (e__ != hipSuccess) return api_fail(code, "%s: %s", what, hipGetErrorString(e__)); \
+        if (e__ != hipSuccess) {                                                       \
+            (void)hipGetLastError(); /* (the runtime keeps the error for the next caller of hipGetLastError otherwise) */ \
+            return api_fail(code, "%s: %s", what, hipGetErrorString(e__));             \
+        }                                                                              \
     } while (0)
 
 struct twm_ctx {
     int ordinal;
+    twm::TraceBuf trace;  // twm_debug_trace: where this context's M = 1 sub-tile launches record their clocks (null: off)
     hipStream_t own_stream;
     hipStream_t stream;
     float *ws;            // split-K partial tiles

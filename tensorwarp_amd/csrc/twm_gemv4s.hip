@@ -321,7 +321,7 @@ __global__ __launch_bounds__(1024) void k_gemv4s_traced(const char *__restrict__
 
 template <int SUB, int RL>
 static hipError_t launch_gemv4s_t(hipStream_t s, const WeightView &w, const void *a, bool a_f32, uint32_t m,
-                                  const OutSpec &out, float *ws, unsigned *counters, uint32_t waves, uint32_t splits)
+                                  const OutSpec &out, float *ws, unsigned *counters, uint32_t waves, uint32_t splits, TraceBuf trace)
 {
     uint32_t n_pad = w.n_tiles * kTileN;  // whole 64-column tiles
     uint32_t sub_tiles = n_pad / SUB;
@@ -337,13 +337,13 @@ static hipError_t launch_gemv4s_t(hipStream_t s, const WeightView &w, const void
                        (const uint16_t *)nullptr, gemv4s_cfg(splits, out.swiglu != nullptr, waves, m, runs), w.k, w.k_chunks, \
                        sub_tiles, cps, w.n, n_pad, ws, counters, out)
     if constexpr (RL == 1) {
-        if (!a_f32 && g_trace.ptr && blocks <= g_trace.capacity) {
+        if (!a_f32 && trace.ptr && blocks <= trace.capacity) {
             if (one)
                 hipLaunchKernelGGL((k_gemv4s_traced<SUB, true>), dim3(blocks), dim3(waves * 64), lds, s, (const char *)w.cq, a, out,
-                                   ws, counters, m, w.k, w.n, n_pad, w.k_chunks, sub_tiles, splits, cps, g_trace.ptr);
+                                   ws, counters, m, w.k, w.n, n_pad, w.k_chunks, sub_tiles, splits, cps, trace.ptr);
             else
                 hipLaunchKernelGGL((k_gemv4s_traced<SUB, false>), dim3(blocks), dim3(waves * 64), lds, s, (const char *)w.cq, a, out,
-                                   ws, counters, m, w.k, w.n, n_pad, w.k_chunks, sub_tiles, splits, cps, g_trace.ptr);
+                                   ws, counters, m, w.k, w.n, n_pad, w.k_chunks, sub_tiles, splits, cps, trace.ptr);
             return hipGetLastError();
         }
     }
@@ -378,7 +378,7 @@ static hipError_t launch_gemv4s_t(hipStream_t s, const WeightView &w, const void
 // sub = 32 or 16 columns per workgroup; waves 1 .. 16; out.swiglu set: the gated store of a paired weight.
 // m <= 4 with f16 or f32 activations, m = 5 .. 16 with f16 activations.
 hipError_t launch_gemv4s(hipStream_t s, const WeightView &w, const void *a, bool a_f32, uint32_t m, const OutSpec &out,
-                         float *ws, unsigned *counters, uint32_t sub, uint32_t waves, uint32_t splits)
+                         float *ws, unsigned *counters, uint32_t sub, uint32_t waves, uint32_t splits, TraceBuf trace)
 {
     if (m == 0 || w.n == 0) return hipSuccess;
     if (m > 16 || (m > 4 && a_f32) || splits == 0 || !w.cq) return hipErrorInvalidValue;
@@ -387,11 +387,11 @@ hipError_t launch_gemv4s(hipStream_t s, const WeightView &w, const void *a, bool
     if (sub != 32 && sub != 16) return hipErrorInvalidValue;
 #define TWM_S_CASE(SUBV)                                                                                       \
     if (sub == SUBV) {                                                                                         \
-        if (m == 1) return launch_gemv4s_t<SUBV, 1>(s, w, a, a_f32, m, out, ws, counters, waves, splits);      \
-        if (m == 2) return launch_gemv4s_t<SUBV, 2>(s, w, a, a_f32, m, out, ws, counters, waves, splits);      \
-        if (m <= 4) return launch_gemv4s_t<SUBV, 4>(s, w, a, a_f32, m, out, ws, counters, waves, splits);      \
-        if (m <= 8) return launch_gemv4s_t<SUBV, 8>(s, w, a, a_f32, m, out, ws, counters, waves, splits);      \
-        return launch_gemv4s_t<SUBV, 16>(s, w, a, a_f32, m, out, ws, counters, waves, splits);                 \
+        if (m == 1) return launch_gemv4s_t<SUBV, 1>(s, w, a, a_f32, m, out, ws, counters, waves, splits, trace); \
+        if (m == 2) return launch_gemv4s_t<SUBV, 2>(s, w, a, a_f32, m, out, ws, counters, waves, splits, trace); \
+        if (m <= 4) return launch_gemv4s_t<SUBV, 4>(s, w, a, a_f32, m, out, ws, counters, waves, splits, trace); \
+        if (m <= 8) return launch_gemv4s_t<SUBV, 8>(s, w, a, a_f32, m, out, ws, counters, waves, splits, trace); \
+        return launch_gemv4s_t<SUBV, 16>(s, w, a, a_f32, m, out, ws, counters, waves, splits, trace);          \
     }
     TWM_S_CASE(32)
     TWM_S_CASE(16)

@@ -86,6 +86,8 @@ struct DecodePlan {
 // ---- host-side helpers shared by the files that hold C-ABI entry points ---------------
 // records the message for twm_last_error() on the calling thread and returns `code`
 int api_fail(int code, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
+// the DeviceError variant of the failure just recorded by api_fail (TWM_KIND_*), where the code alone does not tell
+void set_error_kind(int kind);
 // K % 32 == 0 and K x N within the ABI's limit, else TWM_SHAPE_ERROR with the message set
 int check_kn(const char *who, uint32_t k, uint32_t n);
 // What the dispatch of the GEMV on the reference's arrays needs from its caller: the stream, the knobs, and the
@@ -112,7 +114,6 @@ struct TraceBuf {
     uint32_t *ptr;
     uint32_t capacity;
 };
-extern TraceBuf g_trace;
 
 // ---- launchers (all asynchronous on `s`, return the launch status) ---------------
 hipError_t launch_fill_zero(hipStream_t s, void *ptr, size_t bytes);
@@ -124,6 +125,7 @@ hipError_t launch_fuse_one(hipStream_t s, const uint8_t *packed_in, const uint16
                            uint32_t ni, uint32_t total_n, uint32_t col_off, uint8_t *packed_out, uint16_t *scales_out);
 hipError_t launch_dequant(hipStream_t s, const uint8_t *packed, const uint16_t *scales, uint32_t k, uint32_t n,
                           void *out, bool f16_out);
+hipError_t launch_cast(hipStream_t s, const void *src, void *dst, size_t count, bool to_f16);
 hipError_t launch_split_qkv(hipStream_t s, const float *qkv, float *q, float *kk, float *v, uint32_t h,
                             uint32_t kv, uint32_t batch);
 hipError_t launch_split_gate_up(hipStream_t s, const float *gu, float *g, float *u, uint32_t ffn, uint32_t batch);
@@ -150,7 +152,7 @@ hipError_t launch_weight_dequant_f16_col(hipStream_t s, const WeightView &w, uin
 // swiglu_out != nullptr (the weight in the paired gate_up column order, N = 2*ffn a multiple of 64): instead
 // of the N columns, write silu(gate) * up of every feature to swiglu_out[m][ffn]; `out` is ignored.
 hipError_t launch_gemv4s(hipStream_t s, const WeightView &w, const void *a, bool a_f32, uint32_t m, const OutSpec &out,
-                         float *ws, unsigned *counters, uint32_t sub, uint32_t waves, uint32_t splits);
+                         float *ws, unsigned *counters, uint32_t sub, uint32_t waves, uint32_t splits, TraceBuf trace = TraceBuf{nullptr, 0});
 hipError_t launch_gemv4s_ref(hipStream_t s, const uint8_t *packed, const uint16_t *scales, uint32_t k, uint32_t n,
                              const float *a, float *c, float *ws, unsigned *counters, uint32_t sub, uint32_t waves,
                              uint32_t splits);

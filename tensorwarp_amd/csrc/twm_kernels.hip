@@ -60,6 +60,32 @@ hipError_t launch_fill_zero(hipStream_t s, void *ptr, size_t bytes)
 }
 
 // ---------------------------------------------------------------------------------
+// casts between f32 and f16 rows (crates/kernels/src/fp16.rs:133-166): round to nearest even, as __float2half
+// ---------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void k_cast_f32_f16(const float *__restrict__ src, _Float16 *__restrict__ dst, size_t count)
+{
+    size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    size_t stride = (size_t)gridDim.x * 256;
+    for (; i < count; i += stride) dst[i] = (_Float16)src[i];
+}
+__global__ __launch_bounds__(256) void k_cast_f16_f32(const _Float16 *__restrict__ src, float *__restrict__ dst, size_t count)
+{
+    size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    size_t stride = (size_t)gridDim.x * 256;
+    for (; i < count; i += stride) dst[i] = (float)src[i];
+}
+
+hipError_t launch_cast(hipStream_t s, const void *src, void *dst, size_t count, bool to_f16)
+{
+    if (count == 0) return hipSuccess;
+    size_t blocks = (count + 255) / 256;
+    if (blocks > 4096) blocks = 4096;
+    if (to_f16) hipLaunchKernelGGL(k_cast_f32_f16, dim3((unsigned)blocks), dim3(256), 0, s, (const float *)src, (_Float16 *)dst, count);
+    else hipLaunchKernelGGL(k_cast_f16_f32, dim3((unsigned)blocks), dim3(256), 0, s, (const _Float16 *)src, (float *)dst, count);
+    return hipGetLastError();
+}
+
+// ---------------------------------------------------------------------------------
 // quantizer: one thread per (group, column)
 // ---------------------------------------------------------------------------------
 struct QGroup {

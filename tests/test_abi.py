@@ -103,6 +103,18 @@ def test_no_gpu_means_clean_failure():
     with pytest.raises(T.DeviceError) as e:
         T.WarpDevice(0)
     assert e.value.code == _lib.DEVICE_ERROR
+    assert lib.twm_last_error_kind() == 1        # TWM_KIND_INIT: DeviceError::Init (device.rs:278-292)
+
+
+def test_error_kinds_of_argument_errors():
+    # an error that never reached the device maps to no DeviceError variant; the new entries reject null handles
+    lib = _lib.load()
+    assert lib.twm_ctx_sync(None) == _lib.INVALID_HANDLE and lib.twm_last_error_kind() == 0
+    assert lib.twm_stream_create(None) is None and lib.twm_last_error_kind() == 0
+    assert lib.twm_stream_sync(None, None) == _lib.INVALID_HANDLE
+    assert lib.twm_stream_destroy(None, None) == _lib.INVALID_HANDLE
+    assert lib.twm_cast_f32_to_f16(None, None, None, 4) == _lib.INVALID_HANDLE
+    assert lib.twm_cast_f16_to_f32(None, None, None, 4) == _lib.INVALID_HANDLE
 
 
 def test_product_package_does_not_touch_the_oracle():

@@ -287,6 +287,67 @@ def test_gemm_geglu_gate(dev, m, splits):
     w.free()
 
 
+def test_stream_objects_casts_and_error_kinds(dev):
+    # stream objects (device.rs:230-265), the f32 <-> f16 casts (fp16.rs:133-166) bit-exact against numpy's IEEE
+    # conversion, and the DeviceError variant of a failure (device.rs:278-292)
+    lib = T._lib.load()
+    s = lib.twm_stream_create(dev.handle)
+    assert s
+    own = lib.twm_ctx_stream(dev.handle)
+    assert lib.twm_ctx_set_stream(dev.handle, s) == T._lib.OK
+    assert lib.twm_stream_destroy(dev.handle, s) == T._lib.UNSUPPORTED_OP      # still in use by the context
+    x = (O.synth_normal_f32(70001, 77) * np.float32(300.0)).astype(np.float32)
+    x[:6] = [0.0, -0.0, 65504.0, 65520.0, 1e-8, -6.0e-8]                      # edge of the range, ties, subnormals
+    xd = T.GpuTensor.from_host(dev, x)
+    hd = T.GpuTensor.zeros(dev, (x.size,), "f16")
+    assert lib.twm_cast_f32_to_f16(dev.handle, xd.ptr, hd.ptr, x.size) == T._lib.OK
+    assert lib.twm_stream_sync(dev.handle, s) == T._lib.OK
+    with np.errstate(over="ignore"):
+        want = x.astype(np.float16)
+    assert np.array_equal(hd.to_host().view(np.uint16), want.view(np.uint16))
+    back = T.GpuTensor.zeros(dev, (x.size,), "f32")
+    assert lib.twm_cast_f16_to_f32(dev.handle, hd.ptr, back.ptr, x.size) == T._lib.OK
+    assert lib.twm_stream_sync(dev.handle, s) == T._lib.OK
+    assert np.array_equal(back.to_host().view(np.uint32), want.astype(np.float32).view(np.uint32))
+    assert lib.twm_ctx_set_stream(dev.handle, None) == T._lib.OK
+    assert lib.twm_ctx_stream(dev.handle) == own
+    assert lib.twm_stream_destroy(dev.handle, own) == T._lib.INVALID_HANDLE    # the context's own stream
+    assert lib.twm_stream_destroy(dev.handle, s) == T._lib.OK
+    # a shape error is no DeviceError variant; an allocation the device cannot serve is Memory
+    assert lib.twm_gemm_tw_marlin_m1(dev.handle, xd.ptr, xd.ptr, xd.ptr, xd.ptr, 64, 100) == T._lib.SHAPE_ERROR
+    assert lib.twm_last_error_kind() == 0
+    assert lib.twm_malloc(dev.handle, 1 << 60) is None and lib.twm_last_error_kind() == 5
+    for t in (xd, hd, back):
+        t.free()
+
+
+def test_debug_trace_belongs_to_its_context(dev):
+    # a trace buffer set on one context does not reroute another context's launches
+    lib = T._lib.load()
+    k, n = 3584, 640
+    packed, scales, a16 = synth(k, n, 1, 4242)
+    with T.WarpDevice(0) as other:
+        w_a = T.MarlinWeight.upload(dev, packed, scales, k, n)
+        w_b = T.MarlinWeight.upload(other, packed, scales, k, n)
+        trace = T.GpuTensor.zeros(dev, (4 * 4096,), "i32")
+        assert lib.twm_debug_trace(dev.handle, trace.ptr, 4096) == T._lib.OK
+        try:
+            cb = T.GpuTensor.zeros(other, (n,), "f32")
+            T.gemm(other, w_b, T.GpuTensor.from_host(other, a16, "f16"), 1, cb)
+            other.synchronize()
+            dev.synchronize()
+            assert not trace.to_host().any()                   # the other context's launch left no trace
+            ca = T.GpuTensor.zeros(dev, (n,), "f32")
+            T.gemm(dev, w_a, T.GpuTensor.from_host(dev, a16, "f16"), 1, ca)
+            dev.synchronize()
+            assert trace.to_host().any()
+            assert np.array_equal(ca.to_host(), cb.to_host())   # the traced twin computes the same bits
+        finally:
+            assert lib.twm_debug_trace(dev.handle, None, 0) == T._lib.OK
+        w_a.free()
+        w_b.free()
+
+
 def test_argmax_bit_exact(dev):
     # index output: bit exact against the oracle's sequential scan, including ties (first wins), values at or
     # below the -1e30 starting value, NaN, infinities, a vocabulary-sized row and an empty one
