@@ -125,6 +125,9 @@ int twm_ctx_info(twm_ctx *ctx, char *buf, size_t buf_len);
  *                   the reference's split-K rule and float atomics (bit-equal to the reference order when that
  *                   rule yields one split); 0 (default) = the MFMA kernel
  *   "m1_splits"     twm_gemm_tw_marlin_m1: split-K factor of the MFMA kernel (0 .. 64)
+ *   "m1_align16"    twm_gemm_tw_marlin_m1: 1 = a call whose activations or packed weights are not 16-byte aligned (a slab
+ *                   offset that is only 4-byte aligned, the reference kernel's own limit) returns TWM_SHAPE_ERROR instead
+ *                   of silently taking the plain f32 kernel, which is about 3.6 times slower; 0 (default) = take it
  *   "batch_rounded" twm_gemm at M = 17 .. 32: 1 = weights rounded to f16 and summed over K by the MFMAs, the arithmetic
  *                   of the prefill GEMM; 0 (default) = exact weights with f32 group scales as for M <= 16
  * Values outside these sets return TWM_SHAPE_ERROR, unknown keys TWM_UNSUPPORTED_OP. */

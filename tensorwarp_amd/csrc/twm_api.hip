@@ -67,6 +67,7 @@ twm_ctx *twm_ctx_create(int ordinal)
     c->dequant_src = 0;
     c->weight_copies = 0;
     c->m1_exact = 0;
+    c->m1_align16 = 0;
     c->m1_splits = 0;
     c->batch_rounded = 0;
     c->prefill_bm = 0;
@@ -246,6 +247,11 @@ int twm_ctx_set_option(twm_ctx *ctx, const char *key, int value)
     if (strcmp(key, "dequant_src") == 0) {
         if (value != 0 && value != 1) return api_fail(TWM_SHAPE_ERROR, "twm_ctx_set_option: dequant_src must be 0 or 1");
         ctx->dequant_src = value;
+        return TWM_OK;
+    }
+    if (strcmp(key, "m1_align16") == 0) {
+        if (value != 0 && value != 1) return api_fail(TWM_SHAPE_ERROR, "twm_ctx_set_option: m1_align16 must be 0 or 1");
+        ctx->m1_align16 = value;
         return TWM_OK;
     }
     if (strcmp(key, "m1_exact") == 0) {
@@ -712,6 +718,9 @@ int twm_gemm_tw_marlin_m1(twm_ctx *ctx, const float *a_dev, const uint8_t *packe
                           float *c_dev, uint32_t n, uint32_t k)
 {
     if (!ctx) return api_fail(TWM_INVALID_HANDLE, "twm_gemm_tw_marlin_m1: null context");
+    if (ctx->m1_align16 && !ctx->m1_exact && ((((uintptr_t)a_dev | (uintptr_t)packed_dev) & 15) != 0))
+        return api_fail(TWM_SHAPE_ERROR, "twm_gemm_tw_marlin_m1: activations or packed weights are not 16-byte aligned "
+                                         "(option m1_align16: the 4-byte path, k_ref_gemv, is about 3.6 times slower)");
     const M1Env env = {ctx->stream, ctx->m1_exact, ctx->m1_splits, ctx->force_sub, ctx->force_waves,
                        ctx->ws, ctx->ws_bytes, ctx->counters, ctx->n_counters, false};
     return m1_dispatch(env, "twm_gemm_tw_marlin_m1", a_dev, packed_dev, scales_dev, c_dev, n, k);

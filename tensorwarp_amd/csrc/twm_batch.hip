@@ -286,6 +286,20 @@ __global__ __launch_bounds__(64 * WPS * KS) void k_batch(const uint4v *__restric
 
     // ---- store: lane (c, kb) holds rows 16 mt + 4 kb + r of column 16 tile + c
     const uint32_t n_ld = n_tiles * 16u;
+    if (out.row_scale && !partials) {
+        // f32 rows that were scaled into the f16 range: their sums back, before bias and gate (the K-split's sum kernel
+        // does it for partial sums).  A step of its own ahead of the stores: inside the store loops it moved the main
+        // loop's prefetches of one variant down to their use.
+#pragma unroll
+        for (int mt = 0; mt < MT; mt++)
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                const uint32_t row = 16u * mt + 4u * kb + r;
+                const float rs = out.row_scale[row < m_rows ? row : m_rows - 1u];
+#pragma unroll
+                for (int i = 0; i < TPW; i++) acc[mt][i][r] *= rs;
+            }
+    }
     if (partials) {
         float *dst = partials + (size_t)blockIdx.y * m_rows * n_ld;
 #pragma unroll
@@ -313,10 +327,7 @@ __global__ __launch_bounds__(64 * WPS * KS) void k_batch(const uint4v *__restric
 #pragma unroll
                 for (int r = 0; r < 4; r++) {
                     const uint32_t row = 16u * mt + 4u * kb + r;
-                    if (row < m_rows) {
-                        const float rs = out.row_scale ? out.row_scale[row] : 1.f;  // (f32 rows scaled into the f16 range)
-                        out.swiglu[(size_t)row * ffn + feat] = gated_mul(out.gate_act, acc[mt][0][r] * rs, acc[mt][1][r] * rs);
-                    }
+                    if (row < m_rows) out.swiglu[(size_t)row * ffn + feat] = gated_mul(out.gate_act, acc[mt][0][r], acc[mt][1][r]);
                 }
             return;
         }
@@ -338,10 +349,7 @@ __global__ __launch_bounds__(64 * WPS * KS) void k_batch(const uint4v *__restric
 #pragma unroll
                 for (int r = 0; r < 4; r++) {
                     const uint32_t row = 16u * mt + 4u * kb + r;
-                    if (row < m_rows) {
-                        const float v = out.row_scale ? acc[mt][i][r] * out.row_scale[row] : acc[mt][i][r];
-                        out.seg[sg].ptr[(size_t)row * out.seg[sg].width + rel] = has_b ? v + b : v;
-                    }
+                    if (row < m_rows) out.seg[sg].ptr[(size_t)row * out.seg[sg].width + rel] = has_b ? acc[mt][i][r] + b : acc[mt][i][r];
                 }
         }
     }

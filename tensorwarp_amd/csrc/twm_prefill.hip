@@ -289,12 +289,10 @@ __global__ __launch_bounds__(256) TWM_PF_OCC(HALF) void k_prefill(const uint4v *
 #pragma unroll
             for (int i = 0; i < 4; i++) {
                 const uint32_t row = (lane >> 4) + 4u * i;
-                float4v v = *(const float4v *)(stage + row * 68 + (lane & 15u) * 4u);
+                const float4v v = *(const float4v *)(stage + row * 68 + (lane & 15u) * 4u);
                 const uint32_t om = m0 + mt * 16u + row;
-                if (om < m_rows && col < n_lim && (lane & 15u) * 4u < 16u * NTW) {
-                    if (out.row_scale && !partials) v *= out.row_scale[om];  // (f32 rows scaled into the f16 range)
+                if (om < m_rows && col < n_lim && (lane & 15u) * 4u < 16u * NTW)
                     __builtin_nontemporal_store(v, (float4v *)(dst + (size_t)om * ld + col));
-                }
             }
         }
         return;
@@ -331,11 +329,8 @@ __global__ __launch_bounds__(256) TWM_PF_OCC(HALF) void k_prefill(const uint4v *
 #pragma unroll
             for (int t = 0; t < 2; t++)
 #pragma unroll
-                for (int r = 0; r < 4; r++) {
-                    const uint32_t om = m0 + mt * 16u + kb * 4u + r;
-                    const float rs = out.row_scale && om < m_rows ? out.row_scale[om] : 1.f;
-                    stage[(kb * 4 + r) * 36 + t * 16 + c] = gated_mul(out.gate_act, acc[mt][t][r] * rs, acc[mt][(t + 2) % NTW][r] * rs);
-                }
+                for (int r = 0; r < 4; r++)
+                    stage[(kb * 4 + r) * 36 + t * 16 + c] = gated_mul(out.gate_act, acc[mt][t][r], acc[mt][(t + 2) % NTW][r]);
 #pragma unroll
             for (int i = 0; i < 2; i++) {
                 const uint32_t row = (lane >> 3) + 8u * i;
@@ -363,7 +358,7 @@ __global__ __launch_bounds__(256) TWM_PF_OCC(HALF) void k_prefill(const uint4v *
 #pragma unroll
             for (int r = 0; r < 4; r++) {
                 uint32_t om = m0 + mt * 16u + kb * 4u + r;
-                if (om < m_rows) pf_store_out(out, om, on, out.row_scale ? acc[mt][t][r] * out.row_scale[om] : acc[mt][t][r]);
+                if (om < m_rows) pf_store_out(out, om, on, acc[mt][t][r]);
             }
     }
 }
@@ -416,6 +411,19 @@ __global__ __launch_bounds__(256) void k_splitk_reduce_swiglu(const float *__res
     float4 o = {gated_mul(act, g.x * rs, u.x * rs), gated_mul(act, g.y * rs, u.y * rs), gated_mul(act, g.z * rs, u.z * rs),
                 gated_mul(act, g.w * rs, u.w * rs)};
     *(float4 *)(gate_out + (size_t)row * ffn + feat) = o;
+}
+
+// out[row][:] *= row_scale[row] over every segment, for the rows whose factor is not 1 (a workgroup per row; a row that
+// needs nothing costs its workgroup one load)
+__global__ __launch_bounds__(256) void k_scale_rows(OutSpec out, const float *__restrict__ row_scale)
+{
+    const uint32_t row = blockIdx.x;
+    const float rs = row_scale[row];
+    if (rs == 1.f) return;
+    for (uint32_t sg = 0; sg < out.count && sg < (uint32_t)kMaxSegs; sg++) {
+        float *p = out.seg[sg].ptr + (size_t)row * out.seg[sg].width;
+        for (uint32_t c = threadIdx.x; c < out.seg[sg].width; c += 256u) p[c] *= rs;
+    }
 }
 
 hipError_t launch_splitk_reduce(hipStream_t s, const float *partials, const OutSpec &out, uint32_t m, uint32_t n,
@@ -532,7 +540,7 @@ void prefill_plan_of(uint32_t rows, uint32_t block_rows, uint32_t splits, uint32
 
 template <int MT, int NTW = 4, bool HALF = false>
 static hipError_t launch_prefill_t(hipStream_t s, const WeightView &w, const _Float16 *a, uint32_t m, const OutSpec &out,
-                                   uint32_t splits, float *partials)
+                                   uint32_t splits, float *partials, bool via_partials = false)
 {
     size_t lds = (size_t)2 * 16 * MT * kPfRowStride * sizeof(_Float16);
     uint32_t cps = (w.k_chunks + splits - 1) / splits;
@@ -541,14 +549,17 @@ static hipError_t launch_prefill_t(hipStream_t s, const WeightView &w, const _Fl
     dim3 grid(col_blocks * row_blocks, 1, splits);  // the kernel turns the linear id into an XCD-aware tile
     // 16-byte row stores: into the partial sums always (padded width, a multiple of 64); into the output when it
     // is one plain [M, N] matrix with N a multiple of 4 at a 16-byte aligned address
+    // (via_partials: the sums of a single split go through the partial-sum buffer too and k_splitk_reduce stores them:
+    // it is the store that applies the rows' power-of-two factors of f32 activations ahead of a bias or a gate)
+    via_partials = via_partials && partials != nullptr;
     uint32_t row_store = 1;
-    if (splits == 1)
+    if (splits == 1 && !via_partials)
         row_store = !out.swiglu && out.count == 1 && out.seg[0].start == 0 && out.seg[0].width == w.n && !out.seg[0].bias &&
                     w.n % 4 == 0 && ((uintptr_t)out.seg[0].ptr & 15) == 0;
     if (NTW != 4 && out.swiglu) return hipErrorInvalidValue;
     hipLaunchKernelGGL((k_prefill<MT, NTW, HALF>), grid, dim3(256), lds, s, (const uint4v *)w.qw, (const uint2v *)w.sc, a, out, m, w.k,
-                       w.n, w.n_tiles, w.k_chunks, cps, splits > 1 ? partials : nullptr, row_store, col_blocks, row_blocks);
-    if (splits > 1) return launch_splitk_reduce(s, partials, out, m, w.n, w.n_tiles * 16, splits);
+                       w.n, w.n_tiles, w.k_chunks, cps, splits > 1 || via_partials ? partials : nullptr, row_store, col_blocks, row_blocks);
+    if (splits > 1 || via_partials) return launch_splitk_reduce(s, partials, out, m, w.n, w.n_tiles * 16, splits);
     return hipGetLastError();
 }
 
@@ -574,24 +585,29 @@ hipError_t launch_prefill(hipStream_t s, const WeightView &w, const void *a, boo
 {
     if (m == 0 || w.n == 0) return hipSuccess;
     if (block_rows != 0 && block_rows != 64 && block_rows != 128 && block_rows != 192) return hipErrorInvalidValue;
-    auto run = [&](const _Float16 *a16, uint32_t rows, const OutSpec &o, void *ws, size_t ws_bytes) {
+    auto run = [&](const _Float16 *a16, uint32_t rows, const OutSpec &o, void *ws, size_t ws_bytes, bool via = false) {
         // (a forced 192-column form with the gated store: the 256-column one)
         const uint32_t form = block_rows == 192 && o.swiglu ? 128u : block_rows;
         const PrefillPlan plan = plan_prefill_within(rows, form, splits, w.n_tiles, w.k_chunks, ws ? ws_bytes : 0, o.swiglu != nullptr);
-        if (plan.block_rows == 64) return launch_prefill_t<4>(s, w, a16, rows, o, plan.splits, (float *)ws);
+        if (plan.block_rows == 64) return launch_prefill_t<4>(s, w, a16, rows, o, plan.splits, (float *)ws, via);
         if (plan.block_rows == 192) {
             // more workgroups than CUs: the variant of which two share a CU (4096 -> 11008 at M = 1024, 464 workgroups:
             // 81.6 against 89.5 us; at M = 512, 232 workgroups, 49.0 against 46.4)
             const uint64_t wgs = (uint64_t)((w.n_tiles + 11) / 12) * ((rows + 127) / 128) * plan.splits;
-            return wgs > 256 ? launch_prefill_t<8, 3, true>(s, w, a16, rows, o, plan.splits, (float *)ws)
-                             : launch_prefill_t<8, 3>(s, w, a16, rows, o, plan.splits, (float *)ws);
+            return wgs > 256 ? launch_prefill_t<8, 3, true>(s, w, a16, rows, o, plan.splits, (float *)ws, via)
+                             : launch_prefill_t<8, 3>(s, w, a16, rows, o, plan.splits, (float *)ws, via);
         }
-        return launch_prefill_t<8>(s, w, a16, rows, o, plan.splits, (float *)ws);
+        return launch_prefill_t<8>(s, w, a16, rows, o, plan.splits, (float *)ws, via);
     };
     if (!a_f32) return run((const _Float16 *)a, m, out, scratch, scratch_bytes);
     // f16 copy of the activations (each row scaled by a power of two where it would leave the f16 range, the factors in
-    // front of the copy) at the front of the scratch, partials behind it
-    size_t row_bytes = (size_t)w.k * 2 + 4;
+    // front of the copy) at the front of the scratch, partials behind it.  The factors go back onto the sums in the
+    // K-split's sum kernel where there is one; a launch without a K-split stores plain sums and a small kernel scales
+    // the rows that need it afterwards (most launches: none) -- unless a bias or a gate follows the sum, which the
+    // factor has to come before: then the single split's sums go through the partial-sum buffer and the sum kernel too.
+    bool after_sum = out.swiglu != nullptr;
+    for (uint32_t i = 0; i < out.count; i++) after_sum = after_sum || out.seg[i].bias != nullptr;
+    size_t row_bytes = (size_t)w.k * 2 + 4 + (after_sum ? (size_t)w.n_tiles * 16 * 4 : 0);
     if (!scratch || scratch_bytes < row_bytes + 512) return hipErrorInvalidValue;
     uint32_t slab = (uint32_t)((scratch_bytes - 512) / 2 / row_bytes < m ? (scratch_bytes - 512) / 2 / row_bytes : m);
     if (slab == 0) slab = 1;
@@ -607,8 +623,18 @@ hipError_t launch_prefill(hipStream_t s, const WeightView &w, const void *a, boo
         for (uint32_t i = 0; i < o.count; i++) o.seg[i].ptr += (size_t)r0 * o.seg[i].width;
         if (o.swiglu) o.swiglu += (size_t)r0 * (w.n / 2);
         size_t used = (size_t)((char *)a16 - (char *)scratch) + (((size_t)rows * w.k * 2 + 255) & ~(size_t)255);
-        hipError_t e = run(a16, rows, o, (char *)scratch + used, scratch_bytes - used);
+        hipError_t e = run(a16, rows, o, (char *)scratch + used, scratch_bytes - used, after_sum);
         if (e != hipSuccess) return e;
+        if (!after_sum) {
+            const PrefillPlan plan = plan_prefill_within(rows, block_rows == 192 && o.swiglu ? 128u : block_rows, splits, w.n_tiles, w.k_chunks,
+                                                         scratch_bytes - used, false);
+            const uint32_t cps = (w.k_chunks + plan.splits - 1) / plan.splits;
+            if ((w.k_chunks + cps - 1) / cps == 1) {  // (with a K-split the sum kernel has applied the factors)
+                hipLaunchKernelGGL(k_scale_rows, dim3(rows), dim3(256), 0, s, o, (const float *)row_scale);
+                e = hipGetLastError();
+                if (e != hipSuccess) return e;
+            }
+        }
     }
     return hipGetLastError();
 }

@@ -629,6 +629,14 @@ def test_gemm_tw_marlin_m1_from_buffer_and_errors(dev):
         T.gemm_tw_marlin_m1_from_buffer(dev, T.GpuTensor.from_host(dev, ab), T.GpuTensor.from_host(dev, slab), 36,
                                         T.GpuTensor.from_host(dev, sc_, "f16"), 0, cb, nn, kk)
         assert rel_err(cb.to_host(), O.gemm_f64(ab, pk, sc_, 1, kk, nn)[0]) < TIGHT
+        dev.set_option("m1_align16", 1)                  # a caller can ask to be told instead of taking the slow kernel
+        try:
+            with pytest.raises(T.DeviceError) as e3:
+                T.gemm_tw_marlin_m1_from_buffer(dev, T.GpuTensor.from_host(dev, ab), T.GpuTensor.from_host(dev, slab), 36,
+                                                T.GpuTensor.from_host(dev, sc_, "f16"), 0, cb, nn, kk)
+            assert e3.value.code == T._lib.SHAPE_ERROR and "16-byte" in str(e3.value)
+        finally:
+            dev.set_option("m1_align16", 0)
         with pytest.raises(T.DeviceError) as e2:         # not even 4-byte aligned: a fault in the reference
             T.gemm_tw_marlin_m1_from_buffer(dev, T.GpuTensor.from_host(dev, ab), T.GpuTensor.from_host(dev, slab), 35,
                                             T.GpuTensor.from_host(dev, sc_, "f16"), 0, cb, nn, kk)
