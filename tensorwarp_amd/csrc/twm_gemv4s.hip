@@ -157,11 +157,20 @@ __device__ __forceinline__ void gemv4s_body(const char *__restrict__ cw, const v
     // four independent reads at a time, and the same lane swaps add those - against one thread walking waves * 64 / SUB
     // values one dependent read after the other, which took longer than the unpack of a pass.
     constexpr int E = RL * SUB;       // entries of the workgroup: e = r * SUB + column
+    // (More entries than a wave has lanes, i.e. five rows and more: two lane swaps per row and wave are sixteen to
+    // thirty-two swaps per wave, which with four waves on a SIMD cost more than they save -- 3584 -> 4608 at 16 rows 8.2
+    // against 7.7 us; there every lane writes its sums and the thread that finishes an entry adds the lane groups too.)
+    constexpr bool WIDE = E > 64;
+    if constexpr (WIDE) {
 #pragma unroll
-    for (int r = 0; r < RL; r++) acc[r] = sum_lane_groups<SUB>(acc[r]);
-    if (cg == 0) {
+        for (int r = 0; r < RL; r++) red[(wave * RL + r) * 64 + lane] = acc[r];
+    } else {
 #pragma unroll
-        for (int r = 0; r < RL; r++) red[wave * E + r * SUB + cl] = acc[r];
+        for (int r = 0; r < RL; r++) acc[r] = sum_lane_groups<SUB>(acc[r]);
+        if (cg == 0) {
+#pragma unroll
+            for (int r = 0; r < RL; r++) red[wave * E + r * SUB + cl] = acc[r];
+        }
     }
     __syncthreads();
 
@@ -221,23 +230,31 @@ __device__ __forceinline__ void gemv4s_body(const char *__restrict__ cw, const v
         if (lane == 0) __hip_atomic_store(&counters[st], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         return;
     } else {
-        // more entries than a wave has lanes (four rows on 32 columns, five to sixteen rows): a thread per entry
+        // more entries than a wave has lanes (four rows on 32 columns, five to sixteen rows): a thread per entry, which
+        // adds the waves' lane groups (64 / SUB reads in flight at a time)
         const uint32_t threads = waves * 64u;
+        auto sum_wide = [&](uint32_t r, uint32_t c) {
+            float v = 0.f;
+            for (uint32_t w = 0; w < waves; w++)
+#pragma unroll
+                for (int q = 0; q < CPP; q++) v += red[(w * RL + r) * 64 + q * SUB + c];
+            return v;
+        };
         if (splits == 1) {
             for (uint32_t e = threadIdx.x; e < (uint32_t)E; e += threads) {
                 const uint32_t r = e / SUB, c = e % SUB;
                 if (gated) {
-                    if (c < SUB / 2) finish(r, c, sum_waves(e, 0u, 1u), sum_waves(e + SUB / 2, 0u, 1u), true);
+                    if (c < SUB / 2) finish(r, c, sum_wide(r, c), sum_wide(r, c + SUB / 2), true);
                 } else {
-                    finish(r, c, sum_waves(e, 0u, 1u), 0.f, true);
+                    finish(r, c, sum_wide(r, c), 0.f, true);
                 }
             }
             return;
         }
         for (uint32_t e = threadIdx.x; e < (uint32_t)E; e += threads) {
-            const uint32_t r = e / SUB, on = col_of(e % SUB);
+            const uint32_t r = e / SUB, c = e % SUB, on = col_of(c);
             if (r < m_rows && on < n)
-                __hip_atomic_store(&ws[((size_t)sp * m_rows + r) * n_pad + on], sum_waves(e, 0u, 1u), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                __hip_atomic_store(&ws[((size_t)sp * m_rows + r) * n_pad + on], sum_wide(r, c), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
         __builtin_amdgcn_s_waitcnt(0);  // vmcnt(0): this wave's scratch stores have completed
         __syncthreads();
@@ -329,7 +346,7 @@ static hipError_t launch_gemv4s_t(hipStream_t s, const WeightView &w, const void
     uint32_t cps = (w.k_chunks + splits - 1) / splits;
     splits = (w.k_chunks + cps - 1) / cps;
     uint32_t blocks = ((sub_tiles + 7) / 8) * 8 * splits;
-    size_t lds = (size_t)waves * RL * SUB * sizeof(float);
+    size_t lds = (size_t)waves * RL * (RL * SUB > 64 ? 64 : SUB) * sizeof(float);   // (five rows and more: every lane writes, see gemv4s_body)
     const bool one = (cps + 64 / SUB - 1) / (64 / SUB) <= waves;
     const bool runs = blocks <= 512;  // few workgroups per CU: a contiguous run of sub-tiles per XCD
 #define TWM_S_LAUNCH(AF, ONEV)                                                                                          \
