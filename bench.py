@@ -180,6 +180,44 @@ def trace_decode(T, dev, layers):
         print("%s: %.1f MB in a span of %.2f us = %.2f TB/s inside the kernel" % (name, algo_bytes(k, n) / 1e6, m[7], algo_bytes(k, n) / m[7] / 1e6))
 
 
+def mfma_mix(dev):
+    """FP16 matrix throughput under the instruction mixes of a W4A16 prefill block (twm_debug_mfma_mix): the ceilings
+    the prefill kernel's arrangement was chosen against.  Median of five timed launches per line."""
+    import ctypes as C
+    steps = 8192
+
+    def run(form, parts, per_cu):
+        vals = []
+        for i in range(7):     # (the first two settle the clock)
+            tf = C.c_float(0.0)
+            rc = dev._l.twm_debug_mfma_mix(dev.handle, form, parts, per_cu, steps, C.byref(tf))
+            assert rc == 0, dev._l.twm_last_error()
+            if i >= 2:
+                vals.append(tf.value)
+        return sorted(vals)[2]
+    rows = [
+        (0, 0, "one wave per tile column: the 32 MFMAs of a step alone"),
+        (0, 1, "... + the Q4 unpack of the next step's four B operands (52 vector instructions)"),
+        (0, 3, "... + eight ds_read_b128 (the A operands)"),
+        (0, 7, "... + four global_load_dwordx4 (nibbles, scales, the A tile's direct loads)"),
+        (0, 15, "... + four ds_write_b128 (an A tile staged through registers)"),
+    ]
+    print("| instruction mix per 32-deep step and MFMA-issuing wave | one workgroup of four waves per CU | two per CU |")
+    print("|---|---|---|")
+    for form, parts, text in rows:
+        one, two = run(form, parts, 1), run(form, parts, 2)
+        print("| %s | %.0f TFLOP/s (%.1f %% of 2.5 PFLOP/s) | %.0f TFLOP/s (%.1f %%) |" % (text, one, one / 25.0, two, two / 25.0))
+    print()
+    print("| producers and consumers: eight waves per workgroup, one per CU, 64-deep intervals, one barrier each | TFLOP/s |")
+    print("|---|---|")
+    for parts, text in ((0, "four waves issue MFMAs on operands in registers; four waves only load nibbles"),
+                        (2, "... the MFMA waves read their eight A operands per step from LDS"),
+                        (18, "... and their four B operands per step too (twelve ds_read_b128 per 32 MFMAs)"),
+                        (19, "... and the other four waves unpack the nibbles and write the f16 B tile to LDS")):
+        v = run(1, parts, 1)
+        print("| %s | %.0f (%.1f %% of 2.5 PFLOP/s) |" % (text, v, v / 25.0))
+
+
 def profiler_attached():
     """True when a rocprofiler tool library is preloaded into this process (rocprofv3 does that).  Under it the
     bench issues every launch eagerly: rocprofv3 has crashed on the host inside hipGraphLaunch on this bench's
@@ -272,6 +310,9 @@ def main():
     ap.add_argument("--pmc-copy", action="store_true",
                     help="also run four 64 MiB device-to-device copies: a kernel of known traffic to scale rocprofv3 "
                          "FETCH_SIZE / WRITE_SIZE readings by")
+    ap.add_argument("--mfma-mix", action="store_true",
+                    help="print what the matrix pipes deliver under the instruction mixes of a prefill block "
+                         "(twm_debug_mfma_mix), as a markdown table, and exit")
     ap.add_argument("--trace-decode", action="store_true",
                     help="instead of the timings: run the four M = 1 GEMVs of the layer with the library's per-workgroup "
                          "clock trace (twm_debug_trace) and print where each launch's time goes, as a markdown table")
@@ -315,6 +356,9 @@ def main():
 
     if args.trace_decode:
         trace_decode(T, dev, layers)
+        return
+    if args.mfma_mix:
+        mfma_mix(dev)
         return
 
     if args.pmc_copy:

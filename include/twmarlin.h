@@ -140,6 +140,14 @@ int twm_ctx_set_option(twm_ctx *ctx, const char *key, int value);
  * first wave has unpacked its weights, and at its end, and the hardware id of the CU it ran on (bits 0-15 HW_ID, bits
  * 16-19 the XCD).  NULL or 0 switches it off; the product kernels carry no trace code. */
 int twm_debug_trace(twm_ctx *ctx, uint32_t *trace_dev, uint32_t capacity_workgroups);
+/* Profiling aid, no counterpart in the reference: the FP16 matrix throughput (TFLOP/s, into *tflops) that this GPU
+ * delivers under the instruction mixes of a W4A16 prefill block, measured on constant data by a kernel of its own, one
+ * or two workgroups per CU, `steps` 32-deep steps (a multiple of 16).  form 0: one wave issues the 32 MFMAs of a step
+ * and, between them, the parts selected by bits of `parts`: 1 the Q4 unpack of four B operands, 2 eight ds_read_b128,
+ * 4 four global_load_dwordx4, 8 four ds_write_b128 (parts 0, 1, 3, 5, 7, 15).  form 1: eight waves per workgroup, four
+ * that only read operands from LDS (2: the A operands, 16: the B operands too) and issue MFMAs, four that load, unpack
+ * (1) and write the B operands to LDS (parts 0, 2, 18, 19).  Synchronises; uses the context's scratch. */
+int twm_debug_mfma_mix(twm_ctx *ctx, int form, int parts, int workgroups_per_cu, int steps, float *tflops);
 
 /* ---- device memory (GpuTensor::{zeros,from_host,to_host}, tensor.rs:9-104) ------ */
 

@@ -33,6 +33,7 @@ SIGNATURES = {
     "twm_ctx_info": (_int, [_vp, C.c_char_p, _sz]),
     "twm_ctx_set_option": (_int, [_vp, C.c_char_p, _int]),
     "twm_debug_trace": (_int, [_vp, _vp, _u32]),
+    "twm_debug_mfma_mix": (_int, [_vp, _int, _int, _int, _int, C.POINTER(C.c_float)]),
     "twm_malloc": (_vp, [_vp, _sz]),
     "twm_free": (_int, [_vp, _vp]),
     "twm_memcpy_h2d": (_int, [_vp, _vp, _vp, _sz]),

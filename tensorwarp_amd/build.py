@@ -7,7 +7,7 @@ from concurrent.futures import ThreadPoolExecutor
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libtwmarlin_hip.so")
-SOURCES = ["twm_kernels.hip", "twm_gemv4.hip", "twm_gemv4s.hip", "twm_moe.hip", "twm_stream.hip", "twm_batch.hip", "twm_prefill.hip", "twm_noalloc.hip", "twm_api.hip",
+SOURCES = ["twm_kernels.hip", "twm_gemv4.hip", "twm_gemv4s.hip", "twm_moe.hip", "twm_stream.hip", "twm_batch.hip", "twm_prefill.hip", "twm_debug_mix.hip", "twm_noalloc.hip", "twm_api.hip",
            "twm_api_weights.hip", "twm_api_gemm.hip", "twm_api_moe.hip"]
 # The batched-decode kernels read every MFMA result with vector instructions right away (scale, add):
 # with the default choice the results land in AGPRs and each costs a v_accvgpr_read first.

@@ -48,6 +48,7 @@ def test_null_handles_are_rejected_not_crashed():
     assert lib.twm_graph_begin(None) == _lib.INVALID_HANDLE
     assert lib.twm_graph_launch(None, None) == _lib.INVALID_HANDLE
     assert lib.twm_malloc(None, 16) is None
+    assert lib.twm_debug_mfma_mix(None, 0, 0, 1, 64, None) == _lib.INVALID_HANDLE
     assert lib.twm_weight_upload(None, None, None, 64, 64) is None
     assert lib.twm_weight_bytes(None) == 0
     # the fused stores, the weight cache and the expert banks

@@ -1992,3 +1992,21 @@ def test_graph_of_batched_and_prefill_launches():
                 assert np.array_equal(c.to_host(), want), ("replay", rep)
         graph.destroy()
         w.free()
+
+
+def test_instruction_mix_probe_runs_and_orders_its_rows(dev):
+    # the profiling aid behind bench.py --mfma-mix: matrix instructions alone run near the FP16 peak, every added part
+    # of a prefill block's instruction mix costs throughput, and bad arguments are errors, not launches
+    import ctypes as C
+    lib, tf = T._lib.load(), C.c_float()
+    got = {}
+    for parts in (0, 7):
+        assert lib.twm_debug_mfma_mix(dev.handle, 0, parts, 1, 4096, C.byref(tf)) == T._lib.OK, lib.twm_last_error()
+        got[parts] = tf.value
+    assert 1500 < got[0] < 2600 and 500 < got[7] < got[0], got
+    assert lib.twm_debug_mfma_mix(dev.handle, 1, 19, 1, 4096, C.byref(tf)) == T._lib.OK, lib.twm_last_error()
+    assert 500 < tf.value < 2600, tf.value
+    assert lib.twm_debug_mfma_mix(dev.handle, 0, 4, 1, 4096, C.byref(tf)) == T._lib.UNSUPPORTED_OP
+    assert lib.twm_debug_mfma_mix(dev.handle, 0, 0, 3, 4096, C.byref(tf)) == T._lib.SHAPE_ERROR
+    assert lib.twm_debug_mfma_mix(dev.handle, 1, 0, 2, 4096, C.byref(tf)) == T._lib.SHAPE_ERROR
+    assert lib.twm_debug_mfma_mix(dev.handle, 0, 0, 1, 100, C.byref(tf)) == T._lib.SHAPE_ERROR
