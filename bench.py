@@ -36,7 +36,7 @@ LAYER_05B = [("qkv", 896, 1152), ("o", 896, 896), ("gate_up", 896, 9728), ("down
 CFG0 = [("cfg0", 4096, 4096)]                                                                     # the single-GEMV configuration
 # HBM bytes per gate_up launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, each scaled by
 # what the same counter reads for a 64 MiB copy (profiles/k_gemv4s_gate_up_m1_hbm_traffic.md).
-GATE_UP_TRAFFIC_BYTES = 76679700
+GATE_UP_TRAFFIC_BYTES = 76647700
 
 
 def algo_bytes(k, n, m=1):
