@@ -116,6 +116,10 @@ int twm_ctx_info(twm_ctx *ctx, char *buf, size_t buf_len);
  *                   with the activations shared through LDS (32-row blocks; "nt" 1 / 2 = tiles per wave, 4 / 3 =
  *                   two / three column quads per workgroup, "waves" 8 / 16 = two / four k-slices per workgroup)
  *   "dequant_src"   which repacked copy twm_weight_dequant_f16 unpacks: 0 = 16-column tiles, 1 = column lanes
+ *   "tune_on_upload" new weight handles (twm_weight_upload, twm_weight_from_device, twm_weight_fuse_n; not the paired
+ *                   gate/up handles) get measured plans at once, as if twm_weight_tune had been called on them: 1 = for
+ *                   the decode row counts 1, 4, 8, 16, 32; 2 = also for the prefill row counts 128, 512, 2048; 0 (default)
+ *                   = no.  Costs about half a second per row count and handle; a handle whose tuning fails is not returned.
  *   "weight_copies" the repacked orders a new weight handle is given: 0 or 3 = both, 1 = 16-column tiles only,
  *                   2 = column lanes only (twm_weight_ensure)
  *   "sub_waves"     waves per workgroup of the sub-tile kernels when "sub" forces their width (1 .. 16)

@@ -66,6 +66,7 @@ twm_ctx *twm_ctx_create(int ordinal)
     c->trace = TraceBuf{nullptr, 0};
     c->dequant_src = 0;
     c->weight_copies = 0;
+    c->tune_on_upload = 0;
     c->m1_exact = 0;
     c->m1_align16 = 0;
     c->m1_splits = 0;
@@ -237,6 +238,11 @@ int twm_ctx_set_option(twm_ctx *ctx, const char *key, int value)
     if (strcmp(key, "prefill_min_m") == 0) {
         if (value < 1) return api_fail(TWM_SHAPE_ERROR, "twm_ctx_set_option: prefill_min_m must be >= 1");
         ctx->prefill_min_m = value;
+        return TWM_OK;
+    }
+    if (strcmp(key, "tune_on_upload") == 0) {
+        if (value < 0 || value > 2) return api_fail(TWM_SHAPE_ERROR, "twm_ctx_set_option: tune_on_upload must be 0, 1 or 2");
+        ctx->tune_on_upload = value;
         return TWM_OK;
     }
     if (strcmp(key, "weight_copies") == 0) {
@@ -607,7 +613,11 @@ static M1Form choose_m1_form(int exact, int force_sub, int force_waves, int forc
     // 64-column kernel.
     const uint32_t tiles64 = n_pad / 64, passes16 = (k_chunks + 3) / 4, passes32 = (k_chunks + 1) / 2;
     const bool narrow16 = tiles64 <= 64, wide16 = tiles64 >= 256 && passes16 <= 8;
-    uint32_t sub = narrow16 || wide16 ? 16 : 32, sub_waves = (sub == 16 && passes16 <= 8) ? 8 : 16;
+    // K of 6144 .. 8192 from 128 tiles on: sixteen waves of one pass each on 16 columns (8192 -> 8192 8.9 against 10.0 us on
+    // 32 columns, 8192 -> 10240 11.4 / 14.3, 8192 -> 28672 25.0 / 26.2 on whole tiles, 6144 -> 16384 12.4 / 13.2, 6656 -> 13312
+    // 12.4 / 12.9, 8192 -> 57344 level; not K = 5120 (5120 -> 15360 11.1 / 10.6) nor fewer tiles (7168 -> 7168 8.2 / 7.9))
+    const bool deep16 = tiles64 >= 128 && passes16 >= 12 && passes16 <= 16;
+    uint32_t sub = narrow16 || wide16 || deep16 ? 16 : 32, sub_waves = (sub == 16 && passes16 <= 8) ? 8 : 16;
     // 65 .. 255 tiles on a deeper K: still 32 columns, the waves looping over their passes -- sixteen of them up to 128
     // tiles and 160 chunks, eight beyond (13824 -> 5120 12.2 against 14.6 us on whole tiles with a K-split, 8192 -> 8192
     // 9.4 / 12.4, 18944 -> 4608 15.3 / 17.1, 28672 -> 8192 24.2 / 27.5, 8192 -> 10240 14.2 / 15.1, 5120 -> 15360 10.5 / 11.0)

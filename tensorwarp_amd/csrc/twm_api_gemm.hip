@@ -44,7 +44,7 @@ static DecodePlan plan_gemv4(uint32_t n_tiles, uint32_t k_chunks, int force_nt, 
 struct SubPlan {
     uint32_t sub, waves;
 };
-static SubPlan plan_gemv4_sub(uint32_t tiles64, uint32_t k_chunks, uint32_t m, bool a_f32)
+static SubPlan plan_gemv4_sub(uint32_t tiles64, uint32_t k_chunks, uint32_t m, bool a_f32, bool gated)
 {
     const SubPlan none = {0, 0};
     // shallow K, one row: short-lived workgroups on sub-tiles, whose waves sum by lane swaps and one LDS hop, are ahead
@@ -80,6 +80,18 @@ static SubPlan plan_gemv4_sub(uint32_t tiles64, uint32_t k_chunks, uint32_t m, b
         // rounds: 49.3 against 47.8)
         const uint32_t rounds = (tiles64 + 255) / 256;
         const bool poor_fill = tiles64 * 5 < rounds * 256 * 4;
+        // One row, plain store: since the waves sum by lane swaps and the first wave alone finishes, 16 columns are ahead
+        // on every wide shape measured, whatever the fill and the depth -- f16 row on eight waves (one pass each up to
+        // K = 4096, two or three up front, the pass loop beyond): 4096 -> 28672 12.1 against 12.7 us on whole tiles,
+        // 3584 -> 152064 45.5 / 47.6, 4096 -> 128256 44.4 / 45.8, 8192 -> 28672 21.3 / 23.2, 8192 -> 10240 9.8 / 11.6,
+        // 11008 -> 16384 17.5 / 18.4, 5120 -> 15360 level; f32 row on four waves up to K = 4096 (4096 -> 28672 13.0 / 14.3,
+        // 4096 -> 14336 8.1 / 8.9, 3584 -> 152064 level), eight up to K = 8192 (8192 -> 28672 22.5 / 24.8, 5120 -> 15360
+        // 10.0 / 10.4), four beyond (11008 -> 16384 19.2 / 19.3).  Two rows stay with the rules below (3584 -> 152064 at
+        // M = 2: 48.7 against 47.8), and so does the gated store, which takes 32 columns.
+        if (m == 1 && !gated) {
+            if (a_f32) return SubPlan{16, passes16 <= 8 || passes16 > 64 ? 4u : 8u};
+            return SubPlan{16, passes16 <= 4 ? 4u : passes16 <= 8 ? ((passes16 + 1u) & ~1u) : 8u};
+        }
         // (an even number of waves, so that the workgroups of a CU lie evenly on its four SIMDs and four of them fit:
         // 3584 -> 37888 at M = 1 13.4 us on eight waves, the eighth idle, against 14.2 on seven)
         if (!a_f32 && m <= 2 && passes16 <= 8 && poor_fill) return SubPlan{16, (passes16 + 1u) & ~1u};
@@ -316,7 +328,7 @@ static LaunchForm choose_form(const FormEnv &e, uint32_t n_tiles, uint32_t k_chu
         sub.waves = e.sub_waves ? (uint32_t)e.sub_waves : e.waves ? (uint32_t)e.waves : 8;
     } else if (e.sub == 0 && !e.nt && !e.waves && !splits) {
         // (an explicit nt, waves or split factor asks for the 64-column kernel's plan)
-        sub = plan_gemv4_sub(tiles64, k_chunks, m, a_f32);
+        sub = plan_gemv4_sub(tiles64, k_chunks, m, a_f32, gated);
         // the gated store splits a sub-tile into a gate and an up half: 16 columns would read 128-byte runs
         // (3584 -> 2 x 18944 at M = 1: 17.0 us on 16 columns, 16.3 on 32, 17.1 on whole tiles)
         if (gated && sub.sub == 16) sub = SubPlan{32, 8};

@@ -41,6 +41,7 @@ struct twm_ctx {
     int prefill_bm;       // prefill block form: 0 = choose, 64 = 64 rows x 256 columns, 128 = 128 x 256, 192 = 128 rows x 192 columns
     int prefill_min_m;    // M from which the LDS/MFMA prefill kernel runs instead of 16-row decode blocks
     int dequant_src;      // which copy twm_weight_dequant_f16 unpacks: 0 = 16-column tiles, 1 = column-lane
+    int tune_on_upload;   // new plain weight handles are tuned at once: 0 = no, 1 = decode row counts, 2 = prefill row counts too
     int weight_copies;    // copies a new weight handle is given: 0 or 3 = both, 1 = 16-column tiles only, 2 = column-lane only
     int m1_align16;       // twm_gemm_tw_marlin_m1: 1 = refuse arrays that are not 16-byte aligned instead of running k_ref_gemv
     int m1_exact;         // twm_gemm_tw_marlin_m1: 1 = f32 activations and f32 FMAs in the reference's order

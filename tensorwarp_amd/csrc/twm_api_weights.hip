@@ -98,8 +98,30 @@ int twm_weight_drop(twm_ctx *ctx, twm_weight *w, int copies)
 
 int twm_weight_copies(const twm_weight *w) { return w ? copies_of(w) : 0; }
 
+// Option "tune_on_upload": a new plain weight handle gets its measured plans right away (twm_weight_tune over the row
+// counts of decode, 1 = {1, 4, 8, 16, 32}, and with 2 also of prefill, {128, 512, 2048}).  A handle whose tuning fails is
+// not returned: the caller asked for measured plans.
+static twm_weight *tune_new_weight(twm_ctx *ctx, twm_weight *w)
+{
+    if (!w || !ctx->tune_on_upload || w->n == 0 || w->k == 0) return w;
+    static const uint32_t ms[] = {1, 4, 8, 16, 32, 128, 512, 2048};
+    if (twm_weight_tune(ctx, w, ms, ctx->tune_on_upload >= 2 ? 8u : 5u) != TWM_OK) {
+        twm_weight_destroy(w);
+        return nullptr;
+    }
+    return w;
+}
+
+static twm_weight *weight_from_device(twm_ctx *ctx, const uint8_t *packed_dev, const uint16_t *scales_dev, uint32_t k, uint32_t n);
+
 twm_weight *twm_weight_from_device(twm_ctx *ctx, const uint8_t *packed_dev, const uint16_t *scales_dev, uint32_t k,
                                    uint32_t n)
+{
+    twm_weight *w = weight_from_device(ctx, packed_dev, scales_dev, k, n);
+    return w ? tune_new_weight(ctx, w) : nullptr;
+}
+
+static twm_weight *weight_from_device(twm_ctx *ctx, const uint8_t *packed_dev, const uint16_t *scales_dev, uint32_t k, uint32_t n)
 {
     if (!ctx) { api_fail(TWM_INVALID_HANDLE, "twm_weight_from_device: null context"); return nullptr; }
     if (ctx->capturing) { api_fail(TWM_UNSUPPORTED_OP, "twm_weight_from_device: not allowed inside a graph capture"); return nullptr; }
@@ -179,7 +201,7 @@ twm_weight *twm_weight_fuse_n(twm_ctx *ctx, const twm_weight *const *parts, uint
         weight_release(w);
         return nullptr;
     }
-    return w;
+    return tune_new_weight(ctx, w);
 }
 
 twm_weight *twm_weight_upload(twm_ctx *ctx, const uint8_t *packed_host, const uint16_t *scales_host, uint32_t k,
@@ -189,7 +211,7 @@ twm_weight *twm_weight_upload(twm_ctx *ctx, const uint8_t *packed_host, const ui
     if (ctx->capturing) { api_fail(TWM_UNSUPPORTED_OP, "twm_weight_upload: not allowed inside a graph capture"); return nullptr; }
     if (check_kn("twm_weight_upload", k, n)) return nullptr;
     size_t pbytes = (size_t)(k / 32) * n * 16, sbytes = (size_t)(k / 32) * n * 2;
-    if (pbytes == 0) return twm_weight_from_device(ctx, nullptr, nullptr, k, n);
+    if (pbytes == 0) return weight_from_device(ctx, nullptr, nullptr, k, n);
     if (!packed_host || !scales_host) { api_fail(TWM_INVALID_HANDLE, "twm_weight_upload: null pointer"); return nullptr; }
     void *stage = nullptr;
     hipError_t e = hipMalloc(&stage, pbytes + sbytes);
@@ -198,9 +220,9 @@ twm_weight *twm_weight_upload(twm_ctx *ctx, const uint8_t *packed_host, const ui
     uint16_t *s = (uint16_t *)(p + pbytes);
     twm_weight *w = nullptr;
     if (twm_memcpy_h2d(ctx, p, packed_host, pbytes) == TWM_OK && twm_memcpy_h2d(ctx, s, scales_host, sbytes) == TWM_OK)
-        w = twm_weight_from_device(ctx, p, s, k, n);
+        w = weight_from_device(ctx, p, s, k, n);
     (void)hipFree(stage);
-    return w;
+    return w ? tune_new_weight(ctx, w) : nullptr;
 }
 
 twm_weight *twm_weight_gate_up(twm_ctx *ctx, const uint8_t *gate_packed_dev, const uint16_t *gate_scales_dev,
@@ -213,7 +235,7 @@ twm_weight *twm_weight_gate_up(twm_ctx *ctx, const uint8_t *gate_packed_dev, con
     size_t pbytes = (size_t)(k / 32) * n * 16, sbytes = (size_t)(k / 32) * n * 2;
     twm_weight *w = nullptr;
     if (pbytes == 0) {
-        w = twm_weight_from_device(ctx, nullptr, nullptr, k, n);
+        w = weight_from_device(ctx, nullptr, nullptr, k, n);
     } else {
         void *stage = nullptr;
         hipError_t e = hipMalloc(&stage, pbytes + sbytes);
@@ -221,7 +243,7 @@ twm_weight *twm_weight_gate_up(twm_ctx *ctx, const uint8_t *gate_packed_dev, con
         uint8_t *p = (uint8_t *)stage;
         uint16_t *sc = (uint16_t *)(p + pbytes);
         if (twm_pair_gate_up(ctx, gate_packed_dev, gate_scales_dev, up_packed_dev, up_scales_dev, k, ffn_dim, p, sc) == TWM_OK)
-            w = twm_weight_from_device(ctx, p, sc, k, n);  // synchronises the stream before returning
+            w = weight_from_device(ctx, p, sc, k, n);  // synchronises the stream before returning
         else
             (void)hipStreamSynchronize(ctx->stream);
         (void)hipFree(stage);

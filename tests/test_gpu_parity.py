@@ -1310,6 +1310,32 @@ def test_weight_tune_keeps_results_and_travels_with_the_blob(dev):
         x.free()
 
 
+def test_tune_on_upload_option(dev):
+    # option "tune_on_upload": a new handle is tuned at once (1 = the decode row counts, 2 = the prefill ones too); whatever
+    # the tuner keeps, results stay inside the bar, and a handle made with the option off has no measured plans
+    k, n = 1024, 640
+    packed, scales = O.synth_packed(k, n, 1600), O.synth_scales(k, n, 1601)
+    lib = T._lib.load()
+    assert lib.twm_ctx_set_option(dev.handle, b"tune_on_upload", 3) == T._lib.SHAPE_ERROR
+    plain = T.MarlinWeight.upload(dev, packed, scales, k, n)
+    assert all(plain.tuned_plan(m) is None for m in (1, 4, 8, 16, 32, 128))
+    try:
+        dev.set_option("tune_on_upload", 2)
+        w = T.MarlinWeight.upload(dev, packed, scales, k, n)
+        fused = T.MarlinWeight.fuse_n(dev, [plain, plain])
+    finally:
+        dev.set_option("tune_on_upload", 0)
+    print("kept plans:", {m: w.tuned_plan(m) for m in (1, 4, 8, 16, 32, 128, 512, 2048)})
+    for m in (1, 8, 32):
+        a16 = O.synth_act_f16(m, k, 1610 + m)
+        truth = O.gemm_f64(f16_as_f32(a16), packed, scales, m, k, n)
+        assert rel_err(run_gemm(dev, w, a16, m, n, 0), truth) < TIGHT, (m, w.tuned_plan(m))
+        got2 = run_gemm(dev, fused, a16, m, 2 * n, 0)
+        assert rel_err(got2[:, :n], truth) < TIGHT and rel_err(got2[:, n:], truth) < TIGHT, (m, fused.tuned_plan(m))
+    for x in (plain, w, fused):
+        x.free()
+
+
 def test_repacked_weight_blob_round_trip_through_a_warp_file(dev, tmp_path):
     from tensorwarp_amd import warp_cache as W
     k, n, ffn = 640, 200, 96

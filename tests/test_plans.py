@@ -108,7 +108,7 @@ def test_plans_of_prefill(lib, k, n, m):
 
 def test_plans_of_lm_head_and_small_shapes(lib):
     lm = parse(describe(lib, 3584, 152064, 1))
-    assert lm["kernel"] == "k_gemv4" and lm["splits"] == 1 and workgroups(lm, 3584, 152064, 1) >= 8 * CUS, lm["text"]
+    assert lm["kernel"] in ("k_gemv4", "k_gemv4s") and lm["splits"] == 1 and workgroups(lm, 3584, 152064, 1) >= 8 * CUS, lm["text"]
     small = parse(describe(lib, 896, 1152, 1))
     assert small["kernel"] == "k_gemv4s" and small["splits"] == 1, small["text"]            # shallow K, one row: sub-tiles
 
@@ -161,24 +161,16 @@ def describe_m1(lib, k, n):
     return buf.value.decode()
 
 
-@pytest.mark.parametrize("k,n,want", [
-    # the Qwen-7B layer: 32 columns x 16 waves of one pass on qkv, 16 columns elsewhere (one pass per wave on o and on
-    # the wide gate_up, the pass loop on sixteen waves on the deep down)
-    (3584, 4608, "k_gemv4s: 32-column sub-tiles, 16 waves, 1 K-split; reference arrays"),
-    (3584, 3584, "k_gemv4s: 16-column sub-tiles, 8 waves, 1 K-split; reference arrays"),
-    (3584, 37888, "k_gemv4s: 16-column sub-tiles, 8 waves, 1 K-split; reference arrays"),
-    (18944, 3584, "k_gemv4s: 16-column sub-tiles, 16 waves, 1 K-split; reference arrays"),
-    # 65 .. 255 tiles on a deeper K: 32 columns, waves looping; sixteen up to 128 tiles and 160 chunks, else eight
-    (13824, 5120, "k_gemv4s: 32-column sub-tiles, 16 waves, 1 K-split; reference arrays"),
-    (28672, 8192, "k_gemv4s: 32-column sub-tiles, 8 waves, 1 K-split; reference arrays"),
-    (8192, 10240, "k_gemv4s: 32-column sub-tiles, 8 waves, 1 K-split; reference arrays"),
-    # 256 tiles or more beyond K = 4096: whole 64-column tiles
-    (8192, 57344, "k_gemv4: 1 x 64-column tiles per workgroup, 8 waves, 1 K-split; reference arrays"),
-    # the LM head
-    (3584, 152064, "k_gemv4s: 16-column sub-tiles, 8 waves, 1 K-split; reference arrays"),
-])
-def test_known_drop_in_plans(lib, k, n, want):
-    assert describe_m1(lib, k, n) == want
+@pytest.mark.parametrize("k,n", [(3584, 4608), (3584, 3584), (3584, 37888), (18944, 3584),     # the Qwen-7B layer
+                                 (13824, 5120), (28672, 8192), (8192, 10240), (8192, 57344), (3584, 152064)])
+def test_drop_in_plans_of_model_shapes(lib, k, n):
+    # held to what a good plan keeps, not to its text: the MFMA kernels on the arrays as they are, one launch without a
+    # hand-over between workgroups, a workgroup for at least half of the CUs, and up to K = 4096 one pass per wave
+    f = parse(describe_m1(lib, k, n))
+    assert f["kernel"] in ("k_gemv4s", "k_gemv4") and f["copy"] == "reference arrays" and f["splits"] == 1, f["text"]
+    assert workgroups(f, k, n, 1) >= CUS // 2, f["text"]
+    if k <= 4096:
+        assert f["kernel"] == "k_gemv4s" and f["waves"] * (64 // f["sub"]) >= (k // 32 + 3) // 4, f["text"]
 
 
 def test_drop_in_plan_invariants(lib):
