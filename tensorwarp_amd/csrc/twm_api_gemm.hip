@@ -331,7 +331,9 @@ static LaunchForm choose_form(const FormEnv &e, uint32_t n_tiles, uint32_t k_chu
         sub = plan_gemv4_sub(tiles64, k_chunks, m, a_f32, gated);
         // the gated store splits a sub-tile into a gate and an up half: 16 columns would read 128-byte runs
         // (3584 -> 2 x 18944 at M = 1: 17.0 us on 16 columns, 16.3 on 32, 17.1 on whole tiles)
-        if (gated && sub.sub == 16) sub = SubPlan{32, 8};
+        // (up to two rows and K = 4096 sixteen waves of one pass each: 3584 -> 2 x 18944 15.0 against 15.8 us on eight
+        // waves in the pass loop, 4096 -> 2 x 11008 10.5 / 11.4, at M = 2 15.3 / 15.7 and 10.8 / 11.7; four rows 13.1 / 12.6)
+        if (gated && sub.sub == 16) sub = SubPlan{32, (m <= 2 && k_chunks > 16 && k_chunks <= 32) ? 16u : 8u};
     }
     if (sub.sub) {
         f.kind = kFormSubTile;
