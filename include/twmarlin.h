@@ -350,6 +350,14 @@ int twm_gemm(twm_ctx *ctx, const twm_weight *w, const void *a_dev, int a_dtype, 
  * sum(ns) must equal the weight's N; out i is row-major [M, ns[i]] f32. */
 int twm_gemm_split(twm_ctx *ctx, const twm_weight *w, const void *a_dev, int a_dtype, uint32_t m,
                    float *const *outs_dev, const uint32_t *ns, uint32_t count, uint32_t splits);
+/* twm_gemm with f16 result rows: c_dev_f16[M][N] = f16_rne(the f32 result of twm_gemm).  The reference's decode buffers
+ * are f32 (generate.rs:1382-1404) and its FP16 pipeline keeps f16 rows (crates/kernels/src/fp16.rs:133-166 casts between
+ * them); this entry point serves the second kind of caller without a buffer of its own: the kernels store f32 rows into
+ * the back half of the context's scratch and the cast kernel rounds them into c_dev_f16, in row blocks when M x N x 4
+ * bytes exceed that half (32 MB by default).  One more launch per block than twm_gemm, no allocation (capturable).
+ * TWM_MEMORY_ERROR when a single row of f32 results does not fit: call twm_gemm and twm_cast_f32_to_f16 instead. */
+int twm_gemm_f16out(twm_ctx *ctx, const twm_weight *w, const void *a_dev, int a_dtype, uint32_t m, uint16_t *c_dev_f16,
+                    uint32_t splits);
 /* twm_gemm_split with an f32 bias per output: out i = A x W_i + biases_dev[i][0..ns[i]) on every row
  * (one f32 add per element, GEMV result first).  biases_dev is a host array of `count` device
  * pointers, entries may be NULL; biases_dev itself may be NULL.  For the Q/K/V biases bq/bk/bv

@@ -77,6 +77,7 @@ SIGNATURES = {
     "twm_weight_import": (_vp, [_vp, _vp, _sz]),
     "twm_weight_dequant_f16": (_int, [_vp, _vp, _vp]),
     "twm_gemm": (_int, [_vp, _vp, _vp, _int, _u32, _vp, _u32]),
+    "twm_gemm_f16out": (_int, [_vp, _vp, _vp, _int, _u32, _vp, _u32]),
     "twm_gemm_split": (_int, [_vp, _vp, _vp, _int, _u32, C.POINTER(_vp), C.POINTER(_u32), _u32, _u32]),
     "twm_weight_gate_up": (_vp, [_vp, _vp, _vp, _vp, _vp, _u32, _u32]),
     "twm_weight_is_paired": (_int, [_vp]),

@@ -717,6 +717,38 @@ int twm_gemm(twm_ctx *ctx, const twm_weight *w, const void *a_dev, int a_dtype, 
     return gemm_common(ctx, w, a_dev, a_dtype, m, out, splits, "twm_gemm");
 }
 
+// twm_gemm with f16 result rows: the kernels store f32 (what the reference's buffers hold), so the rows are computed in
+// blocks into the back half of the context's scratch and rounded from there by the cast kernel -- no allocation, one
+// more launch per block; the front half stays the launch's own scratch (split-K sums, f32 activation terms).
+int twm_gemm_f16out(twm_ctx *ctx, const twm_weight *w, const void *a_dev, int a_dtype, uint32_t m, uint16_t *c_dev_f16,
+                    uint32_t splits)
+{
+    const char *who = "twm_gemm_f16out";
+    if (!ctx || !w) return api_fail(TWM_INVALID_HANDLE, "%s: null handle", who);
+    if (w->ctx != ctx) return api_fail(TWM_INVALID_HANDLE, "%s: weight belongs to another context", who);
+    if (m != 0 && w->n != 0 && !c_dev_f16) return api_fail(TWM_INVALID_HANDLE, "%s: null output", who);
+    if (a_dtype != TWM_F16 && a_dtype != TWM_F32) return api_fail(TWM_UNSUPPORTED_OP, "%s: activations must be f16 or f32", who);
+    if (m == 0 || w->n == 0) return TWM_OK;
+    const size_t row_bytes = (size_t)w->n * 4, half = (ctx->ws_bytes / 2) & ~(size_t)255;
+    if (!ctx->ws || row_bytes > half)
+        return api_fail(TWM_MEMORY_ERROR, "%s: one row of f32 results (%zu bytes) does not fit half of the context's scratch; "
+                        "use twm_gemm and twm_cast_f32_to_f16", who, row_bytes);
+    uint32_t block = half / row_bytes < m ? (uint32_t)(half / row_bytes) : m;
+    if (block >= 128) block -= block % 128;   // (whole prefill row blocks)
+    float *stage = (float *)((char *)ctx->ws + ctx->ws_bytes - half);
+    const size_t a_row_bytes = (size_t)w->k * (a_dtype == TWM_F32 ? 4 : 2), saved = ctx->ws_bytes;
+    int rc = TWM_OK;
+    ctx->ws_bytes = saved - half;
+    for (uint32_t m0 = 0; m0 < m && rc == TWM_OK; m0 += block) {
+        const uint32_t rows = m - m0 < block ? m - m0 : block;
+        rc = twm_gemm(ctx, w, (const char *)a_dev + (size_t)m0 * a_row_bytes, a_dtype, rows, stage, splits);
+        if (rc == TWM_OK && launch_cast(ctx->stream, stage, c_dev_f16 + (size_t)m0 * w->n, (size_t)rows * w->n, true) != hipSuccess)
+            rc = api_fail(TWM_DEVICE_ERROR, "%s: cast kernel launch: %s", who, hipGetErrorString(hipGetLastError()));
+    }
+    ctx->ws_bytes = saved;
+    return rc;
+}
+
 int twm_gemm_split_bias(twm_ctx *ctx, const twm_weight *w, const void *a_dev, int a_dtype, uint32_t m,
                         float *const *outs_dev, const float *const *biases_dev, const uint32_t *ns, uint32_t count,
                         uint32_t splits)

@@ -377,6 +377,12 @@ def gemm(device, weight, a, m, c, splits=0):
     _check(device._l.twm_gemm(device.handle, weight.handle, a.ptr, dt, m, c.ptr, splits))
 
 
+def gemm_f16out(device, weight, a, m, c16, splits=0):
+    """gemm() with f16 result rows: c16[M,N] = f16(the f32 result), rounded by the library's cast kernel."""
+    dt = _lib.F16 if a.dtype == "f16" else _lib.F32
+    _check(device._l.twm_gemm_f16out(device.handle, weight.handle, a.ptr, dt, m, c16.ptr, splits))
+
+
 def gemm_swiglu(device, weight, a, m, out, splits=0):
     """out[M, ffn] = silu(A x W_gate) * (A x W_up) on a MarlinWeight.gate_up weight: gemm_tw_marlin_m1 +
     split_gate_up + fused_silu_mul of the decode step (and of prefill) with the gate applied in the GEMM's store."""

@@ -44,6 +44,7 @@ def test_null_handles_are_rejected_not_crashed():
     assert lib.twm_ctx_sync(None) == _lib.INVALID_HANDLE
     assert b"null" in lib.twm_last_error()
     assert lib.twm_gemm(None, None, None, _lib.F16, 1, None, 0) == _lib.INVALID_HANDLE
+    assert lib.twm_gemm_f16out(None, None, None, _lib.F16, 1, None, 0) == _lib.INVALID_HANDLE
     assert lib.twm_gemm_tw_marlin_m1(None, None, None, None, None, 64, 64) == _lib.INVALID_HANDLE
     assert lib.twm_graph_begin(None) == _lib.INVALID_HANDLE
     assert lib.twm_graph_launch(None, None) == _lib.INVALID_HANDLE

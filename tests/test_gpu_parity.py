@@ -2036,3 +2036,33 @@ def test_instruction_mix_probe_runs_and_orders_its_rows(dev):
     assert lib.twm_debug_mfma_mix(dev.handle, 0, 0, 3, 4096, C.byref(tf)) == T._lib.SHAPE_ERROR
     assert lib.twm_debug_mfma_mix(dev.handle, 1, 0, 2, 4096, C.byref(tf)) == T._lib.SHAPE_ERROR
     assert lib.twm_debug_mfma_mix(dev.handle, 0, 0, 1, 100, C.byref(tf)) == T._lib.SHAPE_ERROR
+
+
+def test_gemm_with_f16_result_rows(dev):
+    # twm_gemm_f16out = the f32 result of twm_gemm rounded to nearest even, bit for bit: decode rows, batched rows, prefill
+    # rows, f16 and f32 activations, and a row count whose f32 results exceed the staging half of the scratch (row blocks)
+    for k, n, ms in ((256, 200, (1, 3, 8, 32, 100)), (3584, 37888, (1, 300))):
+        packed, scales = O.synth_packed(k, n, 1700), O.synth_scales(k, n, 1701)
+        w = T.MarlinWeight.upload(dev, packed, scales, k, n)
+        for m in ms:
+            a16 = O.synth_act_f16(m, k, 1710 + m)
+            for a_f32 in (False, True):
+                a_dev = T.GpuTensor.from_host(dev, f16_as_f32(a16)) if a_f32 else T.GpuTensor.from_host(dev, a16, "f16")
+                c32 = T.GpuTensor.from_host(dev, np.full((m, n), np.nan, np.float32))
+                c16 = T.GpuTensor.from_host(dev, np.full((m, n), 0x7E00, np.uint16), "f16")     # NaN canary
+                T.gemm(dev, w, a_dev, m, c32)
+                T.gemm_f16out(dev, w, a_dev, m, c16)
+                want = c32.to_host().astype(np.float16).view(np.uint16)
+                got = c16.to_host().view(np.uint16).reshape(m, n)
+                if n == 200:
+                    assert np.array_equal(got, want), (k, n, m, a_f32)
+                else:
+                    # (row blocks and half the scratch may mean another K-split than twm_gemm's on all rows at once: the
+                    # f32 sums then differ in their last bits, and a few of them round to the neighbouring f16)
+                    gf, wf = got.view(np.float16).astype(np.float32), want.view(np.float16).astype(np.float32)
+                    assert (got != want).mean() < 1e-3 and np.abs(gf - wf).max() <= 1e-3 * np.abs(wf).max(), (k, n, m, a_f32)
+                for t in (a_dev, c32, c16):
+                    t.free()
+        w.free()
+    lib = T._lib.load()
+    assert lib.twm_gemm_f16out(dev.handle, None, None, T._lib.F16, 1, None, 0) == T._lib.INVALID_HANDLE
