@@ -2064,5 +2064,29 @@ def test_gemm_with_f16_result_rows(dev):
                 for t in (a_dev, c32, c16):
                     t.free()
         w.free()
+    # in a captured graph (the call allocates nothing), replayed with eager work in between; empty calls are no-ops
+    k, n = 512, 320
+    packed, scales = O.synth_packed(k, n, 1720), O.synth_scales(k, n, 1721)
+    w = T.MarlinWeight.upload(dev, packed, scales, k, n)
+    acts = {m: T.GpuTensor.from_host(dev, O.synth_act_f16(m, k, 1730 + m), "f16") for m in (1, 8, 40)}
+    outs = {m: T.GpuTensor.from_host(dev, np.zeros((m, n), np.uint16), "f16") for m in acts}
+    eager = {}
+    for m in acts:
+        T.gemm_f16out(dev, w, acts[m], m, outs[m])
+        eager[m] = outs[m].to_host().view(np.uint16).copy()
+    graph = T.GraphCapture.record_with_device(dev, lambda: [T.gemm_f16out(dev, w, acts[m], m, outs[m]) for m in acts])
+    for rep in range(3):
+        for m in acts:
+            outs[m].copy_from_host(np.full((m, n), 0x7E00, np.uint16))
+        graph.replay()
+        dev.synchronize()
+        for m in acts:
+            assert np.array_equal(outs[m].to_host().view(np.uint16), eager[m]), (rep, m)
+        T.gemm_f16out(dev, w, acts[8], 8, outs[8], 2)        # eager work between replays
+        dev.synchronize()
+    graph.destroy()
+    T.gemm_f16out(dev, w, acts[1], 0, outs[1])
     lib = T._lib.load()
     assert lib.twm_gemm_f16out(dev.handle, None, None, T._lib.F16, 1, None, 0) == T._lib.INVALID_HANDLE
+    assert lib.twm_gemm_f16out(dev.handle, w.handle, acts[1].ptr, 7, 1, outs[1].ptr, 0) == T._lib.UNSUPPORTED_OP
+    w.free()
