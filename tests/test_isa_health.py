@@ -1,5 +1,5 @@
-"""What the compiler made of the two kernels whose speed hangs on its instruction scheduling, checked on the CPU from the
-gfx950 assembly: no register spills, and no prefetch moved down to its first use.
+"""What the compiler made of the kernels whose speed hangs on its instruction scheduling and register allocation, checked
+on the CPU from the gfx950 assembly: no register spills, and no prefetch moved down to its first use.
 
 k_batch and k_prefill keep several chunks of loads in flight; their source pins every prefetch in place, but the
 compiler's choices move with unrelated code (a multiply added to k_batch's store loops once moved the main loop's weight
@@ -18,7 +18,12 @@ import pytest
 from tensorwarp_amd import build
 
 CSRC = build.CSRC
-FILES = ["twm_batch.hip", "twm_prefill.hip"]
+FILES = ["twm_batch.hip", "twm_prefill.hip", "twm_gemv4s.hip"]
+# The sub-tile kernel's looping forms with many rows (and with four f32 rows on 16 columns) run out of registers with
+# two register sets live.  No planner chooses them (five rows and up run only where one pass per wave covers K; f32
+# rows on a deep K take 32 columns or whole tiles); only the option knobs reach them, and the parity tests do.
+FORCED_ONLY_SPILLS = ("8k_gemv4sILi32ELi16ELb0ELb0ELb0E", "8k_gemv4sILi16ELi4ELb1ELb0ELb0E", "8k_gemv4sILi16ELi8ELb0ELb0ELb0E",
+                      "8k_gemv4sILi16ELi16ELb0ELb0ELb0E")
 
 
 def assembly_of(src, out_dir):
@@ -46,8 +51,8 @@ def kernels():
 
 
 def test_no_kernel_spills(kernels):
-    assert len(kernels) > 40
-    spilled = {name: scratch for name, (body, scratch) in kernels.items() if scratch}
+    assert len(kernels) > 80
+    spilled = {name: scratch for name, (body, scratch) in kernels.items() if scratch and not any(f in name for f in FORCED_ONLY_SPILLS)}
     assert not spilled, spilled
 
 
