@@ -120,6 +120,8 @@ int twm_ctx_info(twm_ctx *ctx, char *buf, size_t buf_len);
  *                   gate/up handles) get measured plans at once, as if twm_weight_tune had been called on them: 1 = for
  *                   the decode row counts 1, 4, 8, 16, 32; 2 = also for the prefill row counts 128, 512, 2048; 0 (default)
  *                   = no.  Costs about half a second per row count and handle; a handle whose tuning fails is not returned.
+ *                   The tuner measures kernels of both repacked orders, so a tuned handle holds both copies whatever
+ *                   "weight_copies" says (twm_weight_drop frees one afterwards).
  *   "weight_copies" the repacked orders a new weight handle is given: 0 or 3 = both, 1 = 16-column tiles only,
  *                   2 = column lanes only (twm_weight_ensure)
  *   "sub_waves"     waves per workgroup of the sub-tile kernels when "sub" forces their width (1 .. 16)
